@@ -1,0 +1,131 @@
+"""KV-cache scatter, paged-attention decode and host slot mapping.  Test infrastructure only.
+
+Follows:
+  ReshapeAndCache call sites   mindformers/modules/paged_attention_mgr.py:60-62,
+                               mindformers/parallel_core/inference/transformer/flash_attention.py:126-127
+  PagedAttention call sites    mindformers/modules/paged_attention_mgr.py:64-70,
+                               mindformers/parallel_core/inference/transformer/flash_attention.py:135-143
+  unfused attention math       mindformers/modules/infer_attention.py:303-340 (scores*scale, fp32 softmax,
+                               probabilities cast to the compute dtype, PV), GQA head repeat :329-340,
+                               mindformers/parallel_core/inference/transformer/dot_product_attention.py:94-133
+  slot mapping                 mindformers/modules/block_tables.py:65-121
+"""
+import numpy as np
+
+from .numerics import round_to
+
+
+def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
+    """In-place scatter: cache.reshape(-1, n_kv, D)[slot[i]] = x[i]; slot < 0 is padding.
+
+    key/value: [T, n_kv*D] (or any shape with T rows); caches: [num_blocks, block_size, n_kv, D].
+    Returns key, as the primitive does (paged_attention_mgr.py:62 returns the op's output which
+    the caller only uses as an ordering edge, infer_attention.py:453-454).
+    """
+    nb, bs, n_kv, d = key_cache.shape
+    kc = key_cache.reshape(nb * bs, n_kv, d)
+    t = len(slot_mapping)
+    k = np.asarray(key).reshape(t, n_kv, d)
+    for i in range(t):
+        s = int(slot_mapping[i])
+        if s < 0:
+            continue
+        kc[s] = k[i]
+    if value is not None and value_cache is not None:
+        vc = value_cache.reshape(nb * bs, n_kv, d)
+        v = np.asarray(value).reshape(t, n_kv, d)
+        for i in range(t):
+            s = int(slot_mapping[i])
+            if s >= 0:
+                vc[s] = v[i]
+    return key
+
+
+def gather_kv(cache, block_table, length):
+    """Rows 0..length-1 of one sequence: token j lives at cache[block_table[j // bs], j % bs]."""
+    nb, bs, n_kv, d = cache.shape
+    j = np.arange(length)
+    blocks = np.asarray(block_table)[j // bs].astype(np.int64)
+    return cache[blocks, j % bs]          # [length, n_kv, D]
+
+
+def paged_attention_decode(query, key_cache, value_cache, block_tables, context_lens,
+                           n_head, n_kv_head, scale, prob_dtype=None):
+    """out[b, h] = softmax(scale * q[b,h] . K_b[:L_b]^T) V_b[:L_b], kv head = h // (n_head/n_kv).
+
+    query [B, n_head*D]; context_lens[b] counts the new token (it is already in the cache:
+    tests/st/test_infer/test_infer_module/test_infer_attention.py:249, block_tables.py:113).
+    Computed in float64; ``prob_dtype`` optionally rounds the probabilities through the compute
+    dtype before the PV product, as the reference's unfused path does (infer_attention.py:324-326).
+    A sequence with L_b <= 0 yields zeros.
+    """
+    nb, bs, n_kv, d = key_cache.shape
+    assert n_kv == n_kv_head
+    b_sz = len(context_lens)
+    q = np.asarray(query, dtype=np.float64).reshape(b_sz, n_head, d)
+    n_rep = n_head // n_kv_head
+    out = np.zeros((b_sz, n_head, d), dtype=np.float64)
+    for b in range(b_sz):
+        length = int(context_lens[b])
+        if length <= 0:
+            continue
+        k = gather_kv(key_cache, block_tables[b], length).astype(np.float64)     # [L, n_kv, D]
+        v = gather_kv(value_cache, block_tables[b], length).astype(np.float64)
+        for h in range(n_head):
+            g = h // n_rep
+            s = (k[:, g, :] @ q[b, h]) * scale
+            s = s - s.max()
+            p = np.exp(s)
+            p = p / p.sum()
+            if prob_dtype is not None:
+                p = round_to(p, prob_dtype).astype(np.float64)
+            out[b, h] = p @ v[:, g, :]
+    return out.reshape(b_sz, n_head * d)
+
+
+def causal_prefill_attention(query, key, value, seq_lens, n_head, n_kv_head, scale):
+    """Varlen causal attention over packed [T, heads*D] rows (FlashAttentionScore, TH layout,
+    flash_attention.py:129-134; unfused form infer_attention.py:342-404).  float64."""
+    t = query.shape[0]
+    d = query.shape[1] // n_head
+    q = np.asarray(query, dtype=np.float64).reshape(t, n_head, d)
+    k = np.asarray(key, dtype=np.float64).reshape(t, n_kv_head, d)
+    v = np.asarray(value, dtype=np.float64).reshape(t, n_kv_head, d)
+    n_rep = n_head // n_kv_head
+    out = np.zeros_like(q)
+    start = 0
+    for length in seq_lens:
+        length = int(length)
+        for i in range(length):
+            for h in range(n_head):
+                g = h // n_rep
+                s = (k[start:start + i + 1, g] @ q[start + i, h]) * scale
+                p = np.exp(s - s.max())
+                p /= p.sum()
+                out[start + i, h] = p @ v[start:start + i + 1, g]
+        start += length
+    return out.reshape(t, n_head * d)
+
+
+def decode_slot_mapping(block_tables, context_lens, block_size):
+    """slot = table[(L-1)//bs]*bs + (L-1)%bs, clamped to the last allocated block
+    (block_tables.py:113-119)."""
+    slots = []
+    for table, length in zip(block_tables, context_lens):
+        table = [int(x) for x in table if int(x) >= 0]
+        cur = int(length) - 1
+        idx = cur // block_size
+        if idx >= len(table):
+            idx = len(table) - 1
+        slots.append(table[idx] * block_size + cur % block_size)
+    return np.asarray(slots, dtype=np.int32)
+
+
+def prefill_slot_mapping(block_tables, context_lens, block_size, max_input_length):
+    """Per-token slots for a padded [B, max_input_length] prefill; padding = -1
+    (block_tables.py:77-96, written as the naive per-token loop)."""
+    out = -np.ones((len(context_lens), max_input_length), dtype=np.int32)
+    for b, length in enumerate(context_lens):
+        for j in range(int(length)):
+            out[b, j] = int(block_tables[b][j // block_size]) * block_size + j % block_size
+    return out.reshape(-1)

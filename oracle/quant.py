@@ -1,0 +1,68 @@
+"""W8A16 / W8A8 quantized linear arithmetic.  Test infrastructure only.
+
+PARITY UNPINNED against the reference: these cells live in the third-party ``mindspore_gs`` package
+(>= 0.6.0, otherwise unpinned; mindformers/version_control.py:326-334) and lower to the Ascend primitives
+WeightQuantBatchMatmul / DynamicQuant / QuantBatchMatmul.  MindFormers only dispatches to them
+(mindformers/modules/quantizers/rtn_quantizer.py:61-67, ptq_quantizer.py:52-59,
+smooth_quant_quantizer.py:61-67; configs mindformers/utils/quantization_config.py:257-300,404-478) and
+its tests pin no numerics for them (tests/st/test_ut/test_models/test_auto/test_auto_quantizer.py:31-77).
+The convention stated here is this build's contract:
+
+  weights     s_n = max_k |W[n,k]| / 127 ; w_i8 = clip(rint(W / s_n), -127, 127)   (rint: ties to even)
+  W8A16       y = (x . w_i8^T) * s_n (+ bias)             x in bf16/fp16, accumulate wide, scale after
+  act quant   xs = x * smooth ; s_t = max_k |xs[t,k]| / 127 (float32) ; q = clip(rint(xs / s_t), -128, 127)
+  W8A8        acc = q . w_i8^T  (exact int32) ; y = acc * s_t * s_n (+ bias)
+
+What *is* fixed independently of convention, and tested: int32 accumulators equal exact integer matmul;
+power-of-two scales with small-integer activations make W8A16 exact; the int8 grid round-trips.
+"""
+import numpy as np
+
+
+def quantize_weight_int8(weight):
+    """Symmetric per-output-channel int8.  weight [out, in] -> (w_i8 [out, in] int8, scale [out] float32)."""
+    w = np.asarray(weight, dtype=np.float32)
+    amax = np.abs(w).max(axis=1)
+    scale = (amax / np.float32(127.0)).astype(np.float32)
+    safe = np.where(scale > 0, scale, np.float32(1.0))
+    q = np.clip(np.rint(w / safe[:, None]), -127, 127).astype(np.int8)
+    return q, scale
+
+
+def w8a16_linear(x, w_i8, scale, bias=None):
+    """float64 reference of y = (x . w_i8^T) * scale (+ bias)."""
+    acc = np.asarray(x, dtype=np.float64) @ np.asarray(w_i8, dtype=np.float64).T
+    y = acc * np.asarray(scale, dtype=np.float64)[None, :]
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)
+    return y
+
+
+def dynamic_quant_per_token(x, smooth=None):
+    """Per-token dynamic int8.  All float32, in this exact operation order:
+    xs = x*smooth; s = max|xs| / 127; q = clip(rint(xs / s), -128, 127).  Zero rows get s = 0, q = 0 ...
+    returns (q int8 [T,K], s float32 [T])."""
+    xs = np.asarray(x, dtype=np.float32)
+    if smooth is not None:
+        xs = (xs * np.asarray(smooth, dtype=np.float32)[None, :]).astype(np.float32)
+    amax = np.abs(xs).max(axis=1).astype(np.float32)
+    s = (amax / np.float32(127.0)).astype(np.float32)
+    safe = np.where(s > 0, s, np.float32(1.0)).astype(np.float32)
+    q = np.clip(np.rint((xs / safe[:, None]).astype(np.float32)), -128, 127).astype(np.int8)
+    return q, s
+
+
+def int8_gemm_i32(xq, w_i8):
+    """Exact int32 accumulators acc[t,n] = sum_k xq[t,k]*w[n,k] (computed in int64, checked to fit)."""
+    acc = np.asarray(xq, dtype=np.int64) @ np.asarray(w_i8, dtype=np.int64).T
+    assert np.abs(acc).max(initial=0) < 2 ** 31
+    return acc.astype(np.int32)
+
+
+def w8a8_linear(xq, x_scale, w_i8, w_scale, bias=None):
+    """float64 reference of y = acc * s_t * s_n (+ bias)."""
+    acc = int8_gemm_i32(xq, w_i8).astype(np.float64)
+    y = acc * np.asarray(x_scale, dtype=np.float64)[:, None] * np.asarray(w_scale, dtype=np.float64)[None, :]
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)
+    return y

@@ -1,0 +1,195 @@
+"""Pin the CPU oracle against every vector the reference's own tests hold for this path.
+
+The fixtures under tests/golden/*.npz were dumped from the reference's numpy-only data files by
+tests/golden/make_fixtures.py: seeded inputs, the fp32 GOLDEN arrays and the bf16 "GPU" arrays.  The
+criterion is the reference's double benchmark (bf16 thresholds), with the oracle output rounded to bf16
+standing where the reference's device output stands.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as O
+
+R = O.round_bf16
+
+
+def _load(golden_dir, name):
+    return np.load(os.path.join(golden_dir, name))
+
+
+def _check(device, gpu, golden, what):
+    res = O.double_benchmark(R(device), gpu, golden, dtype="bfloat16")
+    assert res.ok, f"{what}: {res.messages}"
+
+
+# ---------------------------------------------------------------- flash / paged attention
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_flash_attention_vectors(golden_dir, case, n_kv):
+    z = _load(golden_dir, "flash_attention.npz")
+    nb, bs = int(z["meta_num_blocks"]), int(z["meta_block_size"])
+    nh, hid = int(z["meta_num_heads"]), int(z["meta_hidden_size"])
+    d = hid // nh
+    scale = 0.25          # test_infer_flash_attention.py:41-43
+    pq = R(z[f"in{case}_prefill_query"]).reshape(4, -1)
+    pk = R(z[f"in{case}_prefill_key"]).reshape(4, -1)
+    pv = R(z[f"in{case}_prefill_value"]).reshape(4, -1)
+    pre = O.causal_prefill_attention(pq, pk, pv, [2, 2], nh, n_kv, scale)
+    _check(pre, z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"], "prefill")
+
+    kc = np.zeros((nb, bs, n_kv, d), np.float32)
+    vc = np.zeros_like(kc)
+    O.reshape_and_cache(pk, pv, kc, vc, z[f"in{case}_prefill_slot_mapping"])
+    dk = R(z[f"in{case}_decoder_key"]).reshape(2, -1)
+    dv = R(z[f"in{case}_decoder_value"]).reshape(2, -1)
+    O.reshape_and_cache(dk, dv, kc, vc, z[f"in{case}_decoder_slot_mapping"])
+    bt = -np.ones((2, 11), np.int32)           # run_infer_flash_attention.py:58-60
+    bt[0, 0], bt[1, 0] = 2, 1
+    dq = R(z[f"in{case}_decoder_query"]).reshape(2, -1)
+    dec = O.paged_attention_decode(dq, kc, vc, bt, [3, 3], nh, n_kv, scale)
+    _check(dec, z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"], "decode")
+    # a wrong GQA head mapping or a dropped token must fail the same criterion
+    bad = O.paged_attention_decode(dq, kc, vc, bt, [2, 2], nh, n_kv, scale)
+    assert not O.double_benchmark(R(bad), z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"]).ok
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_self_attention_vectors(golden_dir, case, n_kv):
+    """QKV linear -> [q|k|v] split -> scatter -> prefill FA / decode PA -> projection
+    (attention.py:214-265,344-349; scale 1/sqrt(head_dim), attention.py:135,166)."""
+    z = _load(golden_dir, "attention.npz")
+    nb, bs = int(z["meta_num_blocks"]), int(z["meta_block_size"])
+    nh, hid = int(z["meta_num_heads"]), int(z["meta_hidden_size"])
+    d = hid // nh
+    scale = 1.0 / np.sqrt(d)
+    wqkv, wo = R(z[f"in{case}_qkv_weight"]), R(z[f"in{case}_proj_weight"])
+
+    def qkv(hs):
+        y = R(O.linear(R(hs).reshape(-1, hid), wqkv))
+        return np.split(y, [nh * d, (nh + n_kv) * d], axis=-1)
+
+    q, k, v = qkv(z[f"in{case}_prefill_hidden_states"])
+    pre = R(O.causal_prefill_attention(q, k, v, [2, 2], nh, n_kv, scale))
+    pre = O.linear(pre, wo)
+    _check(pre, z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"], "prefill")
+
+    kc = np.zeros((nb, bs, n_kv, d), np.float32)
+    vc = np.zeros_like(kc)
+    O.reshape_and_cache(k, v, kc, vc, z[f"in{case}_prefill_slot_mapping"])
+    q, k, v = qkv(z[f"in{case}_decoder_hidden_states"])
+    O.reshape_and_cache(k, v, kc, vc, z[f"in{case}_decoder_slot_mapping"])
+    bt = z[f"in{case}_block_tables"].astype(np.int32)
+    dec = R(O.paged_attention_decode(q, kc, vc, bt, [3, 3], nh, n_kv, scale))
+    dec = O.linear(dec, wo)
+    _check(dec, z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"], "decode")
+
+
+# ---------------------------------------------------------------- RoPE
+def _rope_case(z, kind, phase):
+    dim = int(z["meta_kv_channels"])
+    max_pos = int(z["meta_max_position_embedding"])
+    if kind == "rope":
+        inv, n_pos, ms = O.rope_inv_freq_default(dim, 10000), max_pos, 1.0
+    elif kind == "llama3_rope":
+        inv, n_pos, ms = O.rope_inv_freq_llama3(dim, 10000, 8.0, 1.0, 4.0, 512), max_pos, 1.0
+    else:
+        # YaRN: table length = original_max_position * scaling_factor (yarn_rotary_pos_embedding.py:104-112)
+        inv = O.rope_inv_freq_yarn(dim, 10000, 8.0, 512, 32, 1)
+        n_pos = int(512 * 8.0)
+        ms = O.yarn_mscale(8.0, 1.0) / O.yarn_mscale(8.0, 0.0)
+    cos, sin = O.rope_cos_sin_table(inv, n_pos, ms, "bf16")
+    if phase == "prefill":
+        q = R(z["in_prefill_query_for_prefill"])
+        k = R(z["in_prefill_key_for_prefill"])
+        pos = np.array([0, 1, 0, 1])        # two sequences of two tokens, TH layout
+    else:
+        q = R(z["in_decode_query_for_decode"])
+        k = R(z["in_decode_key_for_decode"])
+        pos = np.array([1, 1])              # run_infer_rotary_embedding.py:67 (positions = ones)
+    return (O.apply_rotary_half(q, cos[pos], sin[pos], 1), O.apply_rotary_half(k, cos[pos], sin[pos], 1))
+
+
+@pytest.mark.parametrize("kind", ["rope", "llama3_rope", "yarn_rope"])
+@pytest.mark.parametrize("phase", ["prefill", "decode"])
+def test_rotary_vectors(golden_dir, kind, phase):
+    z = _load(golden_dir, "rotary.npz")
+    q, k = _rope_case(z, kind, phase)
+    _check(q, z[f"gpu_{kind}_q_emb1_for_{phase}"], z[f"golden_{kind}_q_emb1_for_{phase}"], "q")
+    _check(k, z[f"gpu_{kind}_k_emb1_for_{phase}"], z[f"golden_{kind}_k_emb1_for_{phase}"], "k")
+
+
+def test_rotary_wrong_pairing_fails(golden_dir):
+    """The interleaved pairing (format 3) must not pass the rotate-half vectors."""
+    z = _load(golden_dir, "rotary.npz")
+    dim = int(z["meta_kv_channels"])
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(dim), 4, 1.0, "bf16")
+    q = R(z["in_decode_query_for_decode"]).astype(np.float64)
+    pos = np.array([1, 1])
+    c, s = cos[pos].astype(np.float64), sin[pos].astype(np.float64)
+    rot = np.empty_like(q)
+    rot[:, 0::2], rot[:, 1::2] = -q[:, 1::2], q[:, 0::2]
+    bad = q * c + rot * s
+    assert not O.double_benchmark(R(bad), z["gpu_rope_q_emb1_for_decode"], z["golden_rope_q_emb1_for_decode"]).ok
+
+
+# ---------------------------------------------------------------- norm / activation / mlp / linear
+@pytest.mark.parametrize("name,eps", [("rmsnorm_output1", 1e-5), ("rmsnorm_output2", 0.1)])
+def test_rmsnorm_vectors(golden_dir, name, eps):
+    z = _load(golden_dir, "norm.npz")
+    y = O.rms_norm(R(z["in_input"]), R(z["in_weight"]), eps)
+    _check(y, z[f"gpu_{name}"], z[f"golden_{name}"], name)
+
+
+@pytest.mark.parametrize("name,eps", [("layernorm_output1", 1e-5), ("layernorm_output2", 0.1)])
+def test_layernorm_vectors(golden_dir, name, eps):
+    z = _load(golden_dir, "norm.npz")
+    y = O.layer_norm(R(z["in_input"]), R(z["in_weight"]), None, eps)
+    _check(y, z[f"gpu_{name}"], z[f"golden_{name}"], name)
+
+
+def test_silu_mul_vectors(golden_dir):
+    z = _load(golden_dir, "activation.npz")
+    y = O.silu_mul(R(z["in_multiplicand_input"]), R(z["in_multiplier_input"]))
+    _check(y, z["gpu_output"], z["golden_output"], "silu*mul")
+
+
+@pytest.mark.parametrize("name,gated,bias", [("has_bias_gate_output", True, True), ("has_gate_output", True, False),
+                                             ("has_bias_output", False, True), ("output_only", False, False)])
+def test_mlp_vectors(golden_dir, name, gated, bias):
+    z = _load(golden_dir, "mlp.npz")
+    w1 = R(z["in_fc1_gate_weight"] if gated else z["in_fc1_no_gate_weight"])
+    b1 = R(z["in_fc1_gate_bias"] if gated else z["in_fc1_no_gate_bias"]) if bias else None
+    b2 = R(z["in_fc2_bias"]) if bias else None
+    y = O.mlp(R(z["in_input"]), w1, R(z["in_fc2_weight"]), b1, b2, gated=gated, act_dtype="bf16")
+    _check(y, z[f"gpu_{name}"], z[f"golden_{name}"], name)
+
+
+@pytest.mark.parametrize("kind", ["column", "row"])
+def test_parallel_linear_vectors(golden_dir, kind):
+    """Only 'legacy' bf16 device vectors exist for these; compare within two bf16 ulps of the value."""
+    z = _load(golden_dir, f"{kind}_parallel_linear.npz")
+    x, w, b = R(z["in_inputs"]), R(z["in_weight"]), R(z["in_bias"])
+    y0 = R(O.linear(x, w))
+    np.testing.assert_allclose(y0, z["legacy_output_only"], rtol=2 ** -7, atol=1e-6)
+    y1 = R(O.linear(x, w, b))
+    np.testing.assert_allclose(y1, z["legacy_output_with_bias"], rtol=2 ** -7, atol=1e-6)
+    if kind == "column":
+        y2 = R(O.linear(x, R(z["in_weight_tensor_input"]), b))
+        np.testing.assert_allclose(y2, z["legacy_output_use_weight"], rtol=2 ** -7, atol=1e-6)
+
+
+# ---------------------------------------------------------------- MoE layer
+@pytest.mark.parametrize("name,shared", [("tp1", True), ("tp1_no_shared", False)])
+def test_moe_layer_vectors(golden_dir, name, shared):
+    """test_infer_moe.py:31-58: T=16, H=32, E=8, k=2, n_group=topk_group=2, scale 2.5, ffn 8, rtol 4e-3 (:132-140)."""
+    z = _load(golden_dir, "moe.npz")
+    x = R(z["in_input"])
+    y = O.moe_layer(
+        x, R(z["in_router__weight__weight"]), R(z["in_router__expert_bias"]).astype(np.float32),
+        R(z["in_experts__weight1"]), R(z["in_experts__weight2"]), k=2, n_group=2, topk_group=2, scale=2.5,
+        shared_fc1=R(z["in_shared_experts__linear_fc1__weight"]) if shared else None,
+        shared_fc2=R(z["in_shared_experts__linear_fc2__weight"]) if shared else None,
+        act_dtype="bf16", router_dtype="bf16")
+    got = R(y).astype(np.float16).astype(np.float32)
+    np.testing.assert_allclose(got, z[f"golden_{name}"], rtol=4e-3, atol=2e-6)
