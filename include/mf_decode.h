@@ -1,0 +1,161 @@
+/*
+ * mf_decode.h — C ABI of the MI355X (gfx950) kernels behind MindFormers' quantized decode step.
+ *
+ * Every entry point replaces one MindSpore / golden-stick primitive that the reference calls on its
+ * incremental-inference path (the citation on each declaration is the reference call site, relative to
+ * the reference root).  Conventions:
+ *   - all pointers are DEVICE pointers unless the name says host; buffers are owned by the caller;
+ *   - `stream` is a hipStream_t passed as void*; every call only enqueues work on it and returns;
+ *   - the return value is a hipError_t (0 = success); argument errors return hipErrorInvalidValue (1)
+ *     before anything is launched, and mf_last_error() then holds a readable message;
+ *   - `dtype` selects the activation / cache element type: MF_BF16 or MF_FP16;
+ *   - nothing here allocates or frees device memory.
+ */
+#ifndef MF_DECODE_H_
+#define MF_DECODE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MF_BF16 0
+#define MF_FP16 1
+#define MF_FP32 2
+
+/* Library identification and the message of the last argument error on the calling thread. */
+const char* mf_version(void);
+const char* mf_last_error(void);
+
+/* ---- KV cache ------------------------------------------------------------------------------------- */
+
+/* ops.auto_generate.ReshapeAndCache(key, value, key_cache, value_cache, slot_mapping)
+ *   mindformers/modules/paged_attention_mgr.py:50,60-62
+ *   mindformers/parallel_core/inference/transformer/flash_attention.py:94,126-127
+ * cache.view(num_slots, n_kv_heads*head_dim)[slot_mapping[i]] = x[i] for key and value; slot < 0 skips the
+ * row (padding, mindformers/modules/block_tables.py:79-95).  value / value_cache may both be NULL (the MLA
+ * call writes one latent cache, multi_latent_attention.py:401-402).  Pure copy: bit-exact. */
+int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                         const int32_t* slot_mapping, int num_tokens, int n_kv_heads, int head_dim,
+                         int64_t num_slots, int dtype, void* stream);
+
+/* ops.ApplyRotaryPosEmb(cos_format=2)(query, key, cos, sin, batch_valid_length)
+ *   mindformers/modules/infer_attention.py:50-57
+ *   mindformers/parallel_core/inference/base_models/common/embeddings/rotary_pos_embedding.py:75,146
+ * In place, rotate-half pairing (i, i + head_dim/2): x = x*cos + rotate_half(x)*sin in fp32, rounded once.
+ * cos/sin are [num_tokens, head_dim] rows already gathered per token (table_dtype: MF_BF16/MF_FP16/MF_FP32).
+ * key may be NULL. */
+int mf_rope_half(void* query, void* key, const void* cos, const void* sin, int num_tokens, int n_heads,
+                 int n_kv_heads, int head_dim, int dtype, int table_dtype, void* stream);
+
+/* RoPE on q and k followed by the cache scatter of rotated k and of v, one launch (the sequence
+ * infer_attention.py:445,453 performs).  q and k are rotated in place. */
+int mf_rope_and_cache(void* query, void* key, const void* value, const void* cos, const void* sin,
+                      void* key_cache, void* value_cache, const int32_t* slot_mapping, int num_tokens,
+                      int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int dtype,
+                      int table_dtype, void* stream);
+
+/* ---- paged attention (decode) --------------------------------------------------------------------- */
+
+/* Bytes of scratch mf_paged_attention_decode needs for this shape (0 when the context fits one partition). */
+size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, int max_context);
+
+/* ops.auto_generate.PagedAttention(head_num, scale, kv_head_num)(query, key_cache, value_cache,
+ *                                                               block_tables, context_lens)
+ *   mindformers/modules/paged_attention_mgr.py:51-53,64-70
+ *   mindformers/parallel_core/inference/transformer/flash_attention.py:106-107,135-143
+ * out[b,h,:] = softmax(scale * q[b,h,:] . K_b[:L_b]^T) V_b[:L_b]; token j of sequence b lives at
+ * cache[block_tables[b, j / block_size], j % block_size, h / (n_heads/n_kv_heads), :]; L_b = context_lens[b]
+ * counts the token written by this step.  L_b <= 0 gives zeros.  Scores and softmax in fp32; the
+ * probabilities are rounded to `dtype` before the PV product.  head_dim in {32, 64, 128}. */
+int mf_paged_attention_decode(void* out, const void* query, const void* key_cache, const void* value_cache,
+                              const int32_t* block_tables, const int32_t* context_lens, int batch,
+                              int n_heads, int n_kv_heads, int head_dim, int block_size,
+                              int max_blocks_per_seq, int num_blocks, float scale, int dtype,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- norm / activation ---------------------------------------------------------------------------- */
+
+/* P.RmsNorm(eps)(x, gamma): mindformers/models/llama/llama_layer.py:195,225-228;
+ * mindformers/parallel_core/inference/transformer/norm.py:108,113.
+ * y = x * rsqrt(mean(x^2) + eps) * gamma, fp32 inside, one rounding.  gamma_dtype: MF_BF16/MF_FP16/MF_FP32.
+ * If residual != NULL: h = x + residual is formed first (rounded to dtype), written to sum_out, and
+ * normalised — the residual add of llama_transformer.py:1057 fused with the following norm (:1059). */
+int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* residual, const void* gamma, float eps,
+               int rows, int cols, int dtype, int gamma_dtype, void* stream);
+
+/* act(gate) * up with act = SiLU: mindformers/parallel_core/inference/transformer/mlp.py:135-140,
+ * mindformers/models/llama/llama_layer.py:419-440.  gate_up is [rows, 2*cols]; layout 0 = contiguous halves
+ * [gate | up] (mcore), 1 = interleaved columns g,u,g,u (legacy ffn_concat).  silu(gate) is rounded to dtype
+ * before the multiply, as the reference materialises it. */
+int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, int layout, int dtype, void* stream);
+
+/* out = a + b (residual add, llama_transformer.py:1057,1067). */
+int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* stream);
+
+/* ---- quantized linear ----------------------------------------------------------------------------- */
+
+size_t mf_w8a16_workspace_bytes(int m, int n, int k);
+
+/* golden-stick weight-only cell -> WeightQuantBatchMatmul, replacing P.MatMul(transpose_b=True) at
+ *   mindformers/modules/layers.py:479,526; parallel_core/inference/tensor_parallel/layers.py:186,406
+ * (swapped in by Quantizer.preprocess_model, mindformers/modules/quantizers/rtn_quantizer.py:61-67).
+ * y[m,n] = (sum_k x[m,k] * w[n,k]) * scale[n] (+ bias[n]) (+ residual[m,n]); x/y/bias/residual in `dtype`,
+ * w int8 [N,K] row-major, scale float32 [N]; products exact, fp32 accumulation, scale applied to the sum.
+ * With residual: y = round(round(acc*scale+bias) + residual).  K % 64 == 0. */
+int mf_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const void* bias,
+                  const void* residual, int m, int n, int k, int dtype, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
+/* golden-stick DynamicQuant (per-token) with the SmoothQuant multiplier folded in
+ * (quantization_config.py:363-380,438-442: act per_token needs int8 weights and activations).
+ * xs = x*smooth (fp32); s_t = max_k|xs|/127; q = clip(rint(xs/s_t), -128, 127).  smooth may be NULL. */
+int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m, int k,
+                               int dtype, void* stream);
+
+/* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
+ * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
+ * If acc_out != NULL the raw int32 accumulators are also written ([M,N] row-major).  K % 64 == 0. */
+int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const int8_t* w,
+                 const float* w_scale, const void* bias, const void* residual, int m, int n, int k, int dtype,
+                 void* stream);
+
+/* ---- mixture of experts --------------------------------------------------------------------------- */
+
+/* FusedAddTopKDiv(logits, bias, ...) — mindformers/parallel_core/inference/transformer/moe/router.py:129-140;
+ * unfused form research/deepseek3/moe.py:763-778, mindformers/modules/transformer/moe.py:1529-1576.
+ * s = sigmoid(logits); sb = s + bias; per group score = sum of its two largest sb; keep the topk_group best
+ * groups; top-k of sb over kept groups (ties: lower index); w = s[idx]; if renorm w /= sum(w); w *= scale.
+ * logits fp32 [T,E]; bias fp32 [E] or NULL; weights_out in `dtype` [T,k]; index_out int32 [T,k].
+ * E <= 1024, E % n_group == 0; n_group <= 1 or topk_group >= n_group disables group limiting. */
+int mf_moe_route(void* weights_out, int32_t* index_out, const float* logits, const float* bias, int tokens,
+                 int n_experts, int k, int n_group, int topk_group, float scale, int renorm, int dtype,
+                 void* stream);
+
+/* MoeInitRoutingV2(x, expert_index, ..., expert_tokens_count_or_cumsum_flag=2) — moe_layer.py:136-146.
+ * Stable counting sort of the (token, choice) pairs (flattened t*k + j) by expert.  permuted_x [T*k, H];
+ * row_map[t*k+j] = permuted row of that pair; counts int64 [E] (group_list, moe_layer.py:148);
+ * offsets int32 [E+1] = exclusive prefix sum of counts (for the grouped GEMM).  T*k <= 65536. */
+int mf_moe_permute(void* permuted_x, int32_t* row_map, int64_t* counts, int32_t* offsets, const void* x,
+                   const int32_t* expert_index, int tokens, int k, int n_experts, int hidden, int dtype,
+                   void* stream);
+
+/* GroupedMatmulV4(split_item=3, group_type=0, group_list_type=1) with int8 expert weights —
+ * mindformers/parallel_core/inference/transformer/moe/experts.py:116-117,136-137.
+ * Rows offsets[e]..offsets[e+1] of x use expert e: y = (x . w[e]^T) * scale[e].  w int8 [E, N, K] (K
+ * contiguous: the [E, in, out] parameter of experts.py:71-72 stored transposed at load), scale fp32 [E, N]. */
+int mf_grouped_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const int32_t* offsets,
+                          int n_experts, int total_rows, int n, int k, int dtype, void* stream);
+
+/* MoeTokenUnpermute(permuted_tokens, sorted_indices, probs) — moe_layer.py:151-155.
+ * out[t,:] = sum_j probs[t,j] * y[row_map[t*k+j],:] accumulated in fp32 in order j = 0..k-1
+ * (+ shared[t,:] if shared != NULL, the shared-expert add of moe_layer.py:159-160). */
+int mf_moe_unpermute(void* out, const void* y, const int32_t* row_map, const void* probs, const void* shared,
+                     int tokens, int k, int hidden, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MF_DECODE_H_ */

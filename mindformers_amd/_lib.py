@@ -1,0 +1,86 @@
+"""ctypes binding of libmf_decode.so (the C ABI declared in include/mf_decode.h).
+
+The library is the product: if it has not been built, loading fails loudly — there is no CPU fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmf_decode.so")
+
+MF_BF16, MF_FP16, MF_FP32 = 0, 1, 2
+
+_c = ctypes
+_P, _I, _L, _F, _Z = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float, _c.c_size_t
+
+# name -> (restype, argtypes); mirrors include/mf_decode.h one to one
+SIGNATURES = {
+    "mf_version": (_c.c_char_p, []),
+    "mf_last_error": (_c.c_char_p, []),
+    "mf_reshape_and_cache": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _P]),
+    "mf_rope_half": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "mf_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _P]),
+    "mf_paged_attention_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "mf_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _Z, _P]),
+    "mf_rmsnorm": (_I, [_P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P]),
+    "mf_silu_mul": (_I, [_P, _P, _I, _I, _I, _I, _P]),
+    "mf_add": (_I, [_P, _P, _P, _L, _I, _P]),
+    "mf_w8a16_workspace_bytes": (_Z, [_I, _I, _I]),
+    "mf_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
+    "mf_dynamic_quant_per_token": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
+    "mf_w8a8_gemm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mf_moe_route": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P]),
+    "mf_moe_permute": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mf_grouped_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mf_moe_unpermute": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+}
+
+_lib = None
+
+
+class MfKernelError(RuntimeError):
+    """A C-ABI call returned a non-zero hipError_t."""
+
+
+def load():
+    """Load the shared library once; raise if it is missing (build it with mindformers_amd/build.py)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: the HIP kernels are not built. Run `python mindformers_amd/build.py` "
+            "(or __graft_entry__.build()). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = load().mf_last_error().decode() if rc == 1 else ""
+        raise MfKernelError(f"{what} failed with hipError {rc}" + (f": {msg}" if msg else ""))
+
+
+def dtype_code(dtype):
+    if dtype == torch.bfloat16:
+        return MF_BF16
+    if dtype == torch.float16:
+        return MF_FP16
+    if dtype == torch.float32:
+        return MF_FP32
+    raise TypeError(f"unsupported dtype {dtype}")
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device=None):
+    return torch.cuda.current_stream(device).cuda_stream

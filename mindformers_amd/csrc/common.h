@@ -1,0 +1,103 @@
+// Shared device helpers for the gfx950 decode kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/mf_decode.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define MF_WAVE 64
+
+// Host-side argument error: remember the message, return hipErrorInvalidValue.
+void mf_set_error(const char* fmt, ...);
+#define MF_REQUIRE(cond, ...)                         \
+    do {                                              \
+        if (!(cond)) {                                \
+            mf_set_error(__VA_ARGS__);                \
+            return (int)hipErrorInvalidValue;         \
+        }                                             \
+    } while (0)
+
+#define MF_LAUNCH_CHECK() ((int)hipGetLastError())
+
+// ---- element types ---------------------------------------------------------------------------------
+struct BF16 {
+    using vec8 = bf16x8;
+    static constexpr int id = MF_BF16;
+    static __device__ __forceinline__ float to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        // round to nearest even; NaN stays NaN
+        uint32_t u = __float_as_uint(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct FP16 {
+    using vec8 = f16x8;
+    static constexpr int id = MF_FP16;
+    static __device__ __forceinline__ float to_float(uint16_t b) {
+        union { uint16_t u; _Float16 h; } c; c.u = b; return (float)c.h;
+    }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        union { uint16_t u; _Float16 h; } c; c.h = (_Float16)f; return c.u;   // v_cvt_f16_f32: RNE
+    }
+    static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return (uint32_t)T::from_float(lo) | ((uint32_t)T::from_float(hi) << 16);
+}
+
+template <typename T>
+__device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = T::to_float((uint16_t)(v[i] & 0xffffu));
+        f[2 * i + 1] = T::to_float((uint16_t)(v[i] >> 16));
+    }
+}
+
+// value of a float-like table entry by runtime dtype id (used for cos/sin/gamma that may be fp32)
+__device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dt) {
+    if (dt == MF_FP32) return ((const float*)p)[i];
+    uint16_t b = ((const uint16_t*)p)[i];
+    return dt == MF_BF16 ? BF16::to_float(b) : FP16::to_float(b);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+template <typename V, typename U>
+__device__ __forceinline__ V bitcast(const U& u) {
+    static_assert(sizeof(V) == sizeof(U), "size mismatch");
+    V v;
+    __builtin_memcpy(&v, &u, sizeof(V));
+    return v;
+}

@@ -1,0 +1,263 @@
+// Row-wise and elementwise kernels of the decode layer: RMSNorm (optionally fused with the preceding
+// residual add), SiLU*mul, residual add, per-token dynamic int8 quantisation.
+// All are single-pass, HBM-bound, 16-byte lane accesses; one workgroup per row where a row reduction is
+// needed (the row is held in registers between the reduction and the scaled write).
+#include "common.h"
+
+namespace {
+
+constexpr int ROW_THREADS = 256;
+constexpr int ROW_MAX_VEC = 8;   // up to 8 x (8 elements) per thread: cols <= 256*8*8 = 16384
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
+    __syncthreads();
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) t = fmaxf(t, red[i]);
+    __syncthreads();
+    return t;
+}
+
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restrict__ y,
+                                                             uint16_t* __restrict__ sum_out,
+                                                             const uint16_t* __restrict__ x,
+                                                             const uint16_t* __restrict__ residual,
+                                                             const void* __restrict__ gamma, float eps, int cols,
+                                                             int gamma_dtype) {
+    __shared__ float red[ROW_THREADS / 64];
+    const int64_t row = (int64_t)blockIdx.x * cols;
+    const int nvec = cols >> 3;
+    float v[ROW_MAX_VEC][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ROW_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * ROW_THREADS;
+        if (c < nvec) {
+            u32x4 raw = *(const u32x4*)(x + row + 8 * c);
+            unpack8<T>(raw, v[it]);
+            if (residual) {
+                float rr[8];
+                u32x4 rraw = *(const u32x4*)(residual + row + 8 * c);
+                unpack8<T>(rraw, rr);
+                u32x4 s;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[i] = pack2<T>(v[it][2 * i] + rr[2 * i], v[it][2 * i + 1] + rr[2 * i + 1]);
+                *(u32x4*)(sum_out + row + 8 * c) = s;
+                unpack8<T>(s, v[it]);                          // normalise the rounded sum, as two ops would
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += v[it][i] * v[it][i];
+        }
+    }
+    ss = block_sum(ss, red);
+    const float inv = rsqrtf(ss / (float)cols + eps);
+#pragma unroll
+    for (int it = 0; it < ROW_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * ROW_THREADS;
+        if (c < nvec) {
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float g0 = load_as_float(gamma, 8 * c + 2 * i, gamma_dtype);
+                const float g1 = load_as_float(gamma, 8 * c + 2 * i + 1, gamma_dtype);
+                o[i] = pack2<T>(v[it][2 * i] * inv * g0, v[it][2 * i + 1] * inv * g1);
+            }
+            *(u32x4*)(y + row + 8 * c) = o;
+        }
+    }
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
+// layout 0: [gate | up] halves; layout 1: interleaved g,u pairs.  8 outputs per thread.
+template <typename T>
+__global__ void silu_mul_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ gu, int rows, int cols,
+                                int layout) {
+    const int64_t nvec = (int64_t)rows * (cols >> 3);
+    const int vpr = cols >> 3;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = i / vpr;
+        const int c = (int)(i - row * vpr) * 8;
+        float g[8], u[8];
+        const uint16_t* base = gu + row * 2 * cols;
+        if (layout == 0) {
+            unpack8<T>(*(const u32x4*)(base + c), g);
+            unpack8<T>(*(const u32x4*)(base + cols + c), u);
+        } else {
+            float a[8], b[8];
+            unpack8<T>(*(const u32x4*)(base + 2 * c), a);
+            unpack8<T>(*(const u32x4*)(base + 2 * c + 8), b);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                g[j] = a[2 * j]; u[j] = a[2 * j + 1];
+                g[4 + j] = b[2 * j]; u[4 + j] = b[2 * j + 1];
+            }
+        }
+        u32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float a0 = T::to_float(T::from_float(silu_f(g[2 * j])));
+            const float a1 = T::to_float(T::from_float(silu_f(g[2 * j + 1])));
+            o[j] = pack2<T>(a0 * u[2 * j], a1 * u[2 * j + 1]);
+        }
+        *(u32x4*)(out + row * cols + c) = o;
+    }
+}
+
+template <typename T>
+__global__ void add_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ a,
+                           const uint16_t* __restrict__ b, int64_t n) {
+    const int64_t nvec = n >> 3;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
+        float x[8], y[8];
+        unpack8<T>(*(const u32x4*)(a + 8 * i), x);
+        unpack8<T>(*(const u32x4*)(b + 8 * i), y);
+        u32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = pack2<T>(x[2 * j] + y[2 * j], x[2 * j + 1] + y[2 * j + 1]);
+        *(u32x4*)(out + 8 * i) = o;
+    }
+    // tail (n not a multiple of 8)
+    for (int64_t i = (nvec << 3) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        out[i] = T::from_float(T::to_float(a[i]) + T::to_float(b[i]));
+}
+
+// Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
+// The division xs/s is a true IEEE division so that the grid point chosen equals the CPU statement.
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq,
+                                                                   float* __restrict__ x_scale,
+                                                                   const uint16_t* __restrict__ x,
+                                                                   const float* __restrict__ smooth, int cols) {
+    __shared__ float red[ROW_THREADS / 64];
+    const int64_t row = (int64_t)blockIdx.x * cols;
+    const int nvec = cols >> 3;
+    constexpr int MAXV = 12;                                  // cols <= 256*12*8 = 24576
+    float v[MAXV][8];
+    float amax = 0.f;
+#pragma unroll
+    for (int it = 0; it < MAXV; ++it) {
+        const int c = threadIdx.x + it * ROW_THREADS;
+        if (c < nvec) {
+            unpack8<T>(*(const u32x4*)(x + row + 8 * c), v[it]);
+            if (smooth) {
+                const f32x4 s0 = *(const f32x4*)(smooth + 8 * c), s1 = *(const f32x4*)(smooth + 8 * c + 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    v[it][i] = __fmul_rn(v[it][i], s0[i]);
+                    v[it][4 + i] = __fmul_rn(v[it][4 + i], s1[i]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[it][i]));
+        }
+    }
+    amax = block_max(amax, red);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float safe = s > 0.f ? s : 1.0f;
+    if (threadIdx.x == 0) x_scale[blockIdx.x] = s;
+#pragma unroll
+    for (int it = 0; it < MAXV; ++it) {
+        const int c = threadIdx.x + it * ROW_THREADS;
+        if (c < nvec) {
+            uint32_t o[2] = {0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float qf = rintf(__fdiv_rn(v[it][i], safe));
+                qf = fminf(fmaxf(qf, -128.f), 127.f);
+                o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
+            }
+            *(u32x2*)(xq + row + 8 * c) = (u32x2){o[0], o[1]};
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* residual, const void* gamma,
+                          float eps, int rows, int cols, int dtype, int gamma_dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rmsnorm: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32, "rmsnorm: bad gamma dtype");
+    MF_REQUIRE(y && x && gamma, "rmsnorm: null argument");
+    MF_REQUIRE(!residual || sum_out, "rmsnorm: residual given without sum_out");
+    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * ROW_MAX_VEC * 8,
+               "rmsnorm: cols (%d) must be a multiple of 8 and at most %d", cols, ROW_THREADS * ROW_MAX_VEC * 8);
+    MF_REQUIRE((((uintptr_t)y | (uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out) & 15) == 0,
+               "rmsnorm: pointers must be 16-byte aligned");
+    if (rows <= 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(rmsnorm_kernel<BF16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
+                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
+                           gamma_dtype);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<FP16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
+                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
+                           gamma_dtype);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, int layout, int dtype,
+                           void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "silu_mul: dtype must be bf16 or fp16");
+    MF_REQUIRE(out && gate_up, "silu_mul: null argument");
+    MF_REQUIRE(layout == 0 || layout == 1, "silu_mul: layout must be 0 (halves) or 1 (interleaved)");
+    MF_REQUIRE(cols > 0 && cols % 8 == 0, "silu_mul: cols (%d) must be a multiple of 8", cols);
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)gate_up) & 15) == 0, "silu_mul: pointers must be 16-byte aligned");
+    if (rows <= 0) return 0;
+    const int64_t nvec = (int64_t)rows * (cols / 8);
+    const int blocks = (int)min((int64_t)8192, (nvec + 255) / 256);
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(silu_mul_kernel<BF16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)gate_up, rows, cols, layout);
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<FP16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)gate_up, rows, cols, layout);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "add: dtype must be bf16 or fp16");
+    MF_REQUIRE(out && a && b, "add: null argument");
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)a | (uintptr_t)b) & 15) == 0, "add: pointers must be 16-byte aligned");
+    if (n <= 0) return 0;
+    const int blocks = (int)min((int64_t)8192, (n / 8 + 256) / 256);
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(add_kernel<BF16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)a, (const uint16_t*)b, n);
+    else
+        hipLaunchKernelGGL(add_kernel<FP16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)a, (const uint16_t*)b, n);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m,
+                                          int k, int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(xq && x_scale && x, "dynamic_quant: null argument");
+    MF_REQUIRE(k > 0 && k % 8 == 0 && k <= ROW_THREADS * 12 * 8, "dynamic_quant: k (%d) must be a multiple of 8, <= %d",
+               k, ROW_THREADS * 12 * 8);
+    MF_REQUIRE((((uintptr_t)xq & 7) | ((uintptr_t)x & 15) | ((uintptr_t)smooth & 15)) == 0,
+               "dynamic_quant: x/smooth must be 16-byte aligned, xq 8-byte aligned");
+    if (m <= 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(dynamic_quant_kernel<BF16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (const uint16_t*)x, smooth, k);
+    else
+        hipLaunchKernelGGL(dynamic_quant_kernel<FP16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (const uint16_t*)x, smooth, k);
+    return MF_LAUNCH_CHECK();
+}

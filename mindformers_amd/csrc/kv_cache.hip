@@ -1,0 +1,154 @@
+// KV-cache scatter (reshape_and_cache), rotate-half RoPE, and the two fused.
+//
+// All three are tiny HBM-bound copies: a decode step moves num_tokens * n_kv * head_dim * 2 elements.
+// Rows are moved with 16-byte lane accesses, one workgroup per token row.
+#include "common.h"
+
+namespace {
+
+// One workgroup per (token, k-or-v).  row_elems = n_kv * head_dim.
+template <int VEC_BYTES>
+__global__ void reshape_and_cache_kernel(const uint8_t* __restrict__ key, const uint8_t* __restrict__ value,
+                                         uint8_t* __restrict__ key_cache, uint8_t* __restrict__ value_cache,
+                                         const int32_t* __restrict__ slot_mapping, int row_bytes,
+                                         int64_t num_slots) {
+    const int t = blockIdx.x;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0 || slot >= num_slots) return;  // padding (or a corrupt slot: never write out of bounds)
+    const uint8_t* src = (blockIdx.y == 0 ? key : value) + (int64_t)t * row_bytes;
+    uint8_t* dst = (blockIdx.y == 0 ? key_cache : value_cache) + slot * (int64_t)row_bytes;
+    if (VEC_BYTES == 16) {
+        for (int i = threadIdx.x * 16; i < row_bytes; i += blockDim.x * 16)
+            *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
+    } else {
+        for (int i = threadIdx.x * 2; i < row_bytes; i += blockDim.x * 2)
+            *(uint16_t*)(dst + i) = *(const uint16_t*)(src + i);
+    }
+}
+
+// rotate-half on one [heads, D] row; thread p handles the pair (i, i + D/2) of head h.
+template <typename T>
+__device__ __forceinline__ void rope_row(uint16_t* x, int n_heads, int D, const void* cos, const void* sin,
+                                         int64_t table_row, int table_dtype, uint16_t* scatter_dst) {
+    const int half = D >> 1;
+    for (int p = threadIdx.x; p < n_heads * half; p += blockDim.x) {
+        const int h = p / half, i = p - h * half;
+        uint16_t* xr = x + h * D;
+        const float x1 = T::to_float(xr[i]), x2 = T::to_float(xr[i + half]);
+        const float c1 = load_as_float(cos, table_row + i, table_dtype);
+        const float s1 = load_as_float(sin, table_row + i, table_dtype);
+        const float c2 = load_as_float(cos, table_row + i + half, table_dtype);
+        const float s2 = load_as_float(sin, table_row + i + half, table_dtype);
+        const uint16_t o1 = T::from_float(x1 * c1 - x2 * s1);
+        const uint16_t o2 = T::from_float(x2 * c2 + x1 * s2);
+        xr[i] = o1;
+        xr[i + half] = o2;
+        if (scatter_dst) {
+            scatter_dst[h * D + i] = o1;
+            scatter_dst[h * D + i + half] = o2;
+        }
+    }
+}
+
+template <typename T>
+__global__ void rope_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, const void* __restrict__ cos,
+                            const void* __restrict__ sin, int n_heads, int n_kv, int D, int table_dtype) {
+    const int t = blockIdx.x;
+    const int64_t trow = (int64_t)t * D;
+    rope_row<T>(q + (int64_t)t * n_heads * D, n_heads, D, cos, sin, trow, table_dtype, nullptr);
+    if (k) rope_row<T>(k + (int64_t)t * n_kv * D, n_kv, D, cos, sin, trow, table_dtype, nullptr);
+}
+
+template <typename T>
+__global__ void rope_and_cache_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k,
+                                      const uint16_t* __restrict__ v, const void* __restrict__ cos,
+                                      const void* __restrict__ sin, uint16_t* __restrict__ key_cache,
+                                      uint16_t* __restrict__ value_cache,
+                                      const int32_t* __restrict__ slot_mapping, int n_heads, int n_kv, int D,
+                                      int64_t num_slots, int table_dtype) {
+    const int t = blockIdx.x;
+    const int64_t trow = (int64_t)t * D;
+    const int64_t slot = slot_mapping[t];
+    const bool live = slot >= 0 && slot < num_slots;
+    const int row = n_kv * D;
+    rope_row<T>(q + (int64_t)t * n_heads * D, n_heads, D, cos, sin, trow, table_dtype, nullptr);
+    rope_row<T>(k + (int64_t)t * row, n_kv, D, cos, sin, trow, table_dtype,
+                live ? key_cache + slot * row : nullptr);
+    if (live) {
+        const uint16_t* src = v + (int64_t)t * row;
+        uint16_t* dst = value_cache + slot * row;
+        if ((row & 7) == 0) {
+            for (int i = threadIdx.x * 8; i < row; i += blockDim.x * 8)
+                *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
+        } else {
+            for (int i = threadIdx.x; i < row; i += blockDim.x) dst[i] = src[i];
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                                    const int32_t* slot_mapping, int num_tokens, int n_kv_heads, int head_dim,
+                                    int64_t num_slots, int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "reshape_and_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(key && key_cache && slot_mapping, "reshape_and_cache: null key / key_cache / slot_mapping");
+    MF_REQUIRE((value == nullptr) == (value_cache == nullptr),
+               "reshape_and_cache: value and value_cache must both be given or both be null");
+    MF_REQUIRE(num_tokens >= 0 && n_kv_heads > 0 && head_dim > 0 && num_slots > 0, "reshape_and_cache: bad sizes");
+    if (num_tokens == 0) return 0;
+    const int row_bytes = n_kv_heads * head_dim * 2;
+    const bool vec = (row_bytes % 16 == 0) && (((uintptr_t)key | (uintptr_t)key_cache | (uintptr_t)value |
+                                                 (uintptr_t)value_cache) % 16 == 0);
+    dim3 grid(num_tokens, value ? 2 : 1);
+    const int threads = vec ? min(256, max(64, row_bytes / 16)) : 256;
+    if (vec)
+        hipLaunchKernelGGL(reshape_and_cache_kernel<16>, grid, dim3(threads), 0, (hipStream_t)stream,
+                           (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)key_cache, (uint8_t*)value_cache,
+                           slot_mapping, row_bytes, num_slots);
+    else
+        hipLaunchKernelGGL(reshape_and_cache_kernel<2>, grid, dim3(threads), 0, (hipStream_t)stream,
+                           (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)key_cache, (uint8_t*)value_cache,
+                           slot_mapping, row_bytes, num_slots);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_rope_half(void* query, void* key, const void* cos, const void* sin, int num_tokens,
+                            int n_heads, int n_kv_heads, int head_dim, int dtype, int table_dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rope: dtype must be bf16 or fp16");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32, "rope: bad table dtype");
+    MF_REQUIRE(query && cos && sin, "rope: null query / cos / sin");
+    MF_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope: head_dim must be even");
+    if (num_tokens == 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(rope_kernel<BF16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)query,
+                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype);
+    else
+        hipLaunchKernelGGL(rope_kernel<FP16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)query,
+                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_rope_and_cache(void* query, void* key, const void* value, const void* cos, const void* sin,
+                                 void* key_cache, void* value_cache, const int32_t* slot_mapping, int num_tokens,
+                                 int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int dtype,
+                                 int table_dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rope_and_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
+               "rope_and_cache: bad table dtype");
+    MF_REQUIRE(query && key && value && cos && sin && key_cache && value_cache && slot_mapping,
+               "rope_and_cache: null argument");
+    MF_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && num_slots > 0, "rope_and_cache: bad sizes");
+    if (num_tokens == 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(rope_and_cache_kernel<BF16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream,
+                           (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin, (uint16_t*)key_cache,
+                           (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, num_slots,
+                           table_dtype);
+    else
+        hipLaunchKernelGGL(rope_and_cache_kernel<FP16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream,
+                           (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin, (uint16_t*)key_cache,
+                           (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, num_slots,
+                           table_dtype);
+    return MF_LAUNCH_CHECK();
+}

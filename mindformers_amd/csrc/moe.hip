@@ -1,0 +1,262 @@
+// Mixture-of-experts routing kernels: group-limited sigmoid top-k router, counting-sort permute,
+// weighted unpermute.  Index work is exact; the heavy parts (row gather / weighted row sum) are plain
+// HBM-bound copies with 16-byte lane accesses.
+#include "common.h"
+
+namespace {
+
+constexpr int RT_MAX_E = 1024;
+constexpr int RT_MAX_K = 32;
+
+// One wavefront per token.
+template <typename T>
+__global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ weights_out,
+                                                      int32_t* __restrict__ index_out,
+                                                      const float* __restrict__ logits,
+                                                      const float* __restrict__ bias, int E, int k, int n_group,
+                                                      int topk_group, float scale, int renorm) {
+    __shared__ float s_plain[RT_MAX_E];     // sigmoid(logit)
+    __shared__ float s_biased[RT_MAX_E];    // sigmoid(logit) + bias, later masked
+    __shared__ float s_gscore[64];
+    __shared__ float s_thr;
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* lg = logits + (int64_t)t * E;
+
+    for (int e = lane; e < E; e += 64) {
+        const float s = 1.0f / (1.0f + __expf(-lg[e]));
+        s_plain[e] = s;
+        s_biased[e] = s + (bias ? bias[e] : 0.f);
+    }
+    __syncthreads();
+
+    if (n_group > 1 && topk_group < n_group) {
+        const int gs = E / n_group;
+        float score = -INFINITY;
+        if (lane < n_group) {
+            float a = -INFINITY, b = -INFINITY;               // two largest of the group
+            for (int i = 0; i < gs; ++i) {
+                const float v = s_biased[lane * gs + i];
+                if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+            }
+            score = gs >= 2 ? a + b : a;
+            s_gscore[lane] = score;
+        }
+        __syncthreads();
+        if (lane < n_group) {
+            int rank = 0;                                     // groups strictly ahead (ties: lower index first)
+            for (int j = 0; j < n_group; ++j) {
+                const float o = s_gscore[j];
+                rank += (o > score) || (o == score && j < lane);
+            }
+            if (rank == topk_group - 1) s_thr = score;        // the topk_group-th largest group score
+        }
+        __syncthreads();
+        const float thr = s_thr;
+        // keep groups with score >= threshold; experts of dropped groups score 0.0 (masked_fill)
+        for (int e = lane; e < E; e += 64)
+            if (!(s_gscore[e / gs] >= thr)) s_biased[e] = 0.0f;
+        __syncthreads();
+    }
+
+    // top-k by repeated wave-wide argmax (larger value first, ties to the lower index)
+    __shared__ float s_wsel[RT_MAX_K];
+    __shared__ int s_isel[RT_MAX_K];
+    float wsum = 0.f;
+    for (int j = 0; j < k; ++j) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float v = s_biased[e];
+            if (v > best) { best = v; bi = e; }               // ascending e: first maximum wins
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+        }
+        if (bi >= E) bi = 0;                                  // all -inf/NaN rows: keep indices in range
+        const float wv = s_plain[bi];
+        wsum += wv;
+        __syncthreads();
+        if (lane == 0) {
+            s_wsel[j] = wv;
+            s_isel[j] = bi;
+            s_biased[bi] = -INFINITY;
+        }
+        __syncthreads();
+    }
+    if (lane == 0) {
+        for (int j = 0; j < k; ++j) {
+            float wv = s_wsel[j];
+            if (renorm && k > 1) wv = wv / wsum;
+            wv *= scale;
+            weights_out[(int64_t)t * k + j] = T::from_float(wv);
+            index_out[(int64_t)t * k + j] = s_isel[j];
+        }
+    }
+}
+
+// Histogram + exclusive scan + stable rank.  One workgroup of 1024 threads; pairs p = t*k + j.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(int32_t* __restrict__ row_map, int64_t* __restrict__ counts,
+                                                        int32_t* __restrict__ offsets,
+                                                        const int32_t* __restrict__ expert_index, int pairs,
+                                                        int E) {
+    __shared__ int s_cnt[RT_MAX_E];
+    __shared__ int s_cur[RT_MAX_E];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) s_cnt[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < pairs; p += blockDim.x) {
+        const int e = expert_index[p];
+        if (e >= 0 && e < E) atomicAdd(&s_cnt[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {                                           // E <= 1024: a serial scan is a few microseconds
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            s_cur[e] = run;
+            offsets[e] = run;
+            counts[e] = s_cnt[e];
+            run += s_cnt[e];
+        }
+        offsets[E] = run;
+    }
+    __syncthreads();
+    // stable placement: wave 0 walks the pairs in order, 64 at a time
+    if (tid < 64) {
+        const int lane = tid;
+        for (int base = 0; base < pairs; base += 64) {
+            const int p = base + lane;
+            const bool live = p < pairs;
+            int e = live ? expert_index[p] : -1;
+            const bool ok = live && e >= 0 && e < E;
+            if (!ok) e = -1;
+            // lanes holding the same expert (10 index bits + validity)
+            uint64_t same = __ballot(ok);
+#pragma unroll
+            for (int bit = 0; bit < 10; ++bit) {
+                const uint64_t bm = __ballot((e >> bit) & 1);
+                same &= ((e >> bit) & 1) ? bm : ~bm;
+            }
+            if (ok) {
+                const uint64_t below = same & ((1ull << lane) - 1ull);
+                const int rank = __popcll(below);
+                const int dst = s_cur[e] + rank;
+                row_map[p] = dst;
+            } else if (live) {
+                row_map[p] = -1;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (ok && (same & ((1ull << lane) - 1ull)) == 0) s_cur[e] += __popcll(same);   // group leader
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+}
+
+// permuted_x[row_map[p]] = x[p / k]; one workgroup per pair.
+__global__ void moe_gather_kernel(uint16_t* __restrict__ permuted, const uint16_t* __restrict__ x,
+                                  const int32_t* __restrict__ row_map, int k, int hidden, int pairs) {
+    const int p = blockIdx.x;
+    const int dst = row_map[p];
+    if (dst < 0 || dst >= pairs) return;
+    const uint16_t* src = x + (int64_t)(p / k) * hidden;
+    uint16_t* d = permuted + (int64_t)dst * hidden;
+    for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) *(u32x4*)(d + i) = *(const u32x4*)(src + i);
+}
+
+// out[t] = sum_j probs[t,j] * y[row_map[t*k+j]] (+ shared[t]); one workgroup per token.
+template <typename T>
+__global__ void moe_unpermute_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ y,
+                                     const int32_t* __restrict__ row_map, const uint16_t* __restrict__ probs,
+                                     const uint16_t* __restrict__ shared, int k, int hidden, int pairs) {
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < k; ++j) {
+            const int row = row_map[(int64_t)t * k + j];
+            if (row < 0 || row >= pairs) continue;
+            const float pw = T::to_float(probs[(int64_t)t * k + j]);
+            float v[8];
+            unpack8<T>(*(const u32x4*)(y + (int64_t)row * hidden + i), v);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[q] += pw * v[q];
+        }
+        if (shared) {
+            // the routed sum is materialised in the activation dtype before the shared-expert add
+            float v[8];
+            unpack8<T>(*(const u32x4*)(shared + (int64_t)t * hidden + i), v);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[q] = T::to_float(T::from_float(acc[q])) + v[q];
+        }
+        u32x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) o[q] = pack2<T>(acc[2 * q], acc[2 * q + 1]);
+        *(u32x4*)(out + (int64_t)t * hidden + i) = o;
+    }
+}
+
+}  // namespace
+
+extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* logits, const float* bias,
+                            int tokens, int n_experts, int k, int n_group, int topk_group, float scale, int renorm,
+                            int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_route: dtype must be bf16 or fp16");
+    MF_REQUIRE(weights_out && index_out && logits, "moe_route: null argument");
+    MF_REQUIRE(n_experts > 0 && n_experts <= RT_MAX_E, "moe_route: n_experts (%d) must be in 1..%d", n_experts, RT_MAX_E);
+    MF_REQUIRE(k > 0 && k <= RT_MAX_K && k <= n_experts, "moe_route: k (%d) must be in 1..min(%d, n_experts)", k, RT_MAX_K);
+    if (n_group > 1 && topk_group < n_group) {
+        MF_REQUIRE(n_group <= 64 && n_experts % n_group == 0 && topk_group >= 1,
+                   "moe_route: n_group (%d) must divide n_experts, be <= 64, with 1 <= topk_group (%d)", n_group,
+                   topk_group);
+    }
+    if (tokens <= 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(moe_route_kernel<BF16>, dim3(tokens), dim3(64), 0, (hipStream_t)stream, (uint16_t*)weights_out,
+                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<FP16>, dim3(tokens), dim3(64), 0, (hipStream_t)stream, (uint16_t*)weights_out,
+                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_moe_permute(void* permuted_x, int32_t* row_map, int64_t* counts, int32_t* offsets, const void* x,
+                              const int32_t* expert_index, int tokens, int k, int n_experts, int hidden, int dtype,
+                              void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_permute: dtype must be bf16 or fp16");
+    MF_REQUIRE(permuted_x && row_map && counts && offsets && x && expert_index, "moe_permute: null argument");
+    MF_REQUIRE(n_experts > 0 && n_experts <= RT_MAX_E, "moe_permute: n_experts (%d) must be in 1..%d", n_experts, RT_MAX_E);
+    MF_REQUIRE(tokens >= 0 && k > 0 && (int64_t)tokens * k <= 65536, "moe_permute: tokens*k must be <= 65536");
+    MF_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_permute: hidden (%d) must be a multiple of 8", hidden);
+    MF_REQUIRE((((uintptr_t)permuted_x | (uintptr_t)x) & 15) == 0, "moe_permute: rows must be 16-byte aligned");
+    const int pairs = tokens * k;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, row_map, counts, offsets,
+                       expert_index, pairs, n_experts);
+    int rc = MF_LAUNCH_CHECK();
+    if (rc || pairs == 0) return rc;
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(pairs), dim3(256), 0, (hipStream_t)stream, (uint16_t*)permuted_x,
+                       (const uint16_t*)x, row_map, k, hidden, pairs);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_moe_unpermute(void* out, const void* y, const int32_t* row_map, const void* probs,
+                                const void* shared, int tokens, int k, int hidden, int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_unpermute: dtype must be bf16 or fp16");
+    MF_REQUIRE(out && y && row_map && probs, "moe_unpermute: null argument");
+    MF_REQUIRE(k > 0 && hidden > 0 && hidden % 8 == 0, "moe_unpermute: hidden (%d) must be a multiple of 8", hidden);
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)y | (uintptr_t)shared) & 15) == 0,
+               "moe_unpermute: rows must be 16-byte aligned");
+    if (tokens <= 0) return 0;
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(moe_unpermute_kernel<BF16>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)y, row_map, (const uint16_t*)probs, (const uint16_t*)shared, k, hidden,
+                           tokens * k);
+    else
+        hipLaunchKernelGGL(moe_unpermute_kernel<FP16>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)y, row_map, (const uint16_t*)probs, (const uint16_t*)shared, k, hidden,
+                           tokens * k);
+    return MF_LAUNCH_CHECK();
+}

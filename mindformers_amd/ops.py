@@ -1,0 +1,289 @@
+"""Functional wrappers over the C ABI: one Python function per MindSpore primitive on the decode path.
+
+Each wrapper checks shapes, dtypes, contiguity and device on the host (a kernel launched on operands it does
+not expect can fault the GPU), allocates the output with torch (device-memory plumbing only) and enqueues
+the kernel on torch's current stream.  Nothing is computed in Python.
+"""
+import math
+
+import torch
+
+from . import _lib
+from ._lib import check, dtype_code, ptr, stream_ptr
+
+_ACT = (torch.bfloat16, torch.float16)
+_workspaces = {}
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev_ok(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _need(isinstance(t, torch.Tensor) and t.is_cuda, "all tensors must live on the GPU")
+        _need(t.is_contiguous(), "all tensors must be contiguous")
+        dev = dev or t.device
+        _need(t.device == dev, "all tensors must be on the same device")
+    return dev
+
+
+def workspace(nbytes, device, tag="default"):
+    """A cached per-device scratch buffer (grown on demand, never shrunk)."""
+    key = (device, tag)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+# --------------------------------------------------------------------------------------------- KV cache
+def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
+    """ReshapeAndCache(key, value, key_cache, value_cache, slot_mapping) -> key.
+    key/value [T, n_kv*D] (any leading shape with T rows); caches [num_blocks, block_size, n_kv, D]."""
+    lib = _lib.load()
+    dev = _dev_ok(key, value, key_cache, value_cache, slot_mapping)
+    _need(key_cache.dim() == 4, "key_cache must be [num_blocks, block_size, n_kv_heads, head_dim]")
+    nb, bs, n_kv, d = key_cache.shape
+    _need(key.dtype in _ACT and key_cache.dtype == key.dtype, "key and key_cache must share a bf16/fp16 dtype")
+    _need(slot_mapping.dtype == torch.int32 and slot_mapping.dim() == 1, "slot_mapping must be int32 [T]")
+    t = slot_mapping.numel()
+    _need(key.numel() == t * n_kv * d, f"key has {key.numel()} elements, expected {t}*{n_kv}*{d}")
+    if value is not None:
+        _need(value_cache is not None and value_cache.shape == key_cache.shape and value.dtype == key.dtype
+              and value_cache.dtype == key.dtype and value.numel() == key.numel(), "value / value_cache mismatch")
+    else:
+        _need(value_cache is None, "value_cache given without value")
+    check(lib.mf_reshape_and_cache(ptr(key), ptr(value), ptr(key_cache), ptr(value_cache), ptr(slot_mapping), t, n_kv,
+                                   d, nb * bs, dtype_code(key.dtype), stream_ptr(dev)), "mf_reshape_and_cache")
+    return key
+
+
+def apply_rotary_pos_emb(query, key, cos, sin, n_heads, n_kv_heads, head_dim):
+    """ApplyRotaryPosEmb(cos_format=2), in place.  query [T, n_heads*D], key [T, n_kv*D] or None,
+    cos/sin [T, D] (one row per token)."""
+    lib = _lib.load()
+    dev = _dev_ok(query, key, cos, sin)
+    t = query.numel() // (n_heads * head_dim)
+    _need(query.dtype in _ACT and query.numel() == t * n_heads * head_dim, "query shape/dtype")
+    _need(key is None or (key.dtype == query.dtype and key.numel() == t * n_kv_heads * head_dim), "key shape/dtype")
+    _need(cos.dtype == sin.dtype and cos.numel() == t * head_dim and sin.numel() == t * head_dim,
+          "cos/sin must hold one [head_dim] row per token")
+    check(lib.mf_rope_half(ptr(query), ptr(key), ptr(cos), ptr(sin), t, n_heads, n_kv_heads, head_dim,
+                           dtype_code(query.dtype), dtype_code(cos.dtype), stream_ptr(dev)), "mf_rope_half")
+    return query, key
+
+
+def rope_and_cache(query, key, value, cos, sin, key_cache, value_cache, slot_mapping, n_heads):
+    """RoPE on q/k (in place) then scatter of rotated k and v into the caches, one launch."""
+    lib = _lib.load()
+    dev = _dev_ok(query, key, value, cos, sin, key_cache, value_cache, slot_mapping)
+    nb, bs, n_kv, d = key_cache.shape
+    t = slot_mapping.numel()
+    _need(query.dtype in _ACT and key.dtype == query.dtype and value.dtype == query.dtype
+          and key_cache.dtype == query.dtype and value_cache.dtype == query.dtype, "dtype mismatch")
+    _need(value_cache.shape == key_cache.shape, "cache shapes differ")
+    _need(slot_mapping.dtype == torch.int32, "slot_mapping must be int32")
+    _need(query.numel() == t * n_heads * d and key.numel() == t * n_kv * d and value.numel() == t * n_kv * d,
+          "q/k/v sizes do not match slot_mapping and the cache geometry")
+    _need(cos.dtype == sin.dtype and cos.numel() == t * d and sin.numel() == t * d, "cos/sin must be [T, head_dim]")
+    check(lib.mf_rope_and_cache(ptr(query), ptr(key), ptr(value), ptr(cos), ptr(sin), ptr(key_cache),
+                                ptr(value_cache), ptr(slot_mapping), t, n_heads, n_kv, d, nb * bs,
+                                dtype_code(query.dtype), dtype_code(cos.dtype), stream_ptr(dev)), "mf_rope_and_cache")
+    return query, key
+
+
+# --------------------------------------------------------------------------------------------- attention
+def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n_heads, n_kv_heads, scale, out=None):
+    """PagedAttention(head_num, scale, kv_head_num)(query, key_cache, value_cache, block_tables, context_lens)."""
+    lib = _lib.load()
+    dev = _dev_ok(query, key_cache, value_cache, block_tables, context_lens, out)
+    _need(key_cache.dim() == 4 and value_cache.shape == key_cache.shape, "caches must be [blocks, block_size, n_kv, D]")
+    nb, bs, n_kv, d = key_cache.shape
+    _need(n_kv == n_kv_heads, f"cache has {n_kv} kv heads, module says {n_kv_heads}")
+    _need(query.dtype in _ACT and key_cache.dtype == query.dtype and value_cache.dtype == query.dtype, "dtype mismatch")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
+    _need(context_lens.dtype == torch.int32 and context_lens.dim() == 1, "context_lens must be int32 [B]")
+    b = context_lens.numel()
+    _need(block_tables.shape[0] == b, "block_tables rows != batch")
+    _need(query.numel() == b * n_heads * d, f"query has {query.numel()} elements, expected {b}*{n_heads}*{d}")
+    max_blocks = block_tables.shape[1]
+    if out is None:
+        out = torch.empty_like(query)
+    else:
+        _need(out.shape == query.shape and out.dtype == query.dtype, "out mismatch")
+    need = lib.mf_paged_attention_workspace_bytes(b, n_heads, d, max_blocks * bs)
+    ws = workspace(need, dev, "pa") if need else None
+    check(lib.mf_paged_attention_decode(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(block_tables),
+                                        ptr(context_lens), b, n_heads, n_kv_heads, d, bs, max_blocks, nb,
+                                        float(scale), dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,
+                                        stream_ptr(dev)), "mf_paged_attention_decode")
+    return out
+
+
+# --------------------------------------------------------------------------------------------- norm / activation
+def rms_norm(x, gamma, eps, residual=None):
+    """RmsNorm(eps)(x, gamma).  With ``residual``: returns (norm(x + residual), x + residual)."""
+    lib = _lib.load()
+    dev = _dev_ok(x, gamma, residual)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    _need(gamma.numel() == cols, "gamma size")
+    y = torch.empty_like(x)
+    s = None
+    if residual is not None:
+        _need(residual.shape == x.shape and residual.dtype == x.dtype, "residual mismatch")
+        s = torch.empty_like(x)
+    check(lib.mf_rmsnorm(ptr(y), ptr(s), ptr(x), ptr(residual), ptr(gamma), float(eps), rows, cols,
+                         dtype_code(x.dtype), dtype_code(gamma.dtype), stream_ptr(dev)), "mf_rmsnorm")
+    return (y, s) if residual is not None else y
+
+
+def silu_mul(gate_up, interleaved=False):
+    """silu(gate) * up over [rows, 2*F] -> [rows, F]; halves layout (mcore) or interleaved (legacy ffn_concat)."""
+    lib = _lib.load()
+    dev = _dev_ok(gate_up)
+    _need(gate_up.dtype in _ACT and gate_up.shape[-1] % 2 == 0, "gate_up must be bf16/fp16 with an even last dim")
+    cols = gate_up.shape[-1] // 2
+    rows = gate_up.numel() // (2 * cols)
+    out = torch.empty(*gate_up.shape[:-1], cols, dtype=gate_up.dtype, device=dev)
+    check(lib.mf_silu_mul(ptr(out), ptr(gate_up), rows, cols, 1 if interleaved else 0, dtype_code(gate_up.dtype),
+                          stream_ptr(dev)), "mf_silu_mul")
+    return out
+
+
+def add(a, b):
+    lib = _lib.load()
+    dev = _dev_ok(a, b)
+    _need(a.shape == b.shape and a.dtype == b.dtype and a.dtype in _ACT, "add operands mismatch")
+    out = torch.empty_like(a)
+    check(lib.mf_add(ptr(out), ptr(a), ptr(b), a.numel(), dtype_code(a.dtype), stream_ptr(dev)), "mf_add")
+    return out
+
+
+# --------------------------------------------------------------------------------------------- quantized linear
+def w8a16_linear(x, w_i8, scale, bias=None, residual=None):
+    """WeightQuantBatchMatmul: y = (x . w_i8^T) * scale (+bias) (+residual).  x [..., K], w_i8 [N, K] int8."""
+    lib = _lib.load()
+    dev = _dev_ok(x, w_i8, scale, bias, residual)
+    _need(x.dtype in _ACT and w_i8.dtype == torch.int8 and scale.dtype == torch.float32, "dtypes: x bf16/fp16, w int8, scale fp32")
+    n, k = w_i8.shape
+    _need(x.shape[-1] == k and scale.numel() == n, "shape mismatch")
+    m = x.numel() // k
+    y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=dev)
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    _need(residual is None or (residual.dtype == x.dtype and residual.shape == y.shape), "residual mismatch")
+    need = lib.mf_w8a16_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a16_gemm(ptr(y), ptr(x), ptr(w_i8), ptr(scale), ptr(bias), ptr(residual), m, n, k,
+                            dtype_code(x.dtype), ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w8a16_gemm")
+    return y
+
+
+def dynamic_quant(x, smooth=None):
+    """DynamicQuant per token (with the smoothing vector folded in): returns (xq int8 [..., K], scale fp32 [rows])."""
+    lib = _lib.load()
+    dev = _dev_ok(x, smooth)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    k = x.shape[-1]
+    m = x.numel() // k
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [K]")
+    xq = torch.empty(x.shape, dtype=torch.int8, device=dev)
+    xs = torch.empty(m, dtype=torch.float32, device=dev)
+    check(lib.mf_dynamic_quant_per_token(ptr(xq), ptr(xs), ptr(x), ptr(smooth), m, k, dtype_code(x.dtype),
+                                         stream_ptr(dev)), "mf_dynamic_quant_per_token")
+    return xq, xs
+
+
+def w8a8_linear(xq, x_scale, w_i8, w_scale, out_dtype, bias=None, residual=None, return_acc=False):
+    """QuantBatchMatmul: int8 x int8 -> int32 -> * x_scale * w_scale (+bias) (+residual) -> out_dtype."""
+    lib = _lib.load()
+    dev = _dev_ok(xq, x_scale, w_i8, w_scale, bias, residual)
+    _need(xq.dtype == torch.int8 and w_i8.dtype == torch.int8, "xq and w must be int8")
+    _need(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "scales must be fp32")
+    _need(out_dtype in _ACT, "out_dtype must be bf16/fp16")
+    n, k = w_i8.shape
+    _need(xq.shape[-1] == k and w_scale.numel() == n, "shape mismatch")
+    m = xq.numel() // k
+    _need(x_scale.numel() == m, "x_scale must hold one scale per row")
+    y = torch.empty(*xq.shape[:-1], n, dtype=out_dtype, device=dev)
+    _need(bias is None or (bias.dtype == out_dtype and bias.numel() == n), "bias mismatch")
+    _need(residual is None or (residual.dtype == out_dtype and residual.shape == y.shape), "residual mismatch")
+    acc = torch.empty(*xq.shape[:-1], n, dtype=torch.int32, device=dev) if return_acc else None
+    check(lib.mf_w8a8_gemm(ptr(y), ptr(acc), ptr(xq), ptr(x_scale), ptr(w_i8), ptr(w_scale), ptr(bias), ptr(residual),
+                           m, n, k, dtype_code(out_dtype), stream_ptr(dev)), "mf_w8a8_gemm")
+    return (y, acc) if return_acc else y
+
+
+# --------------------------------------------------------------------------------------------- MoE
+def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, renorm=True):
+    """FusedAddTopKDiv: (expert_weight [T,k] out_dtype, expert_index [T,k] int32) from fp32 logits [T,E]."""
+    lib = _lib.load()
+    dev = _dev_ok(logits, expert_bias)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be fp32 [T, E]")
+    t, e = logits.shape
+    _need(expert_bias is None or (expert_bias.dtype == torch.float32 and expert_bias.numel() == e), "bias must be fp32 [E]")
+    w = torch.empty(t, k, dtype=out_dtype, device=dev)
+    idx = torch.empty(t, k, dtype=torch.int32, device=dev)
+    check(lib.mf_moe_route(ptr(w), ptr(idx), ptr(logits), ptr(expert_bias), t, e, k, int(n_group or 0),
+                           int(topk_group or 0), float(scale), 1 if renorm else 0, dtype_code(out_dtype),
+                           stream_ptr(dev)), "mf_moe_route")
+    return w, idx
+
+
+def moe_permute(x, expert_index, n_experts):
+    """MoeInitRoutingV2: returns (permuted_x [T*k,H], row_map int32 [T*k], counts int64 [E], offsets int32 [E+1])."""
+    lib = _lib.load()
+    dev = _dev_ok(x, expert_index)
+    _need(x.dtype in _ACT and x.dim() == 2, "x must be bf16/fp16 [T, H]")
+    _need(expert_index.dtype == torch.int32 and expert_index.dim() == 2 and expert_index.shape[0] == x.shape[0],
+          "expert_index must be int32 [T, k]")
+    t, h = x.shape
+    k = expert_index.shape[1]
+    px = torch.empty(t * k, h, dtype=x.dtype, device=dev)
+    row_map = torch.empty(t * k, dtype=torch.int32, device=dev)
+    counts = torch.empty(n_experts, dtype=torch.int64, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    check(lib.mf_moe_permute(ptr(px), ptr(row_map), ptr(counts), ptr(offsets), ptr(x), ptr(expert_index), t, k,
+                             n_experts, h, dtype_code(x.dtype), stream_ptr(dev)), "mf_moe_permute")
+    return px, row_map, counts, offsets
+
+
+def grouped_w8a16_linear(x, w_i8, scale, offsets):
+    """GroupedMatmulV4 over expert row groups.  x [R, K]; w_i8 [E, N, K]; scale [E, N]; offsets int32 [E+1]."""
+    lib = _lib.load()
+    dev = _dev_ok(x, w_i8, scale, offsets)
+    _need(x.dtype in _ACT and x.dim() == 2 and w_i8.dtype == torch.int8 and w_i8.dim() == 3, "x [R,K] bf16/fp16, w [E,N,K] int8")
+    e, n, k = w_i8.shape
+    _need(x.shape[1] == k and scale.dtype == torch.float32 and scale.numel() == e * n, "shape mismatch")
+    _need(offsets.dtype == torch.int32 and offsets.numel() == e + 1, "offsets must be int32 [E+1]")
+    y = torch.empty(x.shape[0], n, dtype=x.dtype, device=dev)
+    check(lib.mf_grouped_w8a16_gemm(ptr(y), ptr(x), ptr(w_i8), ptr(scale), ptr(offsets), e, x.shape[0], n, k,
+                                    dtype_code(x.dtype), stream_ptr(dev)), "mf_grouped_w8a16_gemm")
+    return y
+
+
+def moe_unpermute(y, row_map, probs, shared=None):
+    """MoeTokenUnpermute: out[t] = sum_j probs[t,j] * y[row_map[t*k+j]] (+ shared[t])."""
+    lib = _lib.load()
+    dev = _dev_ok(y, row_map, probs, shared)
+    t, k = probs.shape
+    h = y.shape[1]
+    _need(y.dtype in _ACT and probs.dtype == y.dtype and row_map.dtype == torch.int32 and row_map.numel() == t * k
+          and y.shape[0] == t * k, "operand mismatch")
+    _need(shared is None or (shared.dtype == y.dtype and shared.shape == (t, h)), "shared mismatch")
+    out = torch.empty(t, h, dtype=y.dtype, device=dev)
+    check(lib.mf_moe_unpermute(ptr(out), ptr(y), ptr(row_map), ptr(probs), ptr(shared), t, k, h, dtype_code(y.dtype),
+                               stream_ptr(dev)), "mf_moe_unpermute")
+    return out
+
+
+def default_scale(head_dim):
+    return 1.0 / math.sqrt(head_dim)

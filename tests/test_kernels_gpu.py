@@ -1,0 +1,410 @@
+"""Parity of the HIP kernels (called through the C ABI) against the CPU oracle.  GPU only.
+
+Bars: bit-exact for the KV scatter, the int8 quantisation grid, int32 accumulators and all index outputs;
+for floating-point outputs |err| <= 1.5 * eps(dtype) * M where M is the magnitude the rounding error of that
+op scales with (sum of |terms| of the dot product / convex combination), eps(bf16) = 2^-8, eps(fp16) = 2^-11.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import EPS, NAME, assert_within, dev, make_paged_cache, rounded, to_np
+
+pytestmark = pytest.mark.gpu
+
+ops = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load_ops():
+    global ops
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from mindformers_amd import ops as _ops
+    ops = _ops
+    yield
+
+
+# ------------------------------------------------------------------------------------------- KV scatter
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n_kv,d,bs,nb", [(64, 8, 128, 128, 40), (4, 2, 64, 16, 64), (7, 1, 32, 16, 9), (3, 3, 20, 4, 11)])
+def test_reshape_and_cache_bit_exact(dtype, t, n_kv, d, bs, nb):
+    rng = np.random.default_rng(1)
+    k = rounded(rng.normal(size=(t, n_kv * d)), dtype)
+    v = rounded(rng.normal(size=(t, n_kv * d)), dtype)
+    kc0 = rounded(rng.normal(size=(nb, bs, n_kv, d)), dtype)
+    vc0 = rounded(rng.normal(size=(nb, bs, n_kv, d)), dtype)
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[rng.integers(0, t)] = -1                       # one padding row
+    kc_ref, vc_ref = kc0.copy(), vc0.copy()
+    O.reshape_and_cache(k, v, kc_ref, vc_ref, slots)
+    kc, vc = dev(kc0, dtype), dev(vc0, dtype)
+    out = ops.reshape_and_cache(dev(k, dtype), dev(v, dtype), kc, vc, dev(slots, torch.int32))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(kc), kc_ref) and np.array_equal(to_np(vc), vc_ref)
+    assert np.array_equal(to_np(out), k)
+
+
+def test_reshape_and_cache_empty_and_key_only():
+    kc = torch.zeros(4, 16, 2, 32, dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros_like(kc)
+    empty = torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda")
+    ops.reshape_and_cache(empty, empty, kc, vc, torch.zeros(0, dtype=torch.int32, device="cuda"))
+    k = torch.randn(3, 64, device="cuda").to(torch.bfloat16)
+    ops.reshape_and_cache(k, None, kc, None, torch.tensor([5, 63, 0], dtype=torch.int32, device="cuda"))
+    torch.cuda.synchronize()
+    flat = kc.view(64, 64)
+    assert torch.equal(flat[5], k[0]) and torch.equal(flat[63], k[1]) and torch.equal(flat[0], k[2])
+    assert int((flat != 0).any(dim=1).sum()) <= 3 and not bool(vc.any())
+
+
+# ------------------------------------------------------------------------------------------- RoPE
+@pytest.mark.parametrize("dtype,table", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32)])
+@pytest.mark.parametrize("t,nh,nkv,d", [(64, 32, 8, 128), (4, 8, 2, 64), (2, 1, 1, 32)])
+def test_rope_half(dtype, table, t, nh, nkv, d):
+    rng = np.random.default_rng(2)
+    q = rounded(rng.normal(size=(t, nh * d)), dtype)
+    k = rounded(rng.normal(size=(t, nkv * d)), dtype)
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 4096, 1.0, "fp32" if table == torch.float32 else NAME[table])
+    pos = rng.integers(0, 4096, t)
+    c, s = cos[pos], sin[pos]
+    qd, kd = dev(q, dtype), dev(k, dtype)
+    ops.apply_rotary_pos_emb(qd, kd, dev(c, table), dev(s, table), nh, nkv, d)
+    for got, x, n in ((qd, q, nh), (kd, k, nkv)):
+        ref = O.apply_rotary_half(x, c, s, n)
+        xh = np.abs(x.reshape(t, n, d))
+        swapped = np.concatenate((xh[..., d // 2:], xh[..., :d // 2]), -1)
+        mag = xh * np.abs(c)[:, None, :] + swapped * np.abs(s)[:, None, :]
+        assert_within(to_np(got), ref, mag.reshape(t, n * d), dtype, ulps=1.0, what="rope")
+
+
+def test_rope_golden_decode_vectors(golden_dir):
+    """The reference's own decode vectors (position 1, bf16 tables), through the kernel."""
+    z = np.load(os.path.join(golden_dir, "rotary.npz"))
+    d = int(z["meta_kv_channels"])
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 8, 1.0, "bf16")
+    q = dev(O.round_bf16(z["in_decode_query_for_decode"]), torch.bfloat16)
+    k = dev(O.round_bf16(z["in_decode_key_for_decode"]), torch.bfloat16)
+    pos = np.array([1, 1])
+    ops.apply_rotary_pos_emb(q, k, dev(cos[pos], torch.bfloat16), dev(sin[pos], torch.bfloat16), 1, 1, d)
+    for got, name in ((q, "q"), (k, "k")):
+        res = O.double_benchmark(to_np(got), z[f"gpu_rope_{name}_emb1_for_decode"], z[f"golden_rope_{name}_emb1_for_decode"])
+        assert res.ok, res.messages
+
+
+def test_rope_and_cache_matches_separate_ops():
+    rng = np.random.default_rng(3)
+    t, nh, nkv, d, bs, nb = 16, 8, 2, 64, 16, 12
+    dtype = torch.float16
+    q = dev(rng.normal(size=(t, nh * d)), dtype)
+    k = dev(rng.normal(size=(t, nkv * d)), dtype)
+    v = dev(rng.normal(size=(t, nkv * d)), dtype)
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 512, 1.0, "fp16")
+    pos = rng.integers(0, 512, t)
+    c, s = dev(cos[pos], dtype), dev(sin[pos], dtype)
+    slots = torch.from_numpy(rng.permutation(nb * bs)[:t].astype(np.int32)).cuda()
+    slots[3] = -1
+    q1, k1 = q.clone(), k.clone()
+    kc1 = torch.zeros(nb, bs, nkv, d, dtype=dtype, device="cuda")
+    vc1 = torch.zeros_like(kc1)
+    ops.apply_rotary_pos_emb(q1, k1, c, s, nh, nkv, d)
+    ops.reshape_and_cache(k1, v, kc1, vc1, slots)
+    q2, k2 = q.clone(), k.clone()
+    kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(kc1)
+    ops.rope_and_cache(q2, k2, v, c, s, kc2, vc2, slots, nh)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+
+
+# ------------------------------------------------------------------------------------------- paged attention
+def _pa_case(rng, dtype, b, nh, nkv, d, bs, lens, max_blocks=None, std=1.0, scale=None):
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype, max_blocks=max_blocks, std=std)
+    q = rounded(rng.normal(0, std, (b, nh * d)), dtype)
+    scale = scale if scale is not None else 1.0 / np.sqrt(d)
+    out = ops.paged_attention(dev(q, dtype), dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32),
+                              dev(np.asarray(lens, np.int32), torch.int32), nh, nkv, scale)
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode(q, kc, vc, tables, lens, nh, nkv, scale)
+    mag = O.paged_attention_decode(q, kc, np.abs(vc), tables, lens, nh, nkv, scale)
+    return to_np(out), ref, mag
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_paged_attention_reference_vectors(golden_dir, case, n_kv):
+    """decode_output_{1,2} of the reference's flash-attention unit test, through scatter + attention kernels."""
+    z = np.load(os.path.join(golden_dir, "flash_attention.npz"))
+    nb, bs = int(z["meta_num_blocks"]), int(z["meta_block_size"])
+    nh, hid = int(z["meta_num_heads"]), int(z["meta_hidden_size"])
+    d = hid // nh
+    dt = torch.bfloat16
+    kc = torch.zeros(nb, bs, n_kv, d, dtype=dt, device="cuda")
+    vc = torch.zeros_like(kc)
+    ops.reshape_and_cache(dev(z[f"in{case}_prefill_key"].reshape(4, -1), dt), dev(z[f"in{case}_prefill_value"].reshape(4, -1), dt),
+                          kc, vc, dev(z[f"in{case}_prefill_slot_mapping"].astype(np.int32), torch.int32))
+    ops.reshape_and_cache(dev(z[f"in{case}_decoder_key"].reshape(2, -1), dt), dev(z[f"in{case}_decoder_value"].reshape(2, -1), dt),
+                          kc, vc, dev(z[f"in{case}_decoder_slot_mapping"].astype(np.int32), torch.int32))
+    bt = -np.ones((2, 11), np.int32)
+    bt[0, 0], bt[1, 0] = 2, 1
+    out = ops.paged_attention(dev(z[f"in{case}_decoder_query"].reshape(2, -1), dt), kc, vc, dev(bt, torch.int32),
+                              torch.tensor([3, 3], dtype=torch.int32, device="cuda"), nh, n_kv, 0.25)
+    res = O.double_benchmark(to_np(out), z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"])
+    assert res.ok, res.messages
+
+
+@pytest.mark.parametrize("dtype,b,nh,nkv,d,bs,lo,hi", [
+    (torch.float16, 4, 8, 2, 64, 16, 32, 256),        # cfg1 shape
+    (torch.bfloat16, 6, 32, 8, 128, 128, 512, 1500),  # cfg2 shape, multi-partition
+    (torch.bfloat16, 3, 28, 4, 128, 128, 600, 700),   # n_rep = 7
+    (torch.bfloat16, 2, 64, 8, 128, 128, 1000, 2100), # n_rep = 8
+    (torch.bfloat16, 2, 40, 2, 64, 32, 100, 900),     # n_rep = 20: two head groups
+    (torch.float16, 3, 2, 2, 32, 16, 1, 40),          # MHA, tiny
+    (torch.bfloat16, 2, 4, 1, 128, 24, 50, 300),      # block size not a multiple of 16
+])
+def test_paged_attention_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi):
+    rng = np.random.default_rng(b * 1000 + nh)
+    lens = rng.integers(lo, hi + 1, b)
+    got, ref, mag = _pa_case(rng, dtype, b, nh, nkv, d, bs, lens)
+    assert_within(got, ref, mag, dtype, ulps=1.5, what="paged attention")
+
+
+def test_paged_attention_edge_lengths():
+    """L = 1 returns the V row; L = 0 returns zeros; L exactly on tile / partition / block boundaries."""
+    rng = np.random.default_rng(11)
+    dtype = torch.bfloat16
+    lens = np.array([1, 0, 16, 32, 33, 512, 513, 1024, 128, 129], dtype=np.int64)
+    b, nh, nkv, d, bs = len(lens), 8, 2, 128, 128
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype)
+    q = rounded(rng.normal(size=(b, nh * d)), dtype)
+    out = to_np(ops.paged_attention(dev(q, dtype), dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32),
+                                    dev(lens.astype(np.int32), torch.int32), nh, nkv, 1 / np.sqrt(d)))
+    ref = O.paged_attention_decode(q, kc, vc, tables, lens, nh, nkv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q, kc, np.abs(vc), tables, lens, nh, nkv, 1 / np.sqrt(d))
+    assert_within(out, ref, mag, dtype, ulps=1.5, what="edge lengths")
+    assert np.all(out[1] == 0)
+    v_row = vc[tables[0, 0], 0]                           # L = 1: softmax over one token is exactly 1
+    assert np.array_equal(out[0].reshape(nkv, nh // nkv, d), np.repeat(v_row[:, None, :], nh // nkv, axis=1))
+    # single-partition path (max context <= 512) with an empty sequence
+    lens2 = np.array([0, 7, 300], dtype=np.int64)
+    kc, vc, tables, nb = make_paged_cache(rng, 3, lens2, nkv, d, bs, dtype, max_blocks=4)
+    q = rounded(rng.normal(size=(3, nh * d)), dtype)
+    out = to_np(ops.paged_attention(dev(q, dtype), dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32),
+                                    dev(lens2.astype(np.int32), torch.int32), nh, nkv, 1 / np.sqrt(d)))
+    ref = O.paged_attention_decode(q, kc, vc, tables, lens2, nh, nkv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q, kc, np.abs(vc), tables, lens2, nh, nkv, 1 / np.sqrt(d))
+    assert_within(out, ref, mag, dtype, ulps=1.5, what="single partition")
+    assert np.all(out[0] == 0)
+
+
+def test_paged_attention_block_permutation_invariant():
+    """Moving the physical blocks (and the table with them) must leave the output bit-identical."""
+    rng = np.random.default_rng(12)
+    dtype = torch.bfloat16
+    b, nh, nkv, d, bs = 4, 32, 8, 128, 128
+    lens = rng.integers(200, 1400, b)
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype)
+    q = dev(rng.normal(size=(b, nh * d)), dtype)
+    ld = dev(lens.astype(np.int32), torch.int32)
+    out1 = ops.paged_attention(q, dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32), ld, nh, nkv, 0.088)
+    perm = rng.permutation(nb)                           # new_id = perm[old_id]
+    kc2, vc2 = np.empty_like(kc), np.empty_like(vc)
+    kc2[perm], vc2[perm] = kc, vc
+    t2 = np.where(tables >= 0, perm[np.maximum(tables, 0)], -1).astype(np.int32)
+    out2 = ops.paged_attention(q, dev(kc2, dtype), dev(vc2, dtype), dev(t2, torch.int32), ld, nh, nkv, 0.088)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2)
+
+
+# ------------------------------------------------------------------------------------------- norm / activation
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols,gdt", [(64, 4096, torch.float32), (4, 512, torch.float16), (3, 8192, torch.bfloat16), (1, 32, torch.float32)])
+def test_rmsnorm(dtype, rows, cols, gdt):
+    rng = np.random.default_rng(4)
+    x = rounded(rng.normal(size=(rows, cols)), dtype)
+    g = rng.normal(1.0, 0.1, cols).astype(np.float32)
+    g = g if gdt == torch.float32 else rounded(g, gdt)
+    y = ops.rms_norm(dev(x, dtype), dev(g, gdt), 1e-5)
+    ref = O.rms_norm(x, g, 1e-5)
+    assert_within(to_np(y), ref, np.abs(ref), dtype, ulps=1.0, extra=1e-7, what="rmsnorm")
+    res = rounded(rng.normal(size=(rows, cols)), dtype)
+    y2, s2 = ops.rms_norm(dev(x, dtype), dev(g, gdt), 1e-5, residual=dev(res, dtype))
+    s_ref = rounded(x.astype(np.float64) + res, dtype)
+    assert np.array_equal(to_np(s2), s_ref)              # one rounding of an exact fp32 sum: bit-exact
+    ref2 = O.rms_norm(s_ref, g, 1e-5)
+    assert_within(to_np(y2), ref2, np.abs(ref2), dtype, ulps=1.0, extra=1e-7, what="add+rmsnorm")
+
+
+def test_rmsnorm_reference_vectors(golden_dir):
+    z = np.load(os.path.join(golden_dir, "norm.npz"))
+    for name, eps in (("rmsnorm_output1", 1e-5), ("rmsnorm_output2", 0.1)):
+        y = ops.rms_norm(dev(z["in_input"], torch.bfloat16), dev(z["in_weight"], torch.bfloat16), eps)
+        res = O.double_benchmark(to_np(y), z[f"gpu_{name}"], z[f"golden_{name}"])
+        assert res.ok, (name, res.messages)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_silu_mul(dtype, interleaved):
+    rng = np.random.default_rng(5)
+    rows, f = 5, 1376
+    gu = rounded(rng.normal(0, 2, (rows, 2 * f)), dtype)
+    out = to_np(ops.silu_mul(dev(gu, dtype), interleaved=interleaved))
+    g, u = (gu[:, 0::2], gu[:, 1::2]) if interleaved else (gu[:, :f], gu[:, f:])
+    act = rounded(O.silu(g), dtype)
+    ref = act.astype(np.float64) * u
+    # silu itself is evaluated with the fast exponential: allow one extra ulp on the activation
+    assert_within(out, ref, np.abs(ref) + EPS[dtype] * np.abs(u) * np.abs(act), dtype, ulps=1.5, extra=1e-7, what="silu_mul")
+
+
+def test_silu_mul_reference_vectors(golden_dir):
+    z = np.load(os.path.join(golden_dir, "activation.npz"))
+    gu = np.concatenate([z["in_multiplicand_input"], z["in_multiplier_input"]], axis=1)
+    out = ops.silu_mul(dev(gu, torch.bfloat16))
+    res = O.double_benchmark(to_np(out), z["gpu_output"], z["golden_output"])
+    assert res.ok, res.messages
+
+
+def test_add_bit_exact():
+    rng = np.random.default_rng(6)
+    a = rounded(rng.normal(size=(64, 4096)), torch.bfloat16)
+    b = rounded(rng.normal(size=(64, 4096)), torch.bfloat16)
+    out = ops.add(dev(a, torch.bfloat16), dev(b, torch.bfloat16))
+    assert np.array_equal(to_np(out), rounded(a.astype(np.float64) + b, torch.bfloat16))
+
+
+# ------------------------------------------------------------------------------------------- W8A16
+def _w8a16_case(rng, dtype, m, n, k, bias, residual):
+    w = rng.normal(0, 0.02, (n, k)).astype(np.float32)
+    wq, s = O.quantize_weight_int8(w)
+    x = rounded(rng.normal(size=(m, k)), dtype)
+    b = rounded(rng.normal(0, 0.1, n), dtype) if bias else None
+    r = rounded(rng.normal(size=(m, n)), dtype) if residual else None
+    y = ops.w8a16_linear(dev(x, dtype), torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda(),
+                         dev(b, dtype) if bias else None, dev(r, dtype) if residual else None)
+    v = O.w8a16_linear(x, wq, s, b)
+    dot_mag = (np.abs(x).astype(np.float64) @ np.abs(wq).astype(np.float64).T) * s[None, :]
+    extra = 2.0 ** -18 * dot_mag + 1e-9                  # fp32 accumulation of exact products
+    if residual:
+        # y = round(round(v) + r): the inner rounding may land one step away when v sits on a tie
+        vr = rounded(v, dtype).astype(np.float64)
+        ref = vr + r
+        return to_np(y), ref, np.abs(ref) + np.abs(vr), extra
+    return to_np(y), v, np.abs(v), extra
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k,bias,residual", [
+    (64, 6144, 4096, False, False), (64, 4096, 4096, False, True), (4, 704, 512, False, False),
+    (4, 512, 1376, True, True), (1, 4096, 4096, False, False), (17, 200, 1024, True, False),
+    (65, 130, 2048, False, False), (128, 256, 512, True, True), (33, 64, 64, False, False),
+])
+def test_w8a16_gemm(dtype, m, n, k, bias, residual):
+    rng = np.random.default_rng(m * 7 + n)
+    got, ref, mag, extra = _w8a16_case(rng, dtype, m, n, k, bias, residual)
+    assert_within(got, ref, mag, dtype, ulps=1.0, extra=extra, what="w8a16")
+
+
+def test_w8a16_exact_on_integer_grid():
+    """Power-of-two scales and small-integer activations make every product and sum exact: the kernel must
+    return exactly the integer matmul (catches a dropped k-step, a wrong row/column or a transposed operand)."""
+    rng = np.random.default_rng(8)
+    m, n, k = 37, 200, 1376
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    s = (2.0 ** rng.integers(-9, -6, n)).astype(np.float32)
+    x = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    y = ops.w8a16_linear(dev(x, torch.float16), torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())
+    exact = (x.astype(np.int64) @ wq.astype(np.int64).T).astype(np.float64) * s
+    assert np.array_equal(to_np(y).astype(np.float64), rounded(exact, torch.float16).astype(np.float64))
+
+
+def test_column_parallel_linear_reference_vectors(golden_dir):
+    """The reference's linear vectors are for the bf16 cell; they pin the W8A16 path's layout ([out, in] weight,
+    bias add): quantise the reference weight, run the kernel, compare with the oracle linear on the dequantised
+    weight, and check the result reproduces the reference's bf16 output to quantisation accuracy."""
+    z = np.load(os.path.join(golden_dir, "column_parallel_linear.npz"))
+    wq, s = O.quantize_weight_int8(z["in_weight"])
+    x = rounded(z["in_inputs"], torch.bfloat16)
+    b = rounded(z["in_bias"], torch.bfloat16)
+    y = ops.w8a16_linear(dev(x, torch.bfloat16), torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda(), dev(b, torch.bfloat16))
+    w_deq = wq.astype(np.float64) * s[:, None]
+    ref = O.linear(x, w_deq, b)
+    assert_within(to_np(y), ref, np.abs(ref), torch.bfloat16, ulps=1.0, extra=1e-7, what="layout")
+    # and the dequantised weight reproduces the reference's bf16 result to quantisation accuracy
+    assert np.abs(to_np(y) - z["legacy_output_with_bias"]).max() < 2e-4
+
+
+# ------------------------------------------------------------------------------------------- W8A8
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,smooth", [(256, 3584, True), (5, 512, False), (64, 18944, True), (1, 64, True)])
+def test_dynamic_quant_bit_exact(dtype, m, k, smooth):
+    rng = np.random.default_rng(9)
+    x = rounded(rng.normal(size=(m, k)), dtype)
+    if m > 2:
+        x[2] = 0                                         # an all-zero token
+    sm = rng.uniform(0.5, 2.0, k).astype(np.float32) if smooth else None
+    xq, xs = ops.dynamic_quant(dev(x, dtype), torch.from_numpy(sm).cuda() if smooth else None)
+    q_ref, s_ref = O.dynamic_quant_per_token(x, sm)
+    assert np.array_equal(to_np(xs), s_ref)
+    assert np.array_equal(to_np(xq), q_ref)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 3584, 3584), (130, 200, 1088), (1, 64, 64), (64, 257, 512)])
+def test_w8a8_gemm_int32_bit_exact(m, n, k):
+    rng = np.random.default_rng(10)
+    dtype = torch.bfloat16
+    xq = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    xs = rng.uniform(0.01, 0.05, m).astype(np.float32)
+    ws = rng.uniform(1e-4, 5e-4, n).astype(np.float32)
+    b = rounded(rng.normal(0, 0.5, n), dtype)
+    y, acc = ops.w8a8_linear(torch.from_numpy(xq).cuda(), torch.from_numpy(xs).cuda(), torch.from_numpy(wq).cuda(),
+                             torch.from_numpy(ws).cuda(), dtype, bias=dev(b, dtype), return_acc=True)
+    acc_ref = O.int8_gemm_i32(xq, wq)
+    assert np.array_equal(to_np(acc), acc_ref)
+    ref = O.w8a8_linear(xq, xs, wq, ws, b)
+    assert_within(to_np(y), ref, np.abs(ref) + np.abs(b), dtype, ulps=1.0, extra=1e-6, what="w8a8 dequant")
+
+
+# ------------------------------------------------------------------------------------------- MoE
+@pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1)])
+def test_moe_route(t, e, k, ng, tg):
+    rng = np.random.default_rng(13)
+    logits = rng.normal(size=(t, e)).astype(np.float32)
+    bias = rng.normal(0, 0.1, e).astype(np.float32)
+    w, idx = ops.moe_route(torch.from_numpy(logits).cuda(), torch.from_numpy(bias).cuda(), k, ng, tg, 2.5, torch.bfloat16)
+    w_ref, idx_ref = O.topk_router(logits, bias, k, ng, tg, 2.5)
+    assert np.array_equal(to_np(idx), idx_ref)
+    assert_within(to_np(w), w_ref, np.abs(w_ref), torch.bfloat16, ulps=1.0, what="router weights")
+
+
+def test_moe_permute_grouped_unpermute():
+    rng = np.random.default_rng(14)
+    dtype = torch.bfloat16
+    t, h, e, k, f = 40, 256, 16, 4, 128
+    x = rounded(rng.normal(size=(t, h)), dtype)
+    idx = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+    idx[:, 0] = np.minimum(idx[:, 0], 5)                 # leave some experts empty, some crowded (> 16 rows)
+    px, row_map, counts, offsets = ops.moe_permute(dev(x, dtype), torch.from_numpy(idx).cuda(), e)
+    px_ref, map_ref, cnt_ref = O.moe_permute(x, idx, e)
+    assert np.array_equal(to_np(row_map), map_ref) and np.array_equal(to_np(counts), cnt_ref)
+    assert np.array_equal(to_np(offsets), np.concatenate(([0], np.cumsum(cnt_ref))).astype(np.int32))
+    assert np.array_equal(to_np(px), px_ref)
+
+    w1 = rng.normal(0, 0.05, (e, 2 * f, h)).astype(np.float32)       # [E, N, K]
+    q1, s1 = zip(*(O.quantize_weight_int8(w1[i]) for i in range(e)))
+    q1, s1 = np.stack(q1), np.stack(s1)
+    y1 = ops.grouped_w8a16_linear(px, torch.from_numpy(q1).cuda(), torch.from_numpy(s1).cuda(), offsets)
+    deq1 = q1.astype(np.float64) * s1[..., None]                      # [E, N, K] -> oracle wants [E, in, out]
+    ref1 = O.grouped_matmul(px_ref, np.transpose(deq1, (0, 2, 1)), cnt_ref)
+    mag1 = O.grouped_matmul(np.abs(px_ref), np.abs(np.transpose(deq1, (0, 2, 1))), cnt_ref)
+    assert_within(to_np(y1), ref1, np.abs(ref1), dtype, ulps=1.0, extra=2.0 ** -18 * mag1 + 1e-9, what="grouped gemm")
+
+    probs = rounded(rng.uniform(0.1, 1.0, (t, k)), dtype)
+    yy = rounded(rng.normal(size=(t * k, h)), dtype)
+    sh = rounded(rng.normal(size=(t, h)), dtype)
+    out = ops.moe_unpermute(dev(yy, dtype), row_map, dev(probs, dtype), shared=dev(sh, dtype))
+    routed = O.moe_unpermute(yy, map_ref, probs)
+    ref = rounded(routed, dtype).astype(np.float64) + sh
+    mag = np.abs(ref) + np.abs(rounded(routed, dtype))
+    assert_within(to_np(out), ref, mag, dtype, ulps=1.5, extra=1e-6, what="unpermute")
