@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized decode step on one MI355X.
+
+A "step" is one pass of one decode layer over one batch: the Llama-3.1-8B-shape W8A16 layer at batch 64
+(hidden 4096, 32 query / 8 KV heads, head_dim 128, FFN 14336, context lengths uniform in [512, 4096], bf16 KV
+cache in 128-token blocks behind a shuffled block table), synthetic seeded inputs already resident in HBM.
+Prints ONE JSON line: decode tokens/s per layer, the HBM roofline of the dominant kernel (paged attention,
+timed live with events on the launch stream) and the CPU restatement of the same path timed on the host
+cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def run_step(case):
+    """One decode step through every layer of the case (1 layer except the 8-layer long-context config)."""
+    h = case["x"]
+    for layer, (kc, vc) in zip(case["layers"], case["caches"]):
+        h = layer(h, kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    return h
+
+
+def time_events(fn, iters, torch):
+    """Average duration (ms) of fn() bracketed by events on the current stream, one pair per call."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    for i in range(iters):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    ts = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
+def kernel_breakdown(case, torch, ops, iters):
+    """Per-op average microseconds for the first layer (each op timed alone, inputs resident)."""
+    layer = case["layers"][0]
+    kc, vc = case["caches"][0]
+    x = case["x"]
+    nq, nkv = layer.n_head * layer.head_dim, layer.n_kv_head * layer.head_dim
+    n1 = ops.rms_norm(x, layer.attn_norm, layer.eps)
+    qkv = layer._linear(n1, "qkv")
+    q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+    attn = ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], layer.n_head, layer.n_kv_head,
+                               layer.scale_value)
+    h = layer._linear(attn, "wo", residual=x)
+    n2 = ops.rms_norm(h, layer.ffn_norm, layer.eps)
+    gu = layer._linear(n2, "fc1")
+    a = ops.silu_mul(gu)
+    steps = {
+        "rmsnorm": lambda: ops.rms_norm(x, layer.attn_norm, layer.eps),
+        "qkv_gemm": lambda: layer._linear(n1, "qkv"),
+        "rope_and_cache": lambda: ops.rope_and_cache(q, k, v, case["cos"], case["sin"], kc, vc, case["slot_mapping"],
+                                                     layer.n_head),
+        "paged_attention": lambda: ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"],
+                                                       layer.n_head, layer.n_kv_head, layer.scale_value),
+        "wo_gemm": lambda: layer._linear(attn, "wo", residual=x),
+        "fc1_gemm": lambda: layer._linear(n2, "fc1"),
+        "silu_mul": lambda: ops.silu_mul(gu),
+        "fc2_gemm": lambda: layer._linear(a, "fc2", residual=h),
+    }
+    out = {}
+    for name, fn in steps.items():
+        for _ in range(3):
+            fn()
+        avg, med = time_events(fn, iters, torch)
+        out[name] = round(avg * 1e3, 2)
+    return out
+
+
+def cpu_baseline(case, torch, sample_seqs, gpu_out):
+    """Time the numpy restatement of the same layer on the host for ``sample_seqs`` sequences of the batch
+    (compact copies of their KV blocks), and compare the GPU rows with it."""
+    import oracle as O
+    cfg = case["cfg"]
+    layer = case["layers"][0]
+    kc, vc = case["caches"][0]
+    bs = cfg["block_size"]
+    idx = list(range(min(sample_seqs, cfg["batch"])))
+    tables = case["block_tables"][idx].cpu().numpy()
+    lens = case["context_lens_host"][idx]
+    used = np.unique(tables[tables >= 0])
+    remap = -np.ones(case["num_blocks"], dtype=np.int64)
+    remap[used] = np.arange(len(used))
+    t2 = np.where(tables >= 0, remap[np.maximum(tables, 0)], -1).astype(np.int32)
+    sel = torch.from_numpy(used).to(kc.device)
+    kcn = kc[sel].float().cpu().numpy()
+    vcn = vc[sel].float().cpu().numpy()
+    slots = case["slot_mapping"][idx].cpu().numpy()
+    slots2 = (remap[slots // bs] * bs + slots % bs).astype(np.int32)
+    p = {}
+    for n in layer.NAMES:
+        p[n + "_w"] = getattr(layer, n + "_w").cpu().numpy()
+        p[n + "_s"] = getattr(layer, n + "_s").cpu().numpy()
+    p["attn_norm"] = layer.attn_norm.cpu().numpy()
+    p["ffn_norm"] = layer.ffn_norm.cpu().numpy()
+    x = case["x"][idx].float().cpu().numpy()
+    cos = case["cos"][idx].float().cpu().numpy()
+    sin = case["sin"][idx].float().cpu().numpy()
+    ocfg = dict(n_head=cfg["n_head"], n_kv_head=cfg["n_kv_head"], head_dim=cfg["head_dim"], eps=1e-5)
+    act = "bf16" if cfg["dtype"] == torch.bfloat16 else "fp16"
+    fn = O.decode_layer_w8a8 if cfg["act_quant"] else O.decode_layer_w8a16
+    if cfg["act_quant"]:
+        for n in layer.NAMES:
+            p[n + "_smooth"] = getattr(layer, n + "_smooth").cpu().numpy()
+    try:
+        from threadpoolctl import threadpool_info
+        cores = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+    except Exception:
+        cores = 1
+    t0 = time.perf_counter()
+    ref = fn(x, p, ocfg, kcn, vcn, t2, lens, slots2, cos, sin, act_dtype=act)
+    dt = time.perf_counter() - t0
+    got = gpu_out[idx].float().cpu().numpy()
+    err = float(np.abs(got - ref).max())
+    scale = float(np.abs(ref).max())
+    return dict(value=len(idx) / dt, unit="tokens/s", cores=int(cores), kind="port",
+                sample=f"one layer step for {len(idx)} of the {cfg['batch']} sequences "
+                       f"({int(lens.sum())} context tokens), numpy float64, {dt:.1f} s"), dict(
+        max_abs_err=err, ref_max_abs=scale, rows=len(idx))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="llama3_8b_w8a16")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
+    ap.add_argument("--kernel-iters", type=int, default=50)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the decode path has no "
+              "collectives and no multi-GPU figure is produced.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from mindformers_amd import _lib, ops, synthetic
+    _lib.load()                                    # fail loudly if the HIP library is not built
+    torch.cuda.set_device(0)
+
+    t0 = time.perf_counter()
+    case = synthetic.make_decode_case(args.workload, seed=1)
+    cfg = case["cfg"]
+    nbytes = synthetic.algorithmic_bytes(case)
+    torch.cuda.synchronize()
+    log(f"[bench] built {args.workload}: batch {cfg['batch']}, sum(ctx) {int(case['context_lens_host'].sum())}, "
+        f"weights {nbytes['weights'] / 1e6:.1f} MB, KV {nbytes['kv'] / 1e6:.1f} MB per layer ({time.perf_counter() - t0:.1f} s)")
+
+    out_eager = run_step(case)
+    torch.cuda.synchronize()
+
+    use_graph = not args.no_graph
+    graph = None
+    if use_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    run_step(case)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out_graph = run_step(case)
+            # replays must reproduce the eager result bit for bit, with eager work in between
+            for _ in range(3):
+                graph.replay()
+                torch.cuda.synchronize()
+                if not torch.equal(out_graph, out_eager):
+                    raise RuntimeError("graph replay differs from the eager result")
+                run_step(case)
+                torch.cuda.synchronize()
+        except Exception as e:                     # fall back to eager launches, say so
+            log(f"[bench] HIP graph capture unavailable ({e}); timing eager launches")
+            graph = None
+    step = graph.replay if graph is not None else (lambda: run_step(case))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    n_layers = cfg["layers"]
+    tokens_per_s_layer = cfg["batch"] * n_layers * args.steps / elapsed
+
+    # dominant kernel: paged attention, event-timed on the launch stream
+    layer = case["layers"][0]
+    kc, vc = case["caches"][0]
+    nq = layer.n_head * layer.head_dim
+    qkv = layer._linear(ops.rms_norm(case["x"], layer.attn_norm, layer.eps), "qkv")
+    q = qkv[:, :nq]
+
+    def attn():
+        return ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], layer.n_head,
+                                   layer.n_kv_head, layer.scale_value)
+    for _ in range(5):
+        attn()
+    attn_ms, attn_med = time_events(attn, args.kernel_iters, torch)
+    achieved = nbytes["kv"] / (attn_ms * 1e-3) / 1e9
+    roofline = dict(bound="hbm", kernel="paged_attention_kernel (+ partition reduce)", achieved=round(achieved, 1),
+                    peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                    bytes_per_launch=nbytes["kv"], avg_launch_us=round(attn_ms * 1e3, 2))
+    breakdown = kernel_breakdown(case, torch, ops, args.kernel_iters)
+    layer_gbps = nbytes["total"] * n_layers / (ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "decode tokens/sec per layer (Llama3-8B shape, W8A16, bs64); % of peak HBM GB/s",
+        "value": round(tokens_per_s_layer, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if cfg["dtype"] == torch.bfloat16 else "fp16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: one decode layer step, batch {cfg['batch']}, hidden {cfg['hidden']}, "
+                               f"{cfg['n_head']}q/{cfg['n_kv_head']}kv heads x {cfg['head_dim']}, ffn {cfg['ffn']}, "
+                               f"ctx U[{cfg['ctx'][0]},{cfg['ctx'][1]}], block {cfg['block_size']}, "
+                               f"{'W8A8' if cfg['act_quant'] else 'W8A16'}, layers {n_layers}",
+                   "launch": "hip_graph" if graph is not None else "eager",
+                   "algorithmic_bytes_per_layer": nbytes["total"]},
+        "layer_hbm_gbps": round(layer_gbps, 1), "layer_hbm_frac": round(layer_gbps / HBM_PEAK_GBPS, 4),
+        "roofline": roofline, "breakdown_us": breakdown,
+    }
+    if not args.no_cpu:
+        cb, parity = cpu_baseline(case, torch, args.cpu_seqs, out_eager)
+        result["cpu_baseline"] = cb
+        result["parity_vs_cpu"] = parity
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -36,26 +36,30 @@ const char* mf_last_error(void);
  *   mindformers/parallel_core/inference/transformer/flash_attention.py:94,126-127
  * cache.view(num_slots, n_kv_heads*head_dim)[slot_mapping[i]] = x[i] for key and value; slot < 0 skips the
  * row (padding, mindformers/modules/block_tables.py:79-95).  value / value_cache may both be NULL (the MLA
- * call writes one latent cache, multi_latent_attention.py:401-402).  Pure copy: bit-exact. */
+ * call writes one latent cache, multi_latent_attention.py:401-402).  Pure copy: bit-exact.
+ * key_row_stride / value_row_stride: elements between consecutive token rows of key / value (0 = dense,
+ * n_kv_heads*head_dim); lets key and value be column slices of one fused [T, q|k|v] projection output. */
 int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
                          const int32_t* slot_mapping, int num_tokens, int n_kv_heads, int head_dim,
-                         int64_t num_slots, int dtype, void* stream);
+                         int64_t num_slots, int64_t key_row_stride, int64_t value_row_stride, int dtype,
+                         void* stream);
 
 /* ops.ApplyRotaryPosEmb(cos_format=2)(query, key, cos, sin, batch_valid_length)
  *   mindformers/modules/infer_attention.py:50-57
  *   mindformers/parallel_core/inference/base_models/common/embeddings/rotary_pos_embedding.py:75,146
  * In place, rotate-half pairing (i, i + head_dim/2): x = x*cos + rotate_half(x)*sin in fp32, rounded once.
  * cos/sin are [num_tokens, head_dim] rows already gathered per token (table_dtype: MF_BF16/MF_FP16/MF_FP32).
- * key may be NULL. */
+ * key may be NULL.  q_row_stride / k_row_stride: elements between token rows (0 = dense). */
 int mf_rope_half(void* query, void* key, const void* cos, const void* sin, int num_tokens, int n_heads,
-                 int n_kv_heads, int head_dim, int dtype, int table_dtype, void* stream);
+                 int n_kv_heads, int head_dim, int64_t q_row_stride, int64_t k_row_stride, int dtype,
+                 int table_dtype, void* stream);
 
 /* RoPE on q and k followed by the cache scatter of rotated k and of v, one launch (the sequence
  * infer_attention.py:445,453 performs).  q and k are rotated in place. */
 int mf_rope_and_cache(void* query, void* key, const void* value, const void* cos, const void* sin,
                       void* key_cache, void* value_cache, const int32_t* slot_mapping, int num_tokens,
-                      int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int dtype,
-                      int table_dtype, void* stream);
+                      int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int64_t q_row_stride,
+                      int64_t k_row_stride, int64_t v_row_stride, int dtype, int table_dtype, void* stream);
 
 /* ---- paged attention (decode) --------------------------------------------------------------------- */
 
@@ -69,12 +73,13 @@ size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, 
  * out[b,h,:] = softmax(scale * q[b,h,:] . K_b[:L_b]^T) V_b[:L_b]; token j of sequence b lives at
  * cache[block_tables[b, j / block_size], j % block_size, h / (n_heads/n_kv_heads), :]; L_b = context_lens[b]
  * counts the token written by this step.  L_b <= 0 gives zeros.  Scores and softmax in fp32; the
- * probabilities are rounded to `dtype` before the PV product.  head_dim in {32, 64, 128}. */
+ * probabilities are rounded to `dtype` before the PV product.  head_dim in {32, 64, 128}.
+ * q_row_stride: elements between the query rows of consecutive sequences (0 = dense); out is dense. */
 int mf_paged_attention_decode(void* out, const void* query, const void* key_cache, const void* value_cache,
                               const int32_t* block_tables, const int32_t* context_lens, int batch,
                               int n_heads, int n_kv_heads, int head_dim, int block_size,
-                              int max_blocks_per_seq, int num_blocks, float scale, int dtype,
-                              void* workspace, size_t workspace_bytes, void* stream);
+                              int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                              int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- norm / activation ---------------------------------------------------------------------------- */
 
@@ -104,7 +109,7 @@ size_t mf_w8a16_workspace_bytes(int m, int n, int k);
  * (swapped in by Quantizer.preprocess_model, mindformers/modules/quantizers/rtn_quantizer.py:61-67).
  * y[m,n] = (sum_k x[m,k] * w[n,k]) * scale[n] (+ bias[n]) (+ residual[m,n]); x/y/bias/residual in `dtype`,
  * w int8 [N,K] row-major, scale float32 [N]; products exact, fp32 accumulation, scale applied to the sum.
- * With residual: y = round(round(acc*scale+bias) + residual).  K % 64 == 0. */
+ * With residual: y = round(round(acc*scale+bias) + residual).  K % 16 == 0. */
 int mf_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const void* bias,
                   const void* residual, int m, int n, int k, int dtype, void* workspace,
                   size_t workspace_bytes, void* stream);
@@ -117,7 +122,8 @@ int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const 
 
 /* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
  * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
- * If acc_out != NULL the raw int32 accumulators are also written ([M,N] row-major).  K % 64 == 0. */
+ * If acc_out != NULL the raw int32 accumulators are also written ([M,N] row-major); y may then be NULL.
+ * K % 16 == 0. */
 int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const int8_t* w,
                  const float* w_scale, const void* bias, const void* residual, int m, int n, int k, int dtype,
                  void* stream);

@@ -19,11 +19,11 @@ _P, _I, _L, _F, _Z = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float, _c.c_size_t
 SIGNATURES = {
     "mf_version": (_c.c_char_p, []),
     "mf_last_error": (_c.c_char_p, []),
-    "mf_reshape_and_cache": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _P]),
-    "mf_rope_half": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
-    "mf_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _P]),
+    "mf_reshape_and_cache": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _P]),
+    "mf_rope_half": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _I, _I, _P]),
+    "mf_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _I, _I, _P]),
     "mf_paged_attention_workspace_bytes": (_Z, [_I, _I, _I, _I]),
-    "mf_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _Z, _P]),
+    "mf_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P, _Z, _P]),
     "mf_rmsnorm": (_I, [_P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P]),
     "mf_silu_mul": (_I, [_P, _P, _I, _I, _I, _I, _P]),
     "mf_add": (_I, [_P, _P, _P, _L, _I, _P]),

@@ -192,6 +192,7 @@ extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* res
                           float eps, int rows, int cols, int dtype, int gamma_dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rmsnorm: dtype must be bf16 or fp16");
     MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32, "rmsnorm: bad gamma dtype");
+    if (rows <= 0) return 0;
     MF_REQUIRE(y && x && gamma, "rmsnorm: null argument");
     MF_REQUIRE(!residual || sum_out, "rmsnorm: residual given without sum_out");
     MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * ROW_MAX_VEC * 8,
@@ -213,6 +214,7 @@ extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* res
 extern "C" int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, int layout, int dtype,
                            void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "silu_mul: dtype must be bf16 or fp16");
+    if (rows <= 0) return 0;
     MF_REQUIRE(out && gate_up, "silu_mul: null argument");
     MF_REQUIRE(layout == 0 || layout == 1, "silu_mul: layout must be 0 (halves) or 1 (interleaved)");
     MF_REQUIRE(cols > 0 && cols % 8 == 0, "silu_mul: cols (%d) must be a multiple of 8", cols);
@@ -231,6 +233,7 @@ extern "C" int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, i
 
 extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "add: dtype must be bf16 or fp16");
+    if (n <= 0) return 0;
     MF_REQUIRE(out && a && b, "add: null argument");
     MF_REQUIRE((((uintptr_t)out | (uintptr_t)a | (uintptr_t)b) & 15) == 0, "add: pointers must be 16-byte aligned");
     if (n <= 0) return 0;
@@ -247,6 +250,7 @@ extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dt
 extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m,
                                           int k, int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant: dtype must be bf16 or fp16");
+    if (m <= 0) return 0;
     MF_REQUIRE(xq && x_scale && x, "dynamic_quant: null argument");
     MF_REQUIRE(k > 0 && k % 8 == 0 && k <= ROW_THREADS * 12 * 8, "dynamic_quant: k (%d) must be a multiple of 8, <= %d",
                k, ROW_THREADS * 12 * 8);

@@ -11,11 +11,12 @@ template <int VEC_BYTES>
 __global__ void reshape_and_cache_kernel(const uint8_t* __restrict__ key, const uint8_t* __restrict__ value,
                                          uint8_t* __restrict__ key_cache, uint8_t* __restrict__ value_cache,
                                          const int32_t* __restrict__ slot_mapping, int row_bytes,
-                                         int64_t num_slots) {
+                                         int64_t num_slots, int64_t key_stride_bytes,
+                                         int64_t value_stride_bytes) {
     const int t = blockIdx.x;
     const int64_t slot = slot_mapping[t];
     if (slot < 0 || slot >= num_slots) return;  // padding (or a corrupt slot: never write out of bounds)
-    const uint8_t* src = (blockIdx.y == 0 ? key : value) + (int64_t)t * row_bytes;
+    const uint8_t* src = blockIdx.y == 0 ? key + (int64_t)t * key_stride_bytes : value + (int64_t)t * value_stride_bytes;
     uint8_t* dst = (blockIdx.y == 0 ? key_cache : value_cache) + slot * (int64_t)row_bytes;
     if (VEC_BYTES == 16) {
         for (int i = threadIdx.x * 16; i < row_bytes; i += blockDim.x * 16)
@@ -52,11 +53,12 @@ __device__ __forceinline__ void rope_row(uint16_t* x, int n_heads, int D, const 
 
 template <typename T>
 __global__ void rope_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, const void* __restrict__ cos,
-                            const void* __restrict__ sin, int n_heads, int n_kv, int D, int table_dtype) {
+                            const void* __restrict__ sin, int n_heads, int n_kv, int D, int table_dtype,
+                            int64_t q_stride, int64_t k_stride) {
     const int t = blockIdx.x;
     const int64_t trow = (int64_t)t * D;
-    rope_row<T>(q + (int64_t)t * n_heads * D, n_heads, D, cos, sin, trow, table_dtype, nullptr);
-    if (k) rope_row<T>(k + (int64_t)t * n_kv * D, n_kv, D, cos, sin, trow, table_dtype, nullptr);
+    rope_row<T>(q + (int64_t)t * q_stride, n_heads, D, cos, sin, trow, table_dtype, nullptr);
+    if (k) rope_row<T>(k + (int64_t)t * k_stride, n_kv, D, cos, sin, trow, table_dtype, nullptr);
 }
 
 template <typename T>
@@ -65,19 +67,20 @@ __global__ void rope_and_cache_kernel(uint16_t* __restrict__ q, uint16_t* __rest
                                       const void* __restrict__ sin, uint16_t* __restrict__ key_cache,
                                       uint16_t* __restrict__ value_cache,
                                       const int32_t* __restrict__ slot_mapping, int n_heads, int n_kv, int D,
-                                      int64_t num_slots, int table_dtype) {
+                                      int64_t num_slots, int table_dtype, int64_t q_stride, int64_t k_stride,
+                                      int64_t v_stride, int vec_ok) {
     const int t = blockIdx.x;
     const int64_t trow = (int64_t)t * D;
     const int64_t slot = slot_mapping[t];
     const bool live = slot >= 0 && slot < num_slots;
     const int row = n_kv * D;
-    rope_row<T>(q + (int64_t)t * n_heads * D, n_heads, D, cos, sin, trow, table_dtype, nullptr);
-    rope_row<T>(k + (int64_t)t * row, n_kv, D, cos, sin, trow, table_dtype,
+    rope_row<T>(q + (int64_t)t * q_stride, n_heads, D, cos, sin, trow, table_dtype, nullptr);
+    rope_row<T>(k + (int64_t)t * k_stride, n_kv, D, cos, sin, trow, table_dtype,
                 live ? key_cache + slot * row : nullptr);
     if (live) {
-        const uint16_t* src = v + (int64_t)t * row;
+        const uint16_t* src = v + (int64_t)t * v_stride;
         uint16_t* dst = value_cache + slot * row;
-        if ((row & 7) == 0) {
+        if (vec_ok) {
             for (int i = threadIdx.x * 8; i < row; i += blockDim.x * 8)
                 *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
         } else {
@@ -90,65 +93,86 @@ __global__ void rope_and_cache_kernel(uint16_t* __restrict__ q, uint16_t* __rest
 
 extern "C" int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
                                     const int32_t* slot_mapping, int num_tokens, int n_kv_heads, int head_dim,
-                                    int64_t num_slots, int dtype, void* stream) {
+                                    int64_t num_slots, int64_t key_row_stride, int64_t value_row_stride, int dtype,
+                                    void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "reshape_and_cache: dtype must be bf16 or fp16");
+    if (num_tokens == 0) return 0;                          // empty step: nothing to check or launch
     MF_REQUIRE(key && key_cache && slot_mapping, "reshape_and_cache: null key / key_cache / slot_mapping");
     MF_REQUIRE((value == nullptr) == (value_cache == nullptr),
                "reshape_and_cache: value and value_cache must both be given or both be null");
-    MF_REQUIRE(num_tokens >= 0 && n_kv_heads > 0 && head_dim > 0 && num_slots > 0, "reshape_and_cache: bad sizes");
-    if (num_tokens == 0) return 0;
+    MF_REQUIRE(num_tokens > 0 && n_kv_heads > 0 && head_dim > 0 && num_slots > 0, "reshape_and_cache: bad sizes");
     const int row_bytes = n_kv_heads * head_dim * 2;
-    const bool vec = (row_bytes % 16 == 0) && (((uintptr_t)key | (uintptr_t)key_cache | (uintptr_t)value |
-                                                 (uintptr_t)value_cache) % 16 == 0);
+    if (key_row_stride <= 0) key_row_stride = (int64_t)n_kv_heads * head_dim;
+    if (value_row_stride <= 0) value_row_stride = (int64_t)n_kv_heads * head_dim;
+    MF_REQUIRE(key_row_stride >= (int64_t)n_kv_heads * head_dim && value_row_stride >= (int64_t)n_kv_heads * head_dim,
+               "reshape_and_cache: row stride smaller than a row");
+    const bool vec = (row_bytes % 16 == 0) && (key_row_stride % 8 == 0) && (value_row_stride % 8 == 0) &&
+                     (((uintptr_t)key | (uintptr_t)key_cache | (uintptr_t)value | (uintptr_t)value_cache) % 16 == 0);
     dim3 grid(num_tokens, value ? 2 : 1);
     const int threads = vec ? min(256, max(64, row_bytes / 16)) : 256;
     if (vec)
         hipLaunchKernelGGL(reshape_and_cache_kernel<16>, grid, dim3(threads), 0, (hipStream_t)stream,
                            (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)key_cache, (uint8_t*)value_cache,
-                           slot_mapping, row_bytes, num_slots);
+                           slot_mapping, row_bytes, num_slots, key_row_stride * 2, value_row_stride * 2);
     else
         hipLaunchKernelGGL(reshape_and_cache_kernel<2>, grid, dim3(threads), 0, (hipStream_t)stream,
                            (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)key_cache, (uint8_t*)value_cache,
-                           slot_mapping, row_bytes, num_slots);
+                           slot_mapping, row_bytes, num_slots, key_row_stride * 2, value_row_stride * 2);
     return MF_LAUNCH_CHECK();
 }
 
 extern "C" int mf_rope_half(void* query, void* key, const void* cos, const void* sin, int num_tokens,
-                            int n_heads, int n_kv_heads, int head_dim, int dtype, int table_dtype, void* stream) {
+                            int n_heads, int n_kv_heads, int head_dim, int64_t q_row_stride, int64_t k_row_stride,
+                            int dtype, int table_dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rope: dtype must be bf16 or fp16");
     MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32, "rope: bad table dtype");
+    if (num_tokens == 0) return 0;
     MF_REQUIRE(query && cos && sin, "rope: null query / cos / sin");
     MF_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope: head_dim must be even");
-    if (num_tokens == 0) return 0;
+    if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * head_dim;
+    if (k_row_stride <= 0) k_row_stride = (int64_t)n_kv_heads * head_dim;
+    MF_REQUIRE(q_row_stride >= (int64_t)n_heads * head_dim && k_row_stride >= (int64_t)n_kv_heads * head_dim,
+               "rope: row stride smaller than a row");
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(rope_kernel<BF16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)query,
-                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype);
+                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype, q_row_stride,
+                           k_row_stride);
     else
         hipLaunchKernelGGL(rope_kernel<FP16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)query,
-                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype);
+                           (uint16_t*)key, cos, sin, n_heads, n_kv_heads, head_dim, table_dtype, q_row_stride,
+                           k_row_stride);
     return MF_LAUNCH_CHECK();
 }
 
 extern "C" int mf_rope_and_cache(void* query, void* key, const void* value, const void* cos, const void* sin,
                                  void* key_cache, void* value_cache, const int32_t* slot_mapping, int num_tokens,
-                                 int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int dtype,
-                                 int table_dtype, void* stream) {
+                                 int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int64_t q_row_stride,
+                                 int64_t k_row_stride, int64_t v_row_stride, int dtype, int table_dtype,
+                                 void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rope_and_cache: dtype must be bf16 or fp16");
     MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
                "rope_and_cache: bad table dtype");
+    if (num_tokens == 0) return 0;
     MF_REQUIRE(query && key && value && cos && sin && key_cache && value_cache && slot_mapping,
                "rope_and_cache: null argument");
     MF_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && num_slots > 0, "rope_and_cache: bad sizes");
-    if (num_tokens == 0) return 0;
+    const int64_t kv_row = (int64_t)n_kv_heads * head_dim;
+    if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * head_dim;
+    if (k_row_stride <= 0) k_row_stride = kv_row;
+    if (v_row_stride <= 0) v_row_stride = kv_row;
+    MF_REQUIRE(q_row_stride >= (int64_t)n_heads * head_dim && k_row_stride >= kv_row && v_row_stride >= kv_row,
+               "rope_and_cache: row stride smaller than a row");
+    const int vec_ok = (kv_row % 8 == 0) && (v_row_stride % 8 == 0) &&
+                       (((uintptr_t)value | (uintptr_t)value_cache) % 16 == 0);
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(rope_and_cache_kernel<BF16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream,
                            (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin, (uint16_t*)key_cache,
                            (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, num_slots,
-                           table_dtype);
+                           table_dtype, q_row_stride, k_row_stride, v_row_stride, vec_ok);
     else
         hipLaunchKernelGGL(rope_and_cache_kernel<FP16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream,
                            (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin, (uint16_t*)key_cache,
                            (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, num_slots,
-                           table_dtype);
+                           table_dtype, q_row_stride, k_row_stride, v_row_stride, vec_ok);
     return MF_LAUNCH_CHECK();
 }

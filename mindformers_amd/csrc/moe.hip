@@ -205,6 +205,7 @@ extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* 
                             int tokens, int n_experts, int k, int n_group, int topk_group, float scale, int renorm,
                             int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_route: dtype must be bf16 or fp16");
+    if (tokens <= 0) return 0;
     MF_REQUIRE(weights_out && index_out && logits, "moe_route: null argument");
     MF_REQUIRE(n_experts > 0 && n_experts <= RT_MAX_E, "moe_route: n_experts (%d) must be in 1..%d", n_experts, RT_MAX_E);
     MF_REQUIRE(k > 0 && k <= RT_MAX_K && k <= n_experts, "moe_route: k (%d) must be in 1..min(%d, n_experts)", k, RT_MAX_K);
@@ -245,6 +246,7 @@ extern "C" int mf_moe_permute(void* permuted_x, int32_t* row_map, int64_t* count
 extern "C" int mf_moe_unpermute(void* out, const void* y, const int32_t* row_map, const void* probs,
                                 const void* shared, int tokens, int k, int hidden, int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_unpermute: dtype must be bf16 or fp16");
+    if (tokens <= 0) return 0;
     MF_REQUIRE(out && y && row_map && probs, "moe_unpermute: null argument");
     MF_REQUIRE(k > 0 && hidden > 0 && hidden % 8 == 0, "moe_unpermute: hidden (%d) must be a multiple of 8", hidden);
     MF_REQUIRE((((uintptr_t)out | (uintptr_t)y | (uintptr_t)shared) & 15) == 0,

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
     int n_rep, int head_groups, int block_size, int max_blocks, int num_blocks, int max_parts,
-    float scale_log2) {
+    float scale_log2, int64_t q_stride) {
     using vec8 = typename T::vec8;
     constexpr int KS = D / 32;
     constexpr int VSTRIDE = PaSmem<D>::VSTRIDE;
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
     const int head = kvh * n_rep + (head_ok ? hh : 0);
     vec8 qreg[KS];
     {
-        const uint16_t* qp = q + ((int64_t)b * n_heads + head) * D + 8 * g;
+        const uint16_t* qp = q + (int64_t)b * q_stride + (int64_t)head * D + 8 * g;
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             u32x4 v = {0u, 0u, 0u, 0u};
@@ -276,7 +276,8 @@ __global__ void paged_attention_reduce_kernel(uint16_t* __restrict__ out, const 
 template <typename T, int D>
 int launch_pa(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads, int n_kv,
-              int block_size, int max_blocks, int num_blocks, float scale, void* workspace, hipStream_t st) {
+              int block_size, int max_blocks, int num_blocks, float scale, int64_t q_stride, void* workspace,
+              hipStream_t st) {
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
@@ -288,7 +289,7 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     hipLaunchKernelGGL((paged_attention_kernel<T, D>), grid, dim3(PA_WAVES * 64), 0, st, (uint16_t*)out, part_out,
                        part_ml, (const uint16_t*)query, (const uint16_t*)key_cache, (const uint16_t*)value_cache,
                        block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, block_size, max_blocks,
-                       num_blocks, max_parts, scale_log2);
+                       num_blocks, max_parts, scale_log2, q_stride);
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (max_parts > 1) {
@@ -318,9 +319,11 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
                                          const void* value_cache, const int32_t* block_tables,
                                          const int32_t* context_lens, int batch, int n_heads, int n_kv_heads,
                                          int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
-                                         float scale, int dtype, void* workspace, size_t workspace_bytes,
+                                         float scale, int64_t q_row_stride, int dtype, void* workspace,
+                                         size_t workspace_bytes,
                                          void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention: dtype must be bf16 or fp16");
+    if (batch == 0) return 0;
     MF_REQUIRE(out && query && key_cache && value_cache && block_tables && context_lens,
                "paged_attention: null argument");
     MF_REQUIRE(batch >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
@@ -328,6 +331,9 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
     MF_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 128,
                "paged_attention: head_dim %d not supported (32, 64, 128)", head_dim);
     MF_REQUIRE(block_size > 0 && max_blocks_per_seq > 0 && num_blocks > 0, "paged_attention: bad block geometry");
+    if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * head_dim;
+    MF_REQUIRE(q_row_stride >= (int64_t)n_heads * head_dim && q_row_stride % 8 == 0,
+               "paged_attention: query row stride must be >= n_heads*head_dim and a multiple of 8 elements");
     MF_REQUIRE((((uintptr_t)out | (uintptr_t)query | (uintptr_t)key_cache | (uintptr_t)value_cache) & 15) == 0,
                "paged_attention: out / query / caches must be 16-byte aligned");
     if (batch == 0) return 0;
@@ -345,7 +351,7 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
     void* ws = need ? workspace : nullptr;
 #define PA_CASE(TT, DD)                                                                                        \
     return launch_pa<TT, DD>(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,   \
-                             n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, ws, st)
+                             n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride, ws, st)
     if (dtype == MF_BF16) {
         if (head_dim == 32) PA_CASE(BF16, 32);
         if (head_dim == 64) PA_CASE(BF16, 64);

@@ -297,6 +297,7 @@ extern "C" int mf_w8a16_gemm(void* y, const void* x, const int8_t* w, const floa
                              const void* residual, int m, int n, int k, int dtype, void* workspace,
                              size_t workspace_bytes, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_gemm: dtype must be bf16 or fp16");
+    if (m == 0) return 0;
     MF_REQUIRE(y && x && w && scale, "w8a16_gemm: null argument");
     MF_REQUIRE(m >= 0 && n > 0 && k > 0, "w8a16_gemm: bad sizes m=%d n=%d k=%d", m, n, k);
     MF_REQUIRE(k % 16 == 0, "w8a16_gemm: K (%d) must be a multiple of 16", k);
@@ -314,6 +315,7 @@ extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const int8_t* w, co
                                      const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype,
                                      void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "grouped_w8a16_gemm: dtype must be bf16 or fp16");
+    if (total_rows == 0) return 0;
     MF_REQUIRE(y && x && w && scale && offsets, "grouped_w8a16_gemm: null argument");
     MF_REQUIRE(n_experts > 0 && n_experts <= 65535 && total_rows >= 0 && n > 0 && k > 0,
                "grouped_w8a16_gemm: bad sizes");

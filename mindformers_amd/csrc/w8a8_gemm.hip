@@ -124,6 +124,7 @@ extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const f
                             const float* w_scale, const void* bias, const void* residual, int m, int n, int k,
                             int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a8_gemm: dtype must be bf16 or fp16");
+    if (m == 0) return 0;
     MF_REQUIRE(xq && w && (y || acc_out), "w8a8_gemm: null argument");
     MF_REQUIRE(!y || (x_scale && w_scale), "w8a8_gemm: scales required for a dequantised output");
     MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 16 == 0, "w8a8_gemm: bad sizes m=%d n=%d k=%d (K %% 16 == 0)", m, n, k);

@@ -1,0 +1,75 @@
+"""One quantized decode layer wired from the kernels: the caller of the hot path.
+
+Mirrors the pre-norm residual layer of the reference (mindformers/models/llama/llama_transformer.py:1036-1070
+LLamaDecodeLayer.construct with the use_past branch of LLamaAttention.construct :467-569, and
+mindformers/parallel_core/inference/transformer/transformer_layer.py:296-355) with the fused projection
+layouts of the Megatron-style stack: linear_qkv rows are [q | k | v] (attention.py:344-349) and linear_fc1
+rows are [gate | hidden] (mlp.py:135-140).
+
+Launch sequence per decode step (one stream, no host synchronisation):
+  rmsnorm -> qkv GEMM -> rope+KV scatter -> paged attention (+ partition reduce) -> wo GEMM (+residual)
+  -> rmsnorm -> fc1 GEMM -> silu*mul -> fc2 GEMM (+residual)
+"""
+import math
+
+import torch
+from torch import nn
+
+from . import ops
+
+
+class QuantDecodeLayer(nn.Module):
+    """W8A16 (``act_quant=False``) or W8A8 per-token-dynamic (``act_quant=True``) decode layer.
+
+    Parameters are plain buffers: ``{qkv,wo,fc1,fc2}_w`` int8 [out, in], ``*_s`` fp32 [out], optional
+    ``*_b`` bias, optional ``*_smooth`` fp32 [in] (W8A8), ``attn_norm`` / ``ffn_norm`` gammas.
+    """
+
+    NAMES = ("qkv", "wo", "fc1", "fc2")
+
+    def __init__(self, hidden, n_head, n_kv_head, head_dim, ffn, eps=1e-5, dtype=torch.bfloat16, act_quant=False,
+                 qkv_bias=False, device="cuda"):
+        super().__init__()
+        self.hidden, self.n_head, self.n_kv_head, self.head_dim, self.ffn = hidden, n_head, n_kv_head, head_dim, ffn
+        self.eps, self.dtype, self.act_quant = eps, dtype, act_quant
+        self.scale_value = 1.0 / math.sqrt(head_dim)
+        shapes = {"qkv": ((n_head + 2 * n_kv_head) * head_dim, hidden), "wo": (hidden, n_head * head_dim),
+                  "fc1": (2 * ffn, hidden), "fc2": (hidden, ffn)}
+        for name, (n, k) in shapes.items():
+            self.register_buffer(f"{name}_w", torch.zeros(n, k, dtype=torch.int8, device=device))
+            self.register_buffer(f"{name}_s", torch.ones(n, dtype=torch.float32, device=device))
+            setattr(self, f"{name}_b", None)
+            if act_quant:
+                self.register_buffer(f"{name}_smooth", torch.ones(k, dtype=torch.float32, device=device))
+        if qkv_bias:
+            self.qkv_b = torch.zeros(shapes["qkv"][0], dtype=dtype, device=device)
+        self.register_buffer("attn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
+        self.register_buffer("ffn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
+
+    def _linear(self, x, name, residual=None):
+        w, s, b = getattr(self, f"{name}_w"), getattr(self, f"{name}_s"), getattr(self, f"{name}_b")
+        if self.act_quant:
+            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"))
+            return ops.w8a8_linear(xq, xs, w, s, self.dtype, bias=b, residual=residual)
+        return ops.w8a16_linear(x, w, s, bias=b, residual=residual)
+
+    def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin):
+        """x [T, hidden]; caches [num_blocks, block_size, n_kv, D]; cos/sin [T, D] rows for this step's
+        positions; batch_valid_length counts the token written by this step."""
+        nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
+        n1 = ops.rms_norm(x, self.attn_norm, self.eps)
+        qkv = self._linear(n1, "qkv")
+        q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+        ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
+        attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
+                                   self.n_kv_head, self.scale_value)
+        h = self._linear(attn, "wo", residual=x)
+        n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
+        gu = self._linear(n2, "fc1")
+        a = ops.silu_mul(gu)
+        return self._linear(a, "fc2", residual=h)
+
+    construct = forward
+
+    def weight_bytes(self):
+        return sum(getattr(self, f"{n}_w").numel() for n in self.NAMES)

@@ -1,0 +1,55 @@
+"""PagedAttentionMgr — same constructor, attributes and calls as the reference's
+mindformers/modules/paged_attention_mgr.py:26-92, on torch tensors and the gfx950 kernels.
+"""
+import math
+
+import torch
+from torch import nn
+
+from .. import ops
+
+
+class PagedAttentionMgr(nn.Module):
+    """Owns the key/value caches [num_blocks, block_size, n_kv_heads, head_dim] and runs
+    reshape_and_cache / paged_attention on them (paged_attention_mgr.py:29-58)."""
+
+    def __init__(self, n_heads, head_dim, n_kv_heads, kv_shape, seq_length=-1, compute_dtype=torch.float16,
+                 parallel_decoding=False, chunk_prefill=False, device="cuda"):
+        super().__init__()
+        if len(kv_shape) != 4:
+            raise ValueError(f"kv_shape must be (num_blocks, block_size, n_kv_heads, head_dim), got {kv_shape}")
+        if kv_shape[2] != n_kv_heads or kv_shape[3] != head_dim:
+            raise ValueError(f"kv_shape {kv_shape} does not match n_kv_heads={n_kv_heads}, head_dim={head_dim}")
+        if parallel_decoding or chunk_prefill:
+            raise NotImplementedError("parallel_decoding / chunk_prefill (masked multi-token PagedAttention) is not built")
+        self.n_heads = n_heads
+        self.head_dim = head_dim
+        self.n_kv_heads = n_kv_heads
+        self.seq_length = seq_length
+        self.is_first_iteration = True
+        self.scale_value = 1 / math.sqrt(self.head_dim)
+        self.register_buffer("key_cache", torch.zeros(kv_shape, dtype=compute_dtype, device=device), persistent=False)
+        self.register_buffer("value_cache", torch.zeros(kv_shape, dtype=compute_dtype, device=device), persistent=False)
+        self.parallel_decoding = parallel_decoding
+        self.chunk_prefill = chunk_prefill
+
+    def forward(self, key, value, slot_mapping, batch_valid_length=None):
+        """The forward compute of KVCache for Paged Attention (paged_attention_mgr.py:60-62)."""
+        return ops.reshape_and_cache(key, value, self.key_cache, self.value_cache, slot_mapping)
+
+    construct = forward
+
+    def paged_attn(self, query, batch_valid_length, block_tables, attn_mask=None, q_seq_lens=None):
+        """The forward compute of Paged Attention (paged_attention_mgr.py:64-70)."""
+        shape = query.shape
+        out = ops.paged_attention(query.reshape(-1, self.n_heads * self.head_dim), self.key_cache, self.value_cache,
+                                  block_tables, batch_valid_length, self.n_heads, self.n_kv_heads, self.scale_value)
+        return out.reshape(shape)
+
+    def paged_attn_with_alibi(self, query, batch_valid_length, block_tables, alibi_tensor):
+        """paged_attention_mgr.py:72-75 — no alibi model is on the built path."""
+        raise NotImplementedError("PagedAttentionMask (alibi) is not built")
+
+    def shard(self, parallel_config):
+        """One GPU: nothing to shard (paged_attention_mgr.py:77-92 only sets layouts)."""
+        return self

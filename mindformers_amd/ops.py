@@ -32,6 +32,29 @@ def _dev_ok(*tensors):
     return dev
 
 
+def _rows(t, width, what):
+    """A [rows, width] view of ``t`` for the kernels: returns (tensor, row_stride_in_elements).  Accepts any
+    contiguous tensor whose element count is a multiple of width, or a 2-D tensor with unit column stride (a
+    column slice of a wider buffer, e.g. q/k/v inside a fused projection output)."""
+    if t.is_contiguous():
+        _need(t.numel() % width == 0, f"{what}: {t.numel()} elements is not a multiple of the row width {width}")
+        return t, width
+    _need(t.dim() == 2 and t.stride(1) == 1 and t.shape[1] == width and t.stride(0) >= width,
+          f"{what}: must be contiguous or a [rows, {width}] column slice with unit column stride")
+    return t, t.stride(0)
+
+
+def _dev_of(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _need(isinstance(t, torch.Tensor) and t.is_cuda, "all tensors must live on the GPU")
+        dev = dev or t.device
+        _need(t.device == dev, "all tensors must be on the same device")
+    return dev
+
+
 def workspace(nbytes, device, tag="default"):
     """A cached per-device scratch buffer (grown on demand, never shrunk)."""
     key = (device, tag)
@@ -47,9 +70,14 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
     """ReshapeAndCache(key, value, key_cache, value_cache, slot_mapping) -> key.
     key/value [T, n_kv*D] (any leading shape with T rows); caches [num_blocks, block_size, n_kv, D]."""
     lib = _lib.load()
-    dev = _dev_ok(key, value, key_cache, value_cache, slot_mapping)
+    _dev_of(key, value)
+    dev = _dev_ok(key_cache, value_cache, slot_mapping)
     _need(key_cache.dim() == 4, "key_cache must be [num_blocks, block_size, n_kv_heads, head_dim]")
     nb, bs, n_kv, d = key_cache.shape
+    key, ks = _rows(key, n_kv * d, "key")
+    vs = 0
+    if value is not None:
+        value, vs = _rows(value, n_kv * d, "value")
     _need(key.dtype in _ACT and key_cache.dtype == key.dtype, "key and key_cache must share a bf16/fp16 dtype")
     _need(slot_mapping.dtype == torch.int32 and slot_mapping.dim() == 1, "slot_mapping must be int32 [T]")
     t = slot_mapping.numel()
@@ -60,7 +88,7 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
     else:
         _need(value_cache is None, "value_cache given without value")
     check(lib.mf_reshape_and_cache(ptr(key), ptr(value), ptr(key_cache), ptr(value_cache), ptr(slot_mapping), t, n_kv,
-                                   d, nb * bs, dtype_code(key.dtype), stream_ptr(dev)), "mf_reshape_and_cache")
+                                   d, nb * bs, ks, vs, dtype_code(key.dtype), stream_ptr(dev)), "mf_reshape_and_cache")
     return key
 
 
@@ -68,13 +96,18 @@ def apply_rotary_pos_emb(query, key, cos, sin, n_heads, n_kv_heads, head_dim):
     """ApplyRotaryPosEmb(cos_format=2), in place.  query [T, n_heads*D], key [T, n_kv*D] or None,
     cos/sin [T, D] (one row per token)."""
     lib = _lib.load()
-    dev = _dev_ok(query, key, cos, sin)
+    _dev_of(query, key)
+    dev = _dev_ok(cos, sin)
+    query, qs = _rows(query, n_heads * head_dim, "query")
+    ks = 0
+    if key is not None:
+        key, ks = _rows(key, n_kv_heads * head_dim, "key")
     t = query.numel() // (n_heads * head_dim)
     _need(query.dtype in _ACT and query.numel() == t * n_heads * head_dim, "query shape/dtype")
     _need(key is None or (key.dtype == query.dtype and key.numel() == t * n_kv_heads * head_dim), "key shape/dtype")
     _need(cos.dtype == sin.dtype and cos.numel() == t * head_dim and sin.numel() == t * head_dim,
           "cos/sin must hold one [head_dim] row per token")
-    check(lib.mf_rope_half(ptr(query), ptr(key), ptr(cos), ptr(sin), t, n_heads, n_kv_heads, head_dim,
+    check(lib.mf_rope_half(ptr(query), ptr(key), ptr(cos), ptr(sin), t, n_heads, n_kv_heads, head_dim, qs, ks,
                            dtype_code(query.dtype), dtype_code(cos.dtype), stream_ptr(dev)), "mf_rope_half")
     return query, key
 
@@ -82,9 +115,13 @@ def apply_rotary_pos_emb(query, key, cos, sin, n_heads, n_kv_heads, head_dim):
 def rope_and_cache(query, key, value, cos, sin, key_cache, value_cache, slot_mapping, n_heads):
     """RoPE on q/k (in place) then scatter of rotated k and v into the caches, one launch."""
     lib = _lib.load()
-    dev = _dev_ok(query, key, value, cos, sin, key_cache, value_cache, slot_mapping)
+    _dev_of(query, key, value)
+    dev = _dev_ok(cos, sin, key_cache, value_cache, slot_mapping)
     nb, bs, n_kv, d = key_cache.shape
     t = slot_mapping.numel()
+    query, qs = _rows(query, n_heads * d, "query")
+    key, ks = _rows(key, n_kv * d, "key")
+    value, vs = _rows(value, n_kv * d, "value")
     _need(query.dtype in _ACT and key.dtype == query.dtype and value.dtype == query.dtype
           and key_cache.dtype == query.dtype and value_cache.dtype == query.dtype, "dtype mismatch")
     _need(value_cache.shape == key_cache.shape, "cache shapes differ")
@@ -93,7 +130,7 @@ def rope_and_cache(query, key, value, cos, sin, key_cache, value_cache, slot_map
           "q/k/v sizes do not match slot_mapping and the cache geometry")
     _need(cos.dtype == sin.dtype and cos.numel() == t * d and sin.numel() == t * d, "cos/sin must be [T, head_dim]")
     check(lib.mf_rope_and_cache(ptr(query), ptr(key), ptr(value), ptr(cos), ptr(sin), ptr(key_cache),
-                                ptr(value_cache), ptr(slot_mapping), t, n_heads, n_kv, d, nb * bs,
+                                ptr(value_cache), ptr(slot_mapping), t, n_heads, n_kv, d, nb * bs, qs, ks, vs,
                                 dtype_code(query.dtype), dtype_code(cos.dtype), stream_ptr(dev)), "mf_rope_and_cache")
     return query, key
 
@@ -102,9 +139,11 @@ def rope_and_cache(query, key, value, cos, sin, key_cache, value_cache, slot_map
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n_heads, n_kv_heads, scale, out=None):
     """PagedAttention(head_num, scale, kv_head_num)(query, key_cache, value_cache, block_tables, context_lens)."""
     lib = _lib.load()
-    dev = _dev_ok(query, key_cache, value_cache, block_tables, context_lens, out)
+    _dev_of(query)
+    dev = _dev_ok(key_cache, value_cache, block_tables, context_lens, out)
     _need(key_cache.dim() == 4 and value_cache.shape == key_cache.shape, "caches must be [blocks, block_size, n_kv, D]")
     nb, bs, n_kv, d = key_cache.shape
+    query, qs = _rows(query, n_heads * d, "query")
     _need(n_kv == n_kv_heads, f"cache has {n_kv} kv heads, module says {n_kv_heads}")
     _need(query.dtype in _ACT and key_cache.dtype == query.dtype and value_cache.dtype == query.dtype, "dtype mismatch")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
@@ -114,14 +153,14 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n
     _need(query.numel() == b * n_heads * d, f"query has {query.numel()} elements, expected {b}*{n_heads}*{d}")
     max_blocks = block_tables.shape[1]
     if out is None:
-        out = torch.empty_like(query)
+        out = torch.empty(query.shape, dtype=query.dtype, device=dev)
     else:
         _need(out.shape == query.shape and out.dtype == query.dtype, "out mismatch")
     need = lib.mf_paged_attention_workspace_bytes(b, n_heads, d, max_blocks * bs)
     ws = workspace(need, dev, "pa") if need else None
     check(lib.mf_paged_attention_decode(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(block_tables),
                                         ptr(context_lens), b, n_heads, n_kv_heads, d, bs, max_blocks, nb,
-                                        float(scale), dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,
+                                        float(scale), qs, dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,
                                         stream_ptr(dev)), "mf_paged_attention_decode")
     return out
 

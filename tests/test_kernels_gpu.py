@@ -286,10 +286,11 @@ def _w8a16_case(rng, dtype, m, n, k, bias, residual):
     dot_mag = (np.abs(x).astype(np.float64) @ np.abs(wq).astype(np.float64).T) * s[None, :]
     extra = 2.0 ** -18 * dot_mag + 1e-9                  # fp32 accumulation of exact products
     if residual:
-        # y = round(round(v) + r): the inner rounding may land one step away when v sits on a tie
+        # y = round(round(v) + r): when v sits on a rounding tie the inner rounding may land one full step
+        # (2 eps |v|) away, on top of the outer rounding (eps |ref|)
         vr = rounded(v, dtype).astype(np.float64)
         ref = vr + r
-        return to_np(y), ref, np.abs(ref) + np.abs(vr), extra
+        return to_np(y), ref, np.abs(ref) + 2 * np.abs(vr), extra
     return to_np(y), v, np.abs(v), extra
 
 
