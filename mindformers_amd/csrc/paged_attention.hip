@@ -1,16 +1,18 @@
 // GQA paged-attention decode for gfx950.
 //
 // Work decomposition
-//   grid = (partitions, n_kv_heads * head_groups, batch); one workgroup of 4 wavefronts owns one
-//   512-token partition of one (sequence, kv head) and ALL query heads that share that kv head (up to 16
+//   grid = batch * max_partitions * n_kv_heads * head_groups (1-D); one workgroup of 4 wavefronts owns one
+//   256- or 512-token partition of one (sequence, kv head) and ALL query heads that share that kv head (up to 16
 //   per head group), so every K/V byte is fetched from HBM exactly once.  Workgroups whose partition
 //   starts beyond the sequence's context length exit at once; ragged batches therefore cost nothing.
 //   The 16 tiles (32 tokens each) of a partition are interleaved over the 4 waves.
 //
 // Per 32-token tile (one wave)
-//   S^T[token, head] = K[token, :] . Q[head, :]      two 16x16 MFMA tiles, k-steps of 32 over head_dim;
-//                                                    K rows are loaded from HBM straight into the MFMA
-//                                                    A-operand layout (lane = token row, 16 B per k-step)
+//   K and V rows are fetched with fully coalesced 16-byte lane loads (consecutive lanes read consecutive
+//   bytes of a token row) and staged through a per-wave LDS tile; the MFMA operand layouts are formed by
+//   the LDS reads.  (Loading K straight into the A-operand layout makes every group of lanes touch 16
+//   different cache lines per instruction and runs at less than half the bandwidth.)
+//   S^T[token, head] = K[token, :] . Q[head, :]      two 16x16 MFMA tiles, k-steps of 32 over head_dim
 //   online softmax in fp32 (exp2 domain); the only cross-lane traffic is two xor-shuffles for the row max
 //   O^T[d, head] += V^T[d, token] . P^T[token, head] the probabilities sit in exactly the B-operand layout
 //                                                    when the 32 tokens are ordered (sub-tile, 4g+i); V is
@@ -24,40 +26,86 @@ namespace {
 
 constexpr int PA_WAVES = 4;
 constexpr int PA_TILE = 32;                                   // tokens per MFMA tile
-constexpr int PA_TILES_PER_WAVE = 4;
-constexpr int PA_PART = PA_WAVES * PA_TILES_PER_WAVE * PA_TILE;  // 512 tokens per workgroup
+constexpr int PA_WAVE_TOKENS = PA_WAVES * PA_TILE;           // tokens one round of the 4 waves covers
 constexpr float PA_NEG = -1.0e30f;
 
 template <int D>
 struct PaSmem {
-    static constexpr int VSTRIDE = D * 2 + 8;                 // bytes per staged V row (+8: bank spread)
+    static constexpr int VSTRIDE = D * 2 + 16;                // bytes per staged row (+16: bank spread, keeps 16-B alignment)
     static constexpr int VBYTES = PA_WAVES * PA_TILE * VSTRIDE;
-    static constexpr int OBYTES = PA_WAVES * 16 * D * 4;
-    static constexpr int BYTES = VBYTES > OBYTES ? VBYTES : OBYTES;
+    static constexpr int BYTES = VBYTES;
+    static_assert(16 * D * 4 <= PA_TILE * VSTRIDE, "a wave's accumulators must fit its staging tile");
 };
 
-template <typename T, int D>
-__global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
+// TPW = tiles per wave: a workgroup covers TPW * 128 tokens.
+template <typename T, int D, int TPW>
+__global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
     int n_rep, int head_groups, int block_size, int max_blocks, int num_blocks, int max_parts,
-    float scale_log2, int64_t q_stride) {
+    float scale_log2, int64_t q_stride, int batch) {
     using vec8 = typename T::vec8;
     constexpr int KS = D / 32;
     constexpr int VSTRIDE = PaSmem<D>::VSTRIDE;
+    constexpr int PART = TPW * PA_WAVE_TOKENS;
+    constexpr int CPR = D / 8;                                // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
+    constexpr int NI = PA_TILE / RPI;                         // loads per lane per tile per tensor
 
     __shared__ __attribute__((aligned(16))) uint8_t smem[PaSmem<D>::BYTES];
     __shared__ float sm_m[PA_WAVES][16];
     __shared__ float sm_l[PA_WAVES][16];
+    __shared__ int sm_count;
 
-    const int b = blockIdx.z;
-    const int kvh = blockIdx.y / head_groups;
-    const int hg = blockIdx.y - kvh * head_groups;
-    const int part = blockIdx.x;
-    const int L = ctx_lens[b];
-    const int part_start = part * PA_PART;
-    if (part_start >= L) return;                              // uniform over the workgroup
+    // Work list: blockIdx.x enumerates the (sequence, kv head, partition) triples that exist, sequence-major
+    // and partition-minor; each wave finds its triple with a prefix sum over ceil(L_b / PART), so a ragged batch
+    // leaves no idle workgroups between busy ones (the unused tail of the grid exits here).  The order
+    // matters for HBM: walking the kv heads fastest pins each XCD (consecutive workgroup ids go to
+    // consecutive XCDs) to one 256-byte lane of every token row and measured 25 % slower.
+    const int nkg = n_kv * head_groups;
+    int b = -1, part = 0, L = 0, kg = 0;
+    {
+        const int pidx = blockIdx.x;
+        const int ln = threadIdx.x & 63;
+        int base = 0;
+        for (int c0 = 0; c0 < batch; c0 += 64) {
+            const int bb = c0 + ln;
+            const int len = bb < batch ? ctx_lens[bb] : 0;
+            int np = len > 0 ? (len + PART - 1) / PART : 0;
+            np = np < max_parts ? np : max_parts;
+            int incl = np * nkg;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int t = __shfl_up(incl, o, 64);
+                if (ln >= o) incl += t;
+            }
+            const int total = __shfl(incl, 63, 64);
+            if (pidx < base + total) {
+                const bool hit = pidx >= base + incl - np * nkg && pidx < base + incl;
+                const uint64_t m = __ballot(hit);
+                const int src = __ffsll((unsigned long long)m) - 1;
+                b = c0 + src;
+                const int rem = pidx - (base + __shfl(incl - np * nkg, src, 64));
+                const int npb = __shfl(np, src, 64);
+                kg = rem / npb;
+                part = rem - kg * npb;
+                L = __shfl(len, src, 64);
+                break;
+            }
+            base += total;
+        }
+    }
+    kg = __builtin_amdgcn_readfirstlane(kg);
+    const int kvh = kg / head_groups;
+    const int hg = kg - kvh * head_groups;
+    if (b < 0) return;                                        // uniform over the workgroup
+    b = __builtin_amdgcn_readfirstlane(b);
+    part = __builtin_amdgcn_readfirstlane(part);
+    L = __builtin_amdgcn_readfirstlane(L);
+    const int part_start = part * PART;
+    if (threadIdx.x == 0) sm_count = 0;
+    __syncthreads();                                          // the only barrier: all waves are still in step here
 
     const int w = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -91,25 +139,74 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
     const int64_t row_elems = (int64_t)n_kv * D;
 
-    for (int it = 0; it < PA_TILES_PER_WAVE; ++it) {
-        const int tstart = part_start + (it * PA_WAVES + w) * PA_TILE;
-        if (tstart >= L) break;                               // uniform over the wave
+    const int lrow = lane / CPR;                              // coalesced-load coordinates of this lane
+    const int lchunk = lane - lrow * CPR;
+    const bool tile_in_block = (block_size % PA_TILE) == 0;   // then a tile never straddles two blocks
+    const int wu = __builtin_amdgcn_readfirstlane(w);         // wave index as a scalar
 
-        // ---- issue K and V loads for the tile (both sub-tiles of 16 tokens)
-        u32x4 kreg[2][KS], vreg[2][KS];
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            int tok = tstart + s * 16 + r;
-            tok = tok < L ? tok : L - 1;                      // rows past the context are masked below
+    // tiles of this wave: it = 0 .. ntiles-1 start at part_start + (it*4 + wave)*32
+    int ntiles = 0;
+    {
+        const int first = part_start + wu * PA_TILE;
+        if (first < L) {
+            const int last_tok = min(L, part_start + PART) - 1;
+            ntiles = (last_tok - first) / (PA_WAVES * PA_TILE) + 1;
+        }
+    }
+    // slot of a tile's first token when the tile lies inside one block (uniform: a scalar load), looked up
+    // two tiles ahead so that no K/V load ever waits on a table load
+    auto tile_slot = [&](int ts) -> int64_t {
+        if (!tile_in_block || ts >= L) return 0;
+        const int bi = ts / block_size;
+        int blk = table[bi];
+        blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;       // never leave the cache allocation
+        return (int64_t)blk * block_size + (ts - bi * block_size);
+    };
+    // element offset of chunk lchunk of token (tstart + lrow + RPI*i); tokens past the context re-read the last
+    // valid row (their scores are masked)
+    auto row_offset = [&](int64_t slot0, int tstart, int i) -> int64_t {
+        int tok = tstart + lrow + RPI * i;
+        tok = tok < L ? tok : L - 1;
+        int64_t slot;
+        if (tile_in_block) {
+            slot = slot0 + (tok - tstart);
+        } else {
             const int bi = tok / block_size;
             int blk = table[bi];
-            blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;   // never leave the cache allocation
-            const int64_t off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_elems +
-                                (int64_t)kvh * D + 8 * g;
+            blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
+            slot = (int64_t)blk * block_size + (tok - bi * block_size);
+        }
+        return slot * row_elems + (int64_t)kvh * D + 8 * lchunk;
+    };
+
+    const int tstep = PA_WAVES * PA_TILE;
+    const int tfirst = part_start + wu * PA_TILE;
+    int64_t slot_cur = tile_slot(tfirst), slot_nxt = tile_slot(tfirst + tstep);
+    u32x4 kreg[NI], vreg[NI];
+    if (ntiles > 0) {
 #pragma unroll
-            for (int j = 0; j < KS; ++j) kreg[s][j] = *(const u32x4*)(kc + off + 32 * j);
+        for (int i = 0; i < NI; ++i) kreg[i] = *(const u32x4*)(kc + row_offset(slot_cur, tfirst, i));
 #pragma unroll
-            for (int j = 0; j < KS; ++j) vreg[s][j] = *(const u32x4*)(vc + off + 32 * j);
+        for (int i = 0; i < NI; ++i) vreg[i] = *(const u32x4*)(vc + row_offset(slot_cur, tfirst, i));
+    }
+
+#pragma unroll 1
+    for (int it = 0; it < ntiles; ++it) {
+        const int tstart = tfirst + it * tstep;
+        const int tnext = tstart + tstep;
+        const bool more = it + 1 < ntiles;
+        const int64_t slot_nn = tile_slot(tnext + tstep);
+
+        // ---- stage K row-major in LDS, read it back as MFMA A operands (lane = token row r, 8 d per k-step)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < NI; ++i) *(u32x4*)(vst + (lrow + RPI * i) * VSTRIDE + 16 * lchunk) = kreg[i];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (more) {                                           // next tile's K streams in behind this tile's math
+#pragma unroll
+            for (int i = 0; i < NI; ++i) kreg[i] = *(const u32x4*)(kc + row_offset(slot_nxt, tnext, i));
         }
 
         // ---- scores: S[s][i] = score of token tstart + 16 s + 4 g + i for head r
@@ -118,7 +215,10 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
         for (int s = 0; s < 2; ++s) {
             sc[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < KS; ++j) sc[s] = T::mfma16(bitcast<vec8>(kreg[s][j]), qreg[j], sc[s]);
+            for (int j = 0; j < KS; ++j) {
+                const u32x4 ka = *(const u32x4*)(vst + (s * 16 + r) * VSTRIDE + (32 * j + 8 * g) * 2);
+                sc[s] = T::mfma16(bitcast<vec8>(ka), qreg[j], sc[s]);
+            }
         }
         float tmax = PA_NEG;
 #pragma unroll
@@ -155,19 +255,19 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
         }
         const vec8 pfrag = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
 
-        // ---- stage V (rows = tokens) in this wave's LDS tile
+        // ---- stage V (rows = tokens) in the same LDS tile
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int j = 0; j < KS; ++j) {
-                uint8_t* p = vst + (s * 16 + r) * VSTRIDE + (32 * j + 8 * g) * 2;
-                *(u32x2*)p = (u32x2){vreg[s][j][0], vreg[s][j][1]};
-                *(u32x2*)(p + 8) = (u32x2){vreg[s][j][2], vreg[s][j][3]};
-            }
+        for (int i = 0; i < NI; ++i) *(u32x4*)(vst + (lrow + RPI * i) * VSTRIDE + 16 * lchunk) = vreg[i];
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) vreg[i] = *(const u32x4*)(vc + row_offset(slot_nxt, tnext, i));
+        }
+        slot_cur = slot_nxt;
+        slot_nxt = slot_nn;
 
         // ---- O^T += V^T P^T ; lane (r, g) reads d = 32u + 2r, 2r+1 for its 8 tokens (16*(e/4) + 4g + e%4)
 #pragma unroll
@@ -189,37 +289,37 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
         }
     }
 
-    // ---- merge the 4 waves
+    // ---- merge the 4 waves without a barrier: every wave parks its (max, sum, acc) in LDS (acc goes into its
+    // own, now idle, staging tile), bumps a counter and leaves; the wave that arrives last combines them.
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
     if (g == 0) {
         sm_m[w][r] = m_run;
         sm_l[w][r] = l_run;
     }
-    __syncthreads();                                          // also: every wave is done with its V tile
-    float M = sm_m[0][r];
-#pragma unroll
-    for (int x = 1; x < PA_WAVES; ++x) M = fmaxf(M, sm_m[x][r]);
-    const float f = __builtin_amdgcn_exp2f(m_run - M);
-    float* obuf = (float*)smem;                               // [wave][head 16][D]
     {
-        float* dst = obuf + ((w * 16 + r) * D) + 8 * g;
+        float* dst = (float*)vst + r * D + 8 * g;             // [head 16][D] floats: fits the staging tile
 #pragma unroll
         for (int u = 0; u < KS; ++u) {
             // acc[u][par][i] is d = 32u + 8g + 2i + par
-            f32x4 lo = {acc[u][0][0] * f, acc[u][1][0] * f, acc[u][0][1] * f, acc[u][1][1] * f};
-            f32x4 hi = {acc[u][0][2] * f, acc[u][1][2] * f, acc[u][0][3] * f, acc[u][1][3] * f};
+            f32x4 lo = {acc[u][0][0], acc[u][1][0], acc[u][0][1], acc[u][1][1]};
+            f32x4 hi = {acc[u][0][2], acc[u][1][2], acc[u][0][3], acc[u][1][3]};
             *(f32x4*)(dst + 32 * u) = lo;
             *(f32x4*)(dst + 32 * u + 4) = hi;
         }
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    int arrived = 0;
+    if (lane == 0) arrived = atomicAdd(&sm_count, 1);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    if (arrived != PA_WAVES - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
     constexpr int D4 = D / 4;
-    for (int idx = threadIdx.x; idx < 16 * D4; idx += PA_WAVES * 64) {
+    for (int idx = lane; idx < 16 * D4; idx += 64) {
         const int hr = idx / D4, d4 = idx - hr * D4;
         const int hq = hg * 16 + hr;
-        if (hq >= n_rep) continue;
+        if (hq >= n_rep) break;                               // heads are ordered: nothing valid follows
         float Mh = sm_m[0][hr];
 #pragma unroll
         for (int x = 1; x < PA_WAVES; ++x) Mh = fmaxf(Mh, sm_m[x][hr]);
@@ -227,8 +327,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int x = 0; x < PA_WAVES; ++x) {
-            lt += sm_l[x][hr] * __builtin_amdgcn_exp2f(sm_m[x][hr] - Mh);
-            sum += *(const f32x4*)(obuf + (x * 16 + hr) * D + 4 * d4);
+            const float f = __builtin_amdgcn_exp2f(sm_m[x][hr] - Mh);
+            lt += sm_l[x][hr] * f;
+            sum += *(const f32x4*)((const float*)(smem + x * (PA_TILE * VSTRIDE)) + hr * D + 4 * d4) * f;
         }
         const int64_t gh = (int64_t)b * n_heads + kvh * n_rep + hq;
         if (max_parts == 1) {
@@ -247,31 +348,65 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void paged_attention_kernel(
 }
 
 // Combine the partitions of one (sequence, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p.
+// One workgroup of D threads per (head, sequence).  The per-partition (max, sum) pairs are read one per lane
+// and reduced across the wave; the weighted accumulator sum runs 8 independent loads deep.
 template <typename T, int D>
-__global__ void paged_attention_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ part_out,
-                                              const float* __restrict__ part_ml,
-                                              const int32_t* __restrict__ ctx_lens, int n_heads, int max_parts) {
+__global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __restrict__ out,
+                                                                  const float* __restrict__ part_out,
+                                                                  const float* __restrict__ part_ml,
+                                                                  const int32_t* __restrict__ ctx_lens, int n_heads,
+                                                                  int max_parts, int part_tokens) {
+    __shared__ float s_f[64];
     const int h = blockIdx.x, b = blockIdx.y;
     const int d = threadIdx.x;
+    const int lane = threadIdx.x & 63;
     const int L = ctx_lens[b];
     const int64_t gh = (int64_t)b * n_heads + h;
-    int np = L <= 0 ? 0 : (L + PA_PART - 1) / PA_PART;
+    int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
     np = np < max_parts ? np : max_parts;
     if (np == 0) {
         out[gh * D + d] = 0;
         return;
     }
     const float* ml = part_ml + gh * max_parts * 2;
+    const float* po = part_out + gh * max_parts * D + d;
+    // pass 1: global maximum (every wave computes it for itself)
     float M = PA_NEG;
-    for (int p = 0; p < np; ++p) M = fmaxf(M, ml[2 * p]);
+    for (int p0 = 0; p0 < np; p0 += 64) {
+        const int p = p0 + lane;
+        M = fmaxf(M, p < np ? ml[2 * p] : PA_NEG);
+    }
+    M = wave_max(M);
+    // pass 2: weights, denominator, weighted sum, 64 partitions at a time
     float num = 0.f, den = 0.f;
-    for (int p = 0; p < np; ++p) {
-        const float f = __builtin_amdgcn_exp2f(ml[2 * p] - M);
-        den += f * ml[2 * p + 1];
-        num += f * part_out[(gh * max_parts + p) * D + d];
+    for (int p0 = 0; p0 < np; p0 += 64) {
+        const int p = p0 + lane;
+        float f = 0.f, l = 0.f;
+        if (p < np) {
+            f = __builtin_amdgcn_exp2f(ml[2 * p] - M);
+            l = ml[2 * p + 1];
+        }
+        den += wave_sum(f * l);
+        __syncthreads();                                      // previous chunk's weights are no longer needed
+        if (threadIdx.x < 64) s_f[lane] = f;
+        __syncthreads();
+        const int cnt = min(64, np - p0);
+        int q = 0;
+        for (; q + 8 <= cnt; q += 8) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = po[(int64_t)(p0 + q + i) * D];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) num += s_f[q + i] * v[i];
+        }
+        for (; q < cnt; ++q) num += s_f[q] * po[(int64_t)(p0 + q) * D];
     }
     out[gh * D + d] = T::from_float(num / den);
 }
+
+// Partition size rule shared by the workspace query and the launch: 256-token partitions keep the tail of
+// the last round of workgroups short; very long contexts use 512 to halve the partial traffic.
+static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 16384 ? 4 : 2; }
 
 template <typename T, int D>
 int launch_pa(void* out, const void* query, const void* key_cache, const void* value_cache,
@@ -281,20 +416,26 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    const int max_parts = (int)((max_ctx + PA_PART - 1) / PA_PART);
+    const int tpw = pa_tiles_per_wave(max_ctx);
+    const int part_tokens = tpw * PA_WAVE_TOKENS;
+    const int max_parts = (int)((max_ctx + part_tokens - 1) / part_tokens);
     float* part_out = (float*)workspace;
     float* part_ml = part_out ? part_out + (int64_t)batch * n_heads * max_parts * D : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
-    dim3 grid(max_parts, n_kv * head_groups, batch);
-    hipLaunchKernelGGL((paged_attention_kernel<T, D>), grid, dim3(PA_WAVES * 64), 0, st, (uint16_t*)out, part_out,
-                       part_ml, (const uint16_t*)query, (const uint16_t*)key_cache, (const uint16_t*)value_cache,
-                       block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, block_size, max_blocks,
-                       num_blocks, max_parts, scale_log2, q_stride);
+    dim3 grid((unsigned)((int64_t)batch * max_parts * n_kv * head_groups));
+#define PA_LAUNCH(TPWV)                                                                                          \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV>), grid, dim3(PA_WAVES * 64), 0, st, (uint16_t*)out,     \
+                       part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,                      \
+                       (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
+                       block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch)
+    if (tpw == 2) PA_LAUNCH(2);
+    else PA_LAUNCH(4);
+#undef PA_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (max_parts > 1) {
         hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D>), dim3(n_heads, batch), dim3(D), 0, st,
-                           (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts);
+                           (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts, part_tokens);
         rc = MF_LAUNCH_CHECK();
     }
     return rc;
@@ -310,7 +451,8 @@ __global__ void pa_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t* 
 }  // namespace
 
 extern "C" size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, int max_context) {
-    const int64_t max_parts = ((int64_t)max_context + PA_PART - 1) / PA_PART;
+    const int part_tokens = pa_tiles_per_wave(max_context) * PA_WAVE_TOKENS;
+    const int64_t max_parts = ((int64_t)max_context + part_tokens - 1) / part_tokens;
     if (max_parts <= 1) return 0;
     return (size_t)batch * n_heads * max_parts * (head_dim + 2) * sizeof(float);
 }
