@@ -102,15 +102,23 @@ int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* 
 
 /* ---- quantized linear ----------------------------------------------------------------------------- */
 
+/* The W8A16 kernels stream the int8 weight in a tiled order (16 output channels x 64 input channels per
+ * 1 KiB tile, tiles ordered [n-tile][k-step], bytes inside a tile in MFMA-operand lane order; N padded to 16
+ * and K to 64 with zeros).  Pack once after the checkpoint is loaded — the counterpart of the format
+ * conversion golden-stick's deploy cells apply to their weight Parameter.  w is int8 [N, K] row-major. */
+size_t mf_w8a16_packed_bytes(int n, int k);
+int mf_w8a16_pack_weight(void* packed, const int8_t* w, int n, int k, void* stream);
+
 size_t mf_w8a16_workspace_bytes(int m, int n, int k);
 
 /* golden-stick weight-only cell -> WeightQuantBatchMatmul, replacing P.MatMul(transpose_b=True) at
  *   mindformers/modules/layers.py:479,526; parallel_core/inference/tensor_parallel/layers.py:186,406
  * (swapped in by Quantizer.preprocess_model, mindformers/modules/quantizers/rtn_quantizer.py:61-67).
  * y[m,n] = (sum_k x[m,k] * w[n,k]) * scale[n] (+ bias[n]) (+ residual[m,n]); x/y/bias/residual in `dtype`,
- * w int8 [N,K] row-major, scale float32 [N]; products exact, fp32 accumulation, scale applied to the sum.
- * With residual: y = round(round(acc*scale+bias) + residual).  K % 16 == 0. */
-int mf_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const void* bias,
+ * w_packed = mf_w8a16_pack_weight of the int8 [N,K] weight, scale float32 [N]; products exact, fp32
+ * accumulation, scale applied to the sum.  With residual: y = round(round(acc*scale+bias) + residual).
+ * K % 8 == 0. */
+int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
                   const void* residual, int m, int n, int k, int dtype, void* workspace,
                   size_t workspace_bytes, void* stream);
 
@@ -150,9 +158,10 @@ int mf_moe_permute(void* permuted_x, int32_t* row_map, int64_t* counts, int32_t*
 
 /* GroupedMatmulV4(split_item=3, group_type=0, group_list_type=1) with int8 expert weights —
  * mindformers/parallel_core/inference/transformer/moe/experts.py:116-117,136-137.
- * Rows offsets[e]..offsets[e+1] of x use expert e: y = (x . w[e]^T) * scale[e].  w int8 [E, N, K] (K
- * contiguous: the [E, in, out] parameter of experts.py:71-72 stored transposed at load), scale fp32 [E, N]. */
-int mf_grouped_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const int32_t* offsets,
+ * Rows offsets[e]..offsets[e+1] of x use expert e: y = (x . w[e]^T) * scale[e].  w_packed holds the E experts
+ * back to back, each mf_w8a16_pack_weight of its int8 [N, K] matrix (the [E, in, out] parameter of
+ * experts.py:71-72 transposed at load), mf_w8a16_packed_bytes(n, k) apart; scale fp32 [E, N]. */
+int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const int32_t* offsets,
                           int n_experts, int total_rows, int n, int k, int dtype, void* stream);
 
 /* MoeTokenUnpermute(permuted_tokens, sorted_indices, probs) — moe_layer.py:151-155.

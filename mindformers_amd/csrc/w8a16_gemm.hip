@@ -1,17 +1,24 @@
-// W8A16 weight-only skinny GEMM for decode (M <= 64 per pass): y = (x . w_i8^T) * scale (+bias) (+residual).
+// W8A16 weight-only skinny GEMM for decode: y = (x . w_i8^T) * scale (+bias) (+residual), dense and grouped.
 //
-// The int8 weight matrix [N, K] is the only large operand: it is streamed from HBM exactly once, each lane
-// loading 16 contiguous bytes of one weight row straight into the MFMA A-operand layout (no LDS), converted
-// to bf16/fp16 in registers (exact: |w| <= 127) and multiplied on the 16x16x32 matrix cores against the
-// activation tile, which every wave re-reads from L2.  A workgroup owns 64 output channels (4 MFMA row tiles) for
-// all M rows; its 4 waves interleave the 64-wide k-steps of the workgroup's k-range and are summed through
-// LDS at the end.  When N is too small to fill the chip the k-range is additionally split across workgroups
-// (fp32 partials + a fused reduce/epilogue kernel).
+// Weight layout ("packed", produced once at load time by mf_w8a16_pack_weight): the int8 matrix [N, K] is cut
+// into tiles of 16 output channels x 64 input channels (1 KiB).  Inside a tile byte (16*g + r)*16 + j holds
+// w[16*t + r][64*s + 16*g + j]: exactly the order in which the 64 lanes of a wavefront want their MFMA
+// A-operand bytes, so one wave-wide 16-byte load reads one whole tile as 1 KiB of contiguous memory.
+// Tiles are ordered [n-tile][k-step]; N is padded to 16 and K to 64 with zeros.  (Loading the same bytes
+// from the row-major matrix makes every group of lanes touch 16 different cache lines per instruction and
+// ran at about a third of the bandwidth.)
 //
-// MFMA roles: A = weights [16 n x 32 k], B = activations [32 k x 16 m], C = y^T tile [16 n x 16 m].
-// k-ordering trick: one 16-byte weight load covers 16 k of a row; bytes 0-7 feed the first MFMA of the
-// step and bytes 8-15 the second, and the activation operand uses the same (permuted) k order, so no
-// shuffling is needed.
+// A workgroup of 4 waves owns 64 output channels (4 n-tiles) for up to 64 rows of x.  The waves interleave
+// the 64-wide k-steps of the workgroup's k-range; each wave streams its tiles HBM -> registers two steps
+// ahead, converts int8 -> bf16/fp16 in registers (exact) and multiplies on the 16x16x32 matrix cores.  The
+// activation tile of a step ([rows, 64], re-read from L2 by every workgroup) is fetched with coalesced
+// 128-byte row pieces and staged through a private, XOR-swizzled LDS tile from which the MFMA B operands are
+// read.  The 4 waves are summed through LDS at the end; when N is too small to fill the chip the k-range is
+// also split across workgroups (fp32 partials + a fused reduce/epilogue kernel).
+//
+// MFMA roles: A = weights [16 n x 32 k], B = activations [32 k x 16 m], C = y^T tile [16 n x 16 m]; the two
+// MFMAs of a k-step take bytes 0-7 and 8-15 of each lane's 16 weight bytes, and the activation operand is
+// gathered in the same k order.
 #include "common.h"
 
 namespace {
@@ -20,6 +27,8 @@ constexpr int GW_WAVES = 4;
 constexpr int GW_NT = 4;                    // 16-row weight tiles per wave
 constexpr int GW_BN = 16 * GW_NT;           // output channels per workgroup
 constexpr int GW_KSTEP = 64;
+constexpr int GW_TILE_BYTES = 16 * GW_KSTEP;
+constexpr int GW_DEPTH = 2;                 // weight k-steps in flight per wave beyond the current one
 
 // 8 int8 (two dwords) -> 8 elements of T, exact.
 template <typename T>
@@ -72,18 +81,19 @@ __device__ __forceinline__ void store4(uint16_t* y, const uint16_t* bias, const 
     }
 }
 
-// One workgroup tile: 64 output channels [n0, n0+64) x 16*MT rows [m0, ...) x k-steps [s_begin, s_end).
-// MT = number of 16-row activation tiles.
-template <typename T, int MT>
+// One workgroup tile: output channels [n0, n0+64) x 16*MT rows [m0, ...) x k-steps [s_begin, s_end).
+// MT = number of 16-row activation tiles; KTAIL = K is not a multiple of 64.  wp = packed weights of this
+// matrix, KS = k-steps per n-tile.
+template <typename T, int MT, bool KTAIL>
 __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __restrict__ partial,
-                                           const uint16_t* __restrict__ x, const int8_t* __restrict__ w,
+                                           const uint16_t* __restrict__ x, const uint8_t* __restrict__ wp,
                                            const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-                                           const uint16_t* __restrict__ residual, int M, int N, int K, int n0,
-                                           int m0, int s_begin, int s_end, int split_index) {
+                                           const uint16_t* __restrict__ residual, int M, int N, int K, int KS, int n0,
+                                           int m0, int s_begin, int s_end, int split_index, uint8_t* smem) {
     using vec8 = typename T::vec8;
-    // red[wave][m][n], 16-byte granules XOR-swizzled by the row so that neither the MFMA-layout writes nor the
-    // row-major reads collide on LDS banks (64 KB at MT = 4, the static limit, so no padding)
-    __shared__ __attribute__((aligned(16))) float red[GW_WAVES][16 * MT][GW_BN];
+    constexpr int XROWS = 16 * MT;
+    constexpr int XTILE = XROWS * 128;                        // bytes of one staged activation tile
+    constexpr int XLD = XROWS / 8;                            // coalesced loads per lane per tile (8 rows each)
 
     const int wv = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -96,71 +106,117 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // per-lane row pointers (rows beyond N / M read row 0 and are zeroed)
-    const int8_t* wrow[GW_NT];
-    bool wok[GW_NT];
+    // Every load below is unconditional and reads an address that exists (indices are clamped), so the loop body
+    // has no divergent branches: tiles beyond N and rows beyond M compute garbage that is never stored, steps
+    // beyond s_end are prefetched from a clamped address and never consumed, and only the activation chunks
+    // past K (last, short k-step) are replaced by zeros with a select.
+    // ---- weights: tile (n-tile t, step s) sits at ((t*KS + s) * 1024) + lane*16
+    const int n_tiles_total = (N + 15) >> 4;
+    const uint8_t* wbase[GW_NT];
 #pragma unroll
     for (int nt = 0; nt < GW_NT; ++nt) {
-        const int n = n0 + nt * 16 + r;
-        wok[nt] = n < N;
-        wrow[nt] = w + (int64_t)(wok[nt] ? n : 0) * K + 16 * g;
+        const int t = min((n0 >> 4) + nt, n_tiles_total - 1);
+        wbase[nt] = wp + (int64_t)t * KS * GW_TILE_BYTES + lane * 16;
     }
-    const uint16_t* xrow[MT];
-    bool xok[MT];
+    // ---- activations: load i of lane (xr, xc) is the 16-byte chunk xc (8 elements) of row xr + 8*i
+    const int xr = lane >> 3, xc = lane & 7;
+    const uint16_t* xptr[XLD];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = m0 + mt * 16 + r;
-        xok[mt] = m < M;
-        xrow[mt] = x + (int64_t)(xok[mt] ? m : 0) * K + 16 * g;
+    for (int i = 0; i < XLD; ++i) {
+        const int m = min(m0 + xr + 8 * i, M - 1);
+        xptr[i] = x + (int64_t)m * K + 8 * xc;
     }
+    uint8_t* xst = smem + wv * XTILE;                         // this wave's staging tile
+    const int s_last = s_end - 1;
+    const int k_last_chunk = K - 8;                           // element offset of the last whole 16-byte chunk
 
-    for (int s = s_begin + wv; s < s_end; s += GW_WAVES) {
-        const int kb = s * GW_KSTEP;
-        const bool kok = kb + 16 * g < K;                     // K is a multiple of 16; the last step may be short
-        u32x4 wreg[GW_NT];
+    const int first = s_begin + wv;
+    u32x4 wreg[GW_DEPTH + 1][GW_NT];
+    u32x4 xreg[XLD];
+    auto load_w = [&](int slot, int s) {
+        const int64_t off = (int64_t)min(s, s_last) * GW_TILE_BYTES;
 #pragma unroll
-        for (int nt = 0; nt < GW_NT; ++nt) {
-            wreg[nt] = (u32x4){0u, 0u, 0u, 0u};
-            if (kok && wok[nt]) wreg[nt] = *(const u32x4*)(wrow[nt] + kb);
-        }
-        u32x4 xreg[MT][2];
+        for (int nt = 0; nt < GW_NT; ++nt) wreg[slot][nt] = *(const u32x4*)(wbase[nt] + off);
+    };
+    auto load_x = [&](int s) {
+        const int kb = min(s, s_last) * GW_KSTEP;
+        if (KTAIL) {
+            // K is not a multiple of 64: chunks past K (last, short step) read a clamped address and are zeroed
+            // with a mask (an AND, so that the load stays unconditional)
+            const bool kok = kb + 8 * xc < K;
+            const int koff = kok ? kb : k_last_chunk - 8 * xc;
+            const uint32_t km = kok ? 0xffffffffu : 0u;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            xreg[mt][0] = (u32x4){0u, 0u, 0u, 0u};
-            xreg[mt][1] = (u32x4){0u, 0u, 0u, 0u};
-            if (kok && xok[mt]) {
-                xreg[mt][0] = *(const u32x4*)(xrow[mt] + kb);
-                xreg[mt][1] = *(const u32x4*)(xrow[mt] + kb + 8);
+            for (int i = 0; i < XLD; ++i) {
+                const u32x4 v = *(const u32x4*)(xptr[i] + koff);
+                xreg[i] = (u32x4){v[0] & km, v[1] & km, v[2] & km, v[3] & km};
             }
+        } else {
+#pragma unroll
+            for (int i = 0; i < XLD; ++i) xreg[i] = *(const u32x4*)(xptr[i] + kb);
         }
+    };
+#pragma unroll
+    for (int d = 0; d <= GW_DEPTH; ++d) load_w(d, first + d * GW_WAVES);
+    load_x(first);
+
+    // the weight registers rotate through GW_DEPTH + 1 slots; the loop body is written once per slot so that
+    // every register index is a compile-time constant
+    auto step = [&](int slot, int s) {
+        // stage this step's activations: physical chunk = logical chunk ^ (row & 7)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < XLD; ++i) *(u32x4*)(xst + (xr + 8 * i) * 128 + ((xc ^ xr) << 4)) = xreg[i];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        load_x(s + GW_WAVES);                                 // next step's activations (L2) behind this step's math
+
+        // B operands: lane (r, g), tile mt, half h reads logical chunk 2g + h of row 16*mt + r
+        vec8 xb[MT][2];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                xb[mt][h] = bitcast<vec8>(*(const u32x4*)(xst + (16 * mt + r) * 128 + (((2 * g + h) ^ (r & 7)) << 4)));
 #pragma unroll
         for (int nt = 0; nt < GW_NT; ++nt) {
-            const vec8 a0 = dequant8<T>(wreg[nt][0], wreg[nt][1]);
-            const vec8 a1 = dequant8<T>(wreg[nt][2], wreg[nt][3]);
+            const vec8 a0 = dequant8<T>(wreg[slot][nt][0], wreg[slot][nt][1]);
+            const vec8 a1 = dequant8<T>(wreg[slot][nt][2], wreg[slot][nt][3]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                acc[nt][mt] = T::mfma16(a0, bitcast<vec8>(xreg[mt][0]), acc[nt][mt]);
-                acc[nt][mt] = T::mfma16(a1, bitcast<vec8>(xreg[mt][1]), acc[nt][mt]);
+                acc[nt][mt] = T::mfma16(a0, xb[mt][0], acc[nt][mt]);
+                acc[nt][mt] = T::mfma16(a1, xb[mt][1], acc[nt][mt]);
             }
         }
+        load_w(slot, s + (GW_DEPTH + 1) * GW_WAVES);
+    };
+    for (int s = first; s < s_end; s += (GW_DEPTH + 1) * GW_WAVES) {
+#pragma unroll
+        for (int slot = 0; slot <= GW_DEPTH; ++slot)
+            if (s + slot * GW_WAVES < s_end) step(slot, s + slot * GW_WAVES);
     }
 
-    // ---- sum the 4 waves through LDS: red[wave][m][n]
+    // ---- sum the 4 waves through LDS: red[wave][m][n], 16-byte granules XOR-swizzled by the row so that
+    // neither the MFMA-layout writes nor the row-major reads collide on LDS banks
+    __syncthreads();                                          // every wave is done with its staging tile
+    float* red = (float*)smem;                                // [GW_WAVES][XROWS][GW_BN]
 #pragma unroll
     for (int nt = 0; nt < GW_NT; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *(f32x4*)&red[wv][mt * 16 + r][((nt * 4 + g) ^ r) << 2] = acc[nt][mt];
+        for (int mt = 0; mt < MT; ++mt)
+            *(f32x4*)(red + ((wv * XROWS + mt * 16 + r) * GW_BN) + (((nt * 4 + g) ^ r) << 2)) = acc[nt][mt];
     __syncthreads();
 
     constexpr int N4 = GW_BN / 4;
-    for (int idx = threadIdx.x; idx < 16 * MT * N4; idx += GW_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < XROWS * N4; idx += GW_WAVES * 64) {
         const int ml = idx / N4, n4 = idx - ml * N4;
         const int m = m0 + ml, n = n0 + 4 * n4;
         if (m >= M || n >= N) continue;
         const int sw = (n4 ^ (ml & 15)) << 2;
-        f32x4 sum = *(const f32x4*)&red[0][ml][sw];
+        f32x4 sum = *(const f32x4*)(red + (ml * GW_BN) + sw);
 #pragma unroll
-        for (int q = 1; q < GW_WAVES; ++q) sum += *(const f32x4*)&red[q][ml][sw];
+        for (int q = 1; q < GW_WAVES; ++q) sum += *(const f32x4*)(red + ((q * XROWS + ml) * GW_BN) + sw);
         if (partial) {
             float* p = partial + ((int64_t)split_index * M + m) * N + n;
             if (n + 3 < N && (N & 3) == 0) {
@@ -176,39 +232,48 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
     }
 }
 
+template <int MT>
+struct GwSmem {
+    // activation staging (4 waves x [16*MT, 64] bf16) and the cross-wave reduction ([4][16*MT][64] fp32) alias
+    static constexpr int BYTES = GW_WAVES * 16 * MT * GW_BN * 4;
+};
+
 // Dense: grid = (ceil(N/64), split_k, ceil(M/(16*MT))).
-template <typename T, int MT>
+template <typename T, int MT, bool KTAIL>
 __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_gemm_kernel(
     uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
-    const int8_t* __restrict__ w, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
+    const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
     const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split) {
-    const int total_steps = (K + GW_KSTEP - 1) / GW_KSTEP;
+    __shared__ __attribute__((aligned(16))) uint8_t smem[GwSmem<MT>::BYTES];
+    const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
     const int s_begin = blockIdx.y * steps_per_split;
-    const int s_end = min(total_steps, s_begin + steps_per_split);
-    w8a16_tile<T, MT>(y, partial, x, w, scale, bias, residual, M, N, K, blockIdx.x * GW_BN,
-                      blockIdx.z * (16 * MT), s_begin, s_end, blockIdx.y);
+    const int s_end = min(KS, s_begin + steps_per_split);
+    w8a16_tile<T, MT, KTAIL>(y, partial, x, wp, scale, bias, residual, M, N, K, KS, blockIdx.x * GW_BN,
+                      blockIdx.z * (16 * MT), s_begin, s_end, blockIdx.y, smem);
 }
 
 // Grouped (experts): grid = (ceil(N/64), n_experts).  Rows offsets[e] .. offsets[e+1] of x use expert e's
-// weights w[e] ([N, K]) and scale[e]; experts with no rows exit at once.  Rows are taken 16 at a time
-// (decode batches route a handful of tokens to each expert), re-streaming the expert's weights per pass.
-template <typename T>
+// packed weights and scale[e]; experts with no rows exit at once.  Rows are taken 16 at a time (decode
+// batches route a handful of tokens to each expert), re-streaming the expert's weights per pass.
+template <typename T, bool KTAIL>
 __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_grouped_kernel(
-    uint16_t* __restrict__ y, const uint16_t* __restrict__ x, const int8_t* __restrict__ w,
-    const float* __restrict__ scale, const int32_t* __restrict__ offsets, int total_rows, int N, int K) {
+    uint16_t* __restrict__ y, const uint16_t* __restrict__ x, const uint8_t* __restrict__ wp,
+    const float* __restrict__ scale, const int32_t* __restrict__ offsets, int total_rows, int N, int K,
+    int64_t expert_bytes) {
+    __shared__ __attribute__((aligned(16))) uint8_t smem[GwSmem<1>::BYTES];
     const int e = blockIdx.y;
     int row0 = offsets[e], row1 = offsets[e + 1];
     row0 = max(0, min(row0, total_rows));
     row1 = max(row0, min(row1, total_rows));
     const int rows = row1 - row0;
     if (rows == 0) return;
-    const int total_steps = (K + GW_KSTEP - 1) / GW_KSTEP;
-    const int8_t* we = w + (int64_t)e * N * K;
+    const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
+    const uint8_t* we = wp + (int64_t)e * expert_bytes;
     const float* se = scale + (int64_t)e * N;
     for (int m0 = 0; m0 < rows; m0 += 16) {
-        w8a16_tile<T, 1>(y + (int64_t)row0 * N, nullptr, x + (int64_t)row0 * K, we, se, nullptr, nullptr, rows, N, K,
-                         blockIdx.x * GW_BN, m0, 0, total_steps, 0);
-        __syncthreads();                                      // the LDS reduction buffer is reused by the next pass
+        w8a16_tile<T, 1, KTAIL>(y + (int64_t)row0 * N, nullptr, x + (int64_t)row0 * K, we, se, nullptr, nullptr, rows, N, K, KS,
+                         blockIdx.x * GW_BN, m0, 0, KS, 0, smem);
+        __syncthreads();                                      // the LDS tile is reused by the next pass
     }
 }
 
@@ -223,17 +288,37 @@ __global__ void w8a16_splitk_reduce_kernel(uint16_t* __restrict__ y, const float
         const int m = (int)(idx / n4cnt);
         const int n = (int)(idx - (int64_t)m * n4cnt) * 4;
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < split_k; ++s) {
-            const float* p = partial + ((int64_t)s * M + m) * N + n;
-            if (n + 3 < N && (N & 3) == 0) {
-                sum += *(const f32x4*)p;
-            } else {
+        if (n + 3 < N && (N & 3) == 0) {
+            for (int s = 0; s < split_k; ++s) sum += *(const f32x4*)(partial + ((int64_t)s * M + m) * N + n);
+        } else {
+            for (int s = 0; s < split_k; ++s)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (n + i < N) sum[i] += p[i];
-            }
+                    if (n + i < N) sum[i] += partial[((int64_t)s * M + m) * N + n + i];
         }
         store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, sum);
+    }
+}
+
+// [N, K] row-major int8 -> packed tiles.  One thread per 16 packed bytes.
+__global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __restrict__ src, int N, int K, int KS,
+                                  int64_t chunks) {
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * blockDim.x) {
+        const int lane = (int)(c & 63);
+        const int64_t tile = c >> 6;
+        const int s = (int)(tile % KS);
+        const int t = (int)(tile / KS);
+        const int n = 16 * t + (lane & 15);
+        const int k0 = 64 * s + 16 * (lane >> 4);
+        uint8_t b[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) b[j] = (n < N && k0 + j < K) ? (uint8_t)src[(int64_t)n * K + k0 + j] : 0;
+        u32x4 v;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            v[q] = (uint32_t)b[4 * q] | ((uint32_t)b[4 * q + 1] << 8) | ((uint32_t)b[4 * q + 2] << 16) |
+                   ((uint32_t)b[4 * q + 3] << 24);
+        *(u32x4*)(dst + c * 16) = v;
     }
 }
 
@@ -251,10 +336,10 @@ GemmPlan plan_w8a16(int m, int n, int k) {
     p.m_blocks = (m + 16 * p.mt - 1) / (16 * p.mt);
     p.n_blocks = (n + GW_BN - 1) / GW_BN;
     const int total_steps = (k + GW_KSTEP - 1) / GW_KSTEP;
-    // aim at two resident workgroups on each of the 256 CUs; keep at least 8 k-steps per workgroup
+    // aim at two resident workgroups on each of the 256 CUs; keep at least 12 k-steps per workgroup
     int sk = 512 / (p.n_blocks * p.m_blocks);
     sk = sk < 1 ? 1 : sk;
-    const int max_sk = total_steps / 8 < 1 ? 1 : total_steps / 8;
+    const int max_sk = total_steps / 12 < 1 ? 1 : total_steps / 12;
     sk = sk > max_sk ? max_sk : sk;
     sk = sk > 16 ? 16 : sk;
     p.steps_per_split = (total_steps + sk - 1) / sk;
@@ -263,18 +348,20 @@ GemmPlan plan_w8a16(int m, int n, int k) {
 }
 
 template <typename T>
-int launch_w8a16(void* y, const void* x, const int8_t* w, const float* scale, const void* bias,
+int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
                  const void* residual, int m, int n, int k, void* workspace, hipStream_t st) {
     const GemmPlan p = plan_w8a16(m, n, k);
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
     dim3 block(GW_WAVES * 64);
-#define GW_LAUNCH(MTV)                                                                                          \
-    hipLaunchKernelGGL((w8a16_gemm_kernel<T, MTV>), grid, block, 0, st, (uint16_t*)y, partial, (const uint16_t*)x, \
-                       w, scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split)
-    if (p.mt == 1) GW_LAUNCH(1);
-    else if (p.mt == 2) GW_LAUNCH(2);
-    else GW_LAUNCH(4);
+#define GW_LAUNCH(MTV, KT)                                                                                       \
+    hipLaunchKernelGGL((w8a16_gemm_kernel<T, MTV, KT>), grid, block, 0, st, (uint16_t*)y, partial,                  \
+                       (const uint16_t*)x, wp, scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,    \
+                       p.steps_per_split)
+    const bool ktail = (k % GW_KSTEP) != 0;
+    if (p.mt == 1) { if (ktail) GW_LAUNCH(1, true); else GW_LAUNCH(1, false); }
+    else if (p.mt == 2) { if (ktail) GW_LAUNCH(2, true); else GW_LAUNCH(2, false); }
+    else { if (ktail) GW_LAUNCH(4, true); else GW_LAUNCH(4, false); }
 #undef GW_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc || !partial) return rc;
@@ -287,47 +374,68 @@ int launch_w8a16(void* y, const void* x, const int8_t* w, const float* scale, co
 
 }  // namespace
 
+extern "C" size_t mf_w8a16_packed_bytes(int n, int k) {
+    if (n <= 0 || k <= 0) return 0;
+    return (size_t)((n + 15) / 16) * ((k + GW_KSTEP - 1) / GW_KSTEP) * GW_TILE_BYTES;
+}
+
+extern "C" int mf_w8a16_pack_weight(void* packed, const int8_t* w, int n, int k, void* stream) {
+    MF_REQUIRE(packed && w, "w8a16_pack_weight: null argument");
+    MF_REQUIRE(n > 0 && k > 0, "w8a16_pack_weight: bad sizes n=%d k=%d", n, k);
+    MF_REQUIRE(((uintptr_t)packed & 15) == 0, "w8a16_pack_weight: packed buffer must be 16-byte aligned");
+    const int KS = (k + GW_KSTEP - 1) / GW_KSTEP;
+    const int64_t chunks = (int64_t)mf_w8a16_packed_bytes(n, k) / 16;
+    const int blocks = (int)((chunks + 255) / 256 > 65535 ? 65535 : (chunks + 255) / 256);
+    hipLaunchKernelGGL(w8a16_pack_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint8_t*)packed, w, n, k, KS,
+                       chunks);
+    return MF_LAUNCH_CHECK();
+}
+
 extern "C" size_t mf_w8a16_workspace_bytes(int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
     const GemmPlan p = plan_w8a16(m, n, k);
     return p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(float) : 0;
 }
 
-extern "C" int mf_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale, const void* bias,
+extern "C" int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
                              const void* residual, int m, int n, int k, int dtype, void* workspace,
                              size_t workspace_bytes, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_gemm: dtype must be bf16 or fp16");
     if (m == 0) return 0;
-    MF_REQUIRE(y && x && w && scale, "w8a16_gemm: null argument");
+    MF_REQUIRE(y && x && w_packed && scale, "w8a16_gemm: null argument");
     MF_REQUIRE(m >= 0 && n > 0 && k > 0, "w8a16_gemm: bad sizes m=%d n=%d k=%d", m, n, k);
-    MF_REQUIRE(k % 16 == 0, "w8a16_gemm: K (%d) must be a multiple of 16", k);
-    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "w8a16_gemm: x and w must be 16-byte aligned");
-    if (m == 0) return 0;
+    MF_REQUIRE(k % 8 == 0, "w8a16_gemm: K (%d) must be a multiple of 8", k);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0, "w8a16_gemm: x and w_packed must be 16-byte aligned");
     const size_t need = mf_w8a16_workspace_bytes(m, n, k);
     MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
                "w8a16_gemm: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     if (dtype == MF_BF16)
-        return launch_w8a16<BF16>(y, x, w, scale, bias, residual, m, n, k, workspace, (hipStream_t)stream);
-    return launch_w8a16<FP16>(y, x, w, scale, bias, residual, m, n, k, workspace, (hipStream_t)stream);
+        return launch_w8a16<BF16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, workspace,
+                                  (hipStream_t)stream);
+    return launch_w8a16<FP16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, workspace,
+                              (hipStream_t)stream);
 }
 
-extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const int8_t* w, const float* scale,
+extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale,
                                      const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype,
                                      void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "grouped_w8a16_gemm: dtype must be bf16 or fp16");
     if (total_rows == 0) return 0;
-    MF_REQUIRE(y && x && w && scale && offsets, "grouped_w8a16_gemm: null argument");
+    MF_REQUIRE(y && x && w_packed && scale && offsets, "grouped_w8a16_gemm: null argument");
     MF_REQUIRE(n_experts > 0 && n_experts <= 65535 && total_rows >= 0 && n > 0 && k > 0,
                "grouped_w8a16_gemm: bad sizes");
-    MF_REQUIRE(k % 16 == 0, "grouped_w8a16_gemm: K (%d) must be a multiple of 16", k);
-    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "grouped_w8a16_gemm: x and w must be 16-byte aligned");
-    if (total_rows == 0) return 0;
+    MF_REQUIRE(k % 8 == 0, "grouped_w8a16_gemm: K (%d) must be a multiple of 8", k);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0,
+               "grouped_w8a16_gemm: x and w_packed must be 16-byte aligned");
+    const int64_t expert_bytes = (int64_t)mf_w8a16_packed_bytes(n, k);
     dim3 grid((n + GW_BN - 1) / GW_BN, n_experts);
-    if (dtype == MF_BF16)
-        hipLaunchKernelGGL(w8a16_grouped_kernel<BF16>, grid, dim3(GW_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
-                           (const uint16_t*)x, w, scale, offsets, total_rows, n, k);
-    else
-        hipLaunchKernelGGL(w8a16_grouped_kernel<FP16>, grid, dim3(GW_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
-                           (const uint16_t*)x, w, scale, offsets, total_rows, n, k);
+#define GG_LAUNCH(TT, KT)                                                                                        \
+    hipLaunchKernelGGL((w8a16_grouped_kernel<TT, KT>), grid, dim3(GW_WAVES * 64), 0, (hipStream_t)stream,           \
+                       (uint16_t*)y, (const uint16_t*)x, (const uint8_t*)w_packed, scale, offsets, total_rows, n, k, \
+                       expert_bytes)
+    const bool ktail = (k % GW_KSTEP) != 0;
+    if (dtype == MF_BF16) { if (ktail) GG_LAUNCH(BF16, true); else GG_LAUNCH(BF16, false); }
+    else { if (ktail) GG_LAUNCH(FP16, true); else GG_LAUNCH(FP16, false); }
+#undef GG_LAUNCH
     return MF_LAUNCH_CHECK();
 }

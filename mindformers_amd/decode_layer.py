@@ -33,6 +33,7 @@ class QuantDecodeLayer(nn.Module):
         self.hidden, self.n_head, self.n_kv_head, self.head_dim, self.ffn = hidden, n_head, n_kv_head, head_dim, ffn
         self.eps, self.dtype, self.act_quant = eps, dtype, act_quant
         self.scale_value = 1.0 / math.sqrt(head_dim)
+        self._packed = {}
         shapes = {"qkv": ((n_head + 2 * n_kv_head) * head_dim, hidden), "wo": (hidden, n_head * head_dim),
                   "fc1": (2 * ffn, hidden), "fc2": (hidden, ffn)}
         for name, (n, k) in shapes.items():
@@ -51,7 +52,17 @@ class QuantDecodeLayer(nn.Module):
         if self.act_quant:
             xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"))
             return ops.w8a8_linear(xq, xs, w, s, self.dtype, bias=b, residual=residual)
-        return ops.w8a16_linear(x, w, s, bias=b, residual=residual)
+        packed = self._packed.get(name)
+        if packed is None:
+            raise RuntimeError("call prepare() after loading the weights (packs them for the W8A16 kernels)")
+        return ops.w8a16_linear(x, packed, bias=b, residual=residual)
+
+    def prepare(self):
+        """Pack the int8 weights into the order the W8A16 kernels stream.  Call once after loading weights."""
+        if not self.act_quant:
+            for name in self.NAMES:
+                self._packed[name] = ops.pack_w8a16(getattr(self, f"{name}_w"), getattr(self, f"{name}_s"))
+        return self
 
     def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin):
         """x [T, hidden]; caches [num_blocks, block_size, n_kv, D]; cos/sin [T, D] rows for this step's

@@ -207,20 +207,54 @@ def add(a, b):
 
 
 # --------------------------------------------------------------------------------------------- quantized linear
-def w8a16_linear(x, w_i8, scale, bias=None, residual=None):
-    """WeightQuantBatchMatmul: y = (x . w_i8^T) * scale (+bias) (+residual).  x [..., K], w_i8 [N, K] int8."""
+class PackedInt8Weight:
+    """An int8 weight [N, K] (or a stack [E, N, K]) in the tiled order the W8A16 kernels stream, plus its
+    per-output-channel scales.  Built once with ``pack_w8a16`` after the weights are loaded."""
+
+    def __init__(self, packed, scale, n, k, experts=None):
+        self.packed, self.scale, self.n, self.k, self.experts = packed, scale, n, k, experts
+
+    @property
+    def shape(self):
+        return (self.n, self.k) if self.experts is None else (self.experts, self.n, self.k)
+
+
+def pack_w8a16(w_i8, scale):
+    """Pack int8 [N, K] or [E, N, K] (K contiguous) into kernel order.  scale fp32 [N] / [E, N]."""
     lib = _lib.load()
-    dev = _dev_ok(x, w_i8, scale, bias, residual)
-    _need(x.dtype in _ACT and w_i8.dtype == torch.int8 and scale.dtype == torch.float32, "dtypes: x bf16/fp16, w int8, scale fp32")
-    n, k = w_i8.shape
-    _need(x.shape[-1] == k and scale.numel() == n, "shape mismatch")
+    dev = _dev_ok(w_i8, scale)
+    _need(w_i8.dtype == torch.int8 and w_i8.dim() in (2, 3), "weight must be int8 [N, K] or [E, N, K]")
+    _need(scale.dtype == torch.float32, "scale must be fp32")
+    experts = w_i8.shape[0] if w_i8.dim() == 3 else None
+    n, k = w_i8.shape[-2:]
+    _need(scale.numel() == (experts or 1) * n, "scale must hold one value per output channel")
+    per = lib.mf_w8a16_packed_bytes(n, k)
+    packed = torch.empty((experts or 1) * per, dtype=torch.uint8, device=dev)
+    mats = w_i8 if experts is not None else w_i8[None]
+    for e in range(mats.shape[0]):
+        check(lib.mf_w8a16_pack_weight(packed.data_ptr() + e * per, ptr(mats[e]), n, k, stream_ptr(dev)),
+              "mf_w8a16_pack_weight")
+    return PackedInt8Weight(packed, scale.contiguous(), n, k, experts)
+
+
+def w8a16_linear(x, w, scale=None, bias=None, residual=None):
+    """WeightQuantBatchMatmul: y = (x . w_i8^T) * scale (+bias) (+residual).  x [..., K]; ``w`` is a
+    PackedInt8Weight (the fast path) or a raw int8 [N, K] tensor with ``scale`` (packed on every call)."""
+    lib = _lib.load()
+    if not isinstance(w, PackedInt8Weight):
+        w = pack_w8a16(w, scale)
+    _need(w.experts is None, "use grouped_w8a16_linear for stacked expert weights")
+    dev = _dev_ok(x, bias, residual)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    n, k = w.n, w.k
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
     m = x.numel() // k
     y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=dev)
     _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
     _need(residual is None or (residual.dtype == x.dtype and residual.shape == y.shape), "residual mismatch")
     need = lib.mf_w8a16_workspace_bytes(m, n, k)
     ws = workspace(need, dev, "gemm") if need else None
-    check(lib.mf_w8a16_gemm(ptr(y), ptr(x), ptr(w_i8), ptr(scale), ptr(bias), ptr(residual), m, n, k,
+    check(lib.mf_w8a16_gemm(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(residual), m, n, k,
                             dtype_code(x.dtype), ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
           "mf_w8a16_gemm")
     return y
@@ -295,16 +329,19 @@ def moe_permute(x, expert_index, n_experts):
     return px, row_map, counts, offsets
 
 
-def grouped_w8a16_linear(x, w_i8, scale, offsets):
-    """GroupedMatmulV4 over expert row groups.  x [R, K]; w_i8 [E, N, K]; scale [E, N]; offsets int32 [E+1]."""
+def grouped_w8a16_linear(x, w, offsets, scale=None):
+    """GroupedMatmulV4 over expert row groups.  x [R, K]; ``w`` a PackedInt8Weight of [E, N, K] (or a raw int8
+    [E, N, K] tensor with ``scale`` [E, N], packed on every call); offsets int32 [E+1]."""
     lib = _lib.load()
-    dev = _dev_ok(x, w_i8, scale, offsets)
-    _need(x.dtype in _ACT and x.dim() == 2 and w_i8.dtype == torch.int8 and w_i8.dim() == 3, "x [R,K] bf16/fp16, w [E,N,K] int8")
-    e, n, k = w_i8.shape
-    _need(x.shape[1] == k and scale.dtype == torch.float32 and scale.numel() == e * n, "shape mismatch")
+    if not isinstance(w, PackedInt8Weight):
+        w = pack_w8a16(w, scale)
+    _need(w.experts is not None, "grouped_w8a16_linear needs stacked expert weights [E, N, K]")
+    dev = _dev_ok(x, offsets)
+    e, n, k = w.experts, w.n, w.k
+    _need(x.dtype in _ACT and x.dim() == 2 and x.shape[1] == k, "x must be bf16/fp16 [R, K]")
     _need(offsets.dtype == torch.int32 and offsets.numel() == e + 1, "offsets must be int32 [E+1]")
     y = torch.empty(x.shape[0], n, dtype=x.dtype, device=dev)
-    check(lib.mf_grouped_w8a16_gemm(ptr(y), ptr(x), ptr(w_i8), ptr(scale), ptr(offsets), e, x.shape[0], n, k,
+    check(lib.mf_grouped_w8a16_gemm(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(offsets), e, x.shape[0], n, k,
                                     dtype_code(x.dtype), stream_ptr(dev)), "mf_grouped_w8a16_gemm")
     return y
 

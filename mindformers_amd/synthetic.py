@@ -58,7 +58,7 @@ def fill_layer(layer, gen, std=0.02):
             getattr(layer, f"{name}_smooth").copy_(torch.rand(k, generator=gen, device=dev) * 1.5 + 0.5)
     layer.attn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
     layer.ffn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
-    return layer
+    return layer.prepare()
 
 
 def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=None):

@@ -395,7 +395,7 @@ def test_moe_permute_grouped_unpermute():
     w1 = rng.normal(0, 0.05, (e, 2 * f, h)).astype(np.float32)       # [E, N, K]
     q1, s1 = zip(*(O.quantize_weight_int8(w1[i]) for i in range(e)))
     q1, s1 = np.stack(q1), np.stack(s1)
-    y1 = ops.grouped_w8a16_linear(px, torch.from_numpy(q1).cuda(), torch.from_numpy(s1).cuda(), offsets)
+    y1 = ops.grouped_w8a16_linear(px, torch.from_numpy(q1).cuda(), offsets, scale=torch.from_numpy(s1).cuda())
     deq1 = q1.astype(np.float64) * s1[..., None]                      # [E, N, K] -> oracle wants [E, in, out]
     ref1 = O.grouped_matmul(px_ref, np.transpose(deq1, (0, 2, 1)), cnt_ref)
     mag1 = O.grouped_matmul(np.abs(px_ref), np.abs(np.transpose(deq1, (0, 2, 1))), cnt_ref)
