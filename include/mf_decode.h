@@ -143,10 +143,12 @@ int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_sca
  * s = sigmoid(logits); sb = s + bias; per group score = sum of its two largest sb; keep the topk_group best
  * groups; top-k of sb over kept groups (ties: lower index); w = s[idx]; if renorm w /= sum(w); w *= scale.
  * logits fp32 [T,E]; bias fp32 [E] or NULL; weights_out in `dtype` [T,k]; index_out int32 [T,k].
- * E <= 1024, E % n_group == 0; n_group <= 1 or topk_group >= n_group disables group limiting. */
+ * E <= 1024, E % n_group == 0; n_group <= 1 or topk_group >= n_group disables group limiting.
+ * biased_weights != 0 returns w = sb[idx] instead (the plain top-k branch of router.py:142-146, which
+ * normalises the biased scores and applies no scale). */
 int mf_moe_route(void* weights_out, int32_t* index_out, const float* logits, const float* bias, int tokens,
-                 int n_experts, int k, int n_group, int topk_group, float scale, int renorm, int dtype,
-                 void* stream);
+                 int n_experts, int k, int n_group, int topk_group, float scale, int renorm, int biased_weights,
+                 int dtype, void* stream);
 
 /* MoeInitRoutingV2(x, expert_index, ..., expert_tokens_count_or_cumsum_flag=2) — moe_layer.py:136-146.
  * Stable counting sort of the (token, choice) pairs (flattened t*k + j) by expert.  permuted_x [T*k, H];

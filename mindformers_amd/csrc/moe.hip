@@ -14,7 +14,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ we
                                                       int32_t* __restrict__ index_out,
                                                       const float* __restrict__ logits,
                                                       const float* __restrict__ bias, int E, int k, int n_group,
-                                                      int topk_group, float scale, int renorm) {
+                                                      int topk_group, float scale, int renorm,
+                                                      int biased_weights) {
     __shared__ float s_plain[RT_MAX_E];     // sigmoid(logit)
     __shared__ float s_biased[RT_MAX_E];    // sigmoid(logit) + bias, later masked
     __shared__ float s_gscore[64];
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ we
             if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
         }
         if (bi >= E) bi = 0;                                  // all -inf/NaN rows: keep indices in range
-        const float wv = s_plain[bi];
+        const float wv = biased_weights ? best : s_plain[bi];
         wsum += wv;
         __syncthreads();
         if (lane == 0) {
@@ -203,7 +204,7 @@ __global__ void moe_unpermute_kernel(uint16_t* __restrict__ out, const uint16_t*
 
 extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* logits, const float* bias,
                             int tokens, int n_experts, int k, int n_group, int topk_group, float scale, int renorm,
-                            int dtype, void* stream) {
+                            int biased_weights, int dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "moe_route: dtype must be bf16 or fp16");
     if (tokens <= 0) return 0;
     MF_REQUIRE(weights_out && index_out && logits, "moe_route: null argument");
@@ -217,10 +218,10 @@ extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* 
     if (tokens <= 0) return 0;
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(moe_route_kernel<BF16>, dim3(tokens), dim3(64), 0, (hipStream_t)stream, (uint16_t*)weights_out,
-                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm);
+                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm, biased_weights);
     else
         hipLaunchKernelGGL(moe_route_kernel<FP16>, dim3(tokens), dim3(64), 0, (hipStream_t)stream, (uint16_t*)weights_out,
-                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm);
+                           index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm, biased_weights);
     return MF_LAUNCH_CHECK();
 }
 

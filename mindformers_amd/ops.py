@@ -296,7 +296,7 @@ def w8a8_linear(xq, x_scale, w_i8, w_scale, out_dtype, bias=None, residual=None,
 
 
 # --------------------------------------------------------------------------------------------- MoE
-def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, renorm=True):
+def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, renorm=True, biased_weights=False):
     """FusedAddTopKDiv: (expert_weight [T,k] out_dtype, expert_index [T,k] int32) from fp32 logits [T,E]."""
     lib = _lib.load()
     dev = _dev_ok(logits, expert_bias)
@@ -306,7 +306,8 @@ def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, ren
     w = torch.empty(t, k, dtype=out_dtype, device=dev)
     idx = torch.empty(t, k, dtype=torch.int32, device=dev)
     check(lib.mf_moe_route(ptr(w), ptr(idx), ptr(logits), ptr(expert_bias), t, e, k, int(n_group or 0),
-                           int(topk_group or 0), float(scale), 1 if renorm else 0, dtype_code(out_dtype),
+                           int(topk_group or 0), float(scale), 1 if renorm else 0, 1 if biased_weights else 0,
+                           dtype_code(out_dtype),
                            stream_ptr(dev)), "mf_moe_route")
     return w, idx
 

@@ -1,0 +1,240 @@
+"""CPU-only tests: the C-ABI library loads and exports what include/mf_decode.h declares, host-side logic
+(block tables, quantization configs and dispatch, rotary tables), and properties that pin the oracle beyond the
+reference's vectors (router brute force, quantisation grid, int32 exactness)."""
+import ctypes
+import itertools
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------------------------------- C ABI
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "mf_decode.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from mindformers_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from mindformers_amd import build
+        build.build(verbose=False)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared_functions()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in mf_decode.h but not exported"
+    # the ctypes table binds exactly the declared entry points
+    assert sorted(_lib.SIGNATURES) == declared
+    loaded = _lib.load()
+    assert loaded.mf_version().decode().startswith("mf_decode")
+    # size queries are pure host functions: callable without a GPU
+    assert loaded.mf_w8a16_packed_bytes(4096, 4096) == 4096 * 4096
+    assert loaded.mf_w8a16_packed_bytes(17, 1376) == 32 * 1408
+    assert loaded.mf_paged_attention_workspace_bytes(64, 32, 128, 256) == 0
+    assert loaded.mf_paged_attention_workspace_bytes(64, 32, 128, 4096) == 64 * 32 * 16 * 130 * 4
+    assert loaded.mf_w8a16_workspace_bytes(0, 10, 16) == 0
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    from mindformers_amd import _lib
+    lib = _lib.load()
+    rc = lib.mf_paged_attention_decode(None, None, None, None, None, None, 1, 32, 8, 100, 128, 4, 10, 0.1, 0, 0, None, 0, None)
+    assert rc == 1 and b"null" in lib.mf_last_error()
+    rc = lib.mf_w8a16_gemm(1, 1, 1, 1, None, None, 4, 8, 12, 0, None, 0, None)
+    assert rc == 1 and b"multiple of 8" in lib.mf_last_error()
+    with pytest.raises(_lib.MfKernelError):
+        _lib.check(rc, "mf_w8a16_gemm")
+
+
+def test_ops_refuse_cpu_tensors():
+    from mindformers_amd import ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.rms_norm(x, torch.ones(64), 1e-5)
+
+
+# ------------------------------------------------------------------------------------------- block tables
+def test_block_tables_match_naive_slot_mapping():
+    from mindformers_amd.modules import BlockTables
+    rng = np.random.default_rng(0)
+    bs, seq, batch = 16, 256, 5
+    bt = BlockTables(num_blocks=128, block_size=bs, seq_length=seq)
+    bt.init_cache_engine(batch)
+    lens = rng.integers(1, 100, batch)
+    tables, slots = bt.assemble_pa_full_inputs(int(lens.max()), lens, [False] * batch)
+    assert tables.shape == (batch, seq // bs) and tables.dtype == np.int32
+    ref = O.prefill_slot_mapping(tables, lens, bs, int(lens.max()))
+    assert np.array_equal(slots, ref)
+    # blocks are handed out first-fit from the free list (cache_engine.py:45-53)
+    used = tables[tables >= 0]
+    assert sorted(used.tolist()) == list(range(len(used)))
+    for step in range(40):                                # decode steps cross block boundaries
+        lens = lens + 1
+        tables, slots = bt.assemble_pa_inc_inputs(lens, [False] * batch)
+        assert np.array_equal(slots, O.decode_slot_mapping(tables, lens, bs))
+    bt.clear_cache()
+    assert len(bt.block_mem_pool.free_blocks) == 128
+    with pytest.raises(RuntimeError):
+        bt.block_mem_pool.allocate_block(129)
+    with pytest.raises(RuntimeError):
+        bt.block_mem_pool.free_block([3])
+
+
+# ------------------------------------------------------------------------------------------- quantization configs
+def test_auto_quantizer_dispatch():
+    """Mirrors tests/st/test_ut/test_models/test_auto/test_auto_quantizer.py:31-77 (dispatch and errors)."""
+    from mindformers_amd.modules.quantizers import (AutoQuantizationConfig, AutoQuantizer, PtqQuantizer, RtnQuantizer,
+                                                    SmoothQuantQuantizer)
+    from mindformers_amd.quantization_config import PtqConfig, RtnConfig, SmoothQuantConfig
+    with pytest.raises(ValueError):
+        AutoQuantizationConfig.from_dict({})
+    with pytest.raises(ValueError):
+        AutoQuantizationConfig.from_dict({"quant_method": "xxx"})
+    cfg = AutoQuantizationConfig.from_dict({"quant_method": "rtn", "weight_dtype": "int8", "modules_to_not_convert": ["lm_head"]})
+    assert isinstance(cfg, RtnConfig) and cfg.opname_blacklist == ["lm_head"]
+    assert isinstance(AutoQuantizer.from_config(cfg), RtnQuantizer)
+    assert isinstance(AutoQuantizer.from_config({"quant_method": "ptq"}), PtqQuantizer)
+    assert isinstance(AutoQuantizationConfig.from_dict({"quant_method": "ptq"}), PtqConfig)
+    sq = AutoQuantizer.from_config({"quant_method": "smooth_quant"})
+    assert isinstance(sq, SmoothQuantQuantizer) and isinstance(sq.quant_config, SmoothQuantConfig)
+
+
+def test_quantization_config_validation():
+    from mindformers_amd.quantization_config import PtqConfig, RtnConfig, SmoothQuantConfig
+    with pytest.raises(ValueError):                      # RTN is weight-only (quantization_config.py:281-286)
+        RtnConfig(activation_dtype="int8")
+    with pytest.raises(ValueError):
+        RtnConfig(outliers_suppression="smooth")
+    with pytest.raises(ValueError):
+        RtnConfig(mode="quantize")
+    with pytest.raises(ValueError):                      # per_token needs W8A8 (:438-442)
+        PtqConfig(weight_dtype="int8", activation_dtype=None, act_quant_granularity="per_token")
+    with pytest.raises(ValueError):
+        PtqConfig(weight_dtype=None, activation_dtype="int8")
+    with pytest.raises(ValueError):
+        PtqConfig(group_size=32)
+    with pytest.raises(TypeError):
+        PtqConfig(layer_policies={"(": {"quant_method": "ptq"}})
+    with pytest.raises(ValueError):                      # SmoothQuant is A8W8 per tensor only (:577-595)
+        SmoothQuantConfig(act_quant_granularity="per_token")
+    with pytest.raises(ValueError):
+        SmoothQuantConfig(activation_dtype=None)
+    ok = PtqConfig(weight_dtype="int8", activation_dtype="int8", act_quant_granularity="per_token",
+                   outliers_suppression="smooth", layer_policies={r".*wo": {"quant_method": "ptq"}})
+    assert ok.to_dict()["act_quant_granularity"] == "per_token" and list(ok.layer_policies) == [r".*wo"]
+
+
+def test_unbuilt_quant_modes_are_rejected_at_conversion():
+    from mindformers_amd.modules.quantizers.base import check_buildable
+    from mindformers_amd.quantization_config import PtqConfig, SmoothQuantConfig
+    with pytest.raises(NotImplementedError):
+        check_buildable(SmoothQuantConfig())             # per-tensor activations
+    with pytest.raises(NotImplementedError):
+        check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=64))
+    with pytest.raises(NotImplementedError):
+        check_buildable(PtqConfig(kvcache_dtype="int8"))
+    check_buildable(PtqConfig())
+
+
+# ------------------------------------------------------------------------------------------- rotary tables (host)
+def test_rotary_modules_build_the_oracle_tables():
+    from mindformers_amd.modules import FreqsMgr, Llama3RotaryEmbedding, RotaryEmbedding, YaRNScalingRotaryEmbedding
+    d = 32
+    r = RotaryEmbedding(d, rotary_cos_format=2, rotary_dtype=torch.bfloat16, max_position_embeddings=64, device="cpu")
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 64, 1.0, "bf16")
+    assert np.array_equal(r.cos_cache.float().numpy(), cos) and np.array_equal(r.sin_cache.float().numpy(), sin)
+    l3 = Llama3RotaryEmbedding(d, rotary_cos_format=2, rotary_dtype=torch.float32, max_position_embeddings=64,
+                               scaling_factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, orig_max_position=512, device="cpu")
+    cos, _ = O.rope_cos_sin_table(O.rope_inv_freq_llama3(d, 10000, 8.0, 1.0, 4.0, 512), 64, 1.0, "fp32")
+    assert np.allclose(l3.cos_cache.numpy(), cos, atol=1e-6)
+    y = YaRNScalingRotaryEmbedding(d, rotary_cos_format=2, rotary_dtype=torch.float32, scaling_factor=8.0,
+                                   original_max_position_embeddings=16, beta_fast=32, beta_slow=1, mscale=1.0,
+                                   mscale_all_dim=0.0, device="cpu")
+    assert y.cos_cache.shape == (128, d)
+    ms = O.yarn_mscale(8.0, 1.0) / O.yarn_mscale(8.0, 0.0)
+    cos, _ = O.rope_cos_sin_table(O.rope_inv_freq_yarn(d, 10000, 8.0, 16, 32, 1), 128, ms, "fp32")
+    assert np.allclose(y.cos_cache.numpy(), cos, atol=1e-6)
+    f = FreqsMgr(d, max_position_embedding=64, rotary_dtype=torch.float32, device="cpu")
+    c, s, _ = f.increment(torch.tensor([1, 5, 64]))
+    ref_c, ref_s = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 64, 1.0, "fp32")
+    assert np.allclose(c.numpy(), ref_c[[0, 4, 63]], atol=1e-6) and np.allclose(s.numpy(), ref_s[[0, 4, 63]], atol=1e-6)
+    with pytest.raises(NotImplementedError):
+        RotaryEmbedding(d, rotary_interleaved=True, device="cpu")
+    with pytest.raises(NotImplementedError):
+        RotaryEmbedding(d, seq_len_interpolation_factor=1.1, device="cpu")
+
+
+# ------------------------------------------------------------------------------------------- oracle properties
+def test_router_matches_brute_force_with_group_limit():
+    """The reference holds no vector with n_group > topk_group; pin the group-limited selection by exhaustive
+    search on small sizes: chosen set = top-k of the biased scores restricted to the best groups."""
+    rng = np.random.default_rng(5)
+    for e, ng, tg, k in ((8, 4, 2, 2), (12, 3, 1, 3), (16, 4, 3, 4)):
+        logits = rng.normal(size=(20, e)).astype(np.float32)
+        bias = rng.normal(0, 0.2, e).astype(np.float32)
+        w, idx = O.topk_router(logits, bias, k, ng, tg, 2.5)
+        s = 1 / (1 + np.exp(-logits.astype(np.float64)))
+        sb = s + bias
+        gs = e // ng
+        for t in range(20):
+            gscore = [np.sort(sb[t, g * gs:(g + 1) * gs])[-2:].sum() for g in range(ng)]
+            best_groups = set(np.argsort(gscore)[-tg:].tolist())
+            allowed = [i for i in range(e) if i // gs in best_groups]
+            best = max(itertools.combinations(allowed, k), key=lambda c: sb[t, list(c)].sum())
+            assert set(idx[t].tolist()) == set(best)
+            assert np.all(np.diff(sb[t, idx[t]]) <= 0)               # descending by biased score
+            ref_w = s[t, idx[t]] / s[t, idx[t]].sum() * 2.5
+            assert np.allclose(w[t], ref_w, rtol=1e-12)
+    # n_group == topk_group reduces to plain biased top-k
+    logits = rng.normal(size=(6, 16)).astype(np.float32)
+    _, a = O.topk_router(logits, None, 4, 4, 4, 1.0)
+    _, b = O.topk_router(logits, None, 4, 1, 1, 1.0)
+    assert np.array_equal(a, b)
+
+
+def test_quantisation_grid_properties():
+    rng = np.random.default_rng(6)
+    w = rng.normal(0, 0.02, (64, 256)).astype(np.float32)
+    q, s = O.quantize_weight_int8(w)
+    assert q.dtype == np.int8 and np.abs(q).max() == 127 and np.all(np.abs(q).max(axis=1) == 127)
+    assert np.abs(q.astype(np.float64) * s[:, None] - w).max() <= s.max() / 2 * (1 + 1e-6)
+    q2, s2 = O.quantize_weight_int8(q.astype(np.float32) * s[:, None])           # idempotent on its own grid
+    assert np.array_equal(q, q2)
+    x = rng.normal(size=(16, 256)).astype(np.float32)
+    xq, xs = O.dynamic_quant_per_token(x, rng.uniform(0.5, 2, 256).astype(np.float32))
+    assert np.all(np.abs(xq.astype(np.int32)).max(axis=1) == 127)
+    # rint: ties go to even
+    xq, _ = O.dynamic_quant_per_token(np.array([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5]], np.float32))
+    assert xq.tolist() == [[127, 0, 2, 2, 0, -2]]
+    # int32 accumulators are exact integer matmul, including the extreme corner
+    a = np.full((2, 512), -128, np.int8)
+    b = np.full((3, 512), -127, np.int8)
+    assert np.all(O.int8_gemm_i32(a, b) == 128 * 127 * 512)
+
+
+def test_moe_permute_is_a_stable_sort_and_unpermute_inverts_it():
+    rng = np.random.default_rng(7)
+    t, k, e, h = 9, 3, 5, 4
+    x = rng.normal(size=(t, h))
+    idx = rng.integers(0, e, (t, k)).astype(np.int32)
+    px, row_map, counts = O.moe_permute(x, idx, e)
+    flat = idx.reshape(-1)
+    assert counts.sum() == t * k and np.array_equal(counts, np.bincount(flat, minlength=e))
+    sorted_experts = np.empty(t * k, dtype=np.int64)
+    sorted_experts[row_map] = flat
+    assert np.all(np.diff(sorted_experts) >= 0)
+    for ex in range(e):                                   # stability: pair order preserved inside an expert
+        rows = row_map[flat == ex]
+        assert np.all(np.diff(rows) > 0)
+    assert np.array_equal(px[row_map], x[np.arange(t * k) // k])
+    ones = np.ones((t, k))
+    assert np.allclose(O.moe_unpermute(px, row_map, ones), k * x)

@@ -1,0 +1,436 @@
+"""The drop-in modules on the GPU, checked against the oracle and the reference's vectors.  GPU only.
+
+These read like the reference's own module tests (tests/st/test_infer/test_infer_module/*,
+tests/st/test_ut/test_parallel_core/test_inference/**): build the cell with the reference's arguments, feed the
+reference's inputs, compare the outputs.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import EPS, assert_within, dev, make_paged_cache, rounded, to_np
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    assert torch.cuda.is_available()
+    from mindformers_amd import _lib
+    _lib.load()
+    yield
+
+
+# ------------------------------------------------------------------------------------------- attention cells
+def test_paged_attention_mgr_surface():
+    """tests/st/test_infer/test_infer_module/test_paged_attention_mgr.py:28-60: all-ones inputs, shape check —
+    plus the values: with identical keys every probability is equal and the output is the mean of V = 1."""
+    from mindformers_amd.modules import PagedAttentionMgr
+    bsz, n_head, head_dim, n_kv, bs, nb = 1, 8, 128, 8, 16, 64
+    mgr = PagedAttentionMgr(n_head, head_dim, n_kv, (nb, bs, n_kv, head_dim), compute_dtype=torch.float16)
+    assert mgr.key_cache.shape == (nb, bs, n_kv, head_dim) and mgr.scale_value == 1 / np.sqrt(head_dim)
+    key = torch.ones(bsz, 1, n_kv * head_dim, dtype=torch.float16, device="cuda")
+    slot = torch.tensor([3], dtype=torch.int32, device="cuda")
+    out_k = mgr(key, key, slot)
+    assert out_k.shape == key.shape
+    q = torch.ones(bsz, 1, n_head * head_dim, dtype=torch.float16, device="cuda")
+    tables = torch.zeros(bsz, 4, dtype=torch.int32, device="cuda")
+    ctx = mgr.paged_attn(q, torch.tensor([4], dtype=torch.int32, device="cuda"), tables)
+    assert ctx.shape == (bsz, 1, n_head * head_dim)
+    # slots 0-2 are zeros, slot 3 holds ones: scores (0,0,0,sqrt(D)) -> weight of the ones row
+    wgt = np.exp(np.sqrt(head_dim)) / (3 + np.exp(np.sqrt(head_dim)))
+    assert np.allclose(to_np(ctx), wgt, rtol=2e-3)
+    with pytest.raises(NotImplementedError):
+        mgr.paged_attn_with_alibi(q, None, tables, None)
+    with pytest.raises(ValueError):
+        PagedAttentionMgr(8, 128, 8, (4, 16, 8))
+
+
+@pytest.mark.parametrize("dynamic", [True, False])
+def test_infer_attention_decode_step(dynamic):
+    """InferAttention decode call (test_infer_attention.py:179-274 calling convention: batch_valid_length counts
+    the new token, freqs_mgr.increment rows) against oracle RoPE -> scatter -> attention."""
+    from mindformers_amd.modules import BlockTables, FreqsMgr, InferAttention
+    rng = np.random.default_rng(3)
+    b, n_head, n_kv, d, bs, nb, seq = 4, 8, 2, 64, 16, 128, 512
+    dt = torch.float16
+    attn = InferAttention(n_head, d, n_kv, scale_value=1 / np.sqrt(d), block_size=bs, num_blocks=nb, seq_length=seq,
+                          is_dynamic=dynamic, rotary_cos_format=2, compute_dtype=dt)
+    assert attn.is_first_iteration and attn.paged_attention_mgr.key_cache.shape == (nb, bs, n_kv, d)
+    with pytest.raises(NotImplementedError):              # prefill is not on the built path
+        attn(None, None, None, None, None, None)
+    attn.is_first_iteration = False
+    mgr = BlockTables(nb, bs, seq)
+    mgr.init_cache_engine(b)
+    past = rng.integers(20, 200, b)
+    mgr.assemble_pa_full_inputs(int(past.max()), past, [False] * b)
+    # fill the cache with an earlier context
+    kc0 = rounded(rng.normal(size=(nb, bs, n_kv, d)), dt)
+    vc0 = rounded(rng.normal(size=(nb, bs, n_kv, d)), dt)
+    attn.paged_attention_mgr.key_cache.copy_(dev(kc0, dt))
+    attn.paged_attention_mgr.value_cache.copy_(dev(vc0, dt))
+    lens = past + 1
+    tables, slots = mgr.assemble_pa_inc_inputs(lens, [False] * b)
+    freqs = FreqsMgr(d, seq_length=seq, max_position_embedding=seq, rotary_dtype=dt)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    freqs_cis = freqs.increment(lens_t)
+    q = rounded(rng.normal(size=(b, n_head * d)), dt)
+    k = rounded(rng.normal(size=(b, n_kv * d)), dt)
+    v = rounded(rng.normal(size=(b, n_kv * d)), dt)
+    shape = (b, n_head * d) if dynamic else (b, 1, n_head * d)
+    out = attn(dev(q, dt).reshape(shape), dev(k, dt).reshape(b, -1) if dynamic else dev(k, dt).reshape(b, 1, -1),
+               dev(v, dt).reshape(b, -1) if dynamic else dev(v, dt).reshape(b, 1, -1), lens_t,
+               torch.from_numpy(tables).cuda(), torch.from_numpy(slots).cuda(), freqs_cis)
+    assert out.shape == shape
+    cos, sin = to_np(freqs_cis[0]), to_np(freqs_cis[1])
+    q_r = rounded(O.apply_rotary_half(q, cos, sin, n_head), dt)
+    k_r = rounded(O.apply_rotary_half(k, cos, sin, n_kv), dt)
+    O.reshape_and_cache(k_r, v, kc0, vc0, slots)
+    ref = O.paged_attention_decode(q_r, kc0, vc0, tables, lens, n_head, n_kv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q_r, kc0, np.abs(vc0), tables, lens, n_head, n_kv, 1 / np.sqrt(d))
+    # rotated q/k may differ from the oracle's by one rounding step: allow it on top of the attention tolerance
+    assert_within(to_np(out).reshape(b, -1), ref, mag, dt, ulps=4.0, what="InferAttention decode")
+    got_k = to_np(attn.paged_attention_mgr.key_cache).reshape(-1, n_kv * d)
+    assert np.abs(got_k[slots] - k_r).max() <= 2 * EPS[dt] * np.abs(k_r).max()
+    assert np.array_equal(to_np(attn.paged_attention_mgr.value_cache).reshape(-1, n_kv * d)[slots], v)
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_mcore_flash_attention_decode_vectors(golden_dir, case, n_kv):
+    """The reference's FlashAttention unit test, decode half (run_infer_flash_attention.py:150-180): caches are
+    passed per call, the cell scatters the new K/V and attends."""
+    from mindformers_amd import ops
+    from mindformers_amd.modules import FlashAttention
+    z = np.load(os.path.join(golden_dir, "flash_attention.npz"))
+    nb, bs, nh, hid = (int(z[k]) for k in ("meta_num_blocks", "meta_block_size", "meta_num_heads", "meta_hidden_size"))
+    d = hid // nh
+    net = FlashAttention(head_num=nh, head_dim=d, keep_prob=1.0, kv_head_num=n_kv, pa_kv_head_num=n_kv, scale_value=0.25)
+    kc = torch.zeros(nb, bs, n_kv, d, dtype=BF, device="cuda")
+    vc = torch.zeros_like(kc)
+    ops.reshape_and_cache(dev(z[f"in{case}_prefill_key"].reshape(4, -1), BF), dev(z[f"in{case}_prefill_value"].reshape(4, -1), BF),
+                          kc, vc, dev(z[f"in{case}_prefill_slot_mapping"].astype(np.int32), torch.int32))
+    with pytest.raises(NotImplementedError):
+        net(None, dev(z[f"in{case}_decoder_key"].reshape(2, -1), BF), dev(z[f"in{case}_decoder_value"].reshape(2, -1), BF),
+            slot_mapping=dev(z[f"in{case}_decoder_slot_mapping"].astype(np.int32), torch.int32), key_cache=kc, value_cache=vc)
+    net.is_prefill = False
+    bt = -np.ones((2, 11), np.int32)
+    bt[0, 0], bt[1, 0] = 2, 1
+    lens = torch.tensor([3, 3], dtype=torch.int32, device="cuda")
+    out = net(query=dev(z[f"in{case}_decoder_query"].reshape(2, -1), BF), key=dev(z[f"in{case}_decoder_key"].reshape(2, -1), BF),
+              value=dev(z[f"in{case}_decoder_value"].reshape(2, -1), BF),
+              slot_mapping=dev(z[f"in{case}_decoder_slot_mapping"].astype(np.int32), torch.int32),
+              block_tables=dev(bt, torch.int32), batch_valid_length=lens, context_lens_tensor=lens, key_cache=kc, value_cache=vc)
+    res = O.double_benchmark(to_np(out), z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"])
+    assert res.ok, res.messages
+
+
+@pytest.mark.parametrize("kind,phase", [("rope", "decode"), ("llama3_rope", "decode"), ("yarn_rope", "decode"), ("rope", "prefill")])
+def test_rotary_embedding_module_vectors(golden_dir, kind, phase):
+    from mindformers_amd.modules import Llama3RotaryEmbedding, RotaryEmbedding, YaRNScalingRotaryEmbedding
+    z = np.load(os.path.join(golden_dir, "rotary.npz"))
+    d, max_pos = int(z["meta_kv_channels"]), int(z["meta_max_position_embedding"])
+    common = dict(kv_channels=d, rotary_cos_format=2, rotary_dtype=BF)
+    if kind == "rope":
+        net = RotaryEmbedding(max_position_embeddings=max_pos, **common)
+    elif kind == "llama3_rope":
+        net = Llama3RotaryEmbedding(max_position_embeddings=max_pos, scaling_factor=8.0, low_freq_factor=1.0,
+                                    high_freq_factor=4.0, orig_max_position=512, **common)
+    else:
+        net = YaRNScalingRotaryEmbedding(scaling_factor=8.0, original_max_position_embeddings=512, beta_fast=32,
+                                         beta_slow=1, mscale=1.0, mscale_all_dim=0.0, **common)
+    if phase == "decode":
+        q, k = dev(z["in_decode_query_for_decode"], BF), dev(z["in_decode_key_for_decode"], BF)
+        cos, sin = net.get_cos_sin_for_decode(torch.ones(2, dtype=torch.int32, device="cuda"))
+    else:
+        q, k = dev(z["in_prefill_query_for_prefill"], BF), dev(z["in_prefill_key_for_prefill"], BF)
+        cos, sin = net.get_cos_sin_for_decode(torch.tensor([0, 1, 0, 1], dtype=torch.int32, device="cuda"))
+    q, k = net(q, k, cos, sin, None)
+    for got, name in ((q, "q"), (k, "k")):
+        res = O.double_benchmark(to_np(got), z[f"gpu_{kind}_{name}_emb1_for_{phase}"], z[f"golden_{kind}_{name}_emb1_for_{phase}"])
+        assert res.ok, (name, res.messages)
+
+
+# ------------------------------------------------------------------------------------------- linears / quantizers
+def _tiny_model():
+    from mindformers_amd.modules import Linear, LlamaRMSNorm
+    from torch import nn
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.wq = Linear(256, 512, has_bias=True, compute_dtype=BF, param_init_type=BF)
+            self.wo = Linear(512, 256, has_bias=False, compute_dtype=BF, param_init_type=BF)
+            self.norm = LlamaRMSNorm(256, eps=1e-5)
+            self.lm_head = Linear(256, 1000, has_bias=False, compute_dtype=BF, param_init_type=BF)
+
+        def forward(self, x):
+            return self.lm_head(self.wo(self.wq(self.norm(x))))
+    return Block()
+
+
+def test_column_parallel_linear_reference_vectors(golden_dir):
+    from mindformers_amd.modules import ColumnParallelLinear, RowParallelLinear
+    from mindformers_amd.transformer_config import TransformerConfig
+    cfg = TransformerConfig(hidden_size=32, num_attention_heads=2)
+    for kind, cls in (("column", ColumnParallelLinear), ("row", RowParallelLinear)):
+        z = np.load(os.path.join(golden_dir, f"{kind}_parallel_linear.npz"))
+        net = cls(32, 32, config=cfg, bias=True, compute_dtype=BF)
+        net.weight.data.copy_(dev(z["in_weight"], BF))
+        net.bias.data.copy_(dev(z["in_bias"], BF))
+        y = net(dev(z["in_inputs"], BF))
+        np.testing.assert_allclose(to_np(y), z["legacy_output_with_bias"], rtol=2 ** -7, atol=1e-6)
+    col = ColumnParallelLinear(32, 32, config=cfg, bias=True, skip_weight_param_allocation=True, compute_dtype=BF)
+    with pytest.raises(ValueError):
+        col(dev(z["in_inputs"], BF))
+
+
+@pytest.mark.parametrize("method", ["rtn", "ptq_w8a8"])
+def test_quantizer_swaps_cells_and_matches_oracle(method):
+    """build_network's hook (build_model.py:97-100): AutoQuantizer.from_config(cfg).preprocess_model(net), then
+    weights, then postprocess.  lm_head stays float (modules_to_not_convert)."""
+    from mindformers_amd.modules import AllQuantLinearInferCell, Linear, WeightQuantLinearCell
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    torch.manual_seed(0)
+    net = _tiny_model()
+    w_q, b_q, w_o = net.wq.weight.data.clone(), net.wq.bias.data.clone(), net.wo.weight.data.clone()
+    cfg = {"quant_method": "rtn", "weight_dtype": "int8", "modules_to_not_convert": ["lm_head"]} if method == "rtn" else \
+        {"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8", "act_quant_granularity": "per_token",
+         "outliers_suppression": "smooth", "modules_to_not_convert": ["lm_head"]}
+    quantizer = AutoQuantizer.from_config(cfg)
+    quantizer.preprocess_model(net)
+    assert net.is_quantized and net.quantization_method == cfg["quant_method"]
+    cell_t = WeightQuantLinearCell if method == "rtn" else AllQuantLinearInferCell
+    assert isinstance(net.wq, cell_t) and isinstance(net.wo, cell_t) and isinstance(net.lm_head, Linear)
+    assert net.wq.has_act_quant == (method != "rtn") and net.wq.layer.weight.dtype == torch.int8
+    quantizer.postprocess_model(net)
+    x = rounded(np.random.default_rng(1).normal(size=(7, 256)), BF)
+    y = net.wq(dev(x, BF))
+    wq_i8, s = O.quantize_weight_int8(w_q.float().cpu().numpy())
+    assert np.array_equal(to_np(net.wq.weight), wq_i8) and np.array_equal(to_np(net.wq.w_scale), s)
+    b = b_q.float().cpu().numpy()
+    if method == "rtn":
+        ref = O.w8a16_linear(x, wq_i8, s, b)
+    else:
+        xq, xs = O.dynamic_quant_per_token(x, np.ones(256, np.float32))
+        ref = O.w8a8_linear(xq, xs, wq_i8, s, b)
+    assert_within(to_np(y), ref, np.abs(ref) + np.abs(b), BF, ulps=1.0, extra=1e-5, what="quant cell")
+    out = net(dev(x, BF))
+    assert out.shape == (7, 1000) and torch.isfinite(out.float()).all()
+
+
+def test_smooth_quant_method_is_rejected_at_conversion():
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    q = AutoQuantizer.from_config({"quant_method": "smooth_quant"})
+    with pytest.raises(NotImplementedError):
+        q.preprocess_model(_tiny_model())
+
+
+# ------------------------------------------------------------------------------------------- norm / mlp
+def test_rmsnorm_cells(golden_dir):
+    from mindformers_amd.modules import LlamaRMSNorm, RMSNorm
+    from mindformers_amd.transformer_config import TransformerConfig
+    z = np.load(os.path.join(golden_dir, "norm.npz"))
+    cfg = TransformerConfig(hidden_size=32, layernorm_compute_dtype="bfloat16")
+    for name, eps in (("rmsnorm_output1", 1e-5), ("rmsnorm_output2", 0.1)):
+        for net in (RMSNorm(cfg, hidden_size=32, eps=eps), LlamaRMSNorm(32, eps=eps, compute_type=BF)):
+            net.weight.data.copy_(dev(z["in_weight"], BF))
+            res = O.double_benchmark(to_np(net(dev(z["in_input"], BF))), z[f"gpu_{name}"], z[f"golden_{name}"])
+            assert res.ok, (name, res.messages)
+
+
+@pytest.mark.parametrize("name,bias", [("has_bias_gate_output", True), ("has_gate_output", False)])
+def test_mcore_mlp_reference_vectors(golden_dir, name, bias):
+    """test_infer_mlp.py:35-61 gated cases through the float cells (library GEMM + HIP silu*mul)."""
+    from mindformers_amd.modules import MLP
+    from mindformers_amd.transformer_config import TransformerConfig
+    z = np.load(os.path.join(golden_dir, "mlp.npz"))
+    cfg = TransformerConfig(hidden_size=32, ffn_hidden_size=32, num_attention_heads=2, add_bias_linear=bias,
+                            gated_linear_unit=True, hidden_act="silu")
+    net = MLP(cfg)
+    net.linear_fc1.weight.data.copy_(dev(z["in_fc1_gate_weight"], BF))
+    net.linear_fc2.weight.data.copy_(dev(z["in_fc2_weight"], BF))
+    if bias:
+        net.linear_fc1.bias.data.copy_(dev(z["in_fc1_gate_bias"], BF))
+        net.linear_fc2.bias.data.copy_(dev(z["in_fc2_bias"], BF))
+    res = O.double_benchmark(to_np(net(dev(z["in_input"], BF))), z[f"gpu_{name}"], z[f"golden_{name}"])
+    assert res.ok, res.messages
+
+
+def test_llama_feed_forward_layouts():
+    """ffn_concat's interleaved (ffn, 2) layout and the separate w1/w3 layout give the same function."""
+    from mindformers_amd.modules import LlamaFeedForward
+    torch.manual_seed(1)
+    a = LlamaFeedForward(64, intermediate_size=96, compute_dtype=BF, param_init_type=BF, ffn_concat=False)
+    b = LlamaFeedForward(64, intermediate_size=96, compute_dtype=BF, param_init_type=BF, ffn_concat=True)
+    wgh = torch.empty(192, 64, dtype=BF, device="cuda")
+    wgh[0::2], wgh[1::2] = a.w1.weight.data, a.w3.weight.data
+    b.w_gate_hidden.weight.data.copy_(wgh)
+    b.w2.weight.data.copy_(a.w2.weight.data)
+    x = torch.randn(5, 64, device="cuda").to(BF)
+    assert torch.equal(a(x), b(x))
+    ref = O.mlp(to_np(x), np.concatenate([to_np(a.w1.weight), to_np(a.w3.weight)]), to_np(a.w2.weight), gated=True, act_dtype="bf16")
+    assert np.abs(to_np(a(x)) - ref).max() <= 4 * EPS[BF] * np.abs(ref).max() + 1e-6
+
+
+# ------------------------------------------------------------------------------------------- MoE layer
+def _moe_config(shared):
+    from mindformers_amd.transformer_config import TransformerConfig
+    return TransformerConfig(num_layers=1, num_attention_heads=8, hidden_size=32, hidden_act="silu", num_moe_experts=8,
+                             moe_router_topk=2, shared_expert_num=1, moe_router_topk_scaling_factor=2.5,
+                             moe_shared_expert_intermediate_size=8 if shared else 0, moe_ffn_hidden_size=8,
+                             moe_router_group_topk=2, moe_router_num_groups=2, add_bias_linear=False,
+                             gated_linear_unit=True, compute_dtype="bfloat16", params_dtype="bfloat16",
+                             moe_router_dtype="bfloat16", moe_router_enable_expert_bias=True,
+                             moe_router_score_function="sigmoid")
+
+
+def _load_moe(net, z, shared):
+    net.router.weight.data.copy_(dev(z["in_router__weight__weight"], BF))
+    net.router.expert_bias.data.copy_(dev(z["in_router__expert_bias"], torch.float32))
+    net.experts.weight1.data.copy_(dev(z["in_experts__weight1"], BF))
+    net.experts.weight2.data.copy_(dev(z["in_experts__weight2"], BF))
+    if shared:
+        net.shared_experts.linear_fc1.weight.data.copy_(dev(z["in_shared_experts__linear_fc1__weight"], BF))
+        net.shared_experts.linear_fc2.weight.data.copy_(dev(z["in_shared_experts__linear_fc2__weight"], BF))
+
+
+@pytest.mark.parametrize("name,shared", [("tp1", True), ("tp1_no_shared", False)])
+def test_moe_layer_reference_vectors(golden_dir, name, shared):
+    """test_infer_moe.py:31-58 through MoELayer with float experts: rtol 4e-3 (:132-140)."""
+    from mindformers_amd.modules import MoELayer
+    z = np.load(os.path.join(golden_dir, "moe.npz"))
+    net = MoELayer(_moe_config(shared))
+    assert (net.shared_experts is not None) == shared
+    _load_moe(net, z, shared)
+    out = net(dev(z["in_input"], BF))
+    got = to_np(out).astype(np.float16).astype(np.float32)
+    np.testing.assert_allclose(got, z[f"golden_{name}"], rtol=4e-3, atol=2e-6)
+
+
+def test_moe_layer_quantized_experts_vs_oracle(golden_dir):
+    """The same layer after the RTN quantizer (W8A16 experts, shared expert and all linears): compared with the
+    oracle evaluated on the dequantised weights, so only kernel arithmetic is in the tolerance."""
+    from mindformers_amd.modules import MoELayer, QuantGroupedMLP, WeightQuantLinearCell
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    z = np.load(os.path.join(golden_dir, "moe.npz"))
+    net = MoELayer(_moe_config(True))
+    _load_moe(net, z, True)
+    q = AutoQuantizer.from_config({"quant_method": "rtn", "weight_dtype": "int8"})
+    q.preprocess_model(net)
+    q.postprocess_model(net)
+    assert isinstance(net.experts, QuantGroupedMLP) and isinstance(net.shared_experts.linear_fc1, WeightQuantLinearCell)
+    x = rounded(z["in_input"], BF)
+    out = to_np(net(dev(x, BF)))
+    deq1 = (to_np(net.experts.weight1).astype(np.float64) * to_np(net.experts.w1_scale)[..., None]).transpose(0, 2, 1)
+    deq2 = (to_np(net.experts.weight2).astype(np.float64) * to_np(net.experts.w2_scale)[..., None]).transpose(0, 2, 1)
+    sf1 = to_np(net.shared_experts.linear_fc1.weight).astype(np.float64) * to_np(net.shared_experts.linear_fc1.w_scale)[:, None]
+    sf2 = to_np(net.shared_experts.linear_fc2.weight).astype(np.float64) * to_np(net.shared_experts.linear_fc2.w_scale)[:, None]
+    ref = O.moe_layer(x, rounded(z["in_router__weight__weight"], BF), z["in_router__expert_bias"].astype(np.float32), deq1, deq2,
+                      k=2, n_group=2, topk_group=2, scale=2.5, shared_fc1=sf1, shared_fc2=sf2, act_dtype="bf16",
+                      router_dtype="bf16")
+    assert np.abs(out - ref).max() <= 6 * EPS[BF] * np.abs(ref).max()
+
+
+def test_router_plain_topk_branch():
+    """moe_router_group_topk unset: biased scores are normalised and returned without scaling (router.py:142-146)."""
+    from mindformers_amd.modules import TopKRouter
+    from mindformers_amd.transformer_config import TransformerConfig
+    cfg = TransformerConfig(hidden_size=64, num_moe_experts=16, moe_router_topk=4, moe_router_dtype="float32",
+                            moe_router_enable_expert_bias=True)
+    r = TopKRouter(cfg)
+    r.expert_bias.data.normal_(0, 0.1)
+    x = torch.randn(9, 64, device="cuda").to(BF)
+    w, idx = r(x)
+    logits = to_np(x).astype(np.float64) @ to_np(r.weight).astype(np.float64).T
+    sb = 1 / (1 + np.exp(-logits)) + to_np(r.expert_bias)
+    ref_idx = np.argsort(-sb, axis=1, kind="stable")[:, :4]
+    assert np.array_equal(to_np(idx), ref_idx)
+    ref_w = np.take_along_axis(sb, ref_idx, 1)
+    ref_w /= ref_w.sum(1, keepdims=True)
+    assert np.abs(to_np(w) - ref_w).max() <= EPS[BF] * 1.01 * ref_w.max() + 1e-6
+
+
+# ------------------------------------------------------------------------------------------- whole layer
+@pytest.mark.parametrize("name", ["tiny_llama_w8a16"])
+def test_decode_layer_matches_oracle(name):
+    """The reference's CPU-runnable configuration, full layer, against the oracle composition."""
+    from mindformers_amd import synthetic
+    case = synthetic.make_decode_case(name, seed=3)
+    cfg, layer = case["cfg"], case["layers"][0]
+    kc, vc = case["caches"][0]
+    kc0, vc0 = to_np(kc), to_np(vc)
+    out = layer(case["x"], kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    p = {}
+    for n in layer.NAMES:
+        p[n + "_w"], p[n + "_s"] = to_np(getattr(layer, n + "_w")), to_np(getattr(layer, n + "_s"))
+    p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+    ref = O.decode_layer_w8a16(to_np(case["x"]), p, dict(n_head=cfg["n_head"], n_kv_head=cfg["n_kv_head"],
+                                                       head_dim=cfg["head_dim"], eps=1e-5), kc0, vc0,
+                               to_np(case["block_tables"]), case["context_lens_host"], to_np(case["slot_mapping"]),
+                               to_np(case["cos"]), to_np(case["sin"]), act_dtype="fp16")
+    got = to_np(out)
+    tol = 8 * EPS[torch.float16] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
+    assert np.all(np.abs(got - ref) <= tol), np.abs(got - ref).max()
+
+
+def test_decode_layer_w8a8_matches_oracle():
+    """Qwen2.5-shaped W8A8 layer at reduced width (heads 7q/1kv x 128, hidden 896, ffn 1024), batch 5."""
+    from mindformers_amd import synthetic
+    from mindformers_amd.decode_layer import QuantDecodeLayer
+    torch.manual_seed(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    layer = synthetic.fill_layer(QuantDecodeLayer(896, 7, 1, 128, 1024, 1e-5, BF, act_quant=True), gen)
+    rng = np.random.default_rng(9)
+    b, bs = 5, 128
+    lens = rng.integers(100, 700, b)
+    kc0, vc0, tables, nb = make_paged_cache(rng, b, lens, 1, 128, bs, BF)
+    kc, vc = dev(kc0, BF), dev(vc0, BF)
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    x = rounded(rng.normal(size=(b, 896)), BF)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    cos, sin = synthetic.rope_rows(lens_t - 1, 128, 1e6, BF, "cuda")
+    out = layer(dev(x, BF), kc, vc, torch.from_numpy(tables).cuda(), lens_t, torch.from_numpy(slots).cuda(), cos, sin)
+    p = {}
+    for n in layer.NAMES:
+        p[n + "_w"], p[n + "_s"] = to_np(getattr(layer, n + "_w")), to_np(getattr(layer, n + "_s"))
+        p[n + "_smooth"] = to_np(getattr(layer, n + "_smooth"))
+    p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+    ref = O.decode_layer_w8a8(x, p, dict(n_head=7, n_kv_head=1, head_dim=128, eps=1e-5), kc0, vc0, tables, lens, slots,
+                              to_np(cos), to_np(sin), act_dtype="bf16")
+    got = to_np(out)
+    # int8 activation grids amplify one-step differences of the bf16 intermediates: compare at row scale
+    tol = 16 * EPS[BF] * np.maximum(np.abs(ref), 0.1 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-3
+    frac_bad = np.mean(np.abs(got - ref) > tol)
+    assert frac_bad < 0.002, (frac_bad, np.abs(got - ref).max())
+
+
+def test_decode_layer_graph_replay_is_bit_identical():
+    """A captured HIP graph of the layer step must reproduce the eager result on every replay, with eager work
+    and synchronisations in between."""
+    from mindformers_amd import synthetic
+    case = synthetic.make_decode_case("tiny_llama_w8a16", seed=4)
+    layer = case["layers"][0]
+    kc, vc = case["caches"][0]
+    args = (case["x"], kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    eager = layer(*args).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            layer(*args)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = layer(*args)
+    for _ in range(4):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        layer(*args)
+        torch.cuda.synchronize()
