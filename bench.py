@@ -85,7 +85,7 @@ def kernel_breakdown(case, torch, ops, iters):
     return out
 
 
-def cpu_baseline(case, torch, sample_seqs, gpu_out):
+def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
     """Time the numpy restatement of the same layer on the host for ``sample_seqs`` sequences of the batch
     (compact copies of their KV blocks), and compare the GPU rows with it."""
     import oracle as O
@@ -125,15 +125,18 @@ def cpu_baseline(case, torch, sample_seqs, gpu_out):
         cores = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
     except Exception:
         cores = 1
-    t0 = time.perf_counter()
-    ref = fn(x, p, ocfg, kcn, vcn, t2, lens, slots2, cos, sin, act_dtype=act)
-    dt = time.perf_counter() - t0
+    passes, dt = 0, 0.0
+    while passes < 16 and dt < min_seconds:        # every pass rewrites the same cache slots with the same rows: identical work
+        t0 = time.perf_counter()
+        ref = fn(x, p, ocfg, kcn, vcn, t2, lens, slots2, cos, sin, act_dtype=act)
+        dt += time.perf_counter() - t0
+        passes += 1
     got = gpu_out[idx].float().cpu().numpy()
     err = float(np.abs(got - ref).max())
     scale = float(np.abs(ref).max())
-    return dict(value=len(idx) / dt, unit="tokens/s", cores=int(cores), kind="port",
-                sample=f"one layer step for {len(idx)} of the {cfg['batch']} sequences "
-                       f"({int(lens.sum())} context tokens), numpy float64, {dt:.1f} s"), dict(
+    return dict(value=len(idx) * passes / dt, unit="tokens/s", cores=int(cores), kind="port",
+                sample=f"{passes} passes of one layer step for {len(idx)} of the {cfg['batch']} sequences "
+                       f"({int(lens.sum())} context tokens), numpy float64, {dt:.1f} s in all"), dict(
         max_abs_err=err, ref_max_abs=scale, rows=len(idx))
 
 
@@ -145,7 +148,7 @@ def main():
     ap.add_argument("--workload", default="llama3_8b_w8a16")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
+    ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-iters", type=int, default=50)
     args = ap.parse_args()
     if args.gpus != 1:

@@ -128,11 +128,12 @@ class _QuantLinearBase(nn.Module):
     def quantize_from_float(self, weight, bias=None):
         """Round-to-nearest, symmetric per-output-channel int8 (what golden-stick's RoundToNearest produces
         offline).  weight float [out, in]."""
-        w = weight.detach().to(device=self.weight.device, dtype=torch.float32)
+        w = weight.detach().to(device=self.weight.device, dtype=torch.float64)
         if tuple(w.shape) != (self.out_channels, self.in_channels):
             raise ValueError(f"weight shape {tuple(w.shape)} != {(self.out_channels, self.in_channels)}")
-        scale = w.abs().amax(dim=1) / 127.0
-        safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+        # float64 quotient: the rounding to the int8 grid then does not depend on how a device divides in float32
+        scale = (w.abs().amax(dim=1) / 127.0).float()
+        safe = torch.where(scale > 0, scale, torch.ones_like(scale)).double()
         self.weight.copy_(torch.clamp(torch.round(w / safe[:, None]), -127, 127).to(torch.int8))
         self.w_scale.copy_(scale)
         if bias is not None and self.bias is not None:

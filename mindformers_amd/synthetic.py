@@ -27,11 +27,11 @@ CONFIGS = {
 
 def quantize_weight_int8(w):
     """Symmetric per-output-channel int8 of a float weight [out, in]: s = max|w|/127, q = clip(rint(w/s), +-127)."""
-    w = w.float()
-    scale = w.abs().amax(dim=1) / 127.0
-    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    w = w.double()
+    scale = (w.abs().amax(dim=1) / 127.0).float()
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale)).double()
     q = torch.clamp(torch.round(w / safe[:, None]), -127, 127).to(torch.int8)
-    return q, scale.float()
+    return q, scale
 
 
 def rope_rows(positions, head_dim, theta, dtype, device):

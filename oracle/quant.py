@@ -21,11 +21,11 @@ import numpy as np
 
 def quantize_weight_int8(weight):
     """Symmetric per-output-channel int8.  weight [out, in] -> (w_i8 [out, in] int8, scale [out] float32)."""
-    w = np.asarray(weight, dtype=np.float32)
+    w = np.asarray(weight, dtype=np.float32).astype(np.float64)
     amax = np.abs(w).max(axis=1)
-    scale = (amax / np.float32(127.0)).astype(np.float32)
-    safe = np.where(scale > 0, scale, np.float32(1.0))
-    q = np.clip(np.rint(w / safe[:, None]), -127, 127).astype(np.int8)
+    scale = (amax / 127.0).astype(np.float32)           # the stored scale is float32
+    safe = np.where(scale > 0, scale, np.float32(1.0)).astype(np.float64)
+    q = np.clip(np.rint(w / safe[:, None]), -127, 127).astype(np.int8)   # quotient in float64, ties to even
     return q, scale
 
 
