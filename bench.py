@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-iters", type=int, default=50)
+    ap.add_argument("--calibrate-counters", action="store_true",
+                    help="also launch add_kernel on 2 x 128 MiB inputs (reads 256 MiB, writes 128 MiB): the known-size "
+                         "kernel that hardware traffic counters of a profiler run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the decode path has no "
@@ -174,6 +177,13 @@ def main():
 
     out_eager = run_step(case)
     torch.cuda.synchronize()
+    if args.calibrate_counters:
+        ca = torch.ones(64 << 20, dtype=torch.bfloat16, device="cuda")
+        cb_ = torch.ones(64 << 20, dtype=torch.bfloat16, device="cuda")
+        for _ in range(3):
+            ops.add(ca, cb_)
+        torch.cuda.synchronize()
+        del ca, cb_
 
     use_graph = not args.no_graph
     graph = None
