@@ -85,6 +85,11 @@ def kernel_breakdown(case, torch, ops, iters):
     return out
 
 
+# (workload, algorithmic KV bytes) -> HBM bytes per attention launch (main kernel + partition reduce) read from
+# FETCH_SIZE / WRITE_SIZE: (289748.4 + 4902.5) KiB x 2.000 + (10126.9 + 512.0) KiB x 1.000
+MEASURED_TRAFFIC_BYTES = {("llama3_8b_w8a16", 589434880): int((294650.9 * 2.0 + 10638.9) * 1024)}
+
+
 def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
     """Time the numpy restatement of the same layer on the host for ``sample_seqs`` sequences of the batch
     (compact copies of their KV blocks), and compare the GPU rows with it."""
@@ -238,8 +243,11 @@ def main():
         attn()
     attn_ms, attn_med = time_events(attn, args.kernel_iters, torch)
     achieved = nbytes["kv"] / (attn_ms * 1e-3) / 1e9
+    # HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE of a profiler run of this command,
+    # scaled by a known-size kernel); only valid for the exact workload it was collected on
+    traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, nbytes["kv"]))
     roofline = dict(bound="hbm", kernel="paged_attention_kernel (+ partition reduce)", achieved=round(achieved, 1),
-                    peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                    peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
                     bytes_per_launch=nbytes["kv"], avg_launch_us=round(attn_ms * 1e3, 2))
     breakdown = kernel_breakdown(case, torch, ops, args.kernel_iters)
     layer_gbps = nbytes["total"] * n_layers / (ms_per_step * 1e-3) / 1e9
