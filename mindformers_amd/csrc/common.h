@@ -18,6 +18,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define MF_WAVE 64
+#define MF_MAX_DEVICES 64                 // per-device one-off kernel configuration flags
 
 // Host-side argument error: remember the message, return hipErrorInvalidValue.
 void mf_set_error(const char* fmt, ...);
