@@ -84,6 +84,18 @@ __device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dt)
     return dt == MF_BF16 ? BF16::to_float(b) : FP16::to_float(b);
 }
 
+// 8 consecutive entries of a float-like table (runtime dtype id) as floats; 16-byte aligned
+__device__ __forceinline__ void load8_as_float(const void* p, int64_t i, int dt, float* f) {
+    if (dt == MF_FP32) {
+        const f32x4 a = *(const f32x4*)((const float*)p + i), b = *(const f32x4*)((const float*)p + i + 4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { f[q] = a[q]; f[4 + q] = b[q]; }
+    } else {
+        const u32x4 v = *(const u32x4*)((const uint16_t*)p + i);
+        if (dt == MF_BF16) unpack8<BF16>(v, f); else unpack8<FP16>(v, f);
+    }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -40,17 +40,19 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restri
     __shared__ float red[ROW_THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
-    float v[ROW_MAX_VEC][8];
+    float v[ROW_MAX_VEC][8], gm[ROW_MAX_VEC][8];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < ROW_MAX_VEC; ++it) {
         const int c = threadIdx.x + it * ROW_THREADS;
         if (c < nvec) {
             u32x4 raw = *(const u32x4*)(x + row + 8 * c);
+            u32x4 rraw;
+            if (residual) rraw = *(const u32x4*)(residual + row + 8 * c);
+            load8_as_float(gamma, 8 * c, gamma_dtype, gm[it]);   // in flight together with the row, used after the sum
             unpack8<T>(raw, v[it]);
             if (residual) {
                 float rr[8];
-                u32x4 rraw = *(const u32x4*)(residual + row + 8 * c);
                 unpack8<T>(rraw, rr);
                 u32x4 s;
 #pragma unroll
@@ -70,11 +72,8 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restri
         if (c < nvec) {
             u32x4 o;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float g0 = load_as_float(gamma, 8 * c + 2 * i, gamma_dtype);
-                const float g1 = load_as_float(gamma, 8 * c + 2 * i + 1, gamma_dtype);
-                o[i] = pack2<T>(v[it][2 * i] * inv * g0, v[it][2 * i + 1] * inv * g1);
-            }
+            for (int i = 0; i < 4; ++i)
+                o[i] = pack2<T>(v[it][2 * i] * inv * gm[it][2 * i], v[it][2 * i + 1] * inv * gm[it][2 * i + 1]);
             *(u32x4*)(y + row + 8 * c) = o;
         }
     }
@@ -197,7 +196,7 @@ extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* res
     MF_REQUIRE(!residual || sum_out, "rmsnorm: residual given without sum_out");
     MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * ROW_MAX_VEC * 8,
                "rmsnorm: cols (%d) must be a multiple of 8 and at most %d", cols, ROW_THREADS * ROW_MAX_VEC * 8);
-    MF_REQUIRE((((uintptr_t)y | (uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out) & 15) == 0,
+    MF_REQUIRE((((uintptr_t)y | (uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out | (uintptr_t)gamma) & 15) == 0,
                "rmsnorm: pointers must be 16-byte aligned");
     if (rows <= 0) return 0;
     if (dtype == MF_BF16)

@@ -89,6 +89,60 @@ __global__ void rope_and_cache_kernel(uint16_t* __restrict__ q, uint16_t* __rest
     }
 }
 
+// Vector form of the fused rotate-and-scatter for head_dim % 16 == 0: one work item = 8 consecutive elements
+// of the first half of a head together with their partners in the second half (16-byte accesses), or one
+// 16-byte piece of the value row.  grid = (tokens, ceil(items / 256)).
+template <typename T>
+__global__ __launch_bounds__(256) void rope_and_cache_vec_kernel(
+    uint16_t* __restrict__ q, uint16_t* __restrict__ k, const uint16_t* __restrict__ v, const void* __restrict__ cos,
+    const void* __restrict__ sin, uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache,
+    const int32_t* __restrict__ slot_mapping, int n_heads, int n_kv, int D, int64_t num_slots, int table_dtype,
+    int64_t q_stride, int64_t k_stride, int64_t v_stride) {
+    const int t = blockIdx.x;
+    const int half = D >> 1;
+    const int cph = half >> 3;                                // rotate items per head
+    const int rot_items = (n_heads + n_kv) * cph;
+    const int v_items = n_kv * D / 8;
+    const int item = blockIdx.y * 256 + threadIdx.x;
+    if (item >= rot_items + v_items) return;
+    const int64_t slot = slot_mapping[t];
+    const bool live = slot >= 0 && slot < num_slots;
+    const int64_t row = (int64_t)n_kv * D;
+    if (item >= rot_items) {
+        if (live) {
+            const int i = (item - rot_items) * 8;
+            *(u32x4*)(value_cache + slot * row + i) = *(const u32x4*)(v + (int64_t)t * v_stride + i);
+        }
+        return;
+    }
+    const int h = item / cph, i = (item - h * cph) * 8;
+    const bool is_k = h >= n_heads;
+    uint16_t* xr = is_k ? k + (int64_t)t * k_stride + (h - n_heads) * D : q + (int64_t)t * q_stride + h * D;
+    float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8];
+    unpack8<T>(*(const u32x4*)(xr + i), x1);
+    unpack8<T>(*(const u32x4*)(xr + i + half), x2);
+    const int64_t trow = (int64_t)t * D;
+    load8_as_float(cos, trow + i, table_dtype, c1);
+    load8_as_float(sin, trow + i, table_dtype, s1);
+    load8_as_float(cos, trow + i + half, table_dtype, c2);
+    load8_as_float(sin, trow + i + half, table_dtype, s2);
+    u32x4 o1, o2;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        o1[e] = pack2<T>(x1[2 * e] * c1[2 * e] - x2[2 * e] * s1[2 * e],
+                         x1[2 * e + 1] * c1[2 * e + 1] - x2[2 * e + 1] * s1[2 * e + 1]);
+        o2[e] = pack2<T>(x2[2 * e] * c2[2 * e] + x1[2 * e] * s2[2 * e],
+                         x2[2 * e + 1] * c2[2 * e + 1] + x1[2 * e + 1] * s2[2 * e + 1]);
+    }
+    *(u32x4*)(xr + i) = o1;
+    *(u32x4*)(xr + i + half) = o2;
+    if (is_k && live) {
+        uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
+        *(u32x4*)(dst + i) = o1;
+        *(u32x4*)(dst + i + half) = o2;
+    }
+}
+
 }  // namespace
 
 extern "C" int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
@@ -164,6 +218,24 @@ extern "C" int mf_rope_and_cache(void* query, void* key, const void* value, cons
                "rope_and_cache: row stride smaller than a row");
     const int vec_ok = (kv_row % 8 == 0) && (v_row_stride % 8 == 0) &&
                        (((uintptr_t)value | (uintptr_t)value_cache) % 16 == 0);
+    const bool all_vec = vec_ok && head_dim % 16 == 0 && q_row_stride % 8 == 0 && k_row_stride % 8 == 0 &&
+                         (((uintptr_t)query | (uintptr_t)key | (uintptr_t)key_cache | (uintptr_t)cos |
+                           (uintptr_t)sin) % 16 == 0);
+    if (all_vec) {
+        const int items = (n_heads + n_kv_heads) * (head_dim / 16) + n_kv_heads * head_dim / 8;
+        dim3 grid(num_tokens, (items + 255) / 256);
+        if (dtype == MF_BF16)
+            hipLaunchKernelGGL(rope_and_cache_vec_kernel<BF16>, grid, dim3(256), 0, (hipStream_t)stream,
+                               (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin,
+                               (uint16_t*)key_cache, (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads,
+                               head_dim, num_slots, table_dtype, q_row_stride, k_row_stride, v_row_stride);
+        else
+            hipLaunchKernelGGL(rope_and_cache_vec_kernel<FP16>, grid, dim3(256), 0, (hipStream_t)stream,
+                               (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin,
+                               (uint16_t*)key_cache, (uint16_t*)value_cache, slot_mapping, n_heads, n_kv_heads,
+                               head_dim, num_slots, table_dtype, q_row_stride, k_row_stride, v_row_stride);
+        return MF_LAUNCH_CHECK();
+    }
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(rope_and_cache_kernel<BF16>, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream,
                            (uint16_t*)query, (uint16_t*)key, (const uint16_t*)value, cos, sin, (uint16_t*)key_cache,
