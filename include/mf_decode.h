@@ -130,11 +130,14 @@ int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const 
 
 /* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
  * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
- * If acc_out != NULL the raw int32 accumulators are also written ([M,N] row-major); y may then be NULL.
- * K % 16 == 0. */
-int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const int8_t* w,
+ * xq int8 [M,K] row-major (what mf_dynamic_quant_per_token writes); w_packed = mf_w8a16_pack_weight of the int8
+ * [N,K] weight (the same tile order serves the int8 matrix cores).  If acc_out != NULL the raw int32 accumulators
+ * are also written ([M,N] row-major); y may then be NULL.  K % 16 == 0.  workspace: mf_w8a8_workspace_bytes
+ * bytes (int32 partial sums when K is split across workgroups; 0 for wide N). */
+size_t mf_w8a8_workspace_bytes(int m, int n, int k);
+int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,
                  const float* w_scale, const void* bias, const void* residual, int m, int n, int k, int dtype,
-                 void* stream);
+                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- mixture of experts --------------------------------------------------------------------------- */
 

@@ -2,140 +2,365 @@
 // (v_mfma_i32_16x16x64_i8), exact int32 accumulation, dequantised to bf16/fp16 in the epilogue:
 //   y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]).
 //
-// Both operands are K-contiguous ([M,K] and [N,K]), which is exactly the MFMA operand layout
-// (lane = row, 16 consecutive k bytes), so tiles go global -> LDS -> registers with 16-byte accesses and no
-// transposition.  A workgroup of 4 waves owns a 128 x 128 output tile; each wave a 64 x 64 quadrant
-// (4 x 4 MFMA tiles, 64 accumulator registers).  K is walked in 64-byte steps, double-buffered in LDS.
+// Weights come in the packed tile order of mf_w8a16_pack_weight (1 KiB tiles of 16 output channels x 64 input
+// channels, bytes in lane order): 16 consecutive k bytes per lane is the int8 MFMA operand layout as well, so a
+// tile is one coalesced wave-wide load and needs no shuffle.  Activations are the row-major int8 [M, K] that
+// mf_dynamic_quant_per_token writes.
+//
+// A workgroup of 4 waves owns BM x BN outputs and walks K in 64-byte steps.  Both operand tiles of a step go
+// global -> LDS with LDS-direct loads (no registers in between), two steps ahead of their use, into a ring of
+// three stages; one barrier per step.  Every wave issues the same number of loads per step and they complete in
+// issue order, so "at most one step's loads outstanding" means this wave's part of the current step has landed.
+// The LDS reads and their waits are asm statements (the compiler would wait for every LDS-direct load before any
+// LDS read); each wait names the registers it makes valid.
+//   M > 64:  waves split the rows (64 each, BM = 256), every wave multiplies its 4 row tiles with all NT weight
+//            tiles of the step (BN = 16*NT): 4 + NT operand reads feed 4*NT matrix instructions.
+//   M <= 64: one row block, waves split the channels (BN = 64*NT).
+// The 64-byte activation rows are XOR-swizzled in LDS (16-byte chunk c of row r sits at chunk c ^ 2*[r & 8]),
+// applied on the global-address side, which makes the operand reads bank-conflict free.
+// Small N cannot fill the chip with output tiles alone: K is then split across workgroups, which write exact
+// int32 partial tiles that a second kernel sums (integer sums do not depend on the order).
 #include "common.h"
 
 namespace {
 
-constexpr int Q_BM = 128, Q_BN = 128, Q_BK = 64;
-constexpr int Q_ROW = Q_BK + 16;   // LDS row pitch in bytes (80): 16-byte aligned, spreads rows over banks
+constexpr int Q_KSTEP = 64;
+constexpr int Q_TILE = 16 * Q_KSTEP;        // bytes of one packed weight tile
+constexpr int Q_STAGES = 3;
 
+template <int NT, bool MSPLIT>
+struct Q2 {
+    static constexpr int WAVES_M = MSPLIT ? 4 : 1;
+    static constexpr int WAVES_N = MSPLIT ? 1 : 4;
+    static constexpr int BM = 64 * WAVES_M;
+    static constexpr int BN = 16 * NT * WAVES_N;
+    static constexpr int XTILE = BM * Q_KSTEP;
+    static constexpr int WTILES = BN / 16;
+    static constexpr int STAGE = XTILE + WTILES * Q_TILE;
+    static constexpr int XL = BM / 64;                        // activation loads (16 rows each) per wave per stage
+    static constexpr int WL = (WTILES + 3) / 4;               // weight tile loads per wave per stage
+    static constexpr int PENDING = (Q_STAGES - 2) * (XL + WL);
+    static_assert(Q_STAGES * STAGE <= 65536, "ring exceeds static LDS");
+};
+
+__device__ __forceinline__ int q2_swizzle_key(int row) { return ((row >> 3) & 1) << 1; }
+
+template <int OFFSET>
+__device__ __forceinline__ i32x4 q2_lds_read16(uint32_t addr) {
+    i32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFFSET) : "memory");
+    return v;
+}
+__device__ __forceinline__ void q2_lds_direct16(const uint8_t* base_uniform, uint32_t lane_offset,
+                                                uint8_t* dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base_uniform + lane_offset),
+                                     (__attribute__((address_space(3))) void*)dst_wave_uniform, 16, 0, 0);
+}
+
+// Dequantising store of 4 consecutive channels of one row.
 template <typename T>
-__global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(uint16_t* __restrict__ y, int32_t* __restrict__ acc_out,
-                                                          const int8_t* __restrict__ xq,
-                                                          const float* __restrict__ x_scale,
-                                                          const int8_t* __restrict__ w,
-                                                          const float* __restrict__ w_scale,
-                                                          const uint16_t* __restrict__ bias,
-                                                          const uint16_t* __restrict__ residual, int M, int N,
-                                                          int K) {
-    __shared__ __attribute__((aligned(16))) uint8_t sA[2][Q_BM * Q_ROW];
-    __shared__ __attribute__((aligned(16))) uint8_t sB[2][Q_BN * Q_ROW];
-
-    const int tid = threadIdx.x;
-    const int wv = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
-    const int wm = wv >> 1, wn = wv & 1;                      // wave quadrant
-    const int m0 = blockIdx.y * Q_BM, n0 = blockIdx.x * Q_BN;
-
-    // cooperative tile load: 128 rows x 64 B = 512 chunks of 16 B per operand, 2 per thread
-    const int lrow = tid >> 2, lchunk = tid & 3;              // rows lrow and lrow + 64
-    const int8_t* ga[2];
-    const int8_t* gb[2];
-    bool oka[2], okb[2];
+__device__ __forceinline__ void q2_store4(uint16_t* y, int32_t* acc_out, const float* x_scale, const float* w_scale,
+                                          const uint16_t* bias, const uint16_t* residual, int m, int n, int N,
+                                          i32x4 a) {
+    const int64_t o = (int64_t)m * N + n;
+    const bool vec = n + 3 < N && (N & 3) == 0;
+    if (acc_out) {
+        if (vec) {
+            *(i32x4*)(acc_out + o) = a;
+        } else {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int am = m0 + lrow + 64 * h, bn = n0 + lrow + 64 * h;
-        oka[h] = am < M;
-        okb[h] = bn < N;
-        ga[h] = xq + (int64_t)(oka[h] ? am : 0) * K + 16 * lchunk;
-        gb[h] = w + (int64_t)(okb[h] ? bn : 0) * K + 16 * lchunk;
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) acc_out[o + i] = a[i];
+        }
     }
-
-    i32x4 acc[4][4];
+    if (!y) return;
+    const float xs = x_scale[m];
+    float v[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = (i32x4){0, 0, 0, 0};
-
-    const int steps = (K + Q_BK - 1) / Q_BK;
-    u32x4 ra[2], rb[2];
-    auto gload = [&](int s) {
-        const int kb = s * Q_BK;
-        const bool kok = kb + 16 * lchunk < K;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            ra[h] = (u32x4){0u, 0u, 0u, 0u};
-            rb[h] = (u32x4){0u, 0u, 0u, 0u};
-            if (kok && oka[h]) ra[h] = *(const u32x4*)(ga[h] + kb);
-            if (kok && okb[h]) rb[h] = *(const u32x4*)(gb[h] + kb);
+    for (int i = 0; i < 4; ++i) {
+        v[i] = 0.f;
+        if (n + i < N) {
+            float t = (float)a[i] * xs * w_scale[n + i];
+            if (bias) t += T::to_float(bias[n + i]);
+            if (residual) t = T::to_float(T::from_float(t)) + T::to_float(residual[o + i]);
+            v[i] = t;
         }
-    };
-    auto sstore = [&](int buf) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            *(u32x4*)(sA[buf] + (lrow + 64 * h) * Q_ROW + 16 * lchunk) = ra[h];
-            *(u32x4*)(sB[buf] + (lrow + 64 * h) * Q_ROW + 16 * lchunk) = rb[h];
-        }
-    };
-
-    gload(0);
-    sstore(0);
-    __syncthreads();
-    for (int s = 0; s < steps; ++s) {
-        const int buf = s & 1;
-        if (s + 1 < steps) gload(s + 1);
-        i32x4 fa[4], fb[4];
+    }
+    if (vec) {
+        *(u32x2*)(y + o) = (u32x2){pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+    } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            fa[i] = *(const i32x4*)(sA[buf] + (wm * 64 + i * 16 + r) * Q_ROW + 16 * g);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            fb[j] = *(const i32x4*)(sB[buf] + (wn * 64 + j * 16 + r) * Q_ROW + 16 * g);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-        if (s + 1 < steps) sstore(buf ^ 1);
-        __syncthreads();
+            if (n + i < N) y[o + i] = T::from_float(v[i]);
     }
+}
 
-    // ---- epilogue: acc[i][j][e] is row m = 4g + e of tile i, column n = r of tile j
+// grid = (n_blocks, split_k, m_blocks)
+template <typename T, int NT, bool MSPLIT, bool KTAIL>
+__global__ __launch_bounds__(256) void w8a8_gemm_kernel(
+    uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
+    const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
+    const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, int M,
+    int N, int K, int steps_per_split) {
+    using C = Q2<NT, MSPLIT>;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Q_STAGES * C::STAGE];
+
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int wm = MSPLIT ? wv : 0, wn = MSPLIT ? 0 : wv;
+    const int KS = (K + Q_KSTEP - 1) / Q_KSTEP;
+    const int s_begin = blockIdx.y * steps_per_split;
+    const int s_end = min(KS, s_begin + steps_per_split);
+    const int s_last = s_end - 1;
+    const int m0 = blockIdx.z * C::BM;
+    const int nb = blockIdx.x * C::BN;                        // first channel of the workgroup
+    const int nw = nb + wn * 16 * NT;                         // first channel this wave computes
+
+    i32x4 acc[NT][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int m = m0 + wm * 64 + i * 16 + 4 * g + e;
-            if (m >= M) continue;
-            const float xs = x_scale[m];
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = (i32x4){0, 0, 0, 0};
+
+    // activation loads: load i of this wave covers rows 16*(wv*XL + i) .. + 15 of the stage, 4 lanes per 64-byte
+    // row; lane -> (row, physical chunk), the global address uses the logical chunk.  Rows past M re-read row M-1.
+    const uint8_t* xbase = (const uint8_t*)xq + (int64_t)m0 * K;
+    uint32_t xlane[C::XL];
+    int xchunk[C::XL];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = n0 + wn * 64 + j * 16 + r;
-                if (n >= N) continue;
-                const int a = acc[i][j][e];
-                const int64_t o = (int64_t)m * N + n;
-                if (acc_out) acc_out[o] = a;
-                if (y) {
-                    float v = (float)a * xs * w_scale[n];
-                    if (bias) v += T::to_float(bias[n]);
-                    if (residual) v = T::to_float(T::from_float(v)) + T::to_float(residual[o]);
-                    y[o] = T::from_float(v);
+    for (int i = 0; i < C::XL; ++i) {
+        const int row = 16 * (wv * C::XL + i) + (lane >> 2);
+        xchunk[i] = 16 * ((lane & 3) ^ q2_swizzle_key(row));
+        xlane[i] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K + xchunk[i];
+    }
+    // weight loads: tile j of the stage is n-tile nb/16 + j; this wave loads tiles wv*WL + i (clamped: a wave with
+    // fewer tiles re-loads the last one onto itself, so that all waves issue the same number of loads)
+    const int n_tiles_total = (N + 15) >> 4;
+    const uint8_t* wtile[C::WL];
+    int wdst[C::WL];
+#pragma unroll
+    for (int i = 0; i < C::WL; ++i) {
+        const int j = min(wv * C::WL + i, C::WTILES - 1);
+        const int t = min((nb >> 4) + j, n_tiles_total - 1);
+        wtile[i] = wp + (int64_t)t * KS * Q_TILE;
+        wdst[i] = C::XTILE + j * Q_TILE;
+    }
+    const uint32_t wlane = lane * 16;
+
+    auto issue = [&](int stage, int s) {
+        const int sc = min(s, s_last);
+        uint8_t* dst = smem + stage * C::STAGE;
+#pragma unroll
+        for (int i = 0; i < C::XL; ++i) {
+            uint32_t off = xlane[i] + (uint32_t)sc * Q_KSTEP;
+            if (KTAIL) {
+                // chunks past K (last, short step) re-read the row's last whole chunk; they meet zero weights
+                const int over = sc * Q_KSTEP + xchunk[i] - (K - 16);
+                off -= over > 0 ? (uint32_t)over : 0u;
+            }
+            q2_lds_direct16(xbase, off, dst + 1024 * (wv * C::XL + i));
+        }
+#pragma unroll
+        for (int i = 0; i < C::WL; ++i)
+            q2_lds_direct16(wtile[i] + (int64_t)sc * Q_TILE, wlane, dst + wdst[i]);
+    };
+    issue(0, s_begin);
+    issue(1, s_begin + 1);
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+    // operand reads: activation tile mt = row 64*wm + 16*mt + r, logical chunk g; weight tile = lane-linear
+    const uint32_t xoff = lds0 + (64 * wm + r) * Q_KSTEP + ((g ^ q2_swizzle_key(r)) << 4);
+    const uint32_t woff = lds0 + C::XTILE + wn * NT * Q_TILE + lane * 16;
+
+    auto step = [&](auto jc, int s) {
+        constexpr int J = decltype(jc)::value;
+        constexpr int SB = J * C::STAGE;
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::PENDING) : "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue((J + 2) % Q_STAGES, s + 2);
+        i32x4 xb[4], wa[NT];
+        xb[0] = q2_lds_read16<SB>(xoff);
+        xb[1] = q2_lds_read16<SB + 1024>(xoff);
+        xb[2] = q2_lds_read16<SB + 2048>(xoff);
+        xb[3] = q2_lds_read16<SB + 3072>(xoff);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (nt == 0) wa[0] = q2_lds_read16<SB>(woff);
+            if (nt == 1) wa[1] = q2_lds_read16<SB + 1 * Q_TILE>(woff);
+            if (nt == 2) wa[2] = q2_lds_read16<SB + 2 * Q_TILE>(woff);
+            if (nt == 3) wa[3] = q2_lds_read16<SB + 3 * Q_TILE>(woff);
+            if (nt == 4) wa[4] = q2_lds_read16<SB + 4 * Q_TILE>(woff);
+            if (nt == 5) wa[5] = q2_lds_read16<SB + 5 * Q_TILE>(woff);
+            if (nt == 6) wa[6] = q2_lds_read16<SB + 6 * Q_TILE>(woff);
+            if (nt == 7) wa[7] = q2_lds_read16<SB + 7 * Q_TILE>(woff);
+        }
+        // the reads return in order: the activation tiles and the first weight tile are enough to start
+        asm volatile("s_waitcnt lgkmcnt(%5)"
+                     : "+v"(xb[0]), "+v"(xb[1]), "+v"(xb[2]), "+v"(xb[3]), "+v"(wa[0])
+                     : "n"(NT - 1)
+                     : "memory");
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (nt == 1) {                                    // the remaining weight tiles have arrived
+                if constexpr (NT == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[1])::"memory");
+                if constexpr (NT == 4)
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3])::"memory");
+                if constexpr (NT == 5)
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4])::"memory");
+                if constexpr (NT == 8)
+                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                 : "+v"(wa[1]), "+v"(wa[2]), "+v"(wa[3]), "+v"(wa[4]), "+v"(wa[5]), "+v"(wa[6]), "+v"(wa[7])
+                                 :
+                                 : "memory");
+            }
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+                acc[nt][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[nt], xb[mt], acc[nt][mt], 0, 0, 0);
+        }
+    };
+    for (int s = s_begin; s < s_end; s += Q_STAGES) {
+        step(std::integral_constant<int, 0>{}, s);
+        if (s + 1 < s_end) step(std::integral_constant<int, 1>{}, s + 1);
+        if (s + 2 < s_end) step(std::integral_constant<int, 2>{}, s + 2);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // loads issued past the end still target the ring
+
+    // epilogue: lane (r, g) holds row m = 16*mt + r, channels 4g .. 4g+3 of each tile
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int m = m0 + 64 * wm + 16 * mt + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int n = nw + 16 * nt + 4 * g;
+            if (n >= N) continue;
+            if (partial) {
+                int32_t* p = partial + ((int64_t)blockIdx.y * M + m) * N + n;
+                if (n + 3 < N && (N & 3) == 0) {
+                    *(i32x4*)p = acc[nt][mt];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < N) p[i] = acc[nt][mt][i];
                 }
+            } else {
+                q2_store4<T>(y, acc_out, x_scale, w_scale, bias, residual, m, n, N, acc[nt][mt]);
             }
         }
+    }
+}
+
+template <typename T>
+__global__ void w8a8_splitk_reduce_kernel(uint16_t* __restrict__ y, int32_t* __restrict__ acc_out,
+                                          const int32_t* __restrict__ partial, const float* __restrict__ x_scale,
+                                          const float* __restrict__ w_scale, const uint16_t* __restrict__ bias,
+                                          const uint16_t* __restrict__ residual, int M, int N, int split_k) {
+    const int n4cnt = (N + 3) / 4;
+    const int64_t total = (int64_t)M * n4cnt;
+    const int64_t stride = (int64_t)M * N;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int m = (int)(idx / n4cnt);
+        const int n = (int)(idx - (int64_t)m * n4cnt) * 4;
+        const int32_t* p = partial + (int64_t)m * N + n;
+        i32x4 sum = {0, 0, 0, 0};
+        if (n + 3 < N && (N & 3) == 0) {
+            for (int s = 0; s < split_k; ++s) sum += *(const i32x4*)(p + s * stride);
+        } else {
+            for (int s = 0; s < split_k; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) sum[i] += p[s * stride + i];
+        }
+        q2_store4<T>(y, acc_out, x_scale, w_scale, bias, residual, m, n, N, sum);
+    }
+}
+
+struct QPlan {
+    bool msplit;
+    int nt;
+    int n_blocks, m_blocks, split_k, steps_per_split;
+};
+
+QPlan plan_w8a8(int m, int n, int k) {
+    QPlan p;
+    p.msplit = m > 64;
+    const int steps = (k + Q_KSTEP - 1) / Q_KSTEP;
+    if (p.msplit) {
+        // 80-channel tiles, two workgroups per CU: close to 512 tiles balance best; wide N only
+        p.nt = n >= 16384 ? 5 : 4;
+        p.m_blocks = (m + 255) / 256;
+    } else {
+        p.nt = 2;
+        p.m_blocks = 1;
+    }
+    const int bn = 16 * p.nt * (p.msplit ? 1 : 4);
+    p.n_blocks = (n + bn - 1) / bn;
+    // split K only as far as needed to give every CU a workgroup, and keep at least 16 steps per split: every
+    // split writes (and the reduce kernel reads back) an int32 copy of the output
+    const int tiles = p.n_blocks * p.m_blocks;
+    int sk = tiles >= 200 ? 1 : (224 + tiles - 1) / tiles;
+    const int max_sk = steps / 16 < 1 ? 1 : steps / 16;
+    sk = sk > max_sk ? max_sk : sk;
+    sk = sk > 32 ? 32 : sk;
+    p.steps_per_split = (steps + sk - 1) / sk;
+    p.split_k = (steps + p.steps_per_split - 1) / p.steps_per_split;
+    return p;
+}
+
+template <typename T>
+int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const uint8_t* wp,
+                const float* w_scale, const void* bias, const void* residual, int m, int n, int k, void* workspace,
+                hipStream_t st) {
+    const QPlan p = plan_w8a8(m, n, k);
+    int32_t* partial = p.split_k > 1 ? (int32_t*)workspace : nullptr;
+    dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
+    const bool ktail = (k % Q_KSTEP) != 0;
+#define Q_LAUNCH(NTV, MS, KT)                                                                                     \
+    hipLaunchKernelGGL((w8a8_gemm_kernel<T, NTV, MS, KT>), grid, dim3(256), 0, st, (uint16_t*)y, acc_out, partial,   \
+                       xq, x_scale, wp, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,          \
+                       p.steps_per_split)
+#define Q_LAUNCH_KT(NTV, MS) do { if (ktail) Q_LAUNCH(NTV, MS, true); else Q_LAUNCH(NTV, MS, false); } while (0)
+    if (!p.msplit) Q_LAUNCH_KT(2, false);
+    else if (p.nt == 5) Q_LAUNCH_KT(5, true);
+    else Q_LAUNCH_KT(4, true);
+#undef Q_LAUNCH_KT
+#undef Q_LAUNCH
+    int rc = MF_LAUNCH_CHECK();
+    if (rc || !partial) return rc;
+    const int64_t total = (int64_t)m * ((n + 3) / 4);
+    const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+    hipLaunchKernelGGL((w8a8_splitk_reduce_kernel<T>), dim3(blocks), dim3(256), 0, st, (uint16_t*)y, acc_out, partial,
+                       x_scale, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, p.split_k);
+    return MF_LAUNCH_CHECK();
 }
 
 }  // namespace
 
-extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const int8_t* w,
+extern "C" size_t mf_w8a8_workspace_bytes(int m, int n, int k) {
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const QPlan p = plan_w8a8(m, n, k);
+    return p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(int32_t) : 0;
+}
+
+extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,
                             const float* w_scale, const void* bias, const void* residual, int m, int n, int k,
-                            int dtype, void* stream) {
+                            int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a8_gemm: dtype must be bf16 or fp16");
     if (m == 0) return 0;
-    MF_REQUIRE(xq && w && (y || acc_out), "w8a8_gemm: null argument");
+    MF_REQUIRE(xq && w_packed && (y || acc_out), "w8a8_gemm: null argument");
     MF_REQUIRE(!y || (x_scale && w_scale), "w8a8_gemm: scales required for a dequantised output");
     MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 16 == 0, "w8a8_gemm: bad sizes m=%d n=%d k=%d (K %% 16 == 0)", m, n, k);
-    MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w) & 15) == 0, "w8a8_gemm: xq and w must be 16-byte aligned");
-    if (m == 0) return 0;
-    dim3 grid((n + Q_BN - 1) / Q_BN, (m + Q_BM - 1) / Q_BM);
+    MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w_packed) & 15) == 0, "w8a8_gemm: xq and w_packed must be 16-byte aligned");
+    const size_t need = mf_w8a8_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a8_gemm: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     if (dtype == MF_BF16)
-        hipLaunchKernelGGL(w8a8_gemm_kernel<BF16>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t*)y, acc_out, xq,
-                           x_scale, w, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k);
-    else
-        hipLaunchKernelGGL(w8a8_gemm_kernel<FP16>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t*)y, acc_out, xq,
-                           x_scale, w, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k);
-    return MF_LAUNCH_CHECK();
+        return launch_w8a8<BF16>(y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
+                                 workspace, (hipStream_t)stream);
+    return launch_w8a8<FP16>(y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
+                             workspace, (hipStream_t)stream);
 }

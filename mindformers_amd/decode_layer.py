@@ -48,20 +48,19 @@ class QuantDecodeLayer(nn.Module):
         self.register_buffer("ffn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
 
     def _linear(self, x, name, residual=None):
-        w, s, b = getattr(self, f"{name}_w"), getattr(self, f"{name}_s"), getattr(self, f"{name}_b")
-        if self.act_quant:
-            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"))
-            return ops.w8a8_linear(xq, xs, w, s, self.dtype, bias=b, residual=residual)
+        b = getattr(self, f"{name}_b")
         packed = self._packed.get(name)
         if packed is None:
-            raise RuntimeError("call prepare() after loading the weights (packs them for the W8A16 kernels)")
+            raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
+        if self.act_quant:
+            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"))
+            return ops.w8a8_linear(xq, xs, packed, out_dtype=self.dtype, bias=b, residual=residual)
         return ops.w8a16_linear(x, packed, bias=b, residual=residual)
 
     def prepare(self):
-        """Pack the int8 weights into the order the W8A16 kernels stream.  Call once after loading weights."""
-        if not self.act_quant:
-            for name in self.NAMES:
-                self._packed[name] = ops.pack_w8a16(getattr(self, f"{name}_w"), getattr(self, f"{name}_s"))
+        """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights."""
+        for name in self.NAMES:
+            self._packed[name] = ops.pack_w8a16(getattr(self, f"{name}_w"), getattr(self, f"{name}_s"))
         return self
 
     def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin):

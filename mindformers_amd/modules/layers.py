@@ -185,11 +185,13 @@ class AllQuantLinearInferCell(_QuantLinearBase):
         return ops.dynamic_quant(x, self.smooth_scale)
 
     def prepare(self):
-        self._packed = True                                   # the int8 GEMM reads the row-major weight directly
+        self._packed = ops.pack_w8a16(self.weight, self.w_scale)
         return self
 
     def _matmul(self, xq, x_scale, residual=None):
-        return ops.w8a8_linear(xq, x_scale, self.weight, self.w_scale, self.dtype, bias=self.bias, residual=residual)
+        if self._packed is None:
+            raise RuntimeError("call prepare() (or Quantizer.postprocess_model) after loading the weights")
+        return ops.w8a8_linear(xq, x_scale, self._packed, out_dtype=self.dtype, bias=self.bias, residual=residual)
 
     def forward(self, x, residual=None):
         out_shape = tuple(x.shape[:-1]) + (self.out_channels,)

@@ -275,23 +275,30 @@ def dynamic_quant(x, smooth=None):
     return xq, xs
 
 
-def w8a8_linear(xq, x_scale, w_i8, w_scale, out_dtype, bias=None, residual=None, return_acc=False):
-    """QuantBatchMatmul: int8 x int8 -> int32 -> * x_scale * w_scale (+bias) (+residual) -> out_dtype."""
+def w8a8_linear(xq, x_scale, w, w_scale=None, out_dtype=torch.bfloat16, bias=None, residual=None, return_acc=False):
+    """QuantBatchMatmul: int8 x int8 -> int32 -> * x_scale * w_scale (+bias) (+residual) -> out_dtype.  ``w`` is a
+    PackedInt8Weight (the fast path) or a raw int8 [N, K] tensor with ``w_scale`` (packed on every call)."""
     lib = _lib.load()
-    dev = _dev_ok(xq, x_scale, w_i8, w_scale, bias, residual)
-    _need(xq.dtype == torch.int8 and w_i8.dtype == torch.int8, "xq and w must be int8")
-    _need(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "scales must be fp32")
+    if not isinstance(w, PackedInt8Weight):
+        w = pack_w8a16(w, w_scale)
+    _need(w.experts is None, "stacked expert weights are not supported by the int8 GEMM")
+    dev = _dev_ok(xq, x_scale, bias, residual)
+    _need(xq.dtype == torch.int8, "xq must be int8")
+    _need(x_scale.dtype == torch.float32, "scales must be fp32")
     _need(out_dtype in _ACT, "out_dtype must be bf16/fp16")
-    n, k = w_i8.shape
-    _need(xq.shape[-1] == k and w_scale.numel() == n, "shape mismatch")
+    n, k = w.n, w.k
+    _need(xq.shape[-1] == k, "shape mismatch")
     m = xq.numel() // k
     _need(x_scale.numel() == m, "x_scale must hold one scale per row")
     y = torch.empty(*xq.shape[:-1], n, dtype=out_dtype, device=dev)
     _need(bias is None or (bias.dtype == out_dtype and bias.numel() == n), "bias mismatch")
     _need(residual is None or (residual.dtype == out_dtype and residual.shape == y.shape), "residual mismatch")
     acc = torch.empty(*xq.shape[:-1], n, dtype=torch.int32, device=dev) if return_acc else None
-    check(lib.mf_w8a8_gemm(ptr(y), ptr(acc), ptr(xq), ptr(x_scale), ptr(w_i8), ptr(w_scale), ptr(bias), ptr(residual),
-                           m, n, k, dtype_code(out_dtype), stream_ptr(dev)), "mf_w8a8_gemm")
+    need = lib.mf_w8a8_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a8_gemm(ptr(y), ptr(acc), ptr(xq), ptr(x_scale), ptr(w.packed), ptr(w.scale), ptr(bias),
+                           ptr(residual), m, n, k, dtype_code(out_dtype), ptr(ws),
+                           ws.numel() if ws is not None else 0, stream_ptr(dev)), "mf_w8a8_gemm")
     return (y, acc) if return_acc else y
 
 

@@ -350,7 +350,8 @@ def test_dynamic_quant_bit_exact(dtype, m, k, smooth):
     assert np.array_equal(to_np(xq), q_ref)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 3584, 3584), (130, 200, 1088), (1, 64, 64), (64, 257, 512)])
+@pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 3584, 3584), (130, 200, 1088), (1, 64, 64), (64, 257, 512),
+                                   (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16), (33, 130, 2064)])
 def test_w8a8_gemm_int32_bit_exact(m, n, k):
     rng = np.random.default_rng(10)
     dtype = torch.bfloat16
