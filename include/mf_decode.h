@@ -124,20 +124,24 @@ int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* sca
 
 /* golden-stick DynamicQuant (per-token) with the SmoothQuant multiplier folded in
  * (quantization_config.py:363-380,438-442: act per_token needs int8 weights and activations).
- * xs = x*smooth (fp32); s_t = max_k|xs|/127; q = clip(rint(xs/s_t), -128, 127).  smooth may be NULL. */
+ * xs = x*smooth (fp32); s_t = max_k|xs|/127; q = clip(rint(xs/s_t), -128, 127).  smooth may be NULL.
+ * layout 0: xq is int8 [M,K] row-major.  layout 1: xq is written in the tile order mf_w8a8_gemm streams
+ * (1 KiB tiles of 16 rows x 64 columns, the order mf_w8a16_pack_weight gives an [M,K] matrix;
+ * mf_w8a16_packed_bytes(m, k) bytes, padding left unwritten). */
 int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m, int k,
-                               int dtype, void* stream);
+                               int dtype, int layout, void* stream);
 
 /* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
  * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
- * xq int8 [M,K] row-major (what mf_dynamic_quant_per_token writes); w_packed = mf_w8a16_pack_weight of the int8
+ * xq int8 [M,K]: row-major (x_layout 0) or tiled (x_layout 1), as mf_dynamic_quant_per_token writes it; the tiled
+ * form is the fast path (whole-line, evenly spread L2 requests).  w_packed = mf_w8a16_pack_weight of the int8
  * [N,K] weight (the same tile order serves the int8 matrix cores).  If acc_out != NULL the raw int32 accumulators
  * are also written ([M,N] row-major); y may then be NULL.  K % 16 == 0.  workspace: mf_w8a8_workspace_bytes
  * bytes (int32 partial sums when K is split across workgroups; 0 for wide N). */
 size_t mf_w8a8_workspace_bytes(int m, int n, int k);
 int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,
                  const float* w_scale, const void* bias, const void* residual, int m, int n, int k, int dtype,
-                 void* workspace, size_t workspace_bytes, void* stream);
+                 int x_layout, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- mixture of experts --------------------------------------------------------------------------- */
 

@@ -141,7 +141,8 @@ template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq,
                                                                    float* __restrict__ x_scale,
                                                                    const uint16_t* __restrict__ x,
-                                                                   const float* __restrict__ smooth, int cols) {
+                                                                   const float* __restrict__ smooth, int cols,
+                                                                   int tiled) {
     __shared__ float red[ROW_THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
@@ -180,7 +181,15 @@ __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __re
                 qf = fminf(fmaxf(qf, -128.f), 127.f);
                 o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
             }
-            *(u32x2*)(xq + row + 8 * c) = (u32x2){o[0], o[1]};
+            if (tiled) {
+                // 1 KiB tiles of 16 rows x 64 columns, [row tile][column step], 16 consecutive columns per lane
+                // (lane = 16*(column/16 % 4) + row % 16): the operand order of the int8 matrix instructions
+                const int m = blockIdx.x, k = 8 * c;
+                const int64_t tile = (int64_t)(m >> 4) * ((cols + 63) >> 6) + (k >> 6);
+                *(u32x2*)(xq + tile * 1024 + ((((k & 63) >> 4) << 4) + (m & 15)) * 16 + (k & 15)) = (u32x2){o[0], o[1]};
+            } else {
+                *(u32x2*)(xq + row + 8 * c) = (u32x2){o[0], o[1]};
+            }
         }
     }
 }
@@ -247,8 +256,9 @@ extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dt
 }
 
 extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m,
-                                          int k, int dtype, void* stream) {
+                                          int k, int dtype, int layout, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(layout == 0 || layout == 1, "dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
     if (m <= 0) return 0;
     MF_REQUIRE(xq && x_scale && x, "dynamic_quant: null argument");
     MF_REQUIRE(k > 0 && k % 8 == 0 && k <= ROW_THREADS * 12 * 8, "dynamic_quant: k (%d) must be a multiple of 8, <= %d",
@@ -258,9 +268,9 @@ extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void
     if (m <= 0) return 0;
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(dynamic_quant_kernel<BF16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)x, smooth, k);
+                           (const uint16_t*)x, smooth, k, layout);
     else
         hipLaunchKernelGGL(dynamic_quant_kernel<FP16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)x, smooth, k);
+                           (const uint16_t*)x, smooth, k, layout);
     return MF_LAUNCH_CHECK();
 }

@@ -24,12 +24,18 @@
 
 namespace {
 
+#ifndef QNT_WIDE
+#define QNT_WIDE 5
+#endif
+#ifndef QST8
+#define QST8 3
+#endif
 constexpr int Q_KSTEP = 64;
 constexpr int Q_TILE = 16 * Q_KSTEP;        // bytes of one packed weight tile
-constexpr int Q_STAGES = 3;
 
-template <int NT, bool MSPLIT>
+template <int NT, bool MSPLIT, int ST>
 struct Q2 {
+    static constexpr int STAGES = ST;
     static constexpr int WAVES_M = MSPLIT ? 4 : 1;
     static constexpr int WAVES_N = MSPLIT ? 1 : 4;
     static constexpr int BM = 64 * WAVES_M;
@@ -39,8 +45,9 @@ struct Q2 {
     static constexpr int STAGE = XTILE + WTILES * Q_TILE;
     static constexpr int XL = BM / 64;                        // activation loads (16 rows each) per wave per stage
     static constexpr int WL = (WTILES + 3) / 4;               // weight tile loads per wave per stage
-    static constexpr int PENDING = (Q_STAGES - 2) * (XL + WL);
-    static_assert(Q_STAGES * STAGE <= 65536, "ring exceeds static LDS");
+    static constexpr int PENDING = (ST - 2) * (XL + WL);      // loads of the ST-2 younger steps may be in flight
+    static constexpr int LDS_BYTES = ST * STAGE;
+    static_assert(LDS_BYTES <= 160 * 1024 && PENDING < 64, "bad pipeline shape");
 };
 
 __device__ __forceinline__ int q2_swizzle_key(int row) { return ((row >> 3) & 1) << 1; }
@@ -48,7 +55,8 @@ __device__ __forceinline__ int q2_swizzle_key(int row) { return ((row >> 3) & 1)
 template <int OFFSET>
 __device__ __forceinline__ i32x4 q2_lds_read16(uint32_t addr) {
     i32x4 v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFFSET) : "memory");
+    if constexpr (OFFSET >= 65536) addr += (OFFSET >> 16) << 16;    // the offset field has 16 bits
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFFSET & 65535) : "memory");
     return v;
 }
 __device__ __forceinline__ void q2_lds_direct16(const uint8_t* base_uniform, uint32_t lane_offset,
@@ -96,14 +104,14 @@ __device__ __forceinline__ void q2_store4(uint16_t* y, int32_t* acc_out, const f
 }
 
 // grid = (n_blocks, split_k, m_blocks)
-template <typename T, int NT, bool MSPLIT, bool KTAIL>
+template <typename T, int NT, bool MSPLIT, int ST, bool KTAIL, bool XT>
 __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
     uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
     const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
     const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, int M,
     int N, int K, int steps_per_split) {
-    using C = Q2<NT, MSPLIT>;
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[Q_STAGES * C::STAGE];
+    using C = Q2<NT, MSPLIT, ST>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];       // C::LDS_BYTES, set by the launcher
 
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -123,16 +131,21 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = (i32x4){0, 0, 0, 0};
 
-    // activation loads: load i of this wave covers rows 16*(wv*XL + i) .. + 15 of the stage, 4 lanes per 64-byte
-    // row; lane -> (row, physical chunk), the global address uses the logical chunk.  Rows past M re-read row M-1.
-    const uint8_t* xbase = (const uint8_t*)xq + (int64_t)m0 * K;
+    // activation loads: load i of this wave covers rows 16*(wv*XL + i) .. + 15 of the stage.
+    //   tiled xq (XT): a 16-row tile of a step is 1 KiB of contiguous memory in operand order, like a weight tile;
+    //   row-major xq: 4 lanes per 64-byte row piece; lane -> (row, physical chunk), the global address uses the
+    //   logical chunk.  Rows (row tiles) past M re-read the last one; their results are never stored.
+    const uint8_t* xbase = (const uint8_t*)xq + (XT ? 0 : (int64_t)m0 * K);
     uint32_t xlane[C::XL];
     int xchunk[C::XL];
+    const uint8_t* xtile[C::XL];
+    const int m_tiles_total = (M + 15) >> 4;
 #pragma unroll
     for (int i = 0; i < C::XL; ++i) {
         const int row = 16 * (wv * C::XL + i) + (lane >> 2);
         xchunk[i] = 16 * ((lane & 3) ^ q2_swizzle_key(row));
         xlane[i] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K + xchunk[i];
+        xtile[i] = xbase + (int64_t)min((m0 >> 4) + wv * C::XL + i, m_tiles_total - 1) * KS * Q_TILE;
     }
     // weight loads: tile j of the stage is n-tile nb/16 + j; this wave loads tiles wv*WL + i (clamped: a wave with
     // fewer tiles re-loads the last one onto itself, so that all waves issue the same number of loads)
@@ -153,6 +166,10 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         uint8_t* dst = smem + stage * C::STAGE;
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
+            if (XT) {
+                q2_lds_direct16(xtile[i] + (int64_t)sc * Q_TILE, wlane, dst + 1024 * (wv * C::XL + i));
+                continue;
+            }
             uint32_t off = xlane[i] + (uint32_t)sc * Q_KSTEP;
             if (KTAIL) {
                 // chunks past K (last, short step) re-read the row's last whole chunk; they meet zero weights
@@ -165,12 +182,13 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         for (int i = 0; i < C::WL; ++i)
             q2_lds_direct16(wtile[i] + (int64_t)sc * Q_TILE, wlane, dst + wdst[i]);
     };
-    issue(0, s_begin);
-    issue(1, s_begin + 1);
+#pragma unroll
+    for (int p = 0; p < ST - 1; ++p) issue(p, s_begin + p);
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
     // operand reads: activation tile mt = row 64*wm + 16*mt + r, logical chunk g; weight tile = lane-linear
-    const uint32_t xoff = lds0 + (64 * wm + r) * Q_KSTEP + ((g ^ q2_swizzle_key(r)) << 4);
+    const uint32_t xoff = XT ? lds0 + 64 * wm * Q_KSTEP + lane * 16
+                             : lds0 + (64 * wm + r) * Q_KSTEP + ((g ^ q2_swizzle_key(r)) << 4);
     const uint32_t woff = lds0 + C::XTILE + wn * NT * Q_TILE + lane * 16;
 
     auto step = [&](auto jc, int s) {
@@ -180,7 +198,7 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::PENDING) : "memory");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue((J + 2) % Q_STAGES, s + 2);
+        issue((J + ST - 1) % ST, s + ST - 1);
         i32x4 xb[4], wa[NT];
         xb[0] = q2_lds_read16<SB>(xoff);
         xb[1] = q2_lds_read16<SB + 1024>(xoff);
@@ -221,10 +239,16 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
                 acc[nt][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[nt], xb[mt], acc[nt][mt], 0, 0, 0);
         }
     };
-    for (int s = s_begin; s < s_end; s += Q_STAGES) {
+    for (int s = s_begin; s < s_end; s += ST) {
         step(std::integral_constant<int, 0>{}, s);
         if (s + 1 < s_end) step(std::integral_constant<int, 1>{}, s + 1);
         if (s + 2 < s_end) step(std::integral_constant<int, 2>{}, s + 2);
+        if constexpr (ST > 3)
+            if (s + 3 < s_end) step(std::integral_constant<int, 3 % ST>{}, s + 3);
+        if constexpr (ST > 4)
+            if (s + 4 < s_end) step(std::integral_constant<int, 4 % ST>{}, s + 4);
+        if constexpr (ST > 5)
+            if (s + 5 < s_end) step(std::integral_constant<int, 5 % ST>{}, s + 5);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // loads issued past the end still target the ring
 
@@ -291,7 +315,7 @@ QPlan plan_w8a8(int m, int n, int k) {
     const int steps = (k + Q_KSTEP - 1) / Q_KSTEP;
     if (p.msplit) {
         // 80-channel tiles, two workgroups per CU: close to 512 tiles balance best; wide N only
-        p.nt = n >= 16384 ? 5 : 4;
+        p.nt = n >= 16384 ? QNT_WIDE : 4;
         p.m_blocks = (m + 255) / 256;
     } else {
         p.nt = 2;
@@ -313,20 +337,38 @@ QPlan plan_w8a8(int m, int n, int k) {
 
 template <typename T>
 int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const uint8_t* wp,
-                const float* w_scale, const void* bias, const void* residual, int m, int n, int k, void* workspace,
-                hipStream_t st) {
+                const float* w_scale, const void* bias, const void* residual, int m, int n, int k, bool x_tiled,
+                void* workspace, hipStream_t st) {
     const QPlan p = plan_w8a8(m, n, k);
     int32_t* partial = p.split_k > 1 ? (int32_t*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
     const bool ktail = (k % Q_KSTEP) != 0;
-#define Q_LAUNCH(NTV, MS, KT)                                                                                     \
-    hipLaunchKernelGGL((w8a8_gemm_kernel<T, NTV, MS, KT>), grid, dim3(256), 0, st, (uint16_t*)y, acc_out, partial,   \
-                       xq, x_scale, wp, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,          \
-                       p.steps_per_split)
-#define Q_LAUNCH_KT(NTV, MS) do { if (ktail) Q_LAUNCH(NTV, MS, true); else Q_LAUNCH(NTV, MS, false); } while (0)
-    if (!p.msplit) Q_LAUNCH_KT(2, false);
-    else if (p.nt == 5) Q_LAUNCH_KT(5, true);
-    else Q_LAUNCH_KT(4, true);
+#define Q_LAUNCH(NTV, MS, STV, KT, XTV)                                                                                \
+    do {                                                                                                         \
+        auto kern = w8a8_gemm_kernel<T, NTV, MS, STV, KT, XTV>;                                                        \
+        constexpr int lds = Q2<NTV, MS, STV>::LDS_BYTES;                                                          \
+        static bool configured[MF_MAX_DEVICES] = {};                                                              \
+        int dev = 0;                                                                                             \
+        hipGetDevice(&dev);                                                                                      \
+        if (dev < 0 || dev >= MF_MAX_DEVICES) return (int)hipErrorInvalidDevice;                                  \
+        if (!configured[dev]) {                                                                                  \
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+            if (e != hipSuccess) return (int)e;                                                                  \
+            configured[dev] = true;                                                                              \
+        }                                                                                                        \
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (uint16_t*)y, acc_out, partial, xq, x_scale, wp, w_scale, \
+                           (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split);         \
+    } while (0)
+#define Q_LAUNCH_KT(NTV, MS, STV)                                                                                 \
+    do {                                                                                                         \
+        if (x_tiled) Q_LAUNCH(NTV, MS, STV, false, true);                                                        \
+        else if (ktail) Q_LAUNCH(NTV, MS, STV, true, false);                                                     \
+        else Q_LAUNCH(NTV, MS, STV, false, false);                                                               \
+    } while (0)
+    if (!p.msplit) Q_LAUNCH_KT(2, false, 4);
+    else if (p.nt == 8) Q_LAUNCH_KT(8, true, QST8);
+    else if (p.nt == 5) Q_LAUNCH_KT(5, true, 3);
+    else Q_LAUNCH_KT(4, true, 3);
 #undef Q_LAUNCH_KT
 #undef Q_LAUNCH
     int rc = MF_LAUNCH_CHECK();
@@ -348,10 +390,11 @@ extern "C" size_t mf_w8a8_workspace_bytes(int m, int n, int k) {
 
 extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,
                             const float* w_scale, const void* bias, const void* residual, int m, int n, int k,
-                            int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+                            int dtype, int x_layout, void* workspace, size_t workspace_bytes, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a8_gemm: dtype must be bf16 or fp16");
     if (m == 0) return 0;
     MF_REQUIRE(xq && w_packed && (y || acc_out), "w8a8_gemm: null argument");
+    MF_REQUIRE(x_layout == 0 || x_layout == 1, "w8a8_gemm: x_layout must be 0 (row-major) or 1 (tiled)");
     MF_REQUIRE(!y || (x_scale && w_scale), "w8a8_gemm: scales required for a dequantised output");
     MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 16 == 0, "w8a8_gemm: bad sizes m=%d n=%d k=%d (K %% 16 == 0)", m, n, k);
     MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w_packed) & 15) == 0, "w8a8_gemm: xq and w_packed must be 16-byte aligned");
@@ -360,7 +403,7 @@ extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const f
                "w8a8_gemm: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     if (dtype == MF_BF16)
         return launch_w8a8<BF16>(y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
-                                 workspace, (hipStream_t)stream);
+                                 x_layout == 1, workspace, (hipStream_t)stream);
     return launch_w8a8<FP16>(y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
-                             workspace, (hipStream_t)stream);
+                             x_layout == 1, workspace, (hipStream_t)stream);
 }

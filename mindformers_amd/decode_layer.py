@@ -53,7 +53,7 @@ class QuantDecodeLayer(nn.Module):
         if packed is None:
             raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
         if self.act_quant:
-            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"))
+            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"), tiled=True)
             return ops.w8a8_linear(xq, xs, packed, out_dtype=self.dtype, bias=b, residual=residual)
         return ops.w8a16_linear(x, packed, bias=b, residual=residual)
 

@@ -182,7 +182,7 @@ class AllQuantLinearInferCell(_QuantLinearBase):
         self.quant_op = self._quant
 
     def _quant(self, x):
-        return ops.dynamic_quant(x, self.smooth_scale)
+        return ops.dynamic_quant(x, self.smooth_scale, tiled=True)
 
     def prepare(self):
         self._packed = ops.pack_w8a16(self.weight, self.w_scale)

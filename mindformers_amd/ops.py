@@ -260,44 +260,62 @@ def w8a16_linear(x, w, scale=None, bias=None, residual=None):
     return y
 
 
-def dynamic_quant(x, smooth=None):
-    """DynamicQuant per token (with the smoothing vector folded in): returns (xq int8 [..., K], scale fp32 [rows])."""
+class TiledInt8Activations:
+    """Per-token quantised activations [M, K] in the 16 x 64 tile order the int8 GEMM streams (the fast path of
+    ``w8a8_linear``); ``shape`` is the logical shape of the activation tensor."""
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+
+
+def dynamic_quant(x, smooth=None, tiled=False):
+    """DynamicQuant per token (with the smoothing vector folded in): returns (xq, scale fp32 [rows]); xq is int8
+    [..., K] row-major, or with ``tiled`` a TiledInt8Activations for ``w8a8_linear``."""
     lib = _lib.load()
     dev = _dev_ok(x, smooth)
     _need(x.dtype in _ACT, "x must be bf16/fp16")
     k = x.shape[-1]
     m = x.numel() // k
     _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [K]")
-    xq = torch.empty(x.shape, dtype=torch.int8, device=dev)
+    if tiled:
+        xq = torch.empty(lib.mf_w8a16_packed_bytes(max(m, 1), k), dtype=torch.int8, device=dev)
+    else:
+        xq = torch.empty(x.shape, dtype=torch.int8, device=dev)
     xs = torch.empty(m, dtype=torch.float32, device=dev)
     check(lib.mf_dynamic_quant_per_token(ptr(xq), ptr(xs), ptr(x), ptr(smooth), m, k, dtype_code(x.dtype),
-                                         stream_ptr(dev)), "mf_dynamic_quant_per_token")
-    return xq, xs
+                                         1 if tiled else 0, stream_ptr(dev)), "mf_dynamic_quant_per_token")
+    return (TiledInt8Activations(xq, x.shape) if tiled else xq), xs
 
 
 def w8a8_linear(xq, x_scale, w, w_scale=None, out_dtype=torch.bfloat16, bias=None, residual=None, return_acc=False):
     """QuantBatchMatmul: int8 x int8 -> int32 -> * x_scale * w_scale (+bias) (+residual) -> out_dtype.  ``w`` is a
-    PackedInt8Weight (the fast path) or a raw int8 [N, K] tensor with ``w_scale`` (packed on every call)."""
+    PackedInt8Weight (the fast path) or a raw int8 [N, K] tensor with ``w_scale`` (packed on every call); ``xq`` is
+    an int8 [..., K] tensor or the TiledInt8Activations of ``dynamic_quant(..., tiled=True)`` (the fast path)."""
     lib = _lib.load()
     if not isinstance(w, PackedInt8Weight):
         w = pack_w8a16(w, w_scale)
     _need(w.experts is None, "stacked expert weights are not supported by the int8 GEMM")
-    dev = _dev_ok(xq, x_scale, bias, residual)
-    _need(xq.dtype == torch.int8, "xq must be int8")
+    tiled = isinstance(xq, TiledInt8Activations)
+    xshape = xq.shape
+    xdata = xq.data if tiled else xq
+    dev = _dev_ok(xdata, x_scale, bias, residual)
+    _need(xdata.dtype == torch.int8, "xq must be int8")
     _need(x_scale.dtype == torch.float32, "scales must be fp32")
     _need(out_dtype in _ACT, "out_dtype must be bf16/fp16")
     n, k = w.n, w.k
-    _need(xq.shape[-1] == k, "shape mismatch")
-    m = xq.numel() // k
+    _need(xshape[-1] == k, "shape mismatch")
+    m = 1
+    for d in xshape[:-1]:
+        m *= d
     _need(x_scale.numel() == m, "x_scale must hold one scale per row")
-    y = torch.empty(*xq.shape[:-1], n, dtype=out_dtype, device=dev)
+    y = torch.empty(*xshape[:-1], n, dtype=out_dtype, device=dev)
     _need(bias is None or (bias.dtype == out_dtype and bias.numel() == n), "bias mismatch")
     _need(residual is None or (residual.dtype == out_dtype and residual.shape == y.shape), "residual mismatch")
-    acc = torch.empty(*xq.shape[:-1], n, dtype=torch.int32, device=dev) if return_acc else None
+    acc = torch.empty(*xshape[:-1], n, dtype=torch.int32, device=dev) if return_acc else None
     need = lib.mf_w8a8_workspace_bytes(m, n, k)
     ws = workspace(need, dev, "gemm") if need else None
-    check(lib.mf_w8a8_gemm(ptr(y), ptr(acc), ptr(xq), ptr(x_scale), ptr(w.packed), ptr(w.scale), ptr(bias),
-                           ptr(residual), m, n, k, dtype_code(out_dtype), ptr(ws),
+    check(lib.mf_w8a8_gemm(ptr(y), ptr(acc), ptr(xdata), ptr(x_scale), ptr(w.packed), ptr(w.scale), ptr(bias),
+                           ptr(residual), m, n, k, dtype_code(out_dtype), 1 if tiled else 0, ptr(ws),
                            ws.numel() if ws is not None else 0, stream_ptr(dev)), "mf_w8a8_gemm")
     return (y, acc) if return_acc else y
 

@@ -368,6 +368,43 @@ def test_w8a8_gemm_int32_bit_exact(m, n, k):
     assert_within(to_np(y), ref, np.abs(ref) + np.abs(b), dtype, ulps=1.0, extra=1e-6, what="w8a8 dequant")
 
 
+def _untile_int8(buf, m, k):
+    """Row-major [m, k] view of a buffer in 16 x 64 tile order (byte (16*g + r)*16 + j of tile (mt, s) holds
+    element [16*mt + r, 64*s + 16*g + j])."""
+    mt, ks = (m + 15) // 16, (k + 63) // 64
+    t = buf[: mt * ks * 1024].reshape(mt, ks, 4, 16, 16)        # [mt, s, g, r, j]
+    return t.transpose(0, 3, 1, 2, 4).reshape(mt * 16, ks * 64)[:m, :k]
+
+
+@pytest.mark.parametrize("m,k", [(256, 3584), (37, 1376), (1, 64), (130, 208)])
+def test_dynamic_quant_tiled_layout_bit_exact(m, k):
+    """The tiled output holds exactly the row-major result, at the positions the int8 GEMM reads."""
+    rng = np.random.default_rng(m + k)
+    x = rounded(rng.normal(size=(m, k)) * 3, torch.bfloat16)
+    sm = rng.uniform(0.5, 2.0, k).astype(np.float32)
+    xt, xs = ops.dynamic_quant(dev(x, torch.bfloat16), torch.from_numpy(sm).cuda(), tiled=True)
+    q_ref, s_ref = O.dynamic_quant_per_token(x, sm)
+    assert np.array_equal(to_np(xs), s_ref)
+    assert np.array_equal(_untile_int8(to_np(xt.data), m, k), q_ref)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16),
+                                   (33, 130, 2064), (1, 64, 64)])
+def test_w8a8_tiled_activations_bit_exact(m, n, k):
+    """dynamic_quant(tiled) -> w8a8 GEMM: int32 accumulators equal the integer matmul of the oracle's quantisation."""
+    rng = np.random.default_rng(3 * m + n)
+    dtype = torch.bfloat16
+    x = rounded(rng.normal(size=(m, k)), dtype)
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    ws = rng.uniform(1e-4, 5e-4, n).astype(np.float32)
+    xt, xs = ops.dynamic_quant(dev(x, dtype), None, tiled=True)
+    y, acc = ops.w8a8_linear(xt, xs, torch.from_numpy(wq).cuda(), torch.from_numpy(ws).cuda(), dtype, return_acc=True)
+    q_ref, s_ref = O.dynamic_quant_per_token(x, None)
+    assert np.array_equal(to_np(acc), O.int8_gemm_i32(q_ref, wq))
+    ref = O.w8a8_linear(q_ref, s_ref, wq, ws, None)
+    assert_within(to_np(y), ref, np.abs(ref), dtype, ulps=1.0, extra=1e-6, what="w8a8 tiled")
+
+
 # ------------------------------------------------------------------------------------------- MoE
 @pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1)])
 def test_moe_route(t, e, k, ng, tg):
