@@ -103,7 +103,7 @@ int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* 
 /* ---- quantized linear ----------------------------------------------------------------------------- */
 
 /* The W8A16 kernels stream the int8 weight in a tiled order (16 output channels x 64 input channels per
- * 1 KiB tile, tiles ordered [n-tile][k-step], bytes inside a tile in MFMA-operand lane order; N padded to 16
+ * 1 KiB tile, tiles ordered [k-step][n-tile], bytes inside a tile in MFMA-operand lane order; N padded to 16
  * and K to 64 with zeros).  Pack once after the checkpoint is loaded — the counterpart of the format
  * conversion golden-stick's deploy cells apply to their weight Parameter.  w is int8 [N, K] row-major. */
 size_t mf_w8a16_packed_bytes(int n, int k);

@@ -182,10 +182,10 @@ __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __re
                 o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
             }
             if (tiled) {
-                // 1 KiB tiles of 16 rows x 64 columns, [row tile][column step], 16 consecutive columns per lane
+                // 1 KiB tiles of 16 rows x 64 columns, [column step][row tile], 16 consecutive columns per lane
                 // (lane = 16*(column/16 % 4) + row % 16): the operand order of the int8 matrix instructions
                 const int m = blockIdx.x, k = 8 * c;
-                const int64_t tile = (int64_t)(m >> 4) * ((cols + 63) >> 6) + (k >> 6);
+                const int64_t tile = (int64_t)(k >> 6) * ((gridDim.x + 15) >> 4) + (m >> 4);
                 *(u32x2*)(xq + tile * 1024 + ((((k & 63) >> 4) << 4) + (m & 15)) * 16 + (k & 15)) = (u32x2){o[0], o[1]};
             } else {
                 *(u32x2*)(xq + row + 8 * c) = (u32x2){o[0], o[1]};

@@ -4,7 +4,9 @@
 // into tiles of 16 output channels x 64 input channels (1 KiB).  Inside a tile byte (16*g + r)*16 + j holds
 // w[16*t + r][64*s + 16*g + j]: exactly the order in which the 64 lanes of a wavefront want their MFMA
 // A-operand bytes, so one wave-wide 16-byte load reads one whole tile as 1 KiB of contiguous memory.
-// Tiles are ordered [n-tile][k-step]; N is padded to 16 and K to 64 with zeros.  (Loading the same bytes
+// Tiles are ordered [k-step][n-tile] (all output channels of one 64-wide slice of K are contiguous, so at any
+// moment the workgroups of a launch read neighbouring memory, spread over all memory channels, instead of
+// addresses a whole row of tiles apart); N is padded to 16 and K to 64 with zeros.  (Loading the same bytes
 // from the row-major matrix makes every group of lanes touch 16 different cache lines per instruction and
 // ran at about a third of the bandwidth.)
 //
@@ -110,13 +112,13 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
     // has no divergent branches: tiles beyond N and rows beyond M compute garbage that is never stored, steps
     // beyond s_end are prefetched from a clamped address and never consumed, and only the activation chunks
     // past K (last, short k-step) are replaced by zeros with a select.
-    // ---- weights: tile (n-tile t, step s) sits at ((t*KS + s) * 1024) + lane*16
+    // ---- weights: tile (n-tile t, step s) sits at ((s*n_tiles + t) * 1024) + lane*16
     const int n_tiles_total = (N + 15) >> 4;
     const uint8_t* wbase[GW_NT];
 #pragma unroll
     for (int nt = 0; nt < GW_NT; ++nt) {
         const int t = min((n0 >> 4) + nt, n_tiles_total - 1);
-        wbase[nt] = wp + (int64_t)t * KS * GW_TILE_BYTES + lane * 16;
+        wbase[nt] = wp + (int64_t)t * GW_TILE_BYTES + lane * 16;
     }
     // ---- activations: load i of lane (xr, xc) is the 16-byte chunk xc (8 elements) of row xr + 8*i
     const int xr = lane >> 3, xc = lane & 7;
@@ -134,7 +136,7 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
     u32x4 wreg[GW_DEPTH + 1][GW_NT];
     u32x4 xreg[XLD];
     auto load_w = [&](int slot, int s) {
-        const int64_t off = (int64_t)min(s, s_last) * GW_TILE_BYTES;
+        const int64_t off = (int64_t)min(s, s_last) * n_tiles_total * GW_TILE_BYTES;
 #pragma unroll
         for (int nt = 0; nt < GW_NT; ++nt) wreg[slot][nt] = *(const u32x4*)(wbase[nt] + off);
     };
@@ -359,12 +361,13 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // weights: tile (n-tile t, step s) sits at (t*KS + s) * 1024 + lane*16; tiles past N are clamped (never stored)
+    // weights: tile (n-tile t, step s) sits at (s*n_tiles + t) * 1024 + lane*16; tiles past N are clamped (never
+    // stored)
     const int n_tiles_total = (N + 15) >> 4;
     const uint8_t* wtile[NT];                                 // wave-uniform: step 0 of this wave's n-tiles
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-        wtile[nt] = wp + (int64_t)min((n0 >> 4) + nt, n_tiles_total - 1) * KS * GW_TILE_BYTES;
+        wtile[nt] = wp + (int64_t)min((n0 >> 4) + nt, n_tiles_total - 1) * GW_TILE_BYTES;
     const uint32_t wlane = lane * 16;
     // activations: load i of this wave covers rows 8*(wv*XL + i) .. + 7 of the stage (HALF: rows 4*wv .. + 3, lanes
     // 0-31); lane -> (row, physical chunk), the global address uses the logical chunk.  Rows past M re-read row
@@ -400,7 +403,8 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            g2_lds_direct16(wtile[nt] + (int64_t)sc * GW_TILE_BYTES, wlane, dst + wlds + nt * GW_TILE_BYTES);
+            g2_lds_direct16(wtile[nt] + (int64_t)sc * n_tiles_total * GW_TILE_BYTES, wlane,
+                            dst + wlds + nt * GW_TILE_BYTES);
     };
 #pragma unroll
     for (int p = 0; p < D; ++p) issue(p, s_begin + p);
@@ -574,8 +578,9 @@ __global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __res
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * blockDim.x) {
         const int lane = (int)(c & 63);
         const int64_t tile = c >> 6;
-        const int s = (int)(tile % KS);
-        const int t = (int)(tile / KS);
+        const int n_tiles = (N + 15) >> 4;
+        const int t = (int)(tile % n_tiles);
+        const int s = (int)(tile / n_tiles);
         const int n = 16 * t + (lane & 15);
         const int k0 = 64 * s + 16 * (lane >> 4);
         uint8_t b[16];

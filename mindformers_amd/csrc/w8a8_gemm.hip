@@ -24,12 +24,6 @@
 
 namespace {
 
-#ifndef QNT_WIDE
-#define QNT_WIDE 5
-#endif
-#ifndef QST8
-#define QST8 3
-#endif
 constexpr int Q_KSTEP = 64;
 constexpr int Q_TILE = 16 * Q_KSTEP;        // bytes of one packed weight tile
 
@@ -105,7 +99,7 @@ __device__ __forceinline__ void q2_store4(uint16_t* y, int32_t* acc_out, const f
 
 // grid = (n_blocks, split_k, m_blocks)
 template <typename T, int NT, bool MSPLIT, int ST, bool KTAIL, bool XT>
-__global__ __launch_bounds__(256) void w8a8_gemm_kernel(
+__global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(
     uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
     const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
     const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, int M,
@@ -132,7 +126,8 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = (i32x4){0, 0, 0, 0};
 
     // activation loads: load i of this wave covers rows 16*(wv*XL + i) .. + 15 of the stage.
-    //   tiled xq (XT): a 16-row tile of a step is 1 KiB of contiguous memory in operand order, like a weight tile;
+    //   tiled xq (XT): a 16-row tile of a step is 1 KiB of contiguous memory in operand order, like a weight tile
+    //   (tiles ordered [step][row tile]);
     //   row-major xq: 4 lanes per 64-byte row piece; lane -> (row, physical chunk), the global address uses the
     //   logical chunk.  Rows (row tiles) past M re-read the last one; their results are never stored.
     const uint8_t* xbase = (const uint8_t*)xq + (XT ? 0 : (int64_t)m0 * K);
@@ -145,7 +140,7 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         const int row = 16 * (wv * C::XL + i) + (lane >> 2);
         xchunk[i] = 16 * ((lane & 3) ^ q2_swizzle_key(row));
         xlane[i] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K + xchunk[i];
-        xtile[i] = xbase + (int64_t)min((m0 >> 4) + wv * C::XL + i, m_tiles_total - 1) * KS * Q_TILE;
+        xtile[i] = xbase + (int64_t)min((m0 >> 4) + wv * C::XL + i, m_tiles_total - 1) * Q_TILE;
     }
     // weight loads: tile j of the stage is n-tile nb/16 + j; this wave loads tiles wv*WL + i (clamped: a wave with
     // fewer tiles re-loads the last one onto itself, so that all waves issue the same number of loads)
@@ -156,7 +151,7 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
     for (int i = 0; i < C::WL; ++i) {
         const int j = min(wv * C::WL + i, C::WTILES - 1);
         const int t = min((nb >> 4) + j, n_tiles_total - 1);
-        wtile[i] = wp + (int64_t)t * KS * Q_TILE;
+        wtile[i] = wp + (int64_t)t * Q_TILE;
         wdst[i] = C::XTILE + j * Q_TILE;
     }
     const uint32_t wlane = lane * 16;
@@ -167,7 +162,7 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
             if (XT) {
-                q2_lds_direct16(xtile[i] + (int64_t)sc * Q_TILE, wlane, dst + 1024 * (wv * C::XL + i));
+                q2_lds_direct16(xtile[i] + (int64_t)sc * m_tiles_total * Q_TILE, wlane, dst + 1024 * (wv * C::XL + i));
                 continue;
             }
             uint32_t off = xlane[i] + (uint32_t)sc * Q_KSTEP;
@@ -180,7 +175,7 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
         }
 #pragma unroll
         for (int i = 0; i < C::WL; ++i)
-            q2_lds_direct16(wtile[i] + (int64_t)sc * Q_TILE, wlane, dst + wdst[i]);
+            q2_lds_direct16(wtile[i] + (int64_t)sc * n_tiles_total * Q_TILE, wlane, dst + wdst[i]);
     };
 #pragma unroll
     for (int p = 0; p < ST - 1; ++p) issue(p, s_begin + p);
@@ -277,6 +272,127 @@ __global__ __launch_bounds__(256) void w8a8_gemm_kernel(
     }
 }
 
+// ---- register-streaming kernel (tiled activations) --------------------------------------------------
+// With the activations in tile order too, both operands of the int8 matrix instruction are 1 KiB tiles that a wave
+// loads with one coalesced 16-byte-per-lane load straight into operand registers: no LDS, no barriers, no
+// shuffles.  The 4 waves of a workgroup form a WM x WN grid; a wave owns MT row tiles x NT channel tiles of the
+// output and keeps the operand tiles of the next three k-steps in flight in a rotating set of registers.  Tiles
+// that several waves of the workgroup need are fetched by each of them (they meet in the L1/L2 caches); what the
+// design buys is memory-level parallelism that does not depend on LDS capacity (4 waves x 3 steps x (MT+NT) KiB in
+// flight per workgroup) and a main loop that is nothing but loads and matrix instructions.
+constexpr int QR_DEPTH = 3;
+
+template <typename T, int WM, int MT, int NT>
+__global__ __launch_bounds__(256) void w8a8_regs_kernel(
+    uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
+    const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
+    const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, int M,
+    int N, int K, int steps_per_split) {
+    constexpr int WN = 4 / WM;
+    constexpr int BM = 16 * MT * WM, BN = 16 * NT * WN;
+    constexpr int D = QR_DEPTH;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int wm = wv % WM, wn = wv / WM;
+    const int KS = (K + Q_KSTEP - 1) / Q_KSTEP;
+    const int s_begin = blockIdx.y * steps_per_split;
+    const int s_end = min(KS, s_begin + steps_per_split);
+    const int s_last = s_end - 1;
+    const int m_tiles_total = (M + 15) >> 4, n_tiles_total = (N + 15) >> 4;
+    const int mt0 = blockIdx.z * (BM / 16) + wm * MT;         // first row tile of this wave
+    const int nt0 = blockIdx.x * (BN / 16) + wn * NT;         // first channel tile of this wave
+
+    // tile (t, step s) of either operand sits at (s * tiles_total + t) * 1024 + lane * 16: a scalar base per step
+    // plus a per-lane 32-bit offset that never changes.  Tiles past the matrix are clamped to the last one (their
+    // results are never stored).
+    uint32_t xoff[MT], woff[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xoff[i] = (uint32_t)min(mt0 + i, m_tiles_total - 1) * Q_TILE + lane * 16;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) woff[j] = (uint32_t)min(nt0 + j, n_tiles_total - 1) * Q_TILE + lane * 16;
+    const int64_t xstep = (int64_t)m_tiles_total * Q_TILE, wstep = (int64_t)n_tiles_total * Q_TILE;
+
+    i32x4 acc[NT][MT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = (i32x4){0, 0, 0, 0};
+
+    // The loads and the wait that makes a slot's registers valid are asm statements: the compiler's own counting
+    // gives up at the loop back-edge and waits for everything there, which would leave one step in flight, not three.
+    i32x4 xr[D][MT], wr[D][NT];
+    auto load = [&](int slot, int s) {                        // slot is a compile-time constant at every call
+        const int sc = min(s, s_last);                        // past the end: re-read the last step, never used
+        const uint8_t* wb = wp + sc * wstep;
+        const uint8_t* xb = (const uint8_t*)xq + sc * xstep;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(wr[slot][j]) : "v"(woff[j]), "s"(wb) : "memory");
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(xr[slot][i]) : "v"(xoff[i]), "s"(xb) : "memory");
+    };
+    // loads complete in issue order: once at most (D-1) steps' worth are outstanding, this slot's have arrived
+    constexpr int PENDING = (D - 1) * (MT + NT);
+    static_assert(PENDING < 64 && (MT == 4 || MT == 8) && (NT == 4 || NT == 5), "the wait below is written for these");
+    auto arrived = [&](int slot) {
+        i32x4* w = wr[slot];
+        i32x4* x = xr[slot];
+        if constexpr (NT == 4)
+            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]) : "n"(PENDING) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(%5)"
+                         : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(w[4])
+                         : "n"(PENDING)
+                         : "memory");
+        asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3])::"memory");
+        if constexpr (MT == 8) asm volatile("" : "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])::"memory");
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load(d, s_begin + d);
+    auto step = [&](int slot, int s) {
+        arrived(slot);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[slot][j], xr[slot][i], acc[j][i], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);                    // the reload must not overtake the slot's last use
+        load(slot, s + D);
+    };
+    for (int s = s_begin; s < s_end; s += D) {
+#pragma unroll
+        for (int slot = 0; slot < D; ++slot)
+            if (s + slot < s_end) step(slot, s + slot);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the reloads of the last steps still target registers
+
+    // epilogue: lane (r, g) holds row m = 16*tile + r, channels 4g .. 4g+3 of each tile
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = 16 * (mt0 + i) + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int n = 16 * (nt0 + j) + 4 * g;
+            if (n >= N) continue;
+            if (partial) {
+                int32_t* p = partial + ((int64_t)blockIdx.y * M + m) * N + n;
+                if (n + 3 < N && (N & 3) == 0) {
+                    *(i32x4*)p = acc[j][i];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) p[e] = acc[j][i][e];
+                }
+            } else {
+                q2_store4<T>(y, acc_out, x_scale, w_scale, bias, residual, m, n, N, acc[j][i]);
+            }
+        }
+    }
+}
+
 template <typename T>
 __global__ void w8a8_splitk_reduce_kernel(uint16_t* __restrict__ y, int32_t* __restrict__ acc_out,
                                           const int32_t* __restrict__ partial, const float* __restrict__ x_scale,
@@ -304,24 +420,32 @@ __global__ void w8a8_splitk_reduce_kernel(uint16_t* __restrict__ y, int32_t* __r
 }
 
 struct QPlan {
+    int regs;        // 0: LDS-staged kernel; 1: register-streaming kernel, 4x1 waves of 64 x 64
     bool msplit;
     int nt;
     int n_blocks, m_blocks, split_k, steps_per_split;
 };
 
-QPlan plan_w8a8(int m, int n, int k) {
+QPlan plan_w8a8(int m, int n, int k, bool x_tiled) {
     QPlan p;
     p.msplit = m > 64;
+    p.regs = 0;
     const int steps = (k + Q_KSTEP - 1) / Q_KSTEP;
-    if (p.msplit) {
+    if (x_tiled && m > 64 && n < 8192) {
+        // narrow outputs: the register-streaming kernel on 256 x 64 tiles (measured faster than the LDS-staged one
+        // there; on wide outputs it re-fetches the activation tiles too often and the LDS-staged kernel wins)
+        p.regs = 1;
+        p.nt = 4;                                             // channel tiles per workgroup
+        p.m_blocks = (m + 255) / 256;
+    } else if (p.msplit) {
         // 80-channel tiles, two workgroups per CU: close to 512 tiles balance best; wide N only
-        p.nt = n >= 16384 ? QNT_WIDE : 4;
+        p.nt = n >= 16384 ? 5 : 4;
         p.m_blocks = (m + 255) / 256;
     } else {
         p.nt = 2;
         p.m_blocks = 1;
     }
-    const int bn = 16 * p.nt * (p.msplit ? 1 : 4);
+    const int bn = 16 * p.nt * (p.regs || p.msplit ? 1 : 4);
     p.n_blocks = (n + bn - 1) / bn;
     // split K only as far as needed to give every CU a workgroup, and keep at least 16 steps per split: every
     // split writes (and the reduce kernel reads back) an int32 copy of the output
@@ -339,7 +463,7 @@ template <typename T>
 int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const uint8_t* wp,
                 const float* w_scale, const void* bias, const void* residual, int m, int n, int k, bool x_tiled,
                 void* workspace, hipStream_t st) {
-    const QPlan p = plan_w8a8(m, n, k);
+    const QPlan p = plan_w8a8(m, n, k, x_tiled);
     int32_t* partial = p.split_k > 1 ? (int32_t*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
     const bool ktail = (k % Q_KSTEP) != 0;
@@ -365,10 +489,15 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
         else if (ktail) Q_LAUNCH(NTV, MS, STV, true, false);                                                     \
         else Q_LAUNCH(NTV, MS, STV, false, false);                                                               \
     } while (0)
-    if (!p.msplit) Q_LAUNCH_KT(2, false, 4);
-    else if (p.nt == 8) Q_LAUNCH_KT(8, true, QST8);
+#define QR_LAUNCH(WMV, MTV, NTV)                                                                                  \
+    hipLaunchKernelGGL((w8a8_regs_kernel<T, WMV, MTV, NTV>), grid, dim3(256), 0, st, (uint16_t*)y, acc_out, partial, \
+                       xq, x_scale, wp, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,          \
+                       p.steps_per_split)
+    if (p.regs == 1) QR_LAUNCH(4, 4, 4);
+    else if (!p.msplit) Q_LAUNCH_KT(2, false, 4);
     else if (p.nt == 5) Q_LAUNCH_KT(5, true, 3);
     else Q_LAUNCH_KT(4, true, 3);
+#undef QR_LAUNCH
 #undef Q_LAUNCH_KT
 #undef Q_LAUNCH
     int rc = MF_LAUNCH_CHECK();
@@ -384,8 +513,13 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
 
 extern "C" size_t mf_w8a8_workspace_bytes(int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
-    const QPlan p = plan_w8a8(m, n, k);
-    return p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(int32_t) : 0;
+    size_t need = 0;                                          // enough for either activation layout
+    for (int tiled = 0; tiled < 2; ++tiled) {
+        const QPlan p = plan_w8a8(m, n, k, tiled != 0);
+        const size_t b = p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(int32_t) : 0;
+        need = b > need ? b : need;
+    }
+    return need;
 }
 
 extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,

@@ -369,11 +369,11 @@ def test_w8a8_gemm_int32_bit_exact(m, n, k):
 
 
 def _untile_int8(buf, m, k):
-    """Row-major [m, k] view of a buffer in 16 x 64 tile order (byte (16*g + r)*16 + j of tile (mt, s) holds
+    """Row-major [m, k] view of a buffer in 16 x 64 tile order (tiles ordered [s][mt]; byte (16*g + r)*16 + j of tile (mt, s) holds
     element [16*mt + r, 64*s + 16*g + j])."""
     mt, ks = (m + 15) // 16, (k + 63) // 64
-    t = buf[: mt * ks * 1024].reshape(mt, ks, 4, 16, 16)        # [mt, s, g, r, j]
-    return t.transpose(0, 3, 1, 2, 4).reshape(mt * 16, ks * 64)[:m, :k]
+    t = buf[: mt * ks * 1024].reshape(ks, mt, 4, 16, 16)        # [s, mt, g, r, j]
+    return t.transpose(1, 3, 0, 2, 4).reshape(mt * 16, ks * 64)[:m, :k]
 
 
 @pytest.mark.parametrize("m,k", [(256, 3584), (37, 1376), (1, 64), (130, 208)])
