@@ -50,7 +50,9 @@ def time_events(fn, iters, torch):
 
 
 def kernel_breakdown(case, torch, ops, iters):
-    """Per-op average microseconds for the first layer (each op timed alone, inputs resident)."""
+    """Per-op microseconds for the first layer: each op launched ``iters`` times back to back between two events
+    (launch overhead overlaps with execution; repeated weights may be served from the memory-side cache, so the
+    GEMM figures are a lower bound of their in-layer time)."""
     layer = case["layers"][0]
     kc, vc = case["caches"][0]
     x = case["x"]
@@ -62,8 +64,7 @@ def kernel_breakdown(case, torch, ops, iters):
                                layer.scale_value)
     h = layer._linear(attn, "wo", residual=x)
     n2 = ops.rms_norm(h, layer.ffn_norm, layer.eps)
-    gu = layer._linear(n2, "fc1")
-    a = ops.silu_mul(gu)
+    a = layer.gate_up(n2)
     steps = {
         "rmsnorm": lambda: ops.rms_norm(x, layer.attn_norm, layer.eps),
         "qkv_gemm": lambda: layer._linear(n1, "qkv"),
@@ -72,16 +73,20 @@ def kernel_breakdown(case, torch, ops, iters):
         "paged_attention": lambda: ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"],
                                                        layer.n_head, layer.n_kv_head, layer.scale_value),
         "wo_gemm": lambda: layer._linear(attn, "wo", residual=x),
-        "fc1_gemm": lambda: layer._linear(n2, "fc1"),
-        "silu_mul": lambda: ops.silu_mul(gu),
+        "gate_up_silu_mul": lambda: layer.gate_up(n2),
         "fc2_gemm": lambda: layer._linear(a, "fc2", residual=h),
     }
     out = {}
     for name, fn in steps.items():
         for _ in range(3):
             fn()
-        avg, med = time_events(fn, iters, torch)
-        out[name] = round(avg * 1e3, 2)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        out[name] = round(start.elapsed_time(end) / iters * 1e3, 2)
     return out
 
 

@@ -122,6 +122,15 @@ int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* sca
                   const void* residual, int m, int n, int k, int dtype, void* workspace,
                   size_t workspace_bytes, void* stream);
 
+/* The gate/up projection of a gated MLP fused with its activation: WeightQuantBatchMatmul followed by
+ * SiLU(gate) * up (mindformers/models/llama/llama_layer.py:419-440 with the interleaved ffn_concat layout,
+ * parallel_core/inference/transformer/mlp.py:130-147).  The packed weight has its [N, K] rows in interleaved
+ * order (row 2j = gate channel j, row 2j+1 = up channel j; scale and bias likewise), N even; y is [M, N/2]:
+ * y[m,j] = round(round(silu(g)) * u) with g, u = round(acc * scale + bias) of rows 2j, 2j+1 - bit-identical to
+ * mf_w8a16_gemm followed by mf_silu_mul(layout 1).  Workspace as for mf_w8a16_gemm. */
+int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
+                           int m, int n, int k, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* golden-stick DynamicQuant (per-token) with the SmoothQuant multiplier folded in
  * (quantization_config.py:363-380,438-442: act per_token needs int8 weights and activations).
  * xs = x*smooth (fp32); s_t = max_k|xs|/127; q = clip(rint(xs/s_t), -128, 127).  smooth may be NULL.

@@ -107,6 +107,8 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
 template <typename V, typename U>
 __device__ __forceinline__ V bitcast(const U& u) {
     static_assert(sizeof(V) == sizeof(U), "size mismatch");

@@ -79,7 +79,6 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restri
     }
 }
 
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 // layout 0: [gate | up] halves; layout 1: interleaved g,u pairs.  8 outputs per thread.
 template <typename T>

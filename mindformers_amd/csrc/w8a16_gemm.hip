@@ -83,6 +83,29 @@ __device__ __forceinline__ void store4(uint16_t* y, const uint16_t* bias, const 
     }
 }
 
+// Gated epilogue for 4 consecutive channels (gate, up, gate, up) of one row: the two activations
+// silu(gate) * up go to columns n/2, n/2 + 1 of a [rows, N/2] output.  Rounding points as the unfused sequence has
+// them: the projection output, silu(gate), and the product are each rounded to T.
+template <typename T>
+__device__ __forceinline__ void store_gated(uint16_t* y, const uint16_t* bias, const float* scale, int m, int n,
+                                            int N, f32x4 acc) {
+    float o[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        float gv = acc[2 * h] * scale[n + 2 * h], uv = acc[2 * h + 1] * scale[n + 2 * h + 1];
+        if (bias) {
+            gv += T::to_float(bias[n + 2 * h]);
+            uv += T::to_float(bias[n + 2 * h + 1]);
+        }
+        gv = T::to_float(T::from_float(gv));
+        uv = T::to_float(T::from_float(uv));
+        o[h] = T::to_float(T::from_float(silu_f(gv))) * uv;
+    }
+    const int64_t at = (int64_t)m * (N >> 1) + (n >> 1);
+    if (n + 3 < N) *(uint32_t*)(y + at) = pack2<T>(o[0], o[1]);
+    else y[at] = T::from_float(o[0]);
+}
+
 // One workgroup tile: output channels [n0, n0+64) x 16*MT rows [m0, ...) x k-steps [s_begin, s_end).
 // MT = number of 16-row activation tiles; KTAIL = K is not a multiple of 64.  wp = packed weights of this
 // matrix, KS = k-steps per n-tile.
@@ -338,7 +361,7 @@ template <typename T, int MT, int NT, bool KTAIL>
 __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
     uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
     const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split) {
+    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated) {
     using vec8 = typename T::vec8;
     using C = G2<MT, NT>;
     constexpr int D = C::DEPTH;
@@ -518,7 +541,9 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const int m = m0 + 16 * mt + r;
-                if (m < M) store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, acc[nt][mt]);
+                if (m >= M) continue;
+                if (gated) store_gated<T>(y, bias, scale, m, n, N, acc[nt][mt]);
+                else store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, acc[nt][mt]);
             }
         }
     }
@@ -552,7 +577,8 @@ __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_grouped_kernel(
 template <typename T>
 __global__ void w8a16_splitk_reduce_kernel(uint16_t* __restrict__ y, const float* __restrict__ partial,
                                            const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-                                           const uint16_t* __restrict__ residual, int M, int N, int split_k) {
+                                           const uint16_t* __restrict__ residual, int M, int N, int split_k,
+                                           int gated) {
     const int n4cnt = (N + 3) / 4;
     const int64_t total = (int64_t)M * n4cnt;
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -561,14 +587,24 @@ __global__ void w8a16_splitk_reduce_kernel(uint16_t* __restrict__ y, const float
         const int n = (int)(idx - (int64_t)m * n4cnt) * 4;
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         if (n + 3 < N && (N & 3) == 0) {
-            for (int s = 0; s < split_k; ++s) sum += *(const f32x4*)(partial + ((int64_t)s * M + m) * N + n);
+            // all splits' loads in flight together (at most 16 splits), summed in split order
+            const float* p = partial + (int64_t)m * N + n;
+            const int64_t stride = (int64_t)M * N;
+            f32x4 v[16];
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < split_k) v[s] = *(const f32x4*)(p + s * stride);
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < split_k) sum += v[s];
         } else {
             for (int s = 0; s < split_k; ++s)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     if (n + i < N) sum[i] += partial[((int64_t)s * M + m) * N + n + i];
         }
-        store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, sum);
+        if (gated) store_gated<T>(y, bias, scale, m, n, N, sum);
+        else store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, sum);
     }
 }
 
@@ -622,7 +658,7 @@ GemmPlan plan_w8a16(int m, int n, int k) {
 
 template <typename T>
 int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
-                 const void* residual, int m, int n, int k, void* workspace, hipStream_t st) {
+                 const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st) {
     const GemmPlan p = plan_w8a16(m, n, k);
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
@@ -641,7 +677,8 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
             configured[dev] = true;                                                                              \
         }                                                                                                        \
         hipLaunchKernelGGL(kern, grid, block, lds, st, (uint16_t*)y, partial, (const uint16_t*)x, wp, scale,      \
-                           (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split);         \
+                           (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split,     \
+                           gated);                                                                               \
     } while (0)
     const bool ktail = (k % GW_KSTEP) != 0;
     if (p.mt == 1) { if (ktail) GW_LAUNCH(1, true); else GW_LAUNCH(1, false); }
@@ -653,7 +690,7 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     const int64_t total = (int64_t)m * ((n + 3) / 4);
     const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
     hipLaunchKernelGGL((w8a16_splitk_reduce_kernel<T>), dim3(blocks), dim3(256), 0, st, (uint16_t*)y, partial, scale,
-                       (const uint16_t*)bias, (const uint16_t*)residual, m, n, p.split_k);
+                       (const uint16_t*)bias, (const uint16_t*)residual, m, n, p.split_k, gated);
     return MF_LAUNCH_CHECK();
 }
 
@@ -682,23 +719,38 @@ extern "C" size_t mf_w8a16_workspace_bytes(int m, int n, int k) {
     return p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(float) : 0;
 }
 
+static int w8a16_gemm_entry(const char* who, void* y, const void* x, const void* w_packed, const float* scale,
+                            const void* bias, const void* residual, int m, int n, int k, int dtype, int gated,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "%s: dtype must be bf16 or fp16", who);
+    if (m == 0) return 0;
+    MF_REQUIRE(y && x && w_packed && scale, "%s: null argument", who);
+    MF_REQUIRE(m >= 0 && n > 0 && k > 0, "%s: bad sizes m=%d n=%d k=%d", who, m, n, k);
+    MF_REQUIRE(k % 8 == 0, "%s: K (%d) must be a multiple of 8", who, k);
+    MF_REQUIRE(!gated || n % 2 == 0, "%s: N (%d) must be even (gate/up pairs)", who, n);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0, "%s: x and w_packed must be 16-byte aligned", who);
+    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "%s: 16-byte aligned workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, gated, workspace,
+                                  (hipStream_t)stream);
+    return launch_w8a16<FP16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, gated, workspace,
+                              (hipStream_t)stream);
+}
+
 extern "C" int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
                              const void* residual, int m, int n, int k, int dtype, void* workspace,
                              size_t workspace_bytes, void* stream) {
-    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_gemm: dtype must be bf16 or fp16");
-    if (m == 0) return 0;
-    MF_REQUIRE(y && x && w_packed && scale, "w8a16_gemm: null argument");
-    MF_REQUIRE(m >= 0 && n > 0 && k > 0, "w8a16_gemm: bad sizes m=%d n=%d k=%d", m, n, k);
-    MF_REQUIRE(k % 8 == 0, "w8a16_gemm: K (%d) must be a multiple of 8", k);
-    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0, "w8a16_gemm: x and w_packed must be 16-byte aligned");
-    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
-    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
-               "w8a16_gemm: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    if (dtype == MF_BF16)
-        return launch_w8a16<BF16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, workspace,
-                                  (hipStream_t)stream);
-    return launch_w8a16<FP16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, workspace,
-                              (hipStream_t)stream);
+    return w8a16_gemm_entry("w8a16_gemm", y, x, w_packed, scale, bias, residual, m, n, k, dtype, 0, workspace,
+                            workspace_bytes, stream);
+}
+
+extern "C" int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale,
+                                      const void* bias, int m, int n, int k, int dtype, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    return w8a16_gemm_entry("w8a16_gemm_silu_mul", y, x, w_packed, scale, bias, nullptr, m, n, k, dtype, 1, workspace,
+                            workspace_bytes, stream);
 }
 
 extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale,

@@ -60,7 +60,10 @@ class QuantDecodeLayer(nn.Module):
     def prepare(self):
         """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights."""
         for name in self.NAMES:
-            self._packed[name] = ops.pack_w8a16(getattr(self, f"{name}_w"), getattr(self, f"{name}_s"))
+            w, s = getattr(self, f"{name}_w"), getattr(self, f"{name}_s")
+            # W8A16: the gate/up projection runs fused with SiLU * mul, which wants gate/up rows interleaved
+            gated = name == "fc1" and not self.act_quant and getattr(self, "fc1_b") is None
+            self._packed[name] = ops.pack_w8a16_gated(w, s, "halves") if gated else ops.pack_w8a16(w, s)
         return self
 
     def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin):
@@ -75,9 +78,14 @@ class QuantDecodeLayer(nn.Module):
                                    self.n_kv_head, self.scale_value)
         h = self._linear(attn, "wo", residual=x)
         n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
-        gu = self._linear(n2, "fc1")
-        a = ops.silu_mul(gu)
-        return self._linear(a, "fc2", residual=h)
+        return self._linear(self.gate_up(n2), "fc2", residual=h)
+
+    def gate_up(self, n2):
+        """silu(gate) * up of the MLP input projection: one fused kernel on the W8A16 path."""
+        fc1 = self._packed.get("fc1")
+        if fc1 is not None and fc1.gated:
+            return ops.w8a16_gated_linear(n2, fc1)
+        return ops.silu_mul(self._linear(n2, "fc1"))
 
     construct = forward
 

@@ -211,8 +211,9 @@ class PackedInt8Weight:
     """An int8 weight [N, K] (or a stack [E, N, K]) in the tiled order the W8A16 kernels stream, plus its
     per-output-channel scales.  Built once with ``pack_w8a16`` after the weights are loaded."""
 
-    def __init__(self, packed, scale, n, k, experts=None):
+    def __init__(self, packed, scale, n, k, experts=None, gated=False):
         self.packed, self.scale, self.n, self.k, self.experts = packed, scale, n, k, experts
+        self.gated = gated                                    # rows interleaved gate/up for the fused gated GEMM
 
     @property
     def shape(self):
@@ -244,6 +245,7 @@ def w8a16_linear(x, w, scale=None, bias=None, residual=None):
     if not isinstance(w, PackedInt8Weight):
         w = pack_w8a16(w, scale)
     _need(w.experts is None, "use grouped_w8a16_linear for stacked expert weights")
+    _need(not w.gated, "a gate/up weight packed for the fused gated GEMM: use w8a16_gated_linear")
     dev = _dev_ok(x, bias, residual)
     _need(x.dtype in _ACT, "x must be bf16/fp16")
     n, k = w.n, w.k
@@ -266,6 +268,46 @@ class TiledInt8Activations:
 
     def __init__(self, data, shape):
         self.data, self.shape = data, tuple(shape)
+
+
+def interleave_gate_up(t, layout="halves"):
+    """Rows (dim 0) of a gate/up projection parameter in the interleaved order the fused gated GEMM wants (row 2j =
+    gate channel j, row 2j+1 = up channel j).  ``layout``: "halves" = [gate | up] contiguous halves (the mcore MLP,
+    parallel_core/inference/transformer/mlp.py:136-140), "interleaved" = already in that order (legacy ffn_concat,
+    mindformers/models/llama/llama_layer.py:419-423)."""
+    if layout == "interleaved":
+        return t.contiguous()
+    _need(layout == "halves", "layout must be 'halves' or 'interleaved'")
+    f = t.shape[0] // 2
+    return torch.stack((t[:f], t[f:]), dim=1).reshape(t.shape).contiguous()
+
+
+def pack_w8a16_gated(w_i8, scale, layout="halves"):
+    """Pack a gate/up projection weight [2F, K] (+ scale [2F]) for ``w8a16_gated_linear``."""
+    _need(w_i8.dim() == 2 and w_i8.shape[0] % 2 == 0, "gate/up weight must be [2F, K]")
+    w = pack_w8a16(interleave_gate_up(w_i8, layout), interleave_gate_up(scale, layout))
+    w.gated = True
+    return w
+
+
+def w8a16_gated_linear(x, w, bias=None):
+    """Gate/up projection fused with SiLU(gate) * up: x [..., K] -> [..., F].  ``w`` from ``pack_w8a16_gated``;
+    ``bias`` [2F] in the same interleaved order.  Bit-identical to w8a16_linear followed by silu_mul."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt8Weight) and w.gated and w.experts is None, "w must come from pack_w8a16_gated")
+    dev = _dev_ok(x, bias)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    n, k = w.n, w.k
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
+    m = x.numel() // k
+    y = torch.empty(*x.shape[:-1], n // 2, dtype=x.dtype, device=dev)
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    need = lib.mf_w8a16_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a16_gemm_silu_mul(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), m, n, k,
+                                     dtype_code(x.dtype), ptr(ws), ws.numel() if ws is not None else 0,
+                                     stream_ptr(dev)), "mf_w8a16_gemm_silu_mul")
+    return y
 
 
 def dynamic_quant(x, smooth=None, tiled=False):

@@ -306,6 +306,37 @@ def test_w8a16_gemm(dtype, m, n, k, bias, residual):
     assert_within(got, ref, mag, dtype, ulps=1.0, extra=extra, what="w8a16")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,f,k,bias,layout", [(64, 14336, 4096, False, "halves"), (4, 688, 512, True, "halves"),
+                                               (17, 104, 1024, True, "interleaved"), (64, 96, 4096, False, "halves"),
+                                               (130, 40, 192, True, "halves")])
+def test_w8a16_gated_gemm_equals_unfused(dtype, m, f, k, bias, layout):
+    """Gate/up GEMM fused with SiLU*mul: bit-identical to the GEMM followed by silu_mul, and within tolerance of the
+    oracle (narrow shapes take the split-K path, whose reduce kernel applies the same epilogue)."""
+    rng = np.random.default_rng(m + f)
+    w = rng.normal(0, 0.02, (2 * f, k)).astype(np.float32)
+    wq, s = O.quantize_weight_int8(w)
+    x = rounded(rng.normal(size=(m, k)), dtype)
+    b = rounded(rng.normal(0, 0.1, 2 * f), dtype) if bias else None
+    wq_t, s_t, x_t = torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda(), dev(x, dtype)
+    b_t = dev(b, dtype) if bias else None
+    packed = ops.pack_w8a16_gated(wq_t, s_t, layout)
+    fused = ops.w8a16_gated_linear(x_t, packed, ops.interleave_gate_up(b_t, layout) if bias else None)
+    gu = ops.w8a16_linear(x_t, wq_t, s_t, b_t)
+    unfused = ops.silu_mul(gu, interleaved=(layout == "interleaved"))
+    assert torch.equal(fused, unfused)
+    gu_ref = rounded(O.w8a16_linear(x, wq, s, b), dtype).astype(np.float64)
+    g_ref, u_ref = (gu_ref[:, :f], gu_ref[:, f:]) if layout == "halves" else (gu_ref[:, 0::2], gu_ref[:, 1::2])
+    ref = rounded(O.silu(g_ref), dtype).astype(np.float64) * u_ref
+    got_gu = to_np(gu).astype(np.float64)
+    # compare on the kernel's own projection output so that only the activation arithmetic is in the tolerance
+    g_k, u_k = (got_gu[:, :f], got_gu[:, f:]) if layout == "halves" else (got_gu[:, 0::2], got_gu[:, 1::2])
+    ref_k = rounded(O.silu(g_k), dtype).astype(np.float64) * u_k
+    # silu evaluated in float32 may round to the neighbouring value of T (2 eps |silu| |u|), then the product rounds
+    assert_within(to_np(fused), ref_k, np.abs(ref_k), dtype, ulps=3.0, extra=1e-7, what="gated")
+    assert ref.shape == ref_k.shape
+
+
 def test_w8a16_exact_on_integer_grid():
     """Power-of-two scales and small-integer activations make every product and sum exact: the kernel must
     return exactly the integer matmul (catches a dropped k-step, a wrong row/column or a transposed operand)."""
