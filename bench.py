@@ -150,6 +150,82 @@ def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
         max_abs_err=err, ref_max_abs=scale, rows=len(idx))
 
 
+def bench_moe(args, torch, ops, _lib):
+    """DeepSeek-V3-shaped MoE layer on one GPU's share (all 256 experts resident): router top-k (sigmoid, 8 groups,
+    4 kept) -> permute -> grouped W8A16 expert MLP -> weighted unpermute + shared expert, 128 bf16 tokens."""
+    lib = _lib.load()
+    H, E, F, K_TOP, T = 7168, 256, 2048, 8, 128
+    dev, dt = "cuda", torch.bfloat16
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    x = torch.randn(T, H, generator=gen, device=dev).to(dt)
+    logits = torch.randn(T, E, generator=gen, device=dev)
+    ebias = torch.zeros(E, device=dev)
+
+    def packed(experts, n, k):
+        # any byte pattern is a valid int8 weight: fill the packed buffer directly
+        per = lib.mf_w8a16_packed_bytes(n, k)
+        buf = torch.randint(-127, 128, ((experts or 1) * per,), dtype=torch.int8, generator=gen, device=dev).view(torch.uint8)
+        sc = torch.full(((experts or 1) * n,), 1e-3 / (k ** 0.5), device=dev)
+        return ops.PackedInt8Weight(buf, sc, n, k, experts)
+    w1, w2 = packed(E, 2 * F, H), packed(E, H, F)
+    s1, s2 = packed(None, 2 * F, H), packed(None, H, F)
+    s1.gated = True
+
+    def step():
+        wgt, idx = ops.moe_route(logits, ebias, K_TOP, 8, 4, 2.5, dt)
+        px, row_map, counts, offsets = ops.moe_permute(x, idx, E)
+        a = ops.silu_mul(ops.grouped_w8a16_linear(px, w1, offsets))
+        y = ops.grouped_w8a16_linear(a, w2, offsets)
+        shared = ops.w8a16_linear(ops.w8a16_gated_linear(x, s1), s2)
+        return ops.moe_unpermute(y, row_map, wgt, shared=shared), counts
+    out, counts = step()
+    torch.cuda.synchronize()
+    n_act = int((counts > 0).sum().item())
+    per_expert = 3 * H * F
+    alg_bytes = (n_act + 1) * per_expert
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        st.record()
+        for _ in range(args.kernel_iters):
+            fn()
+        en.record()
+        torch.cuda.synchronize()
+        return st.elapsed_time(en) / args.kernel_iters
+    wgt, idx = ops.moe_route(logits, ebias, K_TOP, 8, 4, 2.5, dt)
+    px, row_map, counts, offsets = ops.moe_permute(x, idx, E)
+    g1 = timed(lambda: ops.grouped_w8a16_linear(px, w1, offsets))
+    a = ops.silu_mul(ops.grouped_w8a16_linear(px, w1, offsets))
+    g2 = timed(lambda: ops.grouped_w8a16_linear(a, w2, offsets))
+    ach = n_act * per_expert / ((g1 + g2) * 1e-3) / 1e9
+    result = {
+        "metric": "decode tokens/sec per layer (Llama3-8B shape, W8A16, bs64); % of peak HBM GB/s",
+        "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"deepseek_v3_moe_w8a16: one MoE layer step, {T} tokens, hidden {H}, {E} experts x ffn {F}, "
+                               f"top-{K_TOP} of 4/8 groups, 1 shared expert, W8A16; {n_act} experts received rows",
+                   "launch": "eager", "algorithmic_bytes_per_layer": alg_bytes},
+        "layer_hbm_gbps": round(alg_bytes / (ms * 1e-3) / 1e9, 1),
+        "layer_hbm_frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": dict(bound="hbm", kernel="w8a16_grouped_kernel (fc1 + fc2 launches)", achieved=round(ach, 1),
+                         peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(ach / HBM_PEAK_GBPS, 4), traffic=None,
+                         bytes_per_launch=n_act * per_expert, avg_launch_us=round((g1 + g2) * 1e3, 2)),
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -176,6 +252,10 @@ def main():
     from mindformers_amd import _lib, ops, synthetic
     _lib.load()                                    # fail loudly if the HIP library is not built
     torch.cuda.set_device(0)
+
+    if args.workload == "deepseek_v3_moe_w8a16":
+        bench_moe(args, torch, ops, _lib)
+        return
 
     t0 = time.perf_counter()
     case = synthetic.make_decode_case(args.workload, seed=1)
