@@ -122,6 +122,17 @@ int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* sca
                   const void* residual, int m, int n, int k, int dtype, void* workspace,
                   size_t workspace_bytes, void* stream);
 
+/* A row-parallel projection with its residual add, fused with the RMSNorm that follows it in the layer
+ * (mindformers/models/llama/llama_transformer.py:1053-1059; parallel_core/inference/transformer/
+ * transformer_layer.py:296-355): h_out = round(round(x . w^T * scale + bias) + residual),
+ * y_norm = RMSNorm(h_out) * gamma.  Bit-identical to mf_w8a16_gemm(residual) followed by mf_rmsnorm; when K is
+ * split across workgroups the sum of the splits, the add and the norm are one kernel.  N % 8 == 0, N <= 16384.
+ * Workspace as for mf_w8a16_gemm. */
+int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* x, const void* w_packed, const float* scale,
+                              const void* bias, const void* residual, const void* gamma, float eps, int m, int n,
+                              int k, int dtype, int gamma_dtype, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
 /* The gate/up projection of a gated MLP fused with its activation: WeightQuantBatchMatmul followed by
  * SiLU(gate) * up (mindformers/models/llama/llama_layer.py:419-440 with the interleaved ffn_concat layout,
  * parallel_core/inference/transformer/mlp.py:130-147).  The packed weight has its [N, K] rows in interleaved

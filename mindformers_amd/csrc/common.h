@@ -107,6 +107,19 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Sum over a workgroup of THREADS threads (wave sums, then the waves in order): the one reduction tree that every
+// RMSNorm-carrying kernel uses, so that fused and unfused paths agree to the bit.  ``red`` holds THREADS/64 floats.
+template <int THREADS>
+__device__ __forceinline__ float rmsnorm_block_sum(float v, float* red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < THREADS / 64; ++i) t += red[i];
+    return t;
+}
+
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 template <typename V, typename U>

@@ -7,7 +7,8 @@
 namespace {
 
 constexpr int ROW_THREADS = 256;
-constexpr int ROW_MAX_VEC = 8;   // up to 8 x (8 elements) per thread: cols <= 256*8*8 = 16384
+constexpr int NORM_THREADS = 512;  // RMSNorm: the geometry (and summation order) shared with the GEMM-fused norm
+constexpr int NORM_MAX_VEC = 4;    // up to 4 x (8 elements) per thread: cols <= 512*4*8 = 16384
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
     v = wave_sum(v);
@@ -31,20 +32,20 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restrict__ y,
+__global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(uint16_t* __restrict__ y,
                                                              uint16_t* __restrict__ sum_out,
                                                              const uint16_t* __restrict__ x,
                                                              const uint16_t* __restrict__ residual,
                                                              const void* __restrict__ gamma, float eps, int cols,
                                                              int gamma_dtype) {
-    __shared__ float red[ROW_THREADS / 64];
+    __shared__ float red[NORM_THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
-    float v[ROW_MAX_VEC][8], gm[ROW_MAX_VEC][8];
+    float v[NORM_MAX_VEC][8], gm[NORM_MAX_VEC][8];
     float ss = 0.f;
 #pragma unroll
-    for (int it = 0; it < ROW_MAX_VEC; ++it) {
-        const int c = threadIdx.x + it * ROW_THREADS;
+    for (int it = 0; it < NORM_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * NORM_THREADS;
         if (c < nvec) {
             u32x4 raw = *(const u32x4*)(x + row + 8 * c);
             u32x4 rraw;
@@ -61,14 +62,14 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(uint16_t* __restri
                 unpack8<T>(s, v[it]);                          // normalise the rounded sum, as two ops would
             }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss += v[it][i] * v[it][i];
+            for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[it][i], v[it][i], ss);
         }
     }
-    ss = block_sum(ss, red);
+    ss = rmsnorm_block_sum<NORM_THREADS>(ss, red);
     const float inv = rsqrtf(ss / (float)cols + eps);
 #pragma unroll
-    for (int it = 0; it < ROW_MAX_VEC; ++it) {
-        const int c = threadIdx.x + it * ROW_THREADS;
+    for (int it = 0; it < NORM_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * NORM_THREADS;
         if (c < nvec) {
             u32x4 o;
 #pragma unroll
@@ -202,17 +203,17 @@ extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* res
     if (rows <= 0) return 0;
     MF_REQUIRE(y && x && gamma, "rmsnorm: null argument");
     MF_REQUIRE(!residual || sum_out, "rmsnorm: residual given without sum_out");
-    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * ROW_MAX_VEC * 8,
-               "rmsnorm: cols (%d) must be a multiple of 8 and at most %d", cols, ROW_THREADS * ROW_MAX_VEC * 8);
+    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= NORM_THREADS * NORM_MAX_VEC * 8,
+               "rmsnorm: cols (%d) must be a multiple of 8 and at most %d", cols, NORM_THREADS * NORM_MAX_VEC * 8);
     MF_REQUIRE((((uintptr_t)y | (uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out | (uintptr_t)gamma) & 15) == 0,
                "rmsnorm: pointers must be 16-byte aligned");
     if (rows <= 0) return 0;
     if (dtype == MF_BF16)
-        hipLaunchKernelGGL(rmsnorm_kernel<BF16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
+        hipLaunchKernelGGL(rmsnorm_kernel<BF16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
                            (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
                            gamma_dtype);
     else
-        hipLaunchKernelGGL(rmsnorm_kernel<FP16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
+        hipLaunchKernelGGL(rmsnorm_kernel<FP16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
                            (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
                            gamma_dtype);
     return MF_LAUNCH_CHECK();

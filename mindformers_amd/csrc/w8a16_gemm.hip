@@ -58,6 +58,15 @@ __device__ __forceinline__ f16x8 dequant8<FP16>(uint32_t lo, uint32_t hi) {
     return v;
 }
 
+// acc * scale (+ bias) with separately rounded operations: every epilogue below goes through here, so that the
+// fused and the unfused paths give bit-identical values whatever the compiler would contract elsewhere.
+template <typename T>
+__device__ __forceinline__ float dequant_bias(float acc, float scale, const uint16_t* bias, int n) {
+    float v = __fmul_rn(acc, scale);
+    if (bias) v = __fadd_rn(v, T::to_float(bias[n]));
+    return v;
+}
+
 // Epilogue for 4 consecutive output channels of one row.
 template <typename T>
 __device__ __forceinline__ void store4(uint16_t* y, const uint16_t* bias, const uint16_t* residual,
@@ -66,9 +75,8 @@ __device__ __forceinline__ void store4(uint16_t* y, const uint16_t* bias, const 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         if (n + i < N) {
-            float v = acc[i] * scale[n + i];
-            if (bias) v += T::to_float(bias[n + i]);
-            if (residual) v = T::to_float(T::from_float(v)) + T::to_float(residual[row_off + n + i]);
+            float v = dequant_bias<T>(acc[i], scale[n + i], bias, n + i);
+            if (residual) v = __fadd_rn(T::to_float(T::from_float(v)), T::to_float(residual[row_off + n + i]));
             o[i] = v;
         } else {
             o[i] = 0.f;
@@ -92,11 +100,8 @@ __device__ __forceinline__ void store_gated(uint16_t* y, const uint16_t* bias, c
     float o[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        float gv = acc[2 * h] * scale[n + 2 * h], uv = acc[2 * h + 1] * scale[n + 2 * h + 1];
-        if (bias) {
-            gv += T::to_float(bias[n + 2 * h]);
-            uv += T::to_float(bias[n + 2 * h + 1]);
-        }
+        float gv = dequant_bias<T>(acc[2 * h], scale[n + 2 * h], bias, n + 2 * h);
+        float uv = dequant_bias<T>(acc[2 * h + 1], scale[n + 2 * h + 1], bias, n + 2 * h + 1);
         gv = T::to_float(T::from_float(gv));
         uv = T::to_float(T::from_float(uv));
         o[h] = T::to_float(T::from_float(silu_f(gv))) * uv;
@@ -608,6 +613,83 @@ __global__ void w8a16_splitk_reduce_kernel(uint16_t* __restrict__ y, const float
     }
 }
 
+// Split-K reduce fused with the residual add and the RMSNorm that follows a row-parallel projection: one workgroup
+// per row sums the splits in split order, forms h = round(round(acc*scale + bias) + residual) (written to h_out)
+// and y = h * rsqrt(mean(h^2) + eps) * gamma - the same values, rounding for rounding, as the plain reduce kernel
+// followed by the RMSNorm kernel, without the launch and the pass over h in between.
+constexpr int RN_THREADS = 512;
+constexpr int RN_MAX_VEC = 4;                                 // N <= 512 * 4 * 8 = 16384
+constexpr int RN_SPLITS = 8;                                  // splits whose loads are in flight together
+
+template <typename T>
+__global__ __launch_bounds__(RN_THREADS) void w8a16_reduce_add_rmsnorm_kernel(
+    uint16_t* __restrict__ y, uint16_t* __restrict__ h_out, const float* __restrict__ partial,
+    const float* __restrict__ scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual,
+    const void* __restrict__ gamma, float eps, int M, int N, int split_k, int gamma_dtype) {
+    __shared__ float red[RN_THREADS / 64];
+    const int m = blockIdx.x;
+    const int nvec = N >> 3;
+    const int64_t stride = (int64_t)M * N;
+    float v[RN_MAX_VEC][8], gm[RN_MAX_VEC][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < RN_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * RN_THREADS;
+        if (c < nvec) {
+            const int n = 8 * c;
+            const float* p = partial + (int64_t)m * N + n;
+            const f32x4 s_lo = *(const f32x4*)(scale + n), s_hi = *(const f32x4*)(scale + n + 4);
+            const u32x4 rraw = *(const u32x4*)(residual + (int64_t)m * N + n);
+            load8_as_float(gamma, n, gamma_dtype, gm[it]);
+            f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+            for (int s0 = 0; s0 < split_k; s0 += RN_SPLITS) {  // summed in split order
+                f32x4 a[RN_SPLITS], b[RN_SPLITS];
+#pragma unroll
+                for (int q = 0; q < RN_SPLITS; ++q)
+                    if (s0 + q < split_k) {
+                        a[q] = *(const f32x4*)(p + (s0 + q) * stride);
+                        b[q] = *(const f32x4*)(p + (s0 + q) * stride + 4);
+                    }
+#pragma unroll
+                for (int q = 0; q < RN_SPLITS; ++q)
+                    if (s0 + q < split_k) {
+                        lo += a[q];
+                        hi += b[q];
+                    }
+            }
+            float rr[8];
+            unpack8<T>(rraw, rr);
+            u32x4 hp;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float t0 = dequant_bias<T>(lo[i], s_lo[i], bias, n + i);
+                const float t1 = dequant_bias<T>(hi[i], s_hi[i], bias, n + 4 + i);
+                v[it][i] = __fadd_rn(T::to_float(T::from_float(t0)), rr[i]);
+                v[it][4 + i] = __fadd_rn(T::to_float(T::from_float(t1)), rr[4 + i]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) hp[i] = pack2<T>(v[it][2 * i], v[it][2 * i + 1]);
+            *(u32x4*)(h_out + (int64_t)m * N + n) = hp;
+            unpack8<T>(hp, v[it]);                            // the norm sees the rounded h
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[it][i], v[it][i], ss);
+        }
+    }
+    const float tot = rmsnorm_block_sum<RN_THREADS>(ss, red);
+    const float inv = rsqrtf(tot / (float)N + eps);
+#pragma unroll
+    for (int it = 0; it < RN_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * RN_THREADS;
+        if (c < nvec) {
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                o[i] = pack2<T>(v[it][2 * i] * inv * gm[it][2 * i], v[it][2 * i + 1] * inv * gm[it][2 * i + 1]);
+            *(u32x4*)(y + (int64_t)m * N + 8 * c) = o;
+        }
+    }
+}
+
 // [N, K] row-major int8 -> packed tiles.  One thread per 16 packed bytes.
 __global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __restrict__ src, int N, int K, int KS,
                                   int64_t chunks) {
@@ -658,7 +740,8 @@ GemmPlan plan_w8a16(int m, int n, int k) {
 
 template <typename T>
 int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
-                 const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st) {
+                 const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st,
+                 void* norm_out = nullptr, const void* gamma = nullptr, float eps = 0.f, int gamma_dtype = MF_FP32) {
     const GemmPlan p = plan_w8a16(m, n, k);
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
@@ -686,7 +769,16 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     else { if (ktail) GW_LAUNCH(4, true); else GW_LAUNCH(4, false); }
 #undef GW_LAUNCH
     int rc = MF_LAUNCH_CHECK();
-    if (rc || !partial) return rc;
+    if (rc) return rc;
+    if (norm_out && partial) {                                // reduce + residual + RMSNorm in one kernel
+        hipLaunchKernelGGL((w8a16_reduce_add_rmsnorm_kernel<T>), dim3(m), dim3(RN_THREADS), 0, st, (uint16_t*)norm_out,
+                           (uint16_t*)y, partial, scale, (const uint16_t*)bias, (const uint16_t*)residual, gamma, eps, m,
+                           n, p.split_k, gamma_dtype);
+        return MF_LAUNCH_CHECK();
+    }
+    if (norm_out)                                             // no split: the GEMM wrote h; normalise it
+        return mf_rmsnorm(norm_out, nullptr, y, nullptr, gamma, eps, m, n, T::id, gamma_dtype, st);
+    if (!partial) return rc;
     const int64_t total = (int64_t)m * ((n + 3) / 4);
     const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
     hipLaunchKernelGGL((w8a16_splitk_reduce_kernel<T>), dim3(blocks), dim3(256), 0, st, (uint16_t*)y, partial, scale,
@@ -744,6 +836,32 @@ extern "C" int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const
                              size_t workspace_bytes, void* stream) {
     return w8a16_gemm_entry("w8a16_gemm", y, x, w_packed, scale, bias, residual, m, n, k, dtype, 0, workspace,
                             workspace_bytes, stream);
+}
+
+extern "C" int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* x, const void* w_packed,
+                                         const float* scale, const void* bias, const void* residual,
+                                         const void* gamma, float eps, int m, int n, int k, int dtype,
+                                         int gamma_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_gemm_add_rmsnorm: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32,
+               "w8a16_gemm_add_rmsnorm: bad gamma dtype");
+    if (m == 0) return 0;
+    MF_REQUIRE(y_norm && h_out && x && w_packed && scale && residual && gamma, "w8a16_gemm_add_rmsnorm: null argument");
+    MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 8 == 0, "w8a16_gemm_add_rmsnorm: bad sizes m=%d n=%d k=%d", m, n, k);
+    MF_REQUIRE(n % 8 == 0 && n <= RN_THREADS * RN_MAX_VEC * 8,
+               "w8a16_gemm_add_rmsnorm: N (%d) must be a multiple of 8 and at most %d", n, RN_THREADS * RN_MAX_VEC * 8);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)y_norm | (uintptr_t)h_out | (uintptr_t)residual |
+                 (uintptr_t)gamma | (uintptr_t)scale | (uintptr_t)bias) & 15) == 0,
+               "w8a16_gemm_add_rmsnorm: pointers must be 16-byte aligned");
+    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a16_gemm_add_rmsnorm: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(h_out, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
+                                  (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
+    return launch_w8a16<FP16>(h_out, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
+                              (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
 }
 
 extern "C" int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale,

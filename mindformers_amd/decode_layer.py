@@ -76,8 +76,13 @@ class QuantDecodeLayer(nn.Module):
         ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
         attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
                                    self.n_kv_head, self.scale_value)
-        h = self._linear(attn, "wo", residual=x)
-        n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
+        if self.act_quant or self.wo_b is not None:
+            h = self._linear(attn, "wo", residual=x)
+            n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
+        else:                                                 # W8A16: projection + residual + norm in one call
+            if self._packed.get("wo") is None:
+                raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
+            h, n2 = ops.w8a16_linear_add_rmsnorm(attn, self._packed["wo"], x, self.ffn_norm, self.eps)
         return self._linear(self.gate_up(n2), "fc2", residual=h)
 
     def gate_up(self, n2):

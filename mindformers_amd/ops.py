@@ -270,6 +270,30 @@ class TiledInt8Activations:
         self.data, self.shape = data, tuple(shape)
 
 
+def w8a16_linear_add_rmsnorm(x, w, residual, gamma, eps, bias=None):
+    """Row-parallel projection + residual add + the RMSNorm that follows: returns (h, norm(h) * gamma) with
+    h = (x . w^T) * scale (+bias) + residual.  Bit-identical to w8a16_linear(residual=...) followed by rms_norm."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt8Weight) and w.experts is None and not w.gated, "w must be a packed [N, K] weight")
+    dev = _dev_ok(x, bias, residual, gamma)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    n, k = w.n, w.k
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
+    m = x.numel() // k
+    h = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=dev)
+    y = torch.empty_like(h)
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    _need(residual.dtype == x.dtype and residual.shape == h.shape and residual.is_contiguous(), "residual mismatch")
+    _need(gamma.numel() == n, "gamma size")
+    need = lib.mf_w8a16_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a16_gemm_add_rmsnorm(ptr(y), ptr(h), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(residual),
+                                        ptr(gamma), float(eps), m, n, k, dtype_code(x.dtype), dtype_code(gamma.dtype),
+                                        ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w8a16_gemm_add_rmsnorm")
+    return h, y
+
+
 def interleave_gate_up(t, layout="halves"):
     """Rows (dim 0) of a gate/up projection parameter in the interleaved order the fused gated GEMM wants (row 2j =
     gate channel j, row 2j+1 = up channel j).  ``layout``: "halves" = [gate | up] contiguous halves (the mcore MLP,

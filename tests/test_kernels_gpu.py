@@ -337,6 +337,27 @@ def test_w8a16_gated_gemm_equals_unfused(dtype, m, f, k, bias, layout):
     assert ref.shape == ref_k.shape
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k,bias", [(64, 4096, 4096, False), (4, 512, 1376, True), (64, 16384, 512, False),
+                                        (130, 1024, 2048, True), (1, 4096, 14336, False)])
+def test_w8a16_linear_add_rmsnorm_equals_unfused(dtype, m, n, k, bias):
+    """Projection + residual + RMSNorm in one call: bit-identical to the GEMM (with residual) followed by the norm
+    kernel, on shapes that split K (fused reduce) and shapes that do not."""
+    rng = np.random.default_rng(m + n + k)
+    w = rng.normal(0, 0.02, (n, k)).astype(np.float32)
+    wq, s = O.quantize_weight_int8(w)
+    x = dev(rounded(rng.normal(size=(m, k)), dtype), dtype)
+    res = dev(rounded(rng.normal(size=(m, n)), dtype), dtype)
+    gamma = torch.from_numpy((1 + 0.1 * rng.normal(size=n)).astype(np.float32)).cuda()
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())
+    h, y = ops.w8a16_linear_add_rmsnorm(x, packed, res, gamma, 1e-5, bias=b)
+    h_ref = ops.w8a16_linear(x, packed, bias=b, residual=res)
+    y_ref = ops.rms_norm(h_ref, gamma, 1e-5)
+    assert torch.equal(h, h_ref)
+    assert torch.equal(y, y_ref)
+
+
 def test_w8a16_exact_on_integer_grid():
     """Power-of-two scales and small-integer activations make every product and sum exact: the kernel must
     return exactly the integer matmul (catches a dropped k-step, a wrong row/column or a transposed operand)."""
