@@ -133,6 +133,19 @@ int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* x, const vo
                               int k, int dtype, int gamma_dtype, void* workspace, size_t workspace_bytes,
                               void* stream);
 
+/* The fused QKV projection together with what follows it on the decode path: rotate-half RoPE on q and k and the
+ * scatter of the rotated k and of v into the paged caches (mindformers/modules/infer_attention.py:441-463,
+ * parallel_core/inference/transformer/attention.py:164-258).  qkv is [M, (n_heads + 2 n_kv_heads) * head_dim]; on
+ * return its q columns hold the rotated query (row stride = the full width), its k and v columns are
+ * unspecified, and the caches hold the new rows.  Same values as mf_w8a16_gemm followed by mf_rope_and_cache on
+ * the column slices; when K is split across workgroups the sum of the splits, the rotation and the scatter are
+ * one kernel.  head_dim % 16 == 0.  Workspace as for mf_w8a16_gemm with n = the full width. */
+int mf_w8a16_qkv_rope_and_cache(void* qkv, const void* x, const void* w_packed, const float* scale, const void* bias,
+                                const void* cos, const void* sin, void* key_cache, void* value_cache,
+                                const int32_t* slot_mapping, int m, int n_heads, int n_kv_heads, int head_dim,
+                                int64_t num_slots, int k, int dtype, int table_dtype, void* workspace,
+                                size_t workspace_bytes, void* stream);
+
 /* The gate/up projection of a gated MLP fused with its activation: WeightQuantBatchMatmul followed by
  * SiLU(gate) * up (mindformers/models/llama/llama_layer.py:419-440 with the interleaved ffn_concat layout,
  * parallel_core/inference/transformer/mlp.py:130-147).  The packed weight has its [N, K] rows in interleaved

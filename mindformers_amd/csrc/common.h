@@ -120,6 +120,14 @@ __device__ __forceinline__ float rmsnorm_block_sum(float v, float* red) {
     return t;
 }
 
+// Rotate-half pair (x1 at i, x2 at i + D/2) with separately rounded operations, shared by every kernel that
+// applies RoPE so that fused and unfused paths agree to the bit.
+__device__ __forceinline__ void rope_pair(float x1, float x2, float c1, float s1, float c2, float s2, float& o1,
+                                          float& o2) {
+    o1 = __fsub_rn(__fmul_rn(x1, c1), __fmul_rn(x2, s1));
+    o2 = __fadd_rn(__fmul_rn(x2, c2), __fmul_rn(x1, s2));
+}
+
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 template <typename V, typename U>

@@ -40,8 +40,9 @@ __device__ __forceinline__ void rope_row(uint16_t* x, int n_heads, int D, const 
         const float s1 = load_as_float(sin, table_row + i, table_dtype);
         const float c2 = load_as_float(cos, table_row + i + half, table_dtype);
         const float s2 = load_as_float(sin, table_row + i + half, table_dtype);
-        const uint16_t o1 = T::from_float(x1 * c1 - x2 * s1);
-        const uint16_t o2 = T::from_float(x2 * c2 + x1 * s2);
+        float r1, r2;
+        rope_pair(x1, x2, c1, s1, c2, s2, r1, r2);
+        const uint16_t o1 = T::from_float(r1), o2 = T::from_float(r2);
         xr[i] = o1;
         xr[i + half] = o2;
         if (scatter_dst) {
@@ -129,10 +130,11 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec_kernel(
     u32x4 o1, o2;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        o1[e] = pack2<T>(x1[2 * e] * c1[2 * e] - x2[2 * e] * s1[2 * e],
-                         x1[2 * e + 1] * c1[2 * e + 1] - x2[2 * e + 1] * s1[2 * e + 1]);
-        o2[e] = pack2<T>(x2[2 * e] * c2[2 * e] + x1[2 * e] * s2[2 * e],
-                         x2[2 * e + 1] * c2[2 * e + 1] + x1[2 * e + 1] * s2[2 * e + 1]);
+        float a0, b0, a1, b1;
+        rope_pair(x1[2 * e], x2[2 * e], c1[2 * e], s1[2 * e], c2[2 * e], s2[2 * e], a0, b0);
+        rope_pair(x1[2 * e + 1], x2[2 * e + 1], c1[2 * e + 1], s1[2 * e + 1], c2[2 * e + 1], s2[2 * e + 1], a1, b1);
+        o1[e] = pack2<T>(a0, a1);
+        o2[e] = pack2<T>(b0, b1);
     }
     *(u32x4*)(xr + i) = o1;
     *(u32x4*)(xr + i + half) = o2;

@@ -690,6 +690,101 @@ __global__ __launch_bounds__(RN_THREADS) void w8a16_reduce_add_rmsnorm_kernel(
     }
 }
 
+// Split-K reduce of a fused QKV projection together with what follows it in the attention block: rotate-half RoPE
+// on q and k and the scatter of the rotated k and of v into the paged caches.  One work item = 8 consecutive
+// elements of the first half of a q/k head with their partners in the second half, or 8 elements of v; grid =
+// (tokens, ceil(items / 256)).  q is written (rotated) into its columns of qkv; the k and v columns of qkv are
+// not written.  Values and rounding are those of the plain reduce kernel followed by the rope-and-cache kernel.
+template <typename T>
+__device__ __forceinline__ void qkv_reduce8(const float* __restrict__ p, int64_t stride, int split_k,
+                                            const float* __restrict__ scale, const uint16_t* __restrict__ bias,
+                                            int n, float* out) {
+    f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < split_k; s0 += RN_SPLITS) {
+        f32x4 a[RN_SPLITS], b[RN_SPLITS];
+#pragma unroll
+        for (int q = 0; q < RN_SPLITS; ++q)
+            if (s0 + q < split_k) {
+                a[q] = *(const f32x4*)(p + (s0 + q) * stride);
+                b[q] = *(const f32x4*)(p + (s0 + q) * stride + 4);
+            }
+#pragma unroll
+        for (int q = 0; q < RN_SPLITS; ++q)
+            if (s0 + q < split_k) {
+                lo += a[q];
+                hi += b[q];
+            }
+    }
+    const f32x4 s_lo = *(const f32x4*)(scale + n), s_hi = *(const f32x4*)(scale + n + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[i] = T::to_float(T::from_float(dequant_bias<T>(lo[i], s_lo[i], bias, n + i)));
+        out[4 + i] = T::to_float(T::from_float(dequant_bias<T>(hi[i], s_hi[i], bias, n + 4 + i)));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void w8a16_reduce_rope_cache_kernel(
+    uint16_t* __restrict__ qkv, const float* __restrict__ partial, const float* __restrict__ scale,
+    const uint16_t* __restrict__ bias, const void* __restrict__ cos, const void* __restrict__ sin,
+    uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache, const int32_t* __restrict__ slot_mapping,
+    int M, int N, int split_k, int n_heads, int n_kv, int D, int64_t num_slots, int table_dtype) {
+    const int t = blockIdx.x;
+    const int half = D >> 1;
+    const int cph = half >> 3;
+    const int rot_items = (n_heads + n_kv) * cph;
+    const int v_items = n_kv * D / 8;
+    const int item = blockIdx.y * 256 + threadIdx.x;
+    if (item >= rot_items + v_items) return;
+    const int64_t slot = slot_mapping[t];
+    const bool live = slot >= 0 && slot < num_slots;
+    const int64_t row = (int64_t)n_kv * D;
+    const int64_t stride = (int64_t)M * N;
+    const float* prow = partial + (int64_t)t * N;
+    if (item >= rot_items) {
+        if (!live) return;
+        const int i = (item - rot_items) * 8;
+        const int col = (n_heads + n_kv) * D + i;
+        float v[8];
+        qkv_reduce8<T>(prow + col, stride, split_k, scale, bias, col, v);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = pack2<T>(v[2 * e], v[2 * e + 1]);
+        *(u32x4*)(value_cache + slot * row + i) = o;
+        return;
+    }
+    const int h = item / cph, i = (item - h * cph) * 8;
+    const bool is_k = h >= n_heads;
+    if (is_k && !live) return;
+    const int col = h * D + i;                                // q heads, then k heads, are consecutive columns
+    float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8];
+    const int64_t trow = (int64_t)t * D;
+    load8_as_float(cos, trow + i, table_dtype, c1);
+    load8_as_float(sin, trow + i, table_dtype, s1);
+    load8_as_float(cos, trow + i + half, table_dtype, c2);
+    load8_as_float(sin, trow + i + half, table_dtype, s2);
+    qkv_reduce8<T>(prow + col, stride, split_k, scale, bias, col, x1);
+    qkv_reduce8<T>(prow + col + half, stride, split_k, scale, bias, col + half, x2);
+    u32x4 o1, o2;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float a0, b0, a1, b1;
+        rope_pair(x1[2 * e], x2[2 * e], c1[2 * e], s1[2 * e], c2[2 * e], s2[2 * e], a0, b0);
+        rope_pair(x1[2 * e + 1], x2[2 * e + 1], c1[2 * e + 1], s1[2 * e + 1], c2[2 * e + 1], s2[2 * e + 1], a1, b1);
+        o1[e] = pack2<T>(a0, a1);
+        o2[e] = pack2<T>(b0, b1);
+    }
+    if (is_k) {
+        uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
+        *(u32x4*)(dst + i) = o1;
+        *(u32x4*)(dst + i + half) = o2;
+    } else {
+        uint16_t* dst = qkv + (int64_t)t * N + col;
+        *(u32x4*)dst = o1;
+        *(u32x4*)(dst + half) = o2;
+    }
+}
+
 // [N, K] row-major int8 -> packed tiles.  One thread per 16 packed bytes.
 __global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __restrict__ src, int N, int K, int KS,
                                   int64_t chunks) {
@@ -712,6 +807,14 @@ __global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __res
         *(u32x4*)(dst + c * 16) = v;
     }
 }
+
+struct RopeCacheArgs {
+    const void *cos, *sin;
+    void *key_cache, *value_cache;
+    const int32_t* slot_mapping;
+    int n_heads, n_kv, head_dim, table_dtype;
+    int64_t num_slots;
+};
 
 struct GemmPlan {
     int mt;          // activation tiles per pass (1, 2, 4)
@@ -741,7 +844,8 @@ GemmPlan plan_w8a16(int m, int n, int k) {
 template <typename T>
 int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
                  const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st,
-                 void* norm_out = nullptr, const void* gamma = nullptr, float eps = 0.f, int gamma_dtype = MF_FP32) {
+                 void* norm_out = nullptr, const void* gamma = nullptr, float eps = 0.f, int gamma_dtype = MF_FP32,
+                 const RopeCacheArgs* rc_args = nullptr) {
     const GemmPlan p = plan_w8a16(m, n, k);
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
@@ -770,6 +874,22 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
 #undef GW_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
+    if (rc_args && partial) {                                 // reduce + RoPE + cache scatter in one kernel
+        const RopeCacheArgs& a = *rc_args;
+        const int items = (a.n_heads + a.n_kv) * (a.head_dim / 16) + a.n_kv * a.head_dim / 8;
+        hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T>), dim3(m, (items + 255) / 256), dim3(256), 0, st,
+                           (uint16_t*)y, partial, scale, (const uint16_t*)bias, a.cos, a.sin, (uint16_t*)a.key_cache,
+                           (uint16_t*)a.value_cache, a.slot_mapping, m, n, p.split_k, a.n_heads, a.n_kv, a.head_dim,
+                           a.num_slots, a.table_dtype);
+        return MF_LAUNCH_CHECK();
+    }
+    if (rc_args) {                                            // no split: the GEMM wrote qkv; rotate and scatter
+        const RopeCacheArgs& a = *rc_args;
+        uint16_t* q = (uint16_t*)y;
+        return mf_rope_and_cache(q, q + (int64_t)a.n_heads * a.head_dim, q + (int64_t)(a.n_heads + a.n_kv) * a.head_dim,
+                                 a.cos, a.sin, a.key_cache, a.value_cache, a.slot_mapping, m, a.n_heads, a.n_kv,
+                                 a.head_dim, a.num_slots, n, n, n, T::id, a.table_dtype, st);
+    }
     if (norm_out && partial) {                                // reduce + residual + RMSNorm in one kernel
         hipLaunchKernelGGL((w8a16_reduce_add_rmsnorm_kernel<T>), dim3(m), dim3(RN_THREADS), 0, st, (uint16_t*)norm_out,
                            (uint16_t*)y, partial, scale, (const uint16_t*)bias, (const uint16_t*)residual, gamma, eps, m,
@@ -862,6 +982,38 @@ extern "C" int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* 
                                   (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
     return launch_w8a16<FP16>(h_out, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
                               (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
+}
+
+extern "C" int mf_w8a16_qkv_rope_and_cache(void* qkv, const void* x, const void* w_packed, const float* scale,
+                                           const void* bias, const void* cos, const void* sin, void* key_cache,
+                                           void* value_cache, const int32_t* slot_mapping, int m, int n_heads,
+                                           int n_kv_heads, int head_dim, int64_t num_slots, int k, int dtype,
+                                           int table_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_qkv_rope_and_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
+               "w8a16_qkv_rope_and_cache: bad table dtype");
+    if (m == 0) return 0;
+    MF_REQUIRE(qkv && x && w_packed && scale && cos && sin && key_cache && value_cache && slot_mapping,
+               "w8a16_qkv_rope_and_cache: null argument");
+    MF_REQUIRE(m >= 0 && n_heads > 0 && n_kv_heads > 0 && k > 0 && k % 8 == 0 && num_slots > 0,
+               "w8a16_qkv_rope_and_cache: bad sizes");
+    MF_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "w8a16_qkv_rope_and_cache: head_dim (%d) must be a multiple of 16",
+               head_dim);
+    const int n = (n_heads + 2 * n_kv_heads) * head_dim;
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)qkv | (uintptr_t)cos | (uintptr_t)sin |
+                 (uintptr_t)key_cache | (uintptr_t)value_cache | (uintptr_t)scale | (uintptr_t)bias) & 15) == 0,
+               "w8a16_qkv_rope_and_cache: pointers must be 16-byte aligned");
+    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a16_qkv_rope_and_cache: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    const RopeCacheArgs a = {cos, sin, key_cache, value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, table_dtype,
+                             num_slots};
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(qkv, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                                  (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, &a);
+    return launch_w8a16<FP16>(qkv, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                              (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, &a);
 }
 
 extern "C" int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale,

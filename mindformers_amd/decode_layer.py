@@ -71,9 +71,15 @@ class QuantDecodeLayer(nn.Module):
         positions; batch_valid_length counts the token written by this step."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
         n1 = ops.rms_norm(x, self.attn_norm, self.eps)
-        qkv = self._linear(n1, "qkv")
-        q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
-        ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
+        if self.act_quant or self.head_dim % 16:
+            qkv = self._linear(n1, "qkv")
+            q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+            ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
+        else:                                                 # W8A16: projection + RoPE + cache write in one call
+            if self._packed.get("qkv") is None:
+                raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
+            q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
+                                             self.n_head, bias=self.qkv_b)
         attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
                                    self.n_kv_head, self.scale_value)
         if self.act_quant or self.wo_b is not None:

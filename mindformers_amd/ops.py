@@ -294,6 +294,34 @@ def w8a16_linear_add_rmsnorm(x, w, residual, gamma, eps, bias=None):
     return h, y
 
 
+def w8a16_qkv_rope_and_cache(x, w, cos, sin, key_cache, value_cache, slot_mapping, n_heads, bias=None):
+    """Fused QKV projection + RoPE + cache scatter.  Returns the rotated query as a [T, n_heads * D] column view of
+    the projection buffer (row stride = full QKV width), ready for ``paged_attention``; the caches receive the
+    rotated key rows and the value rows."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt8Weight) and w.experts is None and not w.gated, "w must be a packed [N, K] weight")
+    dev = _dev_ok(x, bias, cos, sin, key_cache, value_cache, slot_mapping)
+    _need(x.dtype in _ACT and key_cache.dtype == x.dtype and value_cache.dtype == x.dtype, "dtype mismatch")
+    nb, bs, n_kv, d = key_cache.shape
+    _need(value_cache.shape == key_cache.shape, "cache shapes differ")
+    n, k = w.n, w.k
+    _need(n == (n_heads + 2 * n_kv) * d, "weight rows do not match the head geometry")
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
+    m = x.numel() // k
+    _need(slot_mapping.dtype == torch.int32 and slot_mapping.numel() == m, "slot_mapping must be int32 [T]")
+    _need(cos.dtype == sin.dtype and cos.numel() == m * d and sin.numel() == m * d, "cos/sin must be [T, head_dim]")
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    qkv = torch.empty(m, n, dtype=x.dtype, device=dev)
+    need = lib.mf_w8a16_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a16_qkv_rope_and_cache(ptr(qkv), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(cos), ptr(sin),
+                                          ptr(key_cache), ptr(value_cache), ptr(slot_mapping), m, n_heads, n_kv, d,
+                                          nb * bs, k, dtype_code(x.dtype), dtype_code(cos.dtype), ptr(ws),
+                                          ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w8a16_qkv_rope_and_cache")
+    return qkv[:, :n_heads * d]
+
+
 def interleave_gate_up(t, layout="halves"):
     """Rows (dim 0) of a gate/up projection parameter in the interleaved order the fused gated GEMM wants (row 2j =
     gate channel j, row 2j+1 = up channel j).  ``layout``: "halves" = [gate | up] contiguous halves (the mcore MLP,

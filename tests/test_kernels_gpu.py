@@ -358,6 +358,34 @@ def test_w8a16_linear_add_rmsnorm_equals_unfused(dtype, m, n, k, bias):
     assert torch.equal(y, y_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n_head,n_kv,d,k,bias", [(64, 32, 8, 128, 4096, False), (4, 8, 2, 64, 512, True),
+                                                     (7, 28, 4, 128, 64, True), (33, 4, 4, 32, 2048, False)])
+def test_w8a16_qkv_rope_and_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, bias):
+    """QKV projection + RoPE + cache scatter in one call: the rotated query and both caches are bit-identical to the
+    GEMM followed by rope_and_cache on its column slices (shapes with and without split K; a padding slot)."""
+    rng = np.random.default_rng(t + k)
+    n = (n_head + 2 * n_kv) * d
+    wq, s = O.quantize_weight_int8(rng.normal(0, 0.02, (n, k)).astype(np.float32))
+    x = dev(rounded(rng.normal(size=(t, k)), dtype), dtype)
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())
+    bs, nb = 16, t + 3
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[t // 2] = -1
+    slots_t = torch.from_numpy(slots).cuda()
+    cos = dev(rounded(np.cos(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    sin = dev(rounded(np.sin(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    init = dev(rounded(rng.normal(size=(nb, bs, n_kv, d)), dtype), dtype)
+    kc1, vc1, kc2, vc2 = init.clone(), init.clone() + 1, init.clone(), init.clone() + 1
+    q1 = ops.w8a16_qkv_rope_and_cache(x, packed, cos, sin, kc1, vc1, slots_t, n_head, bias=b)
+    qkv = ops.w8a16_linear(x, packed, bias=b)
+    nq, nkv = n_head * d, n_kv * d
+    q2, _ = ops.rope_and_cache(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], cos, sin, kc2, vc2, slots_t, n_head)
+    assert torch.equal(q1, qkv[:, :nq])
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+
+
 def test_w8a16_exact_on_integer_grid():
     """Power-of-two scales and small-integer activations make every product and sum exact: the kernel must
     return exactly the integer matmul (catches a dropped k-step, a wrong row/column or a transposed operand)."""
