@@ -38,11 +38,7 @@ struct BF16 {
     static constexpr int id = MF_BF16;
     static __device__ __forceinline__ float to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
     static __device__ __forceinline__ uint16_t from_float(float f) {
-        // round to nearest even; NaN stays NaN
-        uint32_t u = __float_as_uint(f);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (uint16_t)(u >> 16);
+        return __builtin_bit_cast(uint16_t, (__bf16)f);       // v_cvt_pk_bf16_f32: round to nearest even
     }
     static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -66,6 +62,12 @@ struct FP16 {
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     return (uint32_t)T::from_float(lo) | ((uint32_t)T::from_float(hi) << 16);
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, bf16x2_t));   // one instruction
 }
 
 template <typename T>
