@@ -179,15 +179,28 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         return slot * row_elems + (int64_t)kvh * D + 8 * lchunk;
     };
 
+    // A tile that lies inside one block and inside the context (all but the last tile of a sequence) is a scalar
+    // base (its first slot) plus per-lane offsets that never change: no per-load address arithmetic.
+    const uint32_t lane_off = (uint32_t)(lrow * (int)row_elems + kvh * D + 8 * lchunk) * 2u;     // bytes
+    auto load_tile = [&](u32x4* reg, const uint16_t* __restrict__ cache, int64_t slot0, int tstart) {
+        if (tile_in_block && tstart + PA_TILE <= L) {
+            const uint8_t* base = (const uint8_t*)(cache + slot0 * row_elems);     // wave-uniform
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+                reg[i] = *(const u32x4*)(base + (int64_t)(RPI * i) * row_elems * 2 + lane_off);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) reg[i] = *(const u32x4*)(cache + row_offset(slot0, tstart, i));
+        }
+    };
+
     const int tstep = PA_WAVES * PA_TILE;
     const int tfirst = part_start + wu * PA_TILE;
     int64_t slot_cur = tile_slot(tfirst), slot_nxt = tile_slot(tfirst + tstep);
     u32x4 kreg[NI], vreg[NI];
     if (ntiles > 0) {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) kreg[i] = *(const u32x4*)(kc + row_offset(slot_cur, tfirst, i));
-#pragma unroll
-        for (int i = 0; i < NI; ++i) vreg[i] = *(const u32x4*)(vc + row_offset(slot_cur, tfirst, i));
+        load_tile(kreg, kc, slot_cur, tfirst);
+        load_tile(vreg, vc, slot_cur, tfirst);
     }
 
 #pragma unroll 1
@@ -205,8 +218,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (more) {                                           // next tile's K streams in behind this tile's math
-#pragma unroll
-            for (int i = 0; i < NI; ++i) kreg[i] = *(const u32x4*)(kc + row_offset(slot_nxt, tnext, i));
+            load_tile(kreg, kc, slot_nxt, tnext);
         }
 
         // ---- scores: S[s][i] = score of token tstart + 16 s + 4 g + i for head r
@@ -263,8 +275,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (more) {
-#pragma unroll
-            for (int i = 0; i < NI; ++i) vreg[i] = *(const u32x4*)(vc + row_offset(slot_nxt, tnext, i));
+            load_tile(vreg, vc, slot_nxt, tnext);
         }
         slot_cur = slot_nxt;
         slot_nxt = slot_nn;

@@ -10,13 +10,15 @@
 // from the row-major matrix makes every group of lanes touch 16 different cache lines per instruction and
 // ran at about a third of the bandwidth.)
 //
-// A workgroup of 4 waves owns 64 output channels (4 n-tiles) for up to 64 rows of x.  The waves interleave
-// the 64-wide k-steps of the workgroup's k-range; each wave streams its tiles HBM -> registers two steps
-// ahead, converts int8 -> bf16/fp16 in registers (exact) and multiplies on the 16x16x32 matrix cores.  The
-// activation tile of a step ([rows, 64], re-read from L2 by every workgroup) is fetched with coalesced
-// 128-byte row pieces and staged through a private, XOR-swizzled LDS tile from which the MFMA B operands are
-// read.  The 4 waves are summed through LDS at the end; when N is too small to fill the chip the k-range is
-// also split across workgroups (fp32 partials + a fused reduce/epilogue kernel).
+// Two kernels share the format.  The dense kernel (w8a16_gemm2_kernel, described where it is defined) stages
+// activation and weight tiles through a ring of LDS-direct loads and serves the decode layer's projections; its
+// epilogue, or the split-K reduce kernels, carry the fused variants (gate/up + SiLU*mul, residual + RMSNorm,
+// QKV + RoPE + cache scatter).  The grouped kernel (experts) keeps the earlier register-streaming tile routine
+// w8a16_tile: a workgroup of 4 waves owns 64 output channels (4 n-tiles) for up to 64 rows of x; the waves
+// interleave the 64-wide k-steps of the workgroup's k-range, each streams its tiles HBM -> registers two steps
+// ahead, converts int8 -> bf16/fp16 in registers (exact) and multiplies on the 16x16x32 matrix cores; the
+// activation tile of a step is staged through a private, XOR-swizzled LDS tile; the 4 waves are summed through
+// LDS at the end.
 //
 // MFMA roles: A = weights [16 n x 32 k], B = activations [32 k x 16 m], C = y^T tile [16 n x 16 m]; the two
 // MFMAs of a k-step take bytes 0-7 and 8-15 of each lane's 16 weight bytes, and the activation operand is
