@@ -91,8 +91,8 @@ def kernel_breakdown(case, torch, ops, iters):
 
 
 # (workload, algorithmic KV bytes) -> HBM bytes per attention launch (main kernel + partition reduce) read from
-# FETCH_SIZE / WRITE_SIZE: (289748.4 + 4902.5) KiB x 2.000 + (10126.9 + 512.0) KiB x 1.000
-MEASURED_TRAFFIC_BYTES = {("llama3_8b_w8a16", 589434880): int((294650.9 * 2.0 + 10638.9) * 1024)}
+# FETCH_SIZE / WRITE_SIZE: (289941.0 + 4902.0) KiB x 2.000 + (10130.6 + 512.0) KiB x 1.000
+MEASURED_TRAFFIC_BYTES = {("llama3_8b_w8a16", 589434880): int((294843.0 * 2.0 + 10642.6) * 1024)}
 
 
 def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
