@@ -81,6 +81,42 @@ int mf_paged_attention_decode(void* out, const void* query, const void* key_cach
                               int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                               int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- attention over several new tokens per sequence (prefill, chunked prefill, parallel decoding) -- */
+
+/* Bytes of scratch mf_paged_attention_prefill needs (0 when one partition spans the context).  max_context is
+ * max_blocks_per_seq * block_size for a paged cache and total_q for contiguous keys. */
+size_t mf_paged_attention_prefill_workspace_bytes(int batch, int total_q, int n_heads, int n_kv_heads,
+                                                  int head_dim, int max_context);
+
+/* Causal attention of q_len_b = q_starts[b+1] - q_starts[b] new query rows per sequence.
+ *
+ * Paged keys (block_tables != NULL) replace PagedAttention called with q_seq_lens and a causal mask:
+ *   ops.auto_generate.PagedAttention(...)(query, key_cache, value_cache, block_tables, batch_valid_length,
+ *                                         None, None, attn_mask, q_seq_lens)
+ *   mindformers/modules/paged_attention_mgr.py:66-69 (parallel_decoding / chunk_prefill)
+ *   mindformers/parallel_core/inference/transformer/flash_attention.py:140-143
+ * The new tokens' keys and values are already in the cache (ReshapeAndCache runs first, flash_attention.py:
+ * 126-127); context_lens[b] counts them.  Query i of sequence b sits at position L_b - q_len_b + i and
+ * attends to cache tokens 0 .. L_b - q_len_b + i.
+ *
+ * Contiguous keys (block_tables == NULL; context_lens, block_size, max_blocks_per_seq, num_blocks ignored)
+ * replace FlashAttentionScore in the TH layout with a causal mask and actual_seq_qlen == actual_seq_kvlen:
+ *   mindformers/parallel_core/inference/transformer/flash_attention.py:96-104,129-134
+ *   mindformers/modules/flash_attention.py (FlashAttention.construct, input_layout "TH")
+ * key_cache / value_cache are then this step's packed keys and values, row q_starts[b] + j = token j of
+ * sequence b, kv_row_stride elements apart (0 = dense n_kv_heads * head_dim; a slice of a fused QKV output
+ * works), and L_b = q_len_b.
+ *
+ * query: total_q rows of n_heads * head_dim, q_row_stride elements apart (0 = dense); out: dense
+ * [total_q, n_heads * head_dim].  q_starts: int32 [batch + 1], non-decreasing.  Rows of no sequence, and
+ * rows beyond a sequence's context, are written as zeros.  Numerics as mf_paged_attention_decode. */
+int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache, const void* value_cache,
+                               const int32_t* block_tables, const int32_t* context_lens,
+                               const int32_t* q_starts, int batch, int total_q, int n_heads, int n_kv_heads,
+                               int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                               float scale, int64_t q_row_stride, int64_t kv_row_stride, int dtype,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- norm / activation ---------------------------------------------------------------------------- */
 
 /* P.RmsNorm(eps)(x, gamma): mindformers/models/llama/llama_layer.py:195,225-228;

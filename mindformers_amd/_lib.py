@@ -24,6 +24,9 @@ SIGNATURES = {
     "mf_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _I, _I, _P]),
     "mf_paged_attention_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "mf_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P, _Z, _P]),
+    "mf_paged_attention_prefill_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I]),
+    "mf_paged_attention_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _L, _L, _I,
+                                        _P, _Z, _P]),
     "mf_rmsnorm": (_I, [_P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P]),
     "mf_silu_mul": (_I, [_P, _P, _I, _I, _I, _I, _P]),
     "mf_add": (_I, [_P, _P, _P, _L, _I, _P]),

@@ -37,18 +37,45 @@ struct PaSmem {
     static_assert(16 * D * 4 <= PA_TILE * VSTRIDE, "a wave's accumulators must fit its staging tile");
 };
 
+// Prefill bookkeeping of sequence s: first query row, number of query rows and context length, made safe
+// (never more queries than context; query rows, and with them contiguous keys, never leave the `rows` passed).
+__device__ inline void pf_seq(int s, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ ctx_lens,
+                              bool contiguous, int rows, int max_ctx, int batch, int& qs, int& ql, int& len) {
+    qs = 0, ql = 0, len = 0;
+    if (s >= batch) return;
+    qs = q_starts[s];
+    ql = q_starts[s + 1] - qs;
+    if (qs < 0 || ql < 0 || qs + ql > rows) ql = 0;           // never leave the query / output rows
+    if (contiguous) {
+        len = ql;
+    } else {
+        len = ctx_lens[s];
+        len = len < 0 ? 0 : (len > max_ctx ? max_ctx : len);  // the block table holds no more
+        ql = ql < 0 ? 0 : (ql > len ? len : ql);
+    }
+}
+
 // TPW = tiles per wave: a workgroup covers TPW * 128 tokens.
-template <typename T, int D, int TPW>
+// PF (prefill / chunked prefill): sequence b brings q_starts[b+1] - q_starts[b] new query rows whose keys and values
+// are already in the cache; query i of the sequence sits at position L_b - q_len + i and attends to the cache
+// tokens up to and including its own.  The 16 MFMA columns of a workgroup, which in decode are the query heads
+// of one kv head, are then 16 consecutive (query, head-of-the-kv-group) pairs, each with its own causal limit.
+// PF with block_tables == nullptr: the keys and values are this step's own packed rows (row q_starts[b] + j is
+// token j of sequence b, pf_kv_stride elements apart) and the context is q_len.
+template <typename T, int D, int TPW, bool PF>
 __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
     int n_rep, int head_groups, int block_size, int max_blocks, int num_blocks, int max_parts,
-    float scale_log2, int64_t q_stride, int batch) {
+    float scale_log2, int64_t q_stride, int batch, const int32_t* __restrict__ q_starts, int pf_part_tokens,
+    int64_t pf_kv_stride, int pf_rows) {
     using vec8 = typename T::vec8;
     constexpr int KS = D / 32;
     constexpr int VSTRIDE = PaSmem<D>::VSTRIDE;
-    constexpr int PART = TPW * PA_WAVE_TOKENS;
+    // tokens per partition: fixed by TPW in decode, chosen by the host (a multiple of 128) in PF, where the
+    // query rows already supply the parallelism and one partition may span the whole context
+    const int PART = PF ? pf_part_tokens : TPW * PA_WAVE_TOKENS;
     constexpr int CPR = D / 8;                                // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
     constexpr int NI = PA_TILE / RPI;                         // loads per lane per tile per tensor
@@ -65,16 +92,24 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     // consecutive XCDs) to one 256-byte lane of every token row and measured 25 % slower.
     const int nkg = n_kv * head_groups;
     int b = -1, part = 0, L = 0, kg = 0;
+    int q_len = 1, q_start = 0, col_groups = head_groups;     // PF: per sequence
     {
         const int pidx = blockIdx.x;
         const int ln = threadIdx.x & 63;
         int base = 0;
         for (int c0 = 0; c0 < batch; c0 += 64) {
             const int bb = c0 + ln;
-            const int len = bb < batch ? ctx_lens[bb] : 0;
+            int len, ql = 1, qs = 0, ncg = head_groups;
+            if constexpr (PF) {
+                pf_seq(bb, q_starts, ctx_lens, block_tables == nullptr, pf_rows, max_blocks * block_size, batch, qs, ql, len);
+                ncg = (ql * n_rep + 15) >> 4;
+            } else {
+                len = bb < batch ? min(ctx_lens[bb], max_blocks * block_size) : 0;   // the table holds no more
+            }
             int np = len > 0 ? (len + PART - 1) / PART : 0;
             np = np < max_parts ? np : max_parts;
-            int incl = np * nkg;
+            const int per_seq = np * (PF ? n_kv * ncg : nkg);
+            int incl = per_seq;
 #pragma unroll
             for (int o = 1; o < 64; o <<= 1) {
                 const int t = __shfl_up(incl, o, 64);
@@ -82,28 +117,44 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             }
             const int total = __shfl(incl, 63, 64);
             if (pidx < base + total) {
-                const bool hit = pidx >= base + incl - np * nkg && pidx < base + incl;
+                const bool hit = pidx >= base + incl - per_seq && pidx < base + incl;
                 const uint64_t m = __ballot(hit);
                 const int src = __ffsll((unsigned long long)m) - 1;
                 b = c0 + src;
-                const int rem = pidx - (base + __shfl(incl - np * nkg, src, 64));
+                const int rem = pidx - (base + __shfl(incl - per_seq, src, 64));
                 const int npb = __shfl(np, src, 64);
                 kg = rem / npb;
                 part = rem - kg * npb;
                 L = __shfl(len, src, 64);
+                if constexpr (PF) {
+                    q_len = __shfl(ql, src, 64);
+                    q_start = __shfl(qs, src, 64);
+                    col_groups = __shfl(ncg, src, 64);
+                }
                 break;
             }
             base += total;
         }
     }
     kg = __builtin_amdgcn_readfirstlane(kg);
-    const int kvh = kg / head_groups;
-    const int hg = kg - kvh * head_groups;
     if (b < 0) return;                                        // uniform over the workgroup
+    col_groups = __builtin_amdgcn_readfirstlane(col_groups);
+    const int kvh = kg / col_groups;
+    const int hg = kg - kvh * col_groups;                     // head group (decode) / column group (PF)
     b = __builtin_amdgcn_readfirstlane(b);
     part = __builtin_amdgcn_readfirstlane(part);
     L = __builtin_amdgcn_readfirstlane(L);
+    q_len = __builtin_amdgcn_readfirstlane(q_len);
+    q_start = __builtin_amdgcn_readfirstlane(q_start);
     const int part_start = part * PART;
+    // PF: the farthest token any column of this group may see; partitions past it have nothing to do (the reduce
+    // kernel counts partitions per query row and never reads them)
+    const int ctx_before = L - q_len;                         // cache tokens older than this step's queries
+    if constexpr (PF) {
+        const int last_q = min(q_len, (hg * 16 + 15) / n_rep + 1);
+        L = ctx_before + last_q;
+        if (part_start >= L) return;
+    }
     if (threadIdx.x == 0) sm_count = 0;
     __syncthreads();                                          // the only barrier: all waves are still in step here
 
@@ -114,11 +165,16 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 
     // ---- Q as MFMA B operand: lane (r, g) holds Q[head r][32j + 8g .. +8]
     const int hh = hg * 16 + r;
-    const bool head_ok = hh < n_rep;
-    const int head = kvh * n_rep + (head_ok ? hh : 0);
+    int qi = 0;                                               // PF: query index of this lane's column
+    if constexpr (PF) qi = hh / n_rep;
+    const int hcol = PF ? hh - qi * n_rep : hh;               // head within the kv group
+    const bool head_ok = PF ? qi < q_len : hh < n_rep;
+    const int head = kvh * n_rep + (head_ok ? hcol : 0);
+    const int q_row = PF ? q_start + (head_ok ? qi : 0) : b;
+    const int Lcol = PF ? (head_ok ? ctx_before + qi + 1 : 0) : L;      // causal limit of this lane's column
     vec8 qreg[KS];
     {
-        const uint16_t* qp = q + (int64_t)b * q_stride + (int64_t)head * D + 8 * g;
+        const uint16_t* qp = q + (int64_t)q_row * q_stride + (int64_t)head * D + 8 * g;
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             u32x4 v = {0u, 0u, 0u, 0u};
@@ -133,15 +189,18 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         acc[u][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
         acc[u][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
-    float m_run = PA_NEG, l_run = 0.f;
+    // PF: a column can find a whole tile masked before it has seen any token; starting the running maximum above
+    // the mask value makes those probabilities 2^(-huge) = 0 instead of 2^0
+    float m_run = PF ? 0.5f * PA_NEG : PA_NEG, l_run = 0.f;
 
     uint8_t* vst = smem + w * (PA_TILE * VSTRIDE);
+    const bool contiguous = PF && block_tables == nullptr;
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
-    const int64_t row_elems = (int64_t)n_kv * D;
+    const int64_t row_elems = PF ? pf_kv_stride : (int64_t)n_kv * D;
 
     const int lrow = lane / CPR;                              // coalesced-load coordinates of this lane
     const int lchunk = lane - lrow * CPR;
-    const bool tile_in_block = (block_size % PA_TILE) == 0;   // then a tile never straddles two blocks
+    const bool tile_in_block = contiguous || (block_size % PA_TILE) == 0;   // then a tile never straddles two blocks
     const int wu = __builtin_amdgcn_readfirstlane(w);         // wave index as a scalar
 
     // tiles of this wave: it = 0 .. ntiles-1 start at part_start + (it*4 + wave)*32
@@ -157,6 +216,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     // two tiles ahead so that no K/V load ever waits on a table load
     auto tile_slot = [&](int ts) -> int64_t {
         if (!tile_in_block || ts >= L) return 0;
+        if (contiguous) return (int64_t)q_start + ts;
         const int bi = ts / block_size;
         int blk = table[bi];
         blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;       // never leave the cache allocation
@@ -238,7 +298,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tok = tstart + s * 16 + 4 * g + i;
-                const float v = tok < L ? sc[s][i] * scale_log2 : PA_NEG;
+                const float v = tok < Lcol ? sc[s][i] * scale_log2 : PA_NEG;
                 sc[s][i] = v;
                 tmax = fmaxf(tmax, v);
             }
@@ -329,8 +389,16 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     constexpr int D4 = D / 4;
     for (int idx = lane; idx < 16 * D4; idx += 64) {
         const int hr = idx / D4, d4 = idx - hr * D4;
-        const int hq = hg * 16 + hr;
-        if (hq >= n_rep) break;                               // heads are ordered: nothing valid follows
+        int hq = hg * 16 + hr;
+        int row = b;
+        if constexpr (PF) {
+            const int qe = hq / n_rep;
+            if (qe >= q_len) break;                           // columns are ordered: nothing valid follows
+            hq -= qe * n_rep;
+            row = q_start + qe;
+        } else {
+            if (hq >= n_rep) break;                           // heads are ordered: nothing valid follows
+        }
         float Mh = sm_m[0][hr];
 #pragma unroll
         for (int x = 1; x < PA_WAVES; ++x) Mh = fmaxf(Mh, sm_m[x][hr]);
@@ -342,7 +410,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             lt += sm_l[x][hr] * f;
             sum += *(const f32x4*)((const float*)(smem + x * (PA_TILE * VSTRIDE)) + hr * D + 4 * d4) * f;
         }
-        const int64_t gh = (int64_t)b * n_heads + kvh * n_rep + hq;
+        const int64_t gh = (int64_t)row * n_heads + kvh * n_rep + hq;
         if (max_parts == 1) {
             const float inv = 1.0f / lt;
             u32x2 o = {pack2<T>(sum[0] * inv, sum[1] * inv), pack2<T>(sum[2] * inv, sum[3] * inv)};
@@ -358,20 +426,40 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     }
 }
 
+// Causal limit (number of cache tokens visible) of query row `row` in a prefill step; 0 for a row that belongs to
+// no sequence (before q_starts[0], from q_starts[batch] on, or beyond its sequence's context).
+__device__ inline int pf_row_limit(int row, const int32_t* __restrict__ q_starts,
+                                   const int32_t* __restrict__ ctx_lens, bool contiguous, int rows, int max_ctx,
+                                   int batch) {
+    int lo = 0, hi = batch;                                   // last sequence with q_starts[s] <= row
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (q_starts[mid] <= row) lo = mid; else hi = mid;
+    }
+    int qs, ql, len;
+    pf_seq(lo, q_starts, ctx_lens, contiguous, rows, max_ctx, batch, qs, ql, len);
+    const int qi = row - qs;
+    return (qi >= 0 && qi < ql) ? len - ql + qi + 1 : 0;
+}
+
 // Combine the partitions of one (sequence, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p.
 // One workgroup of D threads per (head, sequence).  The per-partition (max, sum) pairs are read one per lane
 // and reduced across the wave; the weighted accumulator sum runs 8 independent loads deep.
-template <typename T, int D>
+// PF: blockIdx.y is a query row; its sequence is found in q_starts and its context is its causal limit.  Rows that
+// belong to no sequence (beyond q_starts[batch], or beyond a sequence's context) are written as zeros.
+template <typename T, int D, bool PF>
 __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __restrict__ out,
                                                                   const float* __restrict__ part_out,
                                                                   const float* __restrict__ part_ml,
                                                                   const int32_t* __restrict__ ctx_lens, int n_heads,
-                                                                  int max_parts, int part_tokens) {
+                                                                  int max_parts, int part_tokens,
+                                                                  const int32_t* __restrict__ q_starts, int batch,
+                                                                  bool contiguous, int max_ctx) {
     __shared__ float s_f[64];
-    const int h = blockIdx.x, b = blockIdx.y;
+    const int h = blockIdx.x, b = blockIdx.y;                 // b: sequence (decode) or query row (PF)
     const int d = threadIdx.x;
     const int lane = threadIdx.x & 63;
-    const int L = ctx_lens[b];
+    const int L = PF ? pf_row_limit(b, q_starts, ctx_lens, contiguous, gridDim.y, max_ctx, batch) : ctx_lens[b];
     const int64_t gh = (int64_t)b * n_heads + h;
     int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
     np = np < max_parts ? np : max_parts;
@@ -435,18 +523,20 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid((unsigned)((int64_t)batch * max_parts * n_kv * head_groups));
 #define PA_LAUNCH(TPWV)                                                                                          \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV>), grid, dim3(PA_WAVES * 64), 0, st, (uint16_t*)out,     \
-                       part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,                      \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false>), grid, dim3(PA_WAVES * 64), 0, st,             \
+                       (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,      \
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
-                       block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch)
+                       block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
+                       (const int32_t*)nullptr, 0, (int64_t)0, 0)
     if (tpw == 2) PA_LAUNCH(2);
     else PA_LAUNCH(4);
 #undef PA_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (max_parts > 1) {
-        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D>), dim3(n_heads, batch), dim3(D), 0, st,
-                           (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts, part_tokens);
+        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, false>), dim3(n_heads, batch), dim3(D), 0, st,
+                           (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts, part_tokens,
+                           (const int32_t*)nullptr, batch, false, 0);
         rc = MF_LAUNCH_CHECK();
     }
     return rc;
@@ -459,7 +549,141 @@ __global__ void pa_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t* 
     for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)b * row + i] = 0;
 }
 
+// ---- prefill --------------------------------------------------------------------------------------------------
+// Partitioning rule shared by the workspace query and the launch.  A workgroup serves 16 (query, head) columns of one
+// kv head; when the query rows alone give the chip enough workgroups one partition spans the whole context and no
+// partials are written, otherwise the context is cut so that about a thousand workgroups exist.
+struct PfPlan {
+    int part_tokens;
+    int max_parts;
+    int64_t col_groups;                                       // upper bound over the batch
+};
+
+static inline PfPlan pf_plan(int batch, int64_t total_q, int n_heads, int n_kv, int64_t max_ctx) {
+    const int n_rep = n_heads / n_kv;
+    PfPlan p;
+    p.col_groups = (total_q * n_rep + 15) / 16 + batch;       // each sequence rounds its own columns up
+    const int64_t wgs = std::max<int64_t>(1, (total_q * n_rep + 15) / 16) * n_kv;
+    int64_t want = (1024 + wgs - 1) / wgs;
+    const int64_t most = std::max<int64_t>(1, (max_ctx + 255) / 256);
+    want = std::min(want, most);
+    int64_t pt = (max_ctx + want - 1) / want;
+    pt = std::max<int64_t>(PA_WAVE_TOKENS, (pt + PA_WAVE_TOKENS - 1) / PA_WAVE_TOKENS * PA_WAVE_TOKENS);
+    p.part_tokens = (int)pt;
+    p.max_parts = (int)std::max<int64_t>(1, (max_ctx + pt - 1) / pt);
+    return p;
+}
+
+// zero the rows the single-partition prefill path never writes (rows of no sequence)
+__global__ void pf_zero_rows_kernel(uint16_t* __restrict__ out, const int32_t* __restrict__ q_starts,
+                                    const int32_t* __restrict__ ctx_lens, bool contiguous, int max_ctx, int batch,
+                                    int row) {
+    if (pf_row_limit(blockIdx.x, q_starts, ctx_lens, contiguous, gridDim.x, max_ctx, batch) > 0) return;
+    for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)blockIdx.x * row + i] = 0;
+}
+
+template <typename T, int D>
+int launch_pf(void* out, const void* query, const void* key_cache, const void* value_cache,
+              const int32_t* block_tables, const int32_t* context_lens, const int32_t* q_starts, int batch,
+              int total_q, int n_heads, int n_kv, int block_size, int max_blocks, int num_blocks, float scale,
+              int64_t q_stride, int64_t kv_stride, void* workspace, hipStream_t st) {
+    const int n_rep = n_heads / n_kv;
+    const bool contiguous = block_tables == nullptr;
+    const PfPlan plan = pf_plan(batch, total_q, n_heads, n_kv, contiguous ? total_q : (int64_t)max_blocks * block_size);
+    float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
+    float* part_ml = part_out ? part_out + (int64_t)total_q * n_heads * plan.max_parts * D : nullptr;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const int64_t wgs = plan.col_groups * n_kv * plan.max_parts;
+    if (wgs > 0x7fffffffLL) {
+        mf_set_error("paged_attention_prefill: %lld workgroups exceed the grid limit", (long long)wgs);
+        return 1;
+    }
+    if (plan.max_parts == 1) {
+        hipLaunchKernelGGL(pf_zero_rows_kernel, dim3(total_q), dim3(128), 0, st, (uint16_t*)out, q_starts,
+                           context_lens, contiguous, max_blocks * block_size, batch, n_heads * D);
+        int rc = MF_LAUNCH_CHECK();
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true>), dim3((unsigned)wgs), dim3(PA_WAVES * 64), 0, st,
+                       (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,
+                       (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep,
+                       (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, scale_log2, q_stride,
+                       batch, q_starts, plan.part_tokens, kv_stride, total_q);
+    int rc = MF_LAUNCH_CHECK();
+    if (rc) return rc;
+    if (plan.max_parts > 1) {
+        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, true>), dim3(n_heads, total_q), dim3(D), 0, st,
+                           (uint16_t*)out, part_out, part_ml, context_lens, n_heads, plan.max_parts,
+                           plan.part_tokens, q_starts, batch, contiguous, max_blocks * block_size);
+        rc = MF_LAUNCH_CHECK();
+    }
+    return rc;
+}
+
 }  // namespace
+
+extern "C" size_t mf_paged_attention_prefill_workspace_bytes(int batch, int total_q, int n_heads, int n_kv_heads,
+                                                             int head_dim, int max_context) {
+    if (batch <= 0 || total_q <= 0 || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
+    const PfPlan plan = pf_plan(batch, total_q, n_heads, n_kv_heads, max_context);
+    if (plan.max_parts <= 1) return 0;
+    return (size_t)total_q * n_heads * plan.max_parts * (head_dim + 2) * sizeof(float);
+}
+
+extern "C" int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache,
+                                          const void* value_cache, const int32_t* block_tables,
+                                          const int32_t* context_lens, const int32_t* q_starts, int batch,
+                                          int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                          int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                          int64_t kv_row_stride, int dtype, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention_prefill: dtype must be bf16 or fp16");
+    MF_REQUIRE(batch >= 0 && total_q >= 0, "paged_attention_prefill: negative batch or row count");
+    if (batch == 0 || total_q == 0) return 0;
+    MF_REQUIRE(out && query && key_cache && value_cache && q_starts, "paged_attention_prefill: null argument");
+    const bool contiguous = block_tables == nullptr;
+    MF_REQUIRE(contiguous || context_lens, "paged_attention_prefill: block_tables without context_lens");
+    MF_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+               "paged_attention_prefill: n_heads (%d) must be a positive multiple of n_kv_heads (%d)", n_heads,
+               n_kv_heads);
+    MF_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 128,
+               "paged_attention_prefill: head_dim %d not supported (32, 64, 128)", head_dim);
+    MF_REQUIRE(contiguous || (block_size > 0 && max_blocks_per_seq > 0 && num_blocks > 0),
+               "paged_attention_prefill: bad block geometry");
+    MF_REQUIRE(contiguous || (int64_t)block_size * max_blocks_per_seq <= 0x7fffffffLL,
+               "paged_attention_prefill: context capacity overflows int");
+    if (kv_row_stride <= 0) kv_row_stride = (int64_t)n_kv_heads * head_dim;
+    MF_REQUIRE(kv_row_stride >= (int64_t)n_kv_heads * head_dim && kv_row_stride % 8 == 0,
+               "paged_attention_prefill: key/value row stride must be >= n_kv_heads*head_dim and a multiple of 8");
+    MF_REQUIRE(contiguous || kv_row_stride == (int64_t)n_kv_heads * head_dim,
+               "paged_attention_prefill: a paged cache has dense rows");
+    if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * head_dim;
+    MF_REQUIRE(q_row_stride >= (int64_t)n_heads * head_dim && q_row_stride % 8 == 0,
+               "paged_attention_prefill: query row stride must be >= n_heads*head_dim and a multiple of 8 elements");
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)query | (uintptr_t)key_cache | (uintptr_t)value_cache) & 15) == 0,
+               "paged_attention_prefill: out / query / caches must be 16-byte aligned");
+    const size_t need = mf_paged_attention_prefill_workspace_bytes(
+        batch, total_q, n_heads, n_kv_heads, head_dim, contiguous ? total_q : max_blocks_per_seq * block_size);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need),
+               "paged_attention_prefill: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    MF_REQUIRE(need == 0 || ((uintptr_t)workspace & 15) == 0,
+               "paged_attention_prefill: workspace must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+#define PF_CASE(TT, DD)                                                                                            \
+    return launch_pf<TT, DD>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch,      \
+                             total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale,      \
+                             q_row_stride, kv_row_stride, workspace, st)
+    if (dtype == MF_BF16) {
+        if (head_dim == 32) PF_CASE(BF16, 32);
+        if (head_dim == 64) PF_CASE(BF16, 64);
+        PF_CASE(BF16, 128);
+    } else {
+        if (head_dim == 32) PF_CASE(FP16, 32);
+        if (head_dim == 64) PF_CASE(FP16, 64);
+        PF_CASE(FP16, 128);
+    }
+#undef PF_CASE
+}
 
 extern "C" size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, int max_context) {
     const int part_tokens = pa_tiles_per_wave(max_context) * PA_WAVE_TOKENS;
@@ -484,6 +708,7 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
     MF_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 128,
                "paged_attention: head_dim %d not supported (32, 64, 128)", head_dim);
     MF_REQUIRE(block_size > 0 && max_blocks_per_seq > 0 && num_blocks > 0, "paged_attention: bad block geometry");
+    MF_REQUIRE((int64_t)block_size * max_blocks_per_seq <= 0x7fffffffLL, "paged_attention: context capacity overflows int");
     if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * head_dim;
     MF_REQUIRE(q_row_stride >= (int64_t)n_heads * head_dim && q_row_stride % 8 == 0,
                "paged_attention: query row stride must be >= n_heads*head_dim and a multiple of 8 elements");

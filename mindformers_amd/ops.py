@@ -165,6 +165,77 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n
     return out
 
 
+def _q_starts(q_starts, dev):
+    _need(isinstance(q_starts, torch.Tensor) and q_starts.dtype == torch.int32 and q_starts.dim() == 1 and
+          q_starts.numel() >= 2, "q_starts must be int32 [batch + 1] (cumulative query-row offsets)")
+    _need(q_starts.device == dev and q_starts.is_contiguous(), "q_starts must be a contiguous tensor on the GPU")
+    return q_starts.numel() - 1
+
+
+def paged_attention_prefill(query, key_cache, value_cache, block_tables, context_lens, q_starts, n_heads,
+                            n_kv_heads, scale, out=None):
+    """Causal attention of several new tokens per sequence over the paged cache (their keys/values already
+    scattered): PagedAttention(...)(query, key_cache, value_cache, block_tables, batch_valid_length, None, None,
+    causal_mask, q_seq_lens) with q_starts = [0, cumsum(q_seq_lens)]."""
+    lib = _lib.load()
+    _dev_of(query)
+    dev = _dev_ok(key_cache, value_cache, block_tables, context_lens, out)
+    _need(key_cache.dim() == 4 and value_cache.shape == key_cache.shape, "caches must be [blocks, block_size, n_kv, D]")
+    nb, bs, n_kv, d = key_cache.shape
+    query, qs = _rows(query, n_heads * d, "query")
+    _need(n_kv == n_kv_heads, f"cache has {n_kv} kv heads, module says {n_kv_heads}")
+    _need(query.dtype in _ACT and key_cache.dtype == query.dtype and value_cache.dtype == query.dtype, "dtype mismatch")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
+    _need(context_lens.dtype == torch.int32 and context_lens.dim() == 1, "context_lens must be int32 [B]")
+    b = _q_starts(q_starts, dev)
+    _need(context_lens.numel() == b and block_tables.shape[0] == b, "context_lens / block_tables rows != batch")
+    total_q = query.numel() // (n_heads * d) if query.is_contiguous() else query.shape[0]
+    max_blocks = block_tables.shape[1]
+    if out is None:
+        out = torch.empty((total_q, n_heads * d), dtype=query.dtype, device=dev)
+    else:
+        _need(out.numel() == total_q * n_heads * d and out.dtype == query.dtype and out.is_contiguous(), "out mismatch")
+    need = lib.mf_paged_attention_prefill_workspace_bytes(b, total_q, n_heads, n_kv_heads, d, max_blocks * bs)
+    ws = workspace(need, dev, "pa_prefill") if need else None
+    check(lib.mf_paged_attention_prefill(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(block_tables),
+                                         ptr(context_lens), ptr(q_starts), b, total_q, n_heads, n_kv_heads, d, bs,
+                                         max_blocks, nb, float(scale), qs, 0, dtype_code(query.dtype), ptr(ws),
+                                         ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_paged_attention_prefill")
+    return out
+
+
+def causal_attention_varlen(query, key, value, q_starts, n_heads, n_kv_heads, scale, out=None):
+    """FlashAttentionScore in the TH layout with a causal mask and actual_seq_qlen == actual_seq_kvlen: packed
+    rows, sequence b owns rows q_starts[b] .. q_starts[b+1]-1 of query, key and value.  key / value may be column
+    slices of a fused projection output (equal row strides)."""
+    lib = _lib.load()
+    dev = _dev_of(query, key, value)
+    _dev_ok(out)
+    _need(query.dtype in _ACT and key.dtype == query.dtype and value.dtype == query.dtype, "dtype mismatch")
+    _need(query.dim() == 2 and key.dim() == 2 and value.dim() == 2, "query / key / value must be [T, heads * D]")
+    _need(n_heads % n_kv_heads == 0 and query.shape[1] % n_heads == 0, "head counts do not divide the row width")
+    d = query.shape[1] // n_heads
+    query, qs = _rows(query, n_heads * d, "query")
+    key, ks = _rows(key, n_kv_heads * d, "key")
+    value, vs = _rows(value, n_kv_heads * d, "value")
+    _need(ks == vs, "key and value must have the same row stride")
+    total_q = query.shape[0]
+    _need(key.shape[0] == total_q and value.shape[0] == total_q, "query, key and value must have the same number of rows")
+    b = _q_starts(q_starts, dev)
+    if out is None:
+        out = torch.empty((total_q, n_heads * d), dtype=query.dtype, device=dev)
+    else:
+        _need(out.numel() == total_q * n_heads * d and out.dtype == query.dtype and out.is_contiguous(), "out mismatch")
+    need = lib.mf_paged_attention_prefill_workspace_bytes(b, total_q, n_heads, n_kv_heads, d, total_q)
+    ws = workspace(need, dev, "pa_prefill") if need else None
+    check(lib.mf_paged_attention_prefill(ptr(out), ptr(query), ptr(key), ptr(value), None, None, ptr(q_starts), b,
+                                         total_q, n_heads, n_kv_heads, d, 0, 0, 0, float(scale), qs, ks,
+                                         dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,
+                                         stream_ptr(dev)), "mf_paged_attention_prefill")
+    return out
+
+
 # --------------------------------------------------------------------------------------------- norm / activation
 def rms_norm(x, gamma, eps, residual=None):
     """RmsNorm(eps)(x, gamma).  With ``residual``: returns (norm(x + residual), x + residual)."""

@@ -14,6 +14,10 @@ Pinning status of each function (what fixes it besides its own formula):
                            flash-attention decode vectors (tests/golden/flash_attention.npz)
   paged_attention_decode   reference vectors decode_output_{1,2} (flash_attention.npz,
                            attention.npz); reduces to softmax(QK^T s)V on the gathered prefix
+  causal_prefill_attention reference vectors prefill_output_{1,2} (flash_attention.npz, attention.npz)
+  paged_attention_prefill  its two special cases are the two pinned functions above: one query per
+                           sequence = paged_attention_decode, empty cache before the step =
+                           causal_prefill_attention (tests); the golden prefill vectors through the cache
   rope tables / apply      reference vectors (rotary.npz: default, Llama3, YaRN; prefill+decode)
   rms_norm / layer_norm    reference vectors (norm.npz)
   silu_mul                 reference vectors (activation.npz)
@@ -30,7 +34,8 @@ Pinning status of each function (what fixes it besides its own formula):
 from .numerics import (round_bf16, round_fp16, round_to, double_benchmark,
                        DoubleBenchmarkResult)
 from .attention import (reshape_and_cache, paged_attention_decode, gather_kv,
-                        decode_slot_mapping, prefill_slot_mapping, causal_prefill_attention)
+                        decode_slot_mapping, prefill_slot_mapping, causal_prefill_attention,
+                        paged_attention_prefill)
 from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_yarn,
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp

@@ -83,6 +83,44 @@ def paged_attention_decode(query, key_cache, value_cache, block_tables, context_
     return out.reshape(b_sz, n_head * d)
 
 
+def paged_attention_prefill(query, key_cache, value_cache, block_tables, context_lens, q_seq_lens,
+                            n_head, n_kv_head, scale, prob_dtype=None):
+    """PagedAttention with several new tokens per sequence and a causal mask among them (paged_attention_mgr.py:66-69
+    called with q_seq_lens; the mask is the lower triangle built by generation/parallel_decoding.py:73-80).
+
+    query [sum(q_seq_lens), n_head*D] packed sequence after sequence; the new tokens are already in the cache and
+    context_lens[b] counts them, so query i of sequence b sees cache tokens 0 .. L_b - q_len_b + i.  float64.
+    Pinned through its two special cases: one query per sequence is `paged_attention_decode`, and an empty
+    cache before the step is `causal_prefill_attention` (both pinned by the reference's golden outputs).
+    """
+    nb, bs, n_kv, d = key_cache.shape
+    assert n_kv == n_kv_head
+    t = int(np.sum(q_seq_lens))
+    q = np.asarray(query, dtype=np.float64).reshape(t, n_head, d)
+    n_rep = n_head // n_kv_head
+    out = np.zeros((t, n_head, d), dtype=np.float64)
+    start = 0
+    for b, q_len in enumerate(q_seq_lens):
+        q_len, length = int(q_len), int(context_lens[b])
+        if length > 0 and q_len > 0:
+            k = gather_kv(key_cache, block_tables[b], length).astype(np.float64)
+            v = gather_kv(value_cache, block_tables[b], length).astype(np.float64)
+            for i in range(q_len):
+                lim = length - q_len + i + 1
+                if lim <= 0:
+                    continue
+                for h in range(n_head):
+                    g = h // n_rep
+                    sc = (k[:lim, g, :] @ q[start + i, h]) * scale
+                    p = np.exp(sc - sc.max())
+                    p = p / p.sum()
+                    if prob_dtype is not None:
+                        p = round_to(p, prob_dtype).astype(np.float64)
+                    out[start + i, h] = p @ v[:lim, g, :]
+        start += q_len
+    return out.reshape(t, n_head * d)
+
+
 def causal_prefill_attention(query, key, value, seq_lens, n_head, n_kv_head, scale):
     """Varlen causal attention over packed [T, heads*D] rows (FlashAttentionScore, TH layout,
     flash_attention.py:129-134; unfused form infer_attention.py:342-404).  float64."""

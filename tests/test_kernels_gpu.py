@@ -216,6 +216,156 @@ def test_paged_attention_block_permutation_invariant():
     assert torch.equal(out1, out2)
 
 
+# ------------------------------------------------------------------------------------------- prefill attention
+def _starts(q_lens):
+    return np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+
+
+def _prefill_case(rng, dtype, nh, nkv, d, bs, lens, q_lens, max_blocks=None, pad_rows=0):
+    b = len(lens)
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype, max_blocks=max_blocks)
+    t = int(np.sum(q_lens))
+    q = rounded(rng.normal(size=(t + pad_rows, nh * d)), dtype)
+    scale = 1.0 / np.sqrt(d)
+    out = ops.paged_attention_prefill(dev(q, dtype), dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32),
+                                      dev(np.asarray(lens, np.int32), torch.int32), dev(_starts(q_lens), torch.int32),
+                                      nh, nkv, scale)
+    torch.cuda.synchronize()
+    ref = O.paged_attention_prefill(q[:t], kc, vc, tables, lens, q_lens, nh, nkv, scale)
+    mag = O.paged_attention_prefill(q[:t], kc, np.abs(vc), tables, lens, q_lens, nh, nkv, scale)
+    return to_np(out), ref, mag
+
+
+@pytest.mark.parametrize("dtype,nh,nkv,d,bs,lens,q_lens", [
+    (torch.bfloat16, 32, 8, 128, 128, [40, 300, 17], [40, 300, 17]),        # first prefill, ragged
+    (torch.bfloat16, 32, 8, 128, 128, [700, 900, 1300], [64, 1, 37]),       # chunks behind a long context
+    (torch.float16, 8, 2, 64, 16, [100, 33, 64, 5], [100, 0, 16, 5]),       # a sequence with no new tokens
+    (torch.bfloat16, 28, 4, 128, 128, [260, 130], [9, 130]),                # n_rep = 7: queries straddle column groups
+    (torch.bfloat16, 40, 2, 64, 32, [150, 90], [5, 90]),                    # n_rep = 20: a query spans two groups
+    (torch.float16, 2, 2, 32, 16, [50, 1], [50, 1]),                        # MHA
+    (torch.bfloat16, 4, 1, 128, 24, [200, 77], [31, 77]),                   # block size not a multiple of 32
+    (torch.bfloat16, 32, 8, 128, 128, [2100], [3]),                         # few queries, long context: partitions
+])
+def test_paged_prefill_vs_oracle(dtype, nh, nkv, d, bs, lens, q_lens):
+    rng = np.random.default_rng(nh * 100 + len(lens))
+    got, ref, mag = _prefill_case(rng, dtype, nh, nkv, d, bs, np.asarray(lens), np.asarray(q_lens))
+    assert_within(got, ref, mag, dtype, ulps=1.5, what="paged prefill")
+
+
+def test_paged_prefill_rows_of_no_sequence_are_zero():
+    """Rows past q_starts[batch] (padding of a fixed-size launch) come back as zeros, on both the single-partition
+    path and the partitioned one; a sequence that claims more queries than context only gets its context's worth."""
+    rng = np.random.default_rng(21)
+    dtype = torch.bfloat16
+    for lens, q_lens, mb in (([70, 20], [30, 20], None), ([1500], [2], None)):
+        got, ref, mag = _prefill_case(rng, dtype, 8, 2, 128, 128, np.asarray(lens), np.asarray(q_lens),
+                                      max_blocks=mb, pad_rows=5)
+        t = int(np.sum(q_lens))
+        assert_within(got[:t], ref, mag, dtype, ulps=1.5, what="padded launch")
+        assert np.all(got[t:] == 0)
+    kc, vc, tables, nb = make_paged_cache(rng, 1, [3], 2, 128, 128, dtype)
+    q = rounded(rng.normal(size=(6, 8 * 128)), dtype)
+    out = to_np(ops.paged_attention_prefill(dev(q, dtype), dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32),
+                                            dev(np.array([3], np.int32), torch.int32),
+                                            dev(np.array([0, 6], np.int32), torch.int32), 8, 2, 0.1))
+    ref = O.paged_attention_prefill(q[:3], kc, vc, tables, [3], [3], 8, 2, 0.1)
+    mag = O.paged_attention_prefill(q[:3], kc, np.abs(vc), tables, [3], [3], 8, 2, 0.1)
+    assert_within(out[:3], ref, mag, dtype, ulps=1.5, what="clamped query count")
+    assert np.all(out[3:] == 0)
+
+
+def test_paged_prefill_one_query_per_sequence_is_decode():
+    rng = np.random.default_rng(22)
+    dtype = torch.bfloat16
+    b, nh, nkv, d, bs = 5, 32, 8, 128, 128
+    lens = rng.integers(100, 1200, b)
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype)
+    q = dev(rng.normal(size=(b, nh * d)), dtype)
+    args = (dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32))
+    dec = to_np(ops.paged_attention(q, *args, nh, nkv, 0.088))
+    pre = to_np(ops.paged_attention_prefill(q, *args, dev(_starts(np.ones(b, np.int64)), torch.int32), nh, nkv, 0.088))
+    mag = O.paged_attention_decode(to_np(q), kc, np.abs(vc), tables, lens, nh, nkv, 0.088)
+    assert_within(pre, dec, mag, dtype, ulps=2.0, what="prefill with one query vs decode")
+
+
+def test_chunked_prefill_matches_whole_prefill():
+    """Scatter and attend chunk by chunk (the cache grows between chunks) against one prefill of the whole prompt."""
+    rng = np.random.default_rng(23)
+    dtype = torch.bfloat16
+    nh, nkv, d, bs = 16, 4, 128, 128
+    lens = np.array([300, 190])
+    b = len(lens)
+    kc0, vc0, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype)
+    t = int(lens.sum())
+    q = rounded(rng.normal(size=(t, nh * d)), dtype)
+    tb, starts = dev(tables, torch.int32), _starts(lens)
+    whole = to_np(ops.paged_attention_prefill(dev(q, dtype), dev(kc0, dtype), dev(vc0, dtype), tb,
+                                              dev(lens.astype(np.int32), torch.int32), dev(starts, torch.int32),
+                                              nh, nkv, 0.09))
+    chunk = 128
+    got = np.zeros_like(whole)
+    done = np.zeros(b, np.int64)
+    while (done < lens).any():
+        step = np.minimum(chunk, lens - done)
+        rows = np.concatenate([np.arange(starts[i] + done[i], starts[i] + done[i] + step[i]) for i in range(b)])
+        done = done + step
+        out = ops.paged_attention_prefill(dev(q[rows], dtype), dev(kc0, dtype), dev(vc0, dtype), tb,
+                                          dev(done.astype(np.int32), torch.int32), dev(_starts(step), torch.int32),
+                                          nh, nkv, 0.09)
+        got[rows] = to_np(out)
+    mag = O.paged_attention_prefill(q, kc0, np.abs(vc0), tables, lens, lens, nh, nkv, 0.09)
+    assert_within(got, whole, mag, dtype, ulps=2.0, what="chunked vs whole prefill")
+
+
+@pytest.mark.parametrize("dtype,nh,nkv,d,q_lens,fused", [
+    (torch.bfloat16, 32, 8, 128, [130, 1, 64], True),
+    (torch.float16, 8, 2, 64, [33, 200], False),
+    (torch.bfloat16, 4, 4, 32, [17], False),
+])
+def test_causal_attention_varlen_vs_oracle(dtype, nh, nkv, d, q_lens, fused):
+    """Keys and values taken from this step's own packed rows (no cache), optionally as column slices of one fused
+    projection output."""
+    rng = np.random.default_rng(nh + d)
+    t = int(np.sum(q_lens))
+    nq, nk = nh * d, nkv * d
+    qkv = rounded(rng.normal(size=(t, nq + 2 * nk)), dtype)
+    qkv_d = dev(qkv, dtype)
+    q, k, v = qkv_d[:, :nq], qkv_d[:, nq:nq + nk], qkv_d[:, nq + nk:]
+    if not fused:
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    scale = 1.0 / np.sqrt(d)
+    out = to_np(ops.causal_attention_varlen(q, k, v, dev(_starts(q_lens), torch.int32), nh, nkv, scale))
+    ref = O.causal_prefill_attention(qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:], q_lens, nh, nkv, scale)
+    mag = O.causal_prefill_attention(qkv[:, :nq], qkv[:, nq:nq + nk], np.abs(qkv[:, nq + nk:]), q_lens, nh, nkv, scale)
+    assert_within(out, ref, mag, dtype, ulps=1.5, what="varlen causal attention")
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_prefill_reference_vectors(golden_dir, case, n_kv):
+    """prefill_output_{1,2} of the reference's flash-attention unit test, from the packed rows and through the cache."""
+    z = np.load(os.path.join(golden_dir, "flash_attention.npz"))
+    nb, bs = int(z["meta_num_blocks"]), int(z["meta_block_size"])
+    nh, hid = int(z["meta_num_heads"]), int(z["meta_hidden_size"])
+    d = hid // nh
+    dt = torch.bfloat16
+    q = dev(z[f"in{case}_prefill_query"].reshape(4, -1), dt)
+    k = dev(z[f"in{case}_prefill_key"].reshape(4, -1), dt)
+    v = dev(z[f"in{case}_prefill_value"].reshape(4, -1), dt)
+    starts = dev(np.array([0, 2, 4], np.int32), torch.int32)
+    out = ops.causal_attention_varlen(q, k, v, starts, nh, n_kv, 0.25)
+    res = O.double_benchmark(to_np(out), z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"])
+    assert res.ok, res.messages
+    kc = torch.zeros(nb, bs, n_kv, d, dtype=dt, device="cuda")
+    vc = torch.zeros_like(kc)
+    ops.reshape_and_cache(k, v, kc, vc, dev(z[f"in{case}_prefill_slot_mapping"].astype(np.int32), torch.int32))
+    bt = -np.ones((2, 11), np.int32)
+    bt[0, 0], bt[1, 0] = 2, 1
+    out2 = ops.paged_attention_prefill(q, kc, vc, dev(bt, torch.int32), dev(np.array([2, 2], np.int32), torch.int32),
+                                       starts, nh, n_kv, 0.25)
+    res = O.double_benchmark(to_np(out2), z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"])
+    assert res.ok, res.messages
+
+
 # ------------------------------------------------------------------------------------------- norm / activation
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,cols,gdt", [(64, 4096, torch.float32), (4, 512, torch.float16), (3, 8192, torch.bfloat16), (1, 32, torch.float32)])

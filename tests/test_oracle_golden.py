@@ -55,6 +55,43 @@ def test_flash_attention_vectors(golden_dir, case, n_kv):
 
 
 @pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_paged_prefill_oracle_is_pinned_by_its_special_cases(golden_dir, case, n_kv):
+    """Several new tokens per sequence over the cache: with an empty cache before the step it must give the
+    reference's prefill vectors, with one query per sequence the decode vectors, and a prefill cut into two
+    chunks must give what the whole prefill gives."""
+    z = _load(golden_dir, "flash_attention.npz")
+    nb, bs = int(z["meta_num_blocks"]), int(z["meta_block_size"])
+    nh, hid = int(z["meta_num_heads"]), int(z["meta_hidden_size"])
+    d = hid // nh
+    scale = 0.25
+    pq = R(z[f"in{case}_prefill_query"]).reshape(4, -1)
+    pk = R(z[f"in{case}_prefill_key"]).reshape(4, -1)
+    pv = R(z[f"in{case}_prefill_value"]).reshape(4, -1)
+    kc = np.zeros((nb, bs, n_kv, d), np.float32)
+    vc = np.zeros_like(kc)
+    O.reshape_and_cache(pk, pv, kc, vc, z[f"in{case}_prefill_slot_mapping"])
+    bt = -np.ones((2, 11), np.int32)
+    bt[0, 0], bt[1, 0] = 2, 1
+    pre = O.paged_attention_prefill(pq, kc, vc, bt, [2, 2], [2, 2], nh, n_kv, scale)
+    _check(pre, z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"], "prefill through the cache")
+    np.testing.assert_allclose(pre, O.causal_prefill_attention(pq, pk, pv, [2, 2], nh, n_kv, scale), rtol=1e-12)
+    # a mask shifted by one token must fail the reference's criterion
+    shifted = O.paged_attention_prefill(pq[[1, 3]], kc, vc, bt, [2, 2], [1, 1], nh, n_kv, scale)
+    first = O.paged_attention_prefill(pq[[0, 2]], kc, vc, bt, [1, 1], [1, 1], nh, n_kv, scale)
+    np.testing.assert_allclose(np.stack([first[0], shifted[0], first[1], shifted[1]]), pre, rtol=1e-12)   # chunks
+    assert not np.allclose(O.paged_attention_prefill(pq[[0, 2]], kc, vc, bt, [2, 2], [1, 1], nh, n_kv, scale),
+                           pre[[0, 2]], rtol=1e-3)
+
+    dk = R(z[f"in{case}_decoder_key"]).reshape(2, -1)
+    dv = R(z[f"in{case}_decoder_value"]).reshape(2, -1)
+    O.reshape_and_cache(dk, dv, kc, vc, z[f"in{case}_decoder_slot_mapping"])
+    dq = R(z[f"in{case}_decoder_query"]).reshape(2, -1)
+    dec = O.paged_attention_prefill(dq, kc, vc, bt, [3, 3], [1, 1], nh, n_kv, scale)
+    _check(dec, z[f"gpu_decode_output_{case}"], z[f"golden_decode_output_{case}"], "one query per sequence")
+    np.testing.assert_allclose(dec, O.paged_attention_decode(dq, kc, vc, bt, [3, 3], nh, n_kv, scale), rtol=1e-12)
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
 def test_self_attention_vectors(golden_dir, case, n_kv):
     """QKV linear -> [q|k|v] split -> scatter -> prefill FA / decode PA -> projection
     (attention.py:214-265,344-349; scale 1/sqrt(head_dim), attention.py:135,166)."""
