@@ -8,7 +8,9 @@ from .. import ops
 
 
 class FlashAttention(nn.Module):
-    """ReshapeAndCache, then FlashAttentionScore (prefill; not built) or PagedAttention (decode)."""
+    """ReshapeAndCache, then FlashAttentionScore (prefill) or PagedAttention (decode; with q_seq_lens: several new
+    tokens per sequence).  Masks are causal: `attn_mask` is accepted for signature parity and taken to be the lower
+    triangle the reference's models build; sparse modes other than the causal default are not built."""
 
     def __init__(self, head_num, head_dim=None, kv_head_num=None, keep_prob=1.0, scale_value=1.0,
                  pre_tokens=2147483647, next_tokens=2147483647, sparse_mode=0, input_layout="TH",
@@ -33,12 +35,37 @@ class FlashAttention(nn.Module):
                 attn_mask=None, padding_mask=None, prefix=None, key_cache=None, value_cache=None):
         """Forward process of the FlashAttention (flash_attention.py:109-145)."""
         ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
-        if self.is_prefill:
-            raise NotImplementedError("prefill (FlashAttentionScore) is not built: set is_prefill = False")
         shape = query.shape
-        out = ops.paged_attention(query.reshape(-1, shape[-1]) if query.dim() > 2 else query, key_cache, value_cache,
-                                  block_tables, batch_valid_length, self.head_num, self.pa_kv_head_num,
-                                  self.scale_value)
+        if query.dim() == 2:
+            q2 = query
+        elif self.input_layout == "TND":
+            q2 = query.reshape(shape[0], -1)
+        else:
+            q2 = query.reshape(-1, shape[-1])
+        if self.is_prefill:
+            # FlashAttentionScore over this step's packed rows (flash_attention.py:129-134); keys are the step's own,
+            # so the query and key lists must agree
+            if actual_seq_kvlen is not None and actual_seq_kvlen is not actual_seq_qlen:
+                if not torch.equal(torch.as_tensor(actual_seq_kvlen).cpu(), torch.as_tensor(actual_seq_qlen).cpu()):
+                    raise NotImplementedError("prefill with actual_seq_kvlen != actual_seq_qlen is not built "
+                                              "(use the decode branch with q_seq_lens for chunked prefill)")
+            if actual_seq_qlen is None:
+                starts = torch.tensor([0, q2.shape[0]], dtype=torch.int32, device=query.device)
+            else:
+                starts = ops.q_starts_from_actual_seq_len(torch.as_tensor(actual_seq_qlen, device=query.device),
+                                                          q2.shape[0])
+            k2 = key if key.dim() == 2 else key.reshape(q2.shape[0], -1)
+            v2 = value if value.dim() == 2 else value.reshape(q2.shape[0], -1)
+            out = ops.causal_attention_varlen(q2, k2, v2, starts, self.head_num,
+                                              self.pa_kv_head_num, self.scale_value)
+            return out.reshape(shape)
+        if q_seq_lens is not None:                            # several new tokens per sequence (flash_attention.py:140-143)
+            out = ops.paged_attention_prefill(q2, key_cache, value_cache, block_tables, batch_valid_length,
+                                              ops.q_starts_from_lens(q_seq_lens), self.head_num,
+                                              self.pa_kv_head_num, self.scale_value)
+            return out.reshape(shape)
+        out = ops.paged_attention(q2, key_cache, value_cache, block_tables, batch_valid_length, self.head_num,
+                                  self.pa_kv_head_num, self.scale_value)
         return out.reshape(shape)
 
     construct = forward

@@ -35,9 +35,11 @@ class InferRotaryEmbedding(nn.Module):
 class InferAttention(nn.Module):
     """Infer Attention Layer (infer_attention.py:209-231 constructor, :441-463 call).
 
-    query [B, 1, n_head*D] (BSH) or [T, n_head*D] (TH); decode only: `is_first_iteration` must be False when
-    called (prefill FlashAttentionScore is not on the built path).  `batch_valid_length` is the context length
-    including the token written by this call."""
+    query [B, S, n_head*D] (BSH) or [T, n_head*D] / [1, T, n_head*D] (TH).  Decode: `batch_valid_length` is the
+    context length including the token written by this call.  Prefill (`is_first_iteration`): causal attention over
+    this call's own keys; in the TH layout `batch_valid_length` (the lengths of the packed sequences, or their
+    increasing row ends) is what the reference hands to FlashAttentionScore (infer_attention.py:459-461), in BSH
+    every batch row is a full sequence of S tokens.  Masks are causal; `attn_mask` is not read."""
 
     def __init__(self, n_head, head_dim, n_kv_head, pa_n_head_split=None, pa_n_kv_head_split=None, keep_prob=1.0,
                  scale_value=1.0, pre_tokens=2147483647, next_tokens=2147483647, sparse_mode=0, block_size=16,
@@ -90,24 +92,40 @@ class InferAttention(nn.Module):
 
     def forward(self, query, key, value, batch_valid_length, block_tables, slot_mapping, freqs_cis=None,
                 attn_mask=None, alibi_mask=None, prefix_keys_values=None, q_seq_lens=None):
-        """Forward process of the Infer Attention Cell (infer_attention.py:441-463), decode branch."""
+        """Forward process of the Infer Attention Cell (infer_attention.py:441-463)."""
         if prefix_keys_values is not None:
             raise NotImplementedError("prefix_keys_values (p-tuning prefix) is not built")
-        if self.is_first_iteration:
-            raise NotImplementedError("prefill attention (FlashAttentionScore) is not built: set "
-                                      "is_first_iteration = False and call with one new token per sequence")
         mgr = self.paged_attention_mgr
+        shape = query.shape
+        q2 = query.reshape(-1, self.n_head * self.head_dim).contiguous()
+        k2 = key.reshape(-1, self.n_kv_head * self.head_dim).contiguous()
+        v2 = value.reshape(-1, self.n_kv_head * self.head_dim).contiguous()
         if self.use_rope_rotary_emb:
             # RoPE + scatter of the rotated key and of value in one launch (infer_attention.py:445,453);
             # same-stream ordering stands in for ops.depend (:454)
             freqs_cos, freqs_sin, _ = freqs_cis
-            query = query.contiguous()
-            key = key.contiguous()
-            ops.rope_and_cache(query, key, value.contiguous(), freqs_cos.contiguous(), freqs_sin.contiguous(),
-                               mgr.key_cache, mgr.value_cache, slot_mapping, self.n_head)
+            ops.rope_and_cache(q2, k2, v2, freqs_cos.contiguous(), freqs_sin.contiguous(), mgr.key_cache,
+                               mgr.value_cache, slot_mapping, self.n_head)
         else:
-            mgr(key, value, slot_mapping, batch_valid_length)
-        return self._incre_attention(query, batch_valid_length, block_tables, alibi_mask, attn_mask, q_seq_lens)
+            mgr(k2, v2, slot_mapping, batch_valid_length)
+        if self.chunk_prefill:                                # infer_attention.py:456-458
+            return mgr.paged_attn(q2, batch_valid_length, block_tables, attn_mask=attn_mask,
+                                  q_seq_lens=q_seq_lens).reshape(shape)
+        if self.is_first_iteration:
+            return self._prefill_attention(q2, k2, v2, attn_mask, alibi_mask, batch_valid_length,
+                                           batch_valid_length, shape).reshape(shape)
+        return self._incre_attention(q2, batch_valid_length, block_tables, alibi_mask, attn_mask,
+                                     q_seq_lens).reshape(shape)
+
+    def _prefill_attention(self, query, key, value, attn_mask, alibi_mask, actual_seq_qlen=None,
+                           actual_seq_kvlen=None, shape=None):
+        """FlashAttentionScore of the first iteration (infer_attention.py:405-431) on packed [T, H] rows."""
+        if self.input_layout == "TH":
+            starts = ops.q_starts_from_actual_seq_len(actual_seq_qlen, query.shape[0])
+        else:                                                 # BSH: every batch row is one sequence of S tokens
+            bsz, seq = shape[0], shape[1]
+            starts = torch.arange(0, bsz + 1, dtype=torch.int32, device=query.device) * seq
+        return ops.causal_attention_varlen(query, key, value, starts, self.n_head, self.n_kv_head, self.scale_value)
 
     construct = forward
 

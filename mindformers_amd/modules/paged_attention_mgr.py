@@ -20,8 +20,6 @@ class PagedAttentionMgr(nn.Module):
             raise ValueError(f"kv_shape must be (num_blocks, block_size, n_kv_heads, head_dim), got {kv_shape}")
         if kv_shape[2] != n_kv_heads or kv_shape[3] != head_dim:
             raise ValueError(f"kv_shape {kv_shape} does not match n_kv_heads={n_kv_heads}, head_dim={head_dim}")
-        if parallel_decoding or chunk_prefill:
-            raise NotImplementedError("parallel_decoding / chunk_prefill (masked multi-token PagedAttention) is not built")
         self.n_heads = n_heads
         self.head_dim = head_dim
         self.n_kv_heads = n_kv_heads
@@ -40,10 +38,20 @@ class PagedAttentionMgr(nn.Module):
     construct = forward
 
     def paged_attn(self, query, batch_valid_length, block_tables, attn_mask=None, q_seq_lens=None):
-        """The forward compute of Paged Attention (paged_attention_mgr.py:64-70)."""
+        """The forward compute of Paged Attention (paged_attention_mgr.py:64-70).  With parallel_decoding or
+        chunk_prefill every sequence brings q_seq_lens[b] new tokens, masked causally among themselves: `attn_mask` is
+        taken to be that lower triangle (generation/parallel_decoding.py:73-80) and is not read."""
         shape = query.shape
-        out = ops.paged_attention(query.reshape(-1, self.n_heads * self.head_dim), self.key_cache, self.value_cache,
-                                  block_tables, batch_valid_length, self.n_heads, self.n_kv_heads, self.scale_value)
+        q2 = query.reshape(-1, self.n_heads * self.head_dim)
+        if self.parallel_decoding or self.chunk_prefill:
+            if q_seq_lens is None:
+                raise ValueError("parallel_decoding / chunk_prefill need q_seq_lens")
+            out = ops.paged_attention_prefill(q2, self.key_cache, self.value_cache, block_tables, batch_valid_length,
+                                              ops.q_starts_from_lens(q_seq_lens), self.n_heads, self.n_kv_heads,
+                                              self.scale_value)
+        else:
+            out = ops.paged_attention(q2, self.key_cache, self.value_cache, block_tables, batch_valid_length,
+                                      self.n_heads, self.n_kv_heads, self.scale_value)
         return out.reshape(shape)
 
     def paged_attn_with_alibi(self, query, batch_valid_length, block_tables, alibi_tensor):

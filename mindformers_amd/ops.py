@@ -172,6 +172,28 @@ def _q_starts(q_starts, dev):
     return q_starts.numel() - 1
 
 
+def q_starts_from_ends(ends):
+    """int32 [B + 1] row offsets from FlashAttentionScore's actual_seq_qlen (increasing ends, the last = T)."""
+    ends = ends.to(torch.int32).reshape(-1)
+    return torch.cat([torch.zeros(1, dtype=torch.int32, device=ends.device), ends])
+
+
+def q_starts_from_actual_seq_len(actual_seq_len, total_rows):
+    """Row offsets from the `actual_seq_qlen` a caller hands to FlashAttentionScore in the TH layout.  The operator
+    documents increasing row ends whose last value is T; the reference's own callers and unit test pass the
+    per-sequence lengths (infer_attention.py:459-461, run_infer_flash_attention.py:110,137-142).  The two readings
+    never disagree when both are valid (then all entries but the last are zero), so the list is taken as ends when
+    it is non-decreasing and ends at T, and as lengths otherwise.  Decided on the device: no host synchronisation."""
+    a = torch.as_tensor(actual_seq_len).reshape(-1).to(torch.int64)
+    is_ends = (a[-1] == total_rows) & torch.all(a[1:] >= a[:-1])
+    return q_starts_from_ends(torch.where(is_ends, a, torch.cumsum(a, 0)))
+
+
+def q_starts_from_lens(q_seq_lens):
+    """int32 [B + 1] row offsets from PagedAttention's q_seq_lens (new tokens per sequence)."""
+    return q_starts_from_ends(torch.cumsum(q_seq_lens.reshape(-1), 0))
+
+
 def paged_attention_prefill(query, key_cache, value_cache, block_tables, context_lens, q_starts, n_heads,
                             n_kv_heads, scale, out=None):
     """Causal attention of several new tokens per sequence over the paged cache (their keys/values already

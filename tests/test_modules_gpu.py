@@ -61,8 +61,6 @@ def test_infer_attention_decode_step(dynamic):
     attn = InferAttention(n_head, d, n_kv, scale_value=1 / np.sqrt(d), block_size=bs, num_blocks=nb, seq_length=seq,
                           is_dynamic=dynamic, rotary_cos_format=2, compute_dtype=dt)
     assert attn.is_first_iteration and attn.paged_attention_mgr.key_cache.shape == (nb, bs, n_kv, d)
-    with pytest.raises(NotImplementedError):              # prefill is not on the built path
-        attn(None, None, None, None, None, None)
     attn.is_first_iteration = False
     mgr = BlockTables(nb, bs, seq)
     mgr.init_cache_engine(b)
@@ -100,6 +98,102 @@ def test_infer_attention_decode_step(dynamic):
 
 
 @pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
+def test_mcore_flash_attention_prefill_vectors(golden_dir, case, n_kv):
+    """The reference's FlashAttention unit test, prefill half (run_infer_flash_attention.py:106-150): the cell
+    scatters the prompt's K/V and runs causal attention over them; actual_seq_qlen is passed as the test passes it
+    (the per-sequence lengths) and as the operator documents it (increasing row ends)."""
+    from mindformers_amd.modules import FlashAttention
+    z = np.load(os.path.join(golden_dir, "flash_attention.npz"))
+    nb, bs, nh, hid = (int(z[k]) for k in ("meta_num_blocks", "meta_block_size", "meta_num_heads", "meta_hidden_size"))
+    d = hid // nh
+    net = FlashAttention(head_num=nh, head_dim=d, keep_prob=1.0, kv_head_num=n_kv, pa_kv_head_num=n_kv, scale_value=0.25)
+    assert net.is_prefill
+    bt = -np.ones((2, 11), np.int32)
+    bt[0, 0], bt[1, 0] = 2, 1
+    mask = torch.triu(torch.ones(2, 2, dtype=BF, device="cuda"), diagonal=1)
+    for lens in ([2, 2], [2, 4]):
+        kc = torch.zeros(nb, bs, n_kv, d, dtype=BF, device="cuda")
+        vc = torch.zeros_like(kc)
+        lens_t = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        out = net(query=dev(z[f"in{case}_prefill_query"].reshape(4, -1), BF), key=dev(z[f"in{case}_prefill_key"].reshape(4, -1), BF),
+                  value=dev(z[f"in{case}_prefill_value"].reshape(4, -1), BF),
+                  slot_mapping=dev(z[f"in{case}_prefill_slot_mapping"].astype(np.int32), torch.int32),
+                  block_tables=dev(bt, torch.int32), actual_seq_qlen=lens_t, actual_seq_kvlen=lens_t,
+                  batch_valid_length=lens_t, context_lens_tensor=lens_t, attn_mask=mask, key_cache=kc, value_cache=vc)
+        res = O.double_benchmark(to_np(out), z[f"gpu_prefill_output_{case}"], z[f"golden_prefill_output_{case}"])
+        assert res.ok, (lens, res.messages)
+        # the prompt's keys are in the cache afterwards
+        slots = z[f"in{case}_prefill_slot_mapping"].astype(np.int64)
+        assert np.array_equal(to_np(kc).reshape(nb * bs, -1)[slots], to_np(dev(z[f"in{case}_prefill_key"].reshape(4, -1), BF)))
+
+
+def test_infer_attention_prefill_chunks_and_decode_agree():
+    """InferAttention over a whole prompt (first iteration, TH and BSH), the same prompt fed in chunks through the
+    chunk_prefill path, and the oracle, all on the same cache and RoPE tables."""
+    from mindformers_amd.modules import FreqsMgr, InferAttention
+    rng = np.random.default_rng(5)
+    n_head, n_kv, d, bs, nb, seq = 8, 2, 64, 16, 64, 256
+    dt = torch.float16
+    lens = np.array([40, 23])
+    b, t = len(lens), int(lens.sum())
+    starts = np.concatenate([[0], np.cumsum(lens)])
+    q = rounded(rng.normal(size=(t, n_head * d)), dt)
+    k = rounded(rng.normal(size=(t, n_kv * d)), dt)
+    v = rounded(rng.normal(size=(t, n_kv * d)), dt)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    freqs = FreqsMgr(d, seq_length=seq, max_position_embedding=seq, rotary_dtype=dt)
+    cos_all, sin_all = freqs.freqs_cos, freqs.freqs_sin
+    pos_t = torch.from_numpy(pos).cuda()
+    freqs_cis = (cos_all[pos_t].contiguous(), sin_all[pos_t].contiguous(), None)
+    tables = np.stack([np.arange(4) + 4 * i for i in range(b)]).astype(np.int32)          # 4 blocks per sequence
+    slots = np.concatenate([tables[i][np.arange(n) // bs] * bs + np.arange(n) % bs for i, n in enumerate(lens)]).astype(np.int32)
+    scale = 1 / np.sqrt(d)
+    q_r = rounded(O.apply_rotary_half(q, to_np(freqs_cis[0]), to_np(freqs_cis[1]), n_head), dt)
+    k_r = rounded(O.apply_rotary_half(k, to_np(freqs_cis[0]), to_np(freqs_cis[1]), n_kv), dt)
+    ref = O.causal_prefill_attention(q_r, k_r, v, lens, n_head, n_kv, scale)
+    mag = O.causal_prefill_attention(q_r, k_r, np.abs(v), lens, n_head, n_kv, scale)
+
+    def make(**kw):
+        return InferAttention(n_head, d, n_kv, scale_value=scale, block_size=bs, num_blocks=nb, seq_length=seq,
+                              rotary_cos_format=2, compute_dtype=dt, **kw)
+
+    attn = make(is_dynamic=True)
+    out = attn(dev(q, dt).reshape(1, t, -1), dev(k, dt).reshape(1, t, -1), dev(v, dt).reshape(1, t, -1),
+               torch.from_numpy(lens.astype(np.int32)).cuda(), torch.from_numpy(tables).cuda(),
+               torch.from_numpy(slots).cuda(), freqs_cis)
+    assert out.shape == (1, t, n_head * d)
+    assert_within(to_np(out).reshape(t, -1), ref, mag, dt, ulps=4.0, what="InferAttention prefill (TH)")
+    got_k = to_np(attn.paged_attention_mgr.key_cache).reshape(-1, n_kv * d)[slots]
+    assert np.abs(got_k - k_r).max() <= 2 * EPS[dt] * np.abs(k_r).max()
+
+    # BSH: one sequence per batch row, equal lengths
+    s_len = 23
+    rows = np.concatenate([np.arange(starts[i], starts[i] + s_len) for i in range(b)])
+    attn_b = make(is_dynamic=False)
+    fc = (freqs_cis[0][rows].contiguous(), freqs_cis[1][rows].contiguous(), None)
+    out_b = attn_b(dev(q[rows], dt).reshape(b, s_len, -1), dev(k[rows], dt).reshape(b, s_len, -1),
+                   dev(v[rows], dt).reshape(b, s_len, -1), torch.full((b,), s_len, dtype=torch.int32, device="cuda"),
+                   torch.from_numpy(tables).cuda(), torch.from_numpy(slots[rows]).cuda(), fc)
+    assert out_b.shape == (b, s_len, n_head * d)
+    assert_within(to_np(out_b).reshape(b * s_len, -1), ref[rows], mag[rows], dt, ulps=4.0, what="InferAttention prefill (BSH)")
+
+    # chunked prefill: 16 new tokens per sequence and call, the cache grows between calls
+    attn_c = make(is_dynamic=True, chunk_prefill=True)
+    got = np.zeros((t, n_head * d), np.float32)
+    done = np.zeros(b, np.int64)
+    while (done < lens).any():
+        step = np.minimum(16, lens - done)
+        rows = np.concatenate([np.arange(starts[i] + done[i], starts[i] + done[i] + step[i]) for i in range(b)])
+        done = done + step
+        fc = (freqs_cis[0][rows].contiguous(), freqs_cis[1][rows].contiguous(), None)
+        o = attn_c(dev(q[rows], dt), dev(k[rows], dt), dev(v[rows], dt), torch.from_numpy(done.astype(np.int32)).cuda(),
+                   torch.from_numpy(tables).cuda(), torch.from_numpy(slots[rows]).cuda(), fc,
+                   q_seq_lens=torch.from_numpy(step.astype(np.int32)).cuda())
+        got[rows] = to_np(o)
+    assert_within(got, ref, mag, dt, ulps=4.0, what="InferAttention chunked prefill")
+
+
+@pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
 def test_mcore_flash_attention_decode_vectors(golden_dir, case, n_kv):
     """The reference's FlashAttention unit test, decode half (run_infer_flash_attention.py:150-180): caches are
     passed per call, the cell scatters the new K/V and attends."""
@@ -113,9 +207,6 @@ def test_mcore_flash_attention_decode_vectors(golden_dir, case, n_kv):
     vc = torch.zeros_like(kc)
     ops.reshape_and_cache(dev(z[f"in{case}_prefill_key"].reshape(4, -1), BF), dev(z[f"in{case}_prefill_value"].reshape(4, -1), BF),
                           kc, vc, dev(z[f"in{case}_prefill_slot_mapping"].astype(np.int32), torch.int32))
-    with pytest.raises(NotImplementedError):
-        net(None, dev(z[f"in{case}_decoder_key"].reshape(2, -1), BF), dev(z[f"in{case}_decoder_value"].reshape(2, -1), BF),
-            slot_mapping=dev(z[f"in{case}_decoder_slot_mapping"].astype(np.int32), torch.int32), key_cache=kc, value_cache=vc)
     net.is_prefill = False
     bt = -np.ones((2, 11), np.int32)
     bt[0, 0], bt[1, 0] = 2, 1
