@@ -226,6 +226,63 @@ def bench_moe(args, torch, ops, _lib):
     print(json.dumps(result), flush=True)
 
 
+def bench_prefill_attention(args, torch, ops):
+    """Causal attention of a Llama-3-8B-shaped prefill step over the paged cache (32 q / 8 kv heads x 128, bf16,
+    block 128): `llama3_8b_prefill_attention` = 4 prompts of 2048 tokens, `llama3_8b_chunked_prefill_attention` =
+    4 sequences adding 512 tokens behind 3584 cached ones.  A step is one attention call; flops = 4 * D * heads *
+    (query, key) pairs inside the causal limit."""
+    nh, nkv, d, bs, dt = 32, 8, 128, 128, torch.bfloat16
+    chunked = args.workload == "llama3_8b_chunked_prefill_attention"
+    lens = np.full(4, 4096 if chunked else 2048)
+    q_lens = np.full(4, 512 if chunked else 2048)
+    need = (lens + bs - 1) // bs
+    nb = int(need.sum()) + 1
+    tables = -np.ones((len(lens), int(need.max())), np.int32)
+    perm, pos = np.random.default_rng(0).permutation(nb), 0
+    for i, n in enumerate(need):
+        tables[i, :n] = perm[pos:pos + n]
+        pos += n
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    kc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
+    vc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
+    t = int(q_lens.sum())
+    q = torch.randn(t, nh * d, generator=gen, device="cuda").to(dt)
+    starts = torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device="cuda")
+    lens_t = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    tb = torch.tensor(tables, device="cuda")
+    out = torch.empty_like(q)
+
+    def step():
+        return ops.paged_attention_prefill(q, kc, vc, tb, lens_t, starts, nh, nkv, d ** -0.5, out=out)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    us = time_events(step, args.kernel_iters, torch)[0] * 1e3
+    pairs = int(sum(int(ql) * (int(L) - int(ql)) + int(ql) * (int(ql) + 1) // 2 for L, ql in zip(lens, q_lens)))
+    flops = 4.0 * d * nh * pairs
+    ach = flops / (us * 1e-6) / 1e12
+    peak = 2500.0
+    result = {
+        "metric": "prefill attention query tokens/sec per layer (Llama3-8B heads, bf16); % of dense bf16 MFMA peak",
+        "value": round(t / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: causal attention over the paged cache, {len(lens)} sequences, "
+                               f"{int(q_lens[0])} new tokens each, context {int(lens[0])}, 32q/8kv heads x 128, block 128",
+                   "launch": "eager", "flops_per_step": flops},
+        "roofline": dict(bound="mfma", kernel="paged_attention_kernel<PF> (+ partition reduce when partitioned)",
+                         achieved=round(ach, 1), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4), traffic=None,
+                         flops_per_launch=flops, avg_launch_us=round(us, 2)),
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,6 +312,9 @@ def main():
 
     if args.workload == "deepseek_v3_moe_w8a16":
         bench_moe(args, torch, ops, _lib)
+        return
+    if args.workload in ("llama3_8b_prefill_attention", "llama3_8b_chunked_prefill_attention"):
+        bench_prefill_attention(args, torch, ops)
         return
 
     t0 = time.perf_counter()
