@@ -26,6 +26,8 @@ Pinning status of each function (what fixes it besides its own formula):
    permute + experts)      group limiting not exercised there)
   topk_router group limit  brute force over subsets on tiny sizes (tests) — the reference
                            holds no vector that exercises n_group > topk_group
+  checkpoint.qkv/ffn_      hand-computed small cases; labelled rows (every output row must carry the
+   concat_hf2mg            (kind, head, channel) label the layout names); closed form (a permutation)
   quantize_weight_int8,    PARITY UNPINNED: the arithmetic lives in mindspore_gs / CANN
   w8a16_linear,            (not vendored, no reference vector).  int32 accumulators are
   dynamic_quant_per_token, pinned against exact integer matmul; rounding mode, clamp range
@@ -41,6 +43,7 @@ from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_ya
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp
 from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token,
                     int8_gemm_i32, w8a8_linear)
+from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,
                   grouped_matmul)
 from .layer import decode_layer_w8a16, decode_layer_w8a8

@@ -530,3 +530,65 @@ def test_decode_layer_graph_replay_is_bit_identical():
         assert torch.equal(out, eager)
         layer(*args)
         torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------------------------------- checkpoint -> layer
+@pytest.mark.parametrize("fmt", ["hf_float", "mg_fused_float", "int8_with_scales"])
+def test_layer_loaded_from_a_checkpoint_matches_oracle(tmp_path, fmt):
+    """A decode layer built from a safetensors checkpoint (HuggingFace names with float weights, the reference's
+    fused per-kv-group / interleaved layouts, or pre-quantized int8 + w_scale) runs the same step as the oracle on
+    the weights quantized with the declared convention."""
+    from safetensors.numpy import save_file
+    from mindformers_amd import checkpoint as C, synthetic
+    rng = np.random.default_rng(13)
+    nh, nkv, d, ffn, layer_idx = 8, 2, 64, 1024, 2
+    hidden = nh * d
+    cfg = dict(num_heads=nh, n_kv_heads=nkv, hidden_size=hidden, intermediate_size=ffn, qkv_concat=False)
+    p = f"model.layers.{layer_idx}."
+    hf = {}
+    for name, shape in (("self_attn.q_proj", (hidden, hidden)), ("self_attn.k_proj", (nkv * d, hidden)),
+                        ("self_attn.v_proj", (nkv * d, hidden)), ("self_attn.o_proj", (hidden, hidden)),
+                        ("mlp.gate_proj", (ffn, hidden)), ("mlp.up_proj", (ffn, hidden)), ("mlp.down_proj", (hidden, ffn))):
+        hf[p + name + ".weight"] = rng.normal(0, 0.03, shape).astype(np.float32)
+    hf[p + "input_layernorm.weight"] = rng.normal(1, 0.1, hidden).astype(np.float32)
+    hf[p + "post_attention_layernorm.weight"] = rng.normal(1, 0.1, hidden).astype(np.float32)
+    ref_arrays = C.read_layer_arrays(hf, layer_idx, cfg)
+    if fmt == "hf_float":
+        path = str(tmp_path / "model.safetensors")
+        save_file(hf, path)
+    elif fmt == "mg_fused_float":
+        src = tmp_path / "hf"
+        src.mkdir()
+        save_file(hf, str(src / "model.safetensors"))
+        path = str(tmp_path / "mg")
+        C.convert_hf_safetensors_multiprocess(str(src), path, None, dict(cfg, qkv_concat=True))
+    else:
+        q = {}
+        for k, v in C.convert_weight_dict(hf, cfg).items():
+            if v.ndim == 2:
+                q[k], q[k[:-len("weight")] + "w_scale"] = C.quantize_rtn_int8(v)
+            else:
+                q[k] = v
+        path = str(tmp_path / "int8.safetensors")
+        save_file(q, path)
+    layer = C.load_decode_layer(path, layer_idx, cfg, dtype=BF)
+    pr = {}
+    for n in layer.NAMES:
+        pr[n + "_w"], pr[n + "_s"] = O.quantize_weight_int8(ref_arrays[n][0])
+        assert np.array_equal(to_np(getattr(layer, n + "_w")), pr[n + "_w"]), n
+        assert np.array_equal(to_np(getattr(layer, n + "_s")), pr[n + "_s"]), n
+    pr["attn_norm"], pr["ffn_norm"] = ref_arrays["attn_norm"], ref_arrays["ffn_norm"]
+    b, bs = 3, 16
+    lens = rng.integers(20, 90, b)
+    kc0, vc0, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, BF)
+    kc, vc = dev(kc0, BF), dev(vc0, BF)
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    x = rounded(rng.normal(size=(b, hidden)), BF)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    cos, sin = synthetic.rope_rows(lens_t - 1, d, 1e4, BF, "cuda")
+    out = layer(dev(x, BF), kc, vc, torch.from_numpy(tables).cuda(), lens_t, torch.from_numpy(slots).cuda(), cos, sin)
+    ref = O.decode_layer_w8a16(x, pr, dict(n_head=nh, n_kv_head=nkv, head_dim=d, eps=1e-5), kc0, vc0, tables, lens, slots,
+                               to_np(cos), to_np(sin), act_dtype="bf16")
+    got = to_np(out)
+    tol = 8 * EPS[BF] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
+    assert np.all(np.abs(got - ref) <= tol), np.abs(got - ref).max()
