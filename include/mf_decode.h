@@ -61,6 +61,16 @@ int mf_rope_and_cache(void* query, void* key, const void* value, const void* cos
                       int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int64_t q_row_stride,
                       int64_t k_row_stride, int64_t v_row_stride, int dtype, int table_dtype, void* stream);
 
+/* mindspore._c_expression.swap_cache(host_cache, device_cache, block_mapping, is_device_to_host), as called per
+ * layer by MindIEModelRunner.swap (mindformers/model_runner.py:478-491): copies whole cache blocks between a host
+ * cache [host_blocks, ...] and a device cache [device_blocks, ...] of block_bytes each.  pairs: HOST int64
+ * [n_pairs][2] = (source block, destination block); device_to_host != 0 copies device[src] -> host[dst], else
+ * host[src] -> device[dst].  Async on `stream` when the host cache is pinned; `pairs` is read before returning.
+ * The primitive lives in MindSpore, not in the reference: the pair order is this build's declared reading. */
+int mf_swap_blocks(void* host_cache, void* device_cache, const int64_t* pairs, int64_t n_pairs,
+                   int64_t block_bytes, int64_t host_blocks, int64_t device_blocks, int device_to_host,
+                   void* stream);
+
 /* ---- paged attention (decode) --------------------------------------------------------------------- */
 
 /* Bytes of scratch mf_paged_attention_decode needs for this shape (0 when the context fits one partition). */

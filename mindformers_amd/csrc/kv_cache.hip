@@ -250,3 +250,96 @@ extern "C" int mf_rope_and_cache(void* query, void* key, const void* value, cons
                            table_dtype, q_row_stride, k_row_stride, v_row_stride, vec_ok);
     return MF_LAUNCH_CHECK();
 }
+
+// Host <-> device swap of whole cache blocks.
+//
+// Scattered blocks: one kernel moves up to SWAP_PAIRS blocks per launch, reading or writing the pinned host cache
+// directly over PCIe (a copy call per 256 KiB block costs more in call overhead than in transfer time).  The pair
+// list travels in the kernel arguments, so nothing is staged in device memory.  Used when the host cache is mapped
+// into the device address space (memory from hipHostMalloc is) and the blocks are 16-byte multiples; otherwise,
+// and for long consecutive runs (where one DMA copy is as fast), the blocks go through hipMemcpyAsync.
+constexpr int SWAP_PAIRS = 240;
+constexpr int SWAP_SPLIT = 16;                                // workgroups per block
+
+struct SwapPairs {
+    int64_t src[SWAP_PAIRS];
+    int64_t dst[SWAP_PAIRS];
+};
+
+__global__ __launch_bounds__(256) void swap_blocks_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                                          SwapPairs pairs, int64_t block_bytes) {
+    const int p = blockIdx.x;
+    const u32x4* s = (const u32x4*)(src + pairs.src[p] * block_bytes);
+    u32x4* d = (u32x4*)(dst + pairs.dst[p] * block_bytes);
+    const int64_t n16 = block_bytes >> 4;
+    const int64_t stride = (int64_t)SWAP_SPLIT * 256;
+    int64_t i = (int64_t)blockIdx.y * 256 + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {           // four 16-byte transfers in flight per lane
+        const u32x4 a = s[i], b = s[i + stride], c = s[i + 2 * stride], e = s[i + 3 * stride];
+        d[i] = a;
+        d[i + stride] = b;
+        d[i + 2 * stride] = c;
+        d[i + 3 * stride] = e;
+    }
+    for (; i < n16; i += stride) d[i] = s[i];
+}
+
+extern "C" int mf_swap_blocks(void* host_cache, void* device_cache, const int64_t* pairs, int64_t n_pairs,
+                              int64_t block_bytes, int64_t host_blocks, int64_t device_blocks, int device_to_host,
+                              void* stream) {
+    MF_REQUIRE(n_pairs >= 0 && block_bytes > 0, "swap_blocks: bad sizes");
+    if (n_pairs == 0) return 0;
+    MF_REQUIRE(host_cache && device_cache && pairs, "swap_blocks: null argument");
+    const int64_t src_blocks = device_to_host ? device_blocks : host_blocks;
+    const int64_t dst_blocks = device_to_host ? host_blocks : device_blocks;
+    for (int64_t i = 0; i < n_pairs; ++i)
+        MF_REQUIRE(pairs[2 * i] >= 0 && pairs[2 * i] < src_blocks && pairs[2 * i + 1] >= 0 &&
+                       pairs[2 * i + 1] < dst_blocks,
+                   "swap_blocks: pair %lld = (%lld, %lld) outside the caches (%lld source, %lld destination blocks)",
+                   (long long)i, (long long)pairs[2 * i], (long long)pairs[2 * i + 1], (long long)src_blocks,
+                   (long long)dst_blocks);
+    hipStream_t st = (hipStream_t)stream;
+    // the device's view of the host cache, if it has one
+    void* host_dev = nullptr;
+    const bool mapped = hipHostGetDevicePointer(&host_dev, host_cache, 0) == hipSuccess && host_dev != nullptr;
+    if (!mapped) (void)hipGetLastError();                      // not an error of this call: the copy path serves it
+    const bool by_kernel = mapped && block_bytes % 16 == 0 &&
+                           (((uintptr_t)host_dev | (uintptr_t)device_cache) & 15) == 0;
+    uint8_t* src = (uint8_t*)(device_to_host ? device_cache : host_cache);
+    uint8_t* dst = (uint8_t*)(device_to_host ? host_cache : device_cache);
+    uint8_t* ksrc = (uint8_t*)(device_to_host ? device_cache : host_dev);
+    uint8_t* kdst = (uint8_t*)(device_to_host ? host_dev : device_cache);
+    const hipMemcpyKind kind = device_to_host ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice;
+    SwapPairs batch;
+    int filled = 0;
+    auto flush = [&]() -> int {
+        if (filled == 0) return 0;
+        hipLaunchKernelGGL(swap_blocks_kernel, dim3(filled, SWAP_SPLIT), dim3(256), 0, st, kdst, ksrc, batch,
+                           block_bytes);
+        filled = 0;
+        return MF_LAUNCH_CHECK();
+    };
+    int64_t i = 0;
+    while (i < n_pairs) {
+        int64_t run = 1;
+        while (i + run < n_pairs && pairs[2 * (i + run)] == pairs[2 * i] + run &&
+               pairs[2 * (i + run) + 1] == pairs[2 * i + 1] + run)
+            ++run;
+        if (!by_kernel || run * block_bytes >= (int64_t)8 << 20) {        // one DMA copy for a long run
+            const hipError_t e = hipMemcpyAsync(dst + pairs[2 * i + 1] * block_bytes, src + pairs[2 * i] * block_bytes,
+                                                (size_t)(run * block_bytes), kind, st);
+            if (e != hipSuccess) return (int)e;
+        } else {
+            for (int64_t j = 0; j < run; ++j) {
+                batch.src[filled] = pairs[2 * (i + j)];
+                batch.dst[filled] = pairs[2 * (i + j) + 1];
+                if (++filled == SWAP_PAIRS) {
+                    const int rc = flush();
+                    if (rc) return rc;
+                }
+            }
+        }
+        i += run;
+    }
+    return flush();
+}

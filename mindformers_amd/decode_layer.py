@@ -66,9 +66,12 @@ class QuantDecodeLayer(nn.Module):
             self._packed[name] = ops.pack_w8a16_gated(w, s, "halves") if gated else ops.pack_w8a16(w, s)
         return self
 
-    def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin):
+    def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin,
+                q_starts=None):
         """x [T, hidden]; caches [num_blocks, block_size, n_kv, D]; cos/sin [T, D] rows for this step's
-        positions; batch_valid_length counts the token written by this step."""
+        positions; batch_valid_length counts the tokens written by this step.  Decode: one token per sequence.
+        Prefill / chunked prefill: ``q_starts`` int32 [B + 1] gives the row range of every sequence in x, its new
+        tokens are scattered first and then attend causally over the cache."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
         n1 = ops.rms_norm(x, self.attn_norm, self.eps)
         if self.act_quant or self.head_dim % 16:
@@ -80,8 +83,12 @@ class QuantDecodeLayer(nn.Module):
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
             q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
                                              self.n_head, bias=self.qkv_b)
-        attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
-                                   self.n_kv_head, self.scale_value)
+        if q_starts is None:
+            attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
+                                       self.n_kv_head, self.scale_value)
+        else:
+            attn = ops.paged_attention_prefill(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts,
+                                               self.n_head, self.n_kv_head, self.scale_value)
         if self.act_quant or self.wo_b is not None:
             h = self._linear(attn, "wo", residual=x)
             n2 = ops.rms_norm(h, self.ffn_norm, self.eps)

@@ -258,6 +258,26 @@ def causal_attention_varlen(query, key, value, q_starts, n_heads, n_kv_heads, sc
     return out
 
 
+def swap_cache(host_cache, device_cache, block_mapping, is_device_to_host):
+    """swap_cache(host_cache, device_cache, block_mapping, is_device_to_host) of MindIEModelRunner.swap: copy the
+    blocks named by ``block_mapping`` ([n, 2] (source, destination), host integers) between a pinned host cache and
+    a device cache with the same per-block shape.  Asynchronous on the current stream."""
+    import numpy as np
+    lib = _lib.load()
+    _need(isinstance(host_cache, torch.Tensor) and not host_cache.is_cuda and host_cache.is_contiguous(),
+          "host_cache must be a contiguous CPU tensor")
+    _need(host_cache.is_pinned(), "host_cache must be pinned (allocate it with pin_memory=True)")
+    dev = _dev_ok(device_cache)
+    _need(host_cache.dtype == device_cache.dtype and host_cache.shape[1:] == device_cache.shape[1:],
+          "host and device caches must share dtype and per-block shape")
+    pairs = np.ascontiguousarray(np.asarray(block_mapping.cpu() if isinstance(block_mapping, torch.Tensor)
+                                            else block_mapping, dtype=np.int64).reshape(-1, 2))
+    block_bytes = device_cache[0].numel() * device_cache.element_size()
+    check(lib.mf_swap_blocks(host_cache.data_ptr(), ptr(device_cache), pairs.ctypes.data, pairs.shape[0], block_bytes,
+                             host_cache.shape[0], device_cache.shape[0], int(bool(is_device_to_host)),
+                             stream_ptr(dev)), "mf_swap_blocks")
+
+
 # --------------------------------------------------------------------------------------------- norm / activation
 def rms_norm(x, gamma, eps, residual=None):
     """RmsNorm(eps)(x, gamma).  With ``residual``: returns (norm(x + residual), x + residual)."""

@@ -16,7 +16,7 @@ fc1 output, silu(gate), silu(gate)*hidden, fc2 output, residual sum.
 """
 import numpy as np
 
-from .attention import paged_attention_decode, reshape_and_cache
+from .attention import paged_attention_decode, paged_attention_prefill, reshape_and_cache
 from .dense import rms_norm, silu
 from .numerics import round_to
 from .quant import dynamic_quant_per_token, w8a16_linear, w8a8_linear
@@ -28,7 +28,7 @@ def _r(x, dt):
 
 
 def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                  act_dtype, lin):
+                  act_dtype, lin, q_seq_lens=None):
     n_head, n_kv, d = cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"]
     eps = cfg.get("eps", 1e-5)
     x = np.asarray(x, dtype=np.float64)
@@ -38,8 +38,12 @@ def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens,
     q = _r(apply_rotary_half(q, cos, sin, n_head), act_dtype)
     k = _r(apply_rotary_half(k, cos, sin, n_kv), act_dtype)
     reshape_and_cache(k.astype(key_cache.dtype), v.astype(value_cache.dtype), key_cache, value_cache, slot_mapping)
-    attn = paged_attention_decode(q, key_cache, value_cache, block_tables, context_lens, n_head, n_kv,
-                                  1.0 / np.sqrt(d), prob_dtype=act_dtype)
+    if q_seq_lens is None:
+        attn = paged_attention_decode(q, key_cache, value_cache, block_tables, context_lens, n_head, n_kv,
+                                      1.0 / np.sqrt(d), prob_dtype=act_dtype)
+    else:                                                     # prefill / chunked prefill: several rows per sequence
+        attn = paged_attention_prefill(q, key_cache, value_cache, block_tables, context_lens, q_seq_lens, n_head,
+                                       n_kv, 1.0 / np.sqrt(d), prob_dtype=act_dtype)
     attn = _r(attn, act_dtype)
     h = _r(x + _r(lin(attn, "wo"), act_dtype), act_dtype)
     n2 = _r(rms_norm(h, p["ffn_norm"], eps), act_dtype)
@@ -51,13 +55,14 @@ def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens,
 
 
 def decode_layer_w8a16(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                       act_dtype="bf16"):
+                       act_dtype="bf16", q_seq_lens=None):
     """p: {name}_w int8 [out,in], {name}_s float32 [out], optional {name}_b for name in qkv, wo, fc1, fc2,
-    plus attn_norm / ffn_norm gammas.  Caches are float32 arrays holding storage-dtype values, updated in place."""
+    plus attn_norm / ffn_norm gammas.  Caches are float32 arrays holding storage-dtype values, updated in place.
+    ``q_seq_lens``: new tokens per sequence for a prefill / chunked-prefill step (None = one each)."""
     def lin(a, name):
         return w8a16_linear(a, p[name + "_w"], p[name + "_s"], p.get(name + "_b"))
     return _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                         act_dtype, lin)
+                         act_dtype, lin, q_seq_lens)
 
 
 def decode_layer_w8a8(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,

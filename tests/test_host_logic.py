@@ -238,3 +238,12 @@ def test_moe_permute_is_a_stable_sort_and_unpermute_inverts_it():
     assert np.array_equal(px[row_map], x[np.arange(t * k) // k])
     ones = np.ones((t, k))
     assert np.allclose(O.moe_unpermute(px, row_map, ones), k * x)
+
+
+def test_cache_sizing_follows_the_reference_formula():
+    """model_runner.py:370-376: blocks = mem // (block_size * kv_heads * head_size * bytes * 2 * layers)."""
+    from mindformers_amd.runner import num_cache_blocks
+    # 1 GiB, block 128, 8 kv heads x 128, 32 layers, bf16: 2^30 / (128*8*128*2*2*32) = 64 blocks
+    assert num_cache_blocks(1, 128, 8, 128, 32, 2) == 64
+    assert num_cache_blocks(1, 128, 8, 128, 32, 1) == 128           # int8 cache
+    assert num_cache_blocks(0, 128, 8, 128, 32, 2) == 0

@@ -1,0 +1,159 @@
+"""The serving-side contract: cache sizing, a prefill step followed by decode steps through block tables, chunked
+prefill, and the host <-> device block swap.  GPU only."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import EPS, dev, rounded, to_np
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _stack(n_layers, hidden, nh, nkv, d, ffn, seed):
+    from mindformers_amd import synthetic
+    from mindformers_amd.decode_layer import QuantDecodeLayer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    return [synthetic.fill_layer(QuantDecodeLayer(hidden, nh, nkv, d, ffn, 1e-5, BF), gen) for _ in range(n_layers)]
+
+
+def _params(layer):
+    p = {}
+    for n in layer.NAMES:
+        p[n + "_w"], p[n + "_s"] = to_np(getattr(layer, n + "_w")), to_np(getattr(layer, n + "_s"))
+    p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+    return p
+
+
+def test_prefill_then_decode_steps_match_the_oracle_and_a_whole_prefill():
+    """Two sequences: prompt prefill, then three decode steps, all through BlockTables; every step is checked
+    against the oracle layer stack on the same cache state, and the decode outputs against the rows a single
+    prefill of the longer sequences produces (the two routes must agree within rounding)."""
+    from mindformers_amd.modules import BlockTables
+    from mindformers_amd.runner import DecodeStackRunner
+    hidden, nh, nkv, d, ffn, bs, n_layers = 512, 8, 2, 64, 1024, 16, 2
+    layers = _stack(n_layers, hidden, nh, nkv, d, ffn, seed=7)
+    run = DecodeStackRunner(layers, npu_mem_size=0.002, cpu_mem_size=0.001, block_size=bs)
+    assert run.npu_num_blocks == int(0.002 * 2 ** 30) // (bs * nkv * d * 2 * 2 * n_layers) and run.phase == "prefill"
+    rng = np.random.default_rng(4)
+    prompt = np.array([37, 21])
+    steps = 3
+    total = prompt + steps
+    b = len(prompt)
+    xs = [rounded(rng.normal(size=(int(t), hidden)), BF) for t in total]
+    mgr = BlockTables(run.npu_num_blocks, bs, 128)
+    mgr.init_cache_engine(b)
+    tables, slots = mgr.assemble_pa_full_inputs(int(prompt.max()), prompt, [False] * b)
+    slots = slots.reshape(b, -1)
+    slots = np.concatenate([slots[i, :prompt[i]] for i in range(b)])           # packed rows, padding dropped
+    x0 = np.concatenate([xs[i][:prompt[i]] for i in range(b)])
+    out0 = to_np(run.forward(dev(x0, BF), prompt, tables, slots, prefill=True))
+    assert run.phase == "increment" and not run.is_first_iteration
+
+    # the oracle on its own copy of the caches
+    cfg = dict(n_head=nh, n_kv_head=nkv, head_dim=d, eps=1e-5)
+    kcs = [np.zeros((run.npu_num_blocks, bs, nkv, d), np.float32) for _ in range(n_layers)]
+    vcs = [np.zeros_like(kcs[0]) for _ in range(n_layers)]
+    inv = 1.0 / (10000.0 ** (np.arange(0, d, 2) / d))
+
+    def rope(pos):
+        ang = np.asarray(pos, np.float64)[:, None] * inv[None, :]
+        emb = np.concatenate([ang, ang], -1).astype(np.float32)
+        return rounded(np.cos(emb), BF), rounded(np.sin(emb), BF)
+
+    def oracle_step(x, lens, tb, sl, pos, q_lens):
+        h = x
+        cos, sin = rope(pos)
+        for i, layer in enumerate(layers):
+            h = O.decode_layer_w8a16(h, _params(layer), cfg, kcs[i], vcs[i], tb, lens, sl, cos, sin, act_dtype="bf16",
+                                     q_seq_lens=q_lens)
+        return h
+
+    def close(got, ref, what, ulps=16):
+        tol = ulps * EPS[BF] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
+        assert np.all(np.abs(got - ref) <= tol), (what, np.abs(got - ref).max())
+
+    pos0 = np.concatenate([np.arange(n) for n in prompt])
+    ref0 = oracle_step(x0, prompt, tables, slots, pos0, prompt)
+    close(out0, ref0, "prefill")
+    decode_rows = []
+    lens = prompt.copy()
+    for s in range(steps):
+        lens = lens + 1
+        tables, slots = mgr.assemble_pa_inc_inputs(lens, [False] * b)
+        x = np.stack([xs[i][lens[i] - 1] for i in range(b)])
+        out = to_np(run.forward(dev(x, BF), lens, tables, slots, prefill=False))
+        ref = oracle_step(x, lens, tables, slots, lens - 1, None)
+        close(out, ref, f"decode step {s}")
+        decode_rows.append(out)
+    for i in range(n_layers):                                   # the caches hold what the oracle's hold
+        used = np.unique(tables[tables >= 0])
+        got_k, ref_k = to_np(run.key_cache[i])[used], kcs[i][used]
+        assert np.abs(got_k - ref_k).max() <= 16 * EPS[BF] * max(np.abs(ref_k).max(), 1.0)
+
+    # one prefill of the full sequences on a fresh runner gives the same rows as the decode steps did
+    run2 = DecodeStackRunner(layers, npu_mem_size=0.002, cpu_mem_size=0, block_size=bs)
+    mgr2 = BlockTables(run2.npu_num_blocks, bs, 128)
+    mgr2.init_cache_engine(b)
+    tables2, slots2 = mgr2.assemble_pa_full_inputs(int(total.max()), total, [False] * b)
+    slots2 = slots2.reshape(b, -1)
+    slots2 = np.concatenate([slots2[i, :total[i]] for i in range(b)])
+    whole = to_np(run2.forward(dev(np.concatenate(xs), BF), total, tables2, slots2, prefill=True))
+    starts = np.concatenate([[0], np.cumsum(total)])
+    for s in range(steps):
+        rows = np.array([starts[i] + prompt[i] + s for i in range(b)])
+        close(decode_rows[s], whole[rows], f"decode step {s} vs whole prefill", ulps=32)
+
+    # chunked prefill of the same sequences: 16 tokens per sequence and call
+    run3 = DecodeStackRunner(layers, npu_mem_size=0.002, cpu_mem_size=0, block_size=bs)
+    got = np.zeros_like(whole)
+    done = np.zeros(b, np.int64)
+    while (done < total).any():
+        step = np.minimum(16, total - done)
+        rows = np.concatenate([np.arange(starts[i] + done[i], starts[i] + done[i] + step[i]) for i in range(b)])
+        done = done + step
+        got[rows] = to_np(run3.forward(dev(np.concatenate(xs)[rows], BF), done, tables2, slots2[rows], prefill=False,
+                                       q_seq_lens=step))
+    close(got, whole, "chunked prefill vs whole prefill", ulps=32)
+
+
+def test_swap_moves_blocks_bit_exactly_both_ways():
+    from mindformers_amd import ops
+    from mindformers_amd.runner import DecodeStackRunner
+    layers = _stack(2, 256, 4, 2, 64, 512, seed=1)
+    run = DecodeStackRunner(layers, npu_mem_size=0.001, cpu_mem_size=0.0005, block_size=16)
+    assert run.cpu_num_blocks >= 8 and run.key_host[0].is_pinned()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    for i in range(2):
+        run.key_cache[i].copy_(torch.randn(run.key_cache[i].shape, generator=gen, device="cuda").to(BF))
+        run.value_cache[i].copy_(torch.randn(run.value_cache[i].shape, generator=gen, device="cuda").to(BF))
+    before_k = [to_np(c).copy() for c in run.key_cache]
+    before_v = [to_np(c).copy() for c in run.value_cache]
+    out_pairs = np.array([[5, 0], [6, 1], [7, 2], [1, 7], [12, 4]])           # device block -> host block
+    run.swap(out_pairs, True)
+    torch.cuda.synchronize()
+    for i in range(2):
+        host_k = run.key_host[i].float().numpy()
+        assert np.array_equal(host_k[out_pairs[:, 1]], before_k[i][out_pairs[:, 0]])
+        assert np.array_equal(run.value_host[i].float().numpy()[out_pairs[:, 1]], before_v[i][out_pairs[:, 0]])
+        untouched = np.setdiff1d(np.arange(run.cpu_num_blocks), out_pairs[:, 1])
+        assert not host_k[untouched].any()
+    # wipe the device blocks, bring them back to other places
+    for i in range(2):
+        run.key_cache[i].zero_()
+        run.value_cache[i].zero_()
+    in_pairs = np.array([[0, 9], [1, 10], [2, 11], [7, 3], [4, 2]])            # host block -> device block
+    run.swap(in_pairs, False)
+    torch.cuda.synchronize()
+    for i in range(2):
+        got = to_np(run.key_cache[i])
+        assert np.array_equal(got[in_pairs[:, 1]], before_k[i][out_pairs[:, 0]])
+        untouched = np.setdiff1d(np.arange(run.npu_num_blocks), in_pairs[:, 1])
+        assert not got[untouched].any()
+    with pytest.raises(RuntimeError):
+        run.swap(np.array([[run.npu_num_blocks, 0]]), True)
+    with pytest.raises(ValueError):
+        ops.swap_cache(torch.zeros(run.key_host[0].shape, dtype=BF), run.key_cache[0], out_pairs, True)   # not pinned
