@@ -91,6 +91,40 @@ int mf_paged_attention_decode(void* out, const void* query, const void* key_cach
                               int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                               int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- int8 KV cache (kvcache_dtype = int8, per-channel) ------------------------------------------------ */
+
+/* The reference sizes an int8 cache (mindformers/model_runner.py:364-368, kvcache_dtype in the quantization
+ * config, mindformers/utils/quantization_config.py:196-250) and hands PagedAttention its antiquant_scale /
+ * antiquant_offset arguments (positions 6-7 of the call in mindformers/modules/paged_attention_mgr.py:66-70);
+ * the cells that fill them belong to golden-stick and the arithmetic to the vendor kernels, so the convention is
+ * this build's own declaration: per channel c of a [n_kv_heads * head_dim] row,
+ *     q = clip(rint(x / scale[c] + offset[c]), -128, 127)        x ~ (q - offset[c]) * scale[c]
+ * scale / offset: float [2][n_kv_heads * head_dim], keys first, then values; offset may be NULL (symmetric).
+ *
+ * mf_quant_reshape_and_cache: the quantizing twin of mf_reshape_and_cache (int8 caches [slots, n_kv*D]). */
+int mf_quant_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                               const int32_t* slot_mapping, const float* scale, const float* offset,
+                               int num_tokens, int n_kv_heads, int head_dim, int64_t num_slots,
+                               int64_t key_row_stride, int64_t value_row_stride, int dtype, void* stream);
+
+/* mf_paged_attention_decode / _prefill on int8 caches: same arguments plus antiquant_scale / antiquant_offset
+ * (offset may be NULL); workspaces as for the 16-bit entry points; paged keys only.  Scores use the query with
+ * the key scale folded in (rounded to dtype); a key offset shifts all scores of a row equally and cancels in the
+ * softmax; out = scale_v * (sum_t p_t v8_t - offset_v) with the int8 values widened exactly. */
+int mf_paged_attention_decode_int8kv(void* out, const void* query, const void* key_cache, const void* value_cache,
+                                     const int32_t* block_tables, const int32_t* context_lens,
+                                     const float* antiquant_scale, const float* antiquant_offset, int batch,
+                                     int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                     int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                     int dtype, void* workspace, size_t workspace_bytes, void* stream);
+int mf_paged_attention_prefill_int8kv(void* out, const void* query, const void* key_cache, const void* value_cache,
+                                      const int32_t* block_tables, const int32_t* context_lens,
+                                      const int32_t* q_starts, const float* antiquant_scale,
+                                      const float* antiquant_offset, int batch, int total_q, int n_heads,
+                                      int n_kv_heads, int head_dim, int block_size, int max_blocks_per_seq,
+                                      int num_blocks, float scale, int64_t q_row_stride, int dtype,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- attention over several new tokens per sequence (prefill, chunked prefill, parallel decoding) -- */
 
 /* Bytes of scratch mf_paged_attention_prefill needs (0 when one partition spans the context).  max_context is

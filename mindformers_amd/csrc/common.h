@@ -139,3 +139,29 @@ __device__ __forceinline__ V bitcast(const U& u) {
     __builtin_memcpy(&v, &u, sizeof(V));
     return v;
 }
+
+// 8 int8 (two dwords) -> 8 elements of T, exact.
+template <typename T>
+__device__ __forceinline__ typename T::vec8 dequant8(uint32_t lo, uint32_t hi);
+
+__device__ __forceinline__ uint32_t i8x2_to_bf16x2(uint32_t w, int shift) {
+    const float f0 = (float)(int)(int8_t)(w >> shift);
+    const float f1 = (float)(int)(int8_t)(w >> (shift + 8));
+    // integers of magnitude <= 128 are exact in bf16: take the high halves
+    return __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+}
+template <>
+__device__ __forceinline__ bf16x8 dequant8<BF16>(uint32_t lo, uint32_t hi) {
+    u32x4 v = {i8x2_to_bf16x2(lo, 0), i8x2_to_bf16x2(lo, 16), i8x2_to_bf16x2(hi, 0), i8x2_to_bf16x2(hi, 16)};
+    return bitcast<bf16x8>(v);
+}
+template <>
+__device__ __forceinline__ f16x8 dequant8<FP16>(uint32_t lo, uint32_t hi) {
+    f16x8 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[i] = (_Float16)(float)(int)(int8_t)(lo >> (8 * i));
+        v[4 + i] = (_Float16)(float)(int)(int8_t)(hi >> (8 * i));
+    }
+    return v;
+}

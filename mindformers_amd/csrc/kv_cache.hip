@@ -145,7 +145,55 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec_kernel(
     }
 }
 
+// Quantize-and-scatter for int8 caches: cache[slot][c] = clip(rint(x[c] / scale[c] + offset[c]), -128, 127), the
+// quotient in double so that the rounding does not depend on how a float division is lowered.  One thread per
+// element; grid (tokens, 2): y = 0 keys, y = 1 values; scale / offset are [2][row].
+template <typename T>
+__global__ void quant_reshape_and_cache_kernel(const uint16_t* __restrict__ key, const uint16_t* __restrict__ value,
+                                               int8_t* __restrict__ key_cache, int8_t* __restrict__ value_cache,
+                                               const int32_t* __restrict__ slot_mapping,
+                                               const float* __restrict__ scale, const float* __restrict__ offset,
+                                               int row, int64_t num_slots, int64_t k_stride, int64_t v_stride) {
+    const int t = blockIdx.x, which = blockIdx.y;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0 || slot >= num_slots) return;
+    const uint16_t* src = which ? value + (int64_t)t * v_stride : key + (int64_t)t * k_stride;
+    int8_t* dst = (which ? value_cache : key_cache) + slot * row;
+    const float* sc = scale + which * row;
+    const float* of = offset ? offset + which * row : nullptr;
+    for (int c = threadIdx.x; c < row; c += blockDim.x) {
+        const double q = (double)T::to_float(src[c]) / (double)sc[c] + (of ? (double)of[c] : 0.0);
+        dst[c] = (int8_t)fmin(fmax(rint(q), -128.0), 127.0);
+    }
+}
+
 }  // namespace
+
+extern "C" int mf_quant_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                                          const int32_t* slot_mapping, const float* scale, const float* offset,
+                                          int num_tokens, int n_kv_heads, int head_dim, int64_t num_slots,
+                                          int64_t key_row_stride, int64_t value_row_stride, int dtype,
+                                          void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "quant_reshape_and_cache: dtype must be bf16 or fp16");
+    if (num_tokens == 0) return 0;
+    MF_REQUIRE(key && value && key_cache && value_cache && slot_mapping && scale,
+               "quant_reshape_and_cache: null argument");
+    MF_REQUIRE(num_tokens > 0 && n_kv_heads > 0 && head_dim > 0 && num_slots > 0, "quant_reshape_and_cache: bad sizes");
+    const int row = n_kv_heads * head_dim;
+    if (key_row_stride <= 0) key_row_stride = row;
+    if (value_row_stride <= 0) value_row_stride = row;
+    MF_REQUIRE(key_row_stride >= row && value_row_stride >= row, "quant_reshape_and_cache: row stride smaller than a row");
+    dim3 grid(num_tokens, 2);
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(quant_reshape_and_cache_kernel<BF16>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)key, (const uint16_t*)value, (int8_t*)key_cache, (int8_t*)value_cache,
+                           slot_mapping, scale, offset, row, num_slots, key_row_stride, value_row_stride);
+    else
+        hipLaunchKernelGGL(quant_reshape_and_cache_kernel<FP16>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)key, (const uint16_t*)value, (int8_t*)key_cache, (int8_t*)value_cache,
+                           slot_mapping, scale, offset, row, num_slots, key_row_stride, value_row_stride);
+    return MF_LAUNCH_CHECK();
+}
 
 extern "C" int mf_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
                                     const int32_t* slot_mapping, int num_tokens, int n_kv_heads, int head_dim,

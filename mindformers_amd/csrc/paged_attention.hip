@@ -62,21 +62,27 @@ __device__ inline void pf_seq(int s, const int32_t* __restrict__ q_starts, const
 // of one kv head, are then 16 consecutive (query, head-of-the-kv-group) pairs, each with its own causal limit.
 // PF with block_tables == nullptr: the keys and values are this step's own packed rows (row q_starts[b] + j is
 // token j of sequence b, pf_kv_stride elements apart) and the context is q_len.
-template <typename T, int D, int TPW, bool PF>
+// KV8: the caches hold int8 (one byte per element, rows of n_kv * D bytes) with per-channel dequantisation
+// x = (q - offset[c]) * scale[c]; kv_scale / kv_offset are float [2][n_kv * D] (keys, then values).  The key scale is
+// folded into the query, the key offset shifts every score of a column by the same amount and drops out of the
+// softmax, the value scale and offset are applied once to the (accumulator, sum) pair; the int8 tiles are widened
+// to T (exactly) when they are staged in LDS, so the MFMA path is the same.
+template <typename T, int D, int TPW, bool PF, bool KV8>
 __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
     int n_rep, int head_groups, int block_size, int max_blocks, int num_blocks, int max_parts,
     float scale_log2, int64_t q_stride, int batch, const int32_t* __restrict__ q_starts, int pf_part_tokens,
-    int64_t pf_kv_stride, int pf_rows) {
+    int64_t pf_kv_stride, int pf_rows, const float* __restrict__ kv_scale, const float* __restrict__ kv_offset) {
     using vec8 = typename T::vec8;
     constexpr int KS = D / 32;
     constexpr int VSTRIDE = PaSmem<D>::VSTRIDE;
     // tokens per partition: fixed by TPW in decode, chosen by the host (a multiple of 128) in PF, where the
     // query rows already supply the parallelism and one partition may span the whole context
     const int PART = PF ? pf_part_tokens : TPW * PA_WAVE_TOKENS;
-    constexpr int CPR = D / 8;                                // 16-byte chunks per row
+    constexpr int EB = KV8 ? 1 : 2;                           // bytes per cache element
+    constexpr int CPR = D * EB / 16;                          // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
     constexpr int NI = PA_TILE / RPI;                         // loads per lane per tile per tensor
 
@@ -179,6 +185,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         for (int j = 0; j < KS; ++j) {
             u32x4 v = {0u, 0u, 0u, 0u};
             if (head_ok) v = *(const u32x4*)(qp + 32 * j);
+            if constexpr (KV8) {                              // fold the per-channel key scale into the query
+                float f[8];
+                unpack8<T>(v, f);
+                const float* ks = kv_scale + kvh * D + 32 * j + 8 * g;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] *= ks[e];
+                v = (u32x4){pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])};
+            }
             qreg[j] = bitcast<vec8>(v);
         }
     }
@@ -196,7 +210,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     uint8_t* vst = smem + w * (PA_TILE * VSTRIDE);
     const bool contiguous = PF && block_tables == nullptr;
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
-    const int64_t row_elems = PF ? pf_kv_stride : (int64_t)n_kv * D;
+    const int64_t row_bytes = (PF ? pf_kv_stride : (int64_t)n_kv * D) * EB;
 
     const int lrow = lane / CPR;                              // coalesced-load coordinates of this lane
     const int lchunk = lane - lrow * CPR;
@@ -222,7 +236,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;       // never leave the cache allocation
         return (int64_t)blk * block_size + (ts - bi * block_size);
     };
-    // element offset of chunk lchunk of token (tstart + lrow + RPI*i); tokens past the context re-read the last
+    // byte offset of chunk lchunk of token (tstart + lrow + RPI*i); tokens past the context re-read the last
     // valid row (their scores are masked)
     auto row_offset = [&](int64_t slot0, int tstart, int i) -> int64_t {
         int tok = tstart + lrow + RPI * i;
@@ -236,21 +250,32 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
             slot = (int64_t)blk * block_size + (tok - bi * block_size);
         }
-        return slot * row_elems + (int64_t)kvh * D + 8 * lchunk;
+        return slot * row_bytes + (int64_t)kvh * D * EB + 16 * lchunk;
     };
 
     // A tile that lies inside one block and inside the context (all but the last tile of a sequence) is a scalar
     // base (its first slot) plus per-lane offsets that never change: no per-load address arithmetic.
-    const uint32_t lane_off = (uint32_t)(lrow * (int)row_elems + kvh * D + 8 * lchunk) * 2u;     // bytes
+    const uint32_t lane_off = (uint32_t)(lrow * (int)row_bytes + kvh * D * EB + 16 * lchunk);
     auto load_tile = [&](u32x4* reg, const uint16_t* __restrict__ cache, int64_t slot0, int tstart) {
         if (tile_in_block && tstart + PA_TILE <= L) {
-            const uint8_t* base = (const uint8_t*)(cache + slot0 * row_elems);     // wave-uniform
+            const uint8_t* base = (const uint8_t*)cache + slot0 * row_bytes;       // wave-uniform
 #pragma unroll
             for (int i = 0; i < NI; ++i)
-                reg[i] = *(const u32x4*)(base + (int64_t)(RPI * i) * row_elems * 2 + lane_off);
+                reg[i] = *(const u32x4*)(base + (int64_t)(RPI * i) * row_bytes + lane_off);
         } else {
 #pragma unroll
-            for (int i = 0; i < NI; ++i) reg[i] = *(const u32x4*)(cache + row_offset(slot0, tstart, i));
+            for (int i = 0; i < NI; ++i)
+                reg[i] = *(const u32x4*)((const uint8_t*)cache + row_offset(slot0, tstart, i));
+        }
+    };
+
+    // a lane's 16 loaded bytes into its place of the staged row (rows hold T elements)
+    auto stage = [&](uint8_t* row, const u32x4& v) {
+        if constexpr (KV8) {
+            *(vec8*)(row + 32 * lchunk) = dequant8<T>(v[0], v[1]);
+            *(vec8*)(row + 32 * lchunk + 16) = dequant8<T>(v[2], v[3]);
+        } else {
+            *(u32x4*)(row + 16 * lchunk) = v;
         }
     };
 
@@ -274,7 +299,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int i = 0; i < NI; ++i) *(u32x4*)(vst + (lrow + RPI * i) * VSTRIDE + 16 * lchunk) = kreg[i];
+        for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, kreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (more) {                                           // next tile's K streams in behind this tile's math
@@ -331,7 +356,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int i = 0; i < NI; ++i) *(u32x4*)(vst + (lrow + RPI * i) * VSTRIDE + 16 * lchunk) = vreg[i];
+        for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, vreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (more) {
@@ -409,6 +434,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             const float f = __builtin_amdgcn_exp2f(sm_m[x][hr] - Mh);
             lt += sm_l[x][hr] * f;
             sum += *(const f32x4*)((const float*)(smem + x * (PA_TILE * VSTRIDE)) + hr * D + 4 * d4) * f;
+        }
+        if constexpr (KV8) {                                  // value dequantisation, linear in (sum, lt)
+            const float* vs = kv_scale + n_kv * D + kvh * D + 4 * d4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float off = kv_offset ? kv_offset[n_kv * D + kvh * D + 4 * d4 + e] : 0.f;
+                sum[e] = vs[e] * (sum[e] - off * lt);
+            }
         }
         const int64_t gh = (int64_t)row * n_heads + kvh * n_rep + hq;
         if (max_parts == 1) {
@@ -507,11 +540,11 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
 // the last round of workgroups short; very long contexts use 512 to halve the partial traffic.
 static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 16384 ? 4 : 2; }
 
-template <typename T, int D>
+template <typename T, int D, bool KV8>
 int launch_pa(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads, int n_kv,
               int block_size, int max_blocks, int num_blocks, float scale, int64_t q_stride, void* workspace,
-              hipStream_t st) {
+              hipStream_t st, const float* kv_scale, const float* kv_offset) {
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
@@ -523,11 +556,11 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid((unsigned)((int64_t)batch * max_parts * n_kv * head_groups));
 #define PA_LAUNCH(TPWV)                                                                                          \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false>), grid, dim3(PA_WAVES * 64), 0, st,             \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false, KV8>), grid, dim3(PA_WAVES * 64), 0, st,        \
                        (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,      \
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
-                       (const int32_t*)nullptr, 0, (int64_t)0, 0)
+                       (const int32_t*)nullptr, 0, (int64_t)0, 0, kv_scale, kv_offset)
     if (tpw == 2) PA_LAUNCH(2);
     else PA_LAUNCH(4);
 #undef PA_LAUNCH
@@ -582,11 +615,12 @@ __global__ void pf_zero_rows_kernel(uint16_t* __restrict__ out, const int32_t* _
     for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)blockIdx.x * row + i] = 0;
 }
 
-template <typename T, int D>
+template <typename T, int D, bool KV8>
 int launch_pf(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, const int32_t* q_starts, int batch,
               int total_q, int n_heads, int n_kv, int block_size, int max_blocks, int num_blocks, float scale,
-              int64_t q_stride, int64_t kv_stride, void* workspace, hipStream_t st) {
+              int64_t q_stride, int64_t kv_stride, void* workspace, hipStream_t st, const float* kv_scale,
+              const float* kv_offset) {
     const int n_rep = n_heads / n_kv;
     const bool contiguous = block_tables == nullptr;
     const PfPlan plan = pf_plan(batch, total_q, n_heads, n_kv, contiguous ? total_q : (int64_t)max_blocks * block_size);
@@ -604,11 +638,11 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
         int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true>), dim3((unsigned)wgs), dim3(PA_WAVES * 64), 0, st,
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, KV8>), dim3((unsigned)wgs), dim3(PA_WAVES * 64), 0, st,
                        (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep,
                        (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, scale_log2, q_stride,
-                       batch, q_starts, plan.part_tokens, kv_stride, total_q);
+                       batch, q_starts, plan.part_tokens, kv_stride, total_q, kv_scale, kv_offset);
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
@@ -630,14 +664,14 @@ extern "C" size_t mf_paged_attention_prefill_workspace_bytes(int batch, int tota
     return (size_t)total_q * n_heads * plan.max_parts * (head_dim + 2) * sizeof(float);
 }
 
-extern "C" int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache,
-                                          const void* value_cache, const int32_t* block_tables,
-                                          const int32_t* context_lens, const int32_t* q_starts, int batch,
-                                          int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
-                                          int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
-                                          int64_t kv_row_stride, int dtype, void* workspace,
-                                          size_t workspace_bytes, void* stream) {
+static int pa_prefill_entry(void* out, const void* query, const void* key_cache, const void* value_cache,
+                            const int32_t* block_tables, const int32_t* context_lens, const int32_t* q_starts,
+                            int batch, int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                            int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                            int64_t kv_row_stride, int dtype, void* workspace, size_t workspace_bytes, void* stream,
+                            bool kv8, const float* kv_scale, const float* kv_offset) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention_prefill: dtype must be bf16 or fp16");
+    MF_REQUIRE(!kv8 || (kv_scale && block_tables), "paged_attention_prefill: an int8 cache needs its scales and a block table");
     MF_REQUIRE(batch >= 0 && total_q >= 0, "paged_attention_prefill: negative batch or row count");
     if (batch == 0 || total_q == 0) return 0;
     MF_REQUIRE(out && query && key_cache && value_cache && q_starts, "paged_attention_prefill: null argument");
@@ -670,9 +704,14 @@ extern "C" int mf_paged_attention_prefill(void* out, const void* query, const vo
                "paged_attention_prefill: workspace must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
 #define PF_CASE(TT, DD)                                                                                            \
-    return launch_pf<TT, DD>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch,      \
-                             total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale,      \
-                             q_row_stride, kv_row_stride, workspace, st)
+    return kv8 ? launch_pf<TT, DD, true>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, \
+                                         batch, total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq,      \
+                                         num_blocks, scale, q_row_stride, kv_row_stride, workspace, st, kv_scale,  \
+                                         kv_offset)                                                                \
+               : launch_pf<TT, DD, false>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, \
+                                          batch, total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq,     \
+                                          num_blocks, scale, q_row_stride, kv_row_stride, workspace, st, nullptr,  \
+                                          nullptr)
     if (dtype == MF_BF16) {
         if (head_dim == 32) PF_CASE(BF16, 32);
         if (head_dim == 64) PF_CASE(BF16, 64);
@@ -685,6 +724,33 @@ extern "C" int mf_paged_attention_prefill(void* out, const void* query, const vo
 #undef PF_CASE
 }
 
+extern "C" int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache,
+                                          const void* value_cache, const int32_t* block_tables,
+                                          const int32_t* context_lens, const int32_t* q_starts, int batch,
+                                          int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                          int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                          int64_t kv_row_stride, int dtype, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    return pa_prefill_entry(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, total_q,
+                            n_heads, n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale,
+                            q_row_stride, kv_row_stride, dtype, workspace, workspace_bytes, stream, false, nullptr,
+                            nullptr);
+}
+
+extern "C" int mf_paged_attention_prefill_int8kv(void* out, const void* query, const void* key_cache,
+                                                 const void* value_cache, const int32_t* block_tables,
+                                                 const int32_t* context_lens, const int32_t* q_starts,
+                                                 const float* antiquant_scale, const float* antiquant_offset,
+                                                 int batch, int total_q, int n_heads, int n_kv_heads, int head_dim,
+                                                 int block_size, int max_blocks_per_seq, int num_blocks, float scale,
+                                                 int64_t q_row_stride, int dtype, void* workspace,
+                                                 size_t workspace_bytes, void* stream) {
+    return pa_prefill_entry(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, total_q,
+                            n_heads, n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale,
+                            q_row_stride, 0, dtype, workspace, workspace_bytes, stream, true, antiquant_scale,
+                            antiquant_offset);
+}
+
 extern "C" size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, int max_context) {
     const int part_tokens = pa_tiles_per_wave(max_context) * PA_WAVE_TOKENS;
     const int64_t max_parts = ((int64_t)max_context + part_tokens - 1) / part_tokens;
@@ -692,14 +758,13 @@ extern "C" size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int
     return (size_t)batch * n_heads * max_parts * (head_dim + 2) * sizeof(float);
 }
 
-extern "C" int mf_paged_attention_decode(void* out, const void* query, const void* key_cache,
-                                         const void* value_cache, const int32_t* block_tables,
-                                         const int32_t* context_lens, int batch, int n_heads, int n_kv_heads,
-                                         int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
-                                         float scale, int64_t q_row_stride, int dtype, void* workspace,
-                                         size_t workspace_bytes,
-                                         void* stream) {
+static int pa_decode_entry(void* out, const void* query, const void* key_cache, const void* value_cache,
+                           const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads,
+                           int n_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                           float scale, int64_t q_row_stride, int dtype, void* workspace, size_t workspace_bytes,
+                           void* stream, bool kv8, const float* kv_scale, const float* kv_offset) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention: dtype must be bf16 or fp16");
+    MF_REQUIRE(!kv8 || kv_scale, "paged_attention: an int8 cache needs its scales");
     if (batch == 0) return 0;
     MF_REQUIRE(out && query && key_cache && value_cache && block_tables && context_lens,
                "paged_attention: null argument");
@@ -728,8 +793,12 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
     }
     void* ws = need ? workspace : nullptr;
 #define PA_CASE(TT, DD)                                                                                        \
-    return launch_pa<TT, DD>(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,   \
-                             n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride, ws, st)
+    return kv8 ? launch_pa<TT, DD, true>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
+                                         n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
+                                         q_row_stride, ws, st, kv_scale, kv_offset)                            \
+               : launch_pa<TT, DD, false>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
+                                          n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
+                                          q_row_stride, ws, st, nullptr, nullptr)
     if (dtype == MF_BF16) {
         if (head_dim == 32) PA_CASE(BF16, 32);
         if (head_dim == 64) PA_CASE(BF16, 64);
@@ -740,4 +809,28 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
         PA_CASE(FP16, 128);
     }
 #undef PA_CASE
+}
+
+extern "C" int mf_paged_attention_decode(void* out, const void* query, const void* key_cache,
+                                         const void* value_cache, const int32_t* block_tables,
+                                         const int32_t* context_lens, int batch, int n_heads, int n_kv_heads,
+                                         int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                                         float scale, int64_t q_row_stride, int dtype, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
+                           n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
+                           dtype, workspace, workspace_bytes, stream, false, nullptr, nullptr);
+}
+
+extern "C" int mf_paged_attention_decode_int8kv(void* out, const void* query, const void* key_cache,
+                                                const void* value_cache, const int32_t* block_tables,
+                                                const int32_t* context_lens, const float* antiquant_scale,
+                                                const float* antiquant_offset, int batch, int n_heads,
+                                                int n_kv_heads, int head_dim, int block_size,
+                                                int max_blocks_per_seq, int num_blocks, float scale,
+                                                int64_t q_row_stride, int dtype, void* workspace,
+                                                size_t workspace_bytes, void* stream) {
+    return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
+                           n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
+                           dtype, workspace, workspace_bytes, stream, true, antiquant_scale, antiquant_offset);
 }

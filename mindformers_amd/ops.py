@@ -172,6 +172,84 @@ def _q_starts(q_starts, dev):
     return q_starts.numel() - 1
 
 
+# --------------------------------------------------------------------------------------------- int8 KV cache
+def _kv_quant_params(scale, offset, row, dev):
+    _need(isinstance(scale, torch.Tensor) and scale.dtype == torch.float32 and scale.numel() == 2 * row and
+          scale.is_contiguous() and scale.device == dev, f"antiquant scale must be float32 [2, {row}] on the GPU")
+    _need(offset is None or (offset.dtype == torch.float32 and offset.numel() == 2 * row and offset.is_contiguous()
+                             and offset.device == dev), f"antiquant offset must be float32 [2, {row}] on the GPU")
+
+
+def quant_reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, scale, offset=None):
+    """Quantize key / value rows per channel (q = clip(rint(x / scale + offset), -128, 127)) and scatter them into
+    the int8 caches [num_blocks, block_size, n_kv, D].  scale / offset: float32 [2, n_kv * D] (keys, values)."""
+    lib = _lib.load()
+    _dev_of(key, value)
+    dev = _dev_ok(key_cache, value_cache, slot_mapping)
+    _need(key_cache.dtype == torch.int8 and value_cache.dtype == torch.int8 and key_cache.dim() == 4 and
+          value_cache.shape == key_cache.shape, "caches must be int8 [blocks, block_size, n_kv, D]")
+    nb, bs, n_kv, d = key_cache.shape
+    row = n_kv * d
+    key, ks = _rows(key, row, "key")
+    value, vs = _rows(value, row, "value")
+    _need(key.dtype in _ACT and value.dtype == key.dtype, "key / value must be bf16 or fp16")
+    _need(slot_mapping.dtype == torch.int32, "slot_mapping must be int32")
+    t = slot_mapping.numel()
+    _need(key.numel() // row == t if key.is_contiguous() else key.shape[0] == t, "key rows != slots")
+    _kv_quant_params(scale, offset, row, dev)
+    check(lib.mf_quant_reshape_and_cache(ptr(key), ptr(value), ptr(key_cache), ptr(value_cache), ptr(slot_mapping),
+                                         ptr(scale), ptr(offset), t, n_kv, d, nb * bs, ks, vs, dtype_code(key.dtype),
+                                         stream_ptr(dev)), "mf_quant_reshape_and_cache")
+    return key
+
+
+def paged_attention_int8kv(query, key_cache, value_cache, block_tables, context_lens, antiquant_scale,
+                           antiquant_offset, n_heads, n_kv_heads, scale, q_starts=None, out=None):
+    """PagedAttention(...)(query, key_cache, value_cache, block_tables, context_lens, antiquant_scale,
+    antiquant_offset[, mask, q_seq_lens]) on int8 caches; ``q_starts`` selects the several-rows-per-sequence form."""
+    lib = _lib.load()
+    _dev_of(query)
+    dev = _dev_ok(key_cache, value_cache, block_tables, context_lens, out)
+    _need(key_cache.dtype == torch.int8 and value_cache.dtype == torch.int8 and key_cache.dim() == 4 and
+          value_cache.shape == key_cache.shape, "caches must be int8 [blocks, block_size, n_kv, D]")
+    nb, bs, n_kv, d = key_cache.shape
+    query, qs = _rows(query, n_heads * d, "query")
+    _need(n_kv == n_kv_heads and query.dtype in _ACT, "head count / dtype mismatch")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
+    _need(context_lens.dtype == torch.int32 and context_lens.dim() == 1, "context_lens must be int32 [B]")
+    _kv_quant_params(antiquant_scale, antiquant_offset, n_kv * d, dev)
+    b = context_lens.numel()
+    _need(block_tables.shape[0] == b, "block_tables rows != batch")
+    max_blocks = block_tables.shape[1]
+    rows = query.numel() // (n_heads * d) if query.is_contiguous() else query.shape[0]
+    if out is None:
+        out = torch.empty((rows, n_heads * d), dtype=query.dtype, device=dev)
+    else:
+        _need(out.numel() == rows * n_heads * d and out.dtype == query.dtype, "out mismatch")
+    if q_starts is None:
+        _need(rows == b, f"query has {rows} rows for {b} sequences")
+        need = lib.mf_paged_attention_workspace_bytes(b, n_heads, d, max_blocks * bs)
+        ws = workspace(need, dev, "pa") if need else None
+        check(lib.mf_paged_attention_decode_int8kv(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache),
+                                                   ptr(block_tables), ptr(context_lens), ptr(antiquant_scale),
+                                                   ptr(antiquant_offset), b, n_heads, n_kv_heads, d, bs, max_blocks, nb,
+                                                   float(scale), qs, dtype_code(query.dtype), ptr(ws),
+                                                   ws.numel() if ws is not None else 0, stream_ptr(dev)),
+              "mf_paged_attention_decode_int8kv")
+    else:
+        _need(_q_starts(q_starts, dev) == b, "q_starts must have batch + 1 entries")
+        need = lib.mf_paged_attention_prefill_workspace_bytes(b, rows, n_heads, n_kv_heads, d, max_blocks * bs)
+        ws = workspace(need, dev, "pa_prefill") if need else None
+        check(lib.mf_paged_attention_prefill_int8kv(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache),
+                                                    ptr(block_tables), ptr(context_lens), ptr(q_starts),
+                                                    ptr(antiquant_scale), ptr(antiquant_offset), b, rows, n_heads,
+                                                    n_kv_heads, d, bs, max_blocks, nb, float(scale), qs,
+                                                    dtype_code(query.dtype), ptr(ws),
+                                                    ws.numel() if ws is not None else 0, stream_ptr(dev)),
+              "mf_paged_attention_prefill_int8kv")
+    return out
+
+
 def q_starts_from_ends(ends):
     """int32 [B + 1] row offsets from FlashAttentionScore's actual_seq_qlen (increasing ends, the last = T)."""
     ends = ends.to(torch.int32).reshape(-1)

@@ -31,7 +31,9 @@ Pinning status of each function (what fixes it besides its own formula):
   quantize_weight_int8,    PARITY UNPINNED: the arithmetic lives in mindspore_gs / CANN
   w8a16_linear,            (not vendored, no reference vector).  int32 accumulators are
   dynamic_quant_per_token, pinned against exact integer matmul; rounding mode, clamp range
-  w8a8_linear              and dequant order are this build's declared convention.
+  w8a8_linear,             and dequant order are this build's declared convention.  The int8 KV cache is
+  quantize_kv_int8,        pinned only through exactness: attention over a dequantised cache equals the
+  dequantize_kv_int8       16-bit oracle on the dequantised values (tests).
 """
 from .numerics import (round_bf16, round_fp16, round_to, double_benchmark,
                        DoubleBenchmarkResult)
@@ -42,7 +44,7 @@ from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_ya
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp
 from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token,
-                    int8_gemm_i32, w8a8_linear)
+                    int8_gemm_i32, w8a8_linear, quantize_kv_int8, dequantize_kv_int8)
 from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,
                   grouped_matmul)

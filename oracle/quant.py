@@ -66,3 +66,21 @@ def w8a8_linear(xq, x_scale, w_i8, w_scale, bias=None):
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)
     return y
+
+
+def quantize_kv_int8(x, scale, offset=None):
+    """Per-channel int8 quantisation of key / value rows: q = clip(rint(x / scale + offset), -128, 127), quotient
+    in float64.  PARITY UNPINNED (the reference only configures an int8 cache, quantization_config.py:196-250;
+    the arithmetic belongs to golden-stick cells and vendor kernels): this build's declared convention."""
+    q = np.asarray(x, dtype=np.float64) / np.asarray(scale, dtype=np.float64)
+    if offset is not None:
+        q = q + np.asarray(offset, dtype=np.float64)
+    return np.clip(np.rint(q), -128, 127).astype(np.int8)
+
+
+def dequantize_kv_int8(q, scale, offset=None):
+    """x ~ (q - offset) * scale in float64 (the inverse convention of quantize_kv_int8)."""
+    x = np.asarray(q, dtype=np.float64)
+    if offset is not None:
+        x = x - np.asarray(offset, dtype=np.float64)
+    return x * np.asarray(scale, dtype=np.float64)

@@ -366,6 +366,89 @@ def test_prefill_reference_vectors(golden_dir, case, n_kv):
     assert res.ok, res.messages
 
 
+# ------------------------------------------------------------------------------------------- int8 KV cache
+def _kv8_case(rng, dtype, b, nh, nkv, d, bs, lens, with_offset, max_blocks=None):
+    """Random 16-bit caches quantised per channel by the oracle; returns int8 caches, the float caches they stand
+    for, tables and the quantisation parameters."""
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype, max_blocks=max_blocks)
+    row = nkv * d
+    scale = np.stack([np.abs(kc).reshape(-1, row).max(0), np.abs(vc).reshape(-1, row).max(0)]).astype(np.float32) / 100.0
+    offset = rng.integers(-20, 21, (2, row)).astype(np.float32) if with_offset else None
+    k8 = O.quantize_kv_int8(kc.reshape(-1, row), scale[0], None if offset is None else offset[0]).reshape(kc.shape)
+    v8 = O.quantize_kv_int8(vc.reshape(-1, row), scale[1], None if offset is None else offset[1]).reshape(vc.shape)
+    kf = O.dequantize_kv_int8(k8.reshape(-1, row), scale[0], None if offset is None else offset[0]).reshape(kc.shape)
+    vf = O.dequantize_kv_int8(v8.reshape(-1, row), scale[1], None if offset is None else offset[1]).reshape(vc.shape)
+    return k8, v8, kf, vf, tables, nb, scale, offset
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("with_offset", [False, True])
+def test_quant_reshape_and_cache_bit_exact(dtype, with_offset):
+    rng = np.random.default_rng(31)
+    t, nkv, d, bs, nb = 37, 4, 64, 16, 12
+    row = nkv * d
+    k = rounded(rng.normal(size=(t, row)), dtype)
+    v = rounded(rng.normal(size=(t, row)) * 3, dtype)                 # some values clip
+    scale = rng.uniform(0.005, 0.03, (2, row)).astype(np.float32)
+    offset = rng.integers(-30, 31, (2, row)).astype(np.float32) if with_offset else None
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[5] = -1
+    kc = torch.full((nb, bs, nkv, d), 7, dtype=torch.int8, device="cuda")
+    vc = torch.full((nb, bs, nkv, d), -9, dtype=torch.int8, device="cuda")
+    ops.quant_reshape_and_cache(dev(k, dtype), dev(v, dtype), kc, vc, dev(slots, torch.int32), dev(scale, torch.float32),
+                                None if offset is None else dev(offset, torch.float32))
+    torch.cuda.synchronize()
+    ref_k = np.full((nb * bs, row), 7, np.int8)
+    ref_v = np.full((nb * bs, row), -9, np.int8)
+    live = slots >= 0
+    ref_k[slots[live]] = O.quantize_kv_int8(k, scale[0], None if offset is None else offset[0])[live]
+    ref_v[slots[live]] = O.quantize_kv_int8(v, scale[1], None if offset is None else offset[1])[live]
+    assert np.array_equal(kc.cpu().numpy().reshape(-1, row), ref_k)
+    assert np.array_equal(vc.cpu().numpy().reshape(-1, row), ref_v)
+    assert (ref_v == 127).any() or (ref_v == -128).any()
+
+
+@pytest.mark.parametrize("dtype,b,nh,nkv,d,bs,lo,hi,with_offset", [
+    (torch.bfloat16, 5, 32, 8, 128, 128, 300, 1500, False),   # bench shape, several partitions
+    (torch.bfloat16, 3, 32, 8, 128, 128, 40, 700, True),
+    (torch.float16, 4, 8, 2, 64, 16, 10, 250, True),
+    (torch.bfloat16, 2, 28, 4, 128, 128, 500, 600, False),    # n_rep = 7
+    (torch.float16, 2, 4, 4, 32, 32, 1, 90, True),            # MHA, head_dim 32
+])
+def test_paged_attention_int8kv_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi, with_offset):
+    """Attention over an int8 cache equals the oracle on the dequantised cache (the only extra rounding is the
+    query times key-scale product, rounded to the compute dtype)."""
+    rng = np.random.default_rng(b * 100 + nh)
+    lens = rng.integers(lo, hi + 1, b)
+    k8, v8, kf, vf, tables, nb, scale, offset = _kv8_case(rng, dtype, b, nh, nkv, d, bs, lens, with_offset)
+    q = rounded(rng.normal(size=(b, nh * d)), dtype)
+    sc = 1.0 / np.sqrt(d)
+    out = ops.paged_attention_int8kv(dev(q, dtype), torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda(),
+                                     dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32),
+                                     dev(scale, torch.float32), None if offset is None else dev(offset, torch.float32),
+                                     nh, nkv, sc)
+    ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, sc)
+    mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, sc)
+    assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="paged attention over an int8 cache")
+
+
+def test_paged_prefill_int8kv_vs_oracle():
+    rng = np.random.default_rng(33)
+    dtype, nh, nkv, d, bs = torch.bfloat16, 16, 4, 128, 128
+    lens, q_lens = np.array([300, 150, 2100]), np.array([60, 150, 3])
+    k8, v8, kf, vf, tables, nb, scale, offset = _kv8_case(rng, dtype, 3, nh, nkv, d, bs, lens, True)
+    t = int(q_lens.sum())
+    q = rounded(rng.normal(size=(t, nh * d)), dtype)
+    sc = 1.0 / np.sqrt(d)
+    out = ops.paged_attention_int8kv(dev(q, dtype), torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda(),
+                                     dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32),
+                                     dev(scale, torch.float32), dev(offset, torch.float32), nh, nkv, sc,
+                                     q_starts=dev(_starts(q_lens), torch.int32))
+    ref = O.paged_attention_prefill(q, kf, vf, tables, lens, q_lens, nh, nkv, sc)
+    mag = O.paged_attention_prefill(q, kf, np.abs(vf), tables, lens, q_lens, nh, nkv, sc)
+    assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="prefill over an int8 cache")
+
+
 # ------------------------------------------------------------------------------------------- norm / activation
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,cols,gdt", [(64, 4096, torch.float32), (4, 512, torch.float16), (3, 8192, torch.bfloat16), (1, 32, torch.float32)])
