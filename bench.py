@@ -60,18 +60,20 @@ def kernel_breakdown(case, torch, ops, iters):
     n1 = ops.rms_norm(x, layer.attn_norm, layer.eps)
     qkv = layer._linear(n1, "qkv")
     q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
-    attn = ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], layer.n_head, layer.n_kv_head,
-                               layer.scale_value)
+    attn = layer.attend(q, kc, vc, case["block_tables"], case["context_lens"])
     h = layer._linear(attn, "wo", residual=x)
     n2 = ops.rms_norm(h, layer.ffn_norm, layer.eps)
     a = layer.gate_up(n2)
     steps = {
         "rmsnorm": lambda: ops.rms_norm(x, layer.attn_norm, layer.eps),
         "qkv_gemm": lambda: layer._linear(n1, "qkv"),
-        "rope_and_cache": lambda: ops.rope_and_cache(q, k, v, case["cos"], case["sin"], kc, vc, case["slot_mapping"],
-                                                     layer.n_head),
-        "paged_attention": lambda: ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"],
-                                                       layer.n_head, layer.n_kv_head, layer.scale_value),
+        "rope_and_cache": (lambda: (ops.apply_rotary_pos_emb(q, k, case["cos"], case["sin"], layer.n_head,
+                                                             layer.n_kv_head, layer.head_dim),
+                                    ops.quant_reshape_and_cache(k, v, kc, vc, case["slot_mapping"], layer.kv_scale,
+                                                                layer.kv_offset))) if kc.dtype == torch.int8 else
+                          (lambda: ops.rope_and_cache(q, k, v, case["cos"], case["sin"], kc, vc, case["slot_mapping"],
+                                                      layer.n_head)),
+        "paged_attention": lambda: layer.attend(q, kc, vc, case["block_tables"], case["context_lens"]),
         "wo_gemm": lambda: layer._linear(attn, "wo", residual=x),
         "gate_up_silu_mul": lambda: layer.gate_up(n2),
         "fc2_gemm": lambda: layer._linear(a, "fc2", residual=h),
@@ -382,8 +384,7 @@ def main():
     q = qkv[:, :nq]
 
     def attn():
-        return ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], layer.n_head,
-                                   layer.n_kv_head, layer.scale_value)
+        return layer.attend(q, kc, vc, case["block_tables"], case["context_lens"])
     for _ in range(5):
         attn()
     attn_ms, attn_med = time_events(attn, args.kernel_iters, torch)
@@ -411,7 +412,9 @@ def main():
         "layer_hbm_gbps": round(layer_gbps, 1), "layer_hbm_frac": round(layer_gbps / HBM_PEAK_GBPS, 4),
         "roofline": roofline, "breakdown_us": breakdown,
     }
-    if not args.no_cpu:
+    if cfg.get("kv_int8"):
+        result["config"]["kv_cache"] = "int8, per-channel scales"
+    if not args.no_cpu and not cfg.get("kv_int8"):            # the CPU restatement of the layer covers 16-bit caches
         cb, parity = cpu_baseline(case, torch, args.cpu_seqs, out_eager)
         result["cpu_baseline"] = cb
         result["parity_vs_cpu"] = parity

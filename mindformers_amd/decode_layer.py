@@ -44,6 +44,8 @@ class QuantDecodeLayer(nn.Module):
                 self.register_buffer(f"{name}_smooth", torch.ones(k, dtype=torch.float32, device=device))
         if qkv_bias:
             self.qkv_b = torch.zeros(shapes["qkv"][0], dtype=dtype, device=device)
+        # int8 KV caches: per-channel dequantisation parameters, float32 [2, n_kv_head * head_dim] (keys, values)
+        self.kv_scale, self.kv_offset = None, None
         self.register_buffer("attn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
         self.register_buffer("ffn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
 
@@ -66,6 +68,29 @@ class QuantDecodeLayer(nn.Module):
             self._packed[name] = ops.pack_w8a16_gated(w, s, "halves") if gated else ops.pack_w8a16(w, s)
         return self
 
+    def set_kv_quant(self, scale, offset=None):
+        """Per-channel parameters of int8 caches: x ~ (q - offset) * scale; float32 [2, n_kv_head * head_dim]."""
+        row = self.n_kv_head * self.head_dim
+        if tuple(scale.shape) != (2, row) or (offset is not None and tuple(offset.shape) != (2, row)):
+            raise ValueError(f"kv scale / offset must be [2, {row}]")
+        self.kv_scale = scale.to(torch.float32).contiguous()
+        self.kv_offset = None if offset is None else offset.to(torch.float32).contiguous()
+        return self
+
+    def attend(self, q, key_cache, value_cache, block_tables, batch_valid_length, q_starts=None):
+        """Attention of this step's queries over the caches (16-bit or int8)."""
+        if key_cache.dtype == torch.int8:
+            if self.kv_scale is None:
+                raise RuntimeError("int8 caches need set_kv_quant(scale, offset)")
+            return ops.paged_attention_int8kv(q, key_cache, value_cache, block_tables, batch_valid_length,
+                                              self.kv_scale, self.kv_offset, self.n_head, self.n_kv_head,
+                                              self.scale_value, q_starts=q_starts)
+        if q_starts is None:
+            return ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
+                                       self.n_kv_head, self.scale_value)
+        return ops.paged_attention_prefill(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts,
+                                           self.n_head, self.n_kv_head, self.scale_value)
+
     def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin,
                 q_starts=None):
         """x [T, hidden]; caches [num_blocks, block_size, n_kv, D]; cos/sin [T, D] rows for this step's
@@ -74,7 +99,14 @@ class QuantDecodeLayer(nn.Module):
         tokens are scattered first and then attend causally over the cache."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
         n1 = ops.rms_norm(x, self.attn_norm, self.eps)
-        if self.act_quant or self.head_dim % 16:
+        if key_cache.dtype == torch.int8:                     # rotate, then quantize into the int8 caches
+            if self.kv_scale is None:
+                raise RuntimeError("int8 caches need set_kv_quant(scale, offset)")
+            qkv = self._linear(n1, "qkv")
+            q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+            ops.apply_rotary_pos_emb(q, k, cos, sin, self.n_head, self.n_kv_head, self.head_dim)
+            ops.quant_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, self.kv_scale, self.kv_offset)
+        elif self.act_quant or self.head_dim % 16:
             qkv = self._linear(n1, "qkv")
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
             ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
@@ -83,12 +115,7 @@ class QuantDecodeLayer(nn.Module):
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
             q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
                                              self.n_head, bias=self.qkv_b)
-        if q_starts is None:
-            attn = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
-                                       self.n_kv_head, self.scale_value)
-        else:
-            attn = ops.paged_attention_prefill(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts,
-                                               self.n_head, self.n_kv_head, self.scale_value)
+        attn = self.attend(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts)
         if self.act_quant or self.wo_b is not None:
             h = self._linear(attn, "wo", residual=x)
             n2 = ops.rms_norm(h, self.ffn_norm, self.eps)

@@ -17,6 +17,10 @@ CONFIGS = {
                              block_size=16, dtype=torch.float16, act_quant=False, theta=10000.0, layers=1),
     "llama3_8b_w8a16": dict(hidden=4096, n_head=32, n_kv_head=8, head_dim=128, ffn=14336, batch=64, ctx=(512, 4096),
                             block_size=128, dtype=torch.bfloat16, act_quant=False, theta=500000.0, layers=1),
+    # the bench shape with an int8 KV cache (per-channel scales): half the attention bytes
+    "llama3_8b_w8a16_kv8": dict(hidden=4096, n_head=32, n_kv_head=8, head_dim=128, ffn=14336, batch=64,
+                                ctx=(512, 4096), block_size=128, dtype=torch.bfloat16, act_quant=False,
+                                theta=500000.0, layers=1, kv_int8=True),
     "qwen2_5_7b_w8a8": dict(hidden=3584, n_head=28, n_kv_head=4, head_dim=128, ffn=18944, batch=256, ctx=(2048, 2048),
                             block_size=128, dtype=torch.bfloat16, act_quant=True, theta=1000000.0, layers=1),
     "qwen2_5_72b_w8a16": dict(hidden=8192, n_head=64, n_kv_head=8, head_dim=128, ffn=29568, batch=16,
@@ -94,14 +98,20 @@ def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=N
         layer = QuantDecodeLayer(cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"], cfg["ffn"], 1e-5, dt,
                                  cfg["act_quant"], device=device)
         layers_.append(fill_layer(layer, gen))
-        kc = torch.empty(kv_shape, dtype=dt, device=device)
-        vc = torch.empty(kv_shape, dtype=dt, device=device)
+        kv8 = bool(cfg.get("kv_int8"))
+        kc = torch.empty(kv_shape, dtype=torch.int8 if kv8 else dt, device=device)
+        vc = torch.empty(kv_shape, dtype=torch.int8 if kv8 else dt, device=device)
         for c in (kc, vc):
             flat = c.view(-1)
             step = 1 << 26
             for o in range(0, flat.numel(), step):
                 n = min(step, flat.numel() - o)
-                flat[o:o + n] = torch.randn(n, generator=gen, device=device).to(dt)
+                r = torch.randn(n, generator=gen, device=device)
+                # int8: N(0, 1) values on a grid of 1/32 (what quantising N(0, 1) rows with scale 1/32 leaves)
+                flat[o:o + n] = torch.clamp(torch.round(r * 32), -128, 127).to(torch.int8) if kv8 else r.to(dt)
+        if kv8:
+            row = cfg["n_kv_head"] * cfg["head_dim"]
+            layer.set_kv_quant(torch.full((2, row), 1.0 / 32, dtype=torch.float32, device=device))
         caches.append((kc, vc))
 
     x = torch.randn(b, cfg["hidden"], generator=gen, device=device).to(dt)
@@ -116,7 +126,7 @@ def algorithmic_bytes(case):
     """HBM bytes one decode step must move per layer: int8 weights once + the K/V rows of every context token
     (2 tensors x n_kv x head_dim x element size).  Activations, scales and the one new KV row are < 0.1 %."""
     cfg = case["cfg"]
-    esz = 2
+    esz = 1 if cfg.get("kv_int8") else 2
     weights = case["layers"][0].weight_bytes()
     kv = int(case["context_lens_host"].astype(np.int64).sum()) * 2 * cfg["n_kv_head"] * cfg["head_dim"] * esz
     return dict(weights=weights, kv=kv, total=weights + kv)

@@ -19,7 +19,8 @@ import numpy as np
 from .attention import paged_attention_decode, paged_attention_prefill, reshape_and_cache
 from .dense import rms_norm, silu
 from .numerics import round_to
-from .quant import dynamic_quant_per_token, w8a16_linear, w8a8_linear
+from .quant import (dequantize_kv_int8, dynamic_quant_per_token, quantize_kv_int8, w8a16_linear,
+                    w8a8_linear)
 from .rope import apply_rotary_half
 
 
@@ -28,7 +29,7 @@ def _r(x, dt):
 
 
 def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                  act_dtype, lin, q_seq_lens=None):
+                  act_dtype, lin, q_seq_lens=None, kv_quant=None):
     n_head, n_kv, d = cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"]
     eps = cfg.get("eps", 1e-5)
     x = np.asarray(x, dtype=np.float64)
@@ -37,7 +38,17 @@ def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens,
     q, k, v = np.split(qkv, [n_head * d, (n_head + n_kv) * d], axis=-1)
     q = _r(apply_rotary_half(q, cos, sin, n_head), act_dtype)
     k = _r(apply_rotary_half(k, cos, sin, n_kv), act_dtype)
-    reshape_and_cache(k.astype(key_cache.dtype), v.astype(value_cache.dtype), key_cache, value_cache, slot_mapping)
+    if kv_quant is None:
+        reshape_and_cache(k.astype(key_cache.dtype), v.astype(value_cache.dtype), key_cache, value_cache, slot_mapping)
+    else:
+        # int8 caches (updated in place); the attention below sees the dequantised values
+        scale, offset = kv_quant
+        ko, vo = (None, None) if offset is None else (offset[0], offset[1])
+        reshape_and_cache(quantize_kv_int8(k, scale[0], ko), quantize_kv_int8(v, scale[1], vo), key_cache,
+                          value_cache, slot_mapping)
+        shape = key_cache.shape
+        key_cache = dequantize_kv_int8(key_cache.reshape(-1, shape[2] * shape[3]), scale[0], ko).reshape(shape)
+        value_cache = dequantize_kv_int8(value_cache.reshape(-1, shape[2] * shape[3]), scale[1], vo).reshape(shape)
     if q_seq_lens is None:
         attn = paged_attention_decode(q, key_cache, value_cache, block_tables, context_lens, n_head, n_kv,
                                       1.0 / np.sqrt(d), prob_dtype=act_dtype)
@@ -55,14 +66,15 @@ def _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens,
 
 
 def decode_layer_w8a16(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                       act_dtype="bf16", q_seq_lens=None):
+                       act_dtype="bf16", q_seq_lens=None, kv_quant=None):
     """p: {name}_w int8 [out,in], {name}_s float32 [out], optional {name}_b for name in qkv, wo, fc1, fc2,
     plus attn_norm / ffn_norm gammas.  Caches are float32 arrays holding storage-dtype values, updated in place.
-    ``q_seq_lens``: new tokens per sequence for a prefill / chunked-prefill step (None = one each)."""
+    ``q_seq_lens``: new tokens per sequence for a prefill / chunked-prefill step (None = one each).
+    ``kv_quant`` = (scale [2, n_kv*D], offset or None): the caches are int8 arrays quantised per channel."""
     def lin(a, name):
         return w8a16_linear(a, p[name + "_w"], p[name + "_s"], p.get(name + "_b"))
     return _decode_layer(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,
-                         act_dtype, lin, q_seq_lens)
+                         act_dtype, lin, q_seq_lens, kv_quant)
 
 
 def decode_layer_w8a8(x, p, cfg, key_cache, value_cache, block_tables, context_lens, slot_mapping, cos, sin,

@@ -592,3 +592,50 @@ def test_layer_loaded_from_a_checkpoint_matches_oracle(tmp_path, fmt):
     got = to_np(out)
     tol = 8 * EPS[BF] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
     assert np.all(np.abs(got - ref) <= tol), np.abs(got - ref).max()
+
+
+@pytest.mark.parametrize("with_offset", [False, True])
+def test_decode_layer_with_int8_kv_cache_matches_oracle(with_offset):
+    """The W8A16 layer over int8 caches: the new K/V rows are rotated, quantised per channel and scattered, the
+    attention reads the int8 cache; against the oracle layer with the same quantisation convention."""
+    from mindformers_amd import synthetic
+    from mindformers_amd.decode_layer import QuantDecodeLayer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    hidden, nh, nkv, d, ffn, bs = 1024, 8, 2, 128, 1536, 128
+    layer = synthetic.fill_layer(QuantDecodeLayer(hidden, nh, nkv, d, ffn, 1e-5, BF), gen)
+    rng = np.random.default_rng(17)
+    b = 4
+    lens = rng.integers(100, 900, b)
+    kc_f, vc_f, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, BF)
+    row = nkv * d
+    scale = np.stack([np.full(row, 4.5 / 127), np.full(row, 4.5 / 127)]).astype(np.float32)
+    scale *= rng.uniform(0.8, 1.2, scale.shape).astype(np.float32)
+    offset = rng.integers(-10, 11, (2, row)).astype(np.float32) if with_offset else None
+    ko, vo = (None, None) if offset is None else (offset[0], offset[1])
+    k8 = O.quantize_kv_int8(kc_f.reshape(-1, row), scale[0], ko).reshape(kc_f.shape)
+    v8 = O.quantize_kv_int8(vc_f.reshape(-1, row), scale[1], vo).reshape(vc_f.shape)
+    layer.set_kv_quant(dev(scale, torch.float32), None if offset is None else dev(offset, torch.float32))
+    kc, vc = torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda()
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    x = rounded(rng.normal(size=(b, hidden)), BF)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    cos, sin = synthetic.rope_rows(lens_t - 1, d, 1e4, BF, "cuda")
+    out = layer(dev(x, BF), kc, vc, torch.from_numpy(tables).cuda(), lens_t, torch.from_numpy(slots).cuda(), cos, sin)
+    p = {}
+    for n in layer.NAMES:
+        p[n + "_w"], p[n + "_s"] = to_np(getattr(layer, n + "_w")), to_np(getattr(layer, n + "_s"))
+    p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+    k8_ref, v8_ref = k8.copy(), v8.copy()
+    ref = O.decode_layer_w8a16(x, p, dict(n_head=nh, n_kv_head=nkv, head_dim=d, eps=1e-5), k8_ref, v8_ref, tables, lens,
+                               slots, to_np(cos), to_np(sin), act_dtype="bf16", kv_quant=(scale, offset))
+    got = to_np(out)
+    tol = 8 * EPS[BF] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
+    assert np.all(np.abs(got - ref) <= tol), np.abs(got - ref).max()
+    # the new rows in the int8 caches: equal to the oracle's up to one quantisation step where the rotated key
+    # differs by a rounding of the compute dtype
+    got_k = kc.cpu().numpy().reshape(-1, row)[slots].astype(np.int32)
+    ref_k = k8_ref.reshape(-1, row)[slots].astype(np.int32)
+    assert np.abs(got_k - ref_k).max() <= 1 and (got_k != ref_k).mean() < 0.05
+    assert np.array_equal(vc.cpu().numpy().reshape(-1, row)[slots], v8_ref.reshape(-1, row)[slots]) or \
+        (np.abs(vc.cpu().numpy().reshape(-1, row)[slots].astype(np.int32) - v8_ref.reshape(-1, row)[slots]).max() <= 1)
