@@ -67,7 +67,7 @@ __device__ inline void pf_seq(int s, const int32_t* __restrict__ q_starts, const
 // folded into the query, the key offset shifts every score of a column by the same amount and drops out of the
 // softmax, the value scale and offset are applied once to the (accumulator, sum) pair; the int8 tiles are widened
 // to T (exactly) when they are staged in LDS, so the MFMA path is the same.
-template <typename T, int D, int TPW, bool PF, bool KV8>
+template <typename T, int D, int TPW, bool PF, bool KV8, bool TIB>
 __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 
     const int lrow = lane / CPR;                              // coalesced-load coordinates of this lane
     const int lchunk = lane - lrow * CPR;
-    const bool tile_in_block = contiguous || (block_size % PA_TILE) == 0;   // then a tile never straddles two blocks
+    constexpr bool tile_in_block = TIB;                       // a tile never straddles two blocks (host-checked)
     const int wu = __builtin_amdgcn_readfirstlane(w);         // wave index as a scalar
 
     // tiles of this wave: it = 0 .. ntiles-1 start at part_start + (it*4 + wave)*32
@@ -253,15 +253,19 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         return slot * row_bytes + (int64_t)kvh * D * EB + 16 * lchunk;
     };
 
-    // A tile that lies inside one block and inside the context (all but the last tile of a sequence) is a scalar
-    // base (its first slot) plus per-lane offsets that never change: no per-load address arithmetic.
-    const uint32_t lane_off = (uint32_t)(lrow * (int)row_bytes + kvh * D * EB + 16 * lchunk);
+    // A tile that lies inside one block (TIB) is a scalar base (its first slot) plus 32-bit per-lane offsets; rows
+    // past the context (last tile of a sequence) re-read the last valid row, whose scores are masked.  The address
+    // arithmetic is free of branches on purpose: the compiler counts outstanding loads exactly (and so lets the next
+    // tile's loads stay in flight behind this tile's math) only where no paths with different loads join.  Block
+    // sizes that tiles straddle (!TIB) need per-lane 64-bit addresses and table lookups.
+    const uint32_t lane_col = (uint32_t)(kvh * D * EB + 16 * lchunk);
     auto load_tile = [&](u32x4* reg, const uint16_t* __restrict__ cache, int64_t slot0, int tstart) {
-        if (tile_in_block && tstart + PA_TILE <= L) {
+        if constexpr (TIB) {
             const uint8_t* base = (const uint8_t*)cache + slot0 * row_bytes;       // wave-uniform
+            const int last_row = min(PA_TILE, L - tstart) - 1;                     // uniform, >= 0 for a live tile
 #pragma unroll
             for (int i = 0; i < NI; ++i)
-                reg[i] = *(const u32x4*)(base + (int64_t)(RPI * i) * row_bytes + lane_off);
+                reg[i] = *(const u32x4*)(base + (uint32_t)(min(lrow + RPI * i, last_row) * (int)row_bytes) + lane_col);
         } else {
 #pragma unroll
             for (int i = 0; i < NI; ++i)
@@ -287,13 +291,18 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         load_tile(kreg, kc, slot_cur, tfirst);
         load_tile(vreg, vc, slot_cur, tfirst);
     }
+    // the query is complete before the tile loop: a load still pending at the loop head from the entry path only
+    // would make the compiler wait for every outstanding load at its first use inside the loop
+#pragma unroll
+    for (int j = 0; j < KS; ++j) asm volatile("" : "+v"(qreg[j]));
 
-#pragma unroll 1
-    for (int it = 0; it < ntiles; ++it) {
+    // One tile.  The last tile of a wave is a copy of the body of its own (more = false at compile time): a branch
+    // around the prefetch inside the loop would make the compiler wait for every outstanding load at the join.
+    auto tile_body = [&](int it, auto more_c) {
+        constexpr bool more = decltype(more_c)::value;
         const int tstart = tfirst + it * tstep;
         const int tnext = tstart + tstep;
-        const bool more = it + 1 < ntiles;
-        const int64_t slot_nn = tile_slot(tnext + tstep);
+        const int64_t slot_nn = more ? tile_slot(tnext + tstep) : 0;
 
         // ---- stage K row-major in LDS, read it back as MFMA A operands (lane = token row r, 8 d per k-step)
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -302,9 +311,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, kreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (more) {                                           // next tile's K streams in behind this tile's math
-            load_tile(kreg, kc, slot_nxt, tnext);
-        }
+        if constexpr (more) load_tile(kreg, kc, slot_nxt, tnext);   // streams in behind this tile's math
 
         // ---- scores: S[s][i] = score of token tstart + 16 s + 4 g + i for head r
         f32x4 sc[2];
@@ -359,9 +366,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, vreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (more) {
-            load_tile(vreg, vc, slot_nxt, tnext);
-        }
+        if constexpr (more) load_tile(vreg, vc, slot_nxt, tnext);
         slot_cur = slot_nxt;
         slot_nxt = slot_nn;
 
@@ -383,7 +388,10 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             acc[u][0] = T::mfma16(bitcast<vec8>(ev), pfrag, acc[u][0]);
             acc[u][1] = T::mfma16(bitcast<vec8>(od), pfrag, acc[u][1]);
         }
-    }
+    };
+#pragma unroll 1
+    for (int it = 0; it + 1 < ntiles; ++it) tile_body(it, std::true_type{});
+    if (ntiles > 0) tile_body(ntiles - 1, std::false_type{});
 
     // ---- merge the 4 waves without a barrier: every wave parks its (max, sum, acc) in LDS (acc goes into its
     // own, now idle, staging tile), bumps a counter and leaves; the wave that arrives last combines them.
@@ -555,14 +563,20 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     float* part_ml = part_out ? part_out + (int64_t)batch * n_heads * max_parts * D : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid((unsigned)((int64_t)batch * max_parts * n_kv * head_groups));
-#define PA_LAUNCH(TPWV)                                                                                          \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false, KV8>), grid, dim3(PA_WAVES * 64), 0, st,        \
+    const bool tib = block_size % PA_TILE == 0;               // a 32-token tile never straddles two blocks
+#define PA_LAUNCH(TPWV, TIBV)                                                                                    \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false, KV8, TIBV>), grid, dim3(PA_WAVES * 64), 0, st,  \
                        (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,      \
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
                        (const int32_t*)nullptr, 0, (int64_t)0, 0, kv_scale, kv_offset)
-    if (tpw == 2) PA_LAUNCH(2);
-    else PA_LAUNCH(4);
+    if (tpw == 2) {
+        if (tib) PA_LAUNCH(2, true);
+        else PA_LAUNCH(2, false);
+    } else {
+        if (tib) PA_LAUNCH(4, true);
+        else PA_LAUNCH(4, false);
+    }
 #undef PA_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
@@ -638,11 +652,17 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
         int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, KV8>), dim3((unsigned)wgs), dim3(PA_WAVES * 64), 0, st,
-                       (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,
-                       (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep,
-                       (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, scale_log2, q_stride,
-                       batch, q_starts, plan.part_tokens, kv_stride, total_q, kv_scale, kv_offset);
+    const bool tib = contiguous || block_size % PA_TILE == 0;  // a 32-token tile never straddles two blocks
+#define PF_LAUNCH(TIBV)                                                                                           \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, KV8, TIBV>), dim3((unsigned)wgs),                    \
+                       dim3(PA_WAVES * 64), 0, st, (uint16_t*)out, part_out, part_ml, (const uint16_t*)query,      \
+                       (const uint16_t*)key_cache, (const uint16_t*)value_cache, block_tables, context_lens,       \
+                       n_heads, n_kv, n_rep, (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, \
+                       scale_log2, q_stride, batch, q_starts, plan.part_tokens, kv_stride, total_q, kv_scale,      \
+                       kv_offset)
+    if (tib) PF_LAUNCH(true);
+    else PF_LAUNCH(false);
+#undef PF_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
