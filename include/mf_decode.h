@@ -161,6 +161,28 @@ int mf_paged_attention_prefill(void* out, const void* query, const void* key_cac
                                float scale, int64_t q_row_stride, int64_t kv_row_stride, int dtype,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- multi-latent attention (MLA) decode -------------------------------------------------------------- */
+
+/* Bytes of scratch mf_mla_paged_attention_decode needs (0 when one partition spans the context). */
+size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads, int max_context);
+
+/* ops.auto_generate.PagedAttention(head_num, scale, kv_head_num=1, mla_v_dim=kv_lora_rank)(query, key_cache,
+ *                                  key_cache, block_tables, batch_valid_length, ...)
+ *   mindformers/parallel_core/inference/transformer/flash_attention.py:106-107,136-139
+ *   mindformers/parallel_core/inference/transformer/multi_latent_attention.py:199-228,344-448 (the caller: one
+ *   latent cache [num_blocks, block_size, 1, kv_lora_rank + rope_dim] written by reshape_and_cache(key, None,
+ *   key_cache, None, slot_mapping) — mf_reshape_and_cache with value = NULL — and queries already multiplied by
+ *   the absorbed key up-projection).
+ * out[b,h,:kv_lora_rank] = softmax(scale * q[b,h,:] . C_b[:L_b]^T) C_b[:L_b, :kv_lora_rank] with C the cache rows
+ * of kv_lora_rank + rope_dim values; query [batch, n_heads * (kv_lora_rank + rope_dim)], q_row_stride elements
+ * apart (0 = dense); out dense [batch, n_heads * kv_lora_rank].  kv_lora_rank = 512, rope_dim = 64 (the DeepSeek
+ * V2 / V3 geometry); block_size a multiple of 32.  Numerics as mf_paged_attention_decode. */
+int mf_mla_paged_attention_decode(void* out, const void* query, const void* latent_cache,
+                                  const int32_t* block_tables, const int32_t* context_lens, int batch,
+                                  int n_heads, int kv_lora_rank, int rope_dim, int block_size,
+                                  int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- norm / activation ---------------------------------------------------------------------------- */
 
 /* P.RmsNorm(eps)(x, gamma): mindformers/models/llama/llama_layer.py:195,225-228;

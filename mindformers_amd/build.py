@@ -15,7 +15,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmf_decode.so")
 
 SOURCES = ["errors.cpp", "kv_cache.hip", "paged_attention.hip", "elementwise.hip", "w8a16_gemm.hip",
-           "w8a8_gemm.hip", "moe.hip"]
+           "w8a8_gemm.hip", "moe.hip", "mla_attention.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 VALU forms are switched off for device code (they have produced silent wrong results on

@@ -172,6 +172,40 @@ def _q_starts(q_starts, dev):
     return q_starts.numel() - 1
 
 
+# --------------------------------------------------------------------------------------------- MLA decode
+def mla_paged_attention(query, latent_cache, block_tables, context_lens, n_heads, kv_lora_rank, scale, out=None):
+    """PagedAttention(head_num, scale, 1, mla_v_dim=kv_lora_rank)(query, cache, cache, block_tables, context_lens):
+    query [B, n_heads * (kv_lora_rank + rope)], latent cache [num_blocks, block_size, 1, kv_lora_rank + rope];
+    returns [B, n_heads * kv_lora_rank]."""
+    lib = _lib.load()
+    _dev_of(query)
+    dev = _dev_ok(latent_cache, block_tables, context_lens, out)
+    _need(latent_cache.dim() == 4 and latent_cache.shape[2] == 1, "latent cache must be [blocks, block_size, 1, rank + rope]")
+    nb, bs, _, dk = latent_cache.shape
+    rope = dk - kv_lora_rank
+    query, qs = _rows(query, n_heads * dk, "query")
+    _need(query.dtype in _ACT and latent_cache.dtype == query.dtype, "dtype mismatch")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
+    _need(context_lens.dtype == torch.int32 and context_lens.dim() == 1, "context_lens must be int32 [B]")
+    b = context_lens.numel()
+    _need(block_tables.shape[0] == b, "block_tables rows != batch")
+    rows = query.numel() // (n_heads * dk) if query.is_contiguous() else query.shape[0]
+    _need(rows == b, f"query has {rows} rows for {b} sequences")
+    max_blocks = block_tables.shape[1]
+    if out is None:
+        out = torch.empty((b, n_heads * kv_lora_rank), dtype=query.dtype, device=dev)
+    else:
+        _need(out.numel() == b * n_heads * kv_lora_rank and out.dtype == query.dtype, "out mismatch")
+    need = lib.mf_mla_paged_attention_workspace_bytes(b, n_heads, max_blocks * bs)
+    ws = workspace(need, dev, "mla") if need else None
+    check(lib.mf_mla_paged_attention_decode(ptr(out), ptr(query), ptr(latent_cache), ptr(block_tables),
+                                            ptr(context_lens), b, n_heads, kv_lora_rank, rope, bs, max_blocks, nb,
+                                            float(scale), qs, dtype_code(query.dtype), ptr(ws),
+                                            ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_mla_paged_attention_decode")
+    return out
+
+
 # --------------------------------------------------------------------------------------------- int8 KV cache
 def _kv_quant_params(scale, offset, row, dev):
     _need(isinstance(scale, torch.Tensor) and scale.dtype == torch.float32 and scale.numel() == 2 * row and

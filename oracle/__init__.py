@@ -18,6 +18,8 @@ Pinning status of each function (what fixes it besides its own formula):
   paged_attention_prefill  its two special cases are the two pinned functions above: one query per
                            sequence = paged_attention_decode, empty cache before the step =
                            causal_prefill_attention (tests); the golden prefill vectors through the cache
+  mla_paged_attention_     its reduction to paged_attention_decode (pinned above) with one kv head: equal
+   decode                  when v_dim = Dk, and its first v_dim columns otherwise (tests)
   rope tables / apply      reference vectors (rotary.npz: default, Llama3, YaRN; prefill+decode)
   rms_norm / layer_norm    reference vectors (norm.npz)
   silu_mul                 reference vectors (activation.npz)
@@ -39,7 +41,7 @@ from .numerics import (round_bf16, round_fp16, round_to, double_benchmark,
                        DoubleBenchmarkResult)
 from .attention import (reshape_and_cache, paged_attention_decode, gather_kv,
                         decode_slot_mapping, prefill_slot_mapping, causal_prefill_attention,
-                        paged_attention_prefill)
+                        paged_attention_prefill, mla_paged_attention_decode)
 from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_yarn,
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp

@@ -121,6 +121,32 @@ def paged_attention_prefill(query, key_cache, value_cache, block_tables, context
     return out.reshape(t, n_head * d)
 
 
+def mla_paged_attention_decode(query, latent_cache, block_tables, context_lens, n_head, v_dim, scale,
+                               prob_dtype=None):
+    """PagedAttention with one shared latent row per token (mla_v_dim = v_dim): the key of every head is the whole
+    cache row, the value its first v_dim entries (flash_attention.py:106-107,136-139 called with key_cache twice;
+    multi_latent_attention.py:199-228).  query [B, n_head * Dk], cache [blocks, bs, 1, Dk]; returns
+    [B, n_head * v_dim].  float64.  Pinned by its reduction to `paged_attention_decode` with one kv head when
+    v_dim = Dk, and by slicing: the output is that result's first v_dim columns per head."""
+    nb, bs, n_kv, dk = latent_cache.shape
+    assert n_kv == 1 and v_dim <= dk
+    b_sz = len(context_lens)
+    q = np.asarray(query, dtype=np.float64).reshape(b_sz, n_head, dk)
+    out = np.zeros((b_sz, n_head, v_dim), dtype=np.float64)
+    for b in range(b_sz):
+        length = int(context_lens[b])
+        if length <= 0:
+            continue
+        c = gather_kv(latent_cache, block_tables[b], length)[:, 0, :].astype(np.float64)      # [L, Dk]
+        s = (q[b] @ c.T) * scale                                                               # [n_head, L]
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p = p / p.sum(axis=1, keepdims=True)
+        if prob_dtype is not None:
+            p = round_to(p, prob_dtype).astype(np.float64)
+        out[b] = p @ c[:, :v_dim]
+    return out.reshape(b_sz, n_head * v_dim)
+
+
 def causal_prefill_attention(query, key, value, seq_lens, n_head, n_kv_head, scale):
     """Varlen causal attention over packed [T, heads*D] rows (FlashAttentionScore, TH layout,
     flash_attention.py:129-134; unfused form infer_attention.py:342-404).  float64."""

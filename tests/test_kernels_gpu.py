@@ -366,6 +366,70 @@ def test_prefill_reference_vectors(golden_dir, case, n_kv):
     assert res.ok, res.messages
 
 
+# ------------------------------------------------------------------------------------------- MLA decode
+def _mla_case(rng, dtype, lens, nh, bs, max_blocks=None):
+    b = len(lens)
+    cache, _, tables, nb = make_paged_cache(rng, b, lens, 1, 576, bs, dtype, max_blocks=max_blocks)
+    q = rounded(rng.normal(size=(b, nh * 576)), dtype)
+    scale = 1.0 / np.sqrt(192)                                  # qk_head_dim + rope of the DeepSeek geometry
+    out = ops.mla_paged_attention(dev(q, dtype), dev(cache, dtype), dev(tables, torch.int32),
+                                  dev(np.asarray(lens, np.int32), torch.int32), nh, 512, scale)
+    torch.cuda.synchronize()
+    ref = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, scale)
+    return to_np(out), ref, _mla_abs(q, cache, tables, lens, nh, scale)
+
+
+def _mla_abs(q, cache, tables, lens, nh, scale):
+    """sum_t p_t |v_t|: the magnitude the rounding of the PV product scales with."""
+    b = len(lens)
+    out = np.zeros((b, nh, 512))
+    for i in range(b):
+        n = int(lens[i])
+        if n <= 0:
+            continue
+        c = O.gather_kv(cache, tables[i], n)[:, 0, :].astype(np.float64)
+        s = (q[i].reshape(nh, 576).astype(np.float64) @ c.T) * scale
+        p = np.exp(s - s.max(1, keepdims=True))
+        p /= p.sum(1, keepdims=True)
+        out[i] = p @ np.abs(c[:, :512])
+    return out.reshape(b, nh * 512)
+
+
+@pytest.mark.parametrize("dtype,nh,bs,lens,max_blocks", [
+    (torch.bfloat16, 128, 128, [700, 130, 1500], None),        # two head blocks, partitions
+    (torch.bfloat16, 16, 128, [64, 33, 200, 1], 2),            # one head group (TP 8), single partition
+    (torch.float16, 64, 32, [95, 400], None),
+    (torch.bfloat16, 40, 64, [257, 0, 31, 32], None),          # heads not a multiple of 16, an empty sequence
+    (torch.bfloat16, 128, 128, [5000], None),                  # one long sequence: many partitions
+])
+def test_mla_paged_attention_vs_oracle(dtype, nh, bs, lens, max_blocks):
+    rng = np.random.default_rng(nh + len(lens))
+    got, ref, mag = _mla_case(rng, dtype, np.asarray(lens), nh, bs, max_blocks)
+    assert_within(got, ref, mag, dtype, ulps=1.5, what="MLA paged attention")
+    for i, n in enumerate(lens):
+        if n == 0:
+            assert not got[i].any()
+
+
+def test_mla_cache_is_written_by_key_only_reshape_and_cache():
+    """multi_latent_attention.py:401-402: the latent row goes in with reshape_and_cache(key, None, cache, None, slots)."""
+    rng = np.random.default_rng(41)
+    dtype, nh, bs = torch.bfloat16, 16, 32
+    lens = np.array([40, 7])
+    cache, _, tables, nb = make_paged_cache(rng, 2, lens, 1, 576, bs, dtype)
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    new = rounded(rng.normal(size=(2, 576)), dtype)
+    cd = dev(cache, dtype)
+    ops.reshape_and_cache(dev(new, dtype), None, cd, None, dev(slots, torch.int32))
+    cache.reshape(-1, 576)[slots] = new
+    assert np.array_equal(to_np(cd), cache)
+    q = rounded(rng.normal(size=(2, nh * 576)), dtype)
+    out = ops.mla_paged_attention(dev(q, dtype), cd, dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32),
+                                  nh, 512, 0.07)
+    ref = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, 0.07)
+    assert_within(to_np(out), ref, _mla_abs(q, cache, tables, lens, nh, 0.07), dtype, ulps=1.5, what="MLA after scatter")
+
+
 # ------------------------------------------------------------------------------------------- int8 KV cache
 def _kv8_case(rng, dtype, b, nh, nkv, d, bs, lens, with_offset, max_blocks=None):
     """Random 16-bit caches quantised per channel by the oracle; returns int8 caches, the float caches they stand

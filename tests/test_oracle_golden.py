@@ -91,6 +91,23 @@ def test_paged_prefill_oracle_is_pinned_by_its_special_cases(golden_dir, case, n
     np.testing.assert_allclose(dec, O.paged_attention_decode(dq, kc, vc, bt, [3, 3], nh, n_kv, scale), rtol=1e-12)
 
 
+def test_mla_oracle_reduces_to_the_pinned_decode_oracle():
+    """One latent row per token shared by all heads: with the value width equal to the key width it is
+    paged_attention_decode with a single kv head (pinned by the reference's decode vectors above); a narrower value
+    is the first columns of that result per head."""
+    rng = np.random.default_rng(6)
+    nb, bs, dk, nh, b = 12, 8, 24, 5, 3
+    cache = rng.normal(size=(nb, bs, 1, dk))
+    lens = np.array([9, 1, 30])
+    tables = np.stack([rng.permutation(nb)[:4] for _ in range(b)]).astype(np.int32)
+    q = rng.normal(size=(b, nh * dk))
+    full = O.paged_attention_decode(q, cache, cache, tables, lens, nh, 1, 0.3)
+    assert np.allclose(O.mla_paged_attention_decode(q, cache, tables, lens, nh, dk, 0.3), full, rtol=1e-12, atol=1e-14)
+    part = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 16, 0.3)
+    assert np.allclose(part.reshape(b, nh, 16), full.reshape(b, nh, dk)[:, :, :16], rtol=1e-12, atol=1e-14)
+    assert not O.mla_paged_attention_decode(q, cache, tables, [0, 1, 30], nh, 16, 0.3)[0].any()
+
+
 @pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
 def test_self_attention_vectors(golden_dir, case, n_kv):
     """QKV linear -> [q|k|v] split -> scatter -> prefill FA / decode PA -> projection
