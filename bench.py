@@ -285,6 +285,58 @@ def bench_prefill_attention(args, torch, ops):
     print(json.dumps(result), flush=True)
 
 
+def bench_mla_decode(args, torch, ops):
+    """DeepSeek-V3-shaped multi-latent attention decode: 128 heads over one latent cache row per token (512 latent
+    + 64 rotary, bf16), batch 64, context lengths uniform in [512, 4096], block 128.  A step is one attention call;
+    flops = 2 * (576 + 512) per (token, head)."""
+    nh, dk, dv, bs, b, dt = 128, 576, 512, 128, 64, torch.bfloat16
+    rng = np.random.default_rng(1)
+    lens = rng.integers(512, 4097, b).astype(np.int32)
+    need = (lens + bs - 1) // bs
+    nb = int(need.sum()) + 2
+    tables = -np.ones((b, 4096 // bs), np.int32)
+    perm, pos = rng.permutation(nb), 0
+    for i, n in enumerate(need):
+        tables[i, :n] = perm[pos:pos + n]
+        pos += n
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4)
+    cache = torch.randn(nb, bs, 1, dk, generator=gen, device="cuda").to(dt)
+    q = torch.randn(b, nh * dk, generator=gen, device="cuda").to(dt)
+    tb, lt = torch.from_numpy(tables).cuda(), torch.from_numpy(lens).cuda()
+    out = torch.empty(b, nh * dv, dtype=dt, device="cuda")
+
+    def step():
+        return ops.mla_paged_attention(q, cache, tb, lt, nh, dv, 192 ** -0.5, out=out)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    us = time_events(step, args.kernel_iters, torch)[0] * 1e3
+    tokens = int(lens.astype(np.int64).sum())
+    flops = 2.0 * (dk + dv) * nh * tokens
+    ach = flops / (us * 1e-6) / 1e12
+    kv_bytes = tokens * dk * 2
+    result = {
+        "metric": "MLA decode attention tokens/sec per layer (DeepSeek-V3 heads, bf16); % of dense bf16 MFMA peak",
+        "value": round(b / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"deepseek_v3_mla_decode: multi-latent attention decode, batch {b}, {nh} heads, latent "
+                               f"512 + rope 64, ctx U[512,4096] (sum {tokens}), block {bs}",
+                   "launch": "eager", "flops_per_step": flops, "cache_bytes_per_step": kv_bytes},
+        "hbm_gbps_on_cache_bytes": round(kv_bytes / (us * 1e-6) / 1e9, 1),
+        "roofline": dict(bound="mfma", kernel="mla_decode_kernel (+ mla_reduce_kernel)", achieved=round(ach, 1),
+                         peak=2500.0, unit="TFLOP/s", frac=round(ach / 2500.0, 4), traffic=None,
+                         flops_per_launch=flops, avg_launch_us=round(us, 2)),
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -314,6 +366,9 @@ def main():
 
     if args.workload == "deepseek_v3_moe_w8a16":
         bench_moe(args, torch, ops, _lib)
+        return
+    if args.workload == "deepseek_v3_mla_decode":
+        bench_mla_decode(args, torch, ops)
         return
     if args.workload in ("llama3_8b_prefill_attention", "llama3_8b_chunked_prefill_attention"):
         bench_prefill_attention(args, torch, ops)

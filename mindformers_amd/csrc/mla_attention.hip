@@ -28,7 +28,10 @@ constexpr int MLA_WAVES = 8;
 constexpr int MLA_THREADS = MLA_WAVES * 64;
 constexpr int MLA_HEADS = 64;                                 // heads per workgroup
 constexpr int MLA_TILE = 32;                                  // tokens per tile
-constexpr int MLA_STRIDE = MLA_DK * 2 + 16;                   // bytes per staged row (+16: bank spread)
+// bytes per staged row: +32 makes the row stride an even, non-multiple-of-4 number of 16-byte slots, which keeps
+// both the 16-byte operand reads (served 16 lanes at a time: rows 0-3, 12-15 of one k-chunk with rows 4-11 of the
+// next) and the transposed 4-byte reads free of bank conflicts
+constexpr int MLA_STRIDE = MLA_DK * 2 + 32;
 constexpr int MLA_TILE_BYTES = MLA_TILE * MLA_STRIDE;
 constexpr int MLA_SMEM = 2 * MLA_TILE_BYTES;
 constexpr int MLA_CPR = MLA_DK * 2 / 16;                      // 16-byte chunks per row

@@ -31,7 +31,10 @@ constexpr float PA_NEG = -1.0e30f;
 
 template <int D>
 struct PaSmem {
-    static constexpr int VSTRIDE = D * 2 + 16;                // bytes per staged row (+16: bank spread, keeps 16-B alignment)
+    // bytes per staged row: +32 makes the row stride an even, non-multiple-of-4 number of 16-byte slots, which
+    // keeps both the 16-byte operand reads (served 16 lanes at a time: rows 0-3, 12-15 of one k-chunk together with
+    // rows 4-11 of the next) and the transposed 4-byte reads free of bank conflicts
+    static constexpr int VSTRIDE = D * 2 + 32;
     static constexpr int VBYTES = PA_WAVES * PA_TILE * VSTRIDE;
     static constexpr int BYTES = VBYTES;
     static_assert(16 * D * 4 <= PA_TILE * VSTRIDE, "a wave's accumulators must fit its staging tile");

@@ -9,15 +9,14 @@ from .. import ops
 
 class FlashAttention(nn.Module):
     """ReshapeAndCache, then FlashAttentionScore (prefill) or PagedAttention (decode; with q_seq_lens: several new
-    tokens per sequence).  Masks are causal: `attn_mask` is accepted for signature parity and taken to be the lower
+    tokens per sequence; with pa_mla_v_dim > 0: multi-latent decode over the single latent cache, whose prefill runs as
+    ordinary attention on the up-projected keys and values).  Masks are causal: `attn_mask` is accepted for signature parity and taken to be the lower
     triangle the reference's models build; sparse modes other than the causal default are not built."""
 
     def __init__(self, head_num, head_dim=None, kv_head_num=None, keep_prob=1.0, scale_value=1.0,
                  pre_tokens=2147483647, next_tokens=2147483647, sparse_mode=0, input_layout="TH",
                  pa_kv_head_num=None, pa_mla_v_dim=0):
         super().__init__()
-        if pa_mla_v_dim > 0:
-            raise NotImplementedError("multi-latent attention (pa_mla_v_dim > 0) is not built")
         if input_layout not in ("TH", "TND"):
             raise ValueError(f"input_layout must be TH or TND, got {input_layout}")
         self.head_num = head_num
@@ -28,13 +27,15 @@ class FlashAttention(nn.Module):
         self.sparse_mode = sparse_mode
         self.is_prefill = True
         self.input_layout = input_layout
-        self.use_multi_latent_attention = False
+        self.pa_mla_v_dim = pa_mla_v_dim
+        self.use_multi_latent_attention = pa_mla_v_dim > 0
 
     def forward(self, query, key, value, slot_mapping=None, block_tables=None, batch_valid_length=None,
                 context_lens_tensor=None, q_seq_lens=None, actual_seq_qlen=None, actual_seq_kvlen=None,
                 attn_mask=None, padding_mask=None, prefix=None, key_cache=None, value_cache=None):
         """Forward process of the FlashAttention (flash_attention.py:109-145)."""
-        ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
+        if not self.use_multi_latent_attention:               # MLA: the caller has written the latent row already
+            ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
         shape = query.shape
         if query.dim() == 2:
             q2 = query
@@ -59,6 +60,12 @@ class FlashAttention(nn.Module):
             out = ops.causal_attention_varlen(q2, k2, v2, starts, self.head_num,
                                               self.pa_kv_head_num, self.scale_value)
             return out.reshape(shape)
+        if self.use_multi_latent_attention:                   # one latent cache, keys = values (flash_attention.py:136-139)
+            if q_seq_lens is not None:
+                raise NotImplementedError("MLA decode with q_seq_lens (several new tokens per sequence) is not built")
+            out = ops.mla_paged_attention(q2, key_cache, block_tables, batch_valid_length, self.head_num,
+                                          self.pa_mla_v_dim, self.scale_value)
+            return out.reshape(*shape[:-1], self.head_num * self.pa_mla_v_dim)
         if q_seq_lens is not None:                            # several new tokens per sequence (flash_attention.py:140-143)
             out = ops.paged_attention_prefill(q2, key_cache, value_cache, block_tables, batch_valid_length,
                                               ops.q_starts_from_lens(q_seq_lens), self.head_num,

@@ -122,11 +122,12 @@ def paged_attention_prefill(query, key_cache, value_cache, block_tables, context
 
 
 def mla_paged_attention_decode(query, latent_cache, block_tables, context_lens, n_head, v_dim, scale,
-                               prob_dtype=None):
+                               prob_dtype=None, abs_values=False):
     """PagedAttention with one shared latent row per token (mla_v_dim = v_dim): the key of every head is the whole
     cache row, the value its first v_dim entries (flash_attention.py:106-107,136-139 called with key_cache twice;
     multi_latent_attention.py:199-228).  query [B, n_head * Dk], cache [blocks, bs, 1, Dk]; returns
-    [B, n_head * v_dim].  float64.  Pinned by its reduction to `paged_attention_decode` with one kv head when
+    [B, n_head * v_dim].  float64.  ``abs_values`` returns sum_t p_t |v_t| instead (the magnitude that the rounding
+    error of the product scales with; used for test tolerances).  Pinned by its reduction to `paged_attention_decode` with one kv head when
     v_dim = Dk, and by slicing: the output is that result's first v_dim columns per head."""
     nb, bs, n_kv, dk = latent_cache.shape
     assert n_kv == 1 and v_dim <= dk
@@ -143,7 +144,7 @@ def mla_paged_attention_decode(query, latent_cache, block_tables, context_lens, 
         p = p / p.sum(axis=1, keepdims=True)
         if prob_dtype is not None:
             p = round_to(p, prob_dtype).astype(np.float64)
-        out[b] = p @ c[:, :v_dim]
+        out[b] = p @ (np.abs(c[:, :v_dim]) if abs_values else c[:, :v_dim])
     return out.reshape(b_sz, n_head * v_dim)
 
 

@@ -381,18 +381,7 @@ def _mla_case(rng, dtype, lens, nh, bs, max_blocks=None):
 
 def _mla_abs(q, cache, tables, lens, nh, scale):
     """sum_t p_t |v_t|: the magnitude the rounding of the PV product scales with."""
-    b = len(lens)
-    out = np.zeros((b, nh, 512))
-    for i in range(b):
-        n = int(lens[i])
-        if n <= 0:
-            continue
-        c = O.gather_kv(cache, tables[i], n)[:, 0, :].astype(np.float64)
-        s = (q[i].reshape(nh, 576).astype(np.float64) @ c.T) * scale
-        p = np.exp(s - s.max(1, keepdims=True))
-        p /= p.sum(1, keepdims=True)
-        out[i] = p @ np.abs(c[:, :512])
-    return out.reshape(b, nh * 512)
+    return O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, scale, abs_values=True)
 
 
 @pytest.mark.parametrize("dtype,nh,bs,lens,max_blocks", [

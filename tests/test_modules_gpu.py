@@ -639,3 +639,31 @@ def test_decode_layer_with_int8_kv_cache_matches_oracle(with_offset):
     assert np.abs(got_k - ref_k).max() <= 1 and (got_k != ref_k).mean() < 0.05
     assert np.array_equal(vc.cpu().numpy().reshape(-1, row)[slots], v8_ref.reshape(-1, row)[slots]) or \
         (np.abs(vc.cpu().numpy().reshape(-1, row)[slots].astype(np.int32) - v8_ref.reshape(-1, row)[slots]).max() <= 1)
+
+
+def test_mcore_flash_attention_mla_decode_branch():
+    """FlashAttention(pa_mla_v_dim=512): the decode call of MLASelfAttention (multi_latent_attention.py:212-228):
+    the caller has written the latent row with reshape_and_cache(key, None, cache, None, slots); the cell attends
+    with the cache as keys and values."""
+    from mindformers_amd import ops
+    from mindformers_amd.modules import FlashAttention
+    rng = np.random.default_rng(19)
+    nh, bs = 32, 32
+    lens = np.array([70, 300, 33])
+    cache, _, tables, nb = make_paged_cache(rng, 3, lens, 1, 576, bs, BF)
+    net = FlashAttention(head_num=nh, head_dim=576, kv_head_num=1, pa_kv_head_num=1, scale_value=0.072, pa_mla_v_dim=512)
+    net.is_prefill = False
+    assert net.use_multi_latent_attention
+    q = rounded(rng.normal(size=(3, nh * 576)), BF)
+    new = rounded(rng.normal(size=(3, 576)), BF)
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    cd = dev(cache, BF)
+    ops.reshape_and_cache(dev(new, BF), None, cd, None, dev(slots, torch.int32))
+    cache.reshape(-1, 576)[slots] = new
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    out = net(query=dev(q, BF), key=None, value=None, slot_mapping=dev(slots, torch.int32),
+              block_tables=dev(tables, torch.int32), batch_valid_length=lens_t, key_cache=cd, value_cache=None)
+    assert out.shape == (3, nh * 512)
+    ref = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, 0.072)
+    mag = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, 0.072, abs_values=True)
+    assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA decode")
