@@ -165,3 +165,10 @@ __device__ __forceinline__ f16x8 dequant8<FP16>(uint32_t lo, uint32_t hi) {
     }
     return v;
 }
+
+// Transposing 64-bit LDS read (ds_read_b64_tr_b16).  Within every group of 16 lanes, lane j names four consecutive
+// 16-bit values M[j][0..3]; lane i receives M[(i >> 2) + 4 e][i & 3] for e = 0..3.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ s16x4 lds_read_tr16(const uint8_t* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+}

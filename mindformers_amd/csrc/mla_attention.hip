@@ -14,8 +14,8 @@
 //   of the output); the PV product, which holds the accumulators, is split between them.
 //   S^T[token, head] = C[token, :576] . Q[head, :576]     18 k-steps of mfma_f32_16x16x32 per 16-token sub-tile
 //   online softmax in fp32 (exp2 domain), probabilities rounded to the cache dtype
-//   O^T[d, head] += C^T[d, token] . P^T[token, head]       the tile is read back transposed, two d-rows per
-//                                                          32-bit LDS read (as in the GQA decode kernel)
+//   O^T[d, head] += C^T[d, token] . P^T[token, head]       the tile is read back through the transposing LDS read
+//                                                          (as in the GQA decode kernel)
 //   No merge inside the workgroup is needed: every wave owns its (heads, columns).  Partitions of a sequence
 //   are combined by the partition-reduce kernel of the GQA path.
 #include "common.h"
@@ -38,7 +38,7 @@ constexpr int MLA_CPR = MLA_DK * 2 / 16;                      // 16-byte chunks 
 constexpr int MLA_CHUNKS = MLA_TILE * MLA_CPR;
 constexpr int MLA_LD = (MLA_CHUNKS + MLA_THREADS - 1) / MLA_THREADS;      // loads per thread per tile
 constexpr int MLA_KS = MLA_DK / 32;                           // k-steps of the score product
-constexpr int MLA_US = MLA_DV / 2 / 32;                       // 32-column steps of one wave's half of the output
+constexpr int MLA_DB = MLA_DV / 2 / 16;                       // 16-column blocks of one wave's half of the output
 constexpr float MLA_NEG = -1.0e30f;
 
 template <typename T>
@@ -139,12 +139,9 @@ __global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
                 *(u32x4*)(buf + lrow[k] * MLA_STRIDE + 16 * lcol[k]) = lreg[k];
     };
 
-    f32x4 acc[MLA_US][2];
+    f32x4 acc[MLA_DB];                                        // acc[db][i]: column 16 db + 4 g + i of this wave's half
 #pragma unroll
-    for (int u = 0; u < MLA_US; ++u) {
-        acc[u][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        acc[u][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
+    for (int db = 0; db < MLA_DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = MLA_NEG, l_run = 0.f;
 
     if (ntiles > 0) {
@@ -173,15 +170,25 @@ __global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
             }
         }
         float tmax = MLA_NEG;
+        if (tstart + MLA_TILE <= L) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int tok = tstart + s * 16 + 4 * g + i;
-                const float v = tok < L ? sc[s][i] * scale_log2 : MLA_NEG;
-                sc[s][i] = v;
-                tmax = fmaxf(tmax, v);
-            }
+                for (int i = 0; i < 4; ++i) {
+                    sc[s][i] *= scale_log2;
+                    tmax = fmaxf(tmax, sc[s][i]);
+                }
+        } else {                                              // last tile of the sequence: mask what lies past it
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int tok = tstart + s * 16 + 4 * g + i;
+                    const float v = tok < L ? sc[s][i] * scale_log2 : MLA_NEG;
+                    sc[s][i] = v;
+                    tmax = fmaxf(tmax, v);
+                }
+        }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float m_new = fmaxf(m_run, tmax);
@@ -199,32 +206,25 @@ __global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
             psum += T::to_float((uint16_t)(pp[2 * s] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s] >> 16)) +
                     T::to_float((uint16_t)(pp[2 * s + 1] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s + 1] >> 16));
         }
-        l_run = l_run * alpha + psum;
+        // when the running maximum moved for no lane of the wave, alpha is exactly 1: skip the rescale
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+            l_run *= alpha;
 #pragma unroll
-        for (int u = 0; u < MLA_US; ++u) {
-            acc[u][0] *= alpha;
-            acc[u][1] *= alpha;
+            for (int db = 0; db < MLA_DB; ++db) acc[db] *= alpha;
         }
+        l_run += psum;
         const vec8 pfrag = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
 
-        // ---- O^T += C^T P^T over this wave's 256 value columns; lane (r, g) reads d, d + 1 for its 8 tokens
+        // ---- O^T += C^T P^T over this wave's 256 value columns.  The A operand (row d, 8 tokens in the order of the
+        // probabilities) comes from the row-major tile through the transposing LDS read: within 16 lanes, lane j
+        // names C[token 4g + (j >> 2)][d0 + 4 (j & 3) ..] and lane r receives C[token 4g + e][d0 + r], e = 0..3.
 #pragma unroll
-        for (int u = 0; u < MLA_US; ++u) {
-            const int d0 = vhalf * (MLA_DV / 2) + 32 * u + 2 * r;
-            uint32_t wv[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int tl = 16 * (e >> 2) + 4 * g + (e & 3);
-                wv[e] = *(const uint32_t*)(tile + tl * MLA_STRIDE + d0 * 2);
-            }
-            u32x4 ev, od;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                ev[e] = __builtin_amdgcn_perm(wv[2 * e + 1], wv[2 * e], 0x05040100u);
-                od[e] = __builtin_amdgcn_perm(wv[2 * e + 1], wv[2 * e], 0x07060302u);
-            }
-            acc[u][0] = T::mfma16(bitcast<vec8>(ev), pfrag, acc[u][0]);
-            acc[u][1] = T::mfma16(bitcast<vec8>(od), pfrag, acc[u][1]);
+        for (int db = 0; db < MLA_DB; ++db) {
+            const int d0 = vhalf * (MLA_DV / 2) + 16 * db;
+            const uint8_t* p0 = tile + (4 * g + (r >> 2)) * MLA_STRIDE + (d0 + 4 * (r & 3)) * 2;
+            const u32x2 l2 = bitcast<u32x2>(lds_read_tr16(p0));
+            const u32x2 h2 = bitcast<u32x2>(lds_read_tr16(p0 + 16 * MLA_STRIDE));
+            acc[db] = T::mfma16(bitcast<vec8>((u32x4){l2[0], l2[1], h2[0], h2[1]}), pfrag, acc[db]);
         }
 
         if (more) store_tile(mla_smem + ((it + 1) & 1) * MLA_TILE_BYTES);
@@ -238,19 +238,13 @@ __global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
     const int64_t gh = (int64_t)b * n_heads + head;
     const float inv = 1.0f / l_run;
 #pragma unroll
-    for (int u = 0; u < MLA_US; ++u) {
-        // acc[u][par][i] is column 32 u + 8 g + 2 i + par of this wave's half
-        const int d = vhalf * (MLA_DV / 2) + 32 * u + 8 * g;
-        const f32x4 lo = {acc[u][0][0], acc[u][1][0], acc[u][0][1], acc[u][1][1]};
-        const f32x4 hi = {acc[u][0][2], acc[u][1][2], acc[u][0][3], acc[u][1][3]};
+    for (int db = 0; db < MLA_DB; ++db) {
+        const int d = vhalf * (MLA_DV / 2) + 16 * db + 4 * g;
         if (max_parts == 1) {
-            const u32x4 o = {pack2<T>(lo[0] * inv, lo[1] * inv), pack2<T>(lo[2] * inv, lo[3] * inv),
-                             pack2<T>(hi[0] * inv, hi[1] * inv), pack2<T>(hi[2] * inv, hi[3] * inv)};
-            *(u32x4*)(out + gh * MLA_DV + d) = o;
+            const u32x2 o = {pack2<T>(acc[db][0] * inv, acc[db][1] * inv), pack2<T>(acc[db][2] * inv, acc[db][3] * inv)};
+            *(u32x2*)(out + gh * MLA_DV + d) = o;
         } else {
-            float* po = part_out + (gh * max_parts + part) * MLA_DV + d;
-            *(f32x4*)po = lo;
-            *(f32x4*)(po + 4) = hi;
+            *(f32x4*)(part_out + (gh * max_parts + part) * MLA_DV + d) = acc[db];
         }
     }
     if (max_parts > 1 && g == 0 && vhalf == 0) {

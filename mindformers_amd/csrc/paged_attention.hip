@@ -16,8 +16,8 @@
 //   online softmax in fp32 (exp2 domain); the only cross-lane traffic is two xor-shuffles for the row max
 //   O^T[d, head] += V^T[d, token] . P^T[token, head] the probabilities sit in exactly the B-operand layout
 //                                                    when the 32 tokens are ordered (sub-tile, 4g+i); V is
-//                                                    staged through a per-wave LDS tile and read back
-//                                                    transposed, two d-rows per 32-bit LDS read
+//                                                    staged through a per-wave LDS tile and read back with
+//                                                    the transposing LDS read (ds_read_b64_tr_b16)
 //   The 4 waves are merged through LDS and the workgroup writes either the final rows (single partition)
 //   or an fp32 partial (acc, max, sum) that a small second kernel combines.
 #include "common.h"
@@ -181,6 +181,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     const int head = kvh * n_rep + (head_ok ? hcol : 0);
     const int q_row = PF ? q_start + (head_ok ? qi : 0) : b;
     const int Lcol = PF ? (head_ok ? ctx_before + qi + 1 : 0) : L;      // causal limit of this lane's column
+    // tiles that end at or before the smallest limit of the group's live columns need no mask (columns past the
+    // sequence's queries are never written)
+    const int Lmask = PF ? ctx_before + (hg * 16) / n_rep + 1 : L;
     vec8 qreg[KS];
     {
         const uint16_t* qp = q + (int64_t)q_row * q_stride + (int64_t)head * D + 8 * g;
@@ -200,12 +203,10 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         }
     }
 
-    f32x4 acc[KS][2];
+    constexpr int DB = D / 16;                                // 16-row blocks of O^T
+    f32x4 acc[DB];                                            // acc[db][i]: d = 16 db + 4 g + i, head r
 #pragma unroll
-    for (int u = 0; u < KS; ++u) {
-        acc[u][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        acc[u][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
+    for (int db = 0; db < DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     // PF: a column can find a whole tile masked before it has seen any token; starting the running maximum above
     // the mask value makes those probabilities 2^(-huge) = 0 instead of 2^0
     float m_run = PF ? 0.5f * PA_NEG : PA_NEG, l_run = 0.f;
@@ -257,18 +258,26 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     };
 
     // A tile that lies inside one block (TIB) is a scalar base (its first slot) plus 32-bit per-lane offsets; rows
-    // past the context (last tile of a sequence) re-read the last valid row, whose scores are masked.  The address
-    // arithmetic is free of branches on purpose: the compiler counts outstanding loads exactly (and so lets the next
+    // past the context (last tile of a sequence) re-read the last valid row, whose scores are masked.  Both paths
+    // issue the same number of loads on purpose: the compiler counts outstanding loads exactly (and so lets the next
     // tile's loads stay in flight behind this tile's math) only where no paths with different loads join.  Block
     // sizes that tiles straddle (!TIB) need per-lane 64-bit addresses and table lookups.
     const uint32_t lane_col = (uint32_t)(kvh * D * EB + 16 * lchunk);
+    const uint32_t lane_off = (uint32_t)(lrow * (int)row_bytes) + lane_col;
     auto load_tile = [&](u32x4* reg, const uint16_t* __restrict__ cache, int64_t slot0, int tstart) {
         if constexpr (TIB) {
             const uint8_t* base = (const uint8_t*)cache + slot0 * row_bytes;       // wave-uniform
-            const int last_row = min(PA_TILE, L - tstart) - 1;                     // uniform, >= 0 for a live tile
+            if (tstart + PA_TILE <= L) {                                           // whole tile: constant lane offset
 #pragma unroll
-            for (int i = 0; i < NI; ++i)
-                reg[i] = *(const u32x4*)(base + (uint32_t)(min(lrow + RPI * i, last_row) * (int)row_bytes) + lane_col);
+                for (int i = 0; i < NI; ++i)
+                    reg[i] = *(const u32x4*)(base + (int64_t)(RPI * i) * row_bytes + lane_off);
+            } else {                                                               // the same loads, rows clamped
+                const int last_row = L - tstart - 1;                               // uniform, >= 0 for a live tile
+#pragma unroll
+                for (int i = 0; i < NI; ++i)
+                    reg[i] = *(const u32x4*)(base + (uint32_t)(min(lrow + RPI * i, last_row) * (int)row_bytes) +
+                                             lane_col);
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < NI; ++i)
@@ -328,15 +337,25 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             }
         }
         float tmax = PA_NEG;
+        if (tstart + PA_TILE <= Lmask) {                      // every token of the tile is visible to every column
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int tok = tstart + s * 16 + 4 * g + i;
-                const float v = tok < Lcol ? sc[s][i] * scale_log2 : PA_NEG;
-                sc[s][i] = v;
-                tmax = fmaxf(tmax, v);
-            }
+                for (int i = 0; i < 4; ++i) {
+                    sc[s][i] *= scale_log2;
+                    tmax = fmaxf(tmax, sc[s][i]);
+                }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int tok = tstart + s * 16 + 4 * g + i;
+                    const float v = tok < Lcol ? sc[s][i] * scale_log2 : PA_NEG;
+                    sc[s][i] = v;
+                    tmax = fmaxf(tmax, v);
+                }
+        }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float m_new = fmaxf(m_run, tmax);
@@ -354,12 +373,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
             psum += T::to_float((uint16_t)(pp[2 * s] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s] >> 16)) +
                     T::to_float((uint16_t)(pp[2 * s + 1] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s + 1] >> 16));
         }
-        l_run = l_run * alpha + psum;
+        // the running maximum of a column rarely moves after the first tiles: when it did not move for any lane of
+        // the wave, alpha is exactly 1 everywhere and the rescale is skipped (bit-identical)
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+            l_run *= alpha;
 #pragma unroll
-        for (int u = 0; u < KS; ++u) {
-            acc[u][0] *= alpha;
-            acc[u][1] *= alpha;
+            for (int db = 0; db < DB; ++db) acc[db] *= alpha;
         }
+        l_run += psum;
         const vec8 pfrag = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
 
         // ---- stage V (rows = tokens) in the same LDS tile
@@ -373,23 +394,16 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         slot_cur = slot_nxt;
         slot_nxt = slot_nn;
 
-        // ---- O^T += V^T P^T ; lane (r, g) reads d = 32u + 2r, 2r+1 for its 8 tokens (16*(e/4) + 4g + e%4)
+        // ---- O^T += V^T P^T.  The A operand (row d, 8 tokens in the order of the probabilities: 4g+e, 16+4g+e) comes
+        // from the row-major tile through the transposing LDS read: within 16 lanes, lane j names the 4 values
+        // V[token 4g + (j >> 2)][16 db + 4 (j & 3) ..] and lane r receives V[token 4g + e][16 db + r], e = 0..3.
 #pragma unroll
-        for (int u = 0; u < KS; ++u) {
-            uint32_t wv[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int tl = 16 * (e >> 2) + 4 * g + (e & 3);
-                wv[e] = *(const uint32_t*)(vst + tl * VSTRIDE + (32 * u + 2 * r) * 2);
-            }
-            u32x4 ev, od;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                ev[e] = __builtin_amdgcn_perm(wv[2 * e + 1], wv[2 * e], 0x05040100u);
-                od[e] = __builtin_amdgcn_perm(wv[2 * e + 1], wv[2 * e], 0x07060302u);
-            }
-            acc[u][0] = T::mfma16(bitcast<vec8>(ev), pfrag, acc[u][0]);
-            acc[u][1] = T::mfma16(bitcast<vec8>(od), pfrag, acc[u][1]);
+        for (int db = 0; db < DB; ++db) {
+            const uint8_t* p0 = vst + (4 * g + (r >> 2)) * VSTRIDE + (16 * db + 4 * (r & 3)) * 2;
+            const s16x4 lo = lds_read_tr16(p0);
+            const s16x4 hi = lds_read_tr16(p0 + 16 * VSTRIDE);
+            const u32x2 l2 = bitcast<u32x2>(lo), h2 = bitcast<u32x2>(hi);
+            acc[db] = T::mfma16(bitcast<vec8>((u32x4){l2[0], l2[1], h2[0], h2[1]}), pfrag, acc[db]);
         }
     };
 #pragma unroll 1
@@ -405,15 +419,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         sm_l[w][r] = l_run;
     }
     {
-        float* dst = (float*)vst + r * D + 8 * g;             // [head 16][D] floats: fits the staging tile
+        float* dst = (float*)vst + r * D + 4 * g;             // [head 16][D] floats: fits the staging tile
 #pragma unroll
-        for (int u = 0; u < KS; ++u) {
-            // acc[u][par][i] is d = 32u + 8g + 2i + par
-            f32x4 lo = {acc[u][0][0], acc[u][1][0], acc[u][0][1], acc[u][1][1]};
-            f32x4 hi = {acc[u][0][2], acc[u][1][2], acc[u][0][3], acc[u][1][3]};
-            *(f32x4*)(dst + 32 * u) = lo;
-            *(f32x4*)(dst + 32 * u + 4) = hi;
-        }
+        for (int db = 0; db < DB; ++db) *(f32x4*)(dst + 16 * db) = acc[db];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     int arrived = 0;
@@ -559,7 +567,9 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    const int tpw = pa_tiles_per_wave(max_ctx);
+    // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
+    // first tile, merge) exposed: twice the tokens per workgroup.  Fewer partitions than the workspace was sized for.
+    const int tpw = KV8 ? 4 : pa_tiles_per_wave(max_ctx);
     const int part_tokens = tpw * PA_WAVE_TOKENS;
     const int max_parts = (int)((max_ctx + part_tokens - 1) / part_tokens);
     float* part_out = (float*)workspace;
