@@ -521,6 +521,30 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
     }
     const float* ml = part_ml + gh * max_parts * 2;
     const float* po = part_out + gh * max_parts * D + d;
+    if (np <= 16) {
+        // common case: every load of the row (the (max, sum) pairs and this thread's accumulator column) is issued
+        // at once, one memory round trip instead of three dependent ones
+        float mv[16], lv[16], pv[16];
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const bool on = p < np;
+            mv[p] = on ? ml[2 * p] : PA_NEG;
+            lv[p] = on ? ml[2 * p + 1] : 0.f;
+            pv[p] = on ? po[(int64_t)p * D] : 0.f;
+        }
+        float M = PA_NEG;
+#pragma unroll
+        for (int p = 0; p < 16; ++p) M = fmaxf(M, mv[p]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const float f = __builtin_amdgcn_exp2f(mv[p] - M);
+            den += f * lv[p];
+            num += f * pv[p];
+        }
+        out[gh * D + d] = T::from_float(num / den);
+        return;
+    }
     // pass 1: global maximum (every wave computes it for itself)
     float M = PA_NEG;
     for (int p0 = 0; p0 < np; p0 += 64) {

@@ -699,8 +699,10 @@ __device__ __forceinline__ void qkv_reduce8(const float* __restrict__ p, int64_t
     }
 }
 
+constexpr int RC_THREADS = 64;            // small workgroups: a 64-row step has only ~450 items per row to spread
+
 template <typename T>
-__global__ __launch_bounds__(256) void w8a16_reduce_rope_cache_kernel(
+__global__ __launch_bounds__(RC_THREADS) void w8a16_reduce_rope_cache_kernel(
     uint16_t* __restrict__ qkv, const float* __restrict__ partial, const float* __restrict__ scale,
     const uint16_t* __restrict__ bias, const void* __restrict__ cos, const void* __restrict__ sin,
     uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache, const int32_t* __restrict__ slot_mapping,
@@ -710,15 +712,14 @@ __global__ __launch_bounds__(256) void w8a16_reduce_rope_cache_kernel(
     const int cph = half >> 3;
     const int rot_items = (n_heads + n_kv) * cph;
     const int v_items = n_kv * D / 8;
-    const int item = blockIdx.y * 256 + threadIdx.x;
+    const int item = blockIdx.y * RC_THREADS + threadIdx.x;
     if (item >= rot_items + v_items) return;
+    // the slot is only needed where a row is stored: no load below waits for it
     const int64_t slot = slot_mapping[t];
-    const bool live = slot >= 0 && slot < num_slots;
     const int64_t row = (int64_t)n_kv * D;
     const int64_t stride = (int64_t)M * N;
     const float* prow = partial + (int64_t)t * N;
     if (item >= rot_items) {
-        if (!live) return;
         const int i = (item - rot_items) * 8;
         const int col = (n_heads + n_kv) * D + i;
         float v[8];
@@ -726,12 +727,11 @@ __global__ __launch_bounds__(256) void w8a16_reduce_rope_cache_kernel(
         u32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = pack2<T>(v[2 * e], v[2 * e + 1]);
-        *(u32x4*)(value_cache + slot * row + i) = o;
+        if (slot >= 0 && slot < num_slots) *(u32x4*)(value_cache + slot * row + i) = o;
         return;
     }
     const int h = item / cph, i = (item - h * cph) * 8;
     const bool is_k = h >= n_heads;
-    if (is_k && !live) return;
     const int col = h * D + i;                                // q heads, then k heads, are consecutive columns
     float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8];
     const int64_t trow = (int64_t)t * D;
@@ -751,9 +751,11 @@ __global__ __launch_bounds__(256) void w8a16_reduce_rope_cache_kernel(
         o2[e] = pack2<T>(b0, b1);
     }
     if (is_k) {
-        uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
-        *(u32x4*)(dst + i) = o1;
-        *(u32x4*)(dst + i + half) = o2;
+        if (slot >= 0 && slot < num_slots) {
+            uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
+            *(u32x4*)(dst + i) = o1;
+            *(u32x4*)(dst + i + half) = o2;
+        }
     } else {
         uint16_t* dst = qkv + (int64_t)t * N + col;
         *(u32x4*)dst = o1;
@@ -853,7 +855,8 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     if (rc_args && partial) {                                 // reduce + RoPE + cache scatter in one kernel
         const RopeCacheArgs& a = *rc_args;
         const int items = (a.n_heads + a.n_kv) * (a.head_dim / 16) + a.n_kv * a.head_dim / 8;
-        hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T>), dim3(m, (items + 255) / 256), dim3(256), 0, st,
+        hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T>), dim3(m, (items + RC_THREADS - 1) / RC_THREADS),
+                           dim3(RC_THREADS), 0, st,
                            (uint16_t*)y, partial, scale, (const uint16_t*)bias, a.cos, a.sin, (uint16_t*)a.key_cache,
                            (uint16_t*)a.value_cache, a.slot_mapping, m, n, p.split_k, a.n_heads, a.n_kv, a.head_dim,
                            a.num_slots, a.table_dtype);

@@ -20,6 +20,9 @@
 // applied on the global-address side, which makes the operand reads bank-conflict free.
 // Small N cannot fill the chip with output tiles alone: K is then split across workgroups, which write exact
 // int32 partial tiles that a second kernel sums (integer sums do not depend on the order).
+// Two more kernels serve the shapes where that one is not the best: a register-streaming kernel for narrow outputs
+// at 65+ rows (w8a8_regs_kernel) and, for very wide outputs at 129+ rows, 256 x 192 tiles on 8 waves with the
+// full-rate v_mfma_i32_32x32x32_i8 and a coalesced, LDS-turned epilogue (w8a8_wide_kernel).
 #include "common.h"
 
 namespace {
@@ -27,18 +30,22 @@ namespace {
 constexpr int Q_KSTEP = 64;
 constexpr int Q_TILE = 16 * Q_KSTEP;        // bytes of one packed weight tile
 
-template <int NT, bool MSPLIT, int ST>
+// MSPLIT: wave grid of a workgroup.  0: 1 x 4 (64 rows, the waves own different channels); 1: 4 x 1 (256 rows, one
+// channel group).
+template <int NT, int MSPLIT, int ST>
 struct Q2 {
     static constexpr int STAGES = ST;
     static constexpr int WAVES_M = MSPLIT ? 4 : 1;
     static constexpr int WAVES_N = MSPLIT ? 1 : 4;
+    static constexpr int WAVES = WAVES_M * WAVES_N;
     static constexpr int BM = 64 * WAVES_M;
     static constexpr int BN = 16 * NT * WAVES_N;
     static constexpr int XTILE = BM * Q_KSTEP;
     static constexpr int WTILES = BN / 16;
     static constexpr int STAGE = XTILE + WTILES * Q_TILE;
-    static constexpr int XL = BM / 64;                        // activation loads (16 rows each) per wave per stage
-    static constexpr int WL = (WTILES + 3) / 4;               // weight tile loads per wave per stage
+    static constexpr int XL = BM / 16 / WAVES;                // activation loads (16 rows each) per wave per stage
+    static constexpr int WL = (WTILES + WAVES - 1) / WAVES;   // weight tile loads per wave per stage
+    static_assert((BM / 16) % WAVES == 0, "activation tiles must divide over the waves");
     static constexpr int PENDING = (ST - 2) * (XL + WL);      // loads of the ST-2 younger steps may be in flight
     static constexpr int LDS_BYTES = ST * STAGE;
     static_assert(LDS_BYTES <= 160 * 1024 && PENDING < 64, "bad pipeline shape");
@@ -98,7 +105,7 @@ __device__ __forceinline__ void q2_store4(uint16_t* y, int32_t* acc_out, const f
 }
 
 // grid = (n_blocks, split_k, m_blocks)
-template <typename T, int NT, bool MSPLIT, int ST, bool KTAIL, bool XT>
+template <typename T, int NT, int MSPLIT, int ST, bool KTAIL, bool XT>
 __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(
     uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
     const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
@@ -282,6 +289,229 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(
 // flight per workgroup) and a main loop that is nothing but loads and matrix instructions.
 constexpr int QR_DEPTH = 3;
 
+// ---- wide outputs at 129+ rows: 256 x 192 tiles on 8 waves with mfma_i32_32x32x32_i8 ----------------------------
+// On gfx950 the 16x16x64 int8 instruction issues at half the rate of the 32x32x32 one (measured: 2.4 against
+// 4.4 POP/s with independent accumulators), so the kernel that is bound by the matrix cores uses the latter.
+// The packed tile format serves it unchanged: rows 32 b .. 32 b + 31 of a k-step are two consecutive 1 KiB
+// tiles, and lane (rho = lane & 31, h = lane >> 5) finds row rho, bytes 32 u + 16 h .. + 15 of the step at
+// tile (rho >> 4), 16-byte slot 16 (2 u + h) + (rho & 15).  Waves 4 (rows) x 2 (channels): a wave owns 64 rows x 96
+// channels = 2 x 3 blocks of 32 x 32.  Both operands go global -> LDS with LDS-direct loads into a ring of stages
+// (counted waits, one barrier per step); the operands of step s + 1 are read from LDS into a second register set
+// while the matrix cores work on step s.  Activations in tile order only.
+struct QW {
+    static constexpr int ST = 5;                              // stages: all that fit in 160 KiB of LDS
+    static constexpr int WAVES = 8;
+    static constexpr int BM = 256, WN = 96, BN = 2 * WN;
+    static constexpr int XTILE = BM * Q_KSTEP;                // 16 KiB
+    static constexpr int WTILES = BN / 16;                    // 12
+    static constexpr int STAGE = XTILE + WTILES * Q_TILE;     // 28 KiB
+    static constexpr int XL = BM / 16 / WAVES;                // 2 activation tile loads per wave per stage
+    static constexpr int WL = (WTILES + WAVES - 1) / WAVES;   // 2 weight tile loads per wave per stage (clamped)
+    static constexpr int L = XL + WL;
+    static constexpr int LDS_BYTES = ST * STAGE;
+};
+
+template <typename T>
+__global__ __launch_bounds__(QW::WAVES * 64, 1) void w8a8_wide_kernel(
+    uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
+    const int8_t* __restrict__ xq, const float* __restrict__ x_scale, const uint8_t* __restrict__ wp,
+    const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, int M,
+    int N, int K, int steps_per_split) {
+    using C = QW;
+    constexpr int ST = C::ST;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int wm = wv & 3, wn = wv >> 2;
+    const int KS = (K + Q_KSTEP - 1) / Q_KSTEP;
+    const int s_begin = blockIdx.y * steps_per_split;
+    const int s_end = min(KS, s_begin + steps_per_split);
+    const int s_last = s_end - 1;
+    const int m0 = blockIdx.z * C::BM;
+    const int nb0 = blockIdx.x * C::BN;
+    const int nw = nb0 + wn * C::WN;
+
+    i32x16 acc[3][2];
+#pragma unroll
+    for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0;
+
+    // loads: tiles past the matrix re-read the last one (their results are never stored); every wave issues the same
+    // number of loads per stage
+    const int m_tiles_total = (M + 15) >> 4, n_tiles_total = (N + 15) >> 4;
+    const uint8_t* xtile[C::XL];
+    const uint8_t* wtile[C::WL];
+    int wdst[C::WL];
+#pragma unroll
+    for (int i = 0; i < C::XL; ++i)
+        xtile[i] = (const uint8_t*)xq + (int64_t)min((m0 >> 4) + wv * C::XL + i, m_tiles_total - 1) * Q_TILE;
+#pragma unroll
+    for (int i = 0; i < C::WL; ++i) {
+        const int j = min(wv * C::WL + i, C::WTILES - 1);
+        wtile[i] = wp + (int64_t)min((nb0 >> 4) + j, n_tiles_total - 1) * Q_TILE;
+        wdst[i] = C::XTILE + j * Q_TILE;
+    }
+    const uint32_t wlane = lane * 16;
+    auto issue = [&](int stage, int s) {
+        const int sc = min(s, s_last);
+        uint8_t* dst = smem + stage * C::STAGE;
+#pragma unroll
+        for (int i = 0; i < C::XL; ++i)
+            q2_lds_direct16(xtile[i] + (int64_t)sc * m_tiles_total * Q_TILE, wlane, dst + 1024 * (wv * C::XL + i));
+#pragma unroll
+        for (int i = 0; i < C::WL; ++i)
+            q2_lds_direct16(wtile[i] + (int64_t)sc * n_tiles_total * Q_TILE, wlane, dst + wdst[i]);
+    };
+#pragma unroll
+    for (int p = 0; p < ST - 1; ++p) issue(p, s_begin + p);
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+    const int rho = lane & 31, h = lane >> 5;
+    const uint32_t lane32 = (uint32_t)((rho >> 4) * Q_TILE + (16 * h + (rho & 15)) * 16);
+    const uint32_t xoff = lds0 + 4 * wm * Q_TILE + lane32;                 // + 2048 mb + 512 u
+    const uint32_t woff = lds0 + C::XTILE + 6 * wn * Q_TILE + lane32;      // + 2048 nb + 512 u
+
+    // operand sets: xb[set][mb][u], wa[set][nb][u]
+    i32x4 xb[2][2][2], wa[2][3][2];
+    auto read_ops = [&](auto jc, int set) {
+        constexpr int SB = decltype(jc)::value * C::STAGE;
+        xb[set][0][0] = q2_lds_read16<SB>(xoff);
+        xb[set][0][1] = q2_lds_read16<SB + 512>(xoff);
+        xb[set][1][0] = q2_lds_read16<SB + 2048>(xoff);
+        xb[set][1][1] = q2_lds_read16<SB + 2048 + 512>(xoff);
+        wa[set][0][0] = q2_lds_read16<SB>(woff);
+        wa[set][0][1] = q2_lds_read16<SB + 512>(woff);
+        wa[set][1][0] = q2_lds_read16<SB + 2048>(woff);
+        wa[set][1][1] = q2_lds_read16<SB + 2048 + 512>(woff);
+        wa[set][2][0] = q2_lds_read16<SB + 4096>(woff);
+        wa[set][2][1] = q2_lds_read16<SB + 4096 + 512>(woff);
+    };
+    auto arrived = [&](int set) {                             // operands read one step ago are in their registers
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(xb[set][0][0]), "+v"(xb[set][0][1]), "+v"(xb[set][1][0]), "+v"(xb[set][1][1]),
+                       "+v"(wa[set][0][0]), "+v"(wa[set][0][1]), "+v"(wa[set][1][0]), "+v"(wa[set][1][1]),
+                       "+v"(wa[set][2][0]), "+v"(wa[set][2][1])
+                     :
+                     : "memory");
+    };
+    // step s_begin's stage has landed when at most the loads of the ST-2 younger steps are in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((ST - 2) * C::L) : "memory");
+    __builtin_amdgcn_s_barrier();
+    read_ops(std::integral_constant<int, 0>{}, 0);
+    auto pstep = [&](auto jc, auto setc, int s) {
+        constexpr int J = decltype(jc)::value;                // stage of step s
+        constexpr int SET = decltype(setc)::value;            // operand register set of step s (the step's parity)
+        __builtin_amdgcn_sched_barrier(0);
+        // the next step's stage must have landed, and this step's operands must be in their registers
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((ST - 3) * C::L) : "memory");
+        arrived(SET);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue((J + ST - 1) % ST, s + ST - 1);
+        read_ops(std::integral_constant<int, (J + 1) % ST>{}, SET ^ 1);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[SET][nb][u], xb[SET][mb][u], acc[nb][mb], 0, 0, 0);
+    };
+    // stages cycle with period ST, register sets with period 2: 2 * ST steps per trip
+#define QW_STEP(I)                                                                                              \
+    if (s + (I) < s_end) pstep(std::integral_constant<int, (I) % ST>{}, std::integral_constant<int, (I) & 1>{}, s + (I))
+    for (int s = s_begin; s < s_end; s += 2 * ST) {
+        QW_STEP(0); QW_STEP(1); QW_STEP(2); QW_STEP(3); QW_STEP(4);
+        QW_STEP(5); QW_STEP(6); QW_STEP(7); QW_STEP(8); QW_STEP(9);
+    }
+#undef QW_STEP
+    static_assert(ST == 5, "the unrolled trip above covers 2 * ST steps");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // look-ahead loads and reads still target the ring
+
+    // epilogue: lane holds row m = 32 mb + rho and, per block, channels 8 q + 4 h .. + 3 for q = 0..3.  Stored
+    // straight from that layout a wave would write 8-byte pieces of 32 different rows per instruction, so the
+    // dequantised tile (64 rows x 96 channels per wave) is turned through the wave's share of the now idle ring and
+    // written out as whole 16-byte pieces of consecutive rows; the int32 / split-K / ragged cases keep the direct path.
+    constexpr int EP_STRIDE = C::WN * 2 + 16;                 // bytes per staged row
+    static_assert(C::WAVES * 64 * EP_STRIDE <= C::LDS_BYTES, "the staged output must fit the ring");
+    if (y && !acc_out && !partial && (N & 7) == 0 && nw + C::WN <= N) {     // uniform per wave
+        __syncthreads();                                      // every wave is done with the ring
+        uint8_t* ep = smem + wv * (64 * EP_STRIDE);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            const int m = min(m0 + 64 * wm + 32 * mb + rho, M - 1);
+            const float xs = x_scale[m];
+#pragma unroll
+            for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = 32 * nb + 8 * q + 4 * h;
+                    const f32x4 ws4 = *(const f32x4*)(w_scale + nw + nl);
+                    float v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        v[i] = (float)acc[nb][mb][4 * q + i] * xs * ws4[i];
+                        if (bias) v[i] += T::to_float(bias[nw + nl + i]);
+                    }
+                    *(u32x2*)(ep + (32 * mb + rho) * EP_STRIDE + nl * 2) =
+                        (u32x2){pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+                }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        constexpr int CPRW = C::WN * 2 / 16;                  // 16-byte pieces per row
+#pragma unroll
+        for (int it = 0; it < 64 * CPRW / 64; ++it) {
+            const int c = it * 64 + lane;
+            const int row = c / CPRW, col = c - row * CPRW;
+            const int m = m0 + 64 * wm + row;
+            u32x4 o = *(const u32x4*)(ep + row * EP_STRIDE + col * 16);
+            if (m < M) {
+                const int64_t off = (int64_t)m * N + nw + 8 * col;
+                if (residual) {
+                    float a[8], rsd[8];
+                    unpack8<T>(o, a);
+                    unpack8<T>(*(const u32x4*)(residual + off), rsd);
+                    o = (u32x4){pack2<T>(a[0] + rsd[0], a[1] + rsd[1]), pack2<T>(a[2] + rsd[2], a[3] + rsd[3]),
+                                pack2<T>(a[4] + rsd[4], a[5] + rsd[5]), pack2<T>(a[6] + rsd[6], a[7] + rsd[7])};
+                }
+                *(u32x4*)(y + off) = o;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        const int m = m0 + 64 * wm + 32 * mb + rho;
+        if (m >= M) continue;
+#pragma unroll
+        for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nw + 32 * nb + 8 * q + 4 * h;
+                if (n >= N) continue;
+                const i32x4 a = {acc[nb][mb][4 * q], acc[nb][mb][4 * q + 1], acc[nb][mb][4 * q + 2],
+                                 acc[nb][mb][4 * q + 3]};
+                if (partial) {
+                    int32_t* p = partial + ((int64_t)blockIdx.y * M + m) * N + n;
+                    if (n + 3 < N && (N & 3) == 0) {
+                        *(i32x4*)p = a;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (n + i < N) p[i] = a[i];
+                    }
+                } else {
+                    q2_store4<T>(y, acc_out, x_scale, w_scale, bias, residual, m, n, N, a);
+                }
+            }
+    }
+}
+
 template <typename T, int WM, int MT, int NT>
 __global__ __launch_bounds__(256) void w8a8_regs_kernel(
     uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, int32_t* __restrict__ partial,
@@ -422,6 +652,7 @@ __global__ void w8a8_splitk_reduce_kernel(uint16_t* __restrict__ y, int32_t* __r
 struct QPlan {
     int regs;        // 0: LDS-staged kernel; 1: register-streaming kernel, 4x1 waves of 64 x 64
     bool msplit;
+    bool wide;       // w8a8_wide_kernel: 8 waves, 256 x 192 tiles
     int nt;
     int n_blocks, m_blocks, split_k, steps_per_split;
 };
@@ -429,6 +660,7 @@ struct QPlan {
 QPlan plan_w8a8(int m, int n, int k, bool x_tiled) {
     QPlan p;
     p.msplit = m > 64;
+    p.wide = false;
     p.regs = 0;
     const int steps = (k + Q_KSTEP - 1) / Q_KSTEP;
     if (x_tiled && m > 64 && n < 8192) {
@@ -440,17 +672,21 @@ QPlan plan_w8a8(int m, int n, int k, bool x_tiled) {
     } else if (p.msplit) {
         // 80-channel tiles, two workgroups per CU: close to 512 tiles balance best; wide N only
         p.nt = n >= 16384 ? 5 : 4;
+        // very wide outputs: 256 x 192 tiles on 8 waves, one workgroup per CU (one staged activation tile serves
+        // more channels, and the 32 x 32 x 32 instruction runs at twice the rate of the 16 x 16 x 64 one)
+        p.wide = x_tiled && n >= 16384 && m > 128;
         p.m_blocks = (m + 255) / 256;
     } else {
         p.nt = 2;
         p.m_blocks = 1;
     }
-    const int bn = 16 * p.nt * (p.regs || p.msplit ? 1 : 4);
+    const int bn = p.wide ? QW::BN : 16 * p.nt * (p.regs || p.msplit ? 1 : 4);
     p.n_blocks = (n + bn - 1) / bn;
     // split K only as far as needed to give every CU a workgroup, and keep at least 16 steps per split: every
     // split writes (and the reduce kernel reads back) an int32 copy of the output
     const int tiles = p.n_blocks * p.m_blocks;
-    int sk = tiles >= 200 ? 1 : (224 + tiles - 1) / tiles;
+    // (the 8-wave tiles hold a whole CU each: from half the CUs up, splitting K would only add partial traffic)
+    int sk = tiles >= (p.wide ? 128 : 200) ? 1 : (224 + tiles - 1) / tiles;
     const int max_sk = steps / 16 < 1 ? 1 : steps / 16;
     sk = sk > max_sk ? max_sk : sk;
     sk = sk > 32 ? 32 : sk;
@@ -480,7 +716,8 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
             if (e != hipSuccess) return (int)e;                                                                  \
             configured[dev] = true;                                                                              \
         }                                                                                                        \
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (uint16_t*)y, acc_out, partial, xq, x_scale, wp, w_scale, \
+        hipLaunchKernelGGL(kern, grid, dim3(Q2<NTV, MS, STV>::WAVES * 64), lds, st, (uint16_t*)y, acc_out, partial, xq,  \
+                           x_scale, wp, w_scale,                                                                  \
                            (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split);         \
     } while (0)
 #define Q_LAUNCH_KT(NTV, MS, STV)                                                                                 \
@@ -494,9 +731,23 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
                        xq, x_scale, wp, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,          \
                        p.steps_per_split)
     if (p.regs == 1) QR_LAUNCH(4, 4, 4);
-    else if (!p.msplit) Q_LAUNCH_KT(2, false, 4);
-    else if (p.nt == 5) Q_LAUNCH_KT(5, true, 3);
-    else Q_LAUNCH_KT(4, true, 3);
+    else if (!p.msplit) Q_LAUNCH_KT(2, 0, 4);
+    else if (p.wide) {
+        static bool configured[MF_MAX_DEVICES] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MF_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+        if (!configured[dev]) {
+            hipError_t e = hipFuncSetAttribute((const void*)w8a8_wide_kernel<T>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, QW::LDS_BYTES);
+            if (e != hipSuccess) return (int)e;
+            configured[dev] = true;
+        }
+        hipLaunchKernelGGL(w8a8_wide_kernel<T>, grid, dim3(QW::WAVES * 64), QW::LDS_BYTES, st, (uint16_t*)y, acc_out,
+                           partial, xq, x_scale, wp, w_scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k,
+                           p.steps_per_split);
+    }
+    else if (p.nt == 5) Q_LAUNCH_KT(5, 1, 3);
+    else Q_LAUNCH_KT(4, 1, 3);
 #undef QR_LAUNCH
 #undef Q_LAUNCH_KT
 #undef Q_LAUNCH

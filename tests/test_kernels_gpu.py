@@ -717,7 +717,8 @@ def test_dynamic_quant_bit_exact(dtype, m, k, smooth):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 3584, 3584), (130, 200, 1088), (1, 64, 64), (64, 257, 512),
-                                   (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16), (33, 130, 2064)])
+                                   (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16), (33, 130, 2064),
+                                   (300, 16500, 208), (130, 16384, 80)])       # the 8-wave 256 x 160 tiles, ragged
 def test_w8a8_gemm_int32_bit_exact(m, n, k):
     rng = np.random.default_rng(10)
     dtype = torch.bfloat16
@@ -755,7 +756,7 @@ def test_dynamic_quant_tiled_layout_bit_exact(m, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16),
-                                   (33, 130, 2064), (1, 64, 64)])
+                                   (33, 130, 2064), (1, 64, 64), (300, 16500, 208), (130, 16384, 80)])
 def test_w8a8_tiled_activations_bit_exact(m, n, k):
     """dynamic_quant(tiled) -> w8a8 GEMM: int32 accumulators equal the integer matmul of the oracle's quantisation."""
     rng = np.random.default_rng(3 * m + n)
