@@ -478,6 +478,317 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     }
 }
 
+// ---- prefill on the 32x32x16 MFMA ---------------------------------------------------------------------------------
+// Prefill has (query, head) columns in abundance.  A workgroup of 4 waves serves 128 consecutive columns of one kv
+// head (32 per wave) and walks the keys and values of their causal range once, 64 tokens at a time: the 256 threads
+// fetch a tile with coalesced 16-byte loads and stage it in LDS (double-buffered, one barrier per tile), and every
+// wave multiplies its own 32 columns against it.  Each K / V byte is thus read from L2 once per 128 columns; with
+// one tile stream per wave the kernel was bound by L2 bandwidth.  The 32x32x16 instruction does twice the work of
+// the 16x16x32 one in the same issue time and halves the LDS reads per column.
+//   S^T[token 32, col 32] = K[token, :] . Q[col, :]    D/16 MFMAs; lane (rho, h) holds row rho, k = 8h .. 8h+7
+//   accumulator register i of lane (rho, h) is token 8 (i / 4) + 4 h + i % 4 of column rho, so registers
+//   8 T .. 8 T + 7 are, in order, exactly the 8 k-values a lane supplies to the B operand of token half T when that
+//   half's 16 tokens are taken in the order (4 h + e, 8 + 4 h + e); the V^T operand is read in the same order with
+//   the transposing LDS read.
+// A wave owns its columns over the whole partition, so there is no merge: it writes final rows (single partition) or
+// fp32 partials for the reduce kernel.
+constexpr int PF_COLS = 128;                                  // columns per workgroup
+constexpr int PF_TOK = 64;                                    // tokens per staged tile
+
+template <int D>
+struct PfSmem {
+    // K rows: an odd number of 16-byte slots keeps the 32-row operand reads (16 consecutive rows of one k-chunk are
+    // served together) free of bank conflicts; V rows: the stride the transposing reads want (see PaSmem)
+    static constexpr int KSTRIDE = D * 2 + 16;
+    static constexpr int VSTRIDE = D * 2 + 32;
+    static constexpr int KBYTES = PF_TOK * KSTRIDE;
+    static constexpr int BUF = KBYTES + PF_TOK * VSTRIDE;
+    static constexpr int BYTES = 2 * BUF;
+};
+
+template <typename T, int D, bool TIB>
+__global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
+    uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+    const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
+    int n_rep, int block_size, int max_blocks, int num_blocks, int max_parts, float scale_log2, int64_t q_stride,
+    int batch, const int32_t* __restrict__ q_starts, int part_tokens, int64_t kv_stride, int rows) {
+    using vec8 = typename T::vec8;
+    constexpr int KS = D / 16;                                // k-steps of the score product
+    constexpr int DB = D / 32;                                // 32-row blocks of O^T
+    constexpr int KSTRIDE = PfSmem<D>::KSTRIDE, VSTRIDE = PfSmem<D>::VSTRIDE;
+    constexpr int CPR = D * 2 / 16;                           // 16-byte chunks per row
+    constexpr int RPP = PA_WAVES * 64 / CPR;                  // rows one workgroup-wide load covers
+    constexpr int NI = (PF_TOK + RPP - 1) / RPP;              // loads per thread per tile per tensor
+    constexpr int TIDS = PA_WAVES * 64;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];
+
+    // work list: see paged_attention_kernel; a sequence has ceil(q_len * n_rep / 128) column groups
+    int b = -1, part = 0, L = 0, kg = 0, q_len = 1, q_start = 0, col_groups = 1;
+    {
+        const int pidx = blockIdx.x;
+        const int ln = threadIdx.x & 63;
+        int base = 0;
+        for (int c0 = 0; c0 < batch; c0 += 64) {
+            const int bb = c0 + ln;
+            int len, ql, qs;
+            pf_seq(bb, q_starts, ctx_lens, block_tables == nullptr, rows, max_blocks * block_size, batch, qs, ql, len);
+            const int ncg = (ql * n_rep + PF_COLS - 1) / PF_COLS;
+            int np = len > 0 ? (len + part_tokens - 1) / part_tokens : 0;
+            np = np < max_parts ? np : max_parts;
+            const int per_seq = np * n_kv * ncg;
+            int incl = per_seq;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int t = __shfl_up(incl, o, 64);
+                if (ln >= o) incl += t;
+            }
+            const int total = __shfl(incl, 63, 64);
+            if (pidx < base + total) {
+                const bool hit = pidx >= base + incl - per_seq && pidx < base + incl;
+                const uint64_t m = __ballot(hit);
+                const int src = __ffsll((unsigned long long)m) - 1;
+                b = c0 + src;
+                const int rem = pidx - (base + __shfl(incl - per_seq, src, 64));
+                const int npb = __shfl(np, src, 64);
+                kg = rem / npb;
+                part = rem - kg * npb;
+                L = __shfl(len, src, 64);
+                q_len = __shfl(ql, src, 64);
+                q_start = __shfl(qs, src, 64);
+                col_groups = __shfl(ncg, src, 64);
+                break;
+            }
+            base += total;
+        }
+    }
+    if (b < 0) return;                                        // uniform over the workgroup
+    kg = __builtin_amdgcn_readfirstlane(kg);
+    col_groups = __builtin_amdgcn_readfirstlane(col_groups);
+    // kv heads fastest: consecutive workgroups go to consecutive XCDs, so with 8 kv heads each XCD's L2 sees the keys
+    // and values of one head only; column groups from the last (longest causal range) to the first, so that the
+    // long workgroups start first and the short ones fill the tail
+    const int kvh = kg % n_kv;
+    const int hg = col_groups - 1 - kg / n_kv;                // column group
+    b = __builtin_amdgcn_readfirstlane(b);
+    part = __builtin_amdgcn_readfirstlane(part);
+    L = __builtin_amdgcn_readfirstlane(L);
+    q_len = __builtin_amdgcn_readfirstlane(q_len);
+    q_start = __builtin_amdgcn_readfirstlane(q_start);
+    const int part_start = part * part_tokens;
+    const int ctx_before = L - q_len;                         // cache tokens older than this step's queries
+    // the farthest token any column of this group may see; partitions past it have nothing to do (the reduce kernel
+    // counts partitions per query row and never reads them)
+    const int Lwg = ctx_before + min(q_len, (hg * PF_COLS + PF_COLS - 1) / n_rep + 1);
+    if (part_start >= Lwg) return;                            // uniform over the workgroup
+
+    const int tid = threadIdx.x;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int rho = lane & 31;
+    const int h = lane >> 5;
+
+    // ---- this wave's 32 columns; Q as B operand: lane (rho, h) holds Q[column rho][16 j + 8 h .. +8]
+    const int c0 = hg * PF_COLS + w * 32;
+    const int hh = c0 + rho;
+    const int qi = hh / n_rep;                                // query index of this lane's column
+    const int hcol = hh - qi * n_rep;                         // head within the kv group
+    const bool col_ok = qi < q_len;
+    const int Lcol = col_ok ? ctx_before + qi + 1 : 0;        // causal limit of this lane's column
+    const int q_first = c0 / n_rep;                           // first query of the wave
+    const int Lw = q_first < q_len ? ctx_before + min(q_len, (c0 + 31) / n_rep + 1) : 0;   // farthest token of the wave
+    const int Lmask = ctx_before + q_first + 1;               // sub-tiles that end at or before it need no mask
+    vec8 qreg[KS];
+    {
+        const uint16_t* qp = q + (int64_t)(q_start + (col_ok ? qi : 0)) * q_stride +
+                             (int64_t)(kvh * n_rep + (col_ok ? hcol : 0)) * D + 8 * h;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (col_ok) v = *(const u32x4*)(qp + 16 * j);
+            qreg[j] = bitcast<vec8>(v);
+        }
+    }
+
+    f32x16 acc[DB];                                           // acc[db][i]: d = 32 db + 8 (i / 4) + 4 h + i % 4
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+    // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
+    // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0
+    float m_run = 0.5f * PA_NEG, l_run = 0.f;
+
+    const bool contiguous = block_tables == nullptr;
+    const int32_t* table = block_tables + (int64_t)b * max_blocks;
+    const int64_t row_bytes = kv_stride * 2;
+    const int lrow = tid / CPR;                               // cooperative-load coordinates of this thread
+    const int lchunk = tid - lrow * CPR;
+    const uint32_t lane_col = (uint32_t)(kvh * D * 2 + 16 * lchunk);
+
+    const int part_end = min(Lwg, part_start + part_tokens);
+    const int ntiles = (part_end - part_start + PF_TOK - 1) / PF_TOK;
+
+    // tile t: rows past the group's range re-read its last row (their scores are masked)
+    auto load_tile = [&](u32x4* kreg, u32x4* vreg, int t) {
+        const int ts = part_start + t * PF_TOK;
+        int64_t slot0 = 0;
+        if constexpr (TIB) {                                  // the tile lies inside one block: one uniform lookup
+            if (contiguous) {
+                slot0 = (int64_t)q_start + ts;
+            } else {
+                const int bi = ts / block_size;
+                int blk = table[bi];
+                blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;   // never leave the cache allocation
+                slot0 = (int64_t)blk * block_size + (ts - bi * block_size);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int row = lrow + RPP * i;
+            if (RPP * (i + 1) > PF_TOK && row >= PF_TOK) break;
+            const int rc = min(row, Lwg - 1 - ts);
+            int64_t off;
+            if constexpr (TIB) {
+                off = (slot0 + rc) * row_bytes + lane_col;
+            } else {
+                const int tok = ts + rc;
+                const int bi = tok / block_size;
+                int blk = table[bi];
+                blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
+                off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_bytes + lane_col;
+            }
+            kreg[i] = *(const u32x4*)((const uint8_t*)kc + off);
+            vreg[i] = *(const u32x4*)((const uint8_t*)vc + off);
+        }
+    };
+    auto store_tile = [&](const u32x4* kreg, const u32x4* vreg, int buf) {
+        uint8_t* kb = pf_smem + buf * PfSmem<D>::BUF;
+        uint8_t* vb = kb + PfSmem<D>::KBYTES;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int row = lrow + RPP * i;
+            if (RPP * (i + 1) > PF_TOK && row >= PF_TOK) break;
+            *(u32x4*)(kb + row * KSTRIDE + 16 * lchunk) = kreg[i];
+            *(u32x4*)(vb + row * VSTRIDE + 16 * lchunk) = vreg[i];
+        }
+    };
+
+    u32x4 kreg[NI], vreg[NI];
+    load_tile(kreg, vreg, 0);
+    store_tile(kreg, vreg, 0);
+    if (ntiles > 1) load_tile(kreg, vreg, 1);
+
+    const int jj = rho & 15;
+    const int voff = (4 * h + (jj >> 2)) * VSTRIDE + ((rho & 16) + 4 * (jj & 3)) * 2;
+#pragma unroll 1
+    for (int t = 0; t < ntiles; ++t) {
+        // tile t is staged and every wave is done with tile t - 1, whose buffer takes tile t + 1
+        __syncthreads();
+        if (t + 1 < ntiles) store_tile(kreg, vreg, (t + 1) & 1);
+        if (t + 2 < ntiles) load_tile(kreg, vreg, t + 2);    // in flight behind this tile's math
+        const uint8_t* kb = pf_smem + (t & 1) * PfSmem<D>::BUF;
+        const uint8_t* vb = kb + PfSmem<D>::KBYTES;
+#pragma unroll
+        for (int s = 0; s < PF_TOK / 32; ++s) {
+            const int tstart = part_start + t * PF_TOK + 32 * s;
+            if (tstart >= Lw) break;                          // nothing this wave's columns may see (wave-uniform)
+            f32x16 sc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+#pragma unroll
+            for (int j = 0; j < KS; ++j) {
+                const u32x4 ka = *(const u32x4*)(kb + (32 * s + rho) * KSTRIDE + (16 * j + 8 * h) * 2);
+                sc = T::mfma32(bitcast<vec8>(ka), qreg[j], sc);
+            }
+            float tmax = PA_NEG;
+            if (tstart + 32 <= Lmask) {                       // every token is visible to every column of the wave
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    sc[i] *= scale_log2;
+                    tmax = fmaxf(tmax, sc[i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int tok = tstart + 8 * (i >> 2) + 4 * h + (i & 3);
+                    const float v = tok < Lcol ? sc[i] * scale_log2 : PA_NEG;
+                    sc[i] = v;
+                    tmax = fmaxf(tmax, v);
+                }
+            }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = fmaxf(m_run, tmax);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            float psum = 0.f;
+            uint32_t pp[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float p0 = __builtin_amdgcn_exp2f(sc[2 * k] - m_new);
+                const float p1 = __builtin_amdgcn_exp2f(sc[2 * k + 1] - m_new);
+                pp[k] = pack2<T>(p0, p1);
+                // the denominator sums the probabilities as the PV product sees them (rounded to T)
+                psum += T::to_float((uint16_t)(pp[k] & 0xffff)) + T::to_float((uint16_t)(pp[k] >> 16));
+            }
+            // the running maximum rarely moves after the first tiles: when it moved for no lane, alpha is exactly 1
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+            }
+            l_run += psum;
+            const vec8 pfrag0 = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
+            const vec8 pfrag1 = bitcast<vec8>((u32x4){pp[4], pp[5], pp[6], pp[7]});
+
+            // ---- O^T += V^T P^T.  Within 16 lanes (d rows rho0 .. rho0+15, token quarter h) lane j names the 4 values
+            // V[token 16 T + 4 h + (j >> 2)][32 db + rho0 + 4 (j & 3) ..] and receives V[token 16 T + 4 h + e][its d
+            // row]; the second read, 8 tokens on, supplies k-values 4 .. 7.
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                for (int th = 0; th < 2; ++th) {
+                    const uint8_t* p0 = vb + (32 * s + 16 * th) * VSTRIDE + voff + 64 * db;
+                    const u32x2 l2 = bitcast<u32x2>(lds_read_tr16(p0));
+                    const u32x2 h2 = bitcast<u32x2>(lds_read_tr16(p0 + 8 * VSTRIDE));
+                    acc[db] = T::mfma32(bitcast<vec8>((u32x4){l2[0], l2[1], h2[0], h2[1]}), th ? pfrag1 : pfrag0,
+                                        acc[db]);
+                }
+            }
+        }
+    }
+
+    // ---- every lane writes its column's values: 4 consecutive d per accumulator quad
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (!col_ok) return;
+    const int64_t gh = (int64_t)(q_start + qi) * n_heads + kvh * n_rep + hcol;
+    if (max_parts == 1) {
+        const float inv = 1.0f / l_run;
+        uint16_t* dst = out + gh * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                *(u32x2*)(dst + 32 * db + 8 * q4) =
+                    (u32x2){pack2<T>(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
+                            pack2<T>(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv)};
+    } else {
+        const int64_t pi = gh * max_parts + part;
+        float* dst = part_out + pi * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                *(f32x4*)(dst + 32 * db + 8 * q4) =
+                    (f32x4){acc[db][4 * q4], acc[db][4 * q4 + 1], acc[db][4 * q4 + 2], acc[db][4 * q4 + 3]};
+        if (h == 0) {
+            part_ml[pi * 2] = m_run;
+            part_ml[pi * 2 + 1] = l_run;
+        }
+    }
+}
+
 // Causal limit (number of cache tokens visible) of query row `row` in a prefill step; 0 for a row that belongs to
 // no sequence (before q_starts[0], from q_starts[batch] on, or beyond its sequence's context).
 __device__ inline int pf_row_limit(int row, const int32_t* __restrict__ q_starts,
@@ -634,20 +945,21 @@ __global__ void pa_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t* 
 }
 
 // ---- prefill --------------------------------------------------------------------------------------------------
-// Partitioning rule shared by the workspace query and the launch.  A workgroup serves 16 (query, head) columns of one
-// kv head; when the query rows alone give the chip enough workgroups one partition spans the whole context and no
-// partials are written, otherwise the context is cut so that about a thousand workgroups exist.
+// Partitioning rule shared by the workspace query and the launch.  A workgroup serves 128 (query, head) columns of
+// one kv head (16 with an int8 cache); when the query rows alone give the chip enough workgroups one partition spans the
+// whole context and no partials are written, otherwise the context is cut so that about a thousand workgroups exist.
 struct PfPlan {
     int part_tokens;
     int max_parts;
-    int64_t col_groups;                                       // upper bound over the batch
+    int64_t col_groups16, col_groups128;                      // upper bounds over the batch, per column-group width
 };
 
 static inline PfPlan pf_plan(int batch, int64_t total_q, int n_heads, int n_kv, int64_t max_ctx) {
     const int n_rep = n_heads / n_kv;
     PfPlan p;
-    p.col_groups = (total_q * n_rep + 15) / 16 + batch;       // each sequence rounds its own columns up
-    const int64_t wgs = std::max<int64_t>(1, (total_q * n_rep + 15) / 16) * n_kv;
+    p.col_groups16 = (total_q * n_rep + 15) / 16 + batch;     // each sequence rounds its own columns up
+    p.col_groups128 = (total_q * n_rep + PF_COLS - 1) / PF_COLS + batch;
+    const int64_t wgs = std::max<int64_t>(1, (total_q * n_rep + PF_COLS - 1) / PF_COLS) * n_kv;
     int64_t want = (1024 + wgs - 1) / wgs;
     const int64_t most = std::max<int64_t>(1, (max_ctx + 255) / 256);
     want = std::min(want, most);
@@ -678,7 +990,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
     float* part_ml = part_out ? part_out + (int64_t)total_q * n_heads * plan.max_parts * D : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
-    const int64_t wgs = plan.col_groups * n_kv * plan.max_parts;
+    const int64_t wgs = (KV8 ? plan.col_groups16 : plan.col_groups128) * n_kv * plan.max_parts;
     if (wgs > 0x7fffffffLL) {
         mf_set_error("paged_attention_prefill: %lld workgroups exceed the grid limit", (long long)wgs);
         return 1;
@@ -689,17 +1001,43 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
         int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
-    const bool tib = contiguous || block_size % PA_TILE == 0;  // a 32-token tile never straddles two blocks
+    if constexpr (KV8) {
+        const bool tib = block_size % PA_TILE == 0;           // a 32-token tile never straddles two blocks
 #define PF_LAUNCH(TIBV)                                                                                           \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, KV8, TIBV>), dim3((unsigned)wgs),                    \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, true, TIBV>), dim3((unsigned)wgs),                   \
                        dim3(PA_WAVES * 64), 0, st, (uint16_t*)out, part_out, part_ml, (const uint16_t*)query,      \
                        (const uint16_t*)key_cache, (const uint16_t*)value_cache, block_tables, context_lens,       \
                        n_heads, n_kv, n_rep, (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, \
                        scale_log2, q_stride, batch, q_starts, plan.part_tokens, kv_stride, total_q, kv_scale,      \
                        kv_offset)
-    if (tib) PF_LAUNCH(true);
-    else PF_LAUNCH(false);
+        if (tib) PF_LAUNCH(true);
+        else PF_LAUNCH(false);
 #undef PF_LAUNCH
+    } else {
+        const bool tib = contiguous || block_size % PF_TOK == 0;   // a staged tile never straddles two blocks
+        static bool lds_set[2][MF_MAX_DEVICES] = {};          // the tile buffers exceed the default dynamic LDS limit
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return (int)e;
+#define PF_LAUNCH(TIBV)                                                                                           \
+    {                                                                                                             \
+        auto kern = prefill_attention_kernel<T, D, TIBV>;                                                         \
+        if (dev < 0 || dev >= MF_MAX_DEVICES || !lds_set[TIBV][dev]) {                                            \
+            e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,                \
+                                    PfSmem<D>::BYTES);                                                            \
+            if (e != hipSuccess) return (int)e;                                                                   \
+            if (dev >= 0 && dev < MF_MAX_DEVICES) lds_set[TIBV][dev] = true;                                      \
+        }                                                                                                         \
+        hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(PA_WAVES * 64), PfSmem<D>::BYTES, st, (uint16_t*)out,  \
+                           part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,                 \
+                           (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep,        \
+                           block_size, max_blocks, num_blocks, plan.max_parts, scale_log2, q_stride, batch,       \
+                           q_starts, plan.part_tokens, kv_stride, total_q);                                       \
+    }
+        if (tib) PF_LAUNCH(true)
+        else PF_LAUNCH(false)
+#undef PF_LAUNCH
+    }
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
