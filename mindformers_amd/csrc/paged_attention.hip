@@ -480,16 +480,24 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 
 // ---- prefill on the 32x32x16 MFMA ---------------------------------------------------------------------------------
 // Prefill has (query, head) columns in abundance.  A workgroup of 4 waves serves 128 consecutive columns of one kv
-// head (32 per wave) and walks the keys and values of their causal range once, 64 tokens at a time: the 256 threads
-// fetch a tile with coalesced 16-byte loads and stage it in LDS (double-buffered, one barrier per tile), and every
-// wave multiplies its own 32 columns against it.  Each K / V byte is thus read from L2 once per 128 columns; with
-// one tile stream per wave the kernel was bound by L2 bandwidth.  The 32x32x16 instruction does twice the work of
-// the 16x16x32 one in the same issue time and halves the LDS reads per column.
+// head (32 per wave) and walks the keys and values of their causal range once, 64 tokens at a time; every wave
+// multiplies its own 32 columns against the shared tile, so each K / V byte is read from L2 once per 128 columns
+// (with one tile stream per wave the kernel was bound by L2 bandwidth).  The 32x32x16 instruction does twice the
+// work of the 16x16x32 one in the same issue time and halves the LDS reads per column.
 //   S^T[token 32, col 32] = K[token, :] . Q[col, :]    D/16 MFMAs; lane (rho, h) holds row rho, k = 8h .. 8h+7
 //   accumulator register i of lane (rho, h) is token 8 (i / 4) + 4 h + i % 4 of column rho, so registers
 //   8 T .. 8 T + 7 are, in order, exactly the 8 k-values a lane supplies to the B operand of token half T when that
 //   half's 16 tokens are taken in the order (4 h + e, 8 + 4 h + e); the V^T operand is read in the same order with
 //   the transposing LDS read.
+// Tiles go from global memory straight into LDS (no registers in between), double-buffered with one barrier per tile.
+// Such a load writes 64 consecutive 16-byte slots, so rows cannot be padded; instead the 16-byte chunks of a row are
+// permuted by the address each lane supplies:
+//   K: chunk c of row t sits in slot c ^ key(t): the 16 rows of one chunk that an operand read serves together
+//      land on 16 different slots;
+//   V: chunk c of row t sits in slot (c + 4 key4(t)) mod chunks-per-row: the 4 tokens x 64 bytes a transposing read
+//      serves together land on different slots.
+// The LDS reads are issued by hand a few MFMAs ahead (the compiler would wait for each before the next), and the
+// exponentials of the tile's second half run beside the first half's PV MFMAs.
 // A wave owns its columns over the whole partition, so there is no merge: it writes final rows (single partition) or
 // fp32 partials for the reduce kernel.
 constexpr int PF_COLS = 128;                                  // columns per workgroup
@@ -497,14 +505,39 @@ constexpr int PF_TOK = 64;                                    // tokens per stag
 
 template <int D>
 struct PfSmem {
-    // K rows: an odd number of 16-byte slots keeps the 32-row operand reads (16 consecutive rows of one k-chunk are
-    // served together) free of bank conflicts; V rows: the stride the transposing reads want (see PaSmem)
-    static constexpr int KSTRIDE = D * 2 + 16;
-    static constexpr int VSTRIDE = D * 2 + 32;
-    static constexpr int KBYTES = PF_TOK * KSTRIDE;
-    static constexpr int BUF = KBYTES + PF_TOK * VSTRIDE;
+    static constexpr int ROWB = D * 2;                        // bytes per staged row
+    static constexpr int KBYTES = PF_TOK * ROWB;
+    static constexpr int BUF = 2 * KBYTES;                    // K tile, then V tile
     static constexpr int BYTES = 2 * BUF;
 };
+
+template <int OFF>
+__device__ __forceinline__ u32x4 pf_lds_read16(uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x2 pf_lds_read_tr(uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
+    u32x2 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void pf_wait_lds() {
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+template <typename F, int... I>
+__device__ __forceinline__ void pf_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void pf_static_for(F&& f) {
+    pf_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <typename T, int D, bool TIB>
 __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
@@ -514,13 +547,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     int n_rep, int block_size, int max_blocks, int num_blocks, int max_parts, float scale_log2, int64_t q_stride,
     int batch, const int32_t* __restrict__ q_starts, int part_tokens, int64_t kv_stride, int rows) {
     using vec8 = typename T::vec8;
+    using S = PfSmem<D>;
     constexpr int KS = D / 16;                                // k-steps of the score product
     constexpr int DB = D / 32;                                // 32-row blocks of O^T
-    constexpr int KSTRIDE = PfSmem<D>::KSTRIDE, VSTRIDE = PfSmem<D>::VSTRIDE;
-    constexpr int CPR = D * 2 / 16;                           // 16-byte chunks per row
-    constexpr int RPP = PA_WAVES * 64 / CPR;                  // rows one workgroup-wide load covers
-    constexpr int NI = (PF_TOK + RPP - 1) / RPP;              // loads per thread per tile per tensor
-    constexpr int TIDS = PA_WAVES * 64;
+    constexpr int ROWB = S::ROWB;
+    constexpr int CPR = ROWB / 16;                            // 16-byte chunks per row
+    constexpr int RPB = 16 / CPR;                             // rows per 256 bytes of LDS
+    constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
+    constexpr int NI = PF_TOK / RPI / PA_WAVES;               // loads per wave per tile per tensor
 
     extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];
 
@@ -598,7 +632,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     const int Lcol = col_ok ? ctx_before + qi + 1 : 0;        // causal limit of this lane's column
     const int q_first = c0 / n_rep;                           // first query of the wave
     const int Lw = q_first < q_len ? ctx_before + min(q_len, (c0 + 31) / n_rep + 1) : 0;   // farthest token of the wave
-    const int Lmask = ctx_before + q_first + 1;               // sub-tiles that end at or before it need no mask
+    const int Lmask = ctx_before + q_first + 1;               // tiles that end at or before it need no mask
     vec8 qreg[KS];
     {
         const uint16_t* qp = q + (int64_t)(q_start + (col_ok ? qi : 0)) * q_stride +
@@ -617,22 +651,33 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
     // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
-    // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0
+    // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0.  Maxima are kept in raw score units: the
+    // (positive) softmax scale is applied inside the exponent.
     float m_run = 0.5f * PA_NEG, l_run = 0.f;
 
     const bool contiguous = block_tables == nullptr;
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
     const int64_t row_bytes = kv_stride * 2;
-    const int lrow = tid / CPR;                               // cooperative-load coordinates of this thread
-    const int lchunk = tid - lrow * CPR;
-    const uint32_t lane_col = (uint32_t)(kvh * D * 2 + 16 * lchunk);
 
+    // ---- tile loads: load i of wave w brings rows (4 i + w) RPI .. + RPI - 1; lane = (row in the group, LDS slot)
+    const int lrow = lane / CPR;
+    const int lslot = lane - lrow * CPR;
+    uint32_t kcol[NI], vcol[NI];                              // byte offset of this lane's chunk within a row
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int row = (PA_WAVES * i + w) * RPI + lrow;
+        const int key = (row / RPB) & (CPR - 1);
+        const int key4 = (row / RPB) & (CPR / 4 - 1);
+        kcol[i] = (uint32_t)(kvh * D * 2 + 16 * (lslot ^ key));
+        vcol[i] = (uint32_t)(kvh * D * 2 + 16 * ((lslot - 4 * key4) & (CPR - 1)));
+    }
     const int part_end = min(Lwg, part_start + part_tokens);
     const int ntiles = (part_end - part_start + PF_TOK - 1) / PF_TOK;
 
-    // tile t: rows past the group's range re-read its last row (their scores are masked)
-    auto load_tile = [&](u32x4* kreg, u32x4* vreg, int t) {
+    // rows past the group's range re-read its last row (their scores are masked)
+    auto issue_tile = [&](int t) {
         const int ts = part_start + t * PF_TOK;
+        uint8_t* kdst = pf_smem + (t & 1) * S::BUF;
         int64_t slot0 = 0;
         if constexpr (TIB) {                                  // the tile lies inside one block: one uniform lookup
             if (contiguous) {
@@ -644,118 +689,155 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
                 slot0 = (int64_t)blk * block_size + (ts - bi * block_size);
             }
         }
+        const int last_row = Lwg - 1 - ts;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int row = lrow + RPP * i;
-            if (RPP * (i + 1) > PF_TOK && row >= PF_TOK) break;
-            const int rc = min(row, Lwg - 1 - ts);
+            const int r0 = (PA_WAVES * i + w) * RPI;
+            const int rc = min(r0 + lrow, last_row);
             int64_t off;
             if constexpr (TIB) {
-                off = (slot0 + rc) * row_bytes + lane_col;
+                off = (slot0 + rc) * row_bytes;
             } else {
                 const int tok = ts + rc;
                 const int bi = tok / block_size;
                 int blk = table[bi];
                 blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
-                off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_bytes + lane_col;
+                off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_bytes;
             }
-            kreg[i] = *(const u32x4*)((const uint8_t*)kc + off);
-            vreg[i] = *(const u32x4*)((const uint8_t*)vc + off);
-        }
-    };
-    auto store_tile = [&](const u32x4* kreg, const u32x4* vreg, int buf) {
-        uint8_t* kb = pf_smem + buf * PfSmem<D>::BUF;
-        uint8_t* vb = kb + PfSmem<D>::KBYTES;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int row = lrow + RPP * i;
-            if (RPP * (i + 1) > PF_TOK && row >= PF_TOK) break;
-            *(u32x4*)(kb + row * KSTRIDE + 16 * lchunk) = kreg[i];
-            *(u32x4*)(vb + row * VSTRIDE + 16 * lchunk) = vreg[i];
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)((const uint8_t*)kc + off + kcol[i]),
+                (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)((const uint8_t*)vc + off + vcol[i]),
+                (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB), 16, 0, 0);
         }
     };
 
-    u32x4 kreg[NI], vreg[NI];
-    load_tile(kreg, vreg, 0);
-    store_tile(kreg, vreg, 0);
-    if (ntiles > 1) load_tile(kreg, vreg, 1);
-
+    // ---- operand read addresses (without the buffer offset)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)pf_smem;
+    const uint32_t krow = lds0 + rho * ROWB;                  // K: row rho (+ 32 rows for the second half)
+    const uint32_t kx = (uint32_t)((16 * h) ^ (16 * ((rho / RPB) & (CPR - 1))));   // chunk 2 j + h, permuted
     const int jj = rho & 15;
-    const int voff = (4 * h + (jj >> 2)) * VSTRIDE + ((rho & 16) + 4 * (jj & 3)) * 2;
+    const int tq = jj >> 2;                                   // token of the quad this lane names
+    const int vkey4 = ((4 * h + tq) / RPB) & (CPR / 4 - 1);
+    const int vchunk = (rho & 16) / 8 + ((jj & 3) >> 1) + 4 * vkey4;   // + 4 db, mod CPR
+    const uint32_t vrow = lds0 + S::KBYTES + (4 * h + tq) * ROWB + (jj & 1) * 8;
+
+    issue_tile(0);
 #pragma unroll 1
     for (int t = 0; t < ntiles; ++t) {
-        // tile t is staged and every wave is done with tile t - 1, whose buffer takes tile t + 1
-        __syncthreads();
-        if (t + 1 < ntiles) store_tile(kreg, vreg, (t + 1) & 1);
-        if (t + 2 < ntiles) load_tile(kreg, vreg, t + 2);    // in flight behind this tile's math
-        const uint8_t* kb = pf_smem + (t & 1) * PfSmem<D>::BUF;
-        const uint8_t* vb = kb + PfSmem<D>::KBYTES;
-#pragma unroll
-        for (int s = 0; s < PF_TOK / 32; ++s) {
-            const int tstart = part_start + t * PF_TOK + 32 * s;
-            if (tstart >= Lw) break;                          // nothing this wave's columns may see (wave-uniform)
-            f32x16 sc;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sc[i] = 0.f;
-#pragma unroll
-            for (int j = 0; j < KS; ++j) {
-                const u32x4 ka = *(const u32x4*)(kb + (32 * s + rho) * KSTRIDE + (16 * j + 8 * h) * 2);
-                sc = T::mfma32(bitcast<vec8>(ka), qreg[j], sc);
-            }
-            float tmax = PA_NEG;
-            if (tstart + 32 <= Lmask) {                       // every token is visible to every column of the wave
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    sc[i] *= scale_log2;
-                    tmax = fmaxf(tmax, sc[i]);
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int tok = tstart + 8 * (i >> 2) + 4 * h + (i & 3);
-                    const float v = tok < Lcol ? sc[i] * scale_log2 : PA_NEG;
-                    sc[i] = v;
-                    tmax = fmaxf(tmax, v);
-                }
-            }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-            const float m_new = fmaxf(m_run, tmax);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            float psum = 0.f;
-            uint32_t pp[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const float p0 = __builtin_amdgcn_exp2f(sc[2 * k] - m_new);
-                const float p1 = __builtin_amdgcn_exp2f(sc[2 * k + 1] - m_new);
-                pp[k] = pack2<T>(p0, p1);
-                // the denominator sums the probabilities as the PV product sees them (rounded to T)
-                psum += T::to_float((uint16_t)(pp[k] & 0xffff)) + T::to_float((uint16_t)(pp[k] >> 16));
-            }
-            // the running maximum rarely moves after the first tiles: when it moved for no lane, alpha is exactly 1
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-                l_run *= alpha;
-#pragma unroll
-                for (int db = 0; db < DB; ++db) acc[db] *= alpha;
-            }
-            l_run += psum;
-            const vec8 pfrag0 = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
-            const vec8 pfrag1 = bitcast<vec8>((u32x4){pp[4], pp[5], pp[6], pp[7]});
+        // tile t has landed for every wave, and every wave is done with tile t - 1, whose buffer takes tile t + 1
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < ntiles) issue_tile(t + 1);               // in flight behind this tile's math
+        const int ts = part_start + t * PF_TOK;
+        if (ts >= Lw) continue;                               // nothing this wave's columns may see (wave-uniform)
+        const uint32_t boff = (t & 1) * S::BUF;
 
-            // ---- O^T += V^T P^T.  Within 16 lanes (d rows rho0 .. rho0+15, token quarter h) lane j names the 4 values
-            // V[token 16 T + 4 h + (j >> 2)][32 db + rho0 + 4 (j & 3) ..] and receives V[token 16 T + 4 h + e][its d
-            // row]; the second read, 8 tokens on, supplies k-values 4 .. 7.
+        // ---- scores of the tile's two 32-token halves (raw).  Read i = 2 j + s: k-step j of half s.
+        f32x16 sc[2];
+        {
+            constexpr int NR = 2 * KS, P = NR < 4 ? NR : 4;
+            u32x4 ka[P];
+            auto rd = [&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int j = i >> 1, s = i & 1;
+                ka[i % P] = pf_lds_read16<32 * s * ROWB>(krow + boff + ((32u * j) ^ kx));
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            pf_static_for<P>(rd);
+            pf_static_for<NR>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int left = NR - 1 - i;              // reads after read i that have been issued
+                pf_wait_lds<(left < P - 1 ? left : P - 1)>();
+                if constexpr (i < 2) {
+                    f32x16 z;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-#pragma unroll
-                for (int th = 0; th < 2; ++th) {
-                    const uint8_t* p0 = vb + (32 * s + 16 * th) * VSTRIDE + voff + 64 * db;
-                    const u32x2 l2 = bitcast<u32x2>(lds_read_tr16(p0));
-                    const u32x2 h2 = bitcast<u32x2>(lds_read_tr16(p0 + 8 * VSTRIDE));
-                    acc[db] = T::mfma32(bitcast<vec8>((u32x4){l2[0], l2[1], h2[0], h2[1]}), th ? pfrag1 : pfrag0,
-                                        acc[db]);
+                    for (int e = 0; e < 16; ++e) z[e] = 0.f;
+                    sc[i & 1] = T::mfma32(bitcast<vec8>(ka[i % P]), qreg[i >> 1], z);
+                } else {
+                    sc[i & 1] = T::mfma32(bitcast<vec8>(ka[i % P]), qreg[i >> 1], sc[i & 1]);
                 }
-            }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (i + P < NR) rd(std::integral_constant<int, i + P>{});
+            });
+        }
+        if (ts + PF_TOK > Lmask) {                            // some token is hidden from some column of the wave
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int tok = ts + 32 * s + 8 * (i >> 2) + 4 * h + (i & 3);
+                    sc[s][i] = tok < Lcol ? sc[s][i] : PA_NEG;
+                }
+        }
+        // one running-maximum update per 64 tokens
+        float tmax = sc[0][0];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sc[s][i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+        m_run = m_new;
+        // the running maximum rarely moves after the first tiles: when it moved for no lane, alpha is exactly 1
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+        }
+        const float nm = -m_new * scale_log2;
+        uint32_t pp[2][8];
+        // probabilities 2 k, 2 k + 1 of half s, rounded to T; the denominator sums them as the PV product sees them
+        auto prob_pair = [&](int s, int k) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[s][2 * k], scale_log2, nm));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[s][2 * k + 1], scale_log2, nm));
+            pp[s][k] = pack2<T>(p0, p1);
+            l_run += T::to_float((uint16_t)(pp[s][k] & 0xffff)) + T::to_float((uint16_t)(pp[s][k] >> 16));
+        };
+#pragma unroll
+        for (int k = 0; k < 8; ++k) prob_pair(0, k);
+
+        // ---- O^T += V^T P^T.  MFMA v = 2 DB s + DB th + db: half s, token half th of it, d block db.  Within 16
+        // lanes (d rows rho0 .. rho0+15, token quarter h) lane j names the 4 values
+        // V[token 32 s + 16 th + 4 h + (j >> 2)][32 db + rho0 + 4 (j & 3) ..] and receives
+        // V[token 32 s + 16 th + 4 h + e][its d row]; the second read, 8 tokens on, supplies k-values 4 .. 7.
+        {
+            constexpr int NV = 4 * DB, P = 4;
+            uint32_t va[DB];
+#pragma unroll
+            for (int db = 0; db < DB; ++db) va[db] = vrow + boff + 16 * ((vchunk + 4 * db) & (CPR - 1));
+            u32x2 lo[P], hi[P];
+            auto rd = [&](auto vc_) {
+                constexpr int v = decltype(vc_)::value;
+                constexpr int s = v / (2 * DB), th = (v / DB) & 1, db = v % DB;
+                lo[v % P] = pf_lds_read_tr<(32 * s + 16 * th) * ROWB>(va[db]);
+                hi[v % P] = pf_lds_read_tr<(32 * s + 16 * th + 8) * ROWB>(va[db]);
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            pf_static_for<P>(rd);
+            pf_static_for<NV>([&](auto vc_) {
+                constexpr int v = decltype(vc_)::value;
+                constexpr int s = v / (2 * DB), th = (v / DB) & 1, db = v % DB;
+                constexpr int left = NV - 1 - v;
+                pf_wait_lds<2 * (left < P - 1 ? left : P - 1)>();
+                const vec8 pf = bitcast<vec8>((u32x4){pp[s][4 * th], pp[s][4 * th + 1], pp[s][4 * th + 2],
+                                                      pp[s][4 * th + 3]});
+                acc[db] = T::mfma32(bitcast<vec8>((u32x4){lo[v % P][0], lo[v % P][1], hi[v % P][0], hi[v % P][1]}),
+                                    pf, acc[db]);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (v + P < NV) rd(std::integral_constant<int, v + P>{});
+                // the second half's exponentials, spread over the first half's MFMAs
+                if constexpr (v < 2 * DB) {
+                    constexpr int per = 8 / (2 * DB);
+#pragma unroll
+                    for (int k = v * per; k < (v + 1) * per; ++k) prob_pair(1, k);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
         }
     }
 
@@ -783,7 +865,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
                 *(f32x4*)(dst + 32 * db + 8 * q4) =
                     (f32x4){acc[db][4 * q4], acc[db][4 * q4 + 1], acc[db][4 * q4 + 2], acc[db][4 * q4 + 3]};
         if (h == 0) {
-            part_ml[pi * 2] = m_run;
+            part_ml[pi * 2] = m_run * scale_log2;
             part_ml[pi * 2 + 1] = l_run;
         }
     }
@@ -1072,6 +1154,7 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
     MF_REQUIRE(out && query && key_cache && value_cache && q_starts, "paged_attention_prefill: null argument");
     const bool contiguous = block_tables == nullptr;
     MF_REQUIRE(contiguous || context_lens, "paged_attention_prefill: block_tables without context_lens");
+    MF_REQUIRE(scale > 0.f, "paged_attention_prefill: the softmax scale must be positive");
     MF_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "paged_attention_prefill: n_heads (%d) must be a positive multiple of n_kv_heads (%d)", n_heads,
                n_kv_heads);
