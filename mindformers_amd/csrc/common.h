@@ -47,6 +47,12 @@ struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // c + both halves of a packed pair, in fp32 (one dot-product instruction)
+    static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_v;
+        const bf16x2_v one = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, pair), one, c, false);
+    }
 };
 
 struct FP16 {
@@ -63,6 +69,11 @@ struct FP16 {
     }
     static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
+        typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_v;
+        const f16x2_v one = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_v, pair), one, c, false);
     }
 };
 

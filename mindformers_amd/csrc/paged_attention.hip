@@ -480,7 +480,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 
 // ---- prefill on the 32x32x16 MFMA ---------------------------------------------------------------------------------
 // Prefill has (query, head) columns in abundance.  A workgroup of 4 waves serves 128 consecutive columns of one kv
-// head (32 per wave) and walks the keys and values of their causal range once, 64 tokens at a time; every wave
+// head (32 per wave) and walks the keys and values of their causal range once, 32 tokens at a time; every wave
 // multiplies its own 32 columns against the shared tile, so each K / V byte is read from L2 once per 128 columns
 // (with one tile stream per wave the kernel was bound by L2 bandwidth).  The 32x32x16 instruction does twice the
 // work of the 16x16x32 one in the same issue time and halves the LDS reads per column.
@@ -489,26 +489,29 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 //   8 T .. 8 T + 7 are, in order, exactly the 8 k-values a lane supplies to the B operand of token half T when that
 //   half's 16 tokens are taken in the order (4 h + e, 8 + 4 h + e); the V^T operand is read in the same order with
 //   the transposing LDS read.
-// Tiles go from global memory straight into LDS (no registers in between), double-buffered with one barrier per tile.
-// Such a load writes 64 consecutive 16-byte slots, so rows cannot be padded; instead the 16-byte chunks of a row are
-// permuted by the address each lane supplies:
+// Tiles go from global memory straight into LDS (no registers in between) through a ring of 4 buffers, two tiles
+// ahead, with one barrier per tile.  Such a load writes 64 consecutive 16-byte slots, so rows cannot be padded;
+// instead the 16-byte chunks of a row are permuted by the address each lane supplies:
 //   K: chunk c of row t sits in slot c ^ key(t): the 16 rows of one chunk that an operand read serves together
 //      land on 16 different slots;
 //   V: chunk c of row t sits in slot (c + 4 key4(t)) mod chunks-per-row: the 4 tokens x 64 bytes a transposing read
 //      serves together land on different slots.
-// The LDS reads are issued by hand a few MFMAs ahead (the compiler would wait for each before the next), and the
-// exponentials of the tile's second half run beside the first half's PV MFMAs.
+// The matrix pipe and the vector ALU work side by side inside a wave: in step t the score MFMAs of tile t are
+// interleaved with the exponentials of tile t - 1, and the PV MFMAs of tile t - 1 with the running-maximum update of
+// tile t.  The LDS reads are issued by hand a few MFMAs ahead and the order of the step is pinned with scheduling
+// barriers (the compiler would otherwise wait for each read and serialise the two pipes).
 // A wave owns its columns over the whole partition, so there is no merge: it writes final rows (single partition) or
 // fp32 partials for the reduce kernel.
 constexpr int PF_COLS = 128;                                  // columns per workgroup
-constexpr int PF_TOK = 64;                                    // tokens per staged tile
+constexpr int PF_TOK = 32;                                    // tokens per staged tile
+constexpr int PF_RING = 4;                                    // staged tiles
 
 template <int D>
 struct PfSmem {
     static constexpr int ROWB = D * 2;                        // bytes per staged row
     static constexpr int KBYTES = PF_TOK * ROWB;
     static constexpr int BUF = 2 * KBYTES;                    // K tile, then V tile
-    static constexpr int BYTES = 2 * BUF;
+    static constexpr int BYTES = PF_RING * BUF;
 };
 
 template <int OFF>
@@ -530,6 +533,13 @@ __device__ __forceinline__ void pf_wait_lds() {
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
     __builtin_amdgcn_sched_barrier(0);
 }
+// maximum of a value over the two lanes l and l ^ 32 (the instruction swaps the upper half of its first operand with
+// the lower half of its second)
+__device__ __forceinline__ float pf_max_xor32(float v) {
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
 template <typename F, int... I>
 __device__ __forceinline__ void pf_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
     (f(std::integral_constant<int, I>{}), ...);
@@ -550,11 +560,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     using S = PfSmem<D>;
     constexpr int KS = D / 16;                                // k-steps of the score product
     constexpr int DB = D / 32;                                // 32-row blocks of O^T
+    constexpr int NV = 2 * DB;                                // PV MFMAs per tile
     constexpr int ROWB = S::ROWB;
     constexpr int CPR = ROWB / 16;                            // 16-byte chunks per row
     constexpr int RPB = 16 / CPR;                             // rows per 256 bytes of LDS
     constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
-    constexpr int NI = PF_TOK / RPI / PA_WAVES;               // loads per wave per tile per tensor
+    constexpr int LOADS = PF_TOK / RPI;                       // wave-wide loads per tile per tensor
+    constexpr int LW = LOADS < PA_WAVES ? LOADS : PA_WAVES;   // waves that load
+    constexpr int NI = LOADS / LW;                            // loads per loading wave per tile per tensor
 
     extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];
 
@@ -631,7 +644,8 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     const bool col_ok = qi < q_len;
     const int Lcol = col_ok ? ctx_before + qi + 1 : 0;        // causal limit of this lane's column
     const int q_first = c0 / n_rep;                           // first query of the wave
-    const int Lw = q_first < q_len ? ctx_before + min(q_len, (c0 + 31) / n_rep + 1) : 0;   // farthest token of the wave
+    // a wave none of whose columns sees a token of this partition only helps with the loads
+    const bool wave_live = q_first < q_len && ctx_before + min(q_len, (c0 + 31) / n_rep + 1) > part_start;
     const int Lmask = ctx_before + q_first + 1;               // tiles that end at or before it need no mask
     vec8 qreg[KS];
     {
@@ -650,34 +664,34 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-    // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
-    // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0.  Maxima are kept in raw score units: the
-    // (positive) softmax scale is applied inside the exponent.
-    float m_run = 0.5f * PA_NEG, l_run = 0.f;
 
     const bool contiguous = block_tables == nullptr;
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
     const int64_t row_bytes = kv_stride * 2;
 
-    // ---- tile loads: load i of wave w brings rows (4 i + w) RPI .. + RPI - 1; lane = (row in the group, LDS slot)
+    // ---- tile loads: load i of wave w brings rows (LW i + w) RPI .. + RPI - 1; lane = (row in the group, LDS slot)
     const int lrow = lane / CPR;
     const int lslot = lane - lrow * CPR;
-    uint32_t kcol[NI], vcol[NI];                              // byte offset of this lane's chunk within a row
+    uint32_t kcol[NI], vcol[NI];                              // byte offset of this lane's chunk within a token row
+    uint32_t kofs[NI], vofs[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int row = (PA_WAVES * i + w) * RPI + lrow;
+        const int row = (LW * i + w) * RPI + lrow;
         const int key = (row / RPB) & (CPR - 1);
         const int key4 = (row / RPB) & (CPR / 4 - 1);
         kcol[i] = (uint32_t)(kvh * D * 2 + 16 * (lslot ^ key));
         vcol[i] = (uint32_t)(kvh * D * 2 + 16 * ((lslot - 4 * key4) & (CPR - 1)));
+        kofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + kcol[i];      // offsets within a whole tile
+        vofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + vcol[i];
     }
     const int part_end = min(Lwg, part_start + part_tokens);
     const int ntiles = (part_end - part_start + PF_TOK - 1) / PF_TOK;
 
     // rows past the group's range re-read its last row (their scores are masked)
     auto issue_tile = [&](int t) {
+        if (LW < PA_WAVES && w >= LW) return;
         const int ts = part_start + t * PF_TOK;
-        uint8_t* kdst = pf_smem + (t & 1) * S::BUF;
+        uint8_t* kdst = pf_smem + (t & (PF_RING - 1)) * S::BUF;
         int64_t slot0 = 0;
         if constexpr (TIB) {                                  // the tile lies inside one block: one uniform lookup
             if (contiguous) {
@@ -690,154 +704,255 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
             }
         }
         const int last_row = Lwg - 1 - ts;
+        if (TIB && last_row >= PF_TOK - 1) {                  // whole tile inside one block: constant lane offsets
+            const uint8_t* kb = (const uint8_t*)kc + slot0 * row_bytes;
+            const uint8_t* vb = (const uint8_t*)vc + slot0 * row_bytes;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int r0 = (LW * i + w) * RPI;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb + kofs[i]),
+                                                 (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(vb + vofs[i]),
+                    (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB), 16, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int r0 = (PA_WAVES * i + w) * RPI;
+            const int r0 = (LW * i + w) * RPI;
             const int rc = min(r0 + lrow, last_row);
-            int64_t off;
-            if constexpr (TIB) {
-                off = (slot0 + rc) * row_bytes;
+            const uint8_t *kp, *vp;
+            if constexpr (TIB) {                              // uniform base, 32-bit lane offset
+                const uint32_t lo = (uint32_t)(rc * (int)row_bytes);
+                kp = (const uint8_t*)kc + slot0 * row_bytes + (lo + kcol[i]);
+                vp = (const uint8_t*)vc + slot0 * row_bytes + (lo + vcol[i]);
             } else {
                 const int tok = ts + rc;
                 const int bi = tok / block_size;
                 int blk = table[bi];
                 blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
-                off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_bytes;
+                const int64_t off = ((int64_t)blk * block_size + (tok - bi * block_size)) * row_bytes;
+                kp = (const uint8_t*)kc + off + kcol[i];
+                vp = (const uint8_t*)vc + off + vcol[i];
             }
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)((const uint8_t*)kc + off + kcol[i]),
-                (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)((const uint8_t*)vc + off + vcol[i]),
-                (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
+                                             (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
+                                             (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB),
+                                             16, 0, 0);
         }
     };
 
-    // ---- operand read addresses (without the buffer offset)
+    // ---- operand read addresses within a ring buffer (the buffer is a compile-time offset of the read)
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)pf_smem;
-    const uint32_t krow = lds0 + rho * ROWB;                  // K: row rho (+ 32 rows for the second half)
     const uint32_t kx = (uint32_t)((16 * h) ^ (16 * ((rho / RPB) & (CPR - 1))));   // chunk 2 j + h, permuted
+    uint32_t klane[KS];                                       // K: row rho, chunk of k-step j
+#pragma unroll
+    for (int j = 0; j < KS; ++j) klane[j] = lds0 + rho * ROWB + ((32u * j) ^ kx);
     const int jj = rho & 15;
     const int tq = jj >> 2;                                   // token of the quad this lane names
     const int vkey4 = ((4 * h + tq) / RPB) & (CPR / 4 - 1);
     const int vchunk = (rho & 16) / 8 + ((jj & 3) >> 1) + 4 * vkey4;   // + 4 db, mod CPR
     const uint32_t vrow = lds0 + S::KBYTES + (4 * h + tq) * ROWB + (jj & 1) * 8;
+    uint32_t vlane[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) vlane[db] = vrow + 16 * ((vchunk + 4 * db) & (CPR - 1));
 
-    issue_tile(0);
-#pragma unroll 1
-    for (int t = 0; t < ntiles; ++t) {
-        // tile t has landed for every wave, and every wave is done with tile t - 1, whose buffer takes tile t + 1
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < ntiles) issue_tile(t + 1);               // in flight behind this tile's math
+    // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
+    // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0.  Maxima are kept in raw score units: the
+    // (positive) softmax scale is applied inside the exponent.
+    float m_run = 0.5f * PA_NEG, l_run = 0.f;
+    float alpha = 1.f, nm = 0.f;                              // of the tile whose scores wait for their exponentials
+    f32x16 sc_a, sc_b;
+
+    // One step: scores of tile t into `cur` (CUR) beside the exponentials of tile t - 1 from `prev` (PREV), then the
+    // PV product of tile t - 1 beside the running-maximum update of tile t.
+    // Tile t lives in ring buffer R = t mod 4 (a compile-time constant of the step), tile t - 1 in buffer R - 1.
+    auto step = [&](int t, auto ring_c, f32x16& cur, f32x16& prev, auto cur_c, auto prev_c) {
+        constexpr bool CUR = decltype(cur_c)::value, PREV = decltype(prev_c)::value;
+        constexpr int R = decltype(ring_c)::value;
+        constexpr int NQ = CUR ? KS : 0, NP = PREV ? NV : 0, NT = NQ + NP, P = 4;
+        constexpr int KOFF = R * S::BUF, VOFF = ((R + PF_RING - 1) % PF_RING) * S::BUF;
         const int ts = part_start + t * PF_TOK;
-        if (ts >= Lw) continue;                               // nothing this wave's columns may see (wave-uniform)
-        const uint32_t boff = (t & 1) * S::BUF;
-
-        // ---- scores of the tile's two 32-token halves (raw).  Read i = 2 j + s: k-step j of half s.
-        f32x16 sc[2];
-        {
-            constexpr int NR = 2 * KS, P = NR < 4 ? NR : 4;
-            u32x4 ka[P];
-            auto rd = [&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                constexpr int j = i >> 1, s = i & 1;
-                ka[i % P] = pf_lds_read16<32 * s * ROWB>(krow + boff + ((32u * j) ^ kx));
-            };
-            __builtin_amdgcn_sched_barrier(0);
-            pf_static_for<P>(rd);
-            pf_static_for<NR>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                constexpr int left = NR - 1 - i;              // reads after read i that have been issued
-                pf_wait_lds<(left < P - 1 ? left : P - 1)>();
-                if constexpr (i < 2) {
+        u32x4 ka[P];
+        u32x2 lo[P], hi[P];
+        uint32_t pp[8];
+        // operand fetch m: K operand of k-step m, or (after the NQ score MFMAs) the V operand of PV MFMA m - NQ =
+        // DB th + db (token half th, d block db), two transposing reads
+        auto fetch = [&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            if constexpr (m < NQ) {
+                ka[m % P] = pf_lds_read16<KOFF>(klane[m]);
+            } else if constexpr (m < NT) {
+                constexpr int v = m - NQ, th = v / DB, db = v % DB;
+                lo[m % P] = pf_lds_read_tr<VOFF + 16 * th * ROWB>(vlane[db]);
+                hi[m % P] = pf_lds_read_tr<VOFF + (16 * th + 8) * ROWB>(vlane[db]);
+            }
+        };
+        // probabilities 2 k, 2 k + 1 of the previous tile, rounded to T; the denominator sums them as the PV product
+        // sees them
+        auto prob_pair = [&](int k) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(prev[2 * k], scale_log2, nm));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(prev[2 * k + 1], scale_log2, nm));
+            pp[k] = pack2<T>(p0, p1);
+            l_run = T::sum2(pp[k], l_run);
+            asm volatile("" : "+v"(pp[k]), "+v"(l_run));    // computed here, not where it is first used
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        pf_static_for<(P < NT ? P : NT)>(fetch);
+        if constexpr (PREV) l_run *= alpha;
+        if constexpr (PREV && !CUR) {                         // last tile: no score MFMAs to work beside
+#pragma unroll
+            for (int k = 0; k < 8; ++k) prob_pair(k);
+        }
+        float tmax = PA_NEG, m_new = 0.f;
+        pf_static_for<NT>([&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            // LDS reads issued after those of fetch m
+            constexpr int last = (m + P < NT ? m + P : NT) - 1;
+            constexpr int k_after = (last < NQ ? last : NQ - 1) - (m < NQ ? m : NQ - 1);
+            constexpr int v_after = (last >= NQ ? last - NQ + 1 : 0) - (m >= NQ ? m - NQ + 1 : 0);
+            if constexpr (PREV && m == NQ) {
+                // between the two halves of the step: the accumulators move to the previous tile's maximum (which
+                // rarely changes after the first tiles: alpha is then exactly 1 in every lane) ...
+                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (CUR && m == NQ) {
+                // ... and tokens hidden from a column leave its scores
+                if (ts + PF_TOK > Lmask) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
+                        cur[i] = tok < Lcol ? cur[i] : PA_NEG;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            pf_wait_lds<k_after + 2 * v_after>();
+            if constexpr (m < NQ) {
+                if constexpr (m == 0) {
                     f32x16 z;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) z[e] = 0.f;
-                    sc[i & 1] = T::mfma32(bitcast<vec8>(ka[i % P]), qreg[i >> 1], z);
+                    cur = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], z);
                 } else {
-                    sc[i & 1] = T::mfma32(bitcast<vec8>(ka[i % P]), qreg[i >> 1], sc[i & 1]);
+                    cur = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], cur);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (i + P < NR) rd(std::integral_constant<int, i + P>{});
-            });
-        }
-        if (ts + PF_TOK > Lmask) {                            // some token is hidden from some column of the wave
+            } else {
+                constexpr int v = m - NQ, th = v / DB, db = v % DB;
+                const vec8 pf = bitcast<vec8>((u32x4){pp[4 * th], pp[4 * th + 1], pp[4 * th + 2], pp[4 * th + 3]});
+                acc[db] = T::mfma32(bitcast<vec8>((u32x4){lo[m % P][0], lo[m % P][1], hi[m % P][0], hi[m % P][1]}),
+                                    pf, acc[db]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(std::integral_constant<int, m + P>{});
+            if constexpr (PREV && m < NQ) {                   // exponentials of tile t - 1 beside the score MFMAs
+                constexpr int per = 8 / KS;
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
+                for (int k = m * per; k < (m + 1) * per; ++k) prob_pair(k);
+            }
+            if constexpr (CUR && m >= NQ) {                   // running maximum of tile t beside the PV MFMAs
+                constexpr int v = m - NQ;
+                constexpr int c_lo = v * 4 / NV, c_hi = (v + 1) * 4 / NV;
+#pragma unroll
+                for (int c = c_lo; c < c_hi; ++c) {
+                    if (c == 0) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) tmax = fmaxf(tmax, cur[i]);
+                    } else if (c == 1) {
+#pragma unroll
+                        for (int i = 8; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
+                        tmax = pf_max_xor32(tmax);
+                    } else if (c == 2) {
+                        m_new = fmaxf(m_run, tmax);
+                        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+                    } else {
+                        m_run = m_new;
+                        nm = -m_new * scale_log2;
+                    }
+                    asm volatile("" : "+v"(tmax), "+v"(m_new), "+v"(alpha), "+v"(nm));   // computed here
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (PREV && !CUR) return;
+        if constexpr (CUR && !PREV) {
+            // first tile: no PV product to work beside
+            if (ts + PF_TOK > Lmask) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int tok = ts + 32 * s + 8 * (i >> 2) + 4 * h + (i & 3);
-                    sc[s][i] = tok < Lcol ? sc[s][i] : PA_NEG;
+                    const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
+                    cur[i] = tok < Lcol ? cur[i] : PA_NEG;
                 }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
+            tmax = pf_max_xor32(tmax);
+            m_new = fmaxf(m_run, tmax);
+            alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+            m_run = m_new;
+            nm = -m_new * scale_log2;
         }
-        // one running-maximum update per 64 tokens
-        float tmax = sc[0][0];
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sc[s][i]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax);
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
-        m_run = m_new;
-        // the running maximum rarely moves after the first tiles: when it moved for no lane, alpha is exactly 1
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-            l_run *= alpha;
-#pragma unroll
-            for (int db = 0; db < DB; ++db) acc[db] *= alpha;
-        }
-        const float nm = -m_new * scale_log2;
-        uint32_t pp[2][8];
-        // probabilities 2 k, 2 k + 1 of half s, rounded to T; the denominator sums them as the PV product sees them
-        auto prob_pair = [&](int s, int k) {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[s][2 * k], scale_log2, nm));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[s][2 * k + 1], scale_log2, nm));
-            pp[s][k] = pack2<T>(p0, p1);
-            l_run += T::to_float((uint16_t)(pp[s][k] & 0xffff)) + T::to_float((uint16_t)(pp[s][k] >> 16));
-        };
-#pragma unroll
-        for (int k = 0; k < 8; ++k) prob_pair(0, k);
+    };
 
-        // ---- O^T += V^T P^T.  MFMA v = 2 DB s + DB th + db: half s, token half th of it, d block db.  Within 16
-        // lanes (d rows rho0 .. rho0+15, token quarter h) lane j names the 4 values
-        // V[token 32 s + 16 th + 4 h + (j >> 2)][32 db + rho0 + 4 (j & 3) ..] and receives
-        // V[token 32 s + 16 th + 4 h + e][its d row]; the second read, 8 tokens on, supplies k-values 4 .. 7.
-        {
-            constexpr int NV = 4 * DB, P = 4;
-            uint32_t va[DB];
+    issue_tile(0);
+    if (ntiles > 1) issue_tile(1);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) va[db] = vrow + boff + 16 * ((vchunk + 4 * db) & (CPR - 1));
-            u32x2 lo[P], hi[P];
-            auto rd = [&](auto vc_) {
-                constexpr int v = decltype(vc_)::value;
-                constexpr int s = v / (2 * DB), th = (v / DB) & 1, db = v % DB;
-                lo[v % P] = pf_lds_read_tr<(32 * s + 16 * th) * ROWB>(va[db]);
-                hi[v % P] = pf_lds_read_tr<(32 * s + 16 * th + 8) * ROWB>(va[db]);
-            };
-            __builtin_amdgcn_sched_barrier(0);
-            pf_static_for<P>(rd);
-            pf_static_for<NV>([&](auto vc_) {
-                constexpr int v = decltype(vc_)::value;
-                constexpr int s = v / (2 * DB), th = (v / DB) & 1, db = v % DB;
-                constexpr int left = NV - 1 - v;
-                pf_wait_lds<2 * (left < P - 1 ? left : P - 1)>();
-                const vec8 pf = bitcast<vec8>((u32x4){pp[s][4 * th], pp[s][4 * th + 1], pp[s][4 * th + 2],
-                                                      pp[s][4 * th + 3]});
-                acc[db] = T::mfma32(bitcast<vec8>((u32x4){lo[v % P][0], lo[v % P][1], hi[v % P][0], hi[v % P][1]}),
-                                    pf, acc[db]);
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (v + P < NV) rd(std::integral_constant<int, v + P>{});
-                // the second half's exponentials, spread over the first half's MFMAs
-                if constexpr (v < 2 * DB) {
-                    constexpr int per = 8 / (2 * DB);
-#pragma unroll
-                    for (int k = v * per; k < (v + 1) * per; ++k) prob_pair(1, k);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            });
+    for (int j = 0; j < KS; ++j) asm volatile("" : "+v"(qreg[j]));   // the query is complete before the loop
+    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 2,
+    // whose buffer takes tile t + 2
+    auto sync_issue = [&](int t) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NI) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 2 < ntiles) issue_tile(t + 2);
+    };
+    constexpr std::true_type yes{};
+    constexpr std::false_type no{};
+    constexpr std::integral_constant<int, 0> r0{};
+    constexpr std::integral_constant<int, 1> r1{};
+    constexpr std::integral_constant<int, 2> r2{};
+    constexpr std::integral_constant<int, 3> r3{};
+    // the scores alternate between two register sets: even tiles in sc_a, odd tiles in sc_b
+    sync_issue(0);
+    if (wave_live) step(0, r0, sc_a, sc_b, yes, no);
+    int t = 1;
+#pragma unroll 1
+    for (; t + 3 < ntiles; t += 4) {
+        sync_issue(t);
+        if (wave_live) step(t, r1, sc_b, sc_a, yes, yes);
+        sync_issue(t + 1);
+        if (wave_live) step(t + 1, r2, sc_a, sc_b, yes, yes);
+        sync_issue(t + 2);
+        if (wave_live) step(t + 2, r3, sc_b, sc_a, yes, yes);
+        sync_issue(t + 3);
+        if (wave_live) step(t + 3, r0, sc_a, sc_b, yes, yes);
+    }
+    if (t < ntiles) {
+        sync_issue(t);
+        if (wave_live) step(t, r1, sc_b, sc_a, yes, yes);
+        if (++t < ntiles) {
+            sync_issue(t);
+            if (wave_live) step(t, r2, sc_a, sc_b, yes, yes);
+            if (++t < ntiles) {
+                sync_issue(t);
+                if (wave_live) step(t, r3, sc_b, sc_a, yes, yes);
+            }
+        }
+    }
+    if (wave_live) {                                          // exponentials and PV product of the last tile
+        switch (ntiles & 3) {
+            case 0: step(ntiles, r0, sc_a, sc_b, no, yes); break;
+            case 1: step(ntiles, r1, sc_b, sc_a, no, yes); break;
+            case 2: step(ntiles, r2, sc_a, sc_b, no, yes); break;
+            default: step(ntiles, r3, sc_b, sc_a, no, yes); break;
         }
     }
 

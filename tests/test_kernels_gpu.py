@@ -245,6 +245,9 @@ def _prefill_case(rng, dtype, nh, nkv, d, bs, lens, q_lens, max_blocks=None, pad
     (torch.float16, 2, 2, 32, 16, [50, 1], [50, 1]),                        # MHA
     (torch.bfloat16, 4, 1, 128, 24, [200, 77], [31, 77]),                   # block size not a multiple of 32
     (torch.bfloat16, 32, 8, 128, 128, [2100], [3]),                         # few queries, long context: partitions
+    (torch.float16, 4, 4, 64, 32, [300], [300]),                            # MHA: 128 queries per workgroup
+    (torch.float16, 16, 4, 128, 64, [1500, 33], [1500, 20]),                # many tiles per workgroup, fp16
+    (torch.bfloat16, 8, 8, 128, 16, [200], [130]),                          # MHA behind a context, small blocks
 ])
 def test_paged_prefill_vs_oracle(dtype, nh, nkv, d, bs, lens, q_lens):
     rng = np.random.default_rng(nh * 100 + len(lens))
