@@ -1144,7 +1144,7 @@ __global__ void pa_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t* 
 // ---- prefill --------------------------------------------------------------------------------------------------
 // Partitioning rule shared by the workspace query and the launch.  A workgroup serves 128 (query, head) columns of
 // one kv head (16 with an int8 cache); when the query rows alone give the chip enough workgroups one partition spans the
-// whole context and no partials are written, otherwise the context is cut so that about a thousand workgroups exist.
+// whole context and no partials are written, otherwise the context is cut so that at least 512 workgroups exist.
 struct PfPlan {
     int part_tokens;
     int max_parts;
@@ -1157,7 +1157,7 @@ static inline PfPlan pf_plan(int batch, int64_t total_q, int n_heads, int n_kv, 
     p.col_groups16 = (total_q * n_rep + 15) / 16 + batch;     // each sequence rounds its own columns up
     p.col_groups128 = (total_q * n_rep + PF_COLS - 1) / PF_COLS + batch;
     const int64_t wgs = std::max<int64_t>(1, (total_q * n_rep + PF_COLS - 1) / PF_COLS) * n_kv;
-    int64_t want = (1024 + wgs - 1) / wgs;
+    int64_t want = (512 + wgs - 1) / wgs;                     // 2 workgroups per CU are resident at a time
     const int64_t most = std::max<int64_t>(1, (max_ctx + 255) / 256);
     want = std::min(want, most);
     int64_t pt = (max_ctx + want - 1) / want;
