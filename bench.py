@@ -278,7 +278,7 @@ def bench_prefill_attention(args, torch, ops):
         "config": {"workload": f"{args.workload}: causal attention over the paged cache, {len(lens)} sequences, "
                                f"{int(q_lens[0])} new tokens each, context {int(lens[0])}, 32q/8kv heads x 128, block 128",
                    "launch": "eager", "flops_per_step": flops},
-        "roofline": dict(bound="mfma", kernel="paged_attention_kernel<PF> (+ partition reduce when partitioned)",
+        "roofline": dict(bound="mfma", kernel="prefill_attention_kernel (+ partition reduce when partitioned)",
                          achieved=round(ach, 1), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4), traffic=None,
                          flops_per_launch=flops, avg_launch_us=round(us, 2)),
     }
