@@ -5,6 +5,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <utility>
+#include <type_traits>
 
 #include "../../include/mf_decode.h"
 
@@ -47,6 +49,11 @@ struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // the same with the accumulator held in the accumulation registers (the compiler is not told that this is a
+    // matrix instruction: a reader of c other than the next such statement has to wait for its 16 passes itself)
+    static __device__ __forceinline__ void mfma32_acc(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
     // c + both halves of a packed pair, in fp32 (one dot-product instruction)
     static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
         typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_v;
@@ -69,6 +76,9 @@ struct FP16 {
     }
     static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mfma32_acc(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
         typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_v;
@@ -190,3 +200,42 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 __device__ __forceinline__ s16x4 lds_read_tr16(const uint8_t* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
 }
+
+// ---- pieces of hand-scheduled inner loops: LDS reads issued as asm statements (the compiler neither moves them nor
+// waits for them), the counted wait that makes the oldest of them valid, and a compile-time loop whose index can
+// select immediate offsets
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read16_at(uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_read_tr16_at(uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
+    u32x2 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void wait_lds_reads() {
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+// maximum of a value over the two lanes l and l ^ 32 (the instruction swaps the upper half of its first operand with
+// the lower half of its second)
+__device__ __forceinline__ float max_xor32(float v) {
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+

@@ -7,42 +7,54 @@
 // HBM: 2 * (576 + 512) flops per (token, head) against 1152 bytes per token.
 //
 // Work decomposition
-//   One workgroup of 8 wavefronts owns one token partition of one sequence and a block of 64 heads.  The cache
-//   tile of 32 tokens (36 KB) is fetched once per workgroup with coalesced 16-byte loads, double-buffered in
-//   LDS, and shared by all 8 waves: wave w serves heads 16 * (w & 3) .. + 15 and the value columns
-//   256 * (w >> 2) .. + 255.  Both waves of a head group compute the scores (they need them for their own half
-//   of the output); the PV product, which holds the accumulators, is split between them.
-//   S^T[token, head] = C[token, :576] . Q[head, :576]     18 k-steps of mfma_f32_16x16x32 per 16-token sub-tile
+//   One workgroup of 4 wavefronts, one per SIMD, owns one token partition of one sequence and a block of 128 heads:
+//   wave w serves heads 32 w .. + 31 and all 512 value columns.  The cache tile of 32 tokens (36 KB) is fetched once
+//   per workgroup and shared by the 4 waves.
+//   S^T[token, head] = C[token, :576] . Q[head, :576]     36 k-steps of mfma_f32_32x32x16
 //   online softmax in fp32 (exp2 domain), probabilities rounded to the cache dtype
 //   O^T[d, head] += C^T[d, token] . P^T[token, head]       the tile is read back through the transposing LDS read
-//                                                          (as in the GQA decode kernel)
-//   No merge inside the workgroup is needed: every wave owns its (heads, columns).  Partitions of a sequence
-//   are combined by the partition-reduce kernel of the GQA path.
+//   No merge inside the workgroup is needed: every wave owns its heads.  Partitions of a sequence are combined by
+//   mla_reduce_kernel.
 #include "common.h"
 
 namespace {
 
 constexpr int MLA_DK = 576;                                   // key width: latent + rotary
 constexpr int MLA_DV = 512;                                   // value width: the latent
-constexpr int MLA_WAVES = 8;
-constexpr int MLA_THREADS = MLA_WAVES * 64;
-constexpr int MLA_HEADS = 64;                                 // heads per workgroup
 constexpr int MLA_TILE = 32;                                  // tokens per tile
-// bytes per staged row: +32 makes the row stride an even, non-multiple-of-4 number of 16-byte slots, which keeps
-// both the 16-byte operand reads (served 16 lanes at a time: rows 0-3, 12-15 of one k-chunk with rows 4-11 of the
-// next) and the transposed 4-byte reads free of bank conflicts
-constexpr int MLA_STRIDE = MLA_DK * 2 + 32;
-constexpr int MLA_TILE_BYTES = MLA_TILE * MLA_STRIDE;
-constexpr int MLA_SMEM = 2 * MLA_TILE_BYTES;
 constexpr int MLA_CPR = MLA_DK * 2 / 16;                      // 16-byte chunks per row
-constexpr int MLA_CHUNKS = MLA_TILE * MLA_CPR;
-constexpr int MLA_LD = (MLA_CHUNKS + MLA_THREADS - 1) / MLA_THREADS;      // loads per thread per tile
-constexpr int MLA_KS = MLA_DK / 32;                           // k-steps of the score product
-constexpr int MLA_DB = MLA_DV / 2 / 16;                       // 16-column blocks of one wave's half of the output
 constexpr float MLA_NEG = -1.0e30f;
 
+// A wave holds 16 accumulator blocks of 32 x 32 (256 registers per lane) in the accumulation registers and its 32
+// query rows (144 registers) in the ordinary ones: one wave per SIMD has 512 registers.  No wave computes a score
+// twice, and a cache tile is fetched once per 128 heads.  Tiles of 32 tokens (36 KB) go from global memory straight
+// into a ring of four LDS buffers, two tiles ahead, one barrier per tile.  Such a load writes 64 consecutive 16-byte
+// slots, so the 1152-byte rows cannot be padded; the chunks of a row are permuted within aligned groups of 8 through
+// the global address each lane supplies: chunk c of row t sits in slot (c & ~7) | ((c & 7) ^ s(t)),
+// s(t) = 4 (t/2 & 1) + (t/4 & 3).  Rows are 72 slots apart (8 mod 16), so the 16 rows of one chunk that an operand
+// read serves together, and the 4 tokens x 64 bytes that a transposing read serves together, both fall on 16
+// different 16-byte bank groups.
+// The reference point of the exponentials follows the running maximum lazily: it moves only when the maximum exceeds
+// it by more than 2^8 in probability, because moving it means rescaling 256 accumulator registers per lane;
+// probabilities then lie in (0, 256], which bf16 and fp16 hold with the same relative precision, and the result
+// does not depend on the reference point.
+constexpr int M2_WAVES = 4;
+constexpr int M2_HEADS = 32 * M2_WAVES;                       // heads per workgroup
+constexpr int M2_ROWB = MLA_DK * 2;                           // bytes per staged row
+constexpr int M2_TILE_BYTES = MLA_TILE * M2_ROWB;
+constexpr int M2_RING = 4;
+constexpr int M2_SMEM = M2_RING * M2_TILE_BYTES;
+constexpr int M2_LOADS = M2_TILE_BYTES / 1024 / M2_WAVES;     // wave-wide 1 KB loads per wave per tile
+constexpr int M2_KS = MLA_DK / 16;                            // k-steps of the score product
+constexpr int M2_DB = MLA_DV / 32;                            // 32-column blocks of the output
+constexpr int M2_NV = 2 * M2_DB;                              // PV MFMAs per tile
+constexpr float M2_LAZY = 8.0f;                               // log2 of the largest probability before the reference moves
+static_assert(M2_TILE_BYTES % (1024 * M2_WAVES) == 0 && M2_SMEM <= 160 * 1024, "tile loads / LDS capacity");
+
+__device__ __forceinline__ int m2_key(int row) { return 4 * ((row >> 1) & 1) + ((row >> 2) & 3); }
+
 template <typename T>
-__global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
+__global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ ctx_lens, int n_heads, int head_blocks, int block_size, int max_blocks,
@@ -89,167 +101,264 @@ __global__ __launch_bounds__(MLA_THREADS) void mla_decode_kernel(
     L = __builtin_amdgcn_readfirstlane(L);
 
     const int tid = threadIdx.x;
-    const int w = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
-    const int hgw = w & 3, vhalf = w >> 2;
-    const int head = hb * MLA_HEADS + hgw * 16 + r;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int rho = lane & 31, h = lane >> 5;
+    const int head = hb * M2_HEADS + w * 32 + rho;
     const bool head_ok = head < n_heads;
 
-    // ---- Q as MFMA B operand: lane (r, g) holds Q[head r][32 j + 8 g .. + 8]
-    vec8 qreg[MLA_KS];
+    // ---- Q as MFMA B operand: lane (rho, h) holds Q[head rho][16 j + 8 h .. + 8]
+    vec8 qreg[M2_KS];
     {
-        const uint16_t* qp = q + (int64_t)b * q_stride + (int64_t)(head_ok ? head : 0) * MLA_DK + 8 * g;
+        const uint16_t* qp = q + (int64_t)b * q_stride + (int64_t)(head_ok ? head : 0) * MLA_DK + 8 * h;
 #pragma unroll
-        for (int j = 0; j < MLA_KS; ++j) {
+        for (int j = 0; j < M2_KS; ++j) {
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (head_ok) v = *(const u32x4*)(qp + 32 * j);
+            if (head_ok) v = *(const u32x4*)(qp + 16 * j);
             qreg[j] = bitcast<vec8>(v);
         }
     }
 
     const int part_start = part * part_tokens;
     const int part_end = min(L, part_start + part_tokens);
-    const int ntiles = (part_end - part_start + MLA_TILE - 1) / MLA_TILE;
+    const int ntiles = (part_end - part_start + MLA_TILE - 1) / MLA_TILE;      // >= 1 for a listed partition
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
 
-    // cooperative tile load: chunk c = row * 72 + col; rows past the context re-read the last valid row
-    int lrow[MLA_LD], lcol[MLA_LD];
+    // ---- tile loads: load i of wave w fills LDS slots 64 (4 i + w) .. + 63 of the tile; slot = 72 row + position
+    uint32_t lofs[M2_LOADS];                                  // byte offset of the lane's chunk within a whole tile
+    int lrow[M2_LOADS], lcol[M2_LOADS];
 #pragma unroll
-    for (int k = 0; k < MLA_LD; ++k) {
-        const int c = tid + k * MLA_THREADS;
-        lrow[k] = c / MLA_CPR;
-        lcol[k] = c - lrow[k] * MLA_CPR;
+    for (int i = 0; i < M2_LOADS; ++i) {
+        const int slot = 64 * (M2_WAVES * i + w) + lane;
+        lrow[i] = slot / MLA_CPR;
+        const int pos = slot - lrow[i] * MLA_CPR;
+        lcol[i] = 16 * ((pos & ~7) | ((pos & 7) ^ m2_key(lrow[i])));          // logical chunk of that position
+        lofs[i] = (uint32_t)(lrow[i] * M2_ROWB + lcol[i]);
     }
-    u32x4 lreg[MLA_LD];
-    auto load_tile = [&](int tstart) {                        // a tile lies inside one block (host-checked)
-        const int bi = tstart / block_size;
+    auto issue_tile = [&](int t) {                            // a tile lies inside one block (host-checked)
+        const int ts = part_start + t * MLA_TILE;
+        const int bi = ts / block_size;
         int blk = table[bi];
         blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;       // never leave the cache allocation
-        const int64_t slot0 = (int64_t)blk * block_size + (tstart - bi * block_size);
-        const uint16_t* base = cache + slot0 * MLA_DK;
-        const int last_row = min(MLA_TILE, L - tstart) - 1;
+        const uint8_t* base = (const uint8_t*)cache + ((int64_t)blk * block_size + (ts - bi * block_size)) * M2_ROWB;
+        uint8_t* dst = mla_smem + (t & (M2_RING - 1)) * M2_TILE_BYTES;
+        const int last_row = L - 1 - ts;                      // rows past the context re-read the last valid row
 #pragma unroll
-        for (int k = 0; k < MLA_LD; ++k)
-            if (k + 1 < MLA_LD || tid + k * MLA_THREADS < MLA_CHUNKS)
-                lreg[k] = *(const u32x4*)(base + (int64_t)min(lrow[k], last_row) * MLA_DK + 8 * lcol[k]);
-    };
-    auto store_tile = [&](uint8_t* buf) {
-#pragma unroll
-        for (int k = 0; k < MLA_LD; ++k)
-            if (k + 1 < MLA_LD || tid + k * MLA_THREADS < MLA_CHUNKS)
-                *(u32x4*)(buf + lrow[k] * MLA_STRIDE + 16 * lcol[k]) = lreg[k];
+        for (int i = 0; i < M2_LOADS; ++i) {
+            const uint32_t off = last_row >= MLA_TILE - 1 ? lofs[i]
+                                                          : (uint32_t)(min(lrow[i], last_row) * M2_ROWB + lcol[i]);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off),
+                                             (__attribute__((address_space(3))) void*)(dst + 1024 * (M2_WAVES * i + w)),
+                                             16, 0, 0);
+        }
     };
 
-    f32x4 acc[MLA_DB];                                        // acc[db][i]: column 16 db + 4 g + i of this wave's half
+    // ---- operand read addresses within a ring buffer
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)mla_smem;
+    // K: row rho, chunk 2 j + h = 8 (j / 4) + 2 (j % 4) + h: one address per j % 4, 128 (j / 4) is an immediate
+    uint32_t klane[2][4];                                     // [half of the ring][j % 4]
 #pragma unroll
-    for (int db = 0; db < MLA_DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_run = MLA_NEG, l_run = 0.f;
-
-    if (ntiles > 0) {
-        load_tile(part_start);
-        store_tile(mla_smem);
+    for (int jb = 0; jb < 4; ++jb) {
+        klane[0][jb] = lds0 + rho * M2_ROWB + ((32u * jb + 16u * h) ^ (16u * m2_key(rho)));
+        klane[1][jb] = klane[0][jb] + 2 * M2_TILE_BYTES;
     }
-    __syncthreads();
+    // V^T: lane j of 16 names token 16 th + 8 e + 4 h + (j >> 2) and the 4 values d = 32 db + rho0 + 4 (j & 3) ..;
+    // chunk 4 db + cl: one address per (e, db % 2), the rest is an immediate
+    const int jj = rho & 15, tq = jj >> 2;
+    const int cl = (rho & 16) / 8 + ((jj & 3) >> 1);
+    uint32_t vlane[2][2][2];                                  // [half of the ring][e][db % 2]
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            const int key = 4 * ((tq >> 1) & 1) + ((2 * e + h) & 3);          // m2_key of that token row
+            vlane[0][e][pb] = lds0 + (8 * e + 4 * h + tq) * M2_ROWB + 16 * ((4 * pb + cl) ^ key) + 8 * (jj & 1);
+            vlane[1][e][pb] = vlane[0][e][pb] + 2 * M2_TILE_BYTES;
+        }
 
-#pragma unroll 1
-    for (int it = 0; it < ntiles; ++it) {
-        const int tstart = part_start + it * MLA_TILE;
-        const bool more = it + 1 < ntiles;
-        const uint8_t* tile = mla_smem + (it & 1) * MLA_TILE_BYTES;
-        if (more) load_tile(tstart + MLA_TILE);               // streams in behind this tile's math
+    // accumulators: acc[db][i]: d = 32 db + 8 (i / 4) + 4 h + i % 4.  They live in the accumulation registers (the
+    // PV MFMAs below are asm statements that name them with the "a" constraint) and leave them only for the rare
+    // rescale and for the final store.
+    f32x16 acc[M2_DB];
+#pragma unroll
+    for (int db = 0; db < M2_DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+    // m_ref: the reference point of the exponentials in raw score units (the positive softmax scale is applied
+    // inside the exponent); it starts above the mask value so that a fully masked tile gives zeros
+    float m_ref = 0.5f * MLA_NEG, l_run = 0.f;
+    const float lazy = M2_LAZY / scale_log2;
 
-        // ---- scores: S[s][i] = score of token tstart + 16 s + 4 g + i for head r
-        f32x4 sc[2];
+    // One tile: scores, softmax, PV product.  With one wave per SIMD nothing is gained by interleaving the matrix and
+    // vector instructions of different tiles (a wave runs its own MFMAs and vector instructions one after the other),
+    // so the phases follow each other; the LDS reads run four operands ahead of the MFMAs that use them.
+    auto step = [&](int t, auto ring_c) {
+        constexpr int R = decltype(ring_c)::value;
+        constexpr int P = 4;
+        // ring buffers 2 and 3 lie beyond the 16-bit offset field of an LDS read: a second set of addresses
+        constexpr int OFF = (R & 1) * M2_TILE_BYTES, HI = R >> 1;
+        const int ts = part_start + t * MLA_TILE;
+
+        // ---- S^T[token, head] = C[token, :576] . Q[head, :576]
+        f32x16 sc;
+        {
+            u32x4 ka[P];
+            auto fetch = [&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                if constexpr (m < M2_KS) ka[m % P] = lds_read16_at<OFF + 128 * (m / 4)>(klane[HI][m % 4]);
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<P>(fetch);
+            static_for<M2_KS>([&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                constexpr int left = M2_KS - 1 - m;
+                wait_lds_reads<(left < P - 1 ? left : P - 1)>();
+                if constexpr (m == 0) {
+                    f32x16 z;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) sc[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    for (int e = 0; e < 16; ++e) z[e] = 0.f;
+                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], z);
+                } else {
+                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], sc);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(std::integral_constant<int, m + P>{});
+            });
+        }
+        if (ts + MLA_TILE > L) {                              // last tile of the sequence: mask what lies past it
 #pragma unroll
-        for (int j = 0; j < MLA_KS; ++j) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const u32x4 ka = *(const u32x4*)(tile + (s * 16 + r) * MLA_STRIDE + (32 * j + 8 * g) * 2);
-                sc[s] = T::mfma16(bitcast<vec8>(ka), qreg[j], sc[s]);
+            for (int i = 0; i < 16; ++i) {
+                const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
+                sc[i] = tok < L ? sc[i] : MLA_NEG;
             }
         }
-        float tmax = MLA_NEG;
-        if (tstart + MLA_TILE <= L) {
+        float tmax = sc[0];
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    sc[s][i] *= scale_log2;
-                    tmax = fmaxf(tmax, sc[s][i]);
-                }
-        } else {                                              // last tile of the sequence: mask what lies past it
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int tok = tstart + s * 16 + 4 * g + i;
-                    const float v = tok < L ? sc[s][i] * scale_log2 : MLA_NEG;
-                    sc[s][i] = v;
-                    tmax = fmaxf(tmax, v);
-                }
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-        uint32_t pp[4];
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const float p0 = __builtin_amdgcn_exp2f(sc[s][0] - m_new), p1 = __builtin_amdgcn_exp2f(sc[s][1] - m_new);
-            const float p2 = __builtin_amdgcn_exp2f(sc[s][2] - m_new), p3 = __builtin_amdgcn_exp2f(sc[s][3] - m_new);
-            pp[2 * s] = pack2<T>(p0, p1);
-            pp[2 * s + 1] = pack2<T>(p2, p3);
-            // the denominator sums the probabilities as the PV product sees them (rounded to T)
-            psum += T::to_float((uint16_t)(pp[2 * s] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s] >> 16)) +
-                    T::to_float((uint16_t)(pp[2 * s + 1] & 0xffff)) + T::to_float((uint16_t)(pp[2 * s + 1] >> 16));
-        }
-        // when the running maximum moved for no lane of the wave, alpha is exactly 1: skip the rescale
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, sc[i]);
+        tmax = max_xor32(tmax);
+        const float m_new = tmax > m_ref + lazy ? tmax : m_ref;
+        if (__builtin_amdgcn_ballot_w64(m_new != m_ref) != 0) {       // the reference point moves: rare
+            const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * scale_log2);
             l_run *= alpha;
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      // the last PV MFMAs have written their registers
 #pragma unroll
-            for (int db = 0; db < MLA_DB; ++db) acc[db] *= alpha;
+            for (int db = 0; db < M2_DB; ++db) {
+                asm volatile("" : "+a"(acc[db]));
+                acc[db] *= alpha;
+                asm volatile("" : "+a"(acc[db]));
+            }
+            asm volatile("s_nop 7" ::: "memory");
+            m_ref = m_new;
         }
-        l_run += psum;
-        const vec8 pfrag = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
-
-        // ---- O^T += C^T P^T over this wave's 256 value columns.  The A operand (row d, 8 tokens in the order of the
-        // probabilities) comes from the row-major tile through the transposing LDS read: within 16 lanes, lane j
-        // names C[token 4g + (j >> 2)][d0 + 4 (j & 3) ..] and lane r receives C[token 4g + e][d0 + r], e = 0..3.
+        const float nm = -m_ref * scale_log2;
+        uint32_t pp[8];
 #pragma unroll
-        for (int db = 0; db < MLA_DB; ++db) {
-            const int d0 = vhalf * (MLA_DV / 2) + 16 * db;
-            const uint8_t* p0 = tile + (4 * g + (r >> 2)) * MLA_STRIDE + (d0 + 4 * (r & 3)) * 2;
-            const u32x2 l2 = bitcast<u32x2>(lds_read_tr16(p0));
-            const u32x2 h2 = bitcast<u32x2>(lds_read_tr16(p0 + 16 * MLA_STRIDE));
-            acc[db] = T::mfma16(bitcast<vec8>((u32x4){l2[0], l2[1], h2[0], h2[1]}), pfrag, acc[db]);
+        for (int k = 0; k < 8; ++k) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[2 * k], scale_log2, nm));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[2 * k + 1], scale_log2, nm));
+            pp[k] = pack2<T>(p0, p1);
+            l_run = T::sum2(pp[k], l_run);                    // sums the probabilities as the PV product sees them
         }
+        const vec8 pf0 = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
+        const vec8 pf1 = bitcast<vec8>((u32x4){pp[4], pp[5], pp[6], pp[7]});
 
-        if (more) store_tile(mla_smem + ((it + 1) & 1) * MLA_TILE_BYTES);
-        __syncthreads();                                      // next tile staged; this tile's readers are done
+        // ---- O^T[d, head] += C^T[d, token] . P^T[token, head]: MFMA v = 16 th + db (token half th, column block db)
+        {
+            u32x2 lo[P], hi[P];
+            auto fetch = [&](auto vc) {
+                constexpr int v = decltype(vc)::value;
+                if constexpr (v < M2_NV) {
+                    constexpr int th = v / M2_DB, db = v % M2_DB;
+                    lo[v % P] = lds_read_tr16_at<OFF + 16 * th * M2_ROWB + 128 * (db / 2)>(vlane[HI][0][db % 2]);
+                    hi[v % P] = lds_read_tr16_at<OFF + 16 * th * M2_ROWB + 128 * (db / 2)>(vlane[HI][1][db % 2]);
+                }
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<P>(fetch);
+            static_for<M2_NV>([&](auto vc) {
+                constexpr int v = decltype(vc)::value;
+                constexpr int th = v / M2_DB, db = v % M2_DB;
+                constexpr int left = M2_NV - 1 - v;
+                wait_lds_reads<2 * (left < P - 1 ? left : P - 1)>();
+                const u32x4 va = {lo[v % P][0], lo[v % P][1], hi[v % P][0], hi[v % P][1]};
+                T::mfma32_acc(acc[db], bitcast<vec8>(va), th ? pf1 : pf0);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(std::integral_constant<int, v + P>{});
+            });
+        }
+    };
+
+    issue_tile(0);
+    if (ntiles > 1) issue_tile(1);
+#pragma unroll
+    for (int j = 0; j < M2_KS; ++j) asm volatile("" : "+v"(qreg[j]));   // the query is complete before the loop
+    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 2,
+    // whose buffer takes tile t + 2
+    auto sync_issue = [&](int t) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(M2_LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 2 < ntiles) issue_tile(t + 2);
+    };
+    constexpr std::integral_constant<int, 0> r0{};
+    constexpr std::integral_constant<int, 1> r1{};
+    constexpr std::integral_constant<int, 2> r2{};
+    constexpr std::integral_constant<int, 3> r3{};
+    int t = 0;
+#pragma unroll 1
+    for (; t + 3 < ntiles; t += 4) {
+        sync_issue(t);
+        step(t, r0);
+        sync_issue(t + 1);
+        step(t + 1, r1);
+        sync_issue(t + 2);
+        step(t + 2, r2);
+        sync_issue(t + 3);
+        step(t + 3, r3);
     }
+    if (t < ntiles) {
+        sync_issue(t);
+        step(t, r0);
+        if (++t < ntiles) {
+            sync_issue(t);
+            step(t, r1);
+            if (++t < ntiles) {
+                sync_issue(t);
+                step(t, r2);
+            }
+        }
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");              // the last PV MFMAs have written their registers
 
-    // ---- write this wave's (heads, columns): the final rows (single partition) or an fp32 partial
-    l_run += __shfl_xor(l_run, 16, 64);
+    // ---- every lane writes its head's values: 4 consecutive columns per accumulator quad
     l_run += __shfl_xor(l_run, 32, 64);
     if (!head_ok) return;
     const int64_t gh = (int64_t)b * n_heads + head;
-    const float inv = 1.0f / l_run;
+    if (max_parts == 1) {
+        const float inv = 1.0f / l_run;
+        uint16_t* dst = out + gh * MLA_DV + 4 * h;
 #pragma unroll
-    for (int db = 0; db < MLA_DB; ++db) {
-        const int d = vhalf * (MLA_DV / 2) + 16 * db + 4 * g;
-        if (max_parts == 1) {
-            const u32x2 o = {pack2<T>(acc[db][0] * inv, acc[db][1] * inv), pack2<T>(acc[db][2] * inv, acc[db][3] * inv)};
-            *(u32x2*)(out + gh * MLA_DV + d) = o;
-        } else {
-            *(f32x4*)(part_out + (gh * max_parts + part) * MLA_DV + d) = acc[db];
+        for (int db = 0; db < M2_DB; ++db)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                *(u32x2*)(dst + 32 * db + 8 * q4) =
+                    (u32x2){pack2<T>(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
+                            pack2<T>(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv)};
+    } else {
+        const int64_t pi = gh * max_parts + part;
+        float* dst = part_out + pi * MLA_DV + 4 * h;
+#pragma unroll
+        for (int db = 0; db < M2_DB; ++db)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+                *(f32x4*)(dst + 32 * db + 8 * q4) =
+                    (f32x4){acc[db][4 * q4], acc[db][4 * q4 + 1], acc[db][4 * q4 + 2], acc[db][4 * q4 + 3]};
+        if (h == 0) {
+            part_ml[pi * 2] = m_ref * scale_log2;
+            part_ml[pi * 2 + 1] = l_run;
         }
-    }
-    if (max_parts > 1 && g == 0 && vhalf == 0) {
-        part_ml[(gh * max_parts + part) * 2] = m_run;
-        part_ml[(gh * max_parts + part) * 2 + 1] = l_run;
     }
 }
 
@@ -297,7 +406,7 @@ struct MlaPlan {
 };
 inline MlaPlan mla_plan(int batch, int n_heads, int64_t max_ctx) {
     MlaPlan p;
-    p.head_blocks = (n_heads + MLA_HEADS - 1) / MLA_HEADS;
+    p.head_blocks = (n_heads + M2_HEADS - 1) / M2_HEADS;
     const int64_t seq_items = std::max<int64_t>(1, (int64_t)batch * p.head_blocks);
     const int64_t want = std::max<int64_t>(1, (512 + seq_items - 1) / seq_items);
     int64_t pt = (max_ctx + want - 1) / want;
@@ -321,7 +430,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
     }
     if (!configured[dev]) {
         e = hipFuncSetAttribute((const void*)mla_decode_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                MLA_SMEM);
+                                M2_SMEM);
         if (e != hipSuccess) return (int)e;
         configured[dev] = true;
     }
@@ -337,7 +446,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
         if (rc) return rc;
     }
     const int64_t wgs = (int64_t)batch * plan.max_parts * plan.head_blocks;
-    hipLaunchKernelGGL(mla_decode_kernel<T>, dim3((unsigned)wgs), dim3(MLA_THREADS), MLA_SMEM, st, (uint16_t*)out,
+    hipLaunchKernelGGL(mla_decode_kernel<T>, dim3((unsigned)wgs), dim3(M2_WAVES * 64), M2_SMEM, st, (uint16_t*)out,
                        part_out, part_ml, (const uint16_t*)query, (const uint16_t*)cache, block_tables, context_lens,
                        n_heads, plan.head_blocks, block_size, max_blocks, num_blocks, plan.max_parts,
                        plan.part_tokens, scale_log2, q_stride, batch);
@@ -373,6 +482,7 @@ extern "C" int mf_mla_paged_attention_decode(void* out, const void* query, const
     MF_REQUIRE(kv_lora_rank == MLA_DV && rope_dim == MLA_DK - MLA_DV,
                "mla_paged_attention: kv_lora_rank %d / rope dim %d not supported (512 / 64)", kv_lora_rank, rope_dim);
     MF_REQUIRE(n_heads > 0, "mla_paged_attention: n_heads must be positive");
+    MF_REQUIRE(scale > 0.f, "mla_paged_attention: the softmax scale must be positive");
     MF_REQUIRE(block_size > 0 && block_size % MLA_TILE == 0 && max_blocks_per_seq > 0 && num_blocks > 0,
                "mla_paged_attention: block_size (%d) must be a positive multiple of %d", block_size, MLA_TILE);
     MF_REQUIRE((int64_t)block_size * max_blocks_per_seq <= 0x7fffffffLL,

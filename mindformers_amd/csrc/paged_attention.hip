@@ -514,41 +514,6 @@ struct PfSmem {
     static constexpr int BYTES = PF_RING * BUF;
 };
 
-template <int OFF>
-__device__ __forceinline__ u32x4 pf_lds_read16(uint32_t addr) {
-    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
-    u32x4 v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
-    return v;
-}
-template <int OFF>
-__device__ __forceinline__ u32x2 pf_lds_read_tr(uint32_t addr) {
-    static_assert(OFF >= 0 && OFF < 65536, "LDS offset field");
-    u32x2 v;
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
-    return v;
-}
-template <int N>
-__device__ __forceinline__ void pf_wait_lds() {
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-// maximum of a value over the two lanes l and l ^ 32 (the instruction swaps the upper half of its first operand with
-// the lower half of its second)
-__device__ __forceinline__ float pf_max_xor32(float v) {
-    float a = v, b = v;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    return fmaxf(a, b);
-}
-template <typename F, int... I>
-__device__ __forceinline__ void pf_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void pf_static_for(F&& f) {
-    pf_static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 template <typename T, int D, bool TIB>
 __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
@@ -783,11 +748,11 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
         auto fetch = [&](auto mc) {
             constexpr int m = decltype(mc)::value;
             if constexpr (m < NQ) {
-                ka[m % P] = pf_lds_read16<KOFF>(klane[m]);
+                ka[m % P] = lds_read16_at<KOFF>(klane[m]);
             } else if constexpr (m < NT) {
                 constexpr int v = m - NQ, th = v / DB, db = v % DB;
-                lo[m % P] = pf_lds_read_tr<VOFF + 16 * th * ROWB>(vlane[db]);
-                hi[m % P] = pf_lds_read_tr<VOFF + (16 * th + 8) * ROWB>(vlane[db]);
+                lo[m % P] = lds_read_tr16_at<VOFF + 16 * th * ROWB>(vlane[db]);
+                hi[m % P] = lds_read_tr16_at<VOFF + (16 * th + 8) * ROWB>(vlane[db]);
             }
         };
         // probabilities 2 k, 2 k + 1 of the previous tile, rounded to T; the denominator sums them as the PV product
@@ -800,14 +765,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
             asm volatile("" : "+v"(pp[k]), "+v"(l_run));    // computed here, not where it is first used
         };
         __builtin_amdgcn_sched_barrier(0);
-        pf_static_for<(P < NT ? P : NT)>(fetch);
+        static_for<(P < NT ? P : NT)>(fetch);
         if constexpr (PREV) l_run *= alpha;
         if constexpr (PREV && !CUR) {                         // last tile: no score MFMAs to work beside
 #pragma unroll
             for (int k = 0; k < 8; ++k) prob_pair(k);
         }
         float tmax = PA_NEG, m_new = 0.f;
-        pf_static_for<NT>([&](auto mc) {
+        static_for<NT>([&](auto mc) {
             constexpr int m = decltype(mc)::value;
             // LDS reads issued after those of fetch m
             constexpr int last = (m + P < NT ? m + P : NT) - 1;
@@ -833,7 +798,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            pf_wait_lds<k_after + 2 * v_after>();
+            wait_lds_reads<k_after + 2 * v_after>();
             if constexpr (m < NQ) {
                 if constexpr (m == 0) {
                     f32x16 z;
@@ -867,7 +832,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
                     } else if (c == 1) {
 #pragma unroll
                         for (int i = 8; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
-                        tmax = pf_max_xor32(tmax);
+                        tmax = max_xor32(tmax);
                     } else if (c == 2) {
                         m_new = fmaxf(m_run, tmax);
                         alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
@@ -892,7 +857,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
-            tmax = pf_max_xor32(tmax);
+            tmax = max_xor32(tmax);
             m_new = fmaxf(m_run, tmax);
             alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
             m_run = m_new;
