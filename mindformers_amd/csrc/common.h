@@ -54,6 +54,13 @@ struct BF16 {
     static __device__ __forceinline__ void mfma32_acc(f32x16& c, vec8 a, vec8 b) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
+    // likewise with the accumulator in ordinary registers: c = a b, then c += a b
+    static __device__ __forceinline__ void mfma32_first(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void mfma32_next(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
     // c + both halves of a packed pair, in fp32 (one dot-product instruction)
     static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
         typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_v;
@@ -79,6 +86,12 @@ struct FP16 {
     }
     static __device__ __forceinline__ void mfma32_acc(f32x16& c, vec8 a, vec8 b) {
         asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void mfma32_first(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void mfma32_next(f32x16& c, vec8 a, vec8 b) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ float sum2(uint32_t pair, float c) {
         typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_v;

@@ -53,17 +53,52 @@ static_assert(M2_TILE_BYTES % (1024 * M2_WAVES) == 0 && M2_SMEM <= 160 * 1024, "
 
 __device__ __forceinline__ int m2_key(int row) { return 4 * ((row >> 1) & 1) + ((row >> 2) & 3); }
 
+// Smallest partition the kernels use: at most 32 partitions per sequence, never less than 256 tokens.
+__host__ __device__ inline int mla_min_part(int max_ctx) {
+    const int p = ((max_ctx + 31) / 32 + 31) / 32 * 32;
+    return p > 256 ? p : 256;
+}
+// Workgroups the partition rule below can produce at most.
+__host__ __device__ inline int mla_free_slots(int batch, int head_blocks, int n_slots) {
+    const int f = n_slots - batch * head_blocks;
+    return f > n_slots / 4 ? f : n_slots / 4;
+}
+// Tokens per partition, chosen from the actual lengths so that the workgroups fit the chip's n_slots compute units in
+// one round (one workgroup is resident per unit): sum_b ceil(L_b / pt) * head_blocks <= total * head_blocks / pt +
+// batch * head_blocks, which is <= n_slots for pt >= total * head_blocks / (n_slots - batch * head_blocks).  Every
+// wave that calls this gets the same value (the main kernel and the reduce kernel both do).
+__device__ inline int mla_part_tokens(const int32_t* __restrict__ ctx_lens, int batch, int max_ctx, int head_blocks,
+                                      int n_slots) {
+    const int ln = threadIdx.x & 63;
+    int64_t total = 0;
+    for (int c0 = 0; c0 < batch; c0 += 64) {
+        const int bb = c0 + ln;
+        const int len = bb < batch ? ctx_lens[bb] : 0;
+        total += len < 0 ? 0 : (len > max_ctx ? max_ctx : len);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o, 64);
+    const int64_t avail = mla_free_slots(batch, head_blocks, n_slots);
+    int64_t pt = (total * head_blocks + avail - 1) / avail;
+    pt = (pt + 31) / 32 * 32;
+    const int lo = mla_min_part(max_ctx);
+    return pt < lo ? lo : (int)pt;
+}
+
 template <typename T>
 __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ ctx_lens, int n_heads, int head_blocks, int block_size, int max_blocks,
-    int num_blocks, int max_parts, int part_tokens, float scale_log2, int64_t q_stride, int batch) {
+    int num_blocks, int max_parts, int n_slots, float scale_log2, int64_t q_stride, int batch) {
     using vec8 = typename T::vec8;
     extern __shared__ __attribute__((aligned(16))) uint8_t mla_smem[];
+    const int part_tokens =
+        max_parts == 1 ? max_blocks * block_size
+                       : mla_part_tokens(ctx_lens, batch, max_blocks * block_size, head_blocks, n_slots);
 
     // ---- work list: (sequence, partition, head block) triples that exist, from a prefix sum over the lengths
-    int b = -1, part = 0, hb = 0, L = 0;
+    int b = -1, part = 0, hb = 0, L = 0, nparts = 1;
     {
         const int pidx = blockIdx.x;
         const int ln = threadIdx.x & 63;
@@ -89,6 +124,7 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
                 part = rem / head_blocks;
                 hb = rem - part * head_blocks;
                 L = __shfl(len, src, 64);
+                nparts = __shfl(np, src, 64);
                 break;
             }
             base += total;
@@ -99,6 +135,7 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     part = __builtin_amdgcn_readfirstlane(part);
     hb = __builtin_amdgcn_readfirstlane(hb);
     L = __builtin_amdgcn_readfirstlane(L);
+    nparts = __builtin_amdgcn_readfirstlane(nparts);
 
     const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -126,14 +163,12 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
 
     // ---- tile loads: load i of wave w fills LDS slots 64 (4 i + w) .. + 63 of the tile; slot = 72 row + position
     uint32_t lofs[M2_LOADS];                                  // byte offset of the lane's chunk within a whole tile
-    int lrow[M2_LOADS], lcol[M2_LOADS];
 #pragma unroll
     for (int i = 0; i < M2_LOADS; ++i) {
         const int slot = 64 * (M2_WAVES * i + w) + lane;
-        lrow[i] = slot / MLA_CPR;
-        const int pos = slot - lrow[i] * MLA_CPR;
-        lcol[i] = 16 * ((pos & ~7) | ((pos & 7) ^ m2_key(lrow[i])));          // logical chunk of that position
-        lofs[i] = (uint32_t)(lrow[i] * M2_ROWB + lcol[i]);
+        const int row = slot / MLA_CPR;
+        const int pos = slot - row * MLA_CPR;
+        lofs[i] = (uint32_t)(row * M2_ROWB + 16 * ((pos & ~7) | ((pos & 7) ^ m2_key(row))));   // its logical chunk
     }
     auto issue_tile = [&](int t) {                            // a tile lies inside one block (host-checked)
         const int ts = part_start + t * MLA_TILE;
@@ -145,8 +180,11 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         const int last_row = L - 1 - ts;                      // rows past the context re-read the last valid row
 #pragma unroll
         for (int i = 0; i < M2_LOADS; ++i) {
-            const uint32_t off = last_row >= MLA_TILE - 1 ? lofs[i]
-                                                          : (uint32_t)(min(lrow[i], last_row) * M2_ROWB + lcol[i]);
+            uint32_t off = lofs[i];
+            if (last_row < MLA_TILE - 1) {                    // last tile of the sequence only
+                const int row = (int)(off / M2_ROWB);
+                off -= (uint32_t)(max(row - last_row, 0) * M2_ROWB);
+            }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off),
                                              (__attribute__((address_space(3))) void*)(dst + 1024 * (M2_WAVES * i + w)),
                                              16, 0, 0);
@@ -199,7 +237,9 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         constexpr int OFF = (R & 1) * M2_TILE_BYTES, HI = R >> 1;
         const int ts = part_start + t * MLA_TILE;
 
-        // ---- S^T[token, head] = C[token, :576] . Q[head, :576]
+        // ---- S^T[token, head] = C[token, :576] . Q[head, :576].  These MFMAs are asm statements as well, with the
+        // scores in ordinary registers: a compiler-chosen accumulation register tuple for them would have to evict an
+        // accumulator block, and the compiler would copy that block without waiting for the asm MFMAs that wrote it.
         f32x16 sc;
         {
             u32x4 ka[P];
@@ -213,17 +253,13 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
                 constexpr int m = decltype(mc)::value;
                 constexpr int left = M2_KS - 1 - m;
                 wait_lds_reads<(left < P - 1 ? left : P - 1)>();
-                if constexpr (m == 0) {
-                    f32x16 z;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) z[e] = 0.f;
-                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], z);
-                } else {
-                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], sc);
-                }
+                if constexpr (m == 0) T::mfma32_first(sc, bitcast<vec8>(ka[m % P]), qreg[m]);
+                else T::mfma32_next(sc, bitcast<vec8>(ka[m % P]), qreg[m]);
                 __builtin_amdgcn_sched_barrier(0);
                 fetch(std::integral_constant<int, m + P>{});
             });
+            // the compiler does not know that sc comes from matrix instructions: their 8 passes end here
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(sc));
         }
         if (ts + MLA_TILE > L) {                              // last tile of the sequence: mask what lies past it
 #pragma unroll
@@ -336,7 +372,7 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     l_run += __shfl_xor(l_run, 32, 64);
     if (!head_ok) return;
     const int64_t gh = (int64_t)b * n_heads + head;
-    if (max_parts == 1) {
+    if (nparts == 1) {                                        // the only partition of its sequence: final rows
         const float inv = 1.0f / l_run;
         uint16_t* dst = out + gh * MLA_DV + 4 * h;
 #pragma unroll
@@ -369,8 +405,10 @@ __global__ __launch_bounds__(MLA_DV) void mla_reduce_kernel(uint16_t* __restrict
                                                             const float* __restrict__ part_out,
                                                             const float* __restrict__ part_ml,
                                                             const int32_t* __restrict__ ctx_lens, int n_heads,
-                                                            int max_parts, int part_tokens, int max_ctx) {
+                                                            int max_parts, int batch, int head_blocks,
+                                                            int n_slots, int max_ctx) {
     const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const int part_tokens = mla_part_tokens(ctx_lens, batch, max_ctx, head_blocks, n_slots);
     const int L = min(ctx_lens[b], max_ctx);
     const int64_t gh = (int64_t)b * n_heads + h;
     int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
@@ -379,6 +417,7 @@ __global__ __launch_bounds__(MLA_DV) void mla_reduce_kernel(uint16_t* __restrict
         out[gh * MLA_DV + d] = 0;
         return;
     }
+    if (np == 1) return;                                      // the main kernel wrote the final row
     const float* ml = part_ml + gh * max_parts * 2;
     const float* po = part_out + gh * max_parts * MLA_DV + d;
     float M = MLA_NEG;
@@ -398,21 +437,16 @@ __global__ void mla_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t*
     for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)blockIdx.x * row + i] = 0;
 }
 
-// Partition rule shared by the workspace query and the launch: about two workgroups per compute unit when the
-// batch allows it, partitions of whole 256-token multiples (fewer, larger partitions keep the fp32 partials,
-// 2 KB per (head, partition), small beside the cache traffic).
+// Host side of the partition rule: the worst-case number of partitions per sequence (which sizes the workspace) and
+// the number of workgroups the device-side rule can produce at most.
 struct MlaPlan {
-    int part_tokens, max_parts, head_blocks;
+    int max_parts, head_blocks;
 };
-inline MlaPlan mla_plan(int batch, int n_heads, int64_t max_ctx) {
+inline MlaPlan mla_plan(int n_heads, int64_t max_ctx) {
     MlaPlan p;
     p.head_blocks = (n_heads + M2_HEADS - 1) / M2_HEADS;
-    const int64_t seq_items = std::max<int64_t>(1, (int64_t)batch * p.head_blocks);
-    const int64_t want = std::max<int64_t>(1, (512 + seq_items - 1) / seq_items);
-    int64_t pt = (max_ctx + want - 1) / want;
-    pt = std::max<int64_t>(256, (pt + 255) / 256 * 256);
-    p.part_tokens = (int)pt;
-    p.max_parts = (int)std::max<int64_t>(1, (max_ctx + pt - 1) / pt);
+    const int lo = mla_min_part((int)max_ctx);
+    p.max_parts = (int)std::max<int64_t>(1, (max_ctx + lo - 1) / lo);
     return p;
 }
 
@@ -421,6 +455,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
                const int32_t* context_lens, int batch, int n_heads, int block_size, int max_blocks, int num_blocks,
                float scale, int64_t q_stride, void* workspace, hipStream_t st) {
     static bool configured[MF_MAX_DEVICES] = {};
+    static int cu_count[MF_MAX_DEVICES] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
@@ -432,10 +467,13 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
         e = hipFuncSetAttribute((const void*)mla_decode_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 M2_SMEM);
         if (e != hipSuccess) return (int)e;
+        e = hipDeviceGetAttribute(&cu_count[dev], hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return (int)e;
         configured[dev] = true;
     }
+    const int n_slots = cu_count[dev] > 0 ? cu_count[dev] : 256;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    const MlaPlan plan = mla_plan(batch, n_heads, max_ctx);
+    const MlaPlan plan = mla_plan(n_heads, max_ctx);
     float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
     float* part_ml = part_out ? part_out + (int64_t)batch * n_heads * plan.max_parts * MLA_DV : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
@@ -445,16 +483,19 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
         const int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
-    const int64_t wgs = (int64_t)batch * plan.max_parts * plan.head_blocks;
+    const int64_t wgs = plan.max_parts == 1
+                            ? (int64_t)batch * plan.head_blocks
+                            : (int64_t)mla_free_slots(batch, plan.head_blocks, n_slots) + (int64_t)batch * plan.head_blocks;
     hipLaunchKernelGGL(mla_decode_kernel<T>, dim3((unsigned)wgs), dim3(M2_WAVES * 64), M2_SMEM, st, (uint16_t*)out,
                        part_out, part_ml, (const uint16_t*)query, (const uint16_t*)cache, block_tables, context_lens,
-                       n_heads, plan.head_blocks, block_size, max_blocks, num_blocks, plan.max_parts,
-                       plan.part_tokens, scale_log2, q_stride, batch);
+                       n_heads, plan.head_blocks, block_size, max_blocks, num_blocks, plan.max_parts, n_slots,
+                       scale_log2, q_stride, batch);
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
         hipLaunchKernelGGL(mla_reduce_kernel<T>, dim3(n_heads, batch), dim3(MLA_DV), 0, st, (uint16_t*)out, part_out,
-                           part_ml, context_lens, n_heads, plan.max_parts, plan.part_tokens, (int)max_ctx);
+                           part_ml, context_lens, n_heads, plan.max_parts, batch, plan.head_blocks, n_slots,
+                           (int)max_ctx);
         rc = MF_LAUNCH_CHECK();
     }
     return rc;
@@ -464,7 +505,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
 
 extern "C" size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads, int max_context) {
     if (batch <= 0 || n_heads <= 0 || max_context <= 0) return 0;
-    const MlaPlan plan = mla_plan(batch, n_heads, max_context);
+    const MlaPlan plan = mla_plan(n_heads, max_context);
     if (plan.max_parts <= 1) return 0;
     return (size_t)batch * n_heads * plan.max_parts * (MLA_DV + 2) * sizeof(float);
 }
