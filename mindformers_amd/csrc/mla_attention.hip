@@ -399,36 +399,50 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
 }
 
 // Combine the partitions of one (sequence, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p.
-// One workgroup of 512 threads (one per value column) per (head, sequence).
+// One workgroup of 128 threads (4 value columns each) per (head, sequence); the loads of up to 8 partitions are
+// issued together, so a row costs one round trip for the lengths, one for the (max, sum) pairs and one for the
+// accumulators.
+constexpr int MR_THREADS = MLA_DV / 4;
 template <typename T>
-__global__ __launch_bounds__(MLA_DV) void mla_reduce_kernel(uint16_t* __restrict__ out,
-                                                            const float* __restrict__ part_out,
-                                                            const float* __restrict__ part_ml,
-                                                            const int32_t* __restrict__ ctx_lens, int n_heads,
-                                                            int max_parts, int batch, int head_blocks,
-                                                            int n_slots, int max_ctx) {
-    const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+__global__ __launch_bounds__(MR_THREADS) void mla_reduce_kernel(uint16_t* __restrict__ out,
+                                                                const float* __restrict__ part_out,
+                                                                const float* __restrict__ part_ml,
+                                                                const int32_t* __restrict__ ctx_lens, int n_heads,
+                                                                int max_parts, int batch, int head_blocks,
+                                                                int n_slots, int max_ctx) {
+    const int h = blockIdx.x, b = blockIdx.y, d = 4 * threadIdx.x;
     const int part_tokens = mla_part_tokens(ctx_lens, batch, max_ctx, head_blocks, n_slots);
     const int L = min(ctx_lens[b], max_ctx);
     const int64_t gh = (int64_t)b * n_heads + h;
     int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
     np = np < max_parts ? np : max_parts;
+    if (np == 1) return;                                      // the main kernel wrote the final row
     if (np == 0) {
-        out[gh * MLA_DV + d] = 0;
+        *(u32x2*)(out + gh * MLA_DV + d) = (u32x2){0u, 0u};
         return;
     }
-    if (np == 1) return;                                      // the main kernel wrote the final row
     const float* ml = part_ml + gh * max_parts * 2;
     const float* po = part_out + gh * max_parts * MLA_DV + d;
     float M = MLA_NEG;
     for (int p = 0; p < np; ++p) M = fmaxf(M, ml[2 * p]);     // uniform addresses: broadcast loads
-    float num = 0.f, den = 0.f;
-    for (int p = 0; p < np; ++p) {
-        const float f = __builtin_amdgcn_exp2f(ml[2 * p] - M);
-        den += f * ml[2 * p + 1];
-        num += f * po[(int64_t)p * MLA_DV];
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    for (int p0 = 0; p0 < np; p0 += 8) {
+        f32x4 v[8];
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool on = p0 + i < np;
+            v[i] = on ? *(const f32x4*)(po + (int64_t)(p0 + i) * MLA_DV) : (f32x4){0.f, 0.f, 0.f, 0.f};
+            f[i] = on ? __builtin_amdgcn_exp2f(ml[2 * (p0 + i)] - M) : 0.f;
+            den += on ? f[i] * ml[2 * (p0 + i) + 1] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) num += v[i] * f[i];
     }
-    out[gh * MLA_DV + d] = T::from_float(num / den);
+    const float inv = 1.0f / den;
+    *(u32x2*)(out + gh * MLA_DV + d) =
+        (u32x2){pack2<T>(num[0] * inv, num[1] * inv), pack2<T>(num[2] * inv, num[3] * inv)};
 }
 
 // zero the rows of sequences with no context when a single partition spans the context (the main kernel skips them)
@@ -493,7 +507,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
-        hipLaunchKernelGGL(mla_reduce_kernel<T>, dim3(n_heads, batch), dim3(MLA_DV), 0, st, (uint16_t*)out, part_out,
+        hipLaunchKernelGGL(mla_reduce_kernel<T>, dim3(n_heads, batch), dim3(MR_THREADS), 0, st, (uint16_t*)out, part_out,
                            part_ml, context_lens, n_heads, plan.max_parts, batch, plan.head_blocks, n_slots,
                            (int)max_ctx);
         rc = MF_LAUNCH_CHECK();
