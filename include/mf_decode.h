@@ -177,7 +177,7 @@ size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads, int max_co
  * out[b,h,:kv_lora_rank] = softmax(scale * q[b,h,:] . C_b[:L_b]^T) C_b[:L_b, :kv_lora_rank] with C the cache rows
  * of kv_lora_rank + rope_dim values; query [batch, n_heads * (kv_lora_rank + rope_dim)], q_row_stride elements
  * apart (0 = dense); out dense [batch, n_heads * kv_lora_rank].  kv_lora_rank = 512, rope_dim = 64 (the DeepSeek
- * V2 / V3 geometry); block_size a multiple of 32.  Numerics as mf_paged_attention_decode. */
+ * V2 / V3 geometry); block_size a multiple of 32; scale positive.  Numerics as mf_paged_attention_decode. */
 int mf_mla_paged_attention_decode(void* out, const void* query, const void* latent_cache,
                                   const int32_t* block_tables, const int32_t* context_lens, int batch,
                                   int n_heads, int kv_lora_rank, int rope_dim, int block_size,
