@@ -727,7 +727,11 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
     // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0.  Maxima are kept in raw score units: the
     // (positive) softmax scale is applied inside the exponent.
+    // m_run follows the running maximum lazily: it moves only when the maximum exceeds it by more than 2^8 in
+    // probability (moving it means rescaling the accumulators); probabilities then lie in (0, 256], which bf16 and
+    // fp16 hold with the same relative precision, and the result does not depend on the reference point.
     float m_run = 0.5f * PA_NEG, l_run = 0.f;
+    const float lazy = 8.0f / scale_log2;
     float alpha = 1.f, nm = 0.f;                              // of the tile whose scores wait for their exponentials
     f32x16 sc_a, sc_b;
 
@@ -834,7 +838,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
                         for (int i = 8; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
                         tmax = max_xor32(tmax);
                     } else if (c == 2) {
-                        m_new = fmaxf(m_run, tmax);
+                        m_new = tmax > m_run + lazy ? tmax : m_run;
                         alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
                     } else {
                         m_run = m_new;
@@ -858,7 +862,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
             tmax = max_xor32(tmax);
-            m_new = fmaxf(m_run, tmax);
+            m_new = tmax > m_run + lazy ? tmax : m_run;
             alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
             m_run = m_new;
             nm = -m_new * scale_log2;
