@@ -393,6 +393,8 @@ def _mla_abs(q, cache, tables, lens, nh, scale):
     (torch.float16, 64, 32, [95, 400], None),
     (torch.bfloat16, 40, 64, [257, 0, 31, 32], None),          # heads not a multiple of 16, an empty sequence
     (torch.bfloat16, 128, 128, [5000], None),                  # one long sequence: many partitions
+    (torch.bfloat16, 200, 32, [300, 600], None),               # two head blocks, the second one partly filled
+    (torch.float16, 128, 128, [9000, 40], None),               # 32 partitions at most: the smallest partition grows
 ])
 def test_mla_paged_attention_vs_oracle(dtype, nh, bs, lens, max_blocks):
     rng = np.random.default_rng(nh + len(lens))
@@ -401,6 +403,32 @@ def test_mla_paged_attention_vs_oracle(dtype, nh, bs, lens, max_blocks):
     for i, n in enumerate(lens):
         if n == 0:
             assert not got[i].any()
+
+
+def test_mla_paged_attention_large_batch():
+    """More sequences than three quarters of the compute units: the partition rule's floor on free workgroups."""
+    rng = np.random.default_rng(77)
+    lens = rng.integers(1, 90, 210)
+    lens[5] = 700                                              # one sequence that is partitioned
+    got, ref, mag = _mla_case(rng, torch.bfloat16, lens, 16, 32)
+    assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what="MLA paged attention, batch 210")
+
+
+def test_attention_rejects_a_non_positive_scale():
+    """Prefill and MLA decode take the maximum over raw scores: the scale must be positive (checked on the host)."""
+    rng = np.random.default_rng(3)
+    dtype = torch.bfloat16
+    cache, _, tables, _ = make_paged_cache(rng, 1, [40], 1, 576, 32, dtype)
+    q = dev(rng.normal(size=(1, 16 * 576)), dtype)
+    with pytest.raises(Exception, match="scale"):
+        ops.mla_paged_attention(q, dev(cache, dtype), dev(tables, torch.int32), dev(np.asarray([40], np.int32), torch.int32),
+                                16, 512, -0.1)
+    kc, vc, tb, _ = make_paged_cache(rng, 1, [40], 2, 64, 32, dtype)
+    qq = dev(rng.normal(size=(40, 4 * 64)), dtype)
+    with pytest.raises(Exception, match="scale"):
+        ops.paged_attention_prefill(qq, dev(kc, dtype), dev(vc, dtype), dev(tb, torch.int32),
+                                    dev(np.asarray([40], np.int32), torch.int32), dev(_starts([40]), torch.int32), 4, 2, 0.0)
+
 
 
 def test_mla_cache_is_written_by_key_only_reshape_and_cache():
