@@ -368,33 +368,55 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");              // the last PV MFMAs have written their registers
 
-    // ---- every lane writes its head's values: 4 consecutive columns per accumulator quad
+    // ---- results.  A lane holds 4 consecutive columns per accumulator quad of one head, which would make 8- and
+    // 16-byte pieces in global memory; the accumulators go through LDS instead (the ring is idle now: a wave takes a
+    // quarter of it, 256 columns of its 32 heads at a time, rows padded by 16 bytes against bank conflicts) and leave
+    // as whole rows: 1 KB of fp32 partials, or 512 bytes of final values, per store instruction.
     l_run += __shfl_xor(l_run, 32, 64);
-    if (!head_ok) return;
-    const int64_t gh = (int64_t)b * n_heads + head;
-    if (nparts == 1) {                                        // the only partition of its sequence: final rows
-        const float inv = 1.0f / l_run;
-        uint16_t* dst = out + gh * MLA_DV + 4 * h;
+    __syncthreads();                                          // every wave has read its last tile
+    constexpr int OROW = 256 * 4 + 16;                        // bytes per staged row of 256 fp32 columns
+    static_assert(32 * OROW <= M2_SMEM / M2_WAVES, "a wave's output rows must fit its quarter of the ring");
+    uint8_t* stage = mla_smem + w * (M2_SMEM / M2_WAVES);
+    const int head0 = hb * M2_HEADS + w * 32;                 // first head of this wave
+    const int live = min(32, n_heads - head0);                // heads of this wave that exist (may be <= 0)
+    const float inv = nparts == 1 ? 1.0f / l_run : 1.0f;
+    if (nparts > 1 && head_ok && h == 0) {
+        const int64_t pi = ((int64_t)b * n_heads + head) * max_parts + part;
+        part_ml[pi * 2] = m_ref * scale_log2;
+        part_ml[pi * 2 + 1] = l_run;
+    }
 #pragma unroll
-        for (int db = 0; db < M2_DB; ++db)
+    for (int hv = 0; hv < 2; ++hv) {                          // unrolled: the accumulator blocks are named statically
+        if (hv) __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int d8 = 0; d8 < M2_DB / 2; ++d8) {
+            const int db = hv * (M2_DB / 2) + d8;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4)
-                *(u32x2*)(dst + 32 * db + 8 * q4) =
-                    (u32x2){pack2<T>(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
-                            pack2<T>(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv)};
-    } else {
-        const int64_t pi = gh * max_parts + part;
-        float* dst = part_out + pi * MLA_DV + 4 * h;
-#pragma unroll
-        for (int db = 0; db < M2_DB; ++db)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4)
-                *(f32x4*)(dst + 32 * db + 8 * q4) =
-                    (f32x4){acc[db][4 * q4], acc[db][4 * q4 + 1], acc[db][4 * q4 + 2], acc[db][4 * q4 + 3]};
-        if (h == 0) {
-            part_ml[pi * 2] = m_ref * scale_log2;
-            part_ml[pi * 2 + 1] = l_run;
+                *(f32x4*)(stage + rho * OROW + (32 * d8 + 8 * q4 + 4 * h) * 4) =
+                    (f32x4){acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv, acc[db][4 * q4 + 2] * inv,
+                            acc[db][4 * q4 + 3] * inv};
         }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (nparts == 1) {                                    // the only partition of its sequence: final rows
+            // two heads per pass: lanes 0-31 one row, lanes 32-63 the next; 8 columns per lane
+            for (int r0 = 0; r0 < live; r0 += 2) {
+                const int r = r0 + h;
+                if (r >= live) continue;
+                const f32x4 lo = *(const f32x4*)(stage + r * OROW + rho * 32);
+                const f32x4 hi = *(const f32x4*)(stage + r * OROW + rho * 32 + 16);
+                const u32x4 o = {pack2<T>(lo[0], lo[1]), pack2<T>(lo[2], lo[3]), pack2<T>(hi[0], hi[1]),
+                                 pack2<T>(hi[2], hi[3])};
+                *(u32x4*)(out + ((int64_t)b * n_heads + head0 + r) * MLA_DV + 256 * hv + 8 * rho) = o;
+            }
+        } else {
+            for (int r = 0; r < live; ++r) {
+                const int64_t pi = ((int64_t)b * n_heads + head0 + r) * max_parts + part;
+                *(f32x4*)(part_out + pi * MLA_DV + 256 * hv + 4 * lane) = *(const f32x4*)(stage + r * OROW + lane * 16);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
 }
 
