@@ -1125,7 +1125,9 @@ static inline PfPlan pf_plan(int batch, int64_t total_q, int n_heads, int n_kv, 
     PfPlan p;
     p.col_groups16 = (total_q * n_rep + 15) / 16 + batch;     // each sequence rounds its own columns up
     p.col_groups128 = (total_q * n_rep + PF_COLS - 1) / PF_COLS + batch;
-    const int64_t wgs = std::max<int64_t>(1, (total_q * n_rep + PF_COLS - 1) / PF_COLS) * n_kv;
+    // column groups over the batch: at least one per sequence that brings a query
+    const int64_t groups = std::max<int64_t>((total_q * n_rep + PF_COLS - 1) / PF_COLS, std::min<int64_t>(batch, total_q));
+    const int64_t wgs = std::max<int64_t>(1, groups) * n_kv;
     int64_t want = (512 + wgs - 1) / wgs;                     // 2 workgroups per CU are resident at a time
     const int64_t most = std::max<int64_t>(1, (max_ctx + 255) / 256);
     want = std::min(want, most);
