@@ -255,6 +255,17 @@ def test_paged_prefill_vs_oracle(dtype, nh, nkv, d, bs, lens, q_lens):
     assert_within(got, ref, mag, dtype, ulps=1.5, what="paged prefill")
 
 
+def test_paged_prefill_many_short_sequences():
+    """More sequences than one wave scans at a time, with empty ones, no new tokens, and one-token contexts."""
+    rng = np.random.default_rng(41)
+    b = 150
+    lens = rng.integers(0, 70, b)
+    q_lens = np.minimum(lens, rng.integers(0, 9, b))
+    lens[7], q_lens[7] = 300, 300                              # one long prompt among them
+    got, ref, mag = _prefill_case(rng, torch.bfloat16, 8, 2, 64, 16, lens, q_lens)
+    assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what="paged prefill, 150 sequences")
+
+
 def test_paged_prefill_rows_of_no_sequence_are_zero():
     """Rows past q_starts[batch] (padding of a fixed-size launch) come back as zeros, on both the single-partition
     path and the partitioned one; a sequence that claims more queries than context only gets its context's worth."""
