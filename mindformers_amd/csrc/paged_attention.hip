@@ -1,6 +1,7 @@
-// GQA paged-attention decode for gfx950.
+// GQA paged attention for gfx950: the decode kernel (one query row per sequence; also the prefill path of int8
+// caches), its partition reduce, and further down the prefill kernel (several causal query rows per sequence).
 //
-// Work decomposition
+// Decode: work decomposition
 //   grid = batch * max_partitions * n_kv_heads * head_groups (1-D); one workgroup of 4 wavefronts owns one
 //   256- or 512-token partition of one (sequence, kv head) and ALL query heads that share that kv head (up to 16
 //   per head group), so every K/V byte is fetched from HBM exactly once.  Workgroups whose partition
