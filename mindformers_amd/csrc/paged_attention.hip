@@ -490,22 +490,23 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
 //   8 T .. 8 T + 7 are, in order, exactly the 8 k-values a lane supplies to the B operand of token half T when that
 //   half's 16 tokens are taken in the order (4 h + e, 8 + 4 h + e); the V^T operand is read in the same order with
 //   the transposing LDS read.
-// Tiles go from global memory straight into LDS (no registers in between) through a ring of 4 buffers, two tiles
+// Tiles go from global memory straight into LDS (no registers in between) through a ring of 3 buffers, two tiles
 // ahead, with one barrier per tile.  Such a load writes 64 consecutive 16-byte slots, so rows cannot be padded;
 // instead the 16-byte chunks of a row are permuted by the address each lane supplies:
 //   K: chunk c of row t sits in slot c ^ key(t): the 16 rows of one chunk that an operand read serves together
 //      land on 16 different slots;
 //   V: chunk c of row t sits in slot (c + 4 key4(t)) mod chunks-per-row: the 4 tokens x 64 bytes a transposing read
 //      serves together land on different slots.
-// The matrix pipe and the vector ALU work side by side inside a wave: in step t the score MFMAs of tile t are
-// interleaved with the exponentials of tile t - 1, and the PV MFMAs of tile t - 1 with the running-maximum update of
-// tile t.  The LDS reads are issued by hand a few MFMAs ahead and the order of the step is pinned with scheduling
-// barriers (the compiler would otherwise wait for each read and serialise the two pipes).
+// The LDS reads are asm statements issued a few MFMAs ahead with counted waits (the compiler would wait for each
+// read before the next), and the order is pinned with scheduling barriers.  Three workgroups are resident per
+// compute unit (48 KB of LDS, at most 168 registers), so a SIMD holds three waves whose matrix and vector phases
+// overlap; a version that interleaved the phases of neighbouring tiles inside a wave needed 216 registers and was
+// no faster with two.
 // A wave owns its columns over the whole partition, so there is no merge: it writes final rows (single partition) or
 // fp32 partials for the reduce kernel.
 constexpr int PF_COLS = 128;                                  // columns per workgroup
 constexpr int PF_TOK = 32;                                    // tokens per staged tile
-constexpr int PF_RING = 4;                                    // staged tiles
+constexpr int PF_RING = 3;                                    // staged tiles
 
 template <int D>
 struct PfSmem {
@@ -516,7 +517,7 @@ struct PfSmem {
 };
 
 template <typename T, int D, bool TIB>
-__global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
+__global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
@@ -657,7 +658,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     auto issue_tile = [&](int t) {
         if (LW < PA_WAVES && w >= LW) return;
         const int ts = part_start + t * PF_TOK;
-        uint8_t* kdst = pf_smem + (t & (PF_RING - 1)) * S::BUF;
+        uint8_t* kdst = pf_smem + (t % PF_RING) * S::BUF;
         int64_t slot0 = 0;
         if constexpr (TIB) {                                  // the tile lies inside one block: one uniform lookup
             if (contiguous) {
@@ -733,140 +734,98 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     // fp16 hold with the same relative precision, and the result does not depend on the reference point.
     float m_run = 0.5f * PA_NEG, l_run = 0.f;
     const float lazy = 8.0f / scale_log2;
-    float alpha = 1.f, nm = 0.f;                              // of the tile whose scores wait for their exponentials
-    f32x16 sc_a, sc_b;
 
-    // One step: scores of tile t into `cur` (CUR) beside the exponentials of tile t - 1 from `prev` (PREV), then the
-    // PV product of tile t - 1 beside the running-maximum update of tile t.
-    // Tile t lives in ring buffer R = t mod 4 (a compile-time constant of the step), tile t - 1 in buffer R - 1.
-    auto step = [&](int t, auto ring_c, f32x16& cur, f32x16& prev, auto cur_c, auto prev_c) {
-        constexpr bool CUR = decltype(cur_c)::value, PREV = decltype(prev_c)::value;
+    // One tile, living in ring buffer R = t mod 3 (a compile-time constant of the step): scores, softmax, PV product,
+    // one phase after the other.  A wave does not overlap its own MFMAs with its own vector instructions, so nothing
+    // is gained by interleaving the phases of neighbouring tiles inside a wave; the other waves of the SIMD (3
+    // workgroups are resident per compute unit) fill the gaps.  The LDS reads run P operands ahead of the MFMAs.
+    auto step = [&](int t, auto ring_c) {
         constexpr int R = decltype(ring_c)::value;
-        constexpr int NQ = CUR ? KS : 0, NP = PREV ? NV : 0, NT = NQ + NP, P = 4;
-        constexpr int KOFF = R * S::BUF, VOFF = ((R + PF_RING - 1) % PF_RING) * S::BUF;
+        constexpr int OFF = R * S::BUF, P = 4;
         const int ts = part_start + t * PF_TOK;
-        u32x4 ka[P];
-        u32x2 lo[P], hi[P];
-        uint32_t pp[8];
-        // operand fetch m: K operand of k-step m, or (after the NQ score MFMAs) the V operand of PV MFMA m - NQ =
-        // DB th + db (token half th, d block db), two transposing reads
-        auto fetch = [&](auto mc) {
-            constexpr int m = decltype(mc)::value;
-            if constexpr (m < NQ) {
-                ka[m % P] = lds_read16_at<KOFF>(klane[m]);
-            } else if constexpr (m < NT) {
-                constexpr int v = m - NQ, th = v / DB, db = v % DB;
-                lo[m % P] = lds_read_tr16_at<VOFF + 16 * th * ROWB>(vlane[db]);
-                hi[m % P] = lds_read_tr16_at<VOFF + (16 * th + 8) * ROWB>(vlane[db]);
-            }
-        };
-        // probabilities 2 k, 2 k + 1 of the previous tile, rounded to T; the denominator sums them as the PV product
-        // sees them
-        auto prob_pair = [&](int k) {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(prev[2 * k], scale_log2, nm));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(prev[2 * k + 1], scale_log2, nm));
-            pp[k] = pack2<T>(p0, p1);
-            l_run = T::sum2(pp[k], l_run);
-            asm volatile("" : "+v"(pp[k]), "+v"(l_run));    // computed here, not where it is first used
-        };
-        __builtin_amdgcn_sched_barrier(0);
-        static_for<(P < NT ? P : NT)>(fetch);
-        if constexpr (PREV) l_run *= alpha;
-        if constexpr (PREV && !CUR) {                         // last tile: no score MFMAs to work beside
-#pragma unroll
-            for (int k = 0; k < 8; ++k) prob_pair(k);
-        }
-        float tmax = PA_NEG, m_new = 0.f;
-        static_for<NT>([&](auto mc) {
-            constexpr int m = decltype(mc)::value;
-            // LDS reads issued after those of fetch m
-            constexpr int last = (m + P < NT ? m + P : NT) - 1;
-            constexpr int k_after = (last < NQ ? last : NQ - 1) - (m < NQ ? m : NQ - 1);
-            constexpr int v_after = (last >= NQ ? last - NQ + 1 : 0) - (m >= NQ ? m - NQ + 1 : 0);
-            if constexpr (PREV && m == NQ) {
-                // between the two halves of the step: the accumulators move to the previous tile's maximum (which
-                // rarely changes after the first tiles: alpha is then exactly 1 in every lane) ...
-                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) acc[db] *= alpha;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if constexpr (CUR && m == NQ) {
-                // ... and tokens hidden from a column leave its scores
-                if (ts + PF_TOK > Lmask) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
-                        cur[i] = tok < Lcol ? cur[i] : PA_NEG;
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            wait_lds_reads<k_after + 2 * v_after>();
-            if constexpr (m < NQ) {
+
+        // ---- S^T[token, col] = K[token, :] . Q[col, :]
+        f32x16 sc;
+        {
+            u32x4 ka[P];
+            auto fetch = [&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                if constexpr (m < KS) ka[m % P] = lds_read16_at<OFF>(klane[m]);
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<(P < KS ? P : KS)>(fetch);
+            static_for<KS>([&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                constexpr int left = KS - 1 - m;
+                wait_lds_reads<(left < P - 1 ? left : P - 1)>();
                 if constexpr (m == 0) {
                     f32x16 z;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) z[e] = 0.f;
-                    cur = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], z);
+                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], z);
                 } else {
-                    cur = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], cur);
+                    sc = T::mfma32(bitcast<vec8>(ka[m % P]), qreg[m], sc);
                 }
-            } else {
-                constexpr int v = m - NQ, th = v / DB, db = v % DB;
-                const vec8 pf = bitcast<vec8>((u32x4){pp[4 * th], pp[4 * th + 1], pp[4 * th + 2], pp[4 * th + 3]});
-                acc[db] = T::mfma32(bitcast<vec8>((u32x4){lo[m % P][0], lo[m % P][1], hi[m % P][0], hi[m % P][1]}),
-                                    pf, acc[db]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(std::integral_constant<int, m + P>{});
+            });
+        }
+        if (ts + PF_TOK > Lmask) {                            // tokens hidden from a column leave its scores
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
+                sc[i] = tok < Lcol ? sc[i] : PA_NEG;
             }
-            __builtin_amdgcn_sched_barrier(0);
-            fetch(std::integral_constant<int, m + P>{});
-            if constexpr (PREV && m < NQ) {                   // exponentials of tile t - 1 beside the score MFMAs
-                constexpr int per = 8 / KS;
+        }
+        float tmax = sc[0];
 #pragma unroll
-                for (int k = m * per; k < (m + 1) * per; ++k) prob_pair(k);
-            }
-            if constexpr (CUR && m >= NQ) {                   // running maximum of tile t beside the PV MFMAs
-                constexpr int v = m - NQ;
-                constexpr int c_lo = v * 4 / NV, c_hi = (v + 1) * 4 / NV;
+        for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, sc[i]);
+        tmax = max_xor32(tmax);
+        const float m_new = tmax > m_run + lazy ? tmax : m_run;
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {      // the reference point moves: rare
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+            l_run *= alpha;
 #pragma unroll
-                for (int c = c_lo; c < c_hi; ++c) {
-                    if (c == 0) {
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) tmax = fmaxf(tmax, cur[i]);
-                    } else if (c == 1) {
-#pragma unroll
-                        for (int i = 8; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
-                        tmax = max_xor32(tmax);
-                    } else if (c == 2) {
-                        m_new = tmax > m_run + lazy ? tmax : m_run;
-                        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
-                    } else {
-                        m_run = m_new;
-                        nm = -m_new * scale_log2;
-                    }
-                    asm volatile("" : "+v"(tmax), "+v"(m_new), "+v"(alpha), "+v"(nm));   // computed here
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        if constexpr (PREV && !CUR) return;
-        if constexpr (CUR && !PREV) {
-            // first tile: no PV product to work beside
-            if (ts + PF_TOK > Lmask) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int tok = ts + 8 * (i >> 2) + 4 * h + (i & 3);
-                    cur[i] = tok < Lcol ? cur[i] : PA_NEG;
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
-            tmax = max_xor32(tmax);
-            m_new = tmax > m_run + lazy ? tmax : m_run;
-            alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+            for (int db = 0; db < DB; ++db) acc[db] *= alpha;
             m_run = m_new;
-            nm = -m_new * scale_log2;
+        }
+        const float nm = -m_run * scale_log2;
+        // probabilities, rounded to T; the denominator sums them as the PV product sees them
+        uint32_t pp[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[2 * k], scale_log2, nm));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[2 * k + 1], scale_log2, nm));
+            pp[k] = pack2<T>(p0, p1);
+            l_run = T::sum2(pp[k], l_run);
+        }
+        const vec8 pf0 = bitcast<vec8>((u32x4){pp[0], pp[1], pp[2], pp[3]});
+        const vec8 pf1 = bitcast<vec8>((u32x4){pp[4], pp[5], pp[6], pp[7]});
+
+        // ---- O^T[d, col] += V^T[d, token] . P^T[token, col]: MFMA v = DB th + db (token half th, d block db), two
+        // transposing reads each
+        {
+            u32x2 lo[P], hi[P];
+            auto fetch = [&](auto vc_) {
+                constexpr int v = decltype(vc_)::value;
+                if constexpr (v < NV) {
+                    constexpr int th = v / DB, db = v % DB;
+                    lo[v % P] = lds_read_tr16_at<OFF + 16 * th * ROWB>(vlane[db]);
+                    hi[v % P] = lds_read_tr16_at<OFF + (16 * th + 8) * ROWB>(vlane[db]);
+                }
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<(P < NV ? P : NV)>(fetch);
+            static_for<NV>([&](auto vc_) {
+                constexpr int v = decltype(vc_)::value;
+                constexpr int th = v / DB, db = v % DB;
+                constexpr int left = NV - 1 - v;
+                wait_lds_reads<2 * (left < P - 1 ? left : P - 1)>();
+                acc[db] = T::mfma32(bitcast<vec8>((u32x4){lo[v % P][0], lo[v % P][1], hi[v % P][0], hi[v % P][1]}),
+                                    th ? pf1 : pf0, acc[db]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(std::integral_constant<int, v + P>{});
+            });
         }
     };
 
@@ -874,7 +833,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
     if (ntiles > 1) issue_tile(1);
 #pragma unroll
     for (int j = 0; j < KS; ++j) asm volatile("" : "+v"(qreg[j]));   // the query is complete before the loop
-    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 2,
+    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 1,
     // whose buffer takes tile t + 2
     auto sync_issue = [&](int t) {
         __builtin_amdgcn_sched_barrier(0);
@@ -884,45 +843,25 @@ __global__ __launch_bounds__(PA_WAVES * 64, 2) void prefill_attention_kernel(
         __builtin_amdgcn_sched_barrier(0);
         if (t + 2 < ntiles) issue_tile(t + 2);
     };
-    constexpr std::true_type yes{};
-    constexpr std::false_type no{};
     constexpr std::integral_constant<int, 0> r0{};
     constexpr std::integral_constant<int, 1> r1{};
     constexpr std::integral_constant<int, 2> r2{};
-    constexpr std::integral_constant<int, 3> r3{};
-    // the scores alternate between two register sets: even tiles in sc_a, odd tiles in sc_b
-    sync_issue(0);
-    if (wave_live) step(0, r0, sc_a, sc_b, yes, no);
-    int t = 1;
+    int t = 0;
 #pragma unroll 1
-    for (; t + 3 < ntiles; t += 4) {
+    for (; t + 2 < ntiles; t += 3) {
         sync_issue(t);
-        if (wave_live) step(t, r1, sc_b, sc_a, yes, yes);
+        if (wave_live) step(t, r0);
         sync_issue(t + 1);
-        if (wave_live) step(t + 1, r2, sc_a, sc_b, yes, yes);
+        if (wave_live) step(t + 1, r1);
         sync_issue(t + 2);
-        if (wave_live) step(t + 2, r3, sc_b, sc_a, yes, yes);
-        sync_issue(t + 3);
-        if (wave_live) step(t + 3, r0, sc_a, sc_b, yes, yes);
+        if (wave_live) step(t + 2, r2);
     }
     if (t < ntiles) {
         sync_issue(t);
-        if (wave_live) step(t, r1, sc_b, sc_a, yes, yes);
+        if (wave_live) step(t, r0);
         if (++t < ntiles) {
             sync_issue(t);
-            if (wave_live) step(t, r2, sc_a, sc_b, yes, yes);
-            if (++t < ntiles) {
-                sync_issue(t);
-                if (wave_live) step(t, r3, sc_b, sc_a, yes, yes);
-            }
-        }
-    }
-    if (wave_live) {                                          // exponentials and PV product of the last tile
-        switch (ntiles & 3) {
-            case 0: step(ntiles, r0, sc_a, sc_b, no, yes); break;
-            case 1: step(ntiles, r1, sc_b, sc_a, no, yes); break;
-            case 2: step(ntiles, r2, sc_a, sc_b, no, yes); break;
-            default: step(ntiles, r3, sc_b, sc_a, no, yes); break;
+            if (wave_live) step(t, r1);
         }
     }
 
