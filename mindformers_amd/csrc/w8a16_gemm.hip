@@ -426,13 +426,11 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
         constexpr int SB = decltype(stagec)::value * C::STAGE;
         wr[P][0] = g2_lds_read16<SB>(woff);
         if constexpr (NT == 2) wr[P][1] = g2_lds_read16<SB + GW_TILE_BYTES>(woff);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            if (mt == 0) { xb[P][0][0] = g2_lds_read16<SB>(xoff0); xb[P][0][1] = g2_lds_read16<SB>(xoff1); }
-            if (mt == 1) { xb[P][1][0] = g2_lds_read16<SB + 2048>(xoff0); xb[P][1][1] = g2_lds_read16<SB + 2048>(xoff1); }
-            if (mt == 2) { xb[P][2][0] = g2_lds_read16<SB + 4096>(xoff0); xb[P][2][1] = g2_lds_read16<SB + 4096>(xoff1); }
-            if (mt == 3) { xb[P][3][0] = g2_lds_read16<SB + 6144>(xoff0); xb[P][3][1] = g2_lds_read16<SB + 6144>(xoff1); }
-        }
+        static_for<MT>([&](auto mc) {
+            constexpr int mt = decltype(mc)::value;
+            xb[P][mt][0] = g2_lds_read16<SB + 2048 * mt>(xoff0);
+            xb[P][mt][1] = g2_lds_read16<SB + 2048 * mt>(xoff1);
+        });
     };
     auto operands_arrived = [&](auto setc) {                  // all LDS reads issued so far have returned
         constexpr int P = decltype(setc)::value;
@@ -834,8 +832,8 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
         constexpr int lds = G2<MTV, G2_NT>::LDS_BYTES;                                                            \
         static bool configured[MF_MAX_DEVICES] = {};                                                              \
         int dev = 0;                                                                                             \
-        hipGetDevice(&dev);                                                                                      \
-        if (dev < 0 || dev >= MF_MAX_DEVICES) return (int)hipErrorInvalidDevice;                                  \
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MF_MAX_DEVICES)                                \
+            return (int)hipErrorInvalidDevice;                                                                   \
         if (!configured[dev]) {                                                                                  \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
             if (e != hipSuccess) return (int)e;                                                                  \

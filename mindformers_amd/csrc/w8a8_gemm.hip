@@ -206,17 +206,10 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(
         xb[1] = q2_lds_read16<SB + 1024>(xoff);
         xb[2] = q2_lds_read16<SB + 2048>(xoff);
         xb[3] = q2_lds_read16<SB + 3072>(xoff);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            if (nt == 0) wa[0] = q2_lds_read16<SB>(woff);
-            if (nt == 1) wa[1] = q2_lds_read16<SB + 1 * Q_TILE>(woff);
-            if (nt == 2) wa[2] = q2_lds_read16<SB + 2 * Q_TILE>(woff);
-            if (nt == 3) wa[3] = q2_lds_read16<SB + 3 * Q_TILE>(woff);
-            if (nt == 4) wa[4] = q2_lds_read16<SB + 4 * Q_TILE>(woff);
-            if (nt == 5) wa[5] = q2_lds_read16<SB + 5 * Q_TILE>(woff);
-            if (nt == 6) wa[6] = q2_lds_read16<SB + 6 * Q_TILE>(woff);
-            if (nt == 7) wa[7] = q2_lds_read16<SB + 7 * Q_TILE>(woff);
-        }
+        static_for<NT>([&](auto nc) {
+            constexpr int nt = decltype(nc)::value;
+            wa[nt] = q2_lds_read16<SB + nt * Q_TILE>(woff);
+        });
         // the reads return in order: the activation tiles and the first weight tile are enough to start
         asm volatile("s_waitcnt lgkmcnt(%5)"
                      : "+v"(xb[0]), "+v"(xb[1]), "+v"(xb[2]), "+v"(xb[3]), "+v"(wa[0])
@@ -709,8 +702,8 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
         constexpr int lds = Q2<NTV, MS, STV>::LDS_BYTES;                                                          \
         static bool configured[MF_MAX_DEVICES] = {};                                                              \
         int dev = 0;                                                                                             \
-        hipGetDevice(&dev);                                                                                      \
-        if (dev < 0 || dev >= MF_MAX_DEVICES) return (int)hipErrorInvalidDevice;                                  \
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MF_MAX_DEVICES)                                \
+            return (int)hipErrorInvalidDevice;                                                                   \
         if (!configured[dev]) {                                                                                  \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
             if (e != hipSuccess) return (int)e;                                                                  \
