@@ -267,6 +267,22 @@ int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const f
 int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m, int k,
                                int dtype, int layout, void* stream);
 
+/* RMSNorm (optionally with the residual add in front, as mf_rmsnorm) whose only reader is a per-token quantised
+ * projection, fused with that quantisation: the norm output is not written, xq / x_scale are what
+ * mf_dynamic_quant_per_token(layout) gives for it.  Bit-identical to mf_rmsnorm followed by
+ * mf_dynamic_quant_per_token (P.RmsNorm, llama_layer.py:195,225-228, in front of the golden-stick DynamicQuant of
+ * the W8A8 qkv and gate/up projections). */
+int mf_rmsnorm_dynamic_quant(int8_t* xq, float* x_scale, void* sum_out, const void* x, const void* residual,
+                             const void* gamma, const float* smooth, float eps, int rows, int cols, int dtype,
+                             int gamma_dtype, int layout, void* stream);
+
+/* act(gate) * up (as mf_silu_mul, gate_up_layout 0 = halves, 1 = interleaved) whose only reader is the per-token
+ * quantised down projection, fused with that quantisation: the product is not written.  Bit-identical to
+ * mf_silu_mul followed by mf_dynamic_quant_per_token (mlp.py:135-140 in front of the golden-stick DynamicQuant of
+ * the W8A8 down projection).  cols = width of the product, at most 24576. */
+int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows, int cols,
+                              int gate_up_layout, int dtype, int layout, void* stream);
+
 /* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
  * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
  * xq int8 [M,K]: row-major (x_layout 0) or tiled (x_layout 1), as mf_dynamic_quant_per_token writes it; the tiled

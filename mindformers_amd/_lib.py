@@ -46,6 +46,8 @@ SIGNATURES = {
     "mf_w8a16_qkv_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm_silu_mul": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_dynamic_quant_per_token": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mf_rmsnorm_dynamic_quant": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P]),
+    "mf_silu_mul_dynamic_quant": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mf_w8a8_workspace_bytes": (_Z, [_I, _I, _I]),
     "mf_w8a8_gemm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_moe_route": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),

@@ -135,8 +135,43 @@ __global__ void add_kernel(uint16_t* __restrict__ out, const uint16_t* __restric
         out[i] = T::from_float(T::to_float(a[i]) + T::to_float(b[i]));
 }
 
+// 8 values of row m, columns k .. k+7, quantised with the row's scale and written in the chosen layout.
+// The division is a true IEEE division so that the grid point chosen equals the CPU statement.
+__device__ __forceinline__ void quant_store8(int8_t* __restrict__ xq, const float* v, float safe, int m, int k, int cols,
+                                             int rows, int tiled) {
+    uint32_t o[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float qf = rintf(__fdiv_rn(v[i], safe));
+        qf = fminf(fmaxf(qf, -128.f), 127.f);
+        o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
+    }
+    if (tiled) {
+        // 1 KiB tiles of 16 rows x 64 columns, [column step][row tile], 16 consecutive columns per lane
+        // (lane = 16*(column/16 % 4) + row % 16): the operand order of the int8 matrix instructions
+        const int64_t tile = (int64_t)(k >> 6) * ((rows + 15) >> 4) + (m >> 4);
+        *(u32x2*)(xq + tile * 1024 + ((((k & 63) >> 4) << 4) + (m & 15)) * 16 + (k & 15)) = (u32x2){o[0], o[1]};
+    } else {
+        *(u32x2*)(xq + (int64_t)m * cols + k) = (u32x2){o[0], o[1]};
+    }
+}
+// x * smooth in place (smooth may be null), returns max |.| of the 8 values
+__device__ __forceinline__ float smooth_absmax8(float* v, const float* __restrict__ smooth, int k) {
+    if (smooth) {
+        const f32x4 s0 = *(const f32x4*)(smooth + k), s1 = *(const f32x4*)(smooth + k + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = __fmul_rn(v[i], s0[i]);
+            v[4 + i] = __fmul_rn(v[4 + i], s1[i]);
+        }
+    }
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a = fmaxf(a, fabsf(v[i]));
+    return a;
+}
+
 // Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
-// The division xs/s is a true IEEE division so that the grid point chosen equals the CPU statement.
 template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq,
                                                                    float* __restrict__ x_scale,
@@ -154,16 +189,7 @@ __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __re
         const int c = threadIdx.x + it * ROW_THREADS;
         if (c < nvec) {
             unpack8<T>(*(const u32x4*)(x + row + 8 * c), v[it]);
-            if (smooth) {
-                const f32x4 s0 = *(const f32x4*)(smooth + 8 * c), s1 = *(const f32x4*)(smooth + 8 * c + 4);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    v[it][i] = __fmul_rn(v[it][i], s0[i]);
-                    v[it][4 + i] = __fmul_rn(v[it][4 + i], s1[i]);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[it][i]));
+            amax = fmaxf(amax, smooth_absmax8(v[it], smooth, 8 * c));
         }
     }
     amax = block_max(amax, red);
@@ -173,24 +199,123 @@ __global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __re
 #pragma unroll
     for (int it = 0; it < MAXV; ++it) {
         const int c = threadIdx.x + it * ROW_THREADS;
-        if (c < nvec) {
-            uint32_t o[2] = {0u, 0u};
+        if (c < nvec) quant_store8(xq, v[it], safe, blockIdx.x, 8 * c, cols, gridDim.x, tiled);
+    }
+}
+
+// RMSNorm (optionally with the residual add before it) followed by the per-token quantisation of its output, which
+// is not written: the quantised GEMM is its only reader.  Rounding points as the two kernels have them: the sum, and
+// the normalised value, are rounded to T before they are used further.
+template <typename T>
+__global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
+    int8_t* __restrict__ xq, float* __restrict__ x_scale, uint16_t* __restrict__ sum_out,
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const void* __restrict__ gamma,
+    const float* __restrict__ smooth, float eps, int cols, int gamma_dtype, int tiled) {
+    __shared__ float red[NORM_THREADS / 64];
+    const int64_t row = (int64_t)blockIdx.x * cols;
+    const int nvec = cols >> 3;
+    float v[NORM_MAX_VEC][8], gm[NORM_MAX_VEC][8];
+    float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float qf = rintf(__fdiv_rn(v[it][i], safe));
-                qf = fminf(fmaxf(qf, -128.f), 127.f);
-                o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
+    for (int it = 0; it < NORM_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * NORM_THREADS;
+        if (c < nvec) {
+            u32x4 raw = *(const u32x4*)(x + row + 8 * c);
+            u32x4 rraw;
+            if (residual) rraw = *(const u32x4*)(residual + row + 8 * c);
+            load8_as_float(gamma, 8 * c, gamma_dtype, gm[it]);
+            unpack8<T>(raw, v[it]);
+            if (residual) {
+                float rr[8];
+                unpack8<T>(rraw, rr);
+                u32x4 sm;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sm[i] = pack2<T>(v[it][2 * i] + rr[2 * i], v[it][2 * i + 1] + rr[2 * i + 1]);
+                *(u32x4*)(sum_out + row + 8 * c) = sm;
+                unpack8<T>(sm, v[it]);
             }
-            if (tiled) {
-                // 1 KiB tiles of 16 rows x 64 columns, [column step][row tile], 16 consecutive columns per lane
-                // (lane = 16*(column/16 % 4) + row % 16): the operand order of the int8 matrix instructions
-                const int m = blockIdx.x, k = 8 * c;
-                const int64_t tile = (int64_t)(k >> 6) * ((gridDim.x + 15) >> 4) + (m >> 4);
-                *(u32x2*)(xq + tile * 1024 + ((((k & 63) >> 4) << 4) + (m & 15)) * 16 + (k & 15)) = (u32x2){o[0], o[1]};
-            } else {
-                *(u32x2*)(xq + row + 8 * c) = (u32x2){o[0], o[1]};
-            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[it][i], v[it][i], ss);
         }
+    }
+    ss = rmsnorm_block_sum<NORM_THREADS>(ss, red);
+    const float inv = rsqrtf(ss / (float)cols + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int it = 0; it < NORM_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * NORM_THREADS;
+        if (c < nvec) {
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                o[i] = pack2<T>(v[it][2 * i] * inv * gm[it][2 * i], v[it][2 * i + 1] * inv * gm[it][2 * i + 1]);
+            unpack8<T>(o, v[it]);                              // the rounded norm output, as the next kernel would read it
+            amax = fmaxf(amax, smooth_absmax8(v[it], smooth, 8 * c));
+        }
+    }
+    amax = block_max(amax, red);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float safe = s > 0.f ? s : 1.0f;
+    if (threadIdx.x == 0) x_scale[blockIdx.x] = s;
+#pragma unroll
+    for (int it = 0; it < NORM_MAX_VEC; ++it) {
+        const int c = threadIdx.x + it * NORM_THREADS;
+        if (c < nvec) quant_store8(xq, v[it], safe, blockIdx.x, 8 * c, cols, gridDim.x, tiled);
+    }
+}
+
+// act(gate) * up followed by the per-token quantisation of the product, which is not written.  One workgroup per
+// row; rounding points as silu_mul_kernel has them.
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void silu_mul_quant_kernel(int8_t* __restrict__ xq,
+                                                                    float* __restrict__ x_scale,
+                                                                    const uint16_t* __restrict__ gu,
+                                                                    const float* __restrict__ smooth, int cols,
+                                                                    int layout, int tiled) {
+    __shared__ float red[ROW_THREADS / 64];
+    const int nvec = cols >> 3;
+    constexpr int MAXV = 12;                                  // cols <= 256*12*8 = 24576
+    float v[MAXV][8];
+    float amax = 0.f;
+    const uint16_t* base = gu + (int64_t)blockIdx.x * 2 * cols;
+#pragma unroll
+    for (int it = 0; it < MAXV; ++it) {
+        const int cv = threadIdx.x + it * ROW_THREADS;
+        if (cv < nvec) {
+            const int c = 8 * cv;
+            float g[8], u[8];
+            if (layout == 0) {
+                unpack8<T>(*(const u32x4*)(base + c), g);
+                unpack8<T>(*(const u32x4*)(base + cols + c), u);
+            } else {
+                float a[8], b[8];
+                unpack8<T>(*(const u32x4*)(base + 2 * c), a);
+                unpack8<T>(*(const u32x4*)(base + 2 * c + 8), b);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    g[j] = a[2 * j]; u[j] = a[2 * j + 1];
+                    g[4 + j] = b[2 * j]; u[4 + j] = b[2 * j + 1];
+                }
+            }
+            u32x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a0 = T::to_float(T::from_float(silu_f(g[2 * j])));
+                const float a1 = T::to_float(T::from_float(silu_f(g[2 * j + 1])));
+                o[j] = pack2<T>(a0 * u[2 * j], a1 * u[2 * j + 1]);
+            }
+            unpack8<T>(o, v[it]);                              // the rounded product, as the next kernel would read it
+            amax = fmaxf(amax, smooth_absmax8(v[it], smooth, c));
+        }
+    }
+    amax = block_max(amax, red);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float safe = s > 0.f ? s : 1.0f;
+    if (threadIdx.x == 0) x_scale[blockIdx.x] = s;
+#pragma unroll
+    for (int it = 0; it < MAXV; ++it) {
+        const int cv = threadIdx.x + it * ROW_THREADS;
+        if (cv < nvec) quant_store8(xq, v[it], safe, blockIdx.x, 8 * cv, cols, gridDim.x, tiled);
     }
 }
 
@@ -272,5 +397,53 @@ extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void
     else
         hipLaunchKernelGGL(dynamic_quant_kernel<FP16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
                            (const uint16_t*)x, smooth, k, layout);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_rmsnorm_dynamic_quant(int8_t* xq, float* x_scale, void* sum_out, const void* x, const void* residual,
+                                        const void* gamma, const float* smooth, float eps, int rows, int cols,
+                                        int dtype, int gamma_dtype, int layout, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rmsnorm_dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32,
+               "rmsnorm_dynamic_quant: bad gamma dtype");
+    MF_REQUIRE(layout == 0 || layout == 1, "rmsnorm_dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
+    if (rows <= 0) return 0;
+    MF_REQUIRE(xq && x_scale && x && gamma, "rmsnorm_dynamic_quant: null argument");
+    MF_REQUIRE(!residual || sum_out, "rmsnorm_dynamic_quant: residual given without sum_out");
+    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= NORM_THREADS * NORM_MAX_VEC * 8,
+               "rmsnorm_dynamic_quant: cols (%d) must be a multiple of 8 and at most %d", cols,
+               NORM_THREADS * NORM_MAX_VEC * 8);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out | (uintptr_t)gamma | (uintptr_t)smooth) & 15) == 0 &&
+                   ((uintptr_t)xq & 7) == 0,
+               "rmsnorm_dynamic_quant: pointers must be 16-byte aligned, xq 8-byte aligned");
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(rmsnorm_quant_kernel<BF16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps, cols,
+                           gamma_dtype, layout);
+    else
+        hipLaunchKernelGGL(rmsnorm_quant_kernel<FP16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps, cols,
+                           gamma_dtype, layout);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows,
+                                         int cols, int gate_up_layout, int dtype, int layout, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "silu_mul_dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(gate_up_layout == 0 || gate_up_layout == 1,
+               "silu_mul_dynamic_quant: gate_up_layout must be 0 (halves) or 1 (interleaved)");
+    MF_REQUIRE(layout == 0 || layout == 1, "silu_mul_dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
+    if (rows <= 0) return 0;
+    MF_REQUIRE(xq && x_scale && gate_up, "silu_mul_dynamic_quant: null argument");
+    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * 12 * 8,
+               "silu_mul_dynamic_quant: cols (%d) must be a multiple of 8, <= %d", cols, ROW_THREADS * 12 * 8);
+    MF_REQUIRE((((uintptr_t)gate_up | (uintptr_t)smooth) & 15) == 0 && ((uintptr_t)xq & 7) == 0,
+               "silu_mul_dynamic_quant: gate_up/smooth must be 16-byte aligned, xq 8-byte aligned");
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(silu_mul_quant_kernel<BF16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout);
+    else
+        hipLaunchKernelGGL(silu_mul_quant_kernel<FP16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
+                           (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout);
     return MF_LAUNCH_CHECK();
 }

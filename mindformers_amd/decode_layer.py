@@ -49,13 +49,14 @@ class QuantDecodeLayer(nn.Module):
         self.register_buffer("attn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
         self.register_buffer("ffn_norm", torch.ones(hidden, dtype=torch.float32, device=device))
 
-    def _linear(self, x, name, residual=None):
+    def _linear(self, x, name, residual=None, quantized=None):
+        """``quantized``: (xq, scale) when the producer of x already quantised it (W8A8 only)."""
         b = getattr(self, f"{name}_b")
         packed = self._packed.get(name)
         if packed is None:
             raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
         if self.act_quant:
-            xq, xs = ops.dynamic_quant(x, getattr(self, f"{name}_smooth"), tiled=True)
+            xq, xs = quantized or ops.dynamic_quant(x, getattr(self, f"{name}_smooth"), tiled=True)
             return ops.w8a8_linear(xq, xs, packed, out_dtype=self.dtype, bias=b, residual=residual)
         return ops.w8a16_linear(x, packed, bias=b, residual=residual)
 
@@ -98,16 +99,19 @@ class QuantDecodeLayer(nn.Module):
         Prefill / chunked prefill: ``q_starts`` int32 [B + 1] gives the row range of every sequence in x, its new
         tokens are scattered first and then attend causally over the cache."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
-        n1 = ops.rms_norm(x, self.attn_norm, self.eps)
+        if self.act_quant:                                    # W8A8: the norm feeds the quantised projection only
+            n1, n1q = None, ops.rms_norm_dynamic_quant(x, self.attn_norm, self.eps, self.qkv_smooth, tiled=True)
+        else:
+            n1, n1q = ops.rms_norm(x, self.attn_norm, self.eps), None
         if key_cache.dtype == torch.int8:                     # rotate, then quantize into the int8 caches
             if self.kv_scale is None:
                 raise RuntimeError("int8 caches need set_kv_quant(scale, offset)")
-            qkv = self._linear(n1, "qkv")
+            qkv = self._linear(n1, "qkv", quantized=n1q)
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
             ops.apply_rotary_pos_emb(q, k, cos, sin, self.n_head, self.n_kv_head, self.head_dim)
             ops.quant_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, self.kv_scale, self.kv_offset)
         elif self.act_quant or self.head_dim % 16:
-            qkv = self._linear(n1, "qkv")
+            qkv = self._linear(n1, "qkv", quantized=n1q)
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
             ops.rope_and_cache(q, k, v, cos, sin, key_cache, value_cache, slot_mapping, self.n_head)
         else:                                                 # W8A16: projection + RoPE + cache write in one call
@@ -116,7 +120,12 @@ class QuantDecodeLayer(nn.Module):
             q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
                                              self.n_head, bias=self.qkv_b)
         attn = self.attend(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts)
-        if self.act_quant or self.wo_b is not None:
+        if self.act_quant:                                    # W8A8: norm + quantisation, gate/up, act + quantisation
+            h = self._linear(attn, "wo", residual=x)
+            n2q = ops.rms_norm_dynamic_quant(h, self.ffn_norm, self.eps, self.fc1_smooth, tiled=True)
+            actq = ops.silu_mul_dynamic_quant(self._linear(None, "fc1", quantized=n2q), self.fc2_smooth, tiled=True)
+            return self._linear(None, "fc2", residual=h, quantized=actq)
+        if self.wo_b is not None:
             h = self._linear(attn, "wo", residual=x)
             n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
         else:                                                 # W8A16: projection + residual + norm in one call

@@ -606,6 +606,53 @@ def dynamic_quant(x, smooth=None, tiled=False):
     return (TiledInt8Activations(xq, x.shape) if tiled else xq), xs
 
 
+def _quant_out(lib, shape, m, k, tiled, dev):
+    if tiled:
+        xq = torch.empty(lib.mf_w8a16_packed_bytes(max(m, 1), k), dtype=torch.int8, device=dev)
+    else:
+        xq = torch.empty(shape, dtype=torch.int8, device=dev)
+    return xq, torch.empty(m, dtype=torch.float32, device=dev)
+
+
+def rms_norm_dynamic_quant(x, gamma, eps, smooth=None, residual=None, tiled=False):
+    """RmsNorm followed by DynamicQuant per token in one kernel (the norm output itself is not materialised).
+    Returns (xq, scale), with ``residual`` also x + residual: bit-identical to rms_norm then dynamic_quant."""
+    lib = _lib.load()
+    dev = _dev_ok(x, gamma, residual, smooth)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    k = x.shape[-1]
+    m = x.numel() // k
+    _need(gamma.numel() == k, "gamma size")
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [K]")
+    s = None
+    if residual is not None:
+        _need(residual.shape == x.shape and residual.dtype == x.dtype, "residual mismatch")
+        s = torch.empty_like(x)
+    xq, xs = _quant_out(lib, x.shape, m, k, tiled, dev)
+    check(lib.mf_rmsnorm_dynamic_quant(ptr(xq), ptr(xs), ptr(s), ptr(x), ptr(residual), ptr(gamma), ptr(smooth),
+                                       float(eps), m, k, dtype_code(x.dtype), dtype_code(gamma.dtype),
+                                       1 if tiled else 0, stream_ptr(dev)), "mf_rmsnorm_dynamic_quant")
+    xq = TiledInt8Activations(xq, x.shape) if tiled else xq
+    return (xq, xs, s) if residual is not None else (xq, xs)
+
+
+def silu_mul_dynamic_quant(gate_up, smooth=None, interleaved=False, tiled=False):
+    """silu(gate) * up followed by DynamicQuant per token in one kernel (the product is not materialised): returns
+    (xq, scale), bit-identical to silu_mul then dynamic_quant."""
+    lib = _lib.load()
+    dev = _dev_ok(gate_up, smooth)
+    _need(gate_up.dtype in _ACT and gate_up.shape[-1] % 2 == 0, "gate_up must be bf16/fp16 with an even last dim")
+    k = gate_up.shape[-1] // 2
+    m = gate_up.numel() // (2 * k)
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [F]")
+    shape = (*gate_up.shape[:-1], k)
+    xq, xs = _quant_out(lib, shape, m, k, tiled, dev)
+    check(lib.mf_silu_mul_dynamic_quant(ptr(xq), ptr(xs), ptr(gate_up), ptr(smooth), m, k, 1 if interleaved else 0,
+                                        dtype_code(gate_up.dtype), 1 if tiled else 0, stream_ptr(dev)),
+          "mf_silu_mul_dynamic_quant")
+    return (TiledInt8Activations(xq, shape) if tiled else xq), xs
+
+
 def w8a8_linear(xq, x_scale, w, w_scale=None, out_dtype=torch.bfloat16, bias=None, residual=None, return_acc=False):
     """QuantBatchMatmul: int8 x int8 -> int32 -> * x_scale * w_scale (+bias) (+residual) -> out_dtype.  ``w`` is a
     PackedInt8Weight (the fast path) or a raw int8 [N, K] tensor with ``w_scale`` (packed on every call); ``xq`` is

@@ -797,6 +797,50 @@ def test_dynamic_quant_tiled_layout_bit_exact(m, k):
     assert np.array_equal(_untile_int8(to_np(xt.data), m, k), q_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,smooth,residual,tiled", [(256, 3584, True, False, True), (5, 512, False, True, False),
+                                                       (33, 16384, True, True, True), (1, 64, True, False, False)])
+def test_rms_norm_dynamic_quant_equals_unfused(dtype, m, k, smooth, residual, tiled):
+    """RMSNorm + per-token quantisation in one kernel: bit-identical to the two kernels in sequence."""
+    rng = np.random.default_rng(m + k)
+    x = dev(rounded(rng.normal(size=(m, k)), dtype), dtype)
+    r = dev(rounded(rng.normal(size=(m, k)), dtype), dtype) if residual else None
+    g = torch.from_numpy(rng.uniform(0.5, 1.5, k).astype(np.float32)).cuda()
+    sm = torch.from_numpy(rng.uniform(0.5, 2.0, k).astype(np.float32)).cuda() if smooth else None
+    if residual:
+        n, h = ops.rms_norm(x, g, 1e-6, residual=r)
+        fq, fs, fh = ops.rms_norm_dynamic_quant(x, g, 1e-6, sm, residual=r, tiled=tiled)
+        assert torch.equal(fh, h)
+    else:
+        n = ops.rms_norm(x, g, 1e-6)
+        fq, fs = ops.rms_norm_dynamic_quant(x, g, 1e-6, sm, tiled=tiled)
+    uq, us = ops.dynamic_quant(n, sm, tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(fs, us)
+    if tiled:
+        assert np.array_equal(_untile_int8(to_np(fq.data), m, k), _untile_int8(to_np(uq.data), m, k))
+    else:
+        assert torch.equal(fq, uq)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,f,smooth,interleaved,tiled", [(256, 18944, True, False, True), (7, 688, False, True, False),
+                                                          (64, 24576, True, True, True), (1, 64, False, False, False)])
+def test_silu_mul_dynamic_quant_equals_unfused(dtype, m, f, smooth, interleaved, tiled):
+    """SiLU(gate) * up + per-token quantisation in one kernel: bit-identical to the two kernels in sequence."""
+    rng = np.random.default_rng(m + f)
+    gu = dev(rounded(rng.normal(size=(m, 2 * f)) * 2, dtype), dtype)
+    sm = torch.from_numpy(rng.uniform(0.5, 2.0, f).astype(np.float32)).cuda() if smooth else None
+    uq, us = ops.dynamic_quant(ops.silu_mul(gu, interleaved=interleaved), sm, tiled=tiled)
+    fq, fs = ops.silu_mul_dynamic_quant(gu, sm, interleaved=interleaved, tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(fs, us)
+    if tiled:
+        assert np.array_equal(_untile_int8(to_np(fq.data), m, f), _untile_int8(to_np(uq.data), m, f))
+    else:
+        assert torch.equal(fq, uq)
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16),
                                    (33, 130, 2064), (1, 64, 64), (300, 16500, 208), (130, 16384, 80)])
 def test_w8a8_tiled_activations_bit_exact(m, n, k):
