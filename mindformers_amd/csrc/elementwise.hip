@@ -6,7 +6,9 @@
 
 namespace {
 
-constexpr int ROW_THREADS = 256;
+constexpr int ROW_THREADS = 256;   // per-token quantisation: threads per row for narrow rows ...
+constexpr int ROW_THREADS_WIDE = 1024;   // ... and for wide ones (one workgroup per row either way: more waves in flight)
+constexpr int ROW_MAX_COLS = 24576;
 constexpr int NORM_THREADS = 512;  // RMSNorm: the geometry (and summation order) shared with the GEMM-fused norm
 constexpr int NORM_MAX_VEC = 4;    // up to 4 x (8 elements) per thread: cols <= 512*4*8 = 16384
 
@@ -172,16 +174,15 @@ __device__ __forceinline__ float smooth_absmax8(float* v, const float* __restric
 }
 
 // Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
-template <typename T>
-__global__ __launch_bounds__(ROW_THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq,
-                                                                   float* __restrict__ x_scale,
-                                                                   const uint16_t* __restrict__ x,
-                                                                   const float* __restrict__ smooth, int cols,
-                                                                   int tiled) {
-    __shared__ float red[ROW_THREADS / 64];
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq, float* __restrict__ x_scale,
+                                                               const uint16_t* __restrict__ x,
+                                                               const float* __restrict__ smooth, int cols, int tiled) {
+    __shared__ float red[THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
-    constexpr int MAXV = 12;                                  // cols <= 256*12*8 = 24576
+    constexpr int ROW_THREADS = THREADS;
+    constexpr int MAXV = ROW_MAX_COLS / 8 / THREADS;
     float v[MAXV][8];
     float amax = 0.f;
 #pragma unroll
@@ -266,15 +267,15 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
 
 // act(gate) * up followed by the per-token quantisation of the product, which is not written.  One workgroup per
 // row; rounding points as silu_mul_kernel has them.
-template <typename T>
-__global__ __launch_bounds__(ROW_THREADS) void silu_mul_quant_kernel(int8_t* __restrict__ xq,
-                                                                    float* __restrict__ x_scale,
-                                                                    const uint16_t* __restrict__ gu,
-                                                                    const float* __restrict__ smooth, int cols,
-                                                                    int layout, int tiled) {
-    __shared__ float red[ROW_THREADS / 64];
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void silu_mul_quant_kernel(int8_t* __restrict__ xq, float* __restrict__ x_scale,
+                                                                const uint16_t* __restrict__ gu,
+                                                                const float* __restrict__ smooth, int cols, int layout,
+                                                                int tiled) {
+    __shared__ float red[THREADS / 64];
     const int nvec = cols >> 3;
-    constexpr int MAXV = 12;                                  // cols <= 256*12*8 = 24576
+    constexpr int ROW_THREADS = THREADS;
+    constexpr int MAXV = ROW_MAX_COLS / 8 / THREADS;
     float v[MAXV][8];
     float amax = 0.f;
     const uint16_t* base = gu + (int64_t)blockIdx.x * 2 * cols;
@@ -386,17 +387,21 @@ extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void
     MF_REQUIRE(layout == 0 || layout == 1, "dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
     if (m <= 0) return 0;
     MF_REQUIRE(xq && x_scale && x, "dynamic_quant: null argument");
-    MF_REQUIRE(k > 0 && k % 8 == 0 && k <= ROW_THREADS * 12 * 8, "dynamic_quant: k (%d) must be a multiple of 8, <= %d",
-               k, ROW_THREADS * 12 * 8);
+    MF_REQUIRE(k > 0 && k % 8 == 0 && k <= ROW_MAX_COLS, "dynamic_quant: k (%d) must be a multiple of 8, <= %d", k,
+               ROW_MAX_COLS);
     MF_REQUIRE((((uintptr_t)xq & 7) | ((uintptr_t)x & 15) | ((uintptr_t)smooth & 15)) == 0,
                "dynamic_quant: x/smooth must be 16-byte aligned, xq 8-byte aligned");
     if (m <= 0) return 0;
-    if (dtype == MF_BF16)
-        hipLaunchKernelGGL(dynamic_quant_kernel<BF16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)x, smooth, k, layout);
-    else
-        hipLaunchKernelGGL(dynamic_quant_kernel<FP16>, dim3(m), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)x, smooth, k, layout);
+#define DQ_LAUNCH(TT, TH)                                                                                        \
+    hipLaunchKernelGGL((dynamic_quant_kernel<TT, TH>), dim3(m), dim3(TH), 0, (hipStream_t)stream, xq, x_scale,    \
+                       (const uint16_t*)x, smooth, k, layout)
+    const bool wide = k > 4096;
+    if (dtype == MF_BF16) {
+        if (wide) DQ_LAUNCH(BF16, ROW_THREADS_WIDE); else DQ_LAUNCH(BF16, ROW_THREADS);
+    } else {
+        if (wide) DQ_LAUNCH(FP16, ROW_THREADS_WIDE); else DQ_LAUNCH(FP16, ROW_THREADS);
+    }
+#undef DQ_LAUNCH
     return MF_LAUNCH_CHECK();
 }
 
@@ -435,15 +440,19 @@ extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void*
     MF_REQUIRE(layout == 0 || layout == 1, "silu_mul_dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
     if (rows <= 0) return 0;
     MF_REQUIRE(xq && x_scale && gate_up, "silu_mul_dynamic_quant: null argument");
-    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_THREADS * 12 * 8,
-               "silu_mul_dynamic_quant: cols (%d) must be a multiple of 8, <= %d", cols, ROW_THREADS * 12 * 8);
+    MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= ROW_MAX_COLS,
+               "silu_mul_dynamic_quant: cols (%d) must be a multiple of 8, <= %d", cols, ROW_MAX_COLS);
     MF_REQUIRE((((uintptr_t)gate_up | (uintptr_t)smooth) & 15) == 0 && ((uintptr_t)xq & 7) == 0,
                "silu_mul_dynamic_quant: gate_up/smooth must be 16-byte aligned, xq 8-byte aligned");
-    if (dtype == MF_BF16)
-        hipLaunchKernelGGL(silu_mul_quant_kernel<BF16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout);
-    else
-        hipLaunchKernelGGL(silu_mul_quant_kernel<FP16>, dim3(rows), dim3(ROW_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout);
+#define SQ_LAUNCH(TT, TH)                                                                                        \
+    hipLaunchKernelGGL((silu_mul_quant_kernel<TT, TH>), dim3(rows), dim3(TH), 0, (hipStream_t)stream, xq, x_scale, \
+                       (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout)
+    const bool wide = cols > 4096;
+    if (dtype == MF_BF16) {
+        if (wide) SQ_LAUNCH(BF16, ROW_THREADS_WIDE); else SQ_LAUNCH(BF16, ROW_THREADS);
+    } else {
+        if (wide) SQ_LAUNCH(FP16, ROW_THREADS_WIDE); else SQ_LAUNCH(FP16, ROW_THREADS);
+    }
+#undef SQ_LAUNCH
     return MF_LAUNCH_CHECK();
 }
