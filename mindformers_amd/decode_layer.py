@@ -93,16 +93,24 @@ class QuantDecodeLayer(nn.Module):
                                            self.n_head, self.n_kv_head, self.scale_value)
 
     def forward(self, x, key_cache, value_cache, block_tables, batch_valid_length, slot_mapping, cos, sin,
-                q_starts=None):
+                q_starts=None, normed=None, next_norm=None):
         """x [T, hidden]; caches [num_blocks, block_size, n_kv, D]; cos/sin [T, D] rows for this step's
         positions; batch_valid_length counts the tokens written by this step.  Decode: one token per sequence.
         Prefill / chunked prefill: ``q_starts`` int32 [B + 1] gives the row range of every sequence in x, its new
-        tokens are scattered first and then attend causally over the cache."""
+        tokens are scattered first and then attend causally over the cache.
+
+        Chaining layers: with ``next_norm`` = (gamma, eps) of the norm that follows this layer (the next layer's
+        attention norm, or the model's final norm) the call returns (out, norm(out) * gamma), and the next layer
+        takes that second tensor as ``normed`` in place of computing its attention norm.  On the W8A16 path the norm
+        then runs inside the kernel that finishes this layer's last projection (same bits, one launch fewer)."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
         if self.act_quant:                                    # W8A8: the norm feeds the quantised projection only
-            n1, n1q = None, ops.rms_norm_dynamic_quant(x, self.attn_norm, self.eps, self.qkv_smooth, tiled=True)
+            if normed is not None:
+                n1, n1q = None, ops.dynamic_quant(normed, self.qkv_smooth, tiled=True)
+            else:
+                n1, n1q = None, ops.rms_norm_dynamic_quant(x, self.attn_norm, self.eps, self.qkv_smooth, tiled=True)
         else:
-            n1, n1q = ops.rms_norm(x, self.attn_norm, self.eps), None
+            n1, n1q = (normed if normed is not None else ops.rms_norm(x, self.attn_norm, self.eps)), None
         if key_cache.dtype == torch.int8:                     # rotate, then quantize into the int8 caches
             if self.kv_scale is None:
                 raise RuntimeError("int8 caches need set_kv_quant(scale, offset)")
@@ -124,7 +132,7 @@ class QuantDecodeLayer(nn.Module):
             h = self._linear(attn, "wo", residual=x)
             n2q = ops.rms_norm_dynamic_quant(h, self.ffn_norm, self.eps, self.fc1_smooth, tiled=True)
             actq = ops.silu_mul_dynamic_quant(self._linear(None, "fc1", quantized=n2q), self.fc2_smooth, tiled=True)
-            return self._linear(None, "fc2", residual=h, quantized=actq)
+            return self._chain(self._linear(None, "fc2", residual=h, quantized=actq), next_norm)
         if self.wo_b is not None:
             h = self._linear(attn, "wo", residual=x)
             n2 = ops.rms_norm(h, self.ffn_norm, self.eps)
@@ -132,7 +140,13 @@ class QuantDecodeLayer(nn.Module):
             if self._packed.get("wo") is None:
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
             h, n2 = ops.w8a16_linear_add_rmsnorm(attn, self._packed["wo"], x, self.ffn_norm, self.eps)
-        return self._linear(self.gate_up(n2), "fc2", residual=h)
+        if next_norm is not None and self.fc2_b is None and self._packed.get("fc2") is not None:
+            return ops.w8a16_linear_add_rmsnorm(self.gate_up(n2), self._packed["fc2"], h, next_norm[0], next_norm[1])
+        return self._chain(self._linear(self.gate_up(n2), "fc2", residual=h), next_norm)
+
+    @staticmethod
+    def _chain(out, next_norm):
+        return out if next_norm is None else (out, ops.rms_norm(out, next_norm[0], next_norm[1]))
 
     def gate_up(self, n2):
         """silu(gate) * up of the MLP input projection: one fused kernel on the W8A16 path."""

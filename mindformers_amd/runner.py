@@ -110,8 +110,15 @@ class DecodeStackRunner:
         tables = torch.as_tensor(block_tables, dtype=torch.int32, device=self.device)
         slots = torch.as_tensor(slot_mapping, dtype=torch.int32, device=self.device)
         h = hidden_states
+        normed = None
         for i, layer in enumerate(self.layers):
-            h = layer(h, self.key_cache[i], self.value_cache[i], tables, lens_t, slots, cos, sin, q_starts=q_starts)
+            # W8A16 stacks: layer i also computes layer i + 1's attention norm, in the kernel that finishes its own
+            # last projection
+            nxt = self.layers[i + 1] if i + 1 < self.num_layers else None
+            chain = nxt is not None and not layer.act_quant and not nxt.act_quant
+            out = layer(h, self.key_cache[i], self.value_cache[i], tables, lens_t, slots, cos, sin, q_starts=q_starts,
+                        normed=normed, next_norm=(nxt.attn_norm, nxt.eps) if chain else None)
+            h, normed = out if chain else (out, None)
         if prefill:
             self.add_flags_custom(is_first_iteration=False)
         return h

@@ -532,6 +532,42 @@ def test_decode_layer_graph_replay_is_bit_identical():
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("act_quant", [False, True])
+def test_chained_layers_are_bit_identical_to_separate_ones(act_quant):
+    """Layer i computing layer i + 1's attention norm (inside the kernel that finishes its last projection on the
+    W8A16 path) must give the bits of every layer computing its own."""
+    from mindformers_amd import synthetic
+    from mindformers_amd.decode_layer import QuantDecodeLayer
+    case = synthetic.make_decode_case("tiny_llama_w8a16", seed=6)
+    layer = case["layers"][0]
+    if act_quant:
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(9)
+        layer = synthetic.fill_layer(QuantDecodeLayer(layer.hidden, layer.n_head, layer.n_kv_head, layer.head_dim,
+                                                      layer.ffn, layer.eps, layer.dtype, act_quant=True), gen)
+    rest = (case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    gammas = [torch.rand(layer.hidden, generator=gen, device="cuda") + 0.5 for _ in range(3)]
+
+    def run(chained):
+        kc, vc = (c.clone() for c in case["caches"][0])
+        h, normed = case["x"], None
+        for i in range(3):                                    # the same weights three times, a norm weight per level
+            layer.attn_norm.copy_(gammas[i])
+            if chained:
+                h, normed = layer(h, kc, vc, *rest, normed=normed, next_norm=(gammas[(i + 1) % 3], layer.eps))
+            else:
+                h = layer(h, kc, vc, *rest)
+        return h, normed, kc, vc
+
+    h0, _, kc0, vc0 = run(False)
+    h1, n1, kc1, vc1 = run(True)
+    assert torch.equal(h0, h1) and torch.equal(kc0, kc1) and torch.equal(vc0, vc1)
+    from mindformers_amd import ops
+    assert torch.equal(n1, ops.rms_norm(h0, gammas[0], layer.eps))
+
+
 # ------------------------------------------------------------------------------------------- checkpoint -> layer
 @pytest.mark.parametrize("fmt", ["hf_float", "mg_fused_float", "int8_with_scales"])
 def test_layer_loaded_from_a_checkpoint_matches_oracle(tmp_path, fmt):
