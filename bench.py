@@ -34,17 +34,15 @@ def run_step(case, repeats=1):
     h, normed = case["x"], case.get("normed")
     layers = case["layers"]
     for i, (layer, (kc, vc)) in ((i, lc) for _ in range(repeats) for i, lc in enumerate(zip(layers, case["caches"]))):
-        if layer.act_quant:
-            h = layer(h, kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"],
-                      case["sin"])
-            continue
-        # W8A16: as in a stack of layers, every layer computes the attention norm of the layer after it (here: of
-        # the same shape, the stack's first layer again after the last) in the kernel that finishes its last
-        # projection, and takes its own normed input from the layer before it.  One step = every projection, the
-        # attention and both norms of each layer, as before; the input norm merely sits at the end of the step.
+        # As in a stack of layers, every layer computes the attention norm of the layer after it (here: of the same
+        # shape, the stack's first layer again after the last; W8A8: with its quantisation) in the kernel that
+        # finishes its last projection, and takes its own normed input from the layer before it.  One step = every
+        # projection, the attention and both norms of each layer, as before; the input norm merely sits at the end
+        # of the step.
         nxt = layers[(i + 1) % len(layers)]
+        nn = (nxt.attn_norm, nxt.eps, nxt.qkv_smooth) if layer.act_quant else (nxt.attn_norm, nxt.eps)
         h, normed = layer(h, kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"],
-                          case["sin"], normed=normed, next_norm=(nxt.attn_norm, nxt.eps))
+                          case["sin"], normed=normed, next_norm=nn)
     return h
 
 
@@ -394,9 +392,12 @@ def main():
     log(f"[bench] built {args.workload}: batch {cfg['batch']}, sum(ctx) {int(case['context_lens_host'].sum())}, "
         f"weights {nbytes['weights'] / 1e6:.1f} MB, KV {nbytes['kv'] / 1e6:.1f} MB per layer ({time.perf_counter() - t0:.1f} s)")
 
-    if not case["layers"][0].act_quant:
-        # what the layer before the first one hands over: its output's norm under the first layer's gamma
-        case["normed"] = ops.rms_norm(case["x"], case["layers"][0].attn_norm, case["layers"][0].eps)
+    # what the layer before the first one hands over: its output's norm under the first layer's gamma (W8A8: quantised)
+    first = case["layers"][0]
+    if first.act_quant:
+        case["normed"] = ops.rms_norm_dynamic_quant(case["x"], first.attn_norm, first.eps, first.qkv_smooth, tiled=True)
+    else:
+        case["normed"] = ops.rms_norm(case["x"], first.attn_norm, first.eps)
     out_eager = run_step(case)
     torch.cuda.synchronize()
     if args.calibrate_counters:

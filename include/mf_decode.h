@@ -295,6 +295,30 @@ int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_sca
                  const float* w_scale, const void* bias, const void* residual, int m, int n, int k, int dtype,
                  int x_layout, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The row-parallel W8A8 projection (attention output, MLP down) together with what follows it in the layer: the
+ * residual add and the RMSNorm whose only reader is the next per-token quantised projection
+ * (llama_layer.py:195,225-228 behind the golden-stick QuantBatchMatmul of wo / w2).  h_out [M,N] =
+ * round(round(acc * x_scale * w_scale + bias) + residual) (residual may be NULL); xq_out / x_scale_out =
+ * mf_rmsnorm_dynamic_quant(h_out, gamma, smooth, eps, out_layout).  Bit-identical to mf_w8a8_gemm(residual)
+ * followed by mf_rmsnorm_dynamic_quant; when K is split across workgroups the integer sum of the splits, the add,
+ * the norm and the quantisation are one kernel.  N % 8 == 0, N <= 16384.  Workspace as for mf_w8a8_gemm. */
+int mf_w8a8_gemm_add_rmsnorm_quant(int8_t* xq_out, float* x_scale_out, void* h_out, const int8_t* xq,
+                                   const float* x_scale, const void* w_packed, const float* w_scale, const void* bias,
+                                   const void* residual, const void* gamma, const float* smooth, float eps, int m,
+                                   int n, int k, int dtype, int gamma_dtype, int x_layout, int out_layout,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* The fused W8A8 QKV projection with RoPE and the cache scatter behind it (infer_attention.py:441-463 behind the
+ * golden-stick QuantBatchMatmul of the fused w_qkv): as mf_w8a16_qkv_rope_and_cache, for int8 activations.  Same
+ * values as mf_w8a8_gemm followed by mf_rope_and_cache on the column slices; when K is split across workgroups the
+ * integer sum of the splits, the dequantisation, the rotation and the scatter are one kernel.  head_dim % 16 == 0.
+ * Workspace as for mf_w8a8_gemm with n = the full QKV width. */
+int mf_w8a8_qkv_rope_and_cache(void* qkv, const int8_t* xq, const float* x_scale, const void* w_packed,
+                               const float* w_scale, const void* bias, const void* cos, const void* sin,
+                               void* key_cache, void* value_cache, const int32_t* slot_mapping, int m, int n_heads,
+                               int n_kv_heads, int head_dim, int64_t num_slots, int k, int dtype, int table_dtype,
+                               int x_layout, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- mixture of experts --------------------------------------------------------------------------- */
 
 /* FusedAddTopKDiv(logits, bias, ...) — mindformers/parallel_core/inference/transformer/moe/router.py:129-140;

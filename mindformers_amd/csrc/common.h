@@ -171,6 +171,14 @@ __device__ __forceinline__ void rope_pair(float x1, float x2, float c1, float s1
     o2 = __fadd_rn(__fmul_rn(x2, c2), __fmul_rn(x1, s2));
 }
 
+// Launcher shared between source files, not part of the C ABI: the RMSNorm + per-token quantisation kernel fed from
+// the int32 split-K partial sums of an int8 GEMM (rows x cols, split_k slabs; row_scale / col_scale / bias
+// dequantise the sums; residual, sum_out, gamma, smooth, layout as in mf_rmsnorm_dynamic_quant).
+__attribute__((visibility("hidden"))) int mf_detail_rmsnorm_quant_from_partial(
+    int8_t* xq, float* x_scale, void* sum_out, const int32_t* partial, int split_k, const float* row_scale,
+    const float* col_scale, const void* bias, const void* residual, const void* gamma, const float* smooth, float eps,
+    int rows, int cols, int dtype, int gamma_dtype, int layout, void* stream);
+
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 template <typename V, typename U>

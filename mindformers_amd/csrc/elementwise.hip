@@ -207,11 +207,22 @@ __global__ __launch_bounds__(THREADS) void dynamic_quant_kernel(int8_t* __restri
 // RMSNorm (optionally with the residual add before it) followed by the per-token quantisation of its output, which
 // is not written: the quantised GEMM is its only reader.  Rounding points as the two kernels have them: the sum, and
 // the normalised value, are rounded to T before they are used further.
-template <typename T>
+// With PARTIAL the input row is not read but formed from the int32 split-K partial sums of the int8 GEMM before it
+// (exact integer sums, then acc * row scale * channel scale (+ bias), rounded to T as that GEMM's own reduce kernel
+// rounds what it stores); without a residual that rounded row goes to sum_out when one is given.
+struct PartialRow {
+    const int32_t* partial;       // [split_k][rows][cols]
+    const float* row_scale;       // [rows]: per-token scale of the GEMM's input
+    const float* col_scale;       // [cols]: per-channel weight scale
+    const uint16_t* bias;         // [cols] or null
+    int split_k;
+};
+
+template <typename T, bool PARTIAL>
 __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
     int8_t* __restrict__ xq, float* __restrict__ x_scale, uint16_t* __restrict__ sum_out,
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const void* __restrict__ gamma,
-    const float* __restrict__ smooth, float eps, int cols, int gamma_dtype, int tiled) {
+    const float* __restrict__ smooth, float eps, int cols, int gamma_dtype, int tiled, PartialRow pr) {
     __shared__ float red[NORM_THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
@@ -221,7 +232,35 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
     for (int it = 0; it < NORM_MAX_VEC; ++it) {
         const int c = threadIdx.x + it * NORM_THREADS;
         if (c < nvec) {
-            u32x4 raw = *(const u32x4*)(x + row + 8 * c);
+            u32x4 raw;
+            if constexpr (PARTIAL) {
+                const int32_t* p = pr.partial + row + 8 * c;
+                const int64_t stride = (int64_t)gridDim.x * cols;
+                i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+                for (int sp = 0; sp < pr.split_k; ++sp) {
+                    lo += *(const i32x4*)(p + sp * stride);
+                    hi += *(const i32x4*)(p + sp * stride + 4);
+                }
+                const float xs = pr.row_scale[blockIdx.x];
+                const f32x4 w_lo = *(const f32x4*)(pr.col_scale + 8 * c), w_hi = *(const f32x4*)(pr.col_scale + 8 * c + 4);
+                float t[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    t[i] = (float)lo[i] * xs * w_lo[i];
+                    t[4 + i] = (float)hi[i] * xs * w_hi[i];
+                }
+                if (pr.bias) {
+                    float bb[8];
+                    unpack8<T>(*(const u32x4*)(pr.bias + 8 * c), bb);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) t[i] += bb[i];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[i] = pack2<T>(t[2 * i], t[2 * i + 1]);
+                if (!residual && sum_out) *(u32x4*)(sum_out + row + 8 * c) = raw;
+            } else {
+                raw = *(const u32x4*)(x + row + 8 * c);
+            }
             u32x4 rraw;
             if (residual) rraw = *(const u32x4*)(residual + row + 8 * c);
             load8_as_float(gamma, 8 * c, gamma_dtype, gm[it]);
@@ -421,14 +460,33 @@ extern "C" int mf_rmsnorm_dynamic_quant(int8_t* xq, float* x_scale, void* sum_ou
     MF_REQUIRE((((uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out | (uintptr_t)gamma | (uintptr_t)smooth) & 15) == 0 &&
                    ((uintptr_t)xq & 7) == 0,
                "rmsnorm_dynamic_quant: pointers must be 16-byte aligned, xq 8-byte aligned");
+    const PartialRow none = {nullptr, nullptr, nullptr, nullptr, 0};
     if (dtype == MF_BF16)
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<BF16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps, cols,
-                           gamma_dtype, layout);
+        hipLaunchKernelGGL((rmsnorm_quant_kernel<BF16, false>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq,
+                           x_scale, (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps,
+                           cols, gamma_dtype, layout, none);
     else
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<FP16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq, x_scale,
-                           (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps, cols,
-                           gamma_dtype, layout);
+        hipLaunchKernelGGL((rmsnorm_quant_kernel<FP16, false>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq,
+                           x_scale, (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, smooth, eps,
+                           cols, gamma_dtype, layout, none);
+    return MF_LAUNCH_CHECK();
+}
+
+// The same kernel fed from the int32 split-K partial sums of an int8 GEMM (called by that GEMM's launcher; arguments
+// checked there).
+int mf_detail_rmsnorm_quant_from_partial(int8_t* xq, float* x_scale, void* sum_out, const int32_t* partial, int split_k,
+                                         const float* row_scale, const float* col_scale, const void* bias,
+                                         const void* residual, const void* gamma, const float* smooth, float eps,
+                                         int rows, int cols, int dtype, int gamma_dtype, int layout, void* stream) {
+    const PartialRow pr = {partial, row_scale, col_scale, (const uint16_t*)bias, split_k};
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL((rmsnorm_quant_kernel<BF16, true>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq,
+                           x_scale, (uint16_t*)sum_out, nullptr, (const uint16_t*)residual, gamma, smooth, eps, cols,
+                           gamma_dtype, layout, pr);
+    else
+        hipLaunchKernelGGL((rmsnorm_quant_kernel<FP16, true>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, xq,
+                           x_scale, (uint16_t*)sum_out, nullptr, (const uint16_t*)residual, gamma, smooth, eps, cols,
+                           gamma_dtype, layout, pr);
     return MF_LAUNCH_CHECK();
 }
 

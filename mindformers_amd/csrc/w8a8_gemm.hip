@@ -642,6 +642,115 @@ __global__ void w8a8_splitk_reduce_kernel(uint16_t* __restrict__ y, int32_t* __r
     }
 }
 
+// Split-K reduce of a fused QKV projection together with the rotate-half RoPE on q and k and the scatter of the
+// rotated k and of v into the paged caches.  One work item = 8 consecutive elements of the first half of a q/k head
+// with their partners in the second half, or 8 elements of v; grid = (tokens, ceil(items / 64)).  q is written
+// (rotated) into its columns of qkv, the k and v columns are not written.  Values and rounding are those of
+// w8a8_splitk_reduce_kernel followed by the rope-and-cache kernel.
+template <typename T>
+__device__ __forceinline__ void q_reduce8(const int32_t* __restrict__ p, int64_t stride, int split_k, float xs,
+                                          const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, int n,
+                                          float* out) {
+    i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+    for (int s = 0; s < split_k; ++s) {
+        lo += *(const i32x4*)(p + s * stride);
+        hi += *(const i32x4*)(p + s * stride + 4);
+    }
+    const f32x4 w_lo = *(const f32x4*)(w_scale + n), w_hi = *(const f32x4*)(w_scale + n + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float a = (float)lo[i] * xs * w_lo[i], b = (float)hi[i] * xs * w_hi[i];
+        if (bias) {
+            a += T::to_float(bias[n + i]);
+            b += T::to_float(bias[n + 4 + i]);
+        }
+        out[i] = T::to_float(T::from_float(a));
+        out[4 + i] = T::to_float(T::from_float(b));
+    }
+}
+
+constexpr int QRC_THREADS = 64;
+
+template <typename T>
+__global__ __launch_bounds__(QRC_THREADS) void w8a8_reduce_rope_cache_kernel(
+    uint16_t* __restrict__ qkv, const int32_t* __restrict__ partial, const float* __restrict__ x_scale,
+    const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, const void* __restrict__ cos,
+    const void* __restrict__ sin, uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache,
+    const int32_t* __restrict__ slot_mapping, int M, int N, int split_k, int n_heads, int n_kv, int D,
+    int64_t num_slots, int table_dtype) {
+    const int t = blockIdx.x;
+    const int half = D >> 1;
+    const int cph = half >> 3;
+    const int rot_items = (n_heads + n_kv) * cph;
+    const int v_items = n_kv * D / 8;
+    const int item = blockIdx.y * QRC_THREADS + threadIdx.x;
+    if (item >= rot_items + v_items) return;
+    const int64_t slot = slot_mapping[t];
+    const float xs = x_scale[t];
+    const int64_t row = (int64_t)n_kv * D;
+    const int64_t stride = (int64_t)M * N;
+    const int32_t* prow = partial + (int64_t)t * N;
+    if (item >= rot_items) {
+        const int i = (item - rot_items) * 8;
+        const int col = (n_heads + n_kv) * D + i;
+        float v[8];
+        q_reduce8<T>(prow + col, stride, split_k, xs, w_scale, bias, col, v);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = pack2<T>(v[2 * e], v[2 * e + 1]);
+        if (slot >= 0 && slot < num_slots) *(u32x4*)(value_cache + slot * row + i) = o;
+        return;
+    }
+    const int h = item / cph, i = (item - h * cph) * 8;
+    const bool is_k = h >= n_heads;
+    const int col = h * D + i;                                // q heads, then k heads, are consecutive columns
+    float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8];
+    const int64_t trow = (int64_t)t * D;
+    load8_as_float(cos, trow + i, table_dtype, c1);
+    load8_as_float(sin, trow + i, table_dtype, s1);
+    load8_as_float(cos, trow + i + half, table_dtype, c2);
+    load8_as_float(sin, trow + i + half, table_dtype, s2);
+    q_reduce8<T>(prow + col, stride, split_k, xs, w_scale, bias, col, x1);
+    q_reduce8<T>(prow + col + half, stride, split_k, xs, w_scale, bias, col + half, x2);
+    u32x4 o1, o2;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float a0, b0, a1, b1;
+        rope_pair(x1[2 * e], x2[2 * e], c1[2 * e], s1[2 * e], c2[2 * e], s2[2 * e], a0, b0);
+        rope_pair(x1[2 * e + 1], x2[2 * e + 1], c1[2 * e + 1], s1[2 * e + 1], c2[2 * e + 1], s2[2 * e + 1], a1, b1);
+        o1[e] = pack2<T>(a0, a1);
+        o2[e] = pack2<T>(b0, b1);
+    }
+    if (is_k) {
+        if (slot >= 0 && slot < num_slots) {
+            uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
+            *(u32x4*)(dst + i) = o1;
+            *(u32x4*)(dst + i + half) = o2;
+        }
+    } else {
+        uint16_t* dst = qkv + (int64_t)t * N + col;
+        *(u32x4*)dst = o1;
+        *(u32x4*)(dst + half) = o2;
+    }
+}
+
+// What may follow the GEMM in the same call, fused with the split-K reduce where K is split.
+struct QNormQuantArgs {           // residual add (through `residual`) + RMSNorm + per-token quantisation
+    int8_t* xq_out;
+    float* x_scale_out;
+    const void* gamma;
+    const float* smooth;
+    float eps;
+    int gamma_dtype, out_layout;
+};
+struct QRopeCacheArgs {           // RoPE on q and k + cache scatter of k and v
+    const void *cos, *sin;
+    void *key_cache, *value_cache;
+    const int32_t* slot_mapping;
+    int n_heads, n_kv, head_dim, table_dtype;
+    int64_t num_slots;
+};
+
 struct QPlan {
     int regs;        // 0: LDS-staged kernel; 1: register-streaming kernel, 4x1 waves of 64 x 64
     bool msplit;
@@ -691,7 +800,8 @@ QPlan plan_w8a8(int m, int n, int k, bool x_tiled) {
 template <typename T>
 int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const uint8_t* wp,
                 const float* w_scale, const void* bias, const void* residual, int m, int n, int k, bool x_tiled,
-                void* workspace, hipStream_t st) {
+                void* workspace, hipStream_t st, const QNormQuantArgs* nq = nullptr,
+                const QRopeCacheArgs* rc = nullptr) {
     const QPlan p = plan_w8a8(m, n, k, x_tiled);
     int32_t* partial = p.split_k > 1 ? (int32_t*)workspace : nullptr;
     dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
@@ -744,8 +854,32 @@ int launch_w8a8(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scal
 #undef QR_LAUNCH
 #undef Q_LAUNCH_KT
 #undef Q_LAUNCH
-    int rc = MF_LAUNCH_CHECK();
-    if (rc || !partial) return rc;
+    int err = MF_LAUNCH_CHECK();
+    if (err) return err;
+    if (nq) {
+        if (partial)                                          // sum of the splits + residual + norm + quantisation
+            return mf_detail_rmsnorm_quant_from_partial(nq->xq_out, nq->x_scale_out, y, partial, p.split_k, x_scale,
+                                                        w_scale, bias, residual, nq->gamma, nq->smooth, nq->eps, m, n,
+                                                        T::id, nq->gamma_dtype, nq->out_layout, st);
+        return mf_rmsnorm_dynamic_quant(nq->xq_out, nq->x_scale_out, nullptr, y, nullptr, nq->gamma, nq->smooth, nq->eps,
+                                        m, n, T::id, nq->gamma_dtype, nq->out_layout, st);   // the GEMM wrote h
+    }
+    if (rc && partial) {
+        const int items = (rc->n_heads + rc->n_kv) * (rc->head_dim / 16) + rc->n_kv * rc->head_dim / 8;
+        hipLaunchKernelGGL((w8a8_reduce_rope_cache_kernel<T>), dim3(m, (items + QRC_THREADS - 1) / QRC_THREADS),
+                           dim3(QRC_THREADS), 0, st, (uint16_t*)y, partial, x_scale, w_scale, (const uint16_t*)bias,
+                           rc->cos, rc->sin, (uint16_t*)rc->key_cache, (uint16_t*)rc->value_cache, rc->slot_mapping, m, n,
+                           p.split_k, rc->n_heads, rc->n_kv, rc->head_dim, rc->num_slots, rc->table_dtype);
+        return MF_LAUNCH_CHECK();
+    }
+    if (rc) {                                                 // no split: the GEMM wrote qkv; rotate and scatter
+        uint16_t* q = (uint16_t*)y;
+        return mf_rope_and_cache(q, q + (int64_t)rc->n_heads * rc->head_dim,
+                                 q + (int64_t)(rc->n_heads + rc->n_kv) * rc->head_dim, rc->cos, rc->sin, rc->key_cache,
+                                 rc->value_cache, rc->slot_mapping, m, rc->n_heads, rc->n_kv, rc->head_dim, rc->num_slots,
+                                 n, n, n, T::id, rc->table_dtype, st);
+    }
+    if (!partial) return 0;
     const int64_t total = (int64_t)m * ((n + 3) / 4);
     const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
     hipLaunchKernelGGL((w8a8_splitk_reduce_kernel<T>), dim3(blocks), dim3(256), 0, st, (uint16_t*)y, acc_out, partial,
@@ -784,4 +918,70 @@ extern "C" int mf_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const f
                                  x_layout == 1, workspace, (hipStream_t)stream);
     return launch_w8a8<FP16>(y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
                              x_layout == 1, workspace, (hipStream_t)stream);
+}
+
+extern "C" int mf_w8a8_gemm_add_rmsnorm_quant(int8_t* xq_out, float* x_scale_out, void* h_out, const int8_t* xq,
+                                              const float* x_scale, const void* w_packed, const float* w_scale,
+                                              const void* bias, const void* residual, const void* gamma,
+                                              const float* smooth, float eps, int m, int n, int k, int dtype,
+                                              int gamma_dtype, int x_layout, int out_layout, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a8_gemm_add_rmsnorm_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32,
+               "w8a8_gemm_add_rmsnorm_quant: bad gamma dtype");
+    MF_REQUIRE((x_layout == 0 || x_layout == 1) && (out_layout == 0 || out_layout == 1),
+               "w8a8_gemm_add_rmsnorm_quant: layouts must be 0 (row-major) or 1 (tiled)");
+    if (m == 0) return 0;
+    MF_REQUIRE(xq_out && x_scale_out && h_out && xq && x_scale && w_packed && w_scale && gamma,
+               "w8a8_gemm_add_rmsnorm_quant: null argument");
+    MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 16 == 0, "w8a8_gemm_add_rmsnorm_quant: bad sizes m=%d n=%d k=%d (K %% 16 == 0)",
+               m, n, k);
+    MF_REQUIRE(n % 8 == 0 && n <= 16384, "w8a8_gemm_add_rmsnorm_quant: N (%d) must be a multiple of 8, at most 16384", n);
+    MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w_packed | (uintptr_t)h_out | (uintptr_t)residual | (uintptr_t)gamma |
+                 (uintptr_t)smooth | (uintptr_t)bias | (uintptr_t)w_scale) & 15) == 0 && ((uintptr_t)xq_out & 7) == 0,
+               "w8a8_gemm_add_rmsnorm_quant: pointers must be 16-byte aligned, xq_out 8-byte aligned");
+    const size_t need = mf_w8a8_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a8_gemm_add_rmsnorm_quant: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    const QNormQuantArgs nq = {xq_out, x_scale_out, gamma, smooth, eps, gamma_dtype, out_layout};
+    if (dtype == MF_BF16)
+        return launch_w8a8<BF16>(h_out, nullptr, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
+                                 x_layout == 1, workspace, (hipStream_t)stream, &nq);
+    return launch_w8a8<FP16>(h_out, nullptr, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, residual, m, n, k,
+                             x_layout == 1, workspace, (hipStream_t)stream, &nq);
+}
+
+extern "C" int mf_w8a8_qkv_rope_and_cache(void* qkv, const int8_t* xq, const float* x_scale, const void* w_packed,
+                                          const float* w_scale, const void* bias, const void* cos, const void* sin,
+                                          void* key_cache, void* value_cache, const int32_t* slot_mapping, int m,
+                                          int n_heads, int n_kv_heads, int head_dim, int64_t num_slots, int k, int dtype,
+                                          int table_dtype, int x_layout, void* workspace, size_t workspace_bytes,
+                                          void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a8_qkv_rope_and_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
+               "w8a8_qkv_rope_and_cache: bad cos/sin dtype");
+    MF_REQUIRE(x_layout == 0 || x_layout == 1, "w8a8_qkv_rope_and_cache: x_layout must be 0 (row-major) or 1 (tiled)");
+    if (m == 0) return 0;
+    MF_REQUIRE(qkv && xq && x_scale && w_packed && w_scale && cos && sin && key_cache && value_cache && slot_mapping,
+               "w8a8_qkv_rope_and_cache: null argument");
+    MF_REQUIRE(m >= 0 && n_heads > 0 && n_kv_heads > 0 && k > 0 && k % 16 == 0 && num_slots > 0,
+               "w8a8_qkv_rope_and_cache: bad sizes m=%d heads=%d/%d k=%d slots=%lld", m, n_heads, n_kv_heads, k,
+               (long long)num_slots);
+    MF_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "w8a8_qkv_rope_and_cache: head_dim (%d) must be a multiple of 16",
+               head_dim);
+    const int n = (n_heads + 2 * n_kv_heads) * head_dim;
+    MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w_packed | (uintptr_t)qkv | (uintptr_t)cos | (uintptr_t)sin |
+                 (uintptr_t)key_cache | (uintptr_t)value_cache | (uintptr_t)bias | (uintptr_t)w_scale) & 15) == 0,
+               "w8a8_qkv_rope_and_cache: pointers must be 16-byte aligned");
+    const size_t need = mf_w8a8_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a8_qkv_rope_and_cache: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    const QRopeCacheArgs rc = {cos, sin, key_cache, value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, table_dtype,
+                               num_slots};
+    if (dtype == MF_BF16)
+        return launch_w8a8<BF16>(qkv, nullptr, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, nullptr, m, n, k,
+                                 x_layout == 1, workspace, (hipStream_t)stream, nullptr, &rc);
+    return launch_w8a8<FP16>(qkv, nullptr, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, nullptr, m, n, k,
+                             x_layout == 1, workspace, (hipStream_t)stream, nullptr, &rc);
 }

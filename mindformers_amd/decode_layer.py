@@ -101,11 +101,15 @@ class QuantDecodeLayer(nn.Module):
 
         Chaining layers: with ``next_norm`` = (gamma, eps) of the norm that follows this layer (the next layer's
         attention norm, or the model's final norm) the call returns (out, norm(out) * gamma), and the next layer
-        takes that second tensor as ``normed`` in place of computing its attention norm.  On the W8A16 path the norm
-        then runs inside the kernel that finishes this layer's last projection (same bits, one launch fewer)."""
+        takes that second tensor as ``normed`` in place of computing its attention norm.  The norm then runs inside
+        the kernel that finishes this layer's last projection (same bits, one launch fewer).  A W8A8 layer takes
+        ``next_norm`` = (gamma, eps, smooth) with the next layer's QKV smoothing vector and hands over the quantised
+        norm output (xq, scale), which is what a W8A8 layer accepts as ``normed``."""
         nq, nkv = self.n_head * self.head_dim, self.n_kv_head * self.head_dim
         if self.act_quant:                                    # W8A8: the norm feeds the quantised projection only
-            if normed is not None:
+            if isinstance(normed, tuple):
+                n1, n1q = None, normed
+            elif normed is not None:
                 n1, n1q = None, ops.dynamic_quant(normed, self.qkv_smooth, tiled=True)
             else:
                 n1, n1q = None, ops.rms_norm_dynamic_quant(x, self.attn_norm, self.eps, self.qkv_smooth, tiled=True)
@@ -118,6 +122,11 @@ class QuantDecodeLayer(nn.Module):
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
             ops.apply_rotary_pos_emb(q, k, cos, sin, self.n_head, self.n_kv_head, self.head_dim)
             ops.quant_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, self.kv_scale, self.kv_offset)
+        elif self.act_quant and self.head_dim % 16 == 0:      # W8A8: projection + RoPE + cache write in one call
+            if self._packed.get("qkv") is None:
+                raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
+            q = ops.w8a8_qkv_rope_and_cache(n1q[0], n1q[1], self._packed["qkv"], cos, sin, key_cache, value_cache,
+                                            slot_mapping, self.n_head, bias=self.qkv_b)
         elif self.act_quant or self.head_dim % 16:
             qkv = self._linear(n1, "qkv", quantized=n1q)
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
@@ -128,11 +137,22 @@ class QuantDecodeLayer(nn.Module):
             q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
                                              self.n_head, bias=self.qkv_b)
         attn = self.attend(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts)
-        if self.act_quant:                                    # W8A8: norm + quantisation, gate/up, act + quantisation
-            h = self._linear(attn, "wo", residual=x)
-            n2q = ops.rms_norm_dynamic_quant(h, self.ffn_norm, self.eps, self.fc1_smooth, tiled=True)
-            actq = ops.silu_mul_dynamic_quant(self._linear(None, "fc1", quantized=n2q), self.fc2_smooth, tiled=True)
-            return self._chain(self._linear(None, "fc2", residual=h, quantized=actq), next_norm)
+        if self.act_quant:
+            # W8A8: wo + residual + norm + quantisation in one call, gate/up, activation + quantisation, and fc2
+            # (+ residual + the next layer's norm and quantisation when layers are chained)
+            if self._packed.get("wo") is None:
+                raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
+            aq, a_s = ops.dynamic_quant(attn, self.wo_smooth, tiled=True)
+            h, n2x, n2s = ops.w8a8_linear_add_rmsnorm_quant(aq, a_s, self._packed["wo"], x, self.ffn_norm, self.eps,
+                                                            self.fc1_smooth, bias=self.wo_b)
+            actq = ops.silu_mul_dynamic_quant(self._linear(None, "fc1", quantized=(n2x, n2s)), self.fc2_smooth,
+                                              tiled=True)
+            if next_norm is None:
+                return self._linear(None, "fc2", residual=h, quantized=actq)
+            gamma, eps, smooth = next_norm
+            out, nx, ns = ops.w8a8_linear_add_rmsnorm_quant(actq[0], actq[1], self._packed["fc2"], h, gamma, eps, smooth,
+                                                            bias=self.fc2_b)
+            return out, (nx, ns)
         if self.wo_b is not None:
             h = self._linear(attn, "wo", residual=x)
             n2 = ops.rms_norm(h, self.ffn_norm, self.eps)

@@ -686,6 +686,72 @@ def w8a8_linear(xq, x_scale, w, w_scale=None, out_dtype=torch.bfloat16, bias=Non
     return (y, acc) if return_acc else y
 
 
+def _w8a8_operands(lib, xq, x_scale, w, what):
+    _need(isinstance(w, PackedInt8Weight) and w.experts is None and not w.gated, "w must be a packed [N, K] weight")
+    tiled = isinstance(xq, TiledInt8Activations)
+    xshape = xq.shape
+    xdata = xq.data if tiled else xq
+    _need(xdata.dtype == torch.int8 and x_scale.dtype == torch.float32, f"{what}: xq must be int8, scales fp32")
+    _need(xshape[-1] == w.k, "shape mismatch")
+    m = 1
+    for d in xshape[:-1]:
+        m *= d
+    _need(x_scale.numel() == m, "x_scale must hold one scale per row")
+    return tiled, xshape, xdata, m
+
+
+def w8a8_linear_add_rmsnorm_quant(xq, x_scale, w, residual, gamma, eps, smooth=None, bias=None, tiled_out=True):
+    """Row-parallel W8A8 projection + residual add + the RMSNorm and per-token quantisation that feed the next
+    quantised projection: returns (h, xq_next, scale_next) with h = x . w^T dequantised (+bias) + residual.
+    Bit-identical to w8a8_linear(residual=...) followed by rms_norm_dynamic_quant."""
+    lib = _lib.load()
+    tiled, xshape, xdata, m = _w8a8_operands(lib, xq, x_scale, w, "w8a8_linear_add_rmsnorm_quant")
+    dev = _dev_ok(xdata, x_scale, bias, residual, gamma, smooth)
+    n, k = w.n, w.k
+    _need(residual.dtype in _ACT and residual.is_contiguous() and residual.numel() == m * n, "residual mismatch")
+    dt = residual.dtype
+    _need(bias is None or (bias.dtype == dt and bias.numel() == n), "bias mismatch")
+    _need(gamma.numel() == n, "gamma size")
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == n), "smooth must be fp32 [N]")
+    h = torch.empty_like(residual)
+    xq_out, xs_out = _quant_out(lib, h.shape, m, n, tiled_out, dev)
+    need = lib.mf_w8a8_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a8_gemm_add_rmsnorm_quant(ptr(xq_out), ptr(xs_out), ptr(h), ptr(xdata), ptr(x_scale), ptr(w.packed),
+                                             ptr(w.scale), ptr(bias), ptr(residual), ptr(gamma), ptr(smooth),
+                                             float(eps), m, n, k, dtype_code(dt), dtype_code(gamma.dtype),
+                                             1 if tiled else 0, 1 if tiled_out else 0, ptr(ws),
+                                             ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w8a8_gemm_add_rmsnorm_quant")
+    return h, (TiledInt8Activations(xq_out, h.shape) if tiled_out else xq_out), xs_out
+
+
+def w8a8_qkv_rope_and_cache(xq, x_scale, w, cos, sin, key_cache, value_cache, slot_mapping, n_heads, bias=None):
+    """Fused W8A8 QKV projection + RoPE + cache scatter; returns the rotated query as a [T, n_heads * D] column view
+    of the projection buffer, as w8a16_qkv_rope_and_cache does."""
+    lib = _lib.load()
+    tiled, xshape, xdata, m = _w8a8_operands(lib, xq, x_scale, w, "w8a8_qkv_rope_and_cache")
+    dev = _dev_ok(xdata, x_scale, bias, cos, sin, key_cache, value_cache, slot_mapping)
+    dt = key_cache.dtype
+    _need(dt in _ACT and value_cache.dtype == dt, "caches must be bf16/fp16")
+    nb, bs, n_kv, d = key_cache.shape
+    _need(value_cache.shape == key_cache.shape, "cache shapes differ")
+    n, k = w.n, w.k
+    _need(n == (n_heads + 2 * n_kv) * d, "weight rows do not match the head geometry")
+    _need(slot_mapping.dtype == torch.int32 and slot_mapping.numel() == m, "slot_mapping must be int32 [T]")
+    _need(cos.dtype == sin.dtype and cos.numel() == m * d and sin.numel() == m * d, "cos/sin must be [T, head_dim]")
+    _need(bias is None or (bias.dtype == dt and bias.numel() == n), "bias mismatch")
+    qkv = torch.empty(m, n, dtype=dt, device=dev)
+    need = lib.mf_w8a8_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a8_qkv_rope_and_cache(ptr(qkv), ptr(xdata), ptr(x_scale), ptr(w.packed), ptr(w.scale), ptr(bias),
+                                         ptr(cos), ptr(sin), ptr(key_cache), ptr(value_cache), ptr(slot_mapping), m,
+                                         n_heads, n_kv, d, nb * bs, k, dtype_code(dt), dtype_code(cos.dtype),
+                                         1 if tiled else 0, ptr(ws), ws.numel() if ws is not None else 0,
+                                         stream_ptr(dev)), "mf_w8a8_qkv_rope_and_cache")
+    return qkv[:, :n_heads * d]
+
+
 # --------------------------------------------------------------------------------------------- MoE
 def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, renorm=True, biased_weights=False):
     """FusedAddTopKDiv: (expert_weight [T,k] out_dtype, expert_index [T,k] int32) from fp32 logits [T,E]."""

@@ -112,12 +112,15 @@ class DecodeStackRunner:
         h = hidden_states
         normed = None
         for i, layer in enumerate(self.layers):
-            # W8A16 stacks: layer i also computes layer i + 1's attention norm, in the kernel that finishes its own
-            # last projection
+            # layer i also computes layer i + 1's attention norm (W8A8: and its quantisation), in the kernel that
+            # finishes its own last projection
             nxt = self.layers[i + 1] if i + 1 < self.num_layers else None
-            chain = nxt is not None and not layer.act_quant and not nxt.act_quant
+            chain = nxt is not None and layer.act_quant == nxt.act_quant
+            nn = None
+            if chain:
+                nn = (nxt.attn_norm, nxt.eps, nxt.qkv_smooth) if nxt.act_quant else (nxt.attn_norm, nxt.eps)
             out = layer(h, self.key_cache[i], self.value_cache[i], tables, lens_t, slots, cos, sin, q_starts=q_starts,
-                        normed=normed, next_norm=(nxt.attn_norm, nxt.eps) if chain else None)
+                        normed=normed, next_norm=nn)
             h, normed = out if chain else (out, None)
         if prefill:
             self.add_flags_custom(is_first_iteration=False)

@@ -54,3 +54,11 @@ def make_paged_cache(rng, batch, ctx_lens, n_kv, head_dim, block_size, dtype, ex
     kc = rounded(rng.normal(0, std, (num_blocks, block_size, n_kv, head_dim)), dtype)
     vc = rounded(rng.normal(0, std, (num_blocks, block_size, n_kv, head_dim)), dtype)
     return kc, vc, tables, num_blocks
+
+
+def untile_int8(buf, m, k):
+    """Row-major [m, k] view of a buffer in 16 x 64 tile order (tiles ordered [s][mt]; byte (16*g + r)*16 + j of tile (mt, s) holds
+    element [16*mt + r, 64*s + 16*g + j])."""
+    mt, ks = (m + 15) // 16, (k + 63) // 64
+    t = buf[: mt * ks * 1024].reshape(ks, mt, 4, 16, 16)        # [s, mt, g, r, j]
+    return t.transpose(1, 3, 0, 2, 4).reshape(mt * 16, ks * 64)[:m, :k]

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import EPS, NAME, assert_within, dev, make_paged_cache, rounded, to_np
+from helpers import EPS, NAME, assert_within, dev, make_paged_cache, rounded, to_np, untile_int8
 
 pytestmark = pytest.mark.gpu
 
@@ -777,14 +777,6 @@ def test_w8a8_gemm_int32_bit_exact(m, n, k):
     assert_within(to_np(y), ref, np.abs(ref) + np.abs(b), dtype, ulps=1.0, extra=1e-6, what="w8a8 dequant")
 
 
-def _untile_int8(buf, m, k):
-    """Row-major [m, k] view of a buffer in 16 x 64 tile order (tiles ordered [s][mt]; byte (16*g + r)*16 + j of tile (mt, s) holds
-    element [16*mt + r, 64*s + 16*g + j])."""
-    mt, ks = (m + 15) // 16, (k + 63) // 64
-    t = buf[: mt * ks * 1024].reshape(ks, mt, 4, 16, 16)        # [s, mt, g, r, j]
-    return t.transpose(1, 3, 0, 2, 4).reshape(mt * 16, ks * 64)[:m, :k]
-
-
 @pytest.mark.parametrize("m,k", [(256, 3584), (37, 1376), (1, 64), (130, 208)])
 def test_dynamic_quant_tiled_layout_bit_exact(m, k):
     """The tiled output holds exactly the row-major result, at the positions the int8 GEMM reads."""
@@ -794,7 +786,7 @@ def test_dynamic_quant_tiled_layout_bit_exact(m, k):
     xt, xs = ops.dynamic_quant(dev(x, torch.bfloat16), torch.from_numpy(sm).cuda(), tiled=True)
     q_ref, s_ref = O.dynamic_quant_per_token(x, sm)
     assert np.array_equal(to_np(xs), s_ref)
-    assert np.array_equal(_untile_int8(to_np(xt.data), m, k), q_ref)
+    assert np.array_equal(untile_int8(to_np(xt.data), m, k), q_ref)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -818,7 +810,7 @@ def test_rms_norm_dynamic_quant_equals_unfused(dtype, m, k, smooth, residual, ti
     torch.cuda.synchronize()
     assert torch.equal(fs, us)
     if tiled:
-        assert np.array_equal(_untile_int8(to_np(fq.data), m, k), _untile_int8(to_np(uq.data), m, k))
+        assert np.array_equal(untile_int8(to_np(fq.data), m, k), untile_int8(to_np(uq.data), m, k))
     else:
         assert torch.equal(fq, uq)
 
@@ -836,7 +828,7 @@ def test_silu_mul_dynamic_quant_equals_unfused(dtype, m, f, smooth, interleaved,
     torch.cuda.synchronize()
     assert torch.equal(fs, us)
     if tiled:
-        assert np.array_equal(_untile_int8(to_np(fq.data), m, f), _untile_int8(to_np(uq.data), m, f))
+        assert np.array_equal(untile_int8(to_np(fq.data), m, f), untile_int8(to_np(uq.data), m, f))
     else:
         assert torch.equal(fq, uq)
 
@@ -859,6 +851,68 @@ def test_w8a8_tiled_activations_bit_exact(m, n, k):
 
 
 # ------------------------------------------------------------------------------------------- MoE
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k,bias,smooth,residual,tiled", [
+    (256, 3584, 3584, False, True, True, True), (256, 3584, 18944, False, True, True, True),
+    (4, 512, 1376 // 16 * 16, True, False, True, False), (130, 1024, 2048, True, True, False, True),
+    (1, 4096, 64, False, False, True, True), (300, 16384, 208, False, True, True, True),
+])
+def test_w8a8_linear_add_rmsnorm_quant_equals_unfused(dtype, m, n, k, bias, smooth, residual, tiled):
+    """Projection + residual + RMSNorm + per-token quantisation in one call: hidden state, quantised norm output and
+    its scales bit-identical to the GEMM (with residual) followed by the fused norm + quantisation kernel, on shapes
+    that split K (the fused reduce) and shapes that do not."""
+    rng = np.random.default_rng(m + n + k)
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    ws = rng.uniform(1e-4, 5e-4, n).astype(np.float32)
+    x = dev(rounded(rng.normal(size=(m, k)), dtype), dtype)
+    xq, xs = ops.dynamic_quant(x, tiled=tiled)
+    res = dev(rounded(rng.normal(size=(m, n)), dtype), dtype)
+    gamma = torch.from_numpy((1 + 0.1 * rng.normal(size=n)).astype(np.float32)).cuda()
+    sm = torch.from_numpy(rng.uniform(0.5, 2.0, n).astype(np.float32)).cuda() if smooth else None
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(ws).cuda())
+    r = res if residual else torch.zeros_like(res)
+    h, nq, ns = ops.w8a8_linear_add_rmsnorm_quant(xq, xs, packed, r, gamma, 1e-5, sm, bias=b, tiled_out=tiled)
+    h_ref = ops.w8a8_linear(xq, xs, packed, out_dtype=dtype, bias=b, residual=r)
+    nq_ref, ns_ref = ops.rms_norm_dynamic_quant(h_ref, gamma, 1e-5, sm, tiled=tiled)
+    assert torch.equal(h, h_ref)
+    assert torch.equal(ns, ns_ref)
+    if tiled:                                                # rows past m in the last 16-row tile are never written
+        assert np.array_equal(untile_int8(to_np(nq.data), m, n), untile_int8(to_np(nq_ref.data), m, n))
+    else:
+        assert torch.equal(nq, nq_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n_head,n_kv,d,k,bias,tiled", [(256, 28, 4, 128, 3584, True, True), (4, 8, 2, 64, 512, True, False),
+                                                           (7, 28, 4, 128, 64, False, True), (130, 4, 4, 32, 2048, False, True)])
+def test_w8a8_qkv_rope_and_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, bias, tiled):
+    """W8A8 QKV projection + RoPE + cache scatter in one call: the rotated query and both caches are bit-identical to
+    the GEMM followed by rope_and_cache on its column slices (shapes with and without split K; a padding slot)."""
+    rng = np.random.default_rng(t + k)
+    n = (n_head + 2 * n_kv) * d
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    ws = rng.uniform(1e-4, 5e-4, n).astype(np.float32)
+    x = dev(rounded(rng.normal(size=(t, k)), dtype), dtype)
+    xq, xs = ops.dynamic_quant(x, tiled=tiled)
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(ws).cuda())
+    bs, nb = 16, t + 3
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[t // 2] = -1
+    slots_t = torch.from_numpy(slots).cuda()
+    cos = dev(rounded(np.cos(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    sin = dev(rounded(np.sin(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    init = dev(rounded(rng.normal(size=(nb, bs, n_kv, d)), dtype), dtype)
+    kc1, vc1, kc2, vc2 = init.clone(), init.clone() + 1, init.clone(), init.clone() + 1
+    q1 = ops.w8a8_qkv_rope_and_cache(xq, xs, packed, cos, sin, kc1, vc1, slots_t, n_head, bias=b)
+    qkv = ops.w8a8_linear(xq, xs, packed, out_dtype=dtype, bias=b)
+    nq, nkv = n_head * d, n_kv * d
+    ops.rope_and_cache(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], cos, sin, kc2, vc2, slots_t, n_head)
+    assert torch.equal(q1, qkv[:, :nq])
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+
+
 @pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1)])
 def test_moe_route(t, e, k, ng, tg):
     rng = np.random.default_rng(13)

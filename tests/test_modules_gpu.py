@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import EPS, assert_within, dev, make_paged_cache, rounded, to_np
+from helpers import EPS, assert_within, dev, make_paged_cache, rounded, to_np, untile_int8
 
 pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
@@ -556,7 +556,8 @@ def test_chained_layers_are_bit_identical_to_separate_ones(act_quant):
         for i in range(3):                                    # the same weights three times, a norm weight per level
             layer.attn_norm.copy_(gammas[i])
             if chained:
-                h, normed = layer(h, kc, vc, *rest, normed=normed, next_norm=(gammas[(i + 1) % 3], layer.eps))
+                nn = (gammas[(i + 1) % 3], layer.eps) + ((layer.qkv_smooth,) if act_quant else ())
+                h, normed = layer(h, kc, vc, *rest, normed=normed, next_norm=nn)
             else:
                 h = layer(h, kc, vc, *rest)
         return h, normed, kc, vc
@@ -565,7 +566,13 @@ def test_chained_layers_are_bit_identical_to_separate_ones(act_quant):
     h1, n1, kc1, vc1 = run(True)
     assert torch.equal(h0, h1) and torch.equal(kc0, kc1) and torch.equal(vc0, vc1)
     from mindformers_amd import ops
-    assert torch.equal(n1, ops.rms_norm(h0, gammas[0], layer.eps))
+    if act_quant:
+        xq, xs = ops.rms_norm_dynamic_quant(h0, gammas[0], layer.eps, layer.qkv_smooth, tiled=True)
+        rows, width = h0.shape
+        assert np.array_equal(untile_int8(to_np(n1[0].data), rows, width), untile_int8(to_np(xq.data), rows, width))
+        assert torch.equal(n1[1], xs)
+    else:
+        assert torch.equal(n1, ops.rms_norm(h0, gammas[0], layer.eps))
 
 
 # ------------------------------------------------------------------------------------------- checkpoint -> layer
