@@ -237,9 +237,20 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
                 const int32_t* p = pr.partial + row + 8 * c;
                 const int64_t stride = (int64_t)gridDim.x * cols;
                 i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-                for (int sp = 0; sp < pr.split_k; ++sp) {
-                    lo += *(const i32x4*)(p + sp * stride);
-                    hi += *(const i32x4*)(p + sp * stride + 4);
+                for (int s0 = 0; s0 < pr.split_k; s0 += 4) {      // four splits' loads in flight together
+                    i32x4 a[4], b[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (s0 + q < pr.split_k) {
+                            a[q] = *(const i32x4*)(p + (s0 + q) * stride);
+                            b[q] = *(const i32x4*)(p + (s0 + q) * stride + 4);
+                        }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (s0 + q < pr.split_k) {
+                            lo += a[q];
+                            hi += b[q];
+                        }
                 }
                 const float xs = pr.row_scale[blockIdx.x];
                 const f32x4 w_lo = *(const f32x4*)(pr.col_scale + 8 * c), w_hi = *(const f32x4*)(pr.col_scale + 8 * c + 4);

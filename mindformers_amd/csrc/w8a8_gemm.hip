@@ -652,9 +652,20 @@ __device__ __forceinline__ void q_reduce8(const int32_t* __restrict__ p, int64_t
                                           const float* __restrict__ w_scale, const uint16_t* __restrict__ bias, int n,
                                           float* out) {
     i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-    for (int s = 0; s < split_k; ++s) {
-        lo += *(const i32x4*)(p + s * stride);
-        hi += *(const i32x4*)(p + s * stride + 4);
+    for (int s0 = 0; s0 < split_k; s0 += 4) {                 // four splits' loads in flight together
+        i32x4 a[4], b[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (s0 + q < split_k) {
+                a[q] = *(const i32x4*)(p + (s0 + q) * stride);
+                b[q] = *(const i32x4*)(p + (s0 + q) * stride + 4);
+            }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (s0 + q < split_k) {
+                lo += a[q];
+                hi += b[q];
+            }
     }
     const f32x4 w_lo = *(const f32x4*)(w_scale + n), w_hi = *(const f32x4*)(w_scale + n + 4);
 #pragma unroll
