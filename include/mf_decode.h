@@ -249,6 +249,17 @@ int mf_w8a16_qkv_rope_and_cache(void* qkv, const void* x, const void* w_packed, 
                                 int64_t num_slots, int k, int dtype, int table_dtype, void* workspace,
                                 size_t workspace_bytes, void* stream);
 
+/* mf_w8a16_qkv_rope_and_cache for int8 caches (kvcache_dtype int8, mindformers/modules/infer_attention.py:225-238):
+ * the rotated k and v rows are quantised on the way into the caches as mf_quant_reshape_and_cache does
+ * (kv_scale / kv_offset float32 [2][n_kv_heads * head_dim], keys then values; kv_offset may be NULL).  Same values as
+ * mf_w8a16_gemm, mf_rope_half on the q and k columns, then mf_quant_reshape_and_cache on the k and v columns. */
+int mf_w8a16_qkv_rope_and_quant_cache(void* qkv, const void* x, const void* w_packed, const float* scale,
+                                      const void* bias, const void* cos, const void* sin, void* key_cache,
+                                      void* value_cache, const int32_t* slot_mapping, const float* kv_scale,
+                                      const float* kv_offset, int m, int n_heads, int n_kv_heads, int head_dim,
+                                      int64_t num_slots, int k, int dtype, int table_dtype, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
 /* The gate/up projection of a gated MLP fused with its activation: WeightQuantBatchMatmul followed by
  * SiLU(gate) * up (mindformers/models/llama/llama_layer.py:419-440 with the interleaved ffn_concat layout,
  * parallel_core/inference/transformer/mlp.py:130-147).  The packed weight has its [N, K] rows in interleaved

@@ -44,6 +44,7 @@ SIGNATURES = {
     "mf_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm_add_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_qkv_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _I, _P, _Z, _P]),
+    "mf_w8a16_qkv_rope_and_quant_cache": (_I, [_P] * 12 + [_I] * 4 + [_L] + [_I] * 3 + [_P, _Z, _P]),
     "mf_w8a16_gemm_silu_mul": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_dynamic_quant_per_token": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mf_rmsnorm_dynamic_quant": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P]),

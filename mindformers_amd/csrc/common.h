@@ -179,6 +179,21 @@ __attribute__((visibility("hidden"))) int mf_detail_rmsnorm_quant_from_partial(
     const float* col_scale, const void* bias, const void* residual, const void* gamma, const float* smooth, float eps,
     int rows, int cols, int dtype, int gamma_dtype, int layout, void* stream);
 
+// Eight cache elements quantised as the int8 KV scatter defines them: clip(rint(x / scale + offset), -128, 127),
+// the quotient in double so that the rounding does not depend on how a float division is lowered; shared by the
+// stand-alone scatter kernel's fused counterparts.  v holds values already rounded to the activation type.
+__device__ __forceinline__ u32x2 quant8_for_cache(const float* v, const float* __restrict__ sc,
+                                                  const float* __restrict__ of) {
+    uint32_t w[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const double q = (double)v[i] / (double)sc[i] + (of ? (double)of[i] : 0.0);
+        const int b = (int)fmin(fmax(rint(q), -128.0), 127.0);
+        w[i >> 2] |= (uint32_t)(b & 0xff) << (8 * (i & 3));
+    }
+    return (u32x2){w[0], w[1]};
+}
+
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 template <typename V, typename U>

@@ -699,12 +699,17 @@ __device__ __forceinline__ void qkv_reduce8(const float* __restrict__ p, int64_t
 
 constexpr int RC_THREADS = 64;            // small workgroups: a 64-row step has only ~450 items per row to spread
 
-template <typename T>
+// KV8: the caches are int8 and the rows are quantised on the way (kv_scale / kv_offset float32 [2][n_kv * D], keys
+// then values), with the values and rounding of the rope kernel followed by the quantising scatter kernel.
+template <typename T, bool KV8>
 __global__ __launch_bounds__(RC_THREADS) void w8a16_reduce_rope_cache_kernel(
     uint16_t* __restrict__ qkv, const float* __restrict__ partial, const float* __restrict__ scale,
     const uint16_t* __restrict__ bias, const void* __restrict__ cos, const void* __restrict__ sin,
-    uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache, const int32_t* __restrict__ slot_mapping,
-    int M, int N, int split_k, int n_heads, int n_kv, int D, int64_t num_slots, int table_dtype) {
+    void* __restrict__ key_cache_, void* __restrict__ value_cache_, const int32_t* __restrict__ slot_mapping,
+    int M, int N, int split_k, int n_heads, int n_kv, int D, int64_t num_slots, int table_dtype,
+    const float* __restrict__ kv_scale, const float* __restrict__ kv_offset) {
+    uint16_t* key_cache = (uint16_t*)key_cache_;
+    uint16_t* value_cache = (uint16_t*)value_cache_;
     const int t = blockIdx.x;
     const int half = D >> 1;
     const int cph = half >> 3;
@@ -722,10 +727,17 @@ __global__ __launch_bounds__(RC_THREADS) void w8a16_reduce_rope_cache_kernel(
         const int col = (n_heads + n_kv) * D + i;
         float v[8];
         qkv_reduce8<T>(prow + col, stride, split_k, scale, bias, col, v);
-        u32x4 o;
+        if (slot >= 0 && slot < num_slots) {
+            if constexpr (KV8) {                              // v already holds values rounded to T
+                *(u32x2*)((int8_t*)value_cache_ + slot * row + i) =
+                    quant8_for_cache(v, kv_scale + row + i, kv_offset ? kv_offset + row + i : nullptr);
+            } else {
+                u32x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = pack2<T>(v[2 * e], v[2 * e + 1]);
-        if (slot >= 0 && slot < num_slots) *(u32x4*)(value_cache + slot * row + i) = o;
+                for (int e = 0; e < 4; ++e) o[e] = pack2<T>(v[2 * e], v[2 * e + 1]);
+                *(u32x4*)(value_cache + slot * row + i) = o;
+            }
+        }
         return;
     }
     const int h = item / cph, i = (item - h * cph) * 8;
@@ -750,9 +762,20 @@ __global__ __launch_bounds__(RC_THREADS) void w8a16_reduce_rope_cache_kernel(
     }
     if (is_k) {
         if (slot >= 0 && slot < num_slots) {
-            uint16_t* dst = key_cache + slot * row + (h - n_heads) * D;
-            *(u32x4*)(dst + i) = o1;
-            *(u32x4*)(dst + i + half) = o2;
+            const int kc = (h - n_heads) * D + i;             // column inside the key row
+            if constexpr (KV8) {
+                float r1[8], r2[8];                           // the rotated key as the rope kernel would store it
+                unpack8<T>(o1, r1);
+                unpack8<T>(o2, r2);
+                int8_t* dst = (int8_t*)key_cache_ + slot * row + kc;
+                *(u32x2*)dst = quant8_for_cache(r1, kv_scale + kc, kv_offset ? kv_offset + kc : nullptr);
+                *(u32x2*)(dst + half) =
+                    quant8_for_cache(r2, kv_scale + kc + half, kv_offset ? kv_offset + kc + half : nullptr);
+            } else {
+                uint16_t* dst = key_cache + slot * row + kc;
+                *(u32x4*)dst = o1;
+                *(u32x4*)(dst + half) = o2;
+            }
         }
     } else {
         uint16_t* dst = qkv + (int64_t)t * N + col;
@@ -790,6 +813,7 @@ struct RopeCacheArgs {
     const int32_t* slot_mapping;
     int n_heads, n_kv, head_dim, table_dtype;
     int64_t num_slots;
+    const float *kv_scale, *kv_offset;        // int8 caches: per-channel parameters [2][n_kv * head_dim]; else null
 };
 
 struct GemmPlan {
@@ -853,12 +877,28 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     if (rc_args && partial) {                                 // reduce + RoPE + cache scatter in one kernel
         const RopeCacheArgs& a = *rc_args;
         const int items = (a.n_heads + a.n_kv) * (a.head_dim / 16) + a.n_kv * a.head_dim / 8;
-        hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T>), dim3(m, (items + RC_THREADS - 1) / RC_THREADS),
-                           dim3(RC_THREADS), 0, st,
-                           (uint16_t*)y, partial, scale, (const uint16_t*)bias, a.cos, a.sin, (uint16_t*)a.key_cache,
-                           (uint16_t*)a.value_cache, a.slot_mapping, m, n, p.split_k, a.n_heads, a.n_kv, a.head_dim,
-                           a.num_slots, a.table_dtype);
+        const dim3 rgrid(m, (items + RC_THREADS - 1) / RC_THREADS);
+        if (a.kv_scale)
+            hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T, true>), rgrid, dim3(RC_THREADS), 0, st, (uint16_t*)y,
+                               partial, scale, (const uint16_t*)bias, a.cos, a.sin, a.key_cache, a.value_cache,
+                               a.slot_mapping, m, n, p.split_k, a.n_heads, a.n_kv, a.head_dim, a.num_slots,
+                               a.table_dtype, a.kv_scale, a.kv_offset);
+        else
+            hipLaunchKernelGGL((w8a16_reduce_rope_cache_kernel<T, false>), rgrid, dim3(RC_THREADS), 0, st, (uint16_t*)y,
+                               partial, scale, (const uint16_t*)bias, a.cos, a.sin, a.key_cache, a.value_cache,
+                               a.slot_mapping, m, n, p.split_k, a.n_heads, a.n_kv, a.head_dim, a.num_slots,
+                               a.table_dtype, (const float*)nullptr, (const float*)nullptr);
         return MF_LAUNCH_CHECK();
+    }
+    if (rc_args && rc_args->kv_scale) {                       // no split, int8 caches: rotate, then quantise and scatter
+        const RopeCacheArgs& a = *rc_args;
+        uint16_t* q = (uint16_t*)y;
+        uint16_t* kk = q + (int64_t)a.n_heads * a.head_dim;
+        int e = mf_rope_half(q, kk, a.cos, a.sin, m, a.n_heads, a.n_kv, a.head_dim, n, n, T::id, a.table_dtype, st);
+        if (e) return e;
+        return mf_quant_reshape_and_cache(kk, kk + (int64_t)a.n_kv * a.head_dim, a.key_cache, a.value_cache,
+                                          a.slot_mapping, a.kv_scale, a.kv_offset, m, a.n_kv, a.head_dim, a.num_slots, n,
+                                          n, T::id, st);
     }
     if (rc_args) {                                            // no split: the GEMM wrote qkv; rotate and scatter
         const RopeCacheArgs& a = *rc_args;
@@ -985,7 +1025,41 @@ extern "C" int mf_w8a16_qkv_rope_and_cache(void* qkv, const void* x, const void*
                "w8a16_qkv_rope_and_cache: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
                workspace_bytes);
     const RopeCacheArgs a = {cos, sin, key_cache, value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, table_dtype,
-                             num_slots};
+                             num_slots, nullptr, nullptr};
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(qkv, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                                  (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, &a);
+    return launch_w8a16<FP16>(qkv, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                              (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, &a);
+}
+
+extern "C" int mf_w8a16_qkv_rope_and_quant_cache(void* qkv, const void* x, const void* w_packed, const float* scale,
+                                                 const void* bias, const void* cos, const void* sin, void* key_cache,
+                                                 void* value_cache, const int32_t* slot_mapping, const float* kv_scale,
+                                                 const float* kv_offset, int m, int n_heads, int n_kv_heads,
+                                                 int head_dim, int64_t num_slots, int k, int dtype, int table_dtype,
+                                                 void* workspace, size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_qkv_rope_and_quant_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
+               "w8a16_qkv_rope_and_quant_cache: bad table dtype");
+    if (m == 0) return 0;
+    MF_REQUIRE(qkv && x && w_packed && scale && cos && sin && key_cache && value_cache && slot_mapping && kv_scale,
+               "w8a16_qkv_rope_and_quant_cache: null argument");
+    MF_REQUIRE(m >= 0 && n_heads > 0 && n_kv_heads > 0 && k > 0 && k % 8 == 0 && num_slots > 0,
+               "w8a16_qkv_rope_and_quant_cache: bad sizes");
+    MF_REQUIRE(head_dim > 0 && head_dim % 16 == 0,
+               "w8a16_qkv_rope_and_quant_cache: head_dim (%d) must be a multiple of 16", head_dim);
+    const int n = (n_heads + 2 * n_kv_heads) * head_dim;
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)qkv | (uintptr_t)cos | (uintptr_t)sin |
+                 (uintptr_t)scale | (uintptr_t)bias) & 15) == 0 &&
+                   (((uintptr_t)key_cache | (uintptr_t)value_cache) & 7) == 0,
+               "w8a16_qkv_rope_and_quant_cache: pointers must be 16-byte aligned, the caches 8-byte aligned");
+    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a16_qkv_rope_and_quant_cache: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    const RopeCacheArgs a = {cos, sin, key_cache, value_cache, slot_mapping, n_heads, n_kv_heads, head_dim, table_dtype,
+                             num_slots, kv_scale, kv_offset};
     if (dtype == MF_BF16)
         return launch_w8a16<BF16>(qkv, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
                                   (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, &a);

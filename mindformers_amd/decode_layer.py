@@ -118,10 +118,15 @@ class QuantDecodeLayer(nn.Module):
         if key_cache.dtype == torch.int8:                     # rotate, then quantize into the int8 caches
             if self.kv_scale is None:
                 raise RuntimeError("int8 caches need set_kv_quant(scale, offset)")
-            qkv = self._linear(n1, "qkv", quantized=n1q)
-            q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
-            ops.apply_rotary_pos_emb(q, k, cos, sin, self.n_head, self.n_kv_head, self.head_dim)
-            ops.quant_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, self.kv_scale, self.kv_offset)
+            if not self.act_quant and self.head_dim % 16 == 0 and self._packed.get("qkv") is not None:
+                q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache,
+                                                 slot_mapping, self.n_head, bias=self.qkv_b, kv_scale=self.kv_scale,
+                                                 kv_offset=self.kv_offset)
+            else:
+                qkv = self._linear(n1, "qkv", quantized=n1q)
+                q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+                ops.apply_rotary_pos_emb(q, k, cos, sin, self.n_head, self.n_kv_head, self.head_dim)
+                ops.quant_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, self.kv_scale, self.kv_offset)
         elif self.act_quant and self.head_dim % 16 == 0:      # W8A8: projection + RoPE + cache write in one call
             if self._packed.get("qkv") is None:
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")

@@ -519,14 +519,19 @@ def w8a16_linear_add_rmsnorm(x, w, residual, gamma, eps, bias=None):
     return h, y
 
 
-def w8a16_qkv_rope_and_cache(x, w, cos, sin, key_cache, value_cache, slot_mapping, n_heads, bias=None):
+def w8a16_qkv_rope_and_cache(x, w, cos, sin, key_cache, value_cache, slot_mapping, n_heads, bias=None,
+                             kv_scale=None, kv_offset=None):
     """Fused QKV projection + RoPE + cache scatter.  Returns the rotated query as a [T, n_heads * D] column view of
     the projection buffer (row stride = full QKV width), ready for ``paged_attention``; the caches receive the
-    rotated key rows and the value rows."""
+    rotated key rows and the value rows.  int8 caches take ``kv_scale`` (and optionally ``kv_offset``), float32
+    [2, n_kv * D] as ``quant_reshape_and_cache`` does, and receive the quantised rows."""
     lib = _lib.load()
     _need(isinstance(w, PackedInt8Weight) and w.experts is None and not w.gated, "w must be a packed [N, K] weight")
     dev = _dev_ok(x, bias, cos, sin, key_cache, value_cache, slot_mapping)
-    _need(x.dtype in _ACT and key_cache.dtype == x.dtype and value_cache.dtype == x.dtype, "dtype mismatch")
+    kv8 = key_cache.dtype == torch.int8
+    _need(x.dtype in _ACT and value_cache.dtype == key_cache.dtype and (kv8 or key_cache.dtype == x.dtype),
+          "dtype mismatch")
+    _need(kv8 == (kv_scale is not None), "kv_scale goes with int8 caches")
     nb, bs, n_kv, d = key_cache.shape
     _need(value_cache.shape == key_cache.shape, "cache shapes differ")
     n, k = w.n, w.k
@@ -539,6 +544,15 @@ def w8a16_qkv_rope_and_cache(x, w, cos, sin, key_cache, value_cache, slot_mappin
     qkv = torch.empty(m, n, dtype=x.dtype, device=dev)
     need = lib.mf_w8a16_workspace_bytes(m, n, k)
     ws = workspace(need, dev, "gemm") if need else None
+    if kv8:
+        _kv_quant_params(kv_scale, kv_offset, n_kv * d, dev)
+        check(lib.mf_w8a16_qkv_rope_and_quant_cache(ptr(qkv), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(cos),
+                                                    ptr(sin), ptr(key_cache), ptr(value_cache), ptr(slot_mapping),
+                                                    ptr(kv_scale), ptr(kv_offset), m, n_heads, n_kv, d, nb * bs, k,
+                                                    dtype_code(x.dtype), dtype_code(cos.dtype), ptr(ws),
+                                                    ws.numel() if ws is not None else 0, stream_ptr(dev)),
+              "mf_w8a16_qkv_rope_and_quant_cache")
+        return qkv[:, :n_heads * d]
     check(lib.mf_w8a16_qkv_rope_and_cache(ptr(qkv), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(cos), ptr(sin),
                                           ptr(key_cache), ptr(value_cache), ptr(slot_mapping), m, n_heads, n_kv, d,
                                           nb * bs, k, dtype_code(x.dtype), dtype_code(cos.dtype), ptr(ws),

@@ -714,6 +714,43 @@ def test_w8a16_qkv_rope_and_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, b
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n_head,n_kv,d,k,bias,with_offset", [(64, 32, 8, 128, 4096, False, False),
+                                                                 (4, 8, 2, 64, 512, True, True),
+                                                                 (7, 28, 4, 128, 64, True, True),
+                                                                 (33, 4, 4, 32, 2048, False, False)])
+def test_w8a16_qkv_rope_and_quant_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, bias, with_offset):
+    """QKV projection + RoPE + quantising scatter into int8 caches in one call: the rotated query and both caches are
+    bit-identical to the GEMM, the in-place rotation and quant_reshape_and_cache on its column slices."""
+    rng = np.random.default_rng(t + k + 1)
+    n = (n_head + 2 * n_kv) * d
+    wq, s = O.quantize_weight_int8(rng.normal(0, 0.02, (n, k)).astype(np.float32))
+    x = dev(rounded(rng.normal(size=(t, k)), dtype), dtype)
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())
+    bs, nb = 16, t + 3
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[t // 2] = -1
+    slots_t = torch.from_numpy(slots).cuda()
+    cos = dev(rounded(np.cos(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    sin = dev(rounded(np.sin(rng.uniform(0, 6, (t, d))), dtype), dtype)
+    row = n_kv * d
+    kv_scale = torch.from_numpy(rng.uniform(0.01, 0.03, (2, row)).astype(np.float32)).cuda()
+    kv_offset = torch.from_numpy(rng.uniform(-4, 4, (2, row)).astype(np.float32)).cuda() if with_offset else None
+    init = torch.from_numpy(rng.integers(-128, 128, (nb, bs, n_kv, d)).astype(np.int8)).cuda()
+    kc1, vc1, kc2, vc2 = init.clone(), init.clone(), init.clone(), init.clone()
+    q1 = ops.w8a16_qkv_rope_and_cache(x, packed, cos, sin, kc1, vc1, slots_t, n_head, bias=b, kv_scale=kv_scale,
+                                      kv_offset=kv_offset)
+    qkv = ops.w8a16_linear(x, packed, bias=b)
+    nq, nkv = n_head * d, n_kv * d
+    q2, k2, v2 = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+    ops.apply_rotary_pos_emb(q2, k2, cos, sin, n_head, n_kv, d)
+    ops.quant_reshape_and_cache(k2, v2, kc2, vc2, slots_t, kv_scale, kv_offset)
+    assert torch.equal(q1, q2)
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    assert not torch.equal(kc1, init)
+
+
 def test_w8a16_exact_on_integer_grid():
     """Power-of-two scales and small-integer activations make every product and sum exact: the kernel must
     return exactly the integer matmul (catches a dropped k-step, a wrong row/column or a transposed operand)."""
