@@ -91,6 +91,19 @@ int mf_paged_attention_decode(void* out, const void* query, const void* key_cach
                               int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                               int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mf_paged_attention_decode for a layer whose output projection is per-token quantised (the golden-stick
+ * DynamicQuant in front of the W8A8 wo, behind flash_attention.py:135-143): besides out, the row of all heads of
+ * every sequence is quantised as mf_dynamic_quant_per_token(smooth, xq_layout) would quantise out: xq int8
+ * [batch, n_heads * head_dim] (or tiled), x_scale float32 [batch].  Same bits as the two calls in sequence; with 2 to
+ * 16 partitions and n_heads * head_dim <= 4096 the partition combine and the quantisation are one kernel.  16-bit
+ * caches.  Workspace as for mf_paged_attention_decode. */
+int mf_paged_attention_decode_dynamic_quant(void* out, int8_t* xq, float* x_scale, const float* smooth, int xq_layout,
+                                            const void* query, const void* key_cache, const void* value_cache,
+                                            const int32_t* block_tables, const int32_t* context_lens, int batch,
+                                            int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                            int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                            int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- int8 KV cache (kvcache_dtype = int8, per-channel) ------------------------------------------------ */
 
 /* The reference sizes an int8 cache (mindformers/model_runner.py:364-368, kvcache_dtype in the quantization

@@ -171,6 +171,55 @@ __device__ __forceinline__ void rope_pair(float x1, float x2, float c1, float s1
     o2 = __fadd_rn(__fmul_rn(x2, c2), __fmul_rn(x1, s2));
 }
 
+// Maximum over the workgroup (red: one float per wave of shared memory); every thread gets the result.
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) t = fmaxf(t, red[i]);
+    __syncthreads();
+    return t;
+}
+
+
+// 8 values of row m, columns k .. k+7, quantised with the row's scale and written in the chosen layout.
+// The division is a true IEEE division so that the grid point chosen equals the CPU statement.
+__device__ __forceinline__ void quant_store8(int8_t* __restrict__ xq, const float* v, float safe, int m, int k, int cols,
+                                             int rows, int tiled) {
+    uint32_t o[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float qf = rintf(__fdiv_rn(v[i], safe));
+        qf = fminf(fmaxf(qf, -128.f), 127.f);
+        o[i >> 2] |= ((uint32_t)((int)qf & 0xff)) << (8 * (i & 3));
+    }
+    if (tiled) {
+        // 1 KiB tiles of 16 rows x 64 columns, [column step][row tile], 16 consecutive columns per lane
+        // (lane = 16*(column/16 % 4) + row % 16): the operand order of the int8 matrix instructions
+        const int64_t tile = (int64_t)(k >> 6) * ((rows + 15) >> 4) + (m >> 4);
+        *(u32x2*)(xq + tile * 1024 + ((((k & 63) >> 4) << 4) + (m & 15)) * 16 + (k & 15)) = (u32x2){o[0], o[1]};
+    } else {
+        *(u32x2*)(xq + (int64_t)m * cols + k) = (u32x2){o[0], o[1]};
+    }
+}
+// x * smooth in place (smooth may be null), returns max |.| of the 8 values
+__device__ __forceinline__ float smooth_absmax8(float* v, const float* __restrict__ smooth, int k) {
+    if (smooth) {
+        const f32x4 s0 = *(const f32x4*)(smooth + k), s1 = *(const f32x4*)(smooth + k + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = __fmul_rn(v[i], s0[i]);
+            v[4 + i] = __fmul_rn(v[4 + i], s1[i]);
+        }
+    }
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a = fmaxf(a, fabsf(v[i]));
+    return a;
+}
+
 // Launcher shared between source files, not part of the C ABI: the RMSNorm + per-token quantisation kernel fed from
 // the int32 split-K partial sums of an int8 GEMM (rows x cols, split_k slabs; row_scale / col_scale / bias
 // dequantise the sums; residual, sum_out, gamma, smooth, layout as in mf_rmsnorm_dynamic_quant).

@@ -916,6 +916,22 @@ __device__ inline int pf_row_limit(int row, const int32_t* __restrict__ q_starts
 // and reduced across the wave; the weighted accumulator sum runs 8 independent loads deep.
 // PF: blockIdx.y is a query row; its sequence is found in q_starts and its context is its causal limit.  Rows that
 // belong to no sequence (beyond q_starts[batch], or beyond a sequence's context) are written as zeros.
+// One output element from up to 16 partitions: (max, sum) pairs mv / lv and the partition accumulators pv of its
+// column (entries past the partition count hold PA_NEG, 0, 0 and contribute nothing).
+__device__ __forceinline__ float pa_combine16(const float* mv, const float* lv, const float* pv) {
+    float M = PA_NEG;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) M = fmaxf(M, mv[p]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+        const float f = __builtin_amdgcn_exp2f(mv[p] - M);
+        den = __fmaf_rn(f, lv[p], den);
+        num = __fmaf_rn(f, pv[p], num);
+    }
+    return __fdiv_rn(num, den);
+}
+
 template <typename T, int D, bool PF>
 __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __restrict__ out,
                                                                   const float* __restrict__ part_out,
@@ -949,17 +965,7 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
             lv[p] = on ? ml[2 * p + 1] : 0.f;
             pv[p] = on ? po[(int64_t)p * D] : 0.f;
         }
-        float M = PA_NEG;
-#pragma unroll
-        for (int p = 0; p < 16; ++p) M = fmaxf(M, mv[p]);
-        float num = 0.f, den = 0.f;
-#pragma unroll
-        for (int p = 0; p < 16; ++p) {
-            const float f = __builtin_amdgcn_exp2f(mv[p] - M);
-            den += f * lv[p];
-            num += f * pv[p];
-        }
-        out[gh * D + d] = T::from_float(num / den);
+        out[gh * D + d] = T::from_float(pa_combine16(mv, lv, pv));
         return;
     }
     // pass 1: global maximum (every wave computes it for itself)
@@ -996,15 +1002,85 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
     out[gh * D + d] = T::from_float(num / den);
 }
 
+// The partition combine of a decode step together with the per-token quantisation of the attention output row (all
+// heads of a sequence) that a W8A8 output projection wants: one workgroup per sequence, a thread per 8 consecutive
+// elements of one head; at most 16 partitions and 512 threads (n_heads * D <= 4096).  out receives the same bits as
+// paged_attention_reduce_kernel writes, xq / x_scale what the per-token quantisation kernel makes of that row.
+constexpr int PA_RQ_THREADS = 512;
+template <typename T, int D>
+__global__ __launch_bounds__(PA_RQ_THREADS) void paged_attention_reduce_quant_kernel(
+    uint16_t* __restrict__ out, int8_t* __restrict__ xq, float* __restrict__ x_scale,
+    const float* __restrict__ part_out, const float* __restrict__ part_ml, const int32_t* __restrict__ ctx_lens,
+    const float* __restrict__ smooth, int n_heads, int max_parts, int part_tokens, int tiled) {
+    __shared__ float red[PA_RQ_THREADS / 64];
+    const int b = blockIdx.x;
+    const int cols = n_heads * D;
+    const int c = threadIdx.x;                                // 8-element piece of the row
+    const bool on_row = c * 8 < cols;
+    const int L = ctx_lens[b];
+    int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
+    np = np < max_parts ? np : max_parts;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    if (on_row && np > 0) {
+        const int h = (c * 8) / D, d = (c * 8) % D;
+        const int64_t gh = (int64_t)b * n_heads + h;
+        const float* ml = part_ml + gh * max_parts * 2;
+        const float* po = part_out + gh * max_parts * D + d;
+        float mv[16], lv[16], pv[8][16];
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const bool on = p < np;
+            mv[p] = on ? ml[2 * p] : PA_NEG;
+            lv[p] = on ? ml[2 * p + 1] : 0.f;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, bq = {0.f, 0.f, 0.f, 0.f};
+            if (on) {
+                a = *(const f32x4*)(po + (int64_t)p * D);
+                bq = *(const f32x4*)(po + (int64_t)p * D + 4);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pv[i][p] = a[i];
+                pv[4 + i][p] = bq[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = pa_combine16(mv, lv, pv[i]);
+    }
+    float amax = 0.f;
+    if (on_row) {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = pack2<T>(v[2 * i], v[2 * i + 1]);
+        *(u32x4*)(out + (int64_t)b * cols + c * 8) = o;
+        unpack8<T>(o, v);                                     // the rounded row, as the quantisation kernel reads it
+        amax = smooth_absmax8(v, smooth, c * 8);
+    }
+    amax = block_max(amax, red);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float safe = s > 0.f ? s : 1.0f;
+    if (threadIdx.x == 0) x_scale[b] = s;
+    if (on_row) quant_store8(xq, v, safe, b, c * 8, cols, gridDim.x, tiled);
+}
+
 // Partition size rule shared by the workspace query and the launch: 256-token partitions keep the tail of
 // the last round of workgroups short; very long contexts use 512 to halve the partial traffic.
 static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 16384 ? 4 : 2; }
+
+// Per-token quantisation of the output rows requested together with the attention itself.
+struct PaQuantArgs {
+    int8_t* xq;
+    float* x_scale;
+    const float* smooth;
+    int layout;
+};
 
 template <typename T, int D, bool KV8>
 int launch_pa(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads, int n_kv,
               int block_size, int max_blocks, int num_blocks, float scale, int64_t q_stride, void* workspace,
-              hipStream_t st, const float* kv_scale, const float* kv_offset) {
+              hipStream_t st, const float* kv_scale, const float* kv_offset, const PaQuantArgs* qa = nullptr) {
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
@@ -1034,12 +1110,22 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
 #undef PA_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
+    if (qa && max_parts > 1 && max_parts <= 16 && n_heads * D <= PA_RQ_THREADS * 8) {
+        // combine of the partitions and quantisation of the row in one kernel
+        hipLaunchKernelGGL((paged_attention_reduce_quant_kernel<T, D>), dim3(batch), dim3(PA_RQ_THREADS), 0, st,
+                           (uint16_t*)out, qa->xq, qa->x_scale, part_out, part_ml, context_lens, qa->smooth, n_heads,
+                           max_parts, part_tokens, qa->layout);
+        return MF_LAUNCH_CHECK();
+    }
     if (max_parts > 1) {
         hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, false>), dim3(n_heads, batch), dim3(D), 0, st,
                            (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts, part_tokens,
                            (const int32_t*)nullptr, batch, false, 0);
         rc = MF_LAUNCH_CHECK();
+        if (rc) return rc;
     }
+    if (qa)
+        return mf_dynamic_quant_per_token(qa->xq, qa->x_scale, out, qa->smooth, batch, n_heads * D, T::id, qa->layout, st);
     return rc;
 }
 
@@ -1266,7 +1352,8 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
                            const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads,
                            int n_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
                            float scale, int64_t q_row_stride, int dtype, void* workspace, size_t workspace_bytes,
-                           void* stream, bool kv8, const float* kv_scale, const float* kv_offset) {
+                           void* stream, bool kv8, const float* kv_scale, const float* kv_offset,
+                           const PaQuantArgs* qa = nullptr) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention: dtype must be bf16 or fp16");
     MF_REQUIRE(!kv8 || kv_scale, "paged_attention: an int8 cache needs its scales");
     if (batch == 0) return 0;
@@ -1299,10 +1386,10 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
 #define PA_CASE(TT, DD)                                                                                        \
     return kv8 ? launch_pa<TT, DD, true>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
                                          n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
-                                         q_row_stride, ws, st, kv_scale, kv_offset)                            \
+                                         q_row_stride, ws, st, kv_scale, kv_offset, qa)                        \
                : launch_pa<TT, DD, false>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
                                           n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
-                                          q_row_stride, ws, st, nullptr, nullptr)
+                                          q_row_stride, ws, st, nullptr, nullptr, qa)
     if (dtype == MF_BF16) {
         if (head_dim == 32) PA_CASE(BF16, 32);
         if (head_dim == 64) PA_CASE(BF16, 64);
@@ -1324,6 +1411,26 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
                            dtype, workspace, workspace_bytes, stream, false, nullptr, nullptr);
+}
+
+extern "C" int mf_paged_attention_decode_dynamic_quant(void* out, int8_t* xq, float* x_scale, const float* smooth,
+                                                       int xq_layout, const void* query, const void* key_cache,
+                                                       const void* value_cache, const int32_t* block_tables,
+                                                       const int32_t* context_lens, int batch, int n_heads,
+                                                       int n_kv_heads, int head_dim, int block_size,
+                                                       int max_blocks_per_seq, int num_blocks, float scale,
+                                                       int64_t q_row_stride, int dtype, void* workspace,
+                                                       size_t workspace_bytes, void* stream) {
+    if (batch == 0) return 0;
+    MF_REQUIRE(xq && x_scale, "paged_attention_decode_dynamic_quant: null argument");
+    MF_REQUIRE(xq_layout == 0 || xq_layout == 1,
+               "paged_attention_decode_dynamic_quant: xq_layout must be 0 (row-major) or 1 (tiled)");
+    MF_REQUIRE(((uintptr_t)xq & 7) == 0 && ((uintptr_t)smooth & 15) == 0,
+               "paged_attention_decode_dynamic_quant: xq must be 8-byte aligned, smooth 16-byte aligned");
+    const PaQuantArgs qa = {xq, x_scale, smooth, xq_layout};
+    return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
+                           n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
+                           dtype, workspace, workspace_bytes, stream, false, nullptr, nullptr, &qa);
 }
 
 extern "C" int mf_paged_attention_decode_int8kv(void* out, const void* query, const void* key_cache,

@@ -141,13 +141,21 @@ class QuantDecodeLayer(nn.Module):
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
             q = ops.w8a16_qkv_rope_and_cache(n1, self._packed["qkv"], cos, sin, key_cache, value_cache, slot_mapping,
                                              self.n_head, bias=self.qkv_b)
-        attn = self.attend(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts)
+        if self.act_quant and q_starts is None and key_cache.dtype != torch.int8:
+            # W8A8 decode: the attention output is only read by wo's per-token quantisation, done with the combine of
+            # the partitions
+            _, aq, a_s = ops.paged_attention(q, key_cache, value_cache, block_tables, batch_valid_length, self.n_head,
+                                             self.n_kv_head, self.scale_value, quant=(self.wo_smooth, True))
+            attn = None
+        else:
+            attn = self.attend(q, key_cache, value_cache, block_tables, batch_valid_length, q_starts)
         if self.act_quant:
             # W8A8: wo + residual + norm + quantisation in one call, gate/up, activation + quantisation, and fc2
             # (+ residual + the next layer's norm and quantisation when layers are chained)
             if self._packed.get("wo") is None:
                 raise RuntimeError("call prepare() after loading the weights (packs them for the GEMM kernels)")
-            aq, a_s = ops.dynamic_quant(attn, self.wo_smooth, tiled=True)
+            if attn is not None:
+                aq, a_s = ops.dynamic_quant(attn, self.wo_smooth, tiled=True)
             h, n2x, n2s = ops.w8a8_linear_add_rmsnorm_quant(aq, a_s, self._packed["wo"], x, self.ffn_norm, self.eps,
                                                             self.fc1_smooth, bias=self.wo_b)
             actq = ops.silu_mul_dynamic_quant(self._linear(None, "fc1", quantized=(n2x, n2s)), self.fc2_smooth,

@@ -136,8 +136,11 @@ def rope_and_cache(query, key, value, cos, sin, key_cache, value_cache, slot_map
 
 
 # --------------------------------------------------------------------------------------------- attention
-def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n_heads, n_kv_heads, scale, out=None):
-    """PagedAttention(head_num, scale, kv_head_num)(query, key_cache, value_cache, block_tables, context_lens)."""
+def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n_heads, n_kv_heads, scale, out=None,
+                    quant=None):
+    """PagedAttention(head_num, scale, kv_head_num)(query, key_cache, value_cache, block_tables, context_lens).
+    ``quant`` = (smooth or None, tiled): also quantise every output row per token, as ``dynamic_quant`` would; the
+    call then returns (out, xq, scale)."""
     lib = _lib.load()
     _dev_of(query)
     dev = _dev_ok(key_cache, value_cache, block_tables, context_lens, out)
@@ -158,6 +161,18 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, n
         _need(out.shape == query.shape and out.dtype == query.dtype, "out mismatch")
     need = lib.mf_paged_attention_workspace_bytes(b, n_heads, d, max_blocks * bs)
     ws = workspace(need, dev, "pa") if need else None
+    if quant is not None:
+        smooth, tiled = quant
+        cols = n_heads * d
+        _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == cols and smooth.device == dev),
+              "smooth must be fp32 [n_heads * D]")
+        xq, xs = _quant_out(lib, (b, cols), b, cols, tiled, dev)
+        check(lib.mf_paged_attention_decode_dynamic_quant(
+            ptr(out), ptr(xq), ptr(xs), ptr(smooth), 1 if tiled else 0, ptr(query), ptr(key_cache), ptr(value_cache),
+            ptr(block_tables), ptr(context_lens), b, n_heads, n_kv_heads, d, bs, max_blocks, nb, float(scale), qs,
+            dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+            "mf_paged_attention_decode_dynamic_quant")
+        return out, (TiledInt8Activations(xq, (b, cols)) if tiled else xq), xs
     check(lib.mf_paged_attention_decode(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(block_tables),
                                         ptr(context_lens), b, n_heads, n_kv_heads, d, bs, max_blocks, nb,
                                         float(scale), qs, dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,

@@ -197,6 +197,34 @@ def test_paged_attention_edge_lengths():
     assert np.all(out[0] == 0)
 
 
+@pytest.mark.parametrize("dtype,b,nh,nkv,d,bs,lo,hi,smooth,tiled", [
+    (torch.bfloat16, 20, 28, 4, 128, 128, 300, 2048, True, True),    # 2..8 partitions: fused combine + quantisation
+    (torch.bfloat16, 5, 32, 8, 128, 128, 1, 200, False, False),      # one partition: attention, then quantisation
+    (torch.float16, 3, 8, 2, 64, 16, 100, 4000, True, True),         # 16 partitions
+    (torch.bfloat16, 2, 64, 8, 128, 128, 600, 900, True, True),      # row wider than the fused kernel takes
+    (torch.bfloat16, 2, 8, 2, 64, 32, 3000, 5000, False, True),      # more than 16 partitions
+])
+def test_paged_attention_with_quantised_output_equals_two_calls(dtype, b, nh, nkv, d, bs, lo, hi, smooth, tiled):
+    """Decode attention that also quantises its output rows per token: out, xq and the scales carry the bits of
+    paged_attention followed by dynamic_quant (a sequence with no context included)."""
+    rng = np.random.default_rng(b + nh + hi)
+    lens = rng.integers(lo, hi + 1, b)
+    lens[0] = 0 if lo > 1 else lens[0]
+    kc, vc, tables, nb = make_paged_cache(rng, b, np.maximum(lens, 1), nkv, d, bs, dtype, max_blocks=(hi + bs - 1) // bs)
+    q = dev(rng.normal(size=(b, nh * d)), dtype)
+    sm = torch.from_numpy(rng.uniform(0.5, 2.0, nh * d).astype(np.float32)).cuda() if smooth else None
+    args = (q, dev(kc, dtype), dev(vc, dtype), dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32), nh, nkv,
+            1.0 / np.sqrt(d))
+    out, xq, xs = ops.paged_attention(*args, quant=(sm, tiled))
+    out_ref = ops.paged_attention(*args)
+    xq_ref, xs_ref = ops.dynamic_quant(out_ref, sm, tiled=tiled)
+    assert torch.equal(out, out_ref) and torch.equal(xs, xs_ref)
+    if tiled:
+        assert np.array_equal(untile_int8(to_np(xq.data), b, nh * d), untile_int8(to_np(xq_ref.data), b, nh * d))
+    else:
+        assert torch.equal(xq, xq_ref)
+
+
 def test_paged_attention_block_permutation_invariant():
     """Moving the physical blocks (and the table with them) must leave the output bit-identical."""
     rng = np.random.default_rng(12)
