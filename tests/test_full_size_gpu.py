@@ -158,3 +158,109 @@ def test_w8a8_accumulators_are_exact(m, n, k, tiled):
     assert np.array_equal(to_np(acc).astype(np.float64), ref)
     yref = ref * to_np(xs).astype(np.float64)[:, None] * ws.astype(np.float64)[None, :]
     assert np.all(np.abs(to_np(y) - yref) <= 1.01 * EPS[BF] * np.abs(yref) + 1e-6)
+
+
+def test_w8a8_layer_step_stage_by_stage_against_the_oracle():
+    """The W8A8 bench layer (Qwen2.5-7B shape, batch 256, context 2048, per-token int8 activations) at full size,
+    first 16 sequences restated by the oracle.  Every stage is compared on identical inputs (what the GPU fed it):
+    quantised activations and their scales must be equal, projections, attention and residual sums within one or two
+    steps of the bf16 grid.  End to end an independent oracle run only agrees statistically: a one-step difference of a
+    bf16 intermediate that crosses a quantisation boundary moves the activation by a whole int8 step, and the random
+    synthetic MLP activations have a coarse grid (row maxima near 50, step 0.39), so the composed outputs are held to
+    a relative error norm instead of an elementwise bound."""
+    from oracle import dense as Dn
+    from oracle import quant as Q
+    from oracle.layer import _r
+    from helpers import assert_within, untile_int8
+    from mindformers_amd import ops, synthetic
+    case = synthetic.make_decode_case("qwen2_5_7b_w8a8", seed=7)
+    cfg, layer = case["cfg"], case["layers"][0]
+    kc, vc = case["caches"][0]
+    n, b, hidden = 16, cfg["batch"], cfg["hidden"]
+    x = case["x"]
+
+    def oq(a, smooth):
+        return Q.dynamic_quant_per_token(np.asarray(a, np.float32), to_np(smooth))
+
+    def same_quant(xq_tiled, xs, a_rows, smooth, width, what):
+        q_ref, s_ref = oq(a_rows, smooth)
+        assert np.array_equal(to_np(xs[:n]), s_ref.astype(np.float32)), what
+        assert np.array_equal(untile_int8(to_np(xq_tiled.data), b, width)[:n], q_ref), what
+        return q_ref, s_ref
+
+    def olin(q, s, name):
+        return Q.w8a8_linear(q, s, to_np(getattr(layer, name + "_w")), to_np(getattr(layer, name + "_s")), None)
+
+    # attention norm + quantisation, QKV projection
+    xq, xs = ops.rms_norm_dynamic_quant(x, layer.attn_norm, layer.eps, layer.qkv_smooth, tiled=True)
+    n1 = ops.rms_norm(x, layer.attn_norm, layer.eps)
+    n1_ref = Dn.rms_norm(to_np(x[:n]).astype(np.float64), to_np(layer.attn_norm), 1e-5)
+    assert_within(to_np(n1[:n]), n1_ref, np.abs(n1_ref), BF, ulps=1.0, extra=1e-6, what="attention norm")
+    q1, s1 = same_quant(xq, xs, to_np(n1[:n]), layer.qkv_smooth, hidden, "qkv activations")
+    qkv = ops.w8a8_linear(xq, xs, layer._packed["qkv"])
+    ref = olin(q1, s1, "qkv")
+    assert_within(to_np(qkv[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=1e-6, what="qkv projection")
+    # RoPE + cache write (bit-exact against the separate ops elsewhere), attention over the real caches
+    kc1, vc1 = kc.clone(), vc.clone()
+    q_rot = ops.w8a8_qkv_rope_and_cache(xq, xs, layer._packed["qkv"], case["cos"], case["sin"], kc1, vc1,
+                                        case["slot_mapping"], layer.n_head)
+    attn, aq, a_s = ops.paged_attention(q_rot, kc1, vc1, case["block_tables"], case["context_lens"], layer.n_head,
+                                        layer.n_kv_head, layer.scale_value, quant=(layer.wo_smooth, True))
+    tables = to_np(case["block_tables"][:n])
+    used = np.unique(tables[tables >= 0])
+    remap = -np.ones(case["num_blocks"], dtype=np.int64)
+    remap[used] = np.arange(len(used))
+    t2 = np.where(tables >= 0, remap[np.maximum(tables, 0)], -1).astype(np.int32)
+    sel = torch.from_numpy(used).cuda()
+    a_ref = O.paged_attention_decode(to_np(q_rot[:n].contiguous()).astype(np.float64), to_np(kc1[sel]), to_np(vc1[sel]), t2,
+                                     case["context_lens_host"][:n], layer.n_head, layer.n_kv_head, layer.scale_value)
+    # magnitude of a softmax-weighted sum: the same attention over |V| (the probabilities round to bf16 one by one)
+    a_mag = O.paged_attention_decode(to_np(q_rot[:n].contiguous()).astype(np.float64), to_np(kc1[sel]),
+                                     np.abs(to_np(vc1[sel])), t2, case["context_lens_host"][:n], layer.n_head,
+                                     layer.n_kv_head, layer.scale_value)
+    assert_within(to_np(attn[:n]), a_ref, a_mag, BF, ulps=1.5, what="attention")
+    q2, s2 = same_quant(aq, a_s, to_np(attn[:n]), layer.wo_smooth, layer.n_head * layer.head_dim, "wo activations")
+    # output projection + residual + MLP norm + quantisation
+    h, n2x, n2s = ops.w8a8_linear_add_rmsnorm_quant(aq, a_s, layer._packed["wo"], x, layer.ffn_norm, layer.eps,
+                                                    layer.fc1_smooth)
+    h_ref = to_np(x[:n]).astype(np.float64) + _r(olin(q2, s2, "wo"), "bf16")
+    assert_within(to_np(h[:n]), h_ref, np.abs(h_ref) + np.abs(to_np(x[:n])), BF, ulps=2.0, extra=1e-6, what="h")
+    n2_ref = _r(Dn.rms_norm(to_np(h[:n]).astype(np.float64), to_np(layer.ffn_norm), 1e-5), "bf16")
+    q3, s3 = oq(n2_ref, layer.fc1_smooth)
+    # the norm's own rounding may move an element by a bf16 step: scales equal, int8 within one step
+    assert np.allclose(to_np(n2s[:n]), s3, rtol=2 * EPS[BF], atol=0)
+    assert np.abs(untile_int8(to_np(n2x.data), b, hidden)[:n].astype(np.int32) - q3).max() <= 1
+    # gate/up, activation + quantisation, down projection + residual
+    gu = layer._linear(None, "fc1", quantized=(n2x, n2s))
+    gq, gs = untile_int8(to_np(n2x.data), b, hidden)[:n], to_np(n2s[:n])
+    ref = olin(gq, gs, "fc1")
+    assert_within(to_np(gu[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=1e-6, what="gate/up projection")
+    f = gu.shape[-1] // 2
+    guf = to_np(gu[:n]).astype(np.float64)
+    act_ref = _r(_r(Dn.silu(guf[:, :f]), "bf16") * guf[:, f:], "bf16")
+    actq = ops.silu_mul_dynamic_quant(gu, layer.fc2_smooth, tiled=True)
+    act = ops.silu_mul(gu)
+    assert_within(to_np(act[:n]), act_ref, np.abs(act_ref), BF, ulps=2.0, extra=1e-6, what="silu * up")
+    q4, s4 = same_quant(actq[0], actq[1], to_np(act[:n]), layer.fc2_smooth, f, "fc2 activations")
+    out = layer._linear(None, "fc2", residual=h, quantized=actq)
+    o_ref = to_np(h[:n]).astype(np.float64) + _r(olin(q4, s4, "fc2"), "bf16")
+    assert_within(to_np(out[:n]), o_ref, np.abs(o_ref) + np.abs(to_np(h[:n])), BF, ulps=2.0, extra=1e-6, what="out")
+    # the layer call is that sequence of stages
+    full = layer(*_step_args(case, kc.clone(), vc.clone()))
+    assert torch.equal(full, out)
+    # end to end against an independent oracle run of the 16 sequences
+    p = {}
+    for name in layer.NAMES:
+        p[name + "_w"], p[name + "_s"] = to_np(getattr(layer, name + "_w")), to_np(getattr(layer, name + "_s"))
+        p[name + "_smooth"] = to_np(getattr(layer, name + "_smooth"))
+    p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+    ocfg = dict(n_head=cfg["n_head"], n_kv_head=cfg["n_kv_head"], head_dim=cfg["head_dim"], eps=1e-5)
+    bs = cfg["block_size"]
+    slots = to_np(case["slot_mapping"][:n]).astype(np.int64)
+    slots2 = (remap[slots // bs] * bs + slots % bs).astype(np.int32)
+    e2e = O.decode_layer_w8a8(to_np(x[:n]), p, ocfg, to_np(kc[sel]), to_np(vc[sel]), t2, case["context_lens_host"][:n],
+                              slots2, to_np(case["cos"][:n]), to_np(case["sin"][:n]), act_dtype="bf16")
+    got = to_np(full[:n]).astype(np.float64)
+    assert np.linalg.norm(got - e2e) / np.linalg.norm(e2e) < 0.05
+    case.clear()
+    torch.cuda.empty_cache()
