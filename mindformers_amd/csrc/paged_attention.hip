@@ -96,7 +96,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     __shared__ int sm_count;
 
     // Work list: blockIdx.x enumerates the (sequence, kv head, partition) triples that exist, sequence-major
-    // and partition-minor; each wave finds its triple with a prefix sum over ceil(L_b / PART), so a ragged batch
+    // and partition-minor (within each of the two regions described below, where there are two); each wave finds its triple with a prefix sum over ceil(L_b / PART), so a ragged batch
     // leaves no idle workgroups between busy ones (the unused tail of the grid exits here).  The order
     // matters for HBM: walking the kv heads fastest pins each XCD (consecutive workgroup ids go to
     // consecutive XCDs) to one 256-byte lane of every token row and measured 25 % slower.
@@ -106,19 +106,44 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     {
         const int pidx = blockIdx.x;
         const int ln = threadIdx.x & 63;
-        int base = 0;
-        for (int c0 = 0; c0 < batch; c0 += 64) {
-            const int bb = c0 + ln;
-            int len, ql = 1, qs = 0, ncg = head_groups;
+        // With 512-token decode partitions (REM_LAST) the full partitions of every sequence come first and the partial
+        // last partitions (at most one per sequence) after them, so that the workgroups that finish the launch are the
+        // short ones (measured with this order: 5 % less time on a ragged int8 cache, no change on 16k-32k bf16
+        // contexts).  With 256-token partitions the short workgroups are better left between the long ones, whose
+        // streaming hides their start-up (bunched at the end they cost 3 % more), and a prefill step keeps the plain
+        // order as well.
+        constexpr bool REM_LAST = !PF && TPW >= 4;
+        auto seq_counts = [&](int bb, int& len, int& ql, int& qs, int& ncg, int& np, int& nfull) {
+            ql = 1; qs = 0; ncg = head_groups;
             if constexpr (PF) {
                 pf_seq(bb, q_starts, ctx_lens, block_tables == nullptr, pf_rows, max_blocks * block_size, batch, qs, ql, len);
                 ncg = (ql * n_rep + 15) >> 4;
             } else {
                 len = bb < batch ? min(ctx_lens[bb], max_blocks * block_size) : 0;   // the table holds no more
             }
-            int np = len > 0 ? (len + PART - 1) / PART : 0;
+            np = len > 0 ? (len + PART - 1) / PART : 0;
             np = np < max_parts ? np : max_parts;
-            const int per_seq = np * (PF ? n_kv * ncg : nkg);
+            nfull = len > 0 ? len / PART : 0;
+            nfull = nfull < np ? nfull : np;
+        };
+        int total_full = 0;
+        if constexpr (REM_LAST) {
+            for (int c0 = 0; c0 < batch; c0 += 64) {
+                int len, ql, qs, ncg, np, nfull;
+                seq_counts(c0 + ln, len, ql, qs, ncg, np, nfull);
+                total_full += nfull * nkg;
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) total_full += __shfl_xor(total_full, o, 64);
+            total_full = __builtin_amdgcn_readfirstlane(total_full);
+        }
+        const bool tail_region = REM_LAST && pidx >= total_full;   // uniform
+        int base = tail_region ? total_full : 0;
+        for (int c0 = 0; c0 < batch; c0 += 64) {
+            int len, ql, qs, ncg, np, nfull;
+            seq_counts(c0 + ln, len, ql, qs, ncg, np, nfull);
+            const int cnt = !REM_LAST ? np : tail_region ? np - nfull : nfull;   // partitions of this sequence in this region
+            const int per_seq = cnt * (PF ? n_kv * ncg : nkg);
             int incl = per_seq;
 #pragma unroll
             for (int o = 1; o < 64; o <<= 1) {
@@ -132,9 +157,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
                 const int src = __ffsll((unsigned long long)m) - 1;
                 b = c0 + src;
                 const int rem = pidx - (base + __shfl(incl - per_seq, src, 64));
-                const int npb = __shfl(np, src, 64);
+                const int npb = __shfl(cnt, src, 64);
                 kg = rem / npb;
-                part = rem - kg * npb;
+                part = rem - kg * npb + (tail_region ? __shfl(nfull, src, 64) : 0);
                 L = __shfl(len, src, 64);
                 if constexpr (PF) {
                     q_len = __shfl(ql, src, 64);
