@@ -72,7 +72,7 @@ __device__ inline void pf_seq(int s, const int32_t* __restrict__ q_starts, const
 // softmax, the value scale and offset are applied once to the (accumulator, sum) pair; the int8 tiles are widened
 // to T (exactly) when they are staged in LDS, so the MFMA path is the same.
 template <typename T, int D, int TPW, bool PF, bool KV8, bool TIB>
-__global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
+__global__ __launch_bounds__(PA_WAVES * 64, (PF || (KV8 && !TIB)) ? 3 : 4) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     __shared__ int sm_count;
 
     // Work list: blockIdx.x enumerates the (sequence, kv head, partition) triples that exist, sequence-major
-    // and partition-minor (within each of the two regions described below, where there are two); each wave finds its triple with a prefix sum over ceil(L_b / PART), so a ragged batch
+    // and partition-minor; each wave finds its triple with a prefix sum over ceil(L_b / PART), so a ragged batch
     // leaves no idle workgroups between busy ones (the unused tail of the grid exits here).  The order
     // matters for HBM: walking the kv heads fastest pins each XCD (consecutive workgroup ids go to
     // consecutive XCDs) to one 256-byte lane of every token row and measured 25 % slower.
@@ -106,44 +106,19 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     {
         const int pidx = blockIdx.x;
         const int ln = threadIdx.x & 63;
-        // With 512-token decode partitions (REM_LAST) the full partitions of every sequence come first and the partial
-        // last partitions (at most one per sequence) after them, so that the workgroups that finish the launch are the
-        // short ones (measured with this order: 5 % less time on a ragged int8 cache, no change on 16k-32k bf16
-        // contexts).  With 256-token partitions the short workgroups are better left between the long ones, whose
-        // streaming hides their start-up (bunched at the end they cost 3 % more), and a prefill step keeps the plain
-        // order as well.
-        constexpr bool REM_LAST = !PF && TPW >= 4;
-        auto seq_counts = [&](int bb, int& len, int& ql, int& qs, int& ncg, int& np, int& nfull) {
-            ql = 1; qs = 0; ncg = head_groups;
+        int base = 0;
+        for (int c0 = 0; c0 < batch; c0 += 64) {
+            const int bb = c0 + ln;
+            int len, ql = 1, qs = 0, ncg = head_groups;
             if constexpr (PF) {
                 pf_seq(bb, q_starts, ctx_lens, block_tables == nullptr, pf_rows, max_blocks * block_size, batch, qs, ql, len);
                 ncg = (ql * n_rep + 15) >> 4;
             } else {
                 len = bb < batch ? min(ctx_lens[bb], max_blocks * block_size) : 0;   // the table holds no more
             }
-            np = len > 0 ? (len + PART - 1) / PART : 0;
+            int np = len > 0 ? (len + PART - 1) / PART : 0;
             np = np < max_parts ? np : max_parts;
-            nfull = len > 0 ? len / PART : 0;
-            nfull = nfull < np ? nfull : np;
-        };
-        int total_full = 0;
-        if constexpr (REM_LAST) {
-            for (int c0 = 0; c0 < batch; c0 += 64) {
-                int len, ql, qs, ncg, np, nfull;
-                seq_counts(c0 + ln, len, ql, qs, ncg, np, nfull);
-                total_full += nfull * nkg;
-            }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) total_full += __shfl_xor(total_full, o, 64);
-            total_full = __builtin_amdgcn_readfirstlane(total_full);
-        }
-        const bool tail_region = REM_LAST && pidx >= total_full;   // uniform
-        int base = tail_region ? total_full : 0;
-        for (int c0 = 0; c0 < batch; c0 += 64) {
-            int len, ql, qs, ncg, np, nfull;
-            seq_counts(c0 + ln, len, ql, qs, ncg, np, nfull);
-            const int cnt = !REM_LAST ? np : tail_region ? np - nfull : nfull;   // partitions of this sequence in this region
-            const int per_seq = cnt * (PF ? n_kv * ncg : nkg);
+            const int per_seq = np * (PF ? n_kv * ncg : nkg);
             int incl = per_seq;
 #pragma unroll
             for (int o = 1; o < 64; o <<= 1) {
@@ -157,9 +132,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
                 const int src = __ffsll((unsigned long long)m) - 1;
                 b = c0 + src;
                 const int rem = pidx - (base + __shfl(incl - per_seq, src, 64));
-                const int npb = __shfl(cnt, src, 64);
+                const int npb = __shfl(np, src, 64);
                 kg = rem / npb;
-                part = rem - kg * npb + (tail_region ? __shfl(nfull, src, 64) : 0);
+                part = rem - kg * npb;
                 L = __shfl(len, src, 64);
                 if constexpr (PF) {
                     q_len = __shfl(ql, src, 64);
@@ -324,10 +299,20 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
     const int tstep = PA_WAVES * PA_TILE;
     const int tfirst = part_start + wu * PA_TILE;
     int64_t slot_cur = tile_slot(tfirst), slot_nxt = tile_slot(tfirst + tstep);
-    u32x4 kreg[NI], vreg[NI];
+    // ONE_BUF (16-bit caches in decode): one register tile serves K and V in turn: V of a tile is fetched while its
+    // scores are computed, K of the next tile during the PV product.  That halves the prefetch registers (32 in place
+    // of 64 at head_dim 128) and lets a fourth workgroup onto the compute unit; a wave's own tile period is several
+    // memory latencies long, so half of it still hides a load.  int8 caches need half the registers per tile anyway
+    // and keep both tiles a full period ahead.
+    constexpr bool ONE_BUF = !KV8 && !PF;
+    u32x4 kreg[NI], vreg2[ONE_BUF ? 1 : NI];
+    auto& vreg = [&]() -> u32x4(&)[NI] {
+        if constexpr (ONE_BUF) return kreg;
+        else return vreg2;
+    }();
     if (ntiles > 0) {
         load_tile(kreg, kc, slot_cur, tfirst);
-        load_tile(vreg, vc, slot_cur, tfirst);
+        if constexpr (!ONE_BUF) load_tile(vreg, vc, slot_cur, tfirst);
     }
     // the query is complete before the tile loop: a load still pending at the loop head from the entry path only
     // would make the compiler wait for every outstanding load at its first use inside the loop
@@ -349,7 +334,8 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, kreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if constexpr (more) load_tile(kreg, kc, slot_nxt, tnext);   // streams in behind this tile's math
+        if constexpr (ONE_BUF) load_tile(vreg, vc, slot_cur, tstart);     // this tile's V behind its scores
+        else if constexpr (more) load_tile(kreg, kc, slot_nxt, tnext);    // streams in behind this tile's math
 
         // ---- scores: S[s][i] = score of token tstart + 16 s + 4 g + i for head r
         f32x4 sc[2];
@@ -416,7 +402,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void paged_attention_kernel(
         for (int i = 0; i < NI; ++i) stage(vst + (lrow + RPI * i) * VSTRIDE, vreg[i]);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if constexpr (more) load_tile(vreg, vc, slot_nxt, tnext);
+        if constexpr (more) load_tile(ONE_BUF ? kreg : vreg, ONE_BUF ? kc : vc, slot_nxt, tnext);
         slot_cur = slot_nxt;
         slot_nxt = slot_nn;
 
