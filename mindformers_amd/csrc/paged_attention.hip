@@ -935,8 +935,14 @@ __device__ __forceinline__ float pa_combine16(const float* mv, const float* lv, 
     return __fdiv_rn(num, den);
 }
 
+// Threads of the combine kernel: one per output column, and never less than a whole wave (the branch for more than
+// 16 partitions spreads the partitions over the 64 lanes of a wave; with head_dim 32 the upper lanes only take
+// part in that and own no column).
+template <int D>
+constexpr int PA_REDUCE_THREADS = D < 64 ? 64 : D;
+
 template <typename T, int D, bool PF>
-__global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __restrict__ out,
+__global__ __launch_bounds__(PA_REDUCE_THREADS<D>) void paged_attention_reduce_kernel(uint16_t* __restrict__ out,
                                                                   const float* __restrict__ part_out,
                                                                   const float* __restrict__ part_ml,
                                                                   const int32_t* __restrict__ ctx_lens, int n_heads,
@@ -945,19 +951,21 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
                                                                   bool contiguous, int max_ctx) {
     __shared__ float s_f[64];
     const int h = blockIdx.x, b = blockIdx.y;                 // b: sequence (decode) or query row (PF)
-    const int d = threadIdx.x;
+    const bool own = (int)threadIdx.x < D;                    // this thread owns an output column
+    const int d = own ? threadIdx.x : 0;
     const int lane = threadIdx.x & 63;
     const int L = PF ? pf_row_limit(b, q_starts, ctx_lens, contiguous, gridDim.y, max_ctx, batch) : ctx_lens[b];
     const int64_t gh = (int64_t)b * n_heads + h;
     int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
     np = np < max_parts ? np : max_parts;
     if (np == 0) {
-        out[gh * D + d] = 0;
+        if (own) out[gh * D + d] = 0;
         return;
     }
     const float* ml = part_ml + gh * max_parts * 2;
     const float* po = part_out + gh * max_parts * D + d;
     if (np <= 16) {
+        if (!own) return;
         // common case: every load of the row (the (max, sum) pairs and this thread's accumulator column) is issued
         // at once, one memory round trip instead of three dependent ones
         float mv[16], lv[16], pv[16];
@@ -1002,7 +1010,7 @@ __global__ __launch_bounds__(D) void paged_attention_reduce_kernel(uint16_t* __r
         }
         for (; q < cnt; ++q) num += s_f[q] * po[(int64_t)(p0 + q) * D];
     }
-    out[gh * D + d] = T::from_float(num / den);
+    if (own) out[gh * D + d] = T::from_float(num / den);
 }
 
 // The partition combine of a decode step together with the per-token quantisation of the attention output row (all
@@ -1070,6 +1078,12 @@ __global__ __launch_bounds__(PA_RQ_THREADS) void paged_attention_reduce_quant_ke
 // Partition size rule shared by the workspace query and the launch: 256-token partitions keep the tail of
 // the last round of workgroups short; very long contexts use 512 to halve the partial traffic.
 static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 16384 ? 4 : 2; }
+// int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
+// first tile, merge) exposed: twice the tokens per workgroup at every context length (fewer partitions than the
+// workspace query, which does not know the cache type, sizes for).
+static inline int pa_launch_tiles_per_wave(int64_t max_context, bool kv8) {
+    return kv8 ? 4 : pa_tiles_per_wave(max_context);
+}
 
 // Per-token quantisation of the output rows requested together with the attention itself.
 struct PaQuantArgs {
@@ -1087,9 +1101,7 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
-    // first tile, merge) exposed: twice the tokens per workgroup.  Fewer partitions than the workspace was sized for.
-    const int tpw = KV8 ? 4 : pa_tiles_per_wave(max_ctx);
+    const int tpw = pa_launch_tiles_per_wave(max_ctx, KV8);
     const int part_tokens = tpw * PA_WAVE_TOKENS;
     const int max_parts = (int)((max_ctx + part_tokens - 1) / part_tokens);
     float* part_out = (float*)workspace;
@@ -1121,7 +1133,8 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
         return MF_LAUNCH_CHECK();
     }
     if (max_parts > 1) {
-        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, false>), dim3(n_heads, batch), dim3(D), 0, st,
+        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, false>), dim3(n_heads, batch),
+                           dim3(PA_REDUCE_THREADS<D>), 0, st,
                            (uint16_t*)out, part_out, part_ml, context_lens, n_heads, max_parts, part_tokens,
                            (const int32_t*)nullptr, batch, false, 0);
         rc = MF_LAUNCH_CHECK();
@@ -1238,7 +1251,8 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
-        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, true>), dim3(n_heads, total_q), dim3(D), 0, st,
+        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, true>), dim3(n_heads, total_q),
+                           dim3(PA_REDUCE_THREADS<D>), 0, st,
                            (uint16_t*)out, part_out, part_ml, context_lens, n_heads, plan.max_parts,
                            plan.part_tokens, q_starts, batch, contiguous, max_blocks * block_size);
         rc = MF_LAUNCH_CHECK();
@@ -1379,7 +1393,10 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
                "paged_attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     MF_REQUIRE(need == 0 || ((uintptr_t)workspace & 15) == 0, "paged_attention: workspace must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    if (need == 0) {
+    // with one partition the attention kernel writes the output rows itself and skips sequences without context
+    const int64_t launch_part_tokens =
+        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kv8) * PA_WAVE_TOKENS;
+    if ((int64_t)max_blocks_per_seq * block_size <= launch_part_tokens) {
         hipLaunchKernelGGL(pa_zero_empty_kernel, dim3(batch), dim3(128), 0, st, (uint16_t*)out, context_lens,
                            n_heads * head_dim);
         int rc = MF_LAUNCH_CHECK();

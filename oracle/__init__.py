@@ -33,9 +33,12 @@ Pinning status of each function (what fixes it besides its own formula):
   quantize_weight_int8,    PARITY UNPINNED: the arithmetic lives in mindspore_gs / CANN
   w8a16_linear,            (not vendored, no reference vector).  int32 accumulators are
   dynamic_quant_per_token, pinned against exact integer matmul; rounding mode, clamp range
-  w8a8_linear,             and dequant order are this build's declared convention.  The int8 KV cache is
-  quantize_kv_int8,        pinned only through exactness: attention over a dequantised cache equals the
-  dequantize_kv_int8       16-bit oracle on the dequantised values (tests).
+  w8a8_linear              and dequant order are this build's declared convention.
+  quantize_kv_int8,        PARITY UNPINNED against the reference for the same reason (the convention, affine per
+  dequantize_kv_int8       channel with ties to even and rails -128 / 127, is declared); the two functions
+                           themselves are pinned against that convention by hand-computed values, the offset's
+                           direction, clipping at the rails, the half-step round trip and torch's affine
+                           per-channel quantiser on power-of-two scales (tests/test_host_logic.py)
 """
 from .numerics import (round_bf16, round_fp16, round_to, double_benchmark,
                        DoubleBenchmarkResult)

@@ -221,6 +221,53 @@ def test_quantisation_grid_properties():
     assert np.all(O.int8_gemm_i32(a, b) == 128 * 127 * 512)
 
 
+def test_kv_int8_oracle_pair_is_pinned_by_what_the_mathematics_fixes():
+    """The int8 KV-cache pair q = clip(rint(x / s + o), -128, 127), x ~ (q - o) * s, pinned without its own formula:
+    hand-computed values, the direction of the offset and the side of the scale (a mirrored sign or a product in
+    place of the quotient fails), clipping at both rails, the half-step round-trip bound inside the rails, and
+    torch's affine per-channel quantiser (x / s rounded, plus an integer zero point) on power-of-two scales."""
+    # hand-computed: 0.26 / 0.1 + 3 = 5.6 -> 6; (6 - 3) * 0.1 = 0.3; -0.26 / 0.1 + 3 = 0.4 -> 0; (0 - 3) * 0.1 = -0.3
+    q = O.quantize_kv_int8(np.array([[0.26, -0.26]]), np.array([0.1, 0.1]), np.array([3.0, 3.0]))
+    assert q.dtype == np.int8 and q.tolist() == [[6, 0]]
+    assert np.allclose(O.dequantize_kv_int8(q, np.array([0.1, 0.1]), np.array([3.0, 3.0])), [[0.3, -0.3]], atol=1e-15)
+    # zero maps to the offset itself (not to its negative) and comes back as zero; k * s maps to k + o exactly
+    s = np.array([0.5, 0.25, 2.0, 0.125])
+    o = np.array([7.0, -11.0, 0.0, 30.0])
+    assert O.quantize_kv_int8(np.zeros((1, 4)), s, o).tolist() == [[7, -11, 0, 30]]
+    assert np.array_equal(O.dequantize_kv_int8(np.array([[7, -11, 0, 30]], np.int8), s, o), np.zeros((1, 4)))
+    ks = np.array([[5, -9, 17, -40]])
+    assert np.array_equal(O.quantize_kv_int8(ks * s, s, o), (ks + o).astype(np.int8))   # a product x * s gives 5 s^2
+    assert np.array_equal(O.dequantize_kv_int8((ks + o).astype(np.int8), s, o), ks * s)
+    # no offset = offset 0
+    x = np.random.default_rng(3).normal(size=(50, 4))
+    assert np.array_equal(O.quantize_kv_int8(x, s), O.quantize_kv_int8(x, s, np.zeros(4)))
+    # clipping at the rails: anything beyond (127 - o) s / (-128 - o) s sticks to 127 / -128
+    big = np.array([[1e6, 1e6, 1e6, 1e6], [-1e6, -1e6, -1e6, -1e6]])
+    assert O.quantize_kv_int8(big, s, o).tolist() == [[127] * 4, [-128] * 4]
+    hi, lo = (127 - o) * s, (-128 - o) * s
+    assert O.quantize_kv_int8(np.stack([hi + 0.6 * s, lo - 0.6 * s]), s, o).tolist() == [[127] * 4, [-128] * 4]
+    # ties go to even (the declared rounding): 2.5 -> 2, 3.5 -> 4, -2.5 -> -2
+    assert O.quantize_kv_int8(np.array([[2.5, 3.5, -2.5]]), np.ones(3)).tolist() == [[2, 4, -2]]
+    # inside the rails the round trip is within half a step, and the step is the scale
+    rng = np.random.default_rng(8)
+    s = rng.uniform(0.005, 0.05, 64)
+    o = rng.integers(-30, 31, 64).astype(np.float64)
+    x = rng.uniform((-128 - o) * s, (127 - o) * s, (500, 64))
+    back = O.dequantize_kv_int8(O.quantize_kv_int8(x, s, o), s, o)
+    assert np.all(np.abs(back - x) <= s / 2 * (1 + 1e-9))
+    assert np.abs(back - x).max() > 0.4 * s.min()                          # a real grid, not a pass-through
+    # a library routine: torch's affine per-channel quantiser, q = clamp(round(x / s) + zero_point), on
+    # power-of-two scales (the quotient is then exact in float32 too) and integer zero points
+    s2 = (2.0 ** rng.integers(-7, -3, 64)).astype(np.float64)
+    zp = rng.integers(-30, 31, 64)
+    xt = torch.from_numpy(rng.normal(0, 1.5, (300, 64)).astype(np.float32))
+    tq = torch.quantize_per_channel(xt, torch.from_numpy(s2), torch.from_numpy(zp), 1, torch.qint8)
+    mine = O.quantize_kv_int8(xt.numpy(), s2, zp.astype(np.float64))
+    assert np.array_equal(mine, tq.int_repr().numpy())
+    assert (mine == 127).any() and (mine == -128).any()                    # the rails are exercised
+    assert np.array_equal(O.dequantize_kv_int8(mine, s2, zp.astype(np.float64)), tq.dequantize().double().numpy())
+
+
 def test_moe_permute_is_a_stable_sort_and_unpermute_inverts_it():
     rng = np.random.default_rng(7)
     t, k, e, h = 9, 3, 5, 4
