@@ -264,3 +264,342 @@ def test_w8a8_layer_step_stage_by_stage_against_the_oracle():
     assert np.linalg.norm(got - e2e) / np.linalg.norm(e2e) < 0.05
     case.clear()
     torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------------------ the W8A16 layer, stage by stage
+def _sub_batch(case, n):
+    """The first n sequences of a case with compact numpy copies of their cache blocks: (remapped tables, block ids
+    as a device tensor, remapped slots, block remap)."""
+    tables = to_np(case["block_tables"][:n])
+    used = np.unique(tables[tables >= 0])
+    remap = -np.ones(case["num_blocks"], dtype=np.int64)
+    remap[used] = np.arange(len(used))
+    t2 = np.where(tables >= 0, remap[np.maximum(tables, 0)], -1).astype(np.int32)
+    bs = case["cfg"]["block_size"]
+    slots = to_np(case["slot_mapping"][:n]).astype(np.int64)
+    slots2 = (remap[slots // bs] * bs + slots % bs).astype(np.int32)
+    return t2, torch.from_numpy(used).cuda(), slots2
+
+
+def _w8a16_stages(case, n, attn_rows=None):
+    """Every stage of one W8A16 decode-layer step on the GPU, compared with the oracle on what the GPU fed that stage
+    (first ``n`` rows; the attention stage on ``attn_rows`` of them).  Returns the stage outputs."""
+    from oracle import dense as Dn
+    from oracle import quant as Q
+    from oracle.layer import _r
+    from oracle.rope import apply_rotary_half
+    from helpers import assert_within
+    from mindformers_amd import ops
+    cfg, layer = case["cfg"], case["layers"][0]
+    kc, vc = (c.clone() for c in case["caches"][0])
+    x = case["x"]
+    nh, nkv, d = layer.n_head, layer.n_kv_head, layer.head_dim
+    nq, nk = nh * d, nkv * d
+    attn_rows = n if attn_rows is None else attn_rows
+
+    def olin(a_rows, name):
+        w, s = to_np(getattr(layer, name + "_w")), to_np(getattr(layer, name + "_s"))
+        a = np.asarray(a_rows, np.float64)
+        y = Q.w8a16_linear(a, w, s)
+        mag = Q.w8a16_linear(np.abs(a), np.abs(w), s)           # sum of |terms|: what the fp32 accumulation error scales with
+        return y, mag
+
+    # attention norm
+    n1 = ops.rms_norm(x, layer.attn_norm, layer.eps)
+    ref = Dn.rms_norm(to_np(x[:n]).astype(np.float64), to_np(layer.attn_norm), 1e-5)
+    assert_within(to_np(n1[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=1e-6, what="attention norm")
+    # QKV projection
+    qkv = ops.w8a16_linear(n1, layer._packed["qkv"])
+    ref, mag = olin(to_np(n1[:n]), "qkv")
+    assert_within(to_np(qkv[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="qkv projection")
+    # RoPE on the GPU's projection output, scatter: rotated rows within a step, cache rows = those rows bit for bit
+    q, k, v = qkv[:, :nq].contiguous(), qkv[:, nq:nq + nk].contiguous(), qkv[:, nq + nk:].contiguous()
+    q_in, k_in = to_np(q[:n]).astype(np.float64), to_np(k[:n]).astype(np.float64)
+    ops.rope_and_cache(q, k, v, case["cos"], case["sin"], kc, vc, case["slot_mapping"], nh)
+    cos, sin = to_np(case["cos"][:n]).astype(np.float64), to_np(case["sin"][:n]).astype(np.float64)
+    for got, src, heads, what in ((q, q_in, nh, "rotated query"), (k, k_in, nkv, "rotated key")):
+        ref = apply_rotary_half(src, cos, sin, heads)
+        xh = np.abs(src.reshape(n, heads, d))
+        swapped = np.concatenate((xh[..., d // 2:], xh[..., :d // 2]), -1)
+        mag = (xh * np.abs(cos)[:, None, :] + swapped * np.abs(sin)[:, None, :]).reshape(n, heads * d)
+        assert_within(to_np(got[:n]), ref, mag, BF, ulps=1.0, what=what)
+    slots = case["slot_mapping"].long()
+    row = nk
+    assert torch.equal(kc.view(-1, row)[slots], k) and torch.equal(vc.view(-1, row)[slots], v)
+    keep = torch.ones(kc.view(-1, row).shape[0], dtype=torch.bool, device="cuda")
+    keep[slots] = False
+    assert torch.equal(kc.view(-1, row)[keep], case["caches"][0][0].view(-1, row)[keep])
+    assert torch.equal(vc.view(-1, row)[keep], case["caches"][0][1].view(-1, row)[keep])
+    # the fused projection + RoPE + scatter writes those same bits
+    kc2, vc2 = (c.clone() for c in case["caches"][0])
+    q2 = ops.w8a16_qkv_rope_and_cache(n1, layer._packed["qkv"], case["cos"], case["sin"], kc2, vc2,
+                                      case["slot_mapping"], nh)
+    assert torch.equal(q2, q) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    # attention over the caches the step wrote
+    attn = ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], nh, nkv, layer.scale_value)
+    t2, sel, _ = _sub_batch(case, attn_rows)
+    lens = case["context_lens_host"][:attn_rows]
+    kcn, vcn = to_np(kc[sel]), to_np(vc[sel])
+    qn = to_np(q[:attn_rows]).astype(np.float64)
+    a_ref = O.paged_attention_decode(qn, kcn, vcn, t2, lens, nh, nkv, layer.scale_value)
+    a_mag = O.paged_attention_decode(qn, kcn, np.abs(vcn), t2, lens, nh, nkv, layer.scale_value)
+    assert_within(to_np(attn[:attn_rows]), a_ref, a_mag, BF, ulps=1.5, what="attention")
+    del kcn, vcn
+    # output projection + residual, MLP norm (one fused call; the unfused pair must give the same bits)
+    h, n2 = ops.w8a16_linear_add_rmsnorm(attn, layer._packed["wo"], x, layer.ffn_norm, layer.eps)
+    h_un = ops.w8a16_linear(attn, layer._packed["wo"], residual=x)
+    assert torch.equal(h, h_un) and torch.equal(n2, ops.rms_norm(h_un, layer.ffn_norm, layer.eps))
+    ref, mag = olin(to_np(attn[:n]), "wo")
+    xr = to_np(x[:n]).astype(np.float64)
+    h_ref = xr + _r(ref, "bf16")
+    assert_within(to_np(h[:n]), h_ref, np.abs(h_ref) + 2 * np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9,
+                  what="wo + residual")
+    ref = Dn.rms_norm(to_np(h[:n]).astype(np.float64), to_np(layer.ffn_norm), 1e-5)
+    assert_within(to_np(n2[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=1e-6, what="MLP norm")
+    # gate/up projection with the activation fused, against the unfused pair bit for bit and against the oracle
+    a = layer.gate_up(n2)
+    gu = ops.w8a16_linear(n2, ops.pack_w8a16(layer.fc1_w, layer.fc1_s))
+    assert torch.equal(a, ops.silu_mul(gu))
+    ref, mag = olin(to_np(n2[:n]), "fc1")
+    assert_within(to_np(gu[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="gate/up projection")
+    f = gu.shape[-1] // 2
+    guf = to_np(gu[:n]).astype(np.float64)
+    act_ref = _r(Dn.silu(guf[:, :f]), "bf16") * guf[:, f:]
+    assert_within(to_np(a[:n]), act_ref, np.abs(act_ref), BF, ulps=2.0, extra=1e-6, what="silu * up")
+    # down projection + residual
+    out = ops.w8a16_linear(a, layer._packed["fc2"], residual=h)
+    ref, mag = olin(to_np(a[:n]), "fc2")
+    hr = to_np(h[:n]).astype(np.float64)
+    o_ref = hr + _r(ref, "bf16")
+    assert_within(to_np(out[:n]), o_ref, np.abs(o_ref) + 2 * np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9,
+                  what="fc2 + residual")
+    # the layer call is that sequence of stages
+    kc3, vc3 = (c.clone() for c in case["caches"][0])
+    full = layer(*_step_args(case, kc3, vc3))
+    assert torch.equal(full, out) and torch.equal(kc3, kc) and torch.equal(vc3, vc)
+    return dict(q=q, kc=kc, vc=vc, attn=attn, out=out)
+
+
+def test_w8a16_layer_step_stage_by_stage_against_the_oracle(llama_case):
+    """The Llama-3-8B W8A16 bench layer at full size (batch 64, contexts U[512, 4096]): every stage against the
+    oracle on the inputs the GPU fed it, all 64 rows (the attention on the first 24 sequences), every fused entry point
+    bit for bit against its unfused sequence, and the layer call against the chain of stages."""
+    _w8a16_stages(llama_case, 64, attn_rows=24)
+
+
+# ------------------------------------------------------------------------------ Qwen2.5-72B long-context decode
+@pytest.fixture(scope="module")
+def qwen72_case():
+    from mindformers_amd import synthetic
+    case = synthetic.make_decode_case("qwen2_5_72b_w8a16", seed=9, layers=1)
+    yield case
+    case.clear()
+    torch.cuda.empty_cache()
+
+
+def test_long_context_attention_properties_and_oracle(qwen72_case):
+    """64 query / 8 kv heads of 128, batch 16, contexts U[16384, 32768] in 128-token blocks: the block table spans
+    more than 16384 tokens, so the 512-token-partition instantiation and the combine over up to 64 partitions run.
+    Bit-identical under moved blocks, a reordered batch and a wider block table (more partition slots in the
+    workspace); three sequences against the oracle."""
+    from helpers import assert_within
+    from mindformers_amd import ops
+    case = qwen72_case
+    cfg = case["cfg"]
+    kc, vc = case["caches"][0]
+    nh, nkv, d = cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"]
+    assert case["block_tables"].shape[1] * cfg["block_size"] > 16384
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(12)
+    q = torch.randn(cfg["batch"], nh * d, generator=gen, device="cuda").to(BF)
+    scale = 1.0 / np.sqrt(d)
+    out = ops.paged_attention(q, kc, vc, case["block_tables"], case["context_lens"], nh, nkv, scale)
+    assert bool(torch.isfinite(out.float()).all())
+    n = 3
+    t2, sel, _ = _sub_batch(case, n)
+    lens = case["context_lens_host"][:n]
+    kcn, vcn = to_np(kc[sel]), to_np(vc[sel])
+    qn = to_np(q[:n]).astype(np.float64)
+    ref = O.paged_attention_decode(qn, kcn, vcn, t2, lens, nh, nkv, scale)
+    mag = O.paged_attention_decode(qn, kcn, np.abs(vcn), t2, lens, nh, nkv, scale)
+    assert_within(to_np(out[:n]), ref, mag, BF, ulps=1.5, what="long-context attention")
+    del kcn, vcn
+    # a wider block table: same partitions, more slots per row in the workspace
+    wide = torch.full((cfg["batch"], case["block_tables"].shape[1] + 37), -1, dtype=torch.int32, device="cuda")
+    wide[:, :case["block_tables"].shape[1]] = case["block_tables"]
+    assert torch.equal(out, ops.paged_attention(q, kc, vc, wide, case["context_lens"], nh, nkv, scale))
+    # the batch in another order
+    order = torch.randperm(cfg["batch"], generator=gen, device="cuda")
+    out3 = ops.paged_attention(q[order].contiguous(), kc, vc, case["block_tables"][order].contiguous(),
+                               case["context_lens"][order].contiguous(), nh, nkv, scale)
+    assert torch.equal(out[order], out3)
+    # physical blocks moved (new id = perm[old id]), the tables following them
+    perm = torch.randperm(case["num_blocks"], generator=gen, device="cuda")
+    kc2 = torch.empty_like(kc)
+    kc2[perm] = kc
+    vc2 = torch.empty_like(vc)
+    vc2[perm] = vc
+    t = case["block_tables"].long()
+    tb2 = torch.where(t >= 0, perm[t.clamp(min=0)], t).to(torch.int32)
+    assert torch.equal(out, ops.paged_attention(q, kc2, vc2, tb2, case["context_lens"], nh, nkv, scale))
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 10240, 8192), (16, 8192, 8192), (16, 59136, 8192), (16, 8192, 29568)])
+def test_w8a16_gemm_is_exact_on_an_integer_grid_long_context_shapes(m, n, k):
+    """The four projections of the Qwen2.5-72B shape at batch 16, exact as in the test above (computed in slabs of
+    output channels to bound host memory)."""
+    from mindformers_amd import ops
+    rng = np.random.default_rng(n + k)
+    wq = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    s = (2.0 ** rng.integers(-12, -9, n)).astype(np.float32)
+    x = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    y = to_np(ops.w8a16_linear(dev(x, BF), torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())).astype(np.float64)
+    x64 = x.astype(np.float64)
+    for c0 in range(0, n, 4096):
+        exact = (x64 @ wq[c0:c0 + 4096].astype(np.float64).T) * s[c0:c0 + 4096]
+        assert np.array_equal(y[:, c0:c0 + 4096], rounded(exact, BF).astype(np.float64)), c0
+
+
+def test_long_context_layer_step_stage_by_stage(qwen72_case):
+    """One layer of the Qwen2.5-72B long-context stack (hidden 8192, FFN 29568, batch 16) stage by stage; the attention
+    stage on two of the sequences."""
+    _w8a16_stages(qwen72_case, 16, attn_rows=2)
+
+
+# ------------------------------------------------------------------------------ DeepSeek-V3 MoE layer at full shape
+@pytest.fixture(scope="module")
+def moe_case():
+    """128 bf16 tokens, hidden 7168, 256 routed experts of FFN 2048 + one shared expert, N(0, 0.02) weights quantised
+    per output channel, router logits N(0, 1), top-8 of 4 of 8 groups."""
+    from mindformers_amd import ops, synthetic
+    T, H, E, F = 128, 7168, 256, 2048
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(21)
+    w1 = torch.empty(E, 2 * F, H, dtype=torch.int8, device="cuda")
+    s1 = torch.empty(E, 2 * F, dtype=torch.float32, device="cuda")
+    w2 = torch.empty(E, H, F, dtype=torch.int8, device="cuda")
+    s2 = torch.empty(E, H, dtype=torch.float32, device="cuda")
+    for e in range(E):
+        w1[e], s1[e] = synthetic.quantize_weight_int8(torch.randn(2 * F, H, generator=gen, device="cuda") * 0.02)
+        w2[e], s2[e] = synthetic.quantize_weight_int8(torch.randn(H, F, generator=gen, device="cuda") * 0.02)
+    sh1, sh1s = synthetic.quantize_weight_int8(torch.randn(2 * F, H, generator=gen, device="cuda") * 0.02)
+    sh2, sh2s = synthetic.quantize_weight_int8(torch.randn(H, F, generator=gen, device="cuda") * 0.02)
+    case = dict(T=T, H=H, E=E, F=F, w1=w1, s1=s1, w2=w2, s2=s2, sh1=sh1, sh1s=sh1s, sh2=sh2, sh2s=sh2s,
+                p1=ops.pack_w8a16(w1, s1), p2=ops.pack_w8a16(w2, s2),
+                ps1=ops.pack_w8a16_gated(sh1, sh1s, "halves"), ps2=ops.pack_w8a16(sh2, sh2s),
+                x=torch.randn(T, H, generator=gen, device="cuda").to(BF),
+                logits=torch.randn(T, E, generator=gen, device="cuda"),
+                bias=torch.randn(E, generator=gen, device="cuda") * 0.1)
+    yield case
+    case.clear()
+    torch.cuda.empty_cache()
+
+
+def test_moe_layer_step_stage_by_stage_against_the_oracle(moe_case):
+    """Router -> permute -> grouped fc1 -> SiLU * mul -> grouped fc2 -> weighted unpermute + shared expert at the
+    DeepSeek-V3 shape.  Index outputs are bit-exact on all tokens; the expert projections are compared with the
+    oracle on the rows of a sample of experts, the combine and the shared expert on all tokens, every stage on the
+    inputs the GPU fed it; and a sample of tokens end to end against the dense sum_k w * MLP_e(x)."""
+    from oracle import dense as Dn
+    from oracle import quant as Q
+    from oracle.layer import _r
+    from helpers import assert_within
+    from mindformers_amd import ops
+    c = moe_case
+    T, H, E, F = c["T"], c["H"], c["E"], c["F"]
+    x = c["x"]
+    wgt, idx = ops.moe_route(c["logits"], c["bias"], 8, 8, 4, 2.5, BF)
+    w_ref, idx_ref = O.topk_router(to_np(c["logits"]), to_np(c["bias"]), 8, 8, 4, 2.5)
+    assert np.array_equal(to_np(idx), idx_ref)
+    assert_within(to_np(wgt), w_ref, np.abs(w_ref), BF, ulps=1.0, what="router weights")
+    px, row_map, counts, offsets = ops.moe_permute(x, idx, E)
+    px_ref, map_ref, cnt_ref = O.moe_permute(to_np(x), idx_ref, E)
+    assert np.array_equal(to_np(row_map), map_ref) and np.array_equal(to_np(counts), cnt_ref)
+    off = np.concatenate(([0], np.cumsum(cnt_ref))).astype(np.int32)
+    assert np.array_equal(to_np(offsets), off) and np.array_equal(to_np(px), px_ref)
+    y1 = ops.grouped_w8a16_linear(px, c["p1"], offsets)
+    a = ops.silu_mul(y1)
+    y2 = ops.grouped_w8a16_linear(a, c["p2"], offsets)
+    busy = np.argsort(-cnt_ref)
+    sample = [int(e) for e in list(busy[:3]) + list(busy[len(busy) // 2:len(busy) // 2 + 3]) +
+              list(np.flatnonzero(cnt_ref > 0)[-3:])]
+    a_np = to_np(a).astype(np.float64)
+    for e in sample:
+        r0, r1 = int(off[e]), int(off[e + 1])
+        if r1 == r0:
+            continue
+        w1, s1 = to_np(c["w1"][e]), to_np(c["s1"][e])
+        ref = Q.w8a16_linear(px_ref[r0:r1], w1, s1)
+        mag = Q.w8a16_linear(np.abs(px_ref[r0:r1]), np.abs(w1), s1)
+        assert_within(to_np(y1[r0:r1]), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9,
+                      what=f"fc1 of expert {e}")
+        w2, s2 = to_np(c["w2"][e]), to_np(c["s2"][e])
+        ref = Q.w8a16_linear(a_np[r0:r1], w2, s2)
+        mag = Q.w8a16_linear(np.abs(a_np[r0:r1]), np.abs(w2), s2)
+        assert_within(to_np(y2[r0:r1]), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9,
+                      what=f"fc2 of expert {e}")
+    g = to_np(y1).astype(np.float64)
+    act_ref = _r(Dn.silu(g[:, :F]), "bf16") * g[:, F:]
+    assert_within(a_np, act_ref, np.abs(act_ref), BF, ulps=2.0, extra=1e-6, what="silu * up")
+    # shared expert: fused gate/up + activation, then the down projection
+    sa = ops.w8a16_gated_linear(x, c["ps1"])
+    su = ops.w8a16_linear(x, ops.pack_w8a16(c["sh1"], c["sh1s"]))
+    assert torch.equal(sa, ops.silu_mul(su))
+    xs = to_np(x).astype(np.float64)
+    ref = Q.w8a16_linear(xs, to_np(c["sh1"]), to_np(c["sh1s"]))
+    mag = Q.w8a16_linear(np.abs(xs), np.abs(to_np(c["sh1"])), to_np(c["sh1s"]))
+    assert_within(to_np(su), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="shared gate/up")
+    shared = ops.w8a16_linear(sa, c["ps2"])
+    san = to_np(sa).astype(np.float64)
+    ref = Q.w8a16_linear(san, to_np(c["sh2"]), to_np(c["sh2s"]))
+    mag = Q.w8a16_linear(np.abs(san), np.abs(to_np(c["sh2"])), to_np(c["sh2s"]))
+    assert_within(to_np(shared), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="shared down")
+    # weighted combine + shared
+    out = ops.moe_unpermute(y2, row_map, wgt, shared=shared)
+    routed = O.moe_unpermute(to_np(y2), map_ref, to_np(wgt))
+    ref = _r(routed, "bf16") + to_np(shared)
+    assert_within(to_np(out), ref, np.abs(ref) + np.abs(_r(routed, "bf16")), BF, ulps=1.5, extra=1e-6, what="unpermute")
+    # end to end on a sample of tokens: dense sum over the chosen experts, every intermediate rounded where the
+    # device writes it; a one-step difference of an intermediate reaches the output through 2048 / 7168-term sums, so
+    # the bound is a few steps of the row's scale
+    for t in (0, 17, 64, 127):
+        xt = xs[t:t + 1]
+        acc = np.zeros((1, H))
+        for j in range(8):
+            e = int(idx_ref[t, j])
+            h1 = _r(Q.w8a16_linear(xt, to_np(c["w1"][e]), to_np(c["s1"][e])), "bf16")
+            at = _r(_r(Dn.silu(h1[:, :F]), "bf16") * h1[:, F:], "bf16")
+            acc += float(to_np(wgt)[t, j]) * _r(Q.w8a16_linear(at, to_np(c["w2"][e]), to_np(c["s2"][e])), "bf16")
+        h1 = _r(Q.w8a16_linear(xt, to_np(c["sh1"]), to_np(c["sh1s"])), "bf16")
+        at = _r(_r(Dn.silu(h1[:, :F]), "bf16") * h1[:, F:], "bf16")
+        e2e = _r(acc, "bf16") + _r(Q.w8a16_linear(at, to_np(c["sh2"]), to_np(c["sh2s"])), "bf16")
+        got = to_np(out[t:t + 1]).astype(np.float64)
+        tol = 4 * EPS[BF] * np.maximum(np.abs(e2e), 0.05 * np.abs(e2e).max()) + 1e-5
+        assert np.mean(np.abs(got - e2e) > tol) < 0.01, (t, np.abs(got - e2e).max())
+
+
+@pytest.mark.parametrize("n,k", [(4096, 7168), (7168, 2048)])
+def test_grouped_w8a16_gemm_is_exact_on_an_integer_grid(n, k):
+    """Both expert projections of the DeepSeek-V3 shape over 256 experts with ragged row groups (empty experts, one
+    with more than 16 rows): power-of-two scales and small-integer activations make the result exact."""
+    from mindformers_amd import ops
+    rng = np.random.default_rng(n)
+    e, rows = 256, 1024
+    cnt = rng.multinomial(rows - 40, np.ones(e) / e)
+    cnt[5] += 40
+    cnt[9] = cnt[200] = 0
+    rows = int(cnt.sum())
+    off = np.concatenate(([0], np.cumsum(cnt))).astype(np.int32)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(n)
+    wq = torch.randint(-127, 128, (e, n, k), dtype=torch.int8, generator=gen, device="cuda")
+    s = (2.0 ** rng.integers(-12, -9, (e, n))).astype(np.float32)
+    x = rng.integers(-3, 4, (rows, k)).astype(np.float32)
+    y = to_np(ops.grouped_w8a16_linear(dev(x, BF), ops.pack_w8a16(wq, torch.from_numpy(s).cuda()),
+                                       torch.from_numpy(off).cuda())).astype(np.float64)
+    for ex in range(e):
+        r0, r1 = int(off[ex]), int(off[ex + 1])
+        if r1 > r0:
+            # every partial sum is an integer below 3 * 127 * 7168 < 2^24: the float32 product is exact
+            exact = (x[r0:r1] @ wq[ex].cpu().numpy().astype(np.float32).T).astype(np.float64) * s[ex]
+            assert np.array_equal(y[r0:r1], rounded(exact, BF).astype(np.float64)), ex

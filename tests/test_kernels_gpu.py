@@ -169,6 +169,26 @@ def test_paged_attention_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi):
     assert_within(got, ref, mag, dtype, ulps=1.5, what="paged attention")
 
 
+@pytest.mark.parametrize("dtype,b,nh,nkv,d,bs,lens,max_blocks", [
+    # 17..64 partitions of 256 tokens (the combine kernel's branch for more than 16 partitions)
+    (torch.bfloat16, 3, 4, 1, 128, 128, [4097, 9000, 16384], 128),
+    (torch.float16, 2, 4, 2, 64, 64, [5000, 12345], 256),
+    # capacity above 16384 tokens: 512-token partitions (four tiles per wave)
+    (torch.bfloat16, 3, 8, 1, 128, 128, [17000, 20000, 300], 160),
+    (torch.float16, 2, 2, 1, 64, 128, [18000, 19999], 157),
+    (torch.bfloat16, 2, 8, 2, 128, 128, [32768, 16385], 256),
+    # head_dim 32 (half a wave of output columns) with more than 32 partitions, both partition sizes
+    (torch.bfloat16, 2, 2, 1, 32, 128, [8193, 12000], 100),
+    (torch.float16, 2, 2, 2, 32, 64, [20000, 17000], 320),
+])
+def test_paged_attention_long_contexts_vs_oracle(dtype, b, nh, nkv, d, bs, lens, max_blocks):
+    """Contexts of 4k-32k tokens against the oracle: many partitions per sequence, both partition sizes, every
+    branch of the kernel that combines them."""
+    rng = np.random.default_rng(sum(lens))
+    got, ref, mag = _pa_case(rng, dtype, b, nh, nkv, d, bs, np.asarray(lens), max_blocks=max_blocks)
+    assert_within(got, ref, mag, dtype, ulps=1.5, what="paged attention, long contexts")
+
+
 def test_paged_attention_edge_lengths():
     """L = 1 returns the V row; L = 0 returns zeros; L exactly on tile / partition / block boundaries."""
     rng = np.random.default_rng(11)
@@ -553,6 +573,26 @@ def test_paged_attention_int8kv_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi, with
     ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, sc)
     mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, sc)
     assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="paged attention over an int8 cache")
+
+
+def test_paged_attention_int8kv_empty_sequence_in_a_short_table():
+    """A block table of 384 tokens is one partition for an int8 cache: the attention kernel writes the rows itself
+    and the row of a sequence without context must still come back as zeros."""
+    rng = np.random.default_rng(35)
+    dtype, nh, nkv, d, bs = torch.bfloat16, 8, 2, 128, 128
+    lens = np.array([0, 300, 384, 7])
+    k8, v8, kf, vf, tables, nb, scale, offset = _kv8_case(rng, dtype, 4, nh, nkv, d, bs, np.maximum(lens, 1), True,
+                                                          max_blocks=3)
+    q = rounded(rng.normal(size=(4, nh * d)), dtype)
+    sc = 1.0 / np.sqrt(d)
+    out = torch.full((4, nh * d), 7.0, dtype=dtype, device="cuda")
+    ops.paged_attention_int8kv(dev(q, dtype), torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda(),
+                               dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32),
+                               dev(scale, torch.float32), dev(offset, torch.float32), nh, nkv, sc, out=out)
+    ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, sc)
+    mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, sc)
+    assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="int8 cache, one partition")
+    assert np.all(to_np(out)[0] == 0)
 
 
 def test_paged_prefill_int8kv_vs_oracle():
