@@ -104,6 +104,22 @@ int mf_paged_attention_decode_dynamic_quant(void* out, int8_t* xq, float* x_scal
                                             int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                                             int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mf_paged_attention_decode for callers that cannot allocate or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments and same result bits as mf_paged_attention_decode, minus workspace / workspace_bytes: the partition
+ * partials go to a device array built into the library (MF_PA_STATIC_SCRATCH_BYTES per GPU, held until the
+ * process ends).  Shapes whose mf_paged_attention_workspace_bytes exceeds that size are rejected with
+ * hipErrorInvalidValue and a message.  The call allocates and frees nothing; the first call on a device looks up
+ * the array's address (make that call outside a stream capture).  All calls on one GPU share the one array:
+ * calls that may overlap on a GPU (different streams, different host threads) race on it and must be serialised
+ * by the caller. */
+#define MF_PA_STATIC_SCRATCH_BYTES (48u << 20)
+int mf_paged_attention_decode_static(void* out, const void* query, const void* key_cache, const void* value_cache,
+                                     const int32_t* block_tables, const int32_t* context_lens, int batch,
+                                     int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                     int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
+                                     int dtype, void* stream);
+
 /* ---- int8 KV cache (kvcache_dtype = int8, per-channel) ------------------------------------------------ */
 
 /* The reference sizes an int8 cache (mindformers/model_runner.py:364-368, kvcache_dtype in the quantization

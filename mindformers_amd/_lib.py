@@ -27,6 +27,7 @@ SIGNATURES = {
     "mf_paged_attention_decode_dynamic_quant": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                                      _F, _L, _I, _P, _Z, _P]),
     "mf_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P, _Z, _P]),
+    "mf_paged_attention_decode_static": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P]),
     "mf_quant_reshape_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _P]),
     "mf_paged_attention_decode_int8kv": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P,
                                               _Z, _P]),

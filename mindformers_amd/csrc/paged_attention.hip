@@ -21,6 +21,8 @@
 //                                                    the transposing LDS read (ds_read_b64_tr_b16)
 //   The 4 waves are merged through LDS and the workgroup writes either the final rows (single partition)
 //   or an fp32 partial (acc, max, sum) that a small second kernel combines.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -1464,4 +1466,52 @@ extern "C" int mf_paged_attention_decode_int8kv(void* out, const void* query, co
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
                            dtype, workspace, workspace_bytes, stream, true, antiquant_scale, antiquant_offset);
+}
+
+// ---- decode attention for callers that cannot allocate ----------------------------------------------------------
+// The partition partials live in a file-scope device array in place of a caller workspace.  Every GPU the library
+// runs on holds its own copy of the array (at its own address) until the process ends; the host-side name of the
+// array is not a device address, so the address is asked for once per device and kept.
+static __device__ __align__(256) unsigned char scratch[MF_PA_STATIC_SCRATCH_BYTES];
+
+static int pa_static_scratch(void** ptr_out) {
+    static std::mutex mu;
+    static void* dev_ptr[MF_MAX_DEVICES] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    MF_REQUIRE(dev >= 0 && dev < MF_MAX_DEVICES, "paged_attention_decode_static: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!dev_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        MF_REQUIRE(p != nullptr, "paged_attention_decode_static: no address for the scratch array");
+        dev_ptr[dev] = p;
+    }
+    *ptr_out = dev_ptr[dev];
+    return 0;
+}
+
+extern "C" int mf_paged_attention_decode_static(void* out, const void* query, const void* key_cache,
+                                                const void* value_cache, const int32_t* block_tables,
+                                                const int32_t* context_lens, int batch, int n_heads, int n_kv_heads,
+                                                int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                                                float scale, int64_t q_row_stride, int dtype, void* stream) {
+    MF_REQUIRE(batch >= 0 && n_heads > 0 && head_dim > 0 && block_size > 0 && max_blocks_per_seq > 0,
+               "paged_attention_decode_static: bad shape");
+    MF_REQUIRE((int64_t)block_size * max_blocks_per_seq <= 0x7fffffffLL,
+               "paged_attention_decode_static: context capacity overflows int");
+    const size_t need = mf_paged_attention_workspace_bytes(batch, n_heads, head_dim, max_blocks_per_seq * block_size);
+    MF_REQUIRE(need <= (size_t)MF_PA_STATIC_SCRATCH_BYTES,
+               "paged_attention_decode_static: batch %d x %d heads x %d context tokens needs %zu bytes of partition "
+               "partials, the built-in scratch holds %zu; use mf_paged_attention_decode with a workspace",
+               batch, n_heads, max_blocks_per_seq * block_size, need, (size_t)MF_PA_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    const int rc = pa_static_scratch(&ws);
+    if (rc) return rc;
+    // every partial a row's combine reads is written by this call's attention kernel first: nothing to clear
+    return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
+                           n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
+                           dtype, ws, (size_t)MF_PA_STATIC_SCRATCH_BYTES, stream, false, nullptr, nullptr);
 }
