@@ -1,26 +1,34 @@
-"""AutoQuantizationConfig / AutoQuantizer — mindformers/modules/quantizers/auto.py:30-114."""
+"""AutoQuantizationConfig / AutoQuantizer: pick the config class and the quantizer class from the ``quant_method``
+string of a quantization config (the dispatch surface of mindformers/modules/quantizers/auto.py:30-114)."""
 from ...quantization_config import PtqConfig, QuantizationConfigMixin, RtnConfig, SmoothQuantConfig
 from .ptq_quantizer import PtqQuantizer
 from .rtn_quantizer import RtnQuantizer
 from .smooth_quant_quantizer import SmoothQuantQuantizer
 
-AUTO_QUANTIZER_MAPPING = {"ptq": PtqQuantizer, "rtn": RtnQuantizer, "smooth_quant": SmoothQuantQuantizer}
-AUTO_QUANTIZATION_CONFIG_MAPPING = {"ptq": PtqConfig, "rtn": RtnConfig, "smooth_quant": SmoothQuantConfig}
+# one registry: method name -> (config class, quantizer class); the two public mappings are its columns
+_METHODS = {"ptq": (PtqConfig, PtqQuantizer), "rtn": (RtnConfig, RtnQuantizer),
+            "smooth_quant": (SmoothQuantConfig, SmoothQuantQuantizer)}
+AUTO_QUANTIZATION_CONFIG_MAPPING = {name: pair[0] for name, pair in _METHODS.items()}
+AUTO_QUANTIZER_MAPPING = {name: pair[1] for name, pair in _METHODS.items()}
 
 __all__ = ["AutoQuantizationConfig", "AutoQuantizer"]
+
+
+def _method_entry(quant_method):
+    if quant_method is None:
+        raise ValueError("quantization config carries no `quant_method`; it must name one of "
+                         f"{sorted(_METHODS)} (is this checkpoint quantized at all?)")
+    try:
+        return _METHODS[quant_method]
+    except (KeyError, TypeError):
+        raise ValueError(f"quant_method {quant_method!r} is not one of the built methods {sorted(_METHODS)}") from None
 
 
 class AutoQuantizationConfig:
     @classmethod
     def from_dict(cls, quantization_config_dict):
-        quant_method = quantization_config_dict.get("quant_method", None)
-        if quant_method is None:
-            raise ValueError("The model's quantization config from the arguments has no `quant_method` attribute. "
-                             "Make sure that the model has been correctly quantized")
-        if quant_method not in AUTO_QUANTIZATION_CONFIG_MAPPING:
-            raise ValueError(f"Unknown quantization type, got {quant_method} - supported types are:"
-                             f" {list(AUTO_QUANTIZER_MAPPING.keys())}")
-        return AUTO_QUANTIZATION_CONFIG_MAPPING[quant_method].from_dict(quantization_config_dict)
+        config_cls, _ = _method_entry(quantization_config_dict.get("quant_method"))
+        return config_cls.from_dict(quantization_config_dict)
 
     @classmethod
     def from_pretrained(cls, pretrained_model_name_or_path, **kwargs):
@@ -33,11 +41,8 @@ class AutoQuantizer:
     def from_config(cls, quantization_config, **kwargs):
         if isinstance(quantization_config, dict):
             quantization_config = AutoQuantizationConfig.from_dict(quantization_config)
-        quant_method = quantization_config.quant_method
-        if quant_method not in AUTO_QUANTIZER_MAPPING:
-            raise ValueError(f"Unknown quantization type, got {quant_method} - supported types are:"
-                             f" {list(AUTO_QUANTIZER_MAPPING.keys())}")
-        return AUTO_QUANTIZER_MAPPING[quant_method](quantization_config, **kwargs)
+        _, quantizer_cls = _method_entry(quantization_config.quant_method)
+        return quantizer_cls(quantization_config, **kwargs)
 
     @classmethod
     def from_pretrained(cls, pretrained_model_name_or_path, **kwargs):

@@ -13,6 +13,7 @@ from ._lib import check, dtype_code, ptr, stream_ptr
 
 _ACT = (torch.bfloat16, torch.float16)
 _workspaces = {}
+_retired = []                                 # outgrown workspaces, kept alive (see workspace())
 
 
 def _need(cond, msg):
@@ -56,11 +57,16 @@ def _dev_of(*tensors):
 
 
 def workspace(nbytes, device, tag="default"):
-    """A cached per-device scratch buffer (grown on demand, never shrunk)."""
-    key = (device, tag)
+    """A cached scratch buffer per (device, stream, purpose), grown on demand and never shrunk.  Two streams never
+    share one (their kernels would race on the partial sums), and a buffer that is outgrown is kept alive rather than
+    freed: a captured HIP graph may still replay into its address."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream, tag)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        if buf is not None:
+            _retired.append(buf)
+        size = max(int(nbytes), 256, 2 * buf.numel() if buf is not None else 0)
+        buf = torch.empty(size, dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
 
