@@ -22,6 +22,19 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0         # MI355X published dense int8 MFMA rate
+
+# metric string per workload; the default workload carries the headline metric
+METRICS = {
+    "llama3_8b_w8a16": "decode tokens/sec per layer (Llama3-8B shape, W8A16, bs64); % of peak HBM GB/s",
+    "llama3_8b_w8a16_kv8": "decode tokens/sec per layer (Llama3-8B shape, W8A16, int8 KV cache, bs64); % of peak HBM GB/s",
+    "tiny_llama_w8a16": "decode tokens/sec per layer (tiny Llama shape, W8A16, bs4); % of peak HBM GB/s",
+    "qwen2_5_7b_w8a8": "decode tokens/sec per layer (Qwen2.5-7B shape, W8A8, bs256); % of peak int8 MFMA TOP/s",
+    "qwen2_5_72b_w8a16": "decode tokens/sec per layer (Qwen2.5-72B shape, W8A16, bs16, ctx 16k-32k); % of peak HBM GB/s",
+    "deepseek_v3_moe_w8a16": "MoE layer tokens/sec (DeepSeek-V3 shape, 256 experts W8A16, 128 tokens); % of peak HBM GB/s",
+}
+TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+ATTENTION_SOURCE = os.path.join(ROOT, "mindformers_amd", "csrc", "paged_attention.hip")
 
 
 def log(*a):
@@ -102,9 +115,63 @@ def kernel_breakdown(case, torch, ops, iters):
     return out
 
 
-# (workload, algorithmic KV bytes) -> HBM bytes per attention launch (main kernel + partition reduce) read from
-# FETCH_SIZE / WRITE_SIZE: (289941.0 + 4902.0) KiB x 2.000 + (10130.6 + 512.0) KiB x 1.000
-MEASURED_TRAFFIC_BYTES = {("llama3_8b_w8a16", 589434880): int((294843.0 * 2.0 + 10642.6) * 1024)}
+def source_sha256(path):
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
+def measured_traffic(workload, kv_bytes):
+    """HBM bytes per attention launch from the committed counter record (FETCH_SIZE / WRITE_SIZE of a profiler run,
+    scaled by a known-size kernel).  Valid only for the workload, the KV byte count and the kernel source it was
+    taken on: otherwise (None, why)."""
+    try:
+        with open(TRAFFIC_RECORD) as f:
+            rec = json.load(f)["paged_attention"]
+    except (OSError, KeyError, ValueError):
+        return None, "no counter record under profiles/"
+    if rec.get("workload") != workload or rec.get("kv_bytes") != kv_bytes:
+        return None, "the counter record covers another workload"
+    if rec.get("kernel_source_sha256") != source_sha256(ATTENTION_SOURCE):
+        return None, "the attention kernel source changed since the counters were read (record of commit %s)" % rec.get("commit")
+    return int(rec["traffic_bytes"]), "profiles/hbm_traffic.json, commit %s" % rec.get("commit")
+
+
+def record_traffic(fetch_csv, write_csv, workload, kv_bytes):
+    """Write profiles/hbm_traffic.json from the counter_collection CSVs of two profiler runs of this benchmark with
+    --calibrate-counters (one with --pmc FETCH_SIZE, one with --pmc WRITE_SIZE): mean counter value per dispatch of
+    the attention kernels, each scaled by what the same counter reads for add_kernel on 2 x 128 MiB inputs."""
+    import csv
+    import subprocess
+
+    def means(path, counter):
+        acc = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") != counter:
+                    continue
+                acc.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    def pick(table, needle, exclude=None):
+        hits = [v for k, v in table.items() if needle in k and not (exclude and exclude in k)]
+        if not hits:
+            raise SystemExit(f"no dispatch of {needle} in the counter file")
+        return hits[0]
+    fetch, write = means(fetch_csv, "FETCH_SIZE"), means(write_csv, "WRITE_SIZE")
+    f_scale = 262144.0 / pick(fetch, "add_kernel")             # add_kernel reads 2 x 128 MiB, writes 128 MiB
+    w_scale = 131072.0 / pick(write, "add_kernel")
+    kib = (pick(fetch, "paged_attention_kernel") + pick(fetch, "paged_attention_reduce_kernel")) * f_scale + \
+          (pick(write, "paged_attention_kernel") + pick(write, "paged_attention_reduce_kernel")) * w_scale
+    commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    rec = {"paged_attention": {"workload": workload, "kv_bytes": int(kv_bytes), "traffic_bytes": int(kib * 1024),
+                               "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4),
+                               "commit": commit or "unknown", "kernel_source": "mindformers_amd/csrc/paged_attention.hip",
+                               "kernel_source_sha256": source_sha256(ATTENTION_SOURCE)}}
+    with open(TRAFFIC_RECORD, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    log(f"[bench] wrote {TRAFFIC_RECORD}: {rec['paged_attention']['traffic_bytes']} bytes per launch")
 
 
 def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
@@ -138,28 +205,160 @@ def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
     sin = case["sin"][idx].float().cpu().numpy()
     ocfg = dict(n_head=cfg["n_head"], n_kv_head=cfg["n_kv_head"], head_dim=cfg["head_dim"], eps=1e-5)
     act = "bf16" if cfg["dtype"] == torch.bfloat16 else "fp16"
-    fn = O.decode_layer_w8a8 if cfg["act_quant"] else O.decode_layer_w8a16
+    got = gpu_out[idx].float().cpu().numpy()
     if cfg["act_quant"]:
+        # W8A8: the numpy restatement (float64 dequantisation around exact integer accumulators)
         for n in layer.NAMES:
             p[n + "_smooth"] = getattr(layer, n + "_smooth").cpu().numpy()
-    try:
-        from threadpoolctl import threadpool_info
-        cores = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
-    except Exception:
-        cores = 1
-    passes, dt = 0, 0.0
-    while passes < 16 and dt < min_seconds:        # every pass rewrites the same cache slots with the same rows: identical work
-        t0 = time.perf_counter()
-        ref = fn(x, p, ocfg, kcn, vcn, t2, lens, slots2, cos, sin, act_dtype=act)
-        dt += time.perf_counter() - t0
-        passes += 1
-    got = gpu_out[idx].float().cpu().numpy()
+        try:
+            from threadpoolctl import threadpool_info
+            cores = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+        except Exception:
+            cores = 1
+        passes, dt = 0, 0.0
+        while passes < 16 and dt < min_seconds:    # every pass rewrites the same cache slots with the same rows: identical work
+            t0 = time.perf_counter()
+            ref = O.decode_layer_w8a8(x, p, ocfg, kcn, vcn, t2, lens, slots2, cos, sin, act_dtype=act)
+            dt += time.perf_counter() - t0
+            passes += 1
+        how = "numpy float64"
+    else:
+        # W8A16: the same layer restated with torch on the host in float32 on all cores (oracle/torch_cpu.py, held to
+        # the float64 oracle by the CPU tests); weights widened to float32 once, outside the timed passes
+        from oracle import torch_cpu
+        cores = torch.get_num_threads()
+        tp = torch_cpu.prepare_params(p)
+        xt, ct, st = torch.from_numpy(x), torch.from_numpy(cos), torch.from_numpy(sin)
+        kct, vct = torch.from_numpy(kcn), torch.from_numpy(vcn)
+        passes, dt = 0, 0.0
+        while passes < 256 and dt < min_seconds:
+            t0 = time.perf_counter()
+            ref = torch_cpu.decode_layer_w8a16_fp32(xt, tp, ocfg, kct, vct, t2, lens, slots2, ct, st, act_dtype=act)
+            dt += time.perf_counter() - t0
+            passes += 1
+        ref = ref.numpy()
+        how = "torch float32 on the host"
     err = float(np.abs(got - ref).max())
     scale = float(np.abs(ref).max())
     return dict(value=len(idx) * passes / dt, unit="tokens/s", cores=int(cores), kind="port",
                 sample=f"{passes} passes of one layer step for {len(idx)} of the {cfg['batch']} sequences "
-                       f"({int(lens.sum())} context tokens), numpy float64, {dt:.1f} s in all"), dict(
+                       f"({int(lens.sum())} context tokens), {how}, {dt:.1f} s in all"), dict(
         max_abs_err=err, ref_max_abs=scale, rows=len(idx))
+
+
+def int8_gemm_roofline(case, torch, ops, iters):
+    """The four int8 GEMMs of a W8A8 layer step (QKV, output, gate/up, down projection), each timed with events on
+    the launch stream on the operands the layer feeds it: int8 ops (2 M N K, summed) over the summed durations
+    against the dense int8 MFMA peak."""
+    layer = case["layers"][0]
+    kc, vc = case["caches"][0]
+    x = case["x"]
+    m = x.shape[0]
+    n1q = ops.rms_norm_dynamic_quant(x, layer.attn_norm, layer.eps, layer.qkv_smooth, tiled=True)
+    qkv = ops.w8a8_linear(n1q[0], n1q[1], layer._packed["qkv"], out_dtype=layer.dtype)
+    attn_q = ops.dynamic_quant(qkv[:, :layer.n_head * layer.head_dim].contiguous(), layer.wo_smooth, tiled=True)
+    h = ops.w8a8_linear(attn_q[0], attn_q[1], layer._packed["wo"], out_dtype=layer.dtype, residual=x)
+    n2q = ops.rms_norm_dynamic_quant(h, layer.ffn_norm, layer.eps, layer.fc1_smooth, tiled=True)
+    gu = ops.w8a8_linear(n2q[0], n2q[1], layer._packed["fc1"], out_dtype=layer.dtype)
+    aq = ops.silu_mul_dynamic_quant(gu, layer.fc2_smooth, tiled=True)
+    calls = {
+        "qkv": lambda: ops.w8a8_linear(n1q[0], n1q[1], layer._packed["qkv"], out_dtype=layer.dtype),
+        "wo": lambda: ops.w8a8_linear(attn_q[0], attn_q[1], layer._packed["wo"], out_dtype=layer.dtype, residual=x),
+        "gate_up": lambda: ops.w8a8_linear(n2q[0], n2q[1], layer._packed["fc1"], out_dtype=layer.dtype),
+        "down": lambda: ops.w8a8_linear(aq[0], aq[1], layer._packed["fc2"], out_dtype=layer.dtype, residual=h),
+    }
+    shapes = {"qkv": layer._packed["qkv"], "wo": layer._packed["wo"], "gate_up": layer._packed["fc1"],
+              "down": layer._packed["fc2"]}
+    us, total_ops, weight_bytes = {}, 0.0, 0
+    for name, fn in calls.items():
+        for _ in range(5):
+            fn()
+        us[name] = round(time_events(fn, iters, torch)[0] * 1e3, 2)
+        total_ops += 2.0 * m * shapes[name].n * shapes[name].k
+        weight_bytes += shapes[name].n * shapes[name].k
+    total_us = sum(us.values())
+    ach = total_ops / (total_us * 1e-6) / 1e12
+    return dict(bound="mfma", kernel="int8 GEMMs of the layer step (w8a8_wide_kernel / w8a8_gemm_kernel / w8a8_regs_kernel "
+                                     "+ split-K reduce): qkv, wo, gate/up, down", achieved=round(ach, 1),
+                peak=INT8_PEAK_TOPS, unit="TOP/s", frac=round(ach / INT8_PEAK_TOPS, 4), traffic=None,
+                ops_per_step=total_ops, avg_launch_us=round(total_us, 2), per_gemm_us=us,
+                weight_stream_gbps=round(weight_bytes / (total_us * 1e-6) / 1e9, 1))
+
+
+def bench_modules(case, torch, ops, args):
+    """The same decode-layer step composed from the drop-in cells a user of the reference's module surface gets, one
+    launch per primitive and nothing fused across cells: LlamaRMSNorm -> WeightQuantLinearCell (QKV) -> InferAttention
+    (RoPE + cache scatter + paged attention on the manager's own caches) -> WeightQuantLinearCell (+ residual) ->
+    LlamaRMSNorm -> WeightQuantLinearCell (gate/up) -> SiLU * mul -> WeightQuantLinearCell (+ residual).  Timed like the
+    fused layer (HIP graph of chained steps) so that the cost of not adopting the fused entry points is on record."""
+    from mindformers_amd.modules import InferAttention, LlamaRMSNorm
+    from mindformers_amd.modules.layers import WeightQuantLinearCell
+    cfg, layer = case["cfg"], case["layers"][0]
+    if layer.act_quant or cfg.get("kv_int8"):
+        return {"skipped": "the module leg covers the W8A16 layer with 16-bit caches"}
+    dt, dev = cfg["dtype"], case["x"].device
+    kc, vc = case["caches"][0]
+    cells = {}
+    for name in layer.NAMES:
+        w = getattr(layer, name + "_w")
+        cell = WeightQuantLinearCell(w.shape[1], w.shape[0], False, dt, device="meta")
+        cell.weight, cell.w_scale = w.to(dev), getattr(layer, name + "_s")
+        cell.prepare()
+        cell.weight = w                                         # the packed copy is what the kernels read
+        cells[name] = cell
+    norm1, norm2 = LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev), LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev)
+    norm1.weight.data, norm2.weight.data = layer.attn_norm, layer.ffn_norm
+    att = InferAttention(cfg["n_head"], cfg["head_dim"], cfg["n_kv_head"], scale_value=layer.scale_value,
+                         block_size=cfg["block_size"], num_blocks=1, rotary_cos_format=2, compute_dtype=dt, device=dev)
+    att.paged_attention_mgr.key_cache, att.paged_attention_mgr.value_cache = kc, vc     # the case's caches, not a copy
+    att.is_first_iteration = False
+    nq, nkv = cfg["n_head"] * cfg["head_dim"], cfg["n_kv_head"] * cfg["head_dim"]
+    freqs = (case["cos"], case["sin"], None)
+
+    def step(x):
+        qkv = cells["qkv"](norm1(x))
+        a = att(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], case["context_lens"], case["block_tables"],
+                case["slot_mapping"], freqs)
+        h = cells["wo"](a, residual=x)
+        return cells["fc2"](ops.silu_mul(cells["fc1"](norm2(h))), residual=h)
+    ref = layer(case["x"], kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    out = step(case["x"])
+    same = bool(torch.equal(out, ref))
+    per = next(g for g in (8, 4, 2, 1) if args.steps % g == 0)
+
+    def chain():
+        h = case["x"]
+        for _ in range(per):
+            h = step(h)
+        return h
+    launch = "eager"
+    fn = chain
+    if not args.no_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    chain()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                chain()
+            fn, launch = g.replay, f"hip_graph, {per} chained layer steps per replay"
+        except Exception as e:
+            log(f"[bench] module leg: graph capture unavailable ({e}); timing eager launches")
+    for _ in range(max(1, args.warmup // per)):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps // per):
+        fn()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    return {"ms_per_step": round(ms, 4), "tokens_per_s": round(cfg["batch"] / (ms * 1e-3), 1), "launch": launch,
+            "bit_identical_to_fused_layer": same,
+            "composition": "LlamaRMSNorm, WeightQuantLinearCell x4, InferAttention, silu_mul"}
 
 
 def bench_moe(args, torch, ops, _lib):
@@ -222,7 +421,7 @@ def bench_moe(args, torch, ops, _lib):
     g2 = timed(lambda: ops.grouped_w8a16_linear(a, w2, offsets))
     ach = n_act * per_expert / ((g1 + g2) * 1e-3) / 1e9
     result = {
-        "metric": "decode tokens/sec per layer (Llama3-8B shape, W8A16, bs64); % of peak HBM GB/s",
+        "metric": METRICS["deepseek_v3_moe_w8a16"],
         "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
@@ -355,6 +554,12 @@ def main():
     ap.add_argument("--workload", default="llama3_8b_w8a16")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--modules", action="store_true",
+                    help="also time the step composed from the drop-in module cells (default for the headline workload)")
+    ap.add_argument("--no-modules", action="store_true", help="skip the drop-in module leg")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter_collection CSVs of two profiler runs of this command with "
+                         "--calibrate-counters (--pmc FETCH_SIZE, --pmc WRITE_SIZE) into profiles/hbm_traffic.json")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-iters", type=int, default=50)
     ap.add_argument("--calibrate-counters", action="store_true",
@@ -365,6 +570,14 @@ def main():
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the decode path has no "
               "collectives and no multi-GPU figure is produced.", file=sys.stderr)
         sys.exit(2)
+
+    if args.record_traffic:
+        from mindformers_amd import synthetic as syn
+        cfg = syn.CONFIGS[args.workload]
+        kv = int(syn.context_lens(args.workload, seed=1).astype(np.int64).sum()) * 2 * cfg["n_kv_head"] * cfg["head_dim"] * \
+            (1 if cfg.get("kv_int8") else 2)
+        record_traffic(args.record_traffic[0], args.record_traffic[1], args.workload, kv)
+        return
 
     import torch
     if not torch.cuda.is_available():
@@ -467,15 +680,23 @@ def main():
     achieved = nbytes["kv"] / (attn_ms * 1e-3) / 1e9
     # HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE of a profiler run of this command,
     # scaled by a known-size kernel); only valid for the exact workload it was collected on
-    traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, nbytes["kv"]))
+    traffic, traffic_note = measured_traffic(args.workload, nbytes["kv"])
     roofline = dict(bound="hbm", kernel="paged_attention_kernel (+ partition reduce)", achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=traffic,
-                    bytes_per_launch=nbytes["kv"], avg_launch_us=round(attn_ms * 1e3, 2))
+                    traffic_source=traffic_note, bytes_per_launch=nbytes["kv"], avg_launch_us=round(attn_ms * 1e3, 2))
     breakdown = kernel_breakdown(case, torch, ops, args.kernel_iters)
     layer_gbps = nbytes["total"] * n_layers / (ms_per_step * 1e-3) / 1e9
+    extra = {}
+    if cfg["act_quant"]:
+        # W8A8: the figure of merit is the int8 matrix rate of the four projections at this batch; the attention
+        # roofline moves to a second key
+        extra["attention_roofline"] = roofline
+        roofline = int8_gemm_roofline(case, torch, ops, args.kernel_iters)
+    if args.modules or (args.workload == "llama3_8b_w8a16" and not args.no_modules):
+        extra["drop_in_modules"] = bench_modules(case, torch, ops, args)
 
     result = {
-        "metric": "decode tokens/sec per layer (Llama3-8B shape, W8A16, bs64); % of peak HBM GB/s",
+        "metric": METRICS.get(args.workload, METRICS["llama3_8b_w8a16"]),
         "value": round(tokens_per_s_layer, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if cfg["dtype"] == torch.bfloat16 else "fp16", "data": "synthetic",
@@ -489,6 +710,7 @@ def main():
         "layer_hbm_gbps": round(layer_gbps, 1), "layer_hbm_frac": round(layer_gbps / HBM_PEAK_GBPS, 4),
         "roofline": roofline, "breakdown_us": breakdown,
     }
+    result.update(extra)
     if cfg.get("kv_int8"):
         result["config"]["kv_cache"] = "int8, per-channel scales"
     if not args.no_cpu and not cfg.get("kv_int8"):            # the CPU restatement of the layer covers 16-bit caches

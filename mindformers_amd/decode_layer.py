@@ -60,13 +60,18 @@ class QuantDecodeLayer(nn.Module):
             return ops.w8a8_linear(xq, xs, packed, out_dtype=self.dtype, bias=b, residual=residual)
         return ops.w8a16_linear(x, packed, bias=b, residual=residual)
 
-    def prepare(self):
-        """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights."""
+    def prepare(self, release_raw=True):
+        """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights.
+        The packed copy is the only one the kernels read: with ``release_raw`` the row-major ``*_w`` buffers move to
+        host memory afterwards (still readable, e.g. for export), so the device holds every weight once."""
+        dev = self.attn_norm.device
         for name in self.NAMES:
-            w, s = getattr(self, f"{name}_w"), getattr(self, f"{name}_s")
+            w, s = getattr(self, f"{name}_w").to(dev), getattr(self, f"{name}_s")
             # W8A16: the gate/up projection runs fused with SiLU * mul, which wants gate/up rows interleaved
             gated = name == "fc1" and not self.act_quant and getattr(self, "fc1_b") is None
             self._packed[name] = ops.pack_w8a16_gated(w, s, "halves") if gated else ops.pack_w8a16(w, s)
+            if release_raw:
+                self._buffers[f"{name}_w"] = w.cpu()
         return self
 
     def set_kv_quant(self, scale, offset=None):

@@ -48,7 +48,7 @@ def rope_rows(positions, head_dim, theta, dtype, device):
 
 def fill_layer(layer, gen, std=0.02):
     """Random N(0, std) weights quantised to int8, unit-ish norm gammas, smoothing vectors U[0.5, 2]."""
-    dev = layer.qkv_w.device
+    dev = layer.attn_norm.device
     for name in layer.NAMES:
         wq = getattr(layer, f"{name}_w")
         n, k = wq.shape
@@ -63,6 +63,13 @@ def fill_layer(layer, gen, std=0.02):
     layer.attn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
     layer.ffn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
     return layer.prepare()
+
+
+def context_lens(name, seed=0, batch=None, ctx=None):
+    """The context lengths make_decode_case draws for a named config (host only)."""
+    cfg = CONFIGS[name]
+    lo, hi = ctx if ctx is not None else cfg["ctx"]
+    return np.random.default_rng(seed).integers(lo, hi + 1, batch if batch is not None else cfg["batch"]).astype(np.int32)
 
 
 def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=None):

@@ -358,7 +358,7 @@ def _w8a16_stages(case, n, attn_rows=None):
     assert_within(to_np(n2[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=1e-6, what="MLP norm")
     # gate/up projection with the activation fused, against the unfused pair bit for bit and against the oracle
     a = layer.gate_up(n2)
-    gu = ops.w8a16_linear(n2, ops.pack_w8a16(layer.fc1_w, layer.fc1_s))
+    gu = ops.w8a16_linear(n2, ops.pack_w8a16(layer.fc1_w.cuda(), layer.fc1_s))
     assert torch.equal(a, ops.silu_mul(gu))
     ref, mag = olin(to_np(n2[:n]), "fc1")
     assert_within(to_np(gu[:n]), ref, np.abs(ref), BF, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="gate/up projection")

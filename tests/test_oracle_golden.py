@@ -247,3 +247,50 @@ def test_moe_layer_vectors(golden_dir, name, shared):
         act_dtype="bf16", router_dtype="bf16")
     got = R(y).astype(np.float16).astype(np.float32)
     np.testing.assert_allclose(got, z[f"golden_{name}"], rtol=4e-3, atol=2e-6)
+
+
+def test_float32_host_layer_follows_the_float64_oracle():
+    """oracle/torch_cpu.py (the float32 restatement that the benchmark times as its CPU baseline) against the
+    float64 oracle layer on a small W8A16 decode step: same rounding points, float32 in between, so the outputs agree
+    to a few steps of the activation dtype, and both write the same cache rows."""
+    import torch
+    from oracle import torch_cpu
+    rng = np.random.default_rng(3)
+    hidden, nh, nkv, d, ffn, b, bs = 256, 4, 2, 64, 352, 3, 16
+    lens = np.array([40, 17, 33])
+    p = {}
+    for name, (n, k) in {"qkv": ((nh + 2 * nkv) * d, hidden), "wo": (hidden, nh * d), "fc1": (2 * ffn, hidden),
+                         "fc2": (hidden, ffn)}.items():
+        p[name + "_w"], p[name + "_s"] = O.quantize_weight_int8(rng.normal(0, 0.05, (n, k)).astype(np.float32))
+    p["attn_norm"] = (1 + 0.1 * rng.normal(size=hidden)).astype(np.float32)
+    p["ffn_norm"] = (1 + 0.1 * rng.normal(size=hidden)).astype(np.float32)
+    cfg = dict(n_head=nh, n_kv_head=nkv, head_dim=d, eps=1e-5)
+    need = (lens + bs - 1) // bs
+    nb = int(need.sum()) + 2
+    perm = rng.permutation(nb)
+    tables = -np.ones((b, int(need.max())), np.int32)
+    pos = 0
+    for i, n in enumerate(need):
+        tables[i, :n] = perm[pos:pos + n]
+        pos += n
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    kc = O.round_bf16(rng.normal(size=(nb, bs, nkv, d)).astype(np.float32))
+    vc = O.round_bf16(rng.normal(size=(nb, bs, nkv, d)).astype(np.float32))
+    x = O.round_bf16(rng.normal(size=(b, hidden)).astype(np.float32))
+    cos, sin = O.rope_cos_sin_table(O.rope_inv_freq_default(d), 64, 1.0, "bf16")
+    cos, sin = cos[lens - 1], sin[lens - 1]
+    kc64, vc64 = kc.copy(), vc.copy()
+    ref = O.decode_layer_w8a16(x, p, cfg, kc64, vc64, tables, lens, slots, cos, sin, act_dtype="bf16")
+    kc32, vc32 = torch.from_numpy(kc.copy()), torch.from_numpy(vc.copy())
+    got = torch_cpu.decode_layer_w8a16_fp32(torch.from_numpy(x), torch_cpu.prepare_params(p), cfg, kc32, vc32, tables,
+                                            lens, slots, torch.from_numpy(cos.astype(np.float32)),
+                                            torch.from_numpy(sin.astype(np.float32)), act_dtype="bf16").numpy()
+    err = np.abs(got - ref)
+    tol = 4 * 2.0 ** -8 * np.maximum(np.abs(ref), 0.1 * np.abs(ref).max(axis=1, keepdims=True))
+    assert np.mean(err > tol) < 0.01 and err.max() < 0.1 * np.abs(ref).max(), (np.mean(err > tol), err.max())
+    row = nkv * d
+    written = np.zeros(nb * bs, bool)
+    written[slots] = True
+    assert np.array_equal(kc32.numpy().reshape(-1, row)[~written], kc.reshape(-1, row)[~written])
+    assert np.abs(kc32.numpy() - kc64).max() <= 2 * 2.0 ** -8 * np.abs(kc64).max()
+    assert np.abs(vc32.numpy() - vc64).max() <= 2 * 2.0 ** -8 * np.abs(vc64).max()
