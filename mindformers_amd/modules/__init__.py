@@ -7,5 +7,5 @@ from .layers import (AllQuantLinearInferCell, ColumnParallelLinear, Linear, QKVP
 from .mlp import MLP, LlamaFeedForward
 from .moe import GroupedMLP, MoELayer, QuantGroupedMLP, SharedExpertMLP, TopKRouter
 from .norm import LlamaRMSNorm, RMSNorm
-from .paged_attention_mgr import PagedAttentionMgr
+from .paged_attention_mgr import PagedAttentionMgr, QuantPagedAttentionMgr
 from .rotary import FreqsMgr, Llama3RotaryEmbedding, RotaryEmbedding, YaRNScalingRotaryEmbedding

@@ -100,13 +100,15 @@ class InferAttention(nn.Module):
         q2 = query.reshape(-1, self.n_head * self.head_dim).contiguous()
         k2 = key.reshape(-1, self.n_kv_head * self.head_dim).contiguous()
         v2 = value.reshape(-1, self.n_kv_head * self.head_dim).contiguous()
-        if self.use_rope_rotary_emb:
+        if self.use_rope_rotary_emb and mgr.key_cache.dtype != torch.int8:
             # RoPE + scatter of the rotated key and of value in one launch (infer_attention.py:445,453);
             # same-stream ordering stands in for ops.depend (:454)
             freqs_cos, freqs_sin, _ = freqs_cis
             ops.rope_and_cache(q2, k2, v2, freqs_cos.contiguous(), freqs_sin.contiguous(), mgr.key_cache,
                                mgr.value_cache, slot_mapping, self.n_head)
         else:
+            if self.use_rope_rotary_emb:                      # int8 caches: rotate, then the manager quantises
+                q2, k2 = self._apply_rotary_pos_emb(q2, k2, freqs_cis, batch_valid_length)
             mgr(k2, v2, slot_mapping, batch_valid_length)
         if self.chunk_prefill:                                # infer_attention.py:456-458
             return mgr.paged_attn(q2, batch_valid_length, block_tables, attn_mask=attn_mask,

@@ -61,3 +61,58 @@ class PagedAttentionMgr(nn.Module):
     def shard(self, parallel_config):
         """One GPU: nothing to shard (paged_attention_mgr.py:77-92 only sets layouts)."""
         return self
+
+
+class QuantPagedAttentionMgr(PagedAttentionMgr):
+    """The manager a quantizer swaps in for ``kvcache_dtype: int8`` (per channel): int8 caches of the same shape,
+    the quantising scatter, and attention that receives the dequantisation parameters where the reference's call
+    passes ``antiquant_scale`` / ``antiquant_offset`` (positions 6-7 of PagedAttention,
+    mindformers/modules/paged_attention_mgr.py:66-70; the cache dtype comes from the quantization config,
+    mindformers/model_runner.py:364-368).  The cell itself belongs to golden-stick in the reference stack, so the
+    parameter names are this build's: ``kv_scale`` / ``kv_offset`` float32 [2, n_kv_heads * head_dim] (keys, values),
+    x ~ (q - offset) * scale, loaded from the checkpoint or set with ``set_kv_quant``."""
+
+    def __init__(self, n_heads, head_dim, n_kv_heads, kv_shape, seq_length=-1, compute_dtype=torch.float16,
+                 parallel_decoding=False, chunk_prefill=False, device="cuda"):
+        super().__init__(n_heads, head_dim, n_kv_heads, (1,) + tuple(kv_shape[1:]), seq_length, compute_dtype,
+                         parallel_decoding, chunk_prefill, device)
+        self.compute_dtype = compute_dtype
+        self.register_buffer("key_cache", torch.zeros(kv_shape, dtype=torch.int8, device=device), persistent=False)
+        self.register_buffer("value_cache", torch.zeros(kv_shape, dtype=torch.int8, device=device), persistent=False)
+        row = n_kv_heads * head_dim
+        self.register_buffer("kv_scale", torch.ones(2, row, dtype=torch.float32, device=device))
+        self.register_buffer("kv_offset", torch.zeros(2, row, dtype=torch.float32, device=device))
+
+    @classmethod
+    def from_float(cls, mgr):
+        """A quantised manager with the geometry of a float one."""
+        kc = mgr.key_cache
+        return cls(mgr.n_heads, mgr.head_dim, mgr.n_kv_heads, tuple(kc.shape), mgr.seq_length, kc.dtype,
+                   mgr.parallel_decoding, mgr.chunk_prefill, kc.device)
+
+    def set_kv_quant(self, scale, offset=None):
+        self.kv_scale.copy_(scale.to(torch.float32))
+        if offset is None:
+            self.kv_offset.zero_()
+        else:
+            self.kv_offset.copy_(offset.to(torch.float32))
+        return self
+
+    def forward(self, key, value, slot_mapping, batch_valid_length=None):
+        return ops.quant_reshape_and_cache(key, value, self.key_cache, self.value_cache, slot_mapping, self.kv_scale,
+                                           self.kv_offset)
+
+    construct = forward
+
+    def paged_attn(self, query, batch_valid_length, block_tables, attn_mask=None, q_seq_lens=None):
+        shape = query.shape
+        q2 = query.reshape(-1, self.n_heads * self.head_dim)
+        starts = None
+        if self.parallel_decoding or self.chunk_prefill:
+            if q_seq_lens is None:
+                raise ValueError("parallel_decoding / chunk_prefill need q_seq_lens")
+            starts = ops.q_starts_from_lens(q_seq_lens)
+        out = ops.paged_attention_int8kv(q2, self.key_cache, self.value_cache, block_tables, batch_valid_length,
+                                         self.kv_scale, self.kv_offset, self.n_heads, self.n_kv_heads,
+                                         self.scale_value, q_starts=starts)
+        return out.reshape(shape)

@@ -8,6 +8,7 @@ import torch
 
 from ..layers import (LINEAR_TYPES, AllQuantLinearInferCell, WeightQuantLinearCell, linear_geometry)
 from ..moe import GroupedMLP, QuantGroupedMLP
+from ..paged_attention_mgr import PagedAttentionMgr, QuantPagedAttentionMgr
 
 
 class Quantizer(ABC):
@@ -100,8 +101,10 @@ def check_buildable(cfg):
         raise NotImplementedError(f"weight_dtype {cfg.weight_quant_dtype!r}: only int8 per-channel weights are built")
     if getattr(cfg, "weight_quant_granularity", "per_channel") != "per_channel":
         raise NotImplementedError("per_group weight quantisation is not built")
-    if cfg.kvcache_quant_dtype is not None:
-        raise NotImplementedError("int8 KV cache is not built")
+    if cfg.kvcache_quant_dtype not in (None, "int8"):
+        raise NotImplementedError(f"kvcache_dtype {cfg.kvcache_quant_dtype!r}: only an int8 KV cache is built")
+    if cfg.kvcache_quant_dtype == "int8" and getattr(cfg, "kvcache_quant_granularity", "per_channel") != "per_channel":
+        raise NotImplementedError("per_token int8 KV cache is not built (per_channel only)")
     if getattr(cfg, "precision_recovery", "none") != "none":
         raise NotImplementedError("GPTQ precision recovery has no deploy-time kernel here")
     if cfg.outliers_suppression not in ("none", "smooth"):
@@ -144,6 +147,11 @@ def convert_linears(model, cfg, layer_policies=None):
                     w = child.weight.data if getattr(child, "transpose_b", True) else child.weight.data.t()
                     cell.quantize_from_float(w, child.bias.data if has_bias else None)
                 setattr(parent, child_name, cell)
+            elif (isinstance(child, PagedAttentionMgr) and not isinstance(child, QuantPagedAttentionMgr)
+                  and pol.kvcache_quant_dtype == "int8"):
+                # kvcache_dtype: int8 - the manager owns int8 caches and hands the attention its dequantisation
+                # parameters (filled from the checkpoint)
+                setattr(parent, child_name, QuantPagedAttentionMgr.from_float(child))
             elif isinstance(child, GroupedMLP):
                 if pol.act_quant_dtype == "int8":
                     raise NotImplementedError("W8A8 experts are not built (W8A16 grouped GEMM only)")

@@ -32,7 +32,8 @@ class DecodeStackRunner:
     ``layers``: prepared ``QuantDecodeLayer``s.  ``npu_mem_size`` / ``cpu_mem_size`` are GiB, as in the reference;
     ``rope_theta`` builds the rotary rows from the positions of each step."""
 
-    def __init__(self, layers, npu_mem_size, cpu_mem_size, block_size, rope_theta=10000.0, device="cuda"):
+    def __init__(self, layers, npu_mem_size, cpu_mem_size, block_size, rope_theta=10000.0, device="cuda",
+                 quantization_config=None):
         if not layers or not all(isinstance(l, QuantDecodeLayer) for l in layers):
             raise TypeError("layers must be a non-empty list of QuantDecodeLayer")
         first = layers[0]
@@ -42,7 +43,22 @@ class DecodeStackRunner:
         self.block_size = int(block_size)
         self.rope_theta = rope_theta
         self.device = torch.device(device)
-        itemsize = torch.empty(0, dtype=self.dtype).element_size()
+        # the cache dtype follows the quantization config when it names one (model_runner.py:364-368); int8 caches
+        # need every layer's dequantisation parameters (QuantDecodeLayer.set_kv_quant)
+        kv_name = getattr(quantization_config, "kvcache_quant_dtype", None) if quantization_config is not None else None
+        if isinstance(quantization_config, dict):
+            kv_name = quantization_config.get("kvcache_dtype")
+        if kv_name not in (None, "int8"):
+            raise NotImplementedError(f"kvcache_dtype {kv_name!r}: only an int8 KV cache is built")
+        if kv_name == "int8":
+            gran = (quantization_config.get("kvcache_quant_granularity", "per_channel") if isinstance(quantization_config, dict)
+                    else getattr(quantization_config, "kvcache_quant_granularity", "per_channel"))
+            if gran != "per_channel":
+                raise NotImplementedError("per_token int8 KV cache is not built (per_channel only)")
+            if any(l.kv_scale is None for l in layers):
+                raise ValueError("kvcache_dtype int8: every layer needs set_kv_quant(scale, offset) first")
+        self.kvcache_dtype = torch.int8 if kv_name == "int8" else self.dtype
+        itemsize = torch.empty(0, dtype=self.kvcache_dtype).element_size()
         args = (self.block_size, self.num_kv_heads, self.head_size, self.num_layers, itemsize)
         self.npu_num_blocks = num_cache_blocks(npu_mem_size, *args)
         self.cpu_num_blocks = num_cache_blocks(cpu_mem_size, *args)
@@ -50,11 +66,11 @@ class DecodeStackRunner:
             raise ValueError(f"npu_mem_size={npu_mem_size} GiB holds no cache block")
         kv_shape = (self.npu_num_blocks, self.block_size, self.num_kv_heads, self.head_size)
         host_shape = (self.cpu_num_blocks,) + kv_shape[1:]
-        self.key_cache = [torch.zeros(kv_shape, dtype=self.dtype, device=self.device) for _ in layers]
-        self.value_cache = [torch.zeros(kv_shape, dtype=self.dtype, device=self.device) for _ in layers]
+        self.key_cache = [torch.zeros(kv_shape, dtype=self.kvcache_dtype, device=self.device) for _ in layers]
+        self.value_cache = [torch.zeros(kv_shape, dtype=self.kvcache_dtype, device=self.device) for _ in layers]
         pin = self.cpu_num_blocks > 0
-        self.key_host = [torch.zeros(host_shape, dtype=self.dtype, pin_memory=pin) for _ in layers]
-        self.value_host = [torch.zeros(host_shape, dtype=self.dtype, pin_memory=pin) for _ in layers]
+        self.key_host = [torch.zeros(host_shape, dtype=self.kvcache_dtype, pin_memory=pin) for _ in layers]
+        self.value_host = [torch.zeros(host_shape, dtype=self.kvcache_dtype, pin_memory=pin) for _ in layers]
         self.is_first_iteration = True
         self.phase = "prefill"
 

@@ -140,8 +140,10 @@ def test_unbuilt_quant_modes_are_rejected_at_conversion():
         check_buildable(SmoothQuantConfig())             # per-tensor activations
     with pytest.raises(NotImplementedError):
         check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=64))
-    with pytest.raises(NotImplementedError):
-        check_buildable(PtqConfig(kvcache_dtype="int8"))
+    with pytest.raises(NotImplementedError):             # an int8 cache is built per channel only
+        check_buildable(PtqConfig(activation_dtype="int8", act_quant_granularity="per_token", kvcache_dtype="int8",
+                                  kvcache_quant_granularity="per_token"))
+    check_buildable(PtqConfig(kvcache_dtype="int8"))
     check_buildable(PtqConfig())
 
 

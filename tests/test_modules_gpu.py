@@ -710,3 +710,110 @@ def test_mcore_flash_attention_mla_decode_branch():
     ref = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, 0.072)
     mag = O.mla_paged_attention_decode(q, cache, tables, lens, nh, 512, 0.072, abs_values=True)
     assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA decode")
+
+
+# ------------------------------------------------------------------------------------------- kvcache_dtype: int8
+@pytest.mark.parametrize("dynamic", [True, False])
+def test_quantizer_swaps_in_the_int8_kv_manager_and_decode_matches_oracle(dynamic):
+    """`kvcache_dtype: int8` in the quantization config (quantization_config.py:196-254) makes the quantizer replace
+    the attention's cache manager by one that owns int8 caches; the InferAttention decode call then rotates,
+    quantises and scatters the new rows and attends over the int8 cache with the manager's dequantisation
+    parameters - against the oracle's RoPE -> quantising scatter -> attention over the dequantised cache."""
+    from torch import nn
+    from mindformers_amd.modules import FreqsMgr, InferAttention, Linear, PagedAttentionMgr, QuantPagedAttentionMgr
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    rng = np.random.default_rng(5)
+    b, n_head, n_kv, d, bs, seq = 3, 8, 2, 64, 16, 512
+    dt = torch.float16
+    lens = rng.integers(30, 300, b)
+    kc_f, vc_f, tables, nb = make_paged_cache(rng, b, lens, n_kv, d, bs, dt, max_blocks=seq // bs)
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.wq = Linear(256, n_head * d, has_bias=False, compute_dtype=dt)
+            self.infer_attention = InferAttention(n_head, d, n_kv, scale_value=1 / np.sqrt(d), block_size=bs,
+                                                  num_blocks=nb, seq_length=seq, is_dynamic=dynamic, rotary_cos_format=2,
+                                                  compute_dtype=dt)
+    net = Block()
+    assert type(net.infer_attention.paged_attention_mgr) is PagedAttentionMgr
+    quantizer = AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "kvcache_dtype": "int8"})
+    quantizer.preprocess_model(net)
+    mgr = net.infer_attention.paged_attention_mgr
+    assert isinstance(mgr, QuantPagedAttentionMgr) and mgr.key_cache.dtype == torch.int8
+    assert mgr.key_cache.shape == (nb, bs, n_kv, d) and mgr.kv_scale.shape == (2, n_kv * d)
+    with pytest.raises(NotImplementedError):                 # per-token cache granularity is refused, not ignored
+        AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8",
+                                   "act_quant_granularity": "per_token", "kvcache_dtype": "int8",
+                                   "kvcache_quant_granularity": "per_token"}).preprocess_model(Block())
+    row = n_kv * d
+    scale = (np.stack([np.abs(kc_f).reshape(-1, row).max(0), np.abs(vc_f).reshape(-1, row).max(0)]) / 110.0).astype(np.float32)
+    offset = rng.integers(-12, 13, (2, row)).astype(np.float32)
+    mgr.set_kv_quant(dev(scale, torch.float32), dev(offset, torch.float32))
+    k8 = O.quantize_kv_int8(kc_f.reshape(-1, row), scale[0], offset[0]).reshape(kc_f.shape)
+    v8 = O.quantize_kv_int8(vc_f.reshape(-1, row), scale[1], offset[1]).reshape(vc_f.shape)
+    mgr.key_cache.copy_(torch.from_numpy(k8))
+    mgr.value_cache.copy_(torch.from_numpy(v8))
+    attn = net.infer_attention
+    attn.is_first_iteration = False
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    freqs = FreqsMgr(d, seq_length=seq, max_position_embedding=seq, rotary_dtype=dt)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    freqs_cis = freqs.increment(lens_t)
+    q = rounded(rng.normal(size=(b, n_head * d)), dt)
+    k = rounded(rng.normal(size=(b, row)), dt)
+    v = rounded(rng.normal(size=(b, row)), dt)
+    shape = (b, n_head * d) if dynamic else (b, 1, n_head * d)
+    kv_shape = (b, row) if dynamic else (b, 1, row)
+    out = attn(dev(q, dt).reshape(shape), dev(k, dt).reshape(kv_shape), dev(v, dt).reshape(kv_shape), lens_t,
+               torch.from_numpy(tables).cuda(), torch.from_numpy(slots).cuda(), freqs_cis)
+    assert out.shape == shape
+    cos, sin = to_np(freqs_cis[0]), to_np(freqs_cis[1])
+    q_r = rounded(O.apply_rotary_half(q, cos, sin, n_head), dt)
+    k_r = rounded(O.apply_rotary_half(k, cos, sin, n_kv), dt)
+    O.reshape_and_cache(O.quantize_kv_int8(k_r, scale[0], offset[0]), O.quantize_kv_int8(v, scale[1], offset[1]), k8, v8, slots)
+    kf = O.dequantize_kv_int8(k8.reshape(-1, row), scale[0], offset[0]).reshape(k8.shape)
+    vf = O.dequantize_kv_int8(v8.reshape(-1, row), scale[1], offset[1]).reshape(v8.shape)
+    ref = O.paged_attention_decode(q_r, kf, vf, tables, lens, n_head, n_kv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q_r, kf, np.abs(vf), tables, lens, n_head, n_kv, 1 / np.sqrt(d))
+    assert_within(to_np(out).reshape(b, -1), ref, mag, dt, ulps=6.0, what="InferAttention decode over an int8 cache")
+    got_k = mgr.key_cache.cpu().numpy().reshape(-1, row)[slots].astype(np.int32)
+    assert np.abs(got_k - k8.reshape(-1, row)[slots]).max() <= 1          # a rotated key one rounding step away
+    assert np.array_equal(mgr.value_cache.cpu().numpy().reshape(-1, row)[slots], v8.reshape(-1, row)[slots])
+    keep = np.ones(nb * bs, bool)
+    keep[slots] = False
+    assert np.array_equal(mgr.key_cache.cpu().numpy().reshape(-1, row)[keep], k8.reshape(-1, row)[keep])
+
+
+def test_mcore_flash_attention_over_int8_caches():
+    """FlashAttention's decode branch with int8 caches passed per call and the antiquant parameters in the
+    PagedAttention positions: the scatter quantises, the attention dequantises; refused without the parameters."""
+    from mindformers_amd.modules import FlashAttention
+    rng = np.random.default_rng(9)
+    b, nh, nkv, d, bs = 3, 8, 2, 128, 128
+    dt = BF
+    lens = rng.integers(100, 700, b)
+    kc_f, vc_f, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dt)
+    row = nkv * d
+    scale = (np.stack([np.abs(kc_f).reshape(-1, row).max(0), np.abs(vc_f).reshape(-1, row).max(0)]) / 120.0).astype(np.float32)
+    k8 = O.quantize_kv_int8(kc_f.reshape(-1, row), scale[0]).reshape(kc_f.shape)
+    v8 = O.quantize_kv_int8(vc_f.reshape(-1, row), scale[1]).reshape(vc_f.shape)
+    kc, vc = torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda()
+    fa = FlashAttention(nh, d, nkv, scale_value=1 / np.sqrt(d), pa_kv_head_num=nkv)
+    fa.is_prefill = False
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    q = rounded(rng.normal(size=(b, nh * d)), dt)
+    k = rounded(rng.normal(size=(b, row)), dt)
+    v = rounded(rng.normal(size=(b, row)), dt)
+    args = dict(slot_mapping=torch.from_numpy(slots).cuda(), block_tables=torch.from_numpy(tables).cuda(),
+                batch_valid_length=torch.from_numpy(lens.astype(np.int32)).cuda(), key_cache=kc, value_cache=vc)
+    with pytest.raises(ValueError):
+        fa(dev(q, dt), dev(k, dt), dev(v, dt), **args)
+    out = fa(dev(q, dt), dev(k, dt), dev(v, dt), antiquant_scale=dev(scale, torch.float32), **args)
+    O.reshape_and_cache(O.quantize_kv_int8(k, scale[0]), O.quantize_kv_int8(v, scale[1]), k8, v8, slots)
+    assert np.array_equal(kc.cpu().numpy(), k8) and np.array_equal(vc.cpu().numpy(), v8)
+    kf = O.dequantize_kv_int8(k8.reshape(-1, row), scale[0]).reshape(k8.shape)
+    vf = O.dequantize_kv_int8(v8.reshape(-1, row), scale[1]).reshape(v8.shape)
+    ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, 1 / np.sqrt(d))
+    assert_within(to_np(out), ref, mag, dt, ulps=3.0, what="FlashAttention over int8 caches")

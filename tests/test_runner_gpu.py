@@ -157,3 +157,80 @@ def test_swap_moves_blocks_bit_exactly_both_ways():
         run.swap(np.array([[run.npu_num_blocks, 0]]), True)
     with pytest.raises(ValueError):
         ops.swap_cache(torch.zeros(run.key_host[0].shape, dtype=BF), run.key_cache[0], out_pairs, True)   # not pinned
+
+
+def test_runner_sizes_and_runs_int8_caches_from_the_quantization_config():
+    """`kvcache_dtype: int8` in the quantization config: the runner sizes the caches with one byte per element
+    (model_runner.py:364-376: twice the blocks in the same memory), allocates int8 device and host caches, and a
+    prefill followed by a decode step matches the oracle stack working on int8 caches with the same parameters."""
+    from mindformers_amd.modules import BlockTables
+    from mindformers_amd.quantization_config import PtqConfig
+    from mindformers_amd.runner import DecodeStackRunner
+    hidden, nh, nkv, d, ffn, bs, n_layers = 512, 8, 2, 64, 1024, 16, 2
+    layers = _stack(n_layers, hidden, nh, nkv, d, ffn, seed=9)
+    qcfg = PtqConfig(weight_dtype="int8", kvcache_dtype="int8")
+    with pytest.raises(ValueError):                          # the layers have no dequantisation parameters yet
+        DecodeStackRunner(layers, 0.002, 0.001, bs, quantization_config=qcfg)
+    rng = np.random.default_rng(6)
+    row = nkv * d
+    scales = [rng.uniform(0.03, 0.05, (2, row)).astype(np.float32) for _ in layers]
+    offsets = [rng.integers(-8, 9, (2, row)).astype(np.float32) for _ in layers]
+    for layer, s, o in zip(layers, scales, offsets):
+        layer.set_kv_quant(dev(s, torch.float32), dev(o, torch.float32))
+    run = DecodeStackRunner(layers, npu_mem_size=0.002, cpu_mem_size=0.001, block_size=bs, quantization_config=qcfg)
+    plain = DecodeStackRunner(layers, npu_mem_size=0.002, cpu_mem_size=0.001, block_size=bs)
+    from mindformers_amd.runner import num_cache_blocks
+    assert run.npu_num_blocks == num_cache_blocks(0.002, bs, nkv, d, n_layers, 1) >= 2 * plain.npu_num_blocks
+    assert run.cpu_num_blocks == num_cache_blocks(0.001, bs, nkv, d, n_layers, 1) >= 2 * plain.cpu_num_blocks
+    assert run.key_cache[0].dtype == torch.int8 and run.key_host[0].dtype == torch.int8 and run.key_host[0].is_pinned()
+    assert plain.key_cache[0].dtype == BF
+    del plain
+    prompt = np.array([29, 18])
+    b = len(prompt)
+    xs = [rounded(rng.normal(size=(int(t) + 1, hidden)), BF) for t in prompt]
+    mgr = BlockTables(run.npu_num_blocks, bs, 128)
+    mgr.init_cache_engine(b)
+    tables, slots = mgr.assemble_pa_full_inputs(int(prompt.max()), prompt, [False] * b)
+    slots = slots.reshape(b, -1)
+    slots = np.concatenate([slots[i, :prompt[i]] for i in range(b)])
+    x0 = np.concatenate([xs[i][:prompt[i]] for i in range(b)])
+    out0 = to_np(run.forward(dev(x0, BF), prompt, tables, slots, prefill=True))
+    cfg = dict(n_head=nh, n_kv_head=nkv, head_dim=d, eps=1e-5)
+    kcs = [np.zeros((run.npu_num_blocks, bs, nkv, d), np.int8) for _ in range(n_layers)]
+    vcs = [np.zeros_like(kcs[0]) for _ in range(n_layers)]
+    inv = 1.0 / (10000.0 ** (np.arange(0, d, 2) / d))
+
+    def rope(pos):
+        ang = np.asarray(pos, np.float64)[:, None] * inv[None, :]
+        emb = np.concatenate([ang, ang], -1).astype(np.float32)
+        return rounded(np.cos(emb), BF), rounded(np.sin(emb), BF)
+
+    def oracle_step(x, lens, tb, sl, pos, q_lens):
+        h = x
+        cos, sin = rope(pos)
+        for i, layer in enumerate(layers):
+            h = O.decode_layer_w8a16(h, _params(layer), cfg, kcs[i], vcs[i], tb, lens, sl, cos, sin, act_dtype="bf16",
+                                     q_seq_lens=q_lens, kv_quant=(scales[i], offsets[i]))
+        return h
+
+    def close(got, ref, what, ulps=16):
+        tol = ulps * EPS[BF] * np.maximum(np.abs(ref), 0.05 * np.abs(ref).max(axis=1, keepdims=True)) + 1e-4
+        assert np.mean(np.abs(got - ref) > tol) < 0.01, (what, np.abs(got - ref).max())
+
+    ref0 = oracle_step(x0, prompt, tables, slots, np.concatenate([np.arange(n) for n in prompt]), prompt)
+    close(out0, ref0, "prefill over int8 caches")
+    lens = prompt + 1
+    tables, slots = mgr.assemble_pa_inc_inputs(lens, [False] * b)
+    x = np.stack([xs[i][lens[i] - 1] for i in range(b)])
+    out = to_np(run.forward(dev(x, BF), lens, tables, slots, prefill=False))
+    close(out, oracle_step(x, lens, tables, slots, lens - 1, None), "decode step over int8 caches")
+    used = np.unique(tables[tables >= 0])
+    diff = np.abs(run.key_cache[0].cpu().numpy()[used].astype(np.int32) - kcs[0][used])
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.05
+    # swap works on the int8 caches as on the 16-bit ones
+    before = run.key_cache[1][used[0]].clone()
+    run.swap(np.array([[used[0], 0]]), True)
+    run.key_cache[1][used[0]].zero_()
+    run.swap(np.array([[0, used[0]]]), False)
+    torch.cuda.synchronize()
+    assert torch.equal(run.key_cache[1][used[0]], before)
