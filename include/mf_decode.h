@@ -307,6 +307,15 @@ int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const f
 int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m, int k,
                                int dtype, int layout, void* stream);
 
+/* golden-stick's static (per-tensor) activation quantisation in front of QuantBatchMatmul, the SmoothQuant method's
+ * A8W8 cells (mindformers/modules/quantizers/smooth_quant_quantizer.py:61-67, act_quant_granularity per_tensor in
+ * mindformers/utils/quantization_config.py:577-595): q = clip(rint(x * smooth / act_scale[0]), -128, 127) with one
+ * calibrated scale for the whole tensor (a float on the device, loaded with the checkpoint; symmetric: this build's
+ * declared convention, the cell's arithmetic is not in the reference).  x_scale receives act_scale[0] for every
+ * row, so mf_w8a8_gemm dequantises as for per-token scales.  Layouts as mf_dynamic_quant_per_token. */
+int mf_static_quant_per_tensor(int8_t* xq, float* x_scale, const void* x, const float* smooth,
+                               const float* act_scale, int m, int k, int dtype, int layout, void* stream);
+
 /* RMSNorm (optionally with the residual add in front, as mf_rmsnorm) whose only reader is a per-token quantised
  * projection, fused with that quantisation: the norm output is not written, xq / x_scale are what
  * mf_dynamic_quant_per_token(layout) gives for it.  Bit-identical to mf_rmsnorm followed by

@@ -50,6 +50,7 @@ SIGNATURES = {
     "mf_w8a16_qkv_rope_and_quant_cache": (_I, [_P] * 12 + [_I] * 4 + [_L] + [_I] * 3 + [_P, _Z, _P]),
     "mf_w8a16_gemm_silu_mul": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_dynamic_quant_per_token": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mf_static_quant_per_tensor": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mf_rmsnorm_dynamic_quant": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P]),
     "mf_silu_mul_dynamic_quant": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mf_w8a8_workspace_bytes": (_Z, [_I, _I, _I]),

@@ -127,10 +127,13 @@ __global__ void add_kernel(uint16_t* __restrict__ out, const uint16_t* __restric
 }
 
 // Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
+// With static_scale (one float on the device: a calibrated per-tensor activation scale) s is that value for every
+// row and no maximum is taken; x_scale still receives s per row, which is what the int8 GEMM's epilogue reads.
 template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq, float* __restrict__ x_scale,
                                                                const uint16_t* __restrict__ x,
-                                                               const float* __restrict__ smooth, int cols, int tiled) {
+                                                               const float* __restrict__ smooth, int cols, int tiled,
+                                                               const float* __restrict__ static_scale) {
     __shared__ float red[THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
@@ -146,8 +149,13 @@ __global__ __launch_bounds__(THREADS) void dynamic_quant_kernel(int8_t* __restri
             amax = fmaxf(amax, smooth_absmax8(v[it], smooth, 8 * c));
         }
     }
-    amax = block_max(amax, red);
-    const float s = __fdiv_rn(amax, 127.0f);
+    float s;
+    if (static_scale) {
+        s = static_scale[0];                                  // uniform: no reduction over the row
+    } else {
+        amax = block_max(amax, red);
+        s = __fdiv_rn(amax, 127.0f);
+    }
     const float safe = s > 0.f ? s : 1.0f;
     if (threadIdx.x == 0) x_scale[blockIdx.x] = s;
 #pragma unroll
@@ -384,8 +392,22 @@ extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dt
     return MF_LAUNCH_CHECK();
 }
 
+static int quant_rows_entry(int8_t* xq, float* x_scale, const void* x, const float* smooth, const float* static_scale,
+                            int m, int k, int dtype, int layout, void* stream);
+
 extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m,
                                           int k, int dtype, int layout, void* stream) {
+    return quant_rows_entry(xq, x_scale, x, smooth, nullptr, m, k, dtype, layout, stream);
+}
+
+extern "C" int mf_static_quant_per_tensor(int8_t* xq, float* x_scale, const void* x, const float* smooth,
+                                          const float* act_scale, int m, int k, int dtype, int layout, void* stream) {
+    MF_REQUIRE(act_scale != nullptr, "static_quant: null activation scale");
+    return quant_rows_entry(xq, x_scale, x, smooth, act_scale, m, k, dtype, layout, stream);
+}
+
+static int quant_rows_entry(int8_t* xq, float* x_scale, const void* x, const float* smooth, const float* static_scale,
+                            int m, int k, int dtype, int layout, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant: dtype must be bf16 or fp16");
     MF_REQUIRE(layout == 0 || layout == 1, "dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
     if (m <= 0) return 0;
@@ -397,7 +419,7 @@ extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void
     if (m <= 0) return 0;
 #define DQ_LAUNCH(TT, TH)                                                                                        \
     hipLaunchKernelGGL((dynamic_quant_kernel<TT, TH>), dim3(m), dim3(TH), 0, (hipStream_t)stream, xq, x_scale,    \
-                       (const uint16_t*)x, smooth, k, layout)
+                       (const uint16_t*)x, smooth, k, layout, static_scale)
     const bool wide = k > 4096;
     if (dtype == MF_BF16) {
         if (wide) DQ_LAUNCH(BF16, ROW_THREADS_WIDE); else DQ_LAUNCH(BF16, ROW_THREADS);

@@ -170,18 +170,27 @@ class WeightQuantLinearCell(_QuantLinearBase):
 
 
 class AllQuantLinearInferCell(_QuantLinearBase):
-    """W8A8 deploy cell: per-token dynamic activation quantisation (with the SmoothQuant multiplier) followed
-    by the int8 MFMA GEMM (DynamicQuant + QuantBatchMatmul in the reference stack)."""
+    """W8A8 deploy cell: per-token dynamic activation quantisation (with the SmoothQuant multiplier), or static
+    per-tensor quantisation with a calibrated scale (``act_quant_granularity="per_tensor"``, the SmoothQuant
+    method), followed by the int8 MFMA GEMM (DynamicQuant / QuantV2 + QuantBatchMatmul in the reference stack)."""
 
     has_act_quant = True
 
     def __init__(self, in_channels, out_channels, has_bias=False, compute_dtype=torch.bfloat16, device="cuda",
-                 layer=None, smooth=True):
+                 layer=None, smooth=True, act_quant_granularity="per_token"):
         super().__init__(in_channels, out_channels, has_bias, compute_dtype, device, layer)
+        if act_quant_granularity not in ("per_token", "per_tensor"):
+            raise ValueError(f"act_quant_granularity must be per_token or per_tensor, got {act_quant_granularity!r}")
+        self.act_quant_granularity = act_quant_granularity
         self.register_buffer("smooth_scale", torch.ones(in_channels, dtype=torch.float32, device=device) if smooth else None)
+        # per_tensor: one calibrated activation scale, loaded with the checkpoint (the SmoothQuant method's cells)
+        self.register_buffer("act_scale", torch.ones(1, dtype=torch.float32, device=device)
+                             if act_quant_granularity == "per_tensor" else None)
         self.quant_op = self._quant
 
     def _quant(self, x):
+        if self.act_quant_granularity == "per_tensor":
+            return ops.static_quant(x, self.act_scale, self.smooth_scale, tiled=True)
         return ops.dynamic_quant(x, self.smooth_scale, tiled=True)
 
     def prepare(self):

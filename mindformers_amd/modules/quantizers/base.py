@@ -109,8 +109,8 @@ def check_buildable(cfg):
         raise NotImplementedError("GPTQ precision recovery has no deploy-time kernel here")
     if cfg.outliers_suppression not in ("none", "smooth"):
         raise NotImplementedError(f"outliers_suppression {cfg.outliers_suppression!r} is not built")
-    if cfg.act_quant_dtype == "int8" and cfg.act_quant_granularity != "per_token":
-        raise NotImplementedError("per-tensor int8 activations are not built (per_token dynamic only)")
+    if cfg.act_quant_dtype == "int8" and cfg.act_quant_granularity not in ("per_token", "per_tensor"):
+        raise NotImplementedError(f"act_quant_granularity {cfg.act_quant_granularity!r} is not built")
 
 
 def convert_linears(model, cfg, layer_policies=None):
@@ -140,7 +140,8 @@ def convert_linears(model, cfg, layer_policies=None):
                 cdt = dt if dt in (torch.bfloat16, torch.float16) else torch.bfloat16
                 if pol.act_quant_dtype == "int8":
                     cell = AllQuantLinearInferCell(fin, fout, has_bias, cdt, dev, layer=child,
-                                                   smooth=pol.outliers_suppression == "smooth")
+                                                   smooth=pol.outliers_suppression == "smooth",
+                                                   act_quant_granularity=pol.act_quant_granularity)
                 else:
                     cell = WeightQuantLinearCell(fin, fout, has_bias, cdt, dev, layer=child)
                 if child.weight is not None:

@@ -1,7 +1,7 @@
-"""SmoothQuantQuantizer — mindformers/modules/quantizers/smooth_quant_quantizer.py:28-78.  The reference's
-SmoothQuant method is A8W8 with per-tensor activations (quantization_config.py:577-582), which these kernels do
-not implement: construction succeeds (dispatch parity), conversion raises NotImplementedError and points to the
-PTQ method with act_quant_granularity="per_token"."""
+"""SmoothQuantQuantizer - mindformers/modules/quantizers/smooth_quant_quantizer.py:28-78.  The reference's
+SmoothQuant method is A8W8 with static per-tensor activations and the smooth multiplier
+(quantization_config.py:577-582): conversion puts AllQuantLinearInferCell(act_quant_granularity="per_tensor") in
+place of every float linear; the calibrated ``act_scale`` / ``smooth_scale`` come with the checkpoint."""
 import torch
 
 from .base import Quantizer, convert_linears, finalize

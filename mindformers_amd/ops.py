@@ -641,6 +641,24 @@ def dynamic_quant(x, smooth=None, tiled=False):
     return (TiledInt8Activations(xq, x.shape) if tiled else xq), xs
 
 
+def static_quant(x, act_scale, smooth=None, tiled=False):
+    """Static per-tensor int8 quantisation (the SmoothQuant method's activation quantiser): q = clip(rint(x * smooth /
+    act_scale), -128, 127) with ``act_scale`` a one-element fp32 tensor on the device.  Returns (xq, scale fp32
+    [rows], every entry = act_scale) in the forms ``dynamic_quant`` returns, ready for ``w8a8_linear``."""
+    lib = _lib.load()
+    dev = _dev_ok(x, smooth, act_scale)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    _need(act_scale.dtype == torch.float32 and act_scale.numel() == 1, "act_scale must be one fp32 value")
+    k = x.shape[-1]
+    m = x.numel() // k
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [K]")
+    xq, xs = _quant_out(lib, x.shape, m, k, tiled, dev)
+    check(lib.mf_static_quant_per_tensor(ptr(xq), ptr(xs), ptr(x), ptr(smooth), ptr(act_scale), m, k,
+                                         dtype_code(x.dtype), 1 if tiled else 0, stream_ptr(dev)),
+          "mf_static_quant_per_tensor")
+    return (TiledInt8Activations(xq, x.shape) if tiled else xq), xs
+
+
 def _quant_out(lib, shape, m, k, tiled, dev):
     if tiled:
         xq = torch.empty(lib.mf_w8a16_packed_bytes(max(m, 1), k), dtype=torch.int8, device=dev)

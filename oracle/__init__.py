@@ -33,6 +33,7 @@ Pinning status of each function (what fixes it besides its own formula):
   quantize_weight_int8,    PARITY UNPINNED: the arithmetic lives in mindspore_gs / CANN
   w8a16_linear,            (not vendored, no reference vector).  int32 accumulators are
   dynamic_quant_per_token, pinned against exact integer matmul; rounding mode, clamp range
+  static_quant_per_tensor,
   w8a8_linear              and dequant order are this build's declared convention.
   quantize_kv_int8,        PARITY UNPINNED against the reference for the same reason (the convention, affine per
   dequantize_kv_int8       channel with ties to even and rails -128 / 127, is declared); the two functions
@@ -48,7 +49,7 @@ from .attention import (reshape_and_cache, paged_attention_decode, gather_kv,
 from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_yarn,
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp
-from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token,
+from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token, static_quant_per_tensor,
                     int8_gemm_i32, w8a8_linear, quantize_kv_int8, dequantize_kv_int8)
 from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,

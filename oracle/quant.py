@@ -52,6 +52,19 @@ def dynamic_quant_per_token(x, smooth=None):
     return q, s
 
 
+def static_quant_per_tensor(x, act_scale, smooth=None):
+    """Static per-tensor int8 (the SmoothQuant method's activation quantiser; PARITY UNPINNED like the per-token
+    form, symmetric by this build's declaration): xs = x*smooth; q = clip(rint(xs / act_scale), -128, 127), float32
+    throughout.  Returns (q int8 [T,K], s float32 [T] = act_scale for every row)."""
+    xs = np.asarray(x, dtype=np.float32)
+    if smooth is not None:
+        xs = (xs * np.asarray(smooth, dtype=np.float32)[None, :]).astype(np.float32)
+    s = np.float32(act_scale)
+    safe = s if s > 0 else np.float32(1.0)
+    q = np.clip(np.rint((xs / safe).astype(np.float32)), -128, 127).astype(np.int8)
+    return q, np.full(xs.shape[0], s, dtype=np.float32)
+
+
 def int8_gemm_i32(xq, w_i8):
     """Exact int32 accumulators acc[t,n] = sum_k xq[t,k]*w[n,k] (computed in int64, checked to fit)."""
     acc = np.asarray(xq, dtype=np.int64) @ np.asarray(w_i8, dtype=np.int64).T

@@ -136,8 +136,7 @@ def test_quantization_config_validation():
 def test_unbuilt_quant_modes_are_rejected_at_conversion():
     from mindformers_amd.modules.quantizers.base import check_buildable
     from mindformers_amd.quantization_config import PtqConfig, SmoothQuantConfig
-    with pytest.raises(NotImplementedError):
-        check_buildable(SmoothQuantConfig())             # per-tensor activations
+    check_buildable(SmoothQuantConfig())                 # static per-tensor activations + smooth: built
     with pytest.raises(NotImplementedError):
         check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=64))
     with pytest.raises(NotImplementedError):             # an int8 cache is built per channel only
@@ -268,6 +267,24 @@ def test_kv_int8_oracle_pair_is_pinned_by_what_the_mathematics_fixes():
     assert np.array_equal(mine, tq.int_repr().numpy())
     assert (mine == 127).any() and (mine == -128).any()                    # the rails are exercised
     assert np.array_equal(O.dequantize_kv_int8(mine, s2, zp.astype(np.float64)), tq.dequantize().double().numpy())
+
+
+def test_static_per_tensor_quant_oracle_properties():
+    """The static per-tensor activation quantiser: hand values, ties to even, both rails, the smoothing multiplier
+    applied before the division, one scale for every row; and agreement with torch's per-tensor affine quantiser on a
+    power-of-two scale."""
+    q, s = O.static_quant_per_tensor(np.array([[0.26, -0.26, 0.25, 0.35, 100.0, -100.0]], np.float32), 0.1)
+    assert q.tolist() == [[3, -3, 2, 4, 127, -128]] and s.tolist() == [np.float32(0.1)]
+    q, _ = O.static_quant_per_tensor(np.array([[1.0, 1.0]], np.float32), 0.5, np.array([2.0, 0.5], np.float32))
+    assert q.tolist() == [[4, 1]]                                         # x * smooth / scale
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 2, (40, 64)).astype(np.float32)
+    q, s = O.static_quant_per_tensor(x, 2.0 ** -5)
+    tq = torch.quantize_per_tensor(torch.from_numpy(x), 2.0 ** -5, 0, torch.qint8)
+    assert np.array_equal(q, tq.int_repr().numpy()) and np.all(s == np.float32(2.0 ** -5))
+    assert (q == 127).any() and (q == -128).any()
+    inside = np.abs(x) < 127 * 2.0 ** -5
+    assert np.abs(q[inside] * 2.0 ** -5 - x[inside]).max() <= 2.0 ** -6
 
 
 def test_moe_permute_is_a_stable_sort_and_unpermute_inverts_it():

@@ -863,6 +863,24 @@ def test_dynamic_quant_bit_exact(dtype, m, k, smooth):
     assert np.array_equal(to_np(xq), q_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,smooth,tiled", [(256, 3584, True, True), (5, 512, False, False), (33, 18944, True, True)])
+def test_static_quant_per_tensor_bit_exact(dtype, m, k, smooth, tiled):
+    """Static per-tensor activation quantisation: int8 values and the per-row copy of the scale equal the oracle's,
+    in both output layouts, with values beyond both rails."""
+    rng = np.random.default_rng(m + k)
+    x = rounded(rng.normal(0, 1.5, (m, k)), dtype)
+    sm = rng.uniform(0.5, 2.0, k).astype(np.float32) if smooth else None
+    act = np.float32(0.021)
+    xq, xs = ops.static_quant(dev(x, dtype), torch.tensor([act], device="cuda"), None if sm is None else dev(sm, torch.float32),
+                              tiled=tiled)
+    q_ref, s_ref = O.static_quant_per_tensor(x, act, sm)
+    assert np.array_equal(to_np(xs), s_ref)
+    got = untile_int8(to_np(xq.data), m, k) if tiled else to_np(xq)
+    assert np.array_equal(got, q_ref)
+    assert (q_ref == 127).any() and (q_ref == -128).any()
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 4608, 3584), (256, 3584, 3584), (130, 200, 1088), (1, 64, 64), (64, 257, 512),
                                    (256, 18944, 3584), (256, 896, 4736), (300, 96, 208), (65, 80, 16), (33, 130, 2064),
                                    (300, 16500, 208), (130, 16384, 80)])       # the 8-wave 256 x 160 tiles, ragged
