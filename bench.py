@@ -373,21 +373,24 @@ def bench_moe(args, torch, ops, _lib):
     logits = torch.randn(T, E, generator=gen, device=dev)
     ebias = torch.zeros(E, device=dev)
 
-    def packed(experts, n, k):
-        # any byte pattern is a valid int8 weight: fill the packed buffer directly
-        per = lib.mf_w8a16_packed_bytes(n, k)
-        buf = torch.randint(-127, 128, ((experts or 1) * per,), dtype=torch.int8, generator=gen, device=dev).view(torch.uint8)
-        sc = torch.full(((experts or 1) * n,), 1e-3 / (k ** 0.5), device=dev)
-        return ops.PackedInt8Weight(buf, sc, n, k, experts)
-    w1, w2 = packed(E, 2 * F, H), packed(E, H, F)
-    s1, s2 = packed(None, 2 * F, H), packed(None, H, F)
-    s1.gated = True
+    from mindformers_amd import synthetic
+
+    def quantized(experts, n, k):
+        # N(0, 0.02) weights quantised per output channel, generated expert by expert
+        w = torch.empty(experts or 1, n, k, dtype=torch.int8, device=dev)
+        sc = torch.empty(experts or 1, n, dtype=torch.float32, device=dev)
+        for e in range(experts or 1):
+            w[e], sc[e] = synthetic.quantize_weight_int8(torch.randn(n, k, generator=gen, device=dev) * 0.02)
+        return (w, sc) if experts else (w[0], sc[0])
+    raw1, raw2 = quantized(E, 2 * F, H), quantized(E, H, F)
+    sraw1, sraw2 = quantized(None, 2 * F, H), quantized(None, H, F)
+    w1, w2 = ops.pack_w8a16_gated(*raw1, "halves"), ops.pack_w8a16(*raw2)      # fc1 with silu(gate) * up in its epilogue
+    s1, s2 = ops.pack_w8a16_gated(*sraw1, "halves"), ops.pack_w8a16(*sraw2)
 
     def step():
         wgt, idx = ops.moe_route(logits, ebias, K_TOP, 8, 4, 2.5, dt)
         px, row_map, counts, offsets = ops.moe_permute(x, idx, E)
-        a = ops.silu_mul(ops.grouped_w8a16_linear(px, w1, offsets))
-        y = ops.grouped_w8a16_linear(a, w2, offsets)
+        y = ops.grouped_w8a16_linear(ops.grouped_w8a16_linear(px, w1, offsets), w2, offsets)
         shared = ops.w8a16_linear(ops.w8a16_gated_linear(x, s1), s2)
         return ops.moe_unpermute(y, row_map, wgt, shared=shared), counts
     out, counts = step()
@@ -417,8 +420,9 @@ def bench_moe(args, torch, ops, _lib):
     wgt, idx = ops.moe_route(logits, ebias, K_TOP, 8, 4, 2.5, dt)
     px, row_map, counts, offsets = ops.moe_permute(x, idx, E)
     g1 = timed(lambda: ops.grouped_w8a16_linear(px, w1, offsets))
-    a = ops.silu_mul(ops.grouped_w8a16_linear(px, w1, offsets))
+    a = ops.grouped_w8a16_linear(px, w1, offsets)
     g2 = timed(lambda: ops.grouped_w8a16_linear(a, w2, offsets))
+    parity = None if args.no_cpu else moe_parity(torch, out, x, logits, ebias, raw1, raw2, sraw1, sraw2, K_TOP, F)
     ach = n_act * per_expert / ((g1 + g2) * 1e-3) / 1e9
     result = {
         "metric": METRICS["deepseek_v3_moe_w8a16"],
@@ -432,9 +436,41 @@ def bench_moe(args, torch, ops, _lib):
         "layer_hbm_frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "roofline": dict(bound="hbm", kernel="w8a16_grouped_kernel (fc1 + fc2 launches)", achieved=round(ach, 1),
                          peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(ach / HBM_PEAK_GBPS, 4), traffic=None,
-                         bytes_per_launch=n_act * per_expert, avg_launch_us=round((g1 + g2) * 1e3, 2)),
+                         bytes_per_launch=n_act * per_expert, avg_launch_us=round((g1 + g2) * 1e3, 2),
+                         per_launch_us={"fc1_silu_mul": round(g1 * 1e3, 2), "fc2": round(g2 * 1e3, 2)}),
     }
+    if parity is not None:
+        result["parity_vs_cpu"] = parity
     print(json.dumps(result), flush=True)
+
+
+def moe_parity(torch, out, x, logits, ebias, raw1, raw2, sraw1, sraw2, k_top, f):
+    """The layer's output rows of a few tokens against the CPU oracle: router choice on all tokens, then the dense
+    sum over the chosen experts of w * fc2(silu(gate) * up) + the shared expert, rounded where the device stores."""
+    import oracle as O
+    from oracle import dense as Dn
+    from oracle import quant as Q
+    from oracle.layer import _r
+
+    def npf(t):
+        return t.float().cpu().numpy() if t.dtype.is_floating_point else t.cpu().numpy()
+    w_ref, idx_ref = O.topk_router(npf(logits), npf(ebias), k_top, 8, 4, 2.5)
+    w_ref = _r(w_ref, "bf16")
+    worst, scale = 0.0, 0.0
+    for t in (0, 31, 64, 127):
+        xt = npf(x[t:t + 1]).astype(np.float64)
+        acc = 0.0
+        for j in range(k_top):
+            e = int(idx_ref[t, j])
+            h1 = _r(Q.w8a16_linear(xt, npf(raw1[0][e]), npf(raw1[1][e])), "bf16")
+            a = _r(_r(Dn.silu(h1[:, :f]), "bf16") * h1[:, f:], "bf16")
+            acc = acc + w_ref[t, j] * _r(Q.w8a16_linear(a, npf(raw2[0][e]), npf(raw2[1][e])), "bf16")
+        h1 = _r(Q.w8a16_linear(xt, npf(sraw1[0]), npf(sraw1[1])), "bf16")
+        a = _r(_r(Dn.silu(h1[:, :f]), "bf16") * h1[:, f:], "bf16")
+        ref = _r(acc, "bf16") + _r(Q.w8a16_linear(a, npf(sraw2[0]), npf(sraw2[1])), "bf16")
+        worst = max(worst, float(np.abs(npf(out[t:t + 1]) - ref).max()))
+        scale = max(scale, float(np.abs(ref).max()))
+    return dict(max_abs_err=worst, ref_max_abs=scale, rows=4)
 
 
 def bench_prefill_attention(args, torch, ops):

@@ -398,6 +398,23 @@ int mf_moe_permute(void* permuted_x, int32_t* row_map, int64_t* counts, int32_t*
 int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const int32_t* offsets,
                           int n_experts, int total_rows, int n, int k, int dtype, void* stream);
 
+/* mf_grouped_w8a16_gemm with the experts' activation in its epilogue (experts.py:151-170: fc1, split into gate and
+ * hidden halves, hidden * silu(gate)): the rows of every expert's weight are interleaved gate / up as for
+ * mf_w8a16_gemm_silu_mul, y is [R, N/2]; same bits as mf_grouped_w8a16_gemm followed by mf_silu_mul(layout 1). */
+int mf_grouped_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale,
+                                   const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype,
+                                   void* stream);
+
+/* GroupedMatmulV4 on int8 activations and weights: the routed experts of a W8A8 checkpoint
+ * (mindformers/parallel_core/inference/transformer/moe/experts.py:116-117,136-137 with the quantization config of
+ * research/deepseek3/deepseek_r1_671b/predict_deepseek_r1_671b_w8a8.yaml:89-92).  xq int8 [R, K] row-major and
+ * x_scale [R] as mf_dynamic_quant_per_token(layout 0) writes them for the permuted rows; w_packed / w_scale / offsets
+ * as for mf_grouped_w8a16_gemm.  Exact int32 accumulators (acc_out int32 [R, N], may be NULL), y = acc * x_scale[r] *
+ * w_scale[e, n] rounded to out_dtype (y may be NULL when only the accumulators are wanted).  K % 16 == 0. */
+int mf_grouped_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale, const void* w_packed,
+                         const float* w_scale, const int32_t* offsets, int n_experts, int total_rows, int n, int k,
+                         int out_dtype, void* stream);
+
 /* MoeTokenUnpermute(permuted_tokens, sorted_indices, probs) — moe_layer.py:151-155.
  * out[t,:] = sum_j probs[t,j] * y[row_map[t*k+j],:] accumulated in fp32 in order j = 0..k-1
  * (+ shared[t,:] if shared != NULL, the shared-expert add of moe_layer.py:159-160). */

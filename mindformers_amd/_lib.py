@@ -60,6 +60,8 @@ SIGNATURES = {
     "mf_moe_route": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
     "mf_moe_permute": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mf_grouped_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mf_grouped_w8a16_gemm_silu_mul": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mf_grouped_w8a8_gemm": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mf_moe_unpermute": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
 }
 

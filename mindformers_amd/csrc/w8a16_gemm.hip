@@ -95,7 +95,8 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
                                            const uint16_t* __restrict__ x, const uint8_t* __restrict__ wp,
                                            const float* __restrict__ scale, const uint16_t* __restrict__ bias,
                                            const uint16_t* __restrict__ residual, int M, int N, int K, int KS, int n0,
-                                           int m0, int s_begin, int s_end, int split_index, uint8_t* smem) {
+                                           int m0, int s_begin, int s_end, int split_index, uint8_t* smem,
+                                           int gated = 0) {
     using vec8 = typename T::vec8;
     constexpr int XROWS = 16 * MT;
     constexpr int XTILE = XROWS * 128;                        // bytes of one staged activation tile
@@ -232,6 +233,8 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
                 for (int i = 0; i < 4; ++i)
                     if (n + i < N) p[i] = sum[i];
             }
+        } else if (gated) {
+            store_gated<T>(y, bias, scale, m, n, N, sum);
         } else {
             store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, sum);
         }
@@ -529,14 +532,16 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
 }
 
 // Grouped (experts): grid = (ceil(N/64), n_experts).  Rows offsets[e] .. offsets[e+1] of x use expert e's
-// packed weights and scale[e]; experts with no rows exit at once.  Rows are taken 16 at a time (decode
-// batches route a handful of tokens to each expert), re-streaming the expert's weights per pass.
+// packed weights and scale[e]; experts with no rows exit at once.  One pass over the expert's weights serves up to
+// 64 rows (decode batches route a handful of tokens to each expert: 16 rows per pass there); experts with more rows
+// repeat the pass.  gated: the rows of the weight are interleaved gate / up and the epilogue writes
+// silu(gate) * up into a [rows, N/2] output, as the dense gated GEMM does.
 template <typename T, bool KTAIL>
 __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_grouped_kernel(
     uint16_t* __restrict__ y, const uint16_t* __restrict__ x, const uint8_t* __restrict__ wp,
     const float* __restrict__ scale, const int32_t* __restrict__ offsets, int total_rows, int N, int K,
-    int64_t expert_bytes) {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[GwSmem<1>::BYTES];
+    int64_t expert_bytes, int gated) {
+    __shared__ __attribute__((aligned(16))) uint8_t smem[GwSmem<4>::BYTES];
     const int e = blockIdx.y;
     int row0 = offsets[e], row1 = offsets[e + 1];
     row0 = max(0, min(row0, total_rows));
@@ -546,10 +551,19 @@ __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_grouped_kernel(
     const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
     const uint8_t* we = wp + (int64_t)e * expert_bytes;
     const float* se = scale + (int64_t)e * N;
-    for (int m0 = 0; m0 < rows; m0 += 16) {
-        w8a16_tile<T, 1, KTAIL>(y + (int64_t)row0 * N, nullptr, x + (int64_t)row0 * K, we, se, nullptr, nullptr, rows, N, K, KS,
-                         blockIdx.x * GW_BN, m0, 0, KS, 0, smem);
-        __syncthreads();                                      // the LDS tile is reused by the next pass
+    uint16_t* ye = y + (int64_t)row0 * (gated ? N >> 1 : N);
+    const uint16_t* xe = x + (int64_t)row0 * K;
+    const int n0 = blockIdx.x * GW_BN;
+    if (rows <= 16) {
+        w8a16_tile<T, 1, KTAIL>(ye, nullptr, xe, we, se, nullptr, nullptr, rows, N, K, KS, n0, 0, 0, KS, 0, smem, gated);
+    } else if (rows <= 32) {
+        w8a16_tile<T, 2, KTAIL>(ye, nullptr, xe, we, se, nullptr, nullptr, rows, N, K, KS, n0, 0, 0, KS, 0, smem, gated);
+    } else {
+        for (int m0 = 0; m0 < rows; m0 += 64) {
+            w8a16_tile<T, 4, KTAIL>(ye, nullptr, xe, we, se, nullptr, nullptr, rows, N, K, KS, n0, m0, 0, KS, 0, smem,
+                                    gated);
+            __syncthreads();                                  // the LDS tile is reused by the next pass
+        }
     }
 }
 
@@ -1074,26 +1088,39 @@ extern "C" int mf_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_pack
                             workspace_bytes, stream);
 }
 
-extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale,
-                                     const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype,
-                                     void* stream) {
-    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "grouped_w8a16_gemm: dtype must be bf16 or fp16");
+static int grouped_w8a16_entry(const char* who, void* y, const void* x, const void* w_packed, const float* scale,
+                               const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype, int gated,
+                               void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "%s: dtype must be bf16 or fp16", who);
     if (total_rows == 0) return 0;
-    MF_REQUIRE(y && x && w_packed && scale && offsets, "grouped_w8a16_gemm: null argument");
-    MF_REQUIRE(n_experts > 0 && n_experts <= 65535 && total_rows >= 0 && n > 0 && k > 0,
-               "grouped_w8a16_gemm: bad sizes");
-    MF_REQUIRE(k % 8 == 0, "grouped_w8a16_gemm: K (%d) must be a multiple of 8", k);
-    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0,
-               "grouped_w8a16_gemm: x and w_packed must be 16-byte aligned");
+    MF_REQUIRE(y && x && w_packed && scale && offsets, "%s: null argument", who);
+    MF_REQUIRE(n_experts > 0 && n_experts <= 65535 && total_rows >= 0 && n > 0 && k > 0, "%s: bad sizes", who);
+    MF_REQUIRE(k % 8 == 0, "%s: K (%d) must be a multiple of 8", who, k);
+    MF_REQUIRE(!gated || n % 4 == 0, "%s: N (%d) must be a multiple of 4 (gate / up pairs)", who, n);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed) & 15) == 0, "%s: x and w_packed must be 16-byte aligned", who);
     const int64_t expert_bytes = (int64_t)mf_w8a16_packed_bytes(n, k);
     dim3 grid((n + GW_BN - 1) / GW_BN, n_experts);
 #define GG_LAUNCH(TT, KT)                                                                                        \
     hipLaunchKernelGGL((w8a16_grouped_kernel<TT, KT>), grid, dim3(GW_WAVES * 64), 0, (hipStream_t)stream,           \
                        (uint16_t*)y, (const uint16_t*)x, (const uint8_t*)w_packed, scale, offsets, total_rows, n, k, \
-                       expert_bytes)
+                       expert_bytes, gated)
     const bool ktail = (k % GW_KSTEP) != 0;
     if (dtype == MF_BF16) { if (ktail) GG_LAUNCH(BF16, true); else GG_LAUNCH(BF16, false); }
     else { if (ktail) GG_LAUNCH(FP16, true); else GG_LAUNCH(FP16, false); }
 #undef GG_LAUNCH
     return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_grouped_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale,
+                                     const int32_t* offsets, int n_experts, int total_rows, int n, int k, int dtype,
+                                     void* stream) {
+    return grouped_w8a16_entry("grouped_w8a16_gemm", y, x, w_packed, scale, offsets, n_experts, total_rows, n, k, dtype,
+                               0, stream);
+}
+
+extern "C" int mf_grouped_w8a16_gemm_silu_mul(void* y, const void* x, const void* w_packed, const float* scale,
+                                              const int32_t* offsets, int n_experts, int total_rows, int n, int k,
+                                              int dtype, void* stream) {
+    return grouped_w8a16_entry("grouped_w8a16_gemm_silu_mul", y, x, w_packed, scale, offsets, n_experts, total_rows, n,
+                               k, dtype, 1, stream);
 }

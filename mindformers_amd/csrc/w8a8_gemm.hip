@@ -745,6 +745,123 @@ __global__ __launch_bounds__(QRC_THREADS) void w8a8_reduce_rope_cache_kernel(
     }
 }
 
+// ---- grouped (experts): rows offsets[e] .. offsets[e+1] of the quantised activations use expert e's weights --------
+// grid = (ceil(N / 64), n_experts); a workgroup of 4 waves owns 64 output channels of one expert for all of its
+// rows.  Decode batches route a handful of tokens to each expert, so the kernel is a weight stream: the waves
+// interleave the 64-wide k-steps, each loads its four 1 KiB weight tiles of a step straight into operand registers
+// (two steps ahead) and the 16 bytes per lane of each 16-row activation tile from the row-major int8 rows (a few KiB
+// per expert, served by L2), and the four waves' exact int32 sums meet in LDS at the end.  Up to 32 rows go through
+// one pass over the weights; experts with more rows repeat the pass per 32 rows.
+constexpr int QG_WAVES = 4;
+constexpr int QG_NT = 4;                                      // 16-channel weight tiles per wave and step
+constexpr int QG_BN = 16 * QG_NT;
+constexpr int QG_MT_MAX = 2;                                  // 16-row activation tiles per pass
+constexpr int QG_SMEM = QG_WAVES * 16 * QG_MT_MAX * QG_BN * 4;
+
+template <typename T, int MT>
+__device__ __forceinline__ void w8a8_group_pass(uint16_t* __restrict__ y, int32_t* __restrict__ acc_out,
+                                                const int8_t* __restrict__ x, const float* __restrict__ xs,
+                                                const uint8_t* __restrict__ wp, const float* __restrict__ ws, int rows,
+                                                int N, int K, int n0, int m0, int32_t* red) {
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int KS = (K + Q_KSTEP - 1) / Q_KSTEP;
+    const int n_tiles_total = (N + 15) >> 4;
+    // operands: every load reads an address that exists (tiles past N, rows past the group and k past K are
+    // clamped; what they contribute is never stored, or meets the zero padding of the packed weights)
+    uint32_t woff[QG_NT];
+#pragma unroll
+    for (int j = 0; j < QG_NT; ++j) woff[j] = (uint32_t)min((n0 >> 4) + j, n_tiles_total - 1) * Q_TILE + lane * 16;
+    const int8_t* xrow[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xrow[i] = x + (int64_t)min(m0 + 16 * i + r, rows - 1) * K;
+    const int64_t wstep = (int64_t)n_tiles_total * Q_TILE;
+    const int k_last = K - 16;                                // byte offset of the last whole 16-byte chunk of a row
+
+    i32x4 acc[QG_NT][MT];
+#pragma unroll
+    for (int j = 0; j < QG_NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = (i32x4){0, 0, 0, 0};
+
+    constexpr int D = 2;                                      // steps in flight beyond the current one
+    i32x4 wr[D + 1][QG_NT], xr[D + 1][MT];
+    auto load = [&](int slot, int s) {
+        const int sc = min(s, KS - 1);
+        const uint8_t* wb = wp + sc * wstep;
+        const int kb = min(sc * Q_KSTEP + 16 * g, k_last);    // chunks past K meet zero weights
+#pragma unroll
+        for (int j = 0; j < QG_NT; ++j) wr[slot][j] = *(const i32x4*)(wb + woff[j]);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) xr[slot][i] = *(const i32x4*)(xrow[i] + kb);
+    };
+    const int first = wv;
+#pragma unroll
+    for (int d = 0; d <= D; ++d) load(d, first + d * QG_WAVES);
+    auto step = [&](int slot, int s) {
+#pragma unroll
+        for (int j = 0; j < QG_NT; ++j)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[slot][j], xr[slot][i], acc[j][i], 0, 0, 0);
+        load(slot, s + (D + 1) * QG_WAVES);
+    };
+    for (int s = first; s < KS; s += (D + 1) * QG_WAVES) {
+#pragma unroll
+        for (int slot = 0; slot <= D; ++slot)
+            if (s + slot * QG_WAVES < KS) step(slot, s + slot * QG_WAVES);
+    }
+
+    // sum of the four waves through LDS: red[wave][row][channel], 16-byte granules XOR-swizzled by the row
+    constexpr int XROWS = 16 * MT;
+    __syncthreads();                                          // the previous pass has been read out
+#pragma unroll
+    for (int j = 0; j < QG_NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            *(i32x4*)(red + ((wv * XROWS + 16 * i + r) * QG_BN) + (((4 * j + g) ^ r) << 2)) = acc[j][i];
+    __syncthreads();
+    constexpr int N4 = QG_BN / 4;
+    for (int idx = threadIdx.x; idx < XROWS * N4; idx += QG_WAVES * 64) {
+        const int ml = idx / N4, n4 = idx - ml * N4;
+        const int m = m0 + ml, n = n0 + 4 * n4;
+        if (m >= rows || n >= N) continue;
+        const int sw = (n4 ^ (ml & 15)) << 2;
+        i32x4 sum = *(const i32x4*)(red + ml * QG_BN + sw);
+#pragma unroll
+        for (int q = 1; q < QG_WAVES; ++q) sum += *(const i32x4*)(red + (q * XROWS + ml) * QG_BN + sw);
+        q2_store4<T>(y, acc_out, xs, ws, nullptr, nullptr, m, n, N, sum);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(QG_WAVES * 64, 2) void w8a8_grouped_kernel(
+    uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, const int8_t* __restrict__ xq,
+    const float* __restrict__ x_scale, const uint8_t* __restrict__ wp, const float* __restrict__ w_scale,
+    const int32_t* __restrict__ offsets, int total_rows, int N, int K, int64_t expert_bytes) {
+    __shared__ __attribute__((aligned(16))) int32_t red[QG_SMEM / 4];
+    const int e = blockIdx.y;
+    int row0 = offsets[e], row1 = offsets[e + 1];
+    row0 = max(0, min(row0, total_rows));
+    row1 = max(row0, min(row1, total_rows));
+    const int rows = row1 - row0;
+    if (rows == 0) return;
+    const uint8_t* we = wp + (int64_t)e * expert_bytes;
+    const float* se = w_scale + (int64_t)e * N;
+    uint16_t* ye = y ? y + (int64_t)row0 * N : nullptr;
+    int32_t* ae = acc_out ? acc_out + (int64_t)row0 * N : nullptr;
+    const int8_t* xe = xq + (int64_t)row0 * K;
+    const float* xse = x_scale + row0;
+    const int n0 = blockIdx.x * QG_BN;
+    if (rows <= 16) {
+        w8a8_group_pass<T, 1>(ye, ae, xe, xse, we, se, rows, N, K, n0, 0, red);
+    } else {
+        for (int m0 = 0; m0 < rows; m0 += 16 * QG_MT_MAX)
+            w8a8_group_pass<T, QG_MT_MAX>(ye, ae, xe, xse, we, se, rows, N, K, n0, m0, red);
+    }
+}
+
 // What may follow the GEMM in the same call, fused with the split-K reduce where K is split.
 struct QNormQuantArgs {           // residual add (through `residual`) + RMSNorm + per-token quantisation
     int8_t* xq_out;
@@ -995,4 +1112,27 @@ extern "C" int mf_w8a8_qkv_rope_and_cache(void* qkv, const int8_t* xq, const flo
                                  x_layout == 1, workspace, (hipStream_t)stream, nullptr, &rc);
     return launch_w8a8<FP16>(qkv, nullptr, xq, x_scale, (const uint8_t*)w_packed, w_scale, bias, nullptr, m, n, k,
                              x_layout == 1, workspace, (hipStream_t)stream, nullptr, &rc);
+}
+
+extern "C" int mf_grouped_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq, const float* x_scale,
+                                    const void* w_packed, const float* w_scale, const int32_t* offsets, int n_experts,
+                                    int total_rows, int n, int k, int out_dtype, void* stream) {
+    MF_REQUIRE(out_dtype == MF_BF16 || out_dtype == MF_FP16, "grouped_w8a8_gemm: out_dtype must be bf16 or fp16");
+    if (total_rows == 0) return 0;
+    MF_REQUIRE((y || acc_out) && xq && x_scale && w_packed && w_scale && offsets, "grouped_w8a8_gemm: null argument");
+    MF_REQUIRE(n_experts > 0 && n_experts <= 65535 && total_rows >= 0 && n > 0 && k > 0, "grouped_w8a8_gemm: bad sizes");
+    MF_REQUIRE(k % 16 == 0, "grouped_w8a8_gemm: K (%d) must be a multiple of 16", k);
+    MF_REQUIRE((((uintptr_t)xq | (uintptr_t)w_packed) & 15) == 0,
+               "grouped_w8a8_gemm: xq and w_packed must be 16-byte aligned");
+    const int64_t expert_bytes = (int64_t)mf_w8a16_packed_bytes(n, k);
+    dim3 grid((n + QG_BN - 1) / QG_BN, n_experts);
+    if (out_dtype == MF_BF16)
+        hipLaunchKernelGGL(w8a8_grouped_kernel<BF16>, grid, dim3(QG_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
+                           acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, offsets, total_rows, n, k,
+                           expert_bytes);
+    else
+        hipLaunchKernelGGL(w8a8_grouped_kernel<FP16>, grid, dim3(QG_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
+                           acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, offsets, total_rows, n, k,
+                           expert_bytes);
+    return MF_LAUNCH_CHECK();
 }

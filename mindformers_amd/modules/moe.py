@@ -93,19 +93,32 @@ class GroupedMLP(nn.Module):
 
 
 class QuantGroupedMLP(nn.Module):
-    """W8A16 experts: int8 weights stored K-contiguous ([E, 2F, H] and [E, H, F], i.e. the reference's
-    [E, in, out] parameters transposed at load) with per-output-channel scales; two grouped HIP GEMMs around
-    the SiLU*mul kernel.  ``offsets`` (int32 [E+1], from moe_permute) addresses the row groups."""
+    """Quantized experts: int8 weights stored K-contiguous ([E, 2F, H] and [E, H, F], i.e. the reference's
+    [E, in, out] parameters transposed at load) with per-output-channel scales.  ``offsets`` (int32 [E+1], from
+    moe_permute) addresses the row groups.
 
-    def __init__(self, num_experts, config, device="cuda"):
+    ``act_quant=None`` (W8A16): two grouped HIP GEMMs, the first with silu(gate) * hidden in its epilogue.
+    ``act_quant="per_token"`` / ``"per_tensor"`` (W8A8, the routed experts of a W8A8 checkpoint such as
+    research/deepseek3/deepseek_r1_671b/predict_deepseek_r1_671b_w8a8.yaml:89-92): the permuted rows are quantised per
+    token, or with one calibrated scale per projection (``act_scale1`` / ``act_scale2``, loaded with the checkpoint),
+    and both projections run on the int8 matrix cores with exact int32 accumulators."""
+
+    def __init__(self, num_experts, config, device="cuda", act_quant=None):
         super().__init__()
+        if act_quant not in (None, "per_token", "per_tensor"):
+            raise ValueError(f"act_quant must be None, 'per_token' or 'per_tensor', got {act_quant!r}")
         self.config = config
         self.num_experts = num_experts
+        self.act_quant = act_quant
+        self.compute_dtype = getattr(config, "compute_dtype", torch.bfloat16)
         f, h = config.moe_ffn_hidden_size, config.hidden_size
         self.register_buffer("weight1", torch.zeros(num_experts, 2 * f, h, dtype=torch.int8, device=device))
         self.register_buffer("w1_scale", torch.ones(num_experts, 2 * f, dtype=torch.float32, device=device))
         self.register_buffer("weight2", torch.zeros(num_experts, h, f, dtype=torch.int8, device=device))
         self.register_buffer("w2_scale", torch.ones(num_experts, h, dtype=torch.float32, device=device))
+        static = act_quant == "per_tensor"
+        self.register_buffer("act_scale1", torch.ones(1, dtype=torch.float32, device=device) if static else None)
+        self.register_buffer("act_scale2", torch.ones(1, dtype=torch.float32, device=device) if static else None)
         self._p1 = self._p2 = None
 
     @torch.no_grad()
@@ -121,9 +134,16 @@ class QuantGroupedMLP(nn.Module):
         return self
 
     def prepare(self):
-        self._p1 = ops.pack_w8a16(self.weight1, self.w1_scale)
+        # W8A16: gate / up rows interleaved, so that the first GEMM's epilogue holds each pair in one lane
+        self._p1 = (ops.pack_w8a16(self.weight1, self.w1_scale) if self.act_quant
+                    else ops.pack_w8a16_gated(self.weight1, self.w1_scale, "halves"))
         self._p2 = ops.pack_w8a16(self.weight2, self.w2_scale)
         return self
+
+    def _quant(self, x, act_scale):
+        if self.act_quant == "per_tensor":
+            return ops.static_quant(x, act_scale)
+        return ops.dynamic_quant(x)
 
     def forward(self, hidden_states, group_list=None, offsets=None):
         if self._p1 is None:
@@ -131,9 +151,17 @@ class QuantGroupedMLP(nn.Module):
         if offsets is None:
             offsets = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=hidden_states.device)
             offsets[1:] = torch.cumsum(group_list, 0).to(torch.int32)
-        h = ops.grouped_w8a16_linear(hidden_states, self._p1, offsets)
-        a = ops.silu_mul(h)
-        return ops.grouped_w8a16_linear(a, self._p2, offsets)
+        if not self.act_quant:
+            a = ops.grouped_w8a16_linear(hidden_states, self._p1, offsets)       # silu(gate) * hidden included
+            return ops.grouped_w8a16_linear(a, self._p2, offsets)
+        dt = hidden_states.dtype
+        xq, xs = self._quant(hidden_states.contiguous(), self.act_scale1)
+        h = ops.grouped_w8a8_linear(xq, xs, self._p1, offsets, out_dtype=dt)
+        if self.act_quant == "per_tensor":
+            aq, a_s = ops.static_quant(ops.silu_mul(h), self.act_scale2)
+        else:
+            aq, a_s = ops.silu_mul_dynamic_quant(h)
+        return ops.grouped_w8a8_linear(aq, a_s, self._p2, offsets, out_dtype=dt)
 
     construct = forward
 

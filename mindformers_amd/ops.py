@@ -582,22 +582,25 @@ def w8a16_qkv_rope_and_cache(x, w, cos, sin, key_cache, value_cache, slot_mappin
     return qkv[:, :n_heads * d]
 
 
-def interleave_gate_up(t, layout="halves"):
-    """Rows (dim 0) of a gate/up projection parameter in the interleaved order the fused gated GEMM wants (row 2j =
-    gate channel j, row 2j+1 = up channel j).  ``layout``: "halves" = [gate | up] contiguous halves (the mcore MLP,
-    parallel_core/inference/transformer/mlp.py:136-140), "interleaved" = already in that order (legacy ffn_concat,
-    mindformers/models/llama/llama_layer.py:419-423)."""
+def interleave_gate_up(t, layout="halves", dim=0):
+    """Entries along ``dim`` of a gate/up projection parameter in the interleaved order the fused gated GEMM wants
+    (entry 2j = gate channel j, entry 2j+1 = up channel j).  ``layout``: "halves" = [gate | up] contiguous halves (the
+    mcore MLP, parallel_core/inference/transformer/mlp.py:136-140), "interleaved" = already in that order (legacy
+    ffn_concat, mindformers/models/llama/llama_layer.py:419-423)."""
     if layout == "interleaved":
         return t.contiguous()
     _need(layout == "halves", "layout must be 'halves' or 'interleaved'")
-    f = t.shape[0] // 2
-    return torch.stack((t[:f], t[f:]), dim=1).reshape(t.shape).contiguous()
+    dim = dim % t.dim()
+    f = t.shape[dim] // 2
+    gate, up = t.narrow(dim, 0, f), t.narrow(dim, f, f)
+    return torch.stack((gate, up), dim=dim + 1).reshape(t.shape).contiguous()
 
 
 def pack_w8a16_gated(w_i8, scale, layout="halves"):
-    """Pack a gate/up projection weight [2F, K] (+ scale [2F]) for ``w8a16_gated_linear``."""
-    _need(w_i8.dim() == 2 and w_i8.shape[0] % 2 == 0, "gate/up weight must be [2F, K]")
-    w = pack_w8a16(interleave_gate_up(w_i8, layout), interleave_gate_up(scale, layout))
+    """Pack a gate/up projection weight [2F, K] or a stack of experts [E, 2F, K] (+ scale [2F] / [E, 2F]) for
+    ``w8a16_gated_linear`` / the gated form of ``grouped_w8a16_linear``."""
+    _need(w_i8.dim() in (2, 3) and w_i8.shape[-2] % 2 == 0, "gate/up weight must be [2F, K] or [E, 2F, K]")
+    w = pack_w8a16(interleave_gate_up(w_i8, layout, dim=-2), interleave_gate_up(scale, layout, dim=-1))
     w.gated = True
     return w
 
@@ -842,7 +845,8 @@ def moe_permute(x, expert_index, n_experts):
 
 def grouped_w8a16_linear(x, w, offsets, scale=None):
     """GroupedMatmulV4 over expert row groups.  x [R, K]; ``w`` a PackedInt8Weight of [E, N, K] (or a raw int8
-    [E, N, K] tensor with ``scale`` [E, N], packed on every call); offsets int32 [E+1]."""
+    [E, N, K] tensor with ``scale`` [E, N], packed on every call); offsets int32 [E+1].  A weight packed with
+    ``pack_w8a16_gated`` runs with silu(gate) * up in the epilogue and returns [R, N/2]."""
     lib = _lib.load()
     if not isinstance(w, PackedInt8Weight):
         w = pack_w8a16(w, scale)
@@ -851,10 +855,31 @@ def grouped_w8a16_linear(x, w, offsets, scale=None):
     e, n, k = w.experts, w.n, w.k
     _need(x.dtype in _ACT and x.dim() == 2 and x.shape[1] == k, "x must be bf16/fp16 [R, K]")
     _need(offsets.dtype == torch.int32 and offsets.numel() == e + 1, "offsets must be int32 [E+1]")
-    y = torch.empty(x.shape[0], n, dtype=x.dtype, device=dev)
-    check(lib.mf_grouped_w8a16_gemm(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(offsets), e, x.shape[0], n, k,
-                                    dtype_code(x.dtype), stream_ptr(dev)), "mf_grouped_w8a16_gemm")
+    y = torch.empty(x.shape[0], n // 2 if w.gated else n, dtype=x.dtype, device=dev)
+    fn = lib.mf_grouped_w8a16_gemm_silu_mul if w.gated else lib.mf_grouped_w8a16_gemm
+    check(fn(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(offsets), e, x.shape[0], n, k, dtype_code(x.dtype),
+             stream_ptr(dev)), "mf_grouped_w8a16_gemm")
     return y
+
+
+def grouped_w8a8_linear(xq, x_scale, w, offsets, out_dtype=torch.bfloat16, return_acc=False):
+    """GroupedMatmulV4 on int8 operands: xq int8 [R, K] row-major with per-row scales (``dynamic_quant`` of the permuted
+    rows), ``w`` a PackedInt8Weight of [E, N, K], offsets int32 [E+1].  Exact int32 accumulators, dequantised to
+    out_dtype; with ``return_acc`` also the int32 [R, N] accumulators."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt8Weight) and w.experts is not None and not w.gated,
+          "grouped_w8a8_linear needs stacked expert weights [E, N, K] (not gated)")
+    dev = _dev_ok(xq, x_scale, offsets)
+    e, n, k = w.experts, w.n, w.k
+    _need(xq.dtype == torch.int8 and xq.dim() == 2 and xq.shape[1] == k, "xq must be int8 [R, K]")
+    _need(x_scale.dtype == torch.float32 and x_scale.numel() == xq.shape[0], "x_scale must be fp32 [R]")
+    _need(offsets.dtype == torch.int32 and offsets.numel() == e + 1, "offsets must be int32 [E+1]")
+    _need(out_dtype in _ACT, "out_dtype must be bf16/fp16")
+    y = torch.empty(xq.shape[0], n, dtype=out_dtype, device=dev)
+    acc = torch.empty(xq.shape[0], n, dtype=torch.int32, device=dev) if return_acc else None
+    check(lib.mf_grouped_w8a8_gemm(ptr(y), ptr(acc), ptr(xq), ptr(x_scale), ptr(w.packed), ptr(w.scale), ptr(offsets), e,
+                                   xq.shape[0], n, k, dtype_code(out_dtype), stream_ptr(dev)), "mf_grouped_w8a8_gemm")
+    return (y, acc) if return_acc else y
 
 
 def moe_unpermute(y, row_map, probs, shared=None):

@@ -603,3 +603,40 @@ def test_grouped_w8a16_gemm_is_exact_on_an_integer_grid(n, k):
             # every partial sum is an integer below 3 * 127 * 7168 < 2^24: the float32 product is exact
             exact = (x[r0:r1] @ wq[ex].cpu().numpy().astype(np.float32).T).astype(np.float64) * s[ex]
             assert np.array_equal(y[r0:r1], rounded(exact, BF).astype(np.float64)), ex
+
+
+@pytest.mark.parametrize("n,k", [(4096, 7168), (7168, 2048)])
+def test_grouped_w8a8_accumulators_are_exact_at_the_moe_shape(n, k):
+    """The int8 expert projections at the DeepSeek-V3 shape over 256 experts with ragged row groups: int32
+    accumulators equal to the integer matmul on a sample of experts (every kind of group: empty, one row, the
+    crowded one), and on all experts to a float64 matmul of the same integers (exact below 2^53)."""
+    from mindformers_amd import ops
+    rng = np.random.default_rng(k)
+    e, rows = 256, 1024
+    cnt = rng.multinomial(rows - 40, np.ones(e) / e)
+    cnt[5] += 40
+    cnt[9] = cnt[200] = 0
+    rows = int(cnt.sum())
+    off = np.concatenate(([0], np.cumsum(cnt))).astype(np.int32)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(k)
+    wq = torch.randint(-127, 128, (e, n, k), dtype=torch.int8, generator=gen, device="cuda")
+    ws = torch.full((e, n), 1e-4, device="cuda")
+    x = rounded(rng.normal(size=(rows, k)), BF)
+    xq, xs = ops.dynamic_quant(dev(x, BF))
+    y, acc = ops.grouped_w8a8_linear(xq, xs, ops.pack_w8a16(wq, ws), torch.from_numpy(off).cuda(), return_acc=True)
+    # all experts at once on the device in float64: |acc| <= 128 * 127 * 7168 < 2^53, so the float64 sums are exact
+    ref_all = torch.empty(rows, n, dtype=torch.float64, device="cuda")
+    xq64 = xq.double()
+    for ex in range(e):
+        r0, r1 = int(off[ex]), int(off[ex + 1])
+        if r1 > r0:
+            ref_all[r0:r1] = xq64[r0:r1] @ wq[ex].double().t()
+    assert torch.equal(acc.double(), ref_all)
+    xq_n, got = to_np(xq), to_np(acc)
+    for ex in (5, 9, 200, int(np.argmin(np.where(cnt > 0, cnt, 99))), 255):
+        r0, r1 = int(off[ex]), int(off[ex + 1])
+        if r1 > r0:
+            assert np.array_equal(got[r0:r1], O.int8_gemm_i32(xq_n[r0:r1], wq[ex].cpu().numpy())), ex
+    yref = ref_all * xs.double()[:, None] * 1e-4
+    assert bool((torch.abs(y.double() - yref) <= 1.01 * EPS[BF] * yref.abs() + 1e-6).all())

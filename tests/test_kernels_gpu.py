@@ -1077,3 +1077,58 @@ def test_moe_permute_grouped_unpermute():
     ref = rounded(routed, dtype).astype(np.float64) + sh
     mag = np.abs(ref) + np.abs(rounded(routed, dtype))
     assert_within(to_np(out), ref, mag, dtype, ulps=1.5, extra=1e-6, what="unpermute")
+
+
+# ------------------------------------------------------------------------------------------- grouped GEMMs, more
+def _ragged_groups(rng, counts):
+    counts = np.asarray(counts, np.int64)
+    return counts, np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_grouped_w8a16_many_rows_and_gated_epilogue(dtype):
+    """Experts with 0, 1, 16, 17, 33 and 70 rows (one, two and four row tiles per pass over the weights, and a
+    repeated pass) against the oracle; the gated form (gate / up rows interleaved at pack time, silu(gate) * up in the
+    epilogue) carries the bits of the plain grouped GEMM followed by silu_mul; K is not a multiple of 64."""
+    rng = np.random.default_rng(23)
+    counts, off = _ragged_groups(rng, [0, 1, 16, 17, 33, 70, 0, 5])
+    e, f, k = len(counts), 96, 328
+    rows = int(counts.sum())
+    x = rounded(rng.normal(size=(rows, k)), dtype)
+    w = rng.normal(0, 0.05, (e, 2 * f, k)).astype(np.float32)
+    q, s = zip(*(O.quantize_weight_int8(w[i]) for i in range(e)))
+    q, s = np.stack(q), np.stack(s)
+    qd, sd, od = torch.from_numpy(q).cuda(), torch.from_numpy(s).cuda(), torch.from_numpy(off).cuda()
+    y = ops.grouped_w8a16_linear(dev(x, dtype), ops.pack_w8a16(qd, sd), od)
+    deq = np.transpose(q.astype(np.float64) * s[..., None], (0, 2, 1))
+    ref = O.grouped_matmul(x, deq, counts)
+    mag = O.grouped_matmul(np.abs(x), np.abs(deq), counts)
+    assert_within(to_np(y), ref, np.abs(ref), dtype, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="grouped gemm, many rows")
+    fused = ops.grouped_w8a16_linear(dev(x, dtype), ops.pack_w8a16_gated(qd, sd, "halves"), od)
+    assert fused.shape == (rows, f) and torch.equal(fused, ops.silu_mul(y))
+
+
+@pytest.mark.parametrize("counts,n,k", [([0, 5, 16, 20, 40, 1, 0, 3], 192, 208), ([4] * 16, 128, 1024), ([33], 80, 64)])
+def test_grouped_w8a8_accumulators_bit_exact(counts, n, k):
+    """The grouped int8 GEMM: exact int32 accumulators per expert (against the integer matmul), dequantised outputs
+    within a rounding of acc * row scale * channel scale; ragged groups, empty experts, more than 32 rows (a repeated
+    pass), K not a multiple of 64, N not a multiple of 64."""
+    rng = np.random.default_rng(n + k)
+    counts, off = _ragged_groups(rng, counts)
+    e, rows = len(counts), int(counts.sum())
+    x = rounded(rng.normal(size=(rows, k)), torch.bfloat16)
+    xq, xs = ops.dynamic_quant(dev(x, torch.bfloat16))
+    wq = rng.integers(-127, 128, (e, n, k)).astype(np.int8)
+    ws = rng.uniform(1e-4, 5e-4, (e, n)).astype(np.float32)
+    w = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(ws).cuda())
+    y, acc = ops.grouped_w8a8_linear(xq, xs, w, torch.from_numpy(off).cuda(), return_acc=True)
+    xq_n, xs_n = to_np(xq), to_np(xs).astype(np.float64)
+    got_acc, got_y = to_np(acc), to_np(y)
+    for ex in range(e):
+        r0, r1 = int(off[ex]), int(off[ex + 1])
+        if r1 == r0:
+            continue
+        ref = O.int8_gemm_i32(xq_n[r0:r1], wq[ex])
+        assert np.array_equal(got_acc[r0:r1], ref), ex
+        yref = ref.astype(np.float64) * xs_n[r0:r1, None] * ws[ex].astype(np.float64)[None, :]
+        assert np.all(np.abs(got_y[r0:r1] - yref) <= 1.01 * EPS[torch.bfloat16] * np.abs(yref) + 1e-6), ex

@@ -839,3 +839,71 @@ def test_mcore_flash_attention_over_int8_caches():
     ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, 1 / np.sqrt(d))
     mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, 1 / np.sqrt(d))
     assert_within(to_np(out), ref, mag, dt, ulps=3.0, what="FlashAttention over int8 caches")
+
+
+@pytest.mark.parametrize("granularity", ["per_token", "per_tensor"])
+def test_moe_layer_w8a8_experts_vs_oracle(granularity):
+    """The reference's own W8A8 recipe for the routed experts (quant_method ptq, int8 weights and activations,
+    research/deepseek3/deepseek_r1_671b/predict_deepseek_r1_671b_w8a8.yaml:89-92; its default activation granularity is
+    per_tensor): the quantizer converts GroupedMLP to int8 experts, and the layer equals the oracle's router and
+    permute around quantise -> exact int8 GEMM -> dequantise per expert, rounding where the device stores."""
+    from oracle import dense as Dn
+    from oracle.layer import _r
+    from mindformers_amd.modules import AllQuantLinearInferCell, MoELayer, QuantGroupedMLP
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    from mindformers_amd.transformer_config import TransformerConfig
+    cfg = TransformerConfig(num_layers=1, num_attention_heads=8, hidden_size=64, hidden_act="silu", num_moe_experts=8,
+                            moe_router_topk=2, shared_expert_num=0, moe_router_topk_scaling_factor=2.5,
+                            moe_shared_expert_intermediate_size=None, moe_ffn_hidden_size=32, moe_router_group_topk=2,
+                            moe_router_num_groups=4, add_bias_linear=False, gated_linear_unit=True,
+                            compute_dtype="bfloat16", params_dtype="bfloat16", moe_router_dtype="bfloat16",
+                            moe_router_enable_expert_bias=True, moe_router_score_function="sigmoid")
+    torch.manual_seed(3)
+    net = MoELayer(cfg)
+    net.router.weight.data.normal_(0, 0.3)
+    net.router.expert_bias.data.normal_(0, 0.1)
+    net.experts.weight1.data.normal_(0, 0.3)
+    net.experts.weight2.data.normal_(0, 0.3)
+    router_w, router_b = to_np(net.router.weight), to_np(net.router.expert_bias)
+    q = AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8",
+                                   "act_quant_granularity": granularity, "modules_to_not_convert": ["router"]})
+    q.preprocess_model(net)
+    assert isinstance(net.experts, QuantGroupedMLP) and net.experts.act_quant == granularity
+    s1, s2 = np.float32(0.03), np.float32(0.25)
+    if granularity == "per_tensor":
+        net.experts.act_scale1.fill_(float(s1))
+        net.experts.act_scale2.fill_(float(s2))
+    q.postprocess_model(net)
+    x = rounded(np.random.default_rng(8).normal(size=(24, 64)), BF)
+    out = to_np(net(dev(x, BF)))
+    ex = net.experts
+    w1, w1s, w2, w2s = to_np(ex.weight1), to_np(ex.w1_scale), to_np(ex.weight2), to_np(ex.w2_scale)
+    e = w1.shape[0]
+    logits = _r(Dn.linear(x, router_w), "bf16")
+    wgt, idx = O.topk_router(logits.astype(np.float32), router_b, 2, 4, 2, 2.5)
+    wgt = _r(wgt, "bf16")
+    px, row_map, counts = O.moe_permute(x, idx, e)
+
+    def quant(a, s):
+        return O.dynamic_quant_per_token(a.astype(np.float32)) if granularity == "per_token" else \
+            O.static_quant_per_tensor(a.astype(np.float32), s)
+    y = np.zeros((px.shape[0], w2.shape[1]))
+    start = 0
+    xq, xs = quant(px, s1)
+    h = np.zeros((px.shape[0], w1.shape[1]))
+    for i, c in enumerate(counts):
+        c = int(c)
+        h[start:start + c] = O.w8a8_linear(xq[start:start + c], xs[start:start + c], w1[i], w1s[i])
+        start += c
+    h = _r(h, "bf16")
+    f = h.shape[1] // 2
+    a = _r(_r(Dn.silu(h[:, :f]), "bf16") * h[:, f:], "bf16")
+    aq, a_s = quant(a, s2)
+    start = 0
+    for i, c in enumerate(counts):
+        c = int(c)
+        y[start:start + c] = O.w8a8_linear(aq[start:start + c], a_s[start:start + c], w2[i], w2s[i])
+        start += c
+    ref = _r(O.moe_unpermute(_r(y, "bf16"), row_map, wgt), "bf16")
+    assert np.abs(out - ref).max() <= 6 * EPS[BF] * np.abs(ref).max()
+    assert np.mean(np.abs(out - ref) > 2 * EPS[BF] * np.abs(ref) + 1e-6) < 0.02
