@@ -73,10 +73,8 @@ class FlashAttention(nn.Module):
                                               self.pa_kv_head_num, self.scale_value)
             return out.reshape(shape)
         if self.use_multi_latent_attention:                   # one latent cache, keys = values (flash_attention.py:136-139)
-            if q_seq_lens is not None:
-                raise NotImplementedError("MLA decode with q_seq_lens (several new tokens per sequence) is not built")
             out = ops.mla_paged_attention(q2, key_cache, block_tables, batch_valid_length, self.head_num,
-                                          self.pa_mla_v_dim, self.scale_value)
+                                          self.pa_mla_v_dim, self.scale_value, q_seq_lens=q_seq_lens)
             return out.reshape(*shape[:-1], self.head_num * self.pa_mla_v_dim)
         if kv8:
             starts = None if q_seq_lens is None else ops.q_starts_from_lens(q_seq_lens)

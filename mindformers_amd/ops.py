@@ -194,10 +194,28 @@ def _q_starts(q_starts, dev):
 
 
 # --------------------------------------------------------------------------------------------- MLA decode
-def mla_paged_attention(query, latent_cache, block_tables, context_lens, n_heads, kv_lora_rank, scale, out=None):
+def mla_paged_attention(query, latent_cache, block_tables, context_lens, n_heads, kv_lora_rank, scale, out=None,
+                        q_seq_lens=None):
     """PagedAttention(head_num, scale, 1, mla_v_dim=kv_lora_rank)(query, cache, cache, block_tables, context_lens):
     query [B, n_heads * (kv_lora_rank + rope)], latent cache [num_blocks, block_size, 1, kv_lora_rank + rope];
-    returns [B, n_heads * kv_lora_rank]."""
+    returns [B, n_heads * kv_lora_rank].
+
+    ``q_seq_lens`` (int32 [B], several new tokens per sequence, causal among themselves: parallel decoding / chunked
+    prefill, flash_attention.py:140-143): query holds sum(q_seq_lens) rows packed sequence after sequence.  Every
+    query row is run as a sequence of its own whose context ends at its own position (its block-table row repeated,
+    built on the device without a host synchronisation), so the result is exactly the one-query kernel's."""
+    if q_seq_lens is not None:
+        _need(q_seq_lens.dtype == torch.int32 and q_seq_lens.numel() == context_lens.numel(), "q_seq_lens must be int32 [B]")
+        dk = latent_cache.shape[-1]
+        rows = query.numel() // (n_heads * dk) if query.is_contiguous() else query.shape[0]
+        b = context_lens.numel()
+        ql = q_seq_lens.to(torch.int64)
+        seq = torch.repeat_interleave(torch.arange(b, device=query.device), ql, output_size=rows)
+        first = torch.cumsum(ql, 0) - ql                          # first query row of every sequence
+        pos = torch.arange(rows, device=query.device) - first[seq]
+        lens = (context_lens.to(torch.int64)[seq] - ql[seq] + pos + 1).clamp(min=0).to(torch.int32)
+        return mla_paged_attention(query, latent_cache, block_tables[seq].contiguous(), lens.contiguous(), n_heads,
+                                   kv_lora_rank, scale, out=out)
     lib = _lib.load()
     _dev_of(query)
     dev = _dev_ok(latent_cache, block_tables, context_lens, out)

@@ -734,6 +734,31 @@ def test_mcore_flash_attention_mla_decode_branch():
     assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA decode")
 
 
+def test_mcore_flash_attention_mla_decode_with_q_seq_lens():
+    """MLA decode with several new tokens per sequence (q_seq_lens: parallel decoding / chunked prefill,
+    flash_attention.py:140-143): every query row sees the latent cache up to its own position; a sequence without new
+    tokens contributes no rows."""
+    from mindformers_amd.modules import FlashAttention
+    rng = np.random.default_rng(29)
+    nh, bs = 16, 32
+    lens = np.array([70, 300, 33, 129])
+    q_lens = np.array([3, 1, 0, 5])
+    cache, _, tables, nb = make_paged_cache(rng, 4, lens, 1, 576, bs, BF)
+    net = FlashAttention(head_num=nh, head_dim=576, kv_head_num=1, pa_kv_head_num=1, scale_value=0.072, pa_mla_v_dim=512)
+    net.is_prefill = False
+    rows = int(q_lens.sum())
+    q = rounded(rng.normal(size=(rows, nh * 576)), BF)
+    out = net(query=dev(q, BF), key=None, value=None, slot_mapping=None, block_tables=dev(tables, torch.int32),
+              batch_valid_length=torch.from_numpy(lens.astype(np.int32)).cuda(),
+              q_seq_lens=torch.from_numpy(q_lens.astype(np.int32)).cuda(), key_cache=dev(cache, BF), value_cache=None)
+    assert out.shape == (rows, nh * 512)
+    seq = np.repeat(np.arange(4), q_lens)
+    limit = np.concatenate([np.arange(l - ql + 1, l + 1) for l, ql in zip(lens, q_lens)])
+    ref = O.mla_paged_attention_decode(q, cache, tables[seq], limit, nh, 512, 0.072)
+    mag = O.mla_paged_attention_decode(q, cache, tables[seq], limit, nh, 512, 0.072, abs_values=True)
+    assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA decode, several tokens per sequence")
+
+
 # ------------------------------------------------------------------------------------------- kvcache_dtype: int8
 @pytest.mark.parametrize("dynamic", [True, False])
 def test_quantizer_swaps_in_the_int8_kv_manager_and_decode_matches_oracle(dynamic):
