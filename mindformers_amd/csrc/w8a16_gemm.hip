@@ -345,7 +345,7 @@ template <typename T, int MT, int NT, bool KTAIL>
 __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
     uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
     const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated) {
+    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated, int split_major) {
     using vec8 = typename T::vec8;
     using C = G2<MT, NT>;
     constexpr int D = C::DEPTH;
@@ -356,10 +356,14 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
     const int lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
     const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
-    const int s_begin = blockIdx.y * steps_per_split;
+    // split_major: the k-split index varies fastest over the workgroup ids, so that (8 splits, workgroup id % 8 =
+    // the XCD) every XCD's L2 fetches one eighth of the activations instead of all of them
+    const int split = split_major ? blockIdx.x : blockIdx.y;
+    const int nblock = split_major ? blockIdx.y : blockIdx.x;
+    const int s_begin = split * steps_per_split;
     const int s_end = min(KS, s_begin + steps_per_split);
     const int s_last = s_end - 1;
-    const int n0 = blockIdx.x * (G2_WAVES * NT * 16) + wv * (NT * 16);      // first output channel of this wave
+    const int n0 = nblock * (G2_WAVES * NT * 16) + wv * (NT * 16);          // first output channel of this wave
     const int m0 = blockIdx.z * C::XROWS;
 
     f32x4 acc[NT][MT];
@@ -510,7 +514,7 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
             for (int mt = 0; mt < MT; ++mt) {
                 const int m = m0 + 16 * mt + r;
                 if (m >= M) continue;
-                float* p = partial + ((int64_t)blockIdx.y * M + m) * N + n;
+                float* p = partial + ((int64_t)split * M + m) * N + n;
                 if (vec) {
                     *(f32x4*)p = acc[nt][mt];
                 } else {
@@ -850,6 +854,7 @@ GemmPlan plan_w8a16(int m, int n, int k) {
     const int max_sk = total_steps / 12 < 1 ? 1 : total_steps / 12;
     sk = sk > max_sk ? max_sk : sk;
     sk = sk > 16 ? 16 : sk;
+    if (sk > 8) sk = 8 * (sk / 8);                             // multiples of 8 can run split-major
     p.steps_per_split = (total_steps + sk - 1) / sk;
     p.split_k = (total_steps + p.steps_per_split - 1) / p.steps_per_split;
     return p;
@@ -862,7 +867,8 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
                  const RopeCacheArgs* rc_args = nullptr) {
     const GemmPlan p = plan_w8a16(m, n, k);
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
-    dim3 grid(p.n_blocks, p.split_k, p.m_blocks);
+    const int split_major = p.split_k % 8 == 0;
+    dim3 grid(split_major ? p.split_k : p.n_blocks, split_major ? p.n_blocks : p.split_k, p.m_blocks);
     dim3 block(G2_WAVES * 64);
 #define GW_LAUNCH(MTV, KT)                                                                                       \
     do {                                                                                                         \
@@ -879,7 +885,7 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
         }                                                                                                        \
         hipLaunchKernelGGL(kern, grid, block, lds, st, (uint16_t*)y, partial, (const uint16_t*)x, wp, scale,      \
                            (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split,     \
-                           gated);                                                                               \
+                           gated, split_major);                                                                  \
     } while (0)
     const bool ktail = (k % GW_KSTEP) != 0;
     if (p.mt == 1) { if (ktail) GW_LAUNCH(1, true); else GW_LAUNCH(1, false); }
