@@ -34,16 +34,38 @@ __global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ we
     if (n_group > 1 && topk_group < n_group) {
         const int gs = E / n_group;
         float score = -INFINITY;
-        if (lane < n_group) {
+        if ((n_group & (n_group - 1)) == 0) {
+            // 64 / n_group lanes share a group: each scans a strided part, the pairs of largest values merge by
+            // shuffles (values only, so the order of the merge does not matter)
+            const int lpg = 64 / n_group;
+            const int grp = lane / lpg, sub = lane - grp * lpg;
             float a = -INFINITY, b = -INFINITY;               // two largest of the group
-            for (int i = 0; i < gs; ++i) {
-                const float v = s_biased[lane * gs + i];
+            for (int i = sub; i < gs; i += lpg) {
+                const float v = s_biased[grp * gs + i];
                 if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
             }
+            for (int o = 1; o < lpg; o <<= 1) {
+                const float oa = __shfl_xor(a, o, 64), ob = __shfl_xor(b, o, 64);
+                const float hi = fmaxf(a, oa);
+                b = a >= oa ? fmaxf(b, oa) : fmaxf(ob, a);
+                a = hi;
+            }
             score = gs >= 2 ? a + b : a;
-            s_gscore[lane] = score;
+            if (sub == 0) s_gscore[grp] = score;
+            __syncthreads();
+            score = lane < n_group ? s_gscore[lane] : -INFINITY;
+        } else {
+            if (lane < n_group) {
+                float a = -INFINITY, b = -INFINITY;
+                for (int i = 0; i < gs; ++i) {
+                    const float v = s_biased[lane * gs + i];
+                    if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+                }
+                score = gs >= 2 ? a + b : a;
+                s_gscore[lane] = score;
+            }
+            __syncthreads();
         }
-        __syncthreads();
         if (lane < n_group) {
             int rank = 0;                                     // groups strictly ahead (ties: lower index first)
             for (int j = 0; j < n_group; ++j) {
@@ -60,16 +82,22 @@ __global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ we
         __syncthreads();
     }
 
-    // top-k by repeated wave-wide argmax (larger value first, ties to the lower index)
+    // top-k by repeated wave-wide argmax (larger value first, ties to the lower index); the candidates live in
+    // registers, expert e = lane + 64 i in slot i
     __shared__ float s_wsel[RT_MAX_K];
     __shared__ int s_isel[RT_MAX_K];
+    constexpr int SLOTS = RT_MAX_E / 64;
+    float cand[SLOTS];
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) cand[i] = lane + 64 * i < E ? s_biased[lane + 64 * i] : -INFINITY;
     float wsum = 0.f;
     for (int j = 0; j < k; ++j) {
         float best = -INFINITY;
         int bi = 0x7fffffff;
-        for (int e = lane; e < E; e += 64) {
-            const float v = s_biased[e];
-            if (v > best) { best = v; bi = e; }               // ascending e: first maximum wins
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i) {
+            const bool live = lane + 64 * i < E;
+            if (live && cand[i] > best) { best = cand[i]; bi = lane + 64 * i; }   // ascending e: first maximum wins
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
@@ -80,14 +108,15 @@ __global__ __launch_bounds__(64) void moe_route_kernel(uint16_t* __restrict__ we
         if (bi >= E) bi = 0;                                  // all -inf/NaN rows: keep indices in range
         const float wv = biased_weights ? best : s_plain[bi];
         wsum += wv;
-        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i)
+            if (bi == lane + 64 * i) cand[i] = -INFINITY;
         if (lane == 0) {
             s_wsel[j] = wv;
             s_isel[j] = bi;
-            s_biased[bi] = -INFINITY;
         }
-        __syncthreads();
     }
+    __syncthreads();
     if (lane == 0) {
         for (int j = 0; j < k; ++j) {
             float wv = s_wsel[j];
@@ -114,15 +143,30 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(int32_t* __restrict__ ro
         if (e >= 0 && e < E) atomicAdd(&s_cnt[e], 1);
     }
     __syncthreads();
-    if (tid == 0) {                                           // E <= 1024: a serial scan is a few microseconds
-        int run = 0;
-        for (int e = 0; e < E; ++e) {
-            s_cur[e] = run;
-            offsets[e] = run;
-            counts[e] = s_cnt[e];
-            run += s_cnt[e];
+    if (tid < 64) {                                           // exclusive scan: a chunk of experts per lane of wave 0
+        const int per = (E + 63) / 64;
+        const int e0 = tid * per;
+        int local = 0;
+        for (int i = 0; i < per; ++i)
+            if (e0 + i < E) local += s_cnt[e0 + i];
+        int incl = local;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, 64);
+            if (tid >= o) incl += up;
         }
-        offsets[E] = run;
+        int run = incl - local;
+        for (int i = 0; i < per; ++i) {
+            const int e = e0 + i;
+            if (e < E) {
+                const int c = s_cnt[e];
+                s_cur[e] = run;
+                offsets[e] = run;
+                counts[e] = c;
+                run += c;
+            }
+        }
+        if (tid == 63) offsets[E] = incl;
     }
     __syncthreads();
     // stable placement: wave 0 walks the pairs in order, 64 at a time
@@ -169,35 +213,57 @@ __global__ void moe_gather_kernel(uint16_t* __restrict__ permuted, const uint16_
     for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) *(u32x4*)(d + i) = *(const u32x4*)(src + i);
 }
 
-// out[t] = sum_j probs[t,j] * y[row_map[t*k+j]] (+ shared[t]); one workgroup per token.
+// out[t] = sum_j probs[t,j] * y[row_map[t*k+j]] (+ shared[t]); grid = (tokens, column chunks of 8 * blockDim.x), one
+// 16-byte item per thread.  The k row indices and weights are read first, then the k rows are loaded in batches of
+// UNP_BATCH independent loads and summed in choice order (the order fixes the fp32 sum).
+constexpr int UNP_BATCH = 8;
 template <typename T>
 __global__ void moe_unpermute_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ y,
                                      const int32_t* __restrict__ row_map, const uint16_t* __restrict__ probs,
                                      const uint16_t* __restrict__ shared, int k, int hidden, int pairs) {
     const int t = blockIdx.x;
-    for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
-        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int j = 0; j < k; ++j) {
-            const int row = row_map[(int64_t)t * k + j];
-            if (row < 0 || row >= pairs) continue;
-            const float pw = T::to_float(probs[(int64_t)t * k + j]);
-            float v[8];
-            unpack8<T>(*(const u32x4*)(y + (int64_t)row * hidden + i), v);
+    const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+    if (i >= hidden) return;
+    u32x4 sh = {0u, 0u, 0u, 0u};
+    if (shared) sh = *(const u32x4*)(shared + (int64_t)t * hidden + i);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j0 = 0; j0 < k; j0 += UNP_BATCH) {
+        int row[UNP_BATCH];
+        float pw[UNP_BATCH];
+        u32x4 v[UNP_BATCH];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) acc[q] += pw * v[q];
+        for (int j = 0; j < UNP_BATCH; ++j) {
+            const int jj = j0 + j;
+            row[j] = jj < k ? row_map[(int64_t)t * k + jj] : -1;
+            pw[j] = jj < k ? T::to_float(probs[(int64_t)t * k + jj]) : 0.f;
         }
-        if (shared) {
-            // the routed sum is materialised in the activation dtype before the shared-expert add
-            float v[8];
-            unpack8<T>(*(const u32x4*)(shared + (int64_t)t * hidden + i), v);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) acc[q] = T::to_float(T::from_float(acc[q])) + v[q];
+        for (int j = 0; j < UNP_BATCH; ++j) {
+            const bool ok = row[j] >= 0 && row[j] < pairs;
+            v[j] = (u32x4){0u, 0u, 0u, 0u};
+            if (ok) v[j] = *(const u32x4*)(y + (int64_t)row[j] * hidden + i);
+            else row[j] = -1;
         }
-        u32x4 o;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) o[q] = pack2<T>(acc[2 * q], acc[2 * q + 1]);
-        *(u32x4*)(out + (int64_t)t * hidden + i) = o;
+        for (int j = 0; j < UNP_BATCH; ++j) {
+            if (row[j] < 0) continue;                         // a skipped choice adds nothing (not even +0)
+            float f[8];
+            unpack8<T>(v[j], f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[q] += pw[j] * f[q];
+        }
     }
+    if (shared) {
+        // the routed sum is materialised in the activation dtype before the shared-expert add
+        float f[8];
+        unpack8<T>(sh, f);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[q] = T::to_float(T::from_float(acc[q])) + f[q];
+    }
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = pack2<T>(acc[2 * q], acc[2 * q + 1]);
+    *(u32x4*)(out + (int64_t)t * hidden + i) = o;
 }
 
 }  // namespace
@@ -253,12 +319,14 @@ extern "C" int mf_moe_unpermute(void* out, const void* y, const int32_t* row_map
     MF_REQUIRE((((uintptr_t)out | (uintptr_t)y | (uintptr_t)shared) & 15) == 0,
                "moe_unpermute: rows must be 16-byte aligned");
     if (tokens <= 0) return 0;
+    constexpr int UNP_THREADS = 128;
+    const dim3 ugrid(tokens, (hidden / 8 + UNP_THREADS - 1) / UNP_THREADS);
     if (dtype == MF_BF16)
-        hipLaunchKernelGGL(moe_unpermute_kernel<BF16>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+        hipLaunchKernelGGL(moe_unpermute_kernel<BF16>, ugrid, dim3(UNP_THREADS), 0, (hipStream_t)stream, (uint16_t*)out,
                            (const uint16_t*)y, row_map, (const uint16_t*)probs, (const uint16_t*)shared, k, hidden,
                            tokens * k);
     else
-        hipLaunchKernelGGL(moe_unpermute_kernel<FP16>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+        hipLaunchKernelGGL(moe_unpermute_kernel<FP16>, ugrid, dim3(UNP_THREADS), 0, (hipStream_t)stream, (uint16_t*)out,
                            (const uint16_t*)y, row_map, (const uint16_t*)probs, (const uint16_t*)shared, k, hidden,
                            tokens * k);
     return MF_LAUNCH_CHECK();
