@@ -1036,7 +1036,8 @@ def test_w8a8_qkv_rope_and_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, bi
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
 
 
-@pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1)])
+@pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1),
+                                         (9, 96, 4, 3, 2), (6, 60, 5, 6, 2), (4, 1024, 32, 16, 8), (3, 640, 7, 64, 9)])
 def test_moe_route(t, e, k, ng, tg):
     rng = np.random.default_rng(13)
     logits = rng.normal(size=(t, e)).astype(np.float32)
@@ -1045,6 +1046,44 @@ def test_moe_route(t, e, k, ng, tg):
     w_ref, idx_ref = O.topk_router(logits, bias, k, ng, tg, 2.5)
     assert np.array_equal(to_np(idx), idx_ref)
     assert_within(to_np(w), w_ref, np.abs(w_ref), torch.bfloat16, ulps=1.0, what="router weights")
+
+
+def test_moe_route_ties_go_to_the_lower_index():
+    """Equal scores (constant logits, and a row of two distinct values): experts and groups are taken in index order."""
+    e, k, ng, tg = 64, 6, 8, 3
+    logits = np.zeros((3, e), np.float32)
+    logits[1, 40:] = 1.0
+    logits[2, ::2] = 0.5
+    bias = np.zeros(e, np.float32)
+    w, idx = ops.moe_route(torch.from_numpy(logits).cuda(), torch.from_numpy(bias).cuda(), k, ng, tg, 1.0, torch.bfloat16)
+    w_ref, idx_ref = O.topk_router(logits, bias, k, ng, tg, 1.0)
+    assert np.array_equal(to_np(idx), idx_ref)
+    assert_within(to_np(w), w_ref, np.abs(w_ref), torch.bfloat16, ulps=1.0, what="router weights")
+
+
+@pytest.mark.parametrize("t,h,e,k", [(5, 64, 300, 1), (130, 7168, 256, 8), (3, 8, 4, 4), (70, 1032, 17, 9)])
+def test_moe_permute_unpermute_shapes(t, h, e, k):
+    """Permute / weighted unpermute at the edges: one choice per token, more experts than lanes of a scan chunk, the
+    full DeepSeek-V3 width, a width that is not a multiple of the column chunk, more than one batch of choices."""
+    rng = np.random.default_rng(t + h + e + k)
+    dtype = torch.bfloat16
+    x = rounded(rng.normal(size=(t, h)), dtype)
+    idx = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+    probs = rounded(rng.uniform(0.1, 1.0, (t, k)), dtype)
+    shared = rounded(rng.normal(size=(t, h)), dtype)
+    px, row_map, counts, offsets = ops.moe_permute(dev(x, dtype), torch.from_numpy(idx).cuda(), e)
+    px_ref, map_ref, cnt_ref = O.moe_permute(x, idx, e)
+    assert np.array_equal(to_np(row_map), map_ref) and np.array_equal(to_np(counts), cnt_ref)
+    assert np.array_equal(to_np(offsets), np.concatenate(([0], np.cumsum(cnt_ref))).astype(np.int32))
+    assert np.array_equal(to_np(px), px_ref)
+    y = rounded(rng.normal(size=(t * k, h)), dtype)
+    for sh in (None, shared):
+        out = ops.moe_unpermute(dev(y, dtype), row_map, dev(probs, dtype), shared=None if sh is None else dev(sh, dtype))
+        ref = O.moe_unpermute(y, map_ref, probs)
+        mag = O.moe_unpermute(np.abs(y), map_ref, probs)
+        if sh is not None:                       # the routed sum is rounded to the activation dtype before the add
+            ref, mag = rounded(ref, dtype) + sh, mag + np.abs(sh)
+        assert_within(to_np(out), ref, mag, dtype, ulps=1.0, extra=2.0 ** -9 * EPS[dtype] * mag + 1e-9, what="unpermute")
 
 
 def test_moe_permute_grouped_unpermute():
