@@ -10,9 +10,10 @@
 // from the row-major matrix makes every group of lanes touch 16 different cache lines per instruction and
 // ran at about a third of the bandwidth.)
 //
-// Two kernels share the format.  The dense kernel (w8a16_gemm2_kernel, described where it is defined) stages
-// activation and weight tiles through a ring of LDS-direct loads and serves the decode layer's projections; its
-// epilogue, or the split-K reduce kernels, carry the fused variants (gate/up + SiLU*mul, residual + RMSNorm,
+// Two kernels share the format.  The dense kernel (w8a16_gemm4_kernel, described where it is defined) loads weight
+// tiles straight into MFMA operand registers, shares one LDS-staged activation tile among the waves of a workgroup
+// and serves the decode layer's projections; its epilogue, or the split-K reduce kernels, carry the fused variants
+// (gate/up + SiLU*mul, residual + RMSNorm,
 // QKV + RoPE + cache scatter).  The grouped kernel (experts) keeps the earlier register-streaming tile routine
 // w8a16_tile: a workgroup of 4 waves owns 64 output channels (4 n-tiles) for up to 64 rows of x; the waves
 // interleave the 64-wide k-steps of the workgroup's k-range, each streams its tiles HBM -> registers two steps
@@ -261,50 +262,9 @@ __global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_gemm_kernel(
                       blockIdx.z * (16 * MT), s_begin, s_end, blockIdx.y, smem);
 }
 
-// ---- dense kernel -----------------------------------------------------------------------------------
-// grid = (ceil(N / (16*NT*G)), split_k, ceil(M / (16*MT))), G waves per workgroup.  The waves of a workgroup walk
-// the same k-steps and own different output channels (wave w: n-tiles [w*NT, (w+1)*NT) of the workgroup's block),
-// so one staged activation tile ([16*MT rows, 64 k] as 128-byte rows) serves all of them.  Activation tiles and
-// weight tiles both go global -> LDS without passing through registers (LDS-direct loads: lane l's 16 bytes land
-// at base + 16*l), DEPTH steps ahead of their use, into a ring of DEPTH + 1 stages; a stage holds the shared
-// activation tile and one private 1 KiB weight tile per wave and n-tile.  The 16-byte chunks of an activation row
-// are XOR-swizzled (physical chunk = logical chunk ^ g2_swizzle_key(row)), applied on the global-address side, so
-// that the operand reads are free of LDS bank conflicts.  Every wave issues the same number of LDS-direct loads
-// per step and they complete in issue order, so "at most DEPTH-1 steps' worth of loads outstanding" means that
-// this wave's loads for step s have landed; one barrier per step makes that true for the whole workgroup and also
-// tells that the stage about to be overwritten has been read by everybody.  (Weight tiles kept in registers
-// instead would mix two kinds of loads under one counter, and those do not complete in order relative to each
-// other.)  Loads past the k-range re-read the last step and are never used, so that the outstanding-load count
-// is the same in every step.
-//
-// The main loop is issue-bound once the memory pipeline is deep enough, so it is kept lean: the loop is unrolled
-// over the ring (every LDS offset is an immediate), global addresses are a scalar base per step plus a per-lane
-// 32-bit offset that never changes, and the only per-byte vector work left is the int8 -> bf16 conversion.
-//
-// The compiler's own wait-count insertion cannot express this pipeline (it waits for *every* LDS-direct load
-// before any LDS read), so the LDS reads of the main loop and their waits are written as asm statements: each
-// wait names the registers it makes valid as in/out operands, which keeps their consumers behind it.
+// ---- dense kernel: helpers ---------------------------------------------------------------------------
 constexpr int G2_WAVES = 4;
-constexpr int G2_NT = 1;                    // weight tiles per wave
-constexpr int G2_BN = G2_WAVES * G2_NT * 16; // output channels per workgroup
-
-template <int MT, int NT>
-struct G2 {
-    static constexpr int XROWS = 16 * MT;
-    static constexpr int XTILE = XROWS * 128;
-    static constexpr int STAGE = XTILE + G2_WAVES * NT * GW_TILE_BYTES;
-    static constexpr int STAGES = 4;
-    static constexpr int DEPTH = STAGES - 1;                  // steps between the issue of a stage's loads and its use
-    // activation loads per wave per stage: whole-wave loads of 8 rows each, or (16 rows over 4 waves) one load of
-    // 4 rows issued by half of the lanes
-    static constexpr bool HALF = 2 * MT < G2_WAVES;
-    static constexpr int XL = HALF ? 1 : 2 * MT / G2_WAVES;
-    // at the top of step s the loads of step s+1 must have landed: those of steps s+2 .. s+DEPTH-1 may be in flight
-    static constexpr int PENDING = (DEPTH - 2) * (XL + NT);
-    static constexpr int LDS_BYTES = STAGES * STAGE;
-    static_assert((HALF ? 4 * MT == G2_WAVES : XL * G2_WAVES == 2 * MT) && PENDING + XL + NT < 64 &&
-                      LDS_BYTES <= 160 * 1024, "bad pipeline shape");
-};
+constexpr int G2_BN = G2_WAVES * 16;        // output channels of a 4-wave workgroup
 
 // A 16-byte-per-lane LDS read is served 16 lanes per cycle over 64 banks (256 bytes); measured on gfx950, the
 // lanes that share a cycle are those of one half of the wave with equal parity of lane bits 2, 3 and 4 - for an
@@ -334,73 +294,89 @@ template <int LGKM>
 __device__ __forceinline__ void g2_wait_lds(u32x4& a, u32x4& b, u32x4& c, u32x4& d) {
     asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(LGKM) : "memory");
 }
-// 16 bytes per lane from (wave-uniform base + per-lane byte offset) to (wave-uniform LDS address + 16*lane)
-__device__ __forceinline__ void g2_lds_direct16(const uint8_t* base_uniform, uint32_t lane_offset,
-                                                uint8_t* dst_wave_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base_uniform + lane_offset),
-                                     (__attribute__((address_space(3))) void*)dst_wave_uniform, 16, 0, 0);
-}
+// ---- dense kernel, weights through registers --------------------------------------------------------------
+// grid = (ceil(N / (16 * tiles)), split_k, ceil(M / (16*MT))) (or (split_k, n-blocks, m-blocks) when split-major).
+// The waves of a workgroup walk the same k-steps and own different 16-channel weight tiles, so one staged activation
+// tile ([16*MT rows, 64 k] as 128-byte rows) serves all of them: 4 waves up to 32 rows, 8 waves beyond (one
+// activation byte per weight byte instead of two; the L2 -> CU path saturates near 11 TB/s, so the activation
+// re-reads are what a skinny GEMM at 64 rows pays most for).  Both operands are fetched by ordinary 16-byte-per-lane
+// loads into registers.  (An earlier version used LDS-direct loads for both.  Measured on this part with the GEMM's
+// own grid and weight order - 448 workgroups x 64 k-steps x 4 KiB, cold - register loads stream 117 MB at 5.3 TB/s
+// and LDS-direct loads at 3.4-3.5 TB/s whatever their number in flight, which is where that version's gate/up launch
+// stood.)  A weight tile in registers is already the MFMA operand (after the int8 -> T conversion), so it never
+// touches LDS; the activation tile is written to LDS by the lanes that loaded it, its 16-byte chunks XOR-swizzled
+// (physical chunk = logical chunk ^ g2_swizzle_key(row), applied on the global-address side) so that the operand
+// reads are free of bank conflicts, and read back as B operands by all waves.  A wave keeps DEPTH steps of
+// loads in flight in a rotating set of registers (loads complete in issue order: the wait in front of a step's first
+// use lets DEPTH-2 steps' worth stay outstanding).  Two LDS stages alternate: the activations of step s+1 are written
+// while the operands of step s (read during step s-1) are multiplied.
+template <int MT, int WAVES>
+struct G4 {
+    static constexpr int XROWS = 16 * MT;
+    static constexpr int XTILE = XROWS * 128;
+    static constexpr int DEPTH = 4;                           // register sets = steps of loads in flight (even)
+    static constexpr int BN = 16 * WAVES;                     // output channels per workgroup, one tile per wave
+    // activation loads (8 rows each) per wave and step: the 2*MT loads of a tile are dealt over the waves; where there
+    // are more waves than loads the surplus waves repeat loads of the others (every wave issues the same number of
+    // loads) and do not write them
+    static constexpr int XL = 2 * MT > WAVES ? 2 * MT / WAVES : 1;
+    static constexpr int XWRITERS = 2 * MT / XL;              // waves that write activations
+    static_assert(XL * XWRITERS == 2 * MT && XWRITERS <= WAVES && XL <= 2, "bad split of the activation loads");
+};
 
-template <typename T, int MT, int NT, bool KTAIL>
-__global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
+template <typename T, int MT, int WAVES, bool KTAIL>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_kernel(
     uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
     const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
     const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated, int split_major) {
     using vec8 = typename T::vec8;
-    using C = G2<MT, NT>;
+    using C = G4<MT, WAVES>;
     constexpr int D = C::DEPTH;
-    static_assert(NT == 1 || NT == 2, "one or two weight tiles per wave");
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];       // C::LDS_BYTES, set by the launcher
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * C::XTILE];
 
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
     const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
-    // split_major: the k-split index varies fastest over the workgroup ids, so that (8 splits, workgroup id % 8 =
-    // the XCD) every XCD's L2 fetches one eighth of the activations instead of all of them
     const int split = split_major ? blockIdx.x : blockIdx.y;
     const int nblock = split_major ? blockIdx.y : blockIdx.x;
     const int s_begin = split * steps_per_split;
     const int s_end = min(KS, s_begin + steps_per_split);
     const int s_last = s_end - 1;
-    const int n0 = nblock * (G2_WAVES * NT * 16) + wv * (NT * 16);          // first output channel of this wave
+    const int n0 = nblock * C::BN + wv * 16;                  // first output channel of this wave
     const int m0 = blockIdx.z * C::XROWS;
 
-    f32x4 acc[NT][MT];
+    f32x4 acc[MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // weights: tile (n-tile t, step s) sits at (s*n_tiles + t) * 1024 + lane*16; tiles past N are clamped (never
-    // stored)
     const int n_tiles_total = (N + 15) >> 4;
-    const uint8_t* wtile[NT];                                 // wave-uniform: step 0 of this wave's n-tiles
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-        wtile[nt] = wp + (int64_t)min((n0 >> 4) + nt, n_tiles_total - 1) * GW_TILE_BYTES;
+    const uint8_t* wtile = wp + (int64_t)min(n0 >> 4, n_tiles_total - 1) * GW_TILE_BYTES;   // wave-uniform
+    const int64_t wstride = (int64_t)n_tiles_total * GW_TILE_BYTES;
     const uint32_t wlane = lane * 16;
-    // activations: load i of this wave covers rows 8*(wv*XL + i) .. + 7 of the stage (HALF: rows 4*wv .. + 3, lanes
-    // 0-31); lane -> (row, physical chunk), the global address uses the logical chunk.  Rows past M re-read row
-    // M-1 (never stored).
-    const uint8_t* xbase = (const uint8_t*)(x + (int64_t)m0 * K);          // wave-uniform
-    uint32_t xlane[C::XL];                                    // byte offset of the lane's chunk at step 0
+    const uint8_t* xbase = (const uint8_t*)(x + (int64_t)m0 * K);                            // wave-uniform
+    uint32_t xlane[C::XL];
     int xchunk8[C::XL];
-    int xdst[C::XL];                                          // first byte of the load inside a stage
-    const bool xactive = !C::HALF || lane < 32;
+    uint32_t xdst[C::XL];                                     // LDS byte of the lane's chunk inside a stage
+    const bool xwrite = wv < C::XWRITERS;
 #pragma unroll
     for (int i = 0; i < C::XL; ++i) {
-        const int row0 = C::HALF ? 4 * wv : 8 * (wv * C::XL + i);
+        const int row0 = 8 * ((wv % C::XWRITERS) * C::XL + i);
         const int row = row0 + (lane >> 3);
-        xdst[i] = row0 * 128;
+        xdst[i] = row0 * 128 + lane * 16;
         xchunk8[i] = 8 * ((lane & 7) ^ g2_swizzle_key(row));
         xlane[i] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K * 2u + 2u * xchunk8[i];
     }
-    const int wlds = C::XTILE + wv * NT * GW_TILE_BYTES;      // this wave's weight tiles inside a stage
 
-    auto issue = [&](int stage, int s) {                      // stage is a compile-time constant at every call
+    // All memory operations below are ordinary loads and stores, so the compiler itself places the counted waits in
+    // front of the first use of every register (a hand-written wait cannot stop the register allocator from copying a
+    // register whose load is still in flight).  For its count to stay exact, the main loop is free of conditional
+    // steps: it runs over whole groups of D steps, the remaining 0 .. D-1 steps follow it.
+    u32x4 wreg[D], xreg[D][C::XL];
+    auto issue = [&](auto setc, int s) {
+        constexpr int S = decltype(setc)::value;
         const int sc = min(s, s_last);
-        uint8_t* dst = smem + stage * C::STAGE;
+        wreg[S] = *(const u32x4*)(wtile + sc * wstride + wlane);
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
             uint32_t off = xlane[i] + (uint32_t)sc * (GW_KSTEP * 2);
@@ -410,127 +386,91 @@ __global__ __launch_bounds__(G2_WAVES * 64) void w8a16_gemm2_kernel(
                 const int over = sc * GW_KSTEP + xchunk8[i] - (K - 8);
                 off -= over > 0 ? 2u * over : 0u;
             }
-            if (xactive) g2_lds_direct16(xbase, off, dst + xdst[i]);
+            xreg[S][i] = *(const u32x4*)(xbase + off);
         }
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            g2_lds_direct16(wtile[nt] + (int64_t)sc * n_tiles_total * GW_TILE_BYTES, wlane,
-                            dst + wlds + nt * GW_TILE_BYTES);
     };
+    auto stage_x = [&](auto setc, int stage) {                // this wave's activation chunks of a set -> LDS stage
+        constexpr int S = decltype(setc)::value;
+        if (xwrite) {
 #pragma unroll
-    for (int p = 0; p < D; ++p) issue(p, s_begin + p);
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+            for (int i = 0; i < C::XL; ++i) *(u32x4*)(smem + stage * C::XTILE + xdst[i]) = xreg[S][i];
+        }
+    };
     // B operands: lane (r, g), tile mt, half h reads logical chunk 2g + h of row 16*mt + r
-    const uint32_t xoff0 = lds0 + r * 128 + (((2 * g) ^ g2_swizzle_key(r)) << 4);
-    const uint32_t xoff1 = lds0 + r * 128 + (((2 * g + 1) ^ g2_swizzle_key(r)) << 4);
-    const uint32_t woff = lds0 + wlds + lane * 16;
+    const int xoff0 = r * 128 + (((2 * g) ^ g2_swizzle_key(r)) << 4);
+    const int xoff1 = r * 128 + (((2 * g + 1) ^ g2_swizzle_key(r)) << 4);
+    u32x4 xb[2][MT][2];
+    auto read_operands = [&](auto stagec) {
+        constexpr int P = decltype(stagec)::value;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            xb[P][mt][0] = *(const u32x4*)(smem + P * C::XTILE + 2048 * mt + xoff0);
+            xb[P][mt][1] = *(const u32x4*)(smem + P * C::XTILE + 2048 * mt + xoff1);
+        }
+    };
 
-    // Register sets for the operands of two consecutive steps: while step s is converted and multiplied out of one
-    // set, the LDS reads of step s+1 fill the other.
-    u32x4 wr[2][NT], xb[2][MT][2];
-    auto read_operands = [&](auto setc, auto stagec) {
-        constexpr int P = decltype(setc)::value;
-        constexpr int SB = decltype(stagec)::value * C::STAGE;
-        wr[P][0] = g2_lds_read16<SB>(woff);
-        if constexpr (NT == 2) wr[P][1] = g2_lds_read16<SB + GW_TILE_BYTES>(woff);
-        static_for<MT>([&](auto mc) {
-            constexpr int mt = decltype(mc)::value;
-            xb[P][mt][0] = g2_lds_read16<SB + 2048 * mt>(xoff0);
-            xb[P][mt][1] = g2_lds_read16<SB + 2048 * mt>(xoff1);
-        });
-    };
-    auto operands_arrived = [&](auto setc) {                  // all LDS reads issued so far have returned
-        constexpr int P = decltype(setc)::value;
-        if constexpr (NT == 1) g2_wait_lds<0>(wr[P][0], xb[P][0][0], xb[P][0][1]);
-        else g2_wait_lds<0>(wr[P][0], wr[P][1], xb[P][0][0], xb[P][0][1]);
-        if constexpr (MT >= 2) g2_wait_lds<0>(xb[P][1][0], xb[P][1][1]);
-        if constexpr (MT == 4) g2_wait_lds<0>(xb[P][2][0], xb[P][2][1], xb[P][3][0], xb[P][3][1]);
-    };
-    // step s: its operands are in register set J & 1 (read during step s-1); stage J + 1 (step s+1) must have
-    // landed for the whole workgroup before it is read, hence the counter wait and the barrier at the top
+    // prologue: D steps of loads in flight, the first step's activations staged and its operands read
+    static_for<D>([&](auto dc) { issue(dc, s_begin + decltype(dc)::value); });
+    stage_x(std::integral_constant<int, 0>{}, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    read_operands(std::integral_constant<int, 0>{});
+
+    // step s: register set J holds its weight tile, LDS stage J & 1 held its activations (operands already in
+    // xb[J & 1]); set J + 1 (step s + 1) is needed now: its activations go to the other stage
     auto step = [&](auto jc, int s) {
-        constexpr int J = decltype(jc)::value;                // ring stage of step s
+        constexpr int J = decltype(jc)::value;
+        constexpr int JN = (J + 1) % D;
         constexpr int P = J & 1;
         __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::PENDING) : "memory");
+        stage_x(std::integral_constant<int, JN>{}, P ^ 1);
+        vec8 wa[2];
+        wa[0] = dequant8<T>(wreg[J][0], wreg[J][1]);
+        wa[1] = dequant8<T>(wreg[J][2], wreg[J][3]);
+        // the conversion happens here, before the set is reloaded (sunk below the reload it would keep the old
+        // registers alive next to the new ones, and the sets would no longer rotate in place)
+        asm volatile("" : "+v"(wa[0]), "+v"(wa[1]));
+        __builtin_amdgcn_sched_barrier(0);
+        issue(jc, s + D);                                     // set J is free: weights converted, activations staged
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // this wave's LDS writes are done
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue((J + D) % C::STAGES, s + D);
-        read_operands(std::integral_constant<int, P ^ 1>{}, std::integral_constant<int, (J + 1) % C::STAGES>{});
+        read_operands(std::integral_constant<int, P ^ 1>{});  // in flight behind the matrix instructions below
         __builtin_amdgcn_sched_barrier(0);
-        vec8 wa[NT][2];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            wa[nt][0] = dequant8<T>(wr[P][nt][0], wr[P][nt][1]);
-            wa[nt][1] = dequant8<T>(wr[P][nt][2], wr[P][nt][3]);
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)                       // dependent accumulations stay MT instructions apart
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    acc[nt][mt] = T::mfma16(wa[nt][h], bitcast<vec8>(xb[P][mt][h]), acc[nt][mt]);
-        }
-        // interleave: the conversion of the first tile, then matrix instructions with the conversion of the
-        // second tile in their shadow (3 vector instructions per matrix instruction), then the rest
-        if constexpr (NT == 2) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 24, 0);
-#pragma unroll
-            for (int q = 0; q < 2 * MT; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, 24 / (2 * MT), 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
-        }
+            for (int mt = 0; mt < MT; ++mt) acc[mt] = T::mfma16(wa[h], bitcast<vec8>(xb[P][mt][h]), acc[mt]);
         __builtin_amdgcn_sched_barrier(0);
-        operands_arrived(std::integral_constant<int, P ^ 1>{});
     };
-    // prologue of the register pipeline: operands of the first step
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::PENDING + C::XL + NT) : "memory");
-    __builtin_amdgcn_s_barrier();
-    read_operands(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-    operands_arrived(std::integral_constant<int, 0>{});
-    static_assert(C::STAGES == 4 || C::STAGES == 6, "the loop below is unrolled for an even ring of 4 or 6 stages");
-    for (int s = s_begin; s < s_end; s += C::STAGES) {
-        step(std::integral_constant<int, 0>{}, s);
-        if (s + 1 < s_end) step(std::integral_constant<int, 1>{}, s + 1);
-        if (s + 2 < s_end) step(std::integral_constant<int, 2>{}, s + 2);
-        if (s + 3 < s_end) step(std::integral_constant<int, 3>{}, s + 3);
-        if constexpr (C::STAGES == 6) {
-            if (s + 4 < s_end) step(std::integral_constant<int, 4>{}, s + 4);
-            if (s + 5 < s_end) step(std::integral_constant<int, 5>{}, s + 5);
-        }
-    }
-    // loads issued for steps past the end still target the staging ring
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    static_assert(D % 2 == 0 && D >= 4, "the two LDS stages alternate with the register sets");
+    int s = s_begin;
+    for (; s + D <= s_end; s += D) static_for<D>([&](auto jc) { step(jc, s + decltype(jc)::value); });
+    static_for<D - 1>([&](auto jc) {
+        if (s + decltype(jc)::value < s_end) step(jc, s + decltype(jc)::value);
+    });
 
     // epilogue straight from the accumulator layout: lane (r, g) holds rows m = 16*mt + r, channels 4g .. 4g+3
+    const int n = n0 + 4 * g;
+    if (n >= N) return;
+    const bool vec = n + 3 < N && (N & 3) == 0;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int n = n0 + 16 * nt + 4 * g;
-        if (n >= N) continue;
-        const bool vec = n + 3 < N && (N & 3) == 0;
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + 16 * mt + r;
+        if (m >= M) continue;
         if (partial) {
+            float* p = partial + ((int64_t)split * M + m) * N + n;
+            if (vec) {
+                *(f32x4*)p = acc[mt];
+            } else {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = m0 + 16 * mt + r;
-                if (m >= M) continue;
-                float* p = partial + ((int64_t)split * M + m) * N + n;
-                if (vec) {
-                    *(f32x4*)p = acc[nt][mt];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        if (n + i < N) p[i] = acc[nt][mt][i];
-                }
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) p[i] = acc[mt][i];
             }
+        } else if (gated) {
+            store_gated<T>(y, bias, scale, m, n, N, acc[mt]);
         } else {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = m0 + 16 * mt + r;
-                if (m >= M) continue;
-                if (gated) store_gated<T>(y, bias, scale, m, n, N, acc[nt][mt]);
-                else store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, acc[nt][mt]);
-            }
+            store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, acc[mt]);
         }
     }
 }
@@ -835,6 +775,7 @@ struct RopeCacheArgs {
 };
 
 struct GemmPlan {
+    int waves;       // waves (16-channel tiles) per workgroup
     int mt;          // activation tiles per pass (1, 2, 4)
     int m_blocks;
     int n_blocks;
@@ -846,12 +787,19 @@ GemmPlan plan_w8a16(int m, int n, int k) {
     GemmPlan p;
     p.mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
     p.m_blocks = (m + 16 * p.mt - 1) / (16 * p.mt);
-    p.n_blocks = (n + G2_BN - 1) / G2_BN;
+    // 33+ rows: 8 waves x 16 channels share one staged activation tile (half the activation bytes per weight byte of
+    // the 4-wave shape), one workgroup per CU
+    p.waves = p.mt == 4 ? 8 : 4;
+    const int bn = 16 * p.waves;
+    p.n_blocks = (n + bn - 1) / bn;
     const int total_steps = (k + GW_KSTEP - 1) / GW_KSTEP;
-    // aim at two resident workgroups on each of the 256 CUs; keep at least 12 k-steps per workgroup
-    int sk = 512 / (p.n_blocks * p.m_blocks);
+    // 4 waves: aim at two resident workgroups on each of the 256 CUs, at least 12 k-steps per workgroup; 8 waves: one
+    // workgroup per CU, at least 8 steps
+    const int target = p.waves == 8 ? 256 : 512;
+    const int min_steps = p.waves == 8 ? 8 : 12;
+    int sk = target / (p.n_blocks * p.m_blocks);
     sk = sk < 1 ? 1 : sk;
-    const int max_sk = total_steps / 12 < 1 ? 1 : total_steps / 12;
+    const int max_sk = total_steps / min_steps < 1 ? 1 : total_steps / min_steps;
     sk = sk > max_sk ? max_sk : sk;
     sk = sk > 16 ? 16 : sk;
     if (sk > 8) sk = 8 * (sk / 8);                             // multiples of 8 can run split-major
@@ -869,29 +817,16 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     const int split_major = p.split_k % 8 == 0;
     dim3 grid(split_major ? p.split_k : p.n_blocks, split_major ? p.n_blocks : p.split_k, p.m_blocks);
-    dim3 block(G2_WAVES * 64);
-#define GW_LAUNCH(MTV, KT)                                                                                       \
-    do {                                                                                                         \
-        auto kern = w8a16_gemm2_kernel<T, MTV, G2_NT, KT>;                                                        \
-        constexpr int lds = G2<MTV, G2_NT>::LDS_BYTES;                                                            \
-        static bool configured[MF_MAX_DEVICES] = {};                                                              \
-        int dev = 0;                                                                                             \
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MF_MAX_DEVICES)                                \
-            return (int)hipErrorInvalidDevice;                                                                   \
-        if (!configured[dev]) {                                                                                  \
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
-            if (e != hipSuccess) return (int)e;                                                                  \
-            configured[dev] = true;                                                                              \
-        }                                                                                                        \
-        hipLaunchKernelGGL(kern, grid, block, lds, st, (uint16_t*)y, partial, (const uint16_t*)x, wp, scale,      \
-                           (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, p.steps_per_split,     \
-                           gated, split_major);                                                                  \
-    } while (0)
     const bool ktail = (k % GW_KSTEP) != 0;
-    if (p.mt == 1) { if (ktail) GW_LAUNCH(1, true); else GW_LAUNCH(1, false); }
-    else if (p.mt == 2) { if (ktail) GW_LAUNCH(2, true); else GW_LAUNCH(2, false); }
-    else { if (ktail) GW_LAUNCH(4, true); else GW_LAUNCH(4, false); }
-#undef GW_LAUNCH
+#define GW4_LAUNCH(MTV, WV, KT)                                                                                  \
+    hipLaunchKernelGGL((w8a16_gemm4_kernel<T, MTV, WV, KT>), grid, dim3(WV * 64), 0, st, (uint16_t*)y, partial,  \
+                       (const uint16_t*)x, wp, scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, \
+                       p.steps_per_split, gated, split_major)
+    if (p.mt == 1) { if (ktail) GW4_LAUNCH(1, 4, true); else GW4_LAUNCH(1, 4, false); }
+    else if (p.mt == 2) { if (ktail) GW4_LAUNCH(2, 4, true); else GW4_LAUNCH(2, 4, false); }
+    else if (p.waves == 8) { if (ktail) GW4_LAUNCH(4, 8, true); else GW4_LAUNCH(4, 8, false); }
+    else { if (ktail) GW4_LAUNCH(4, 4, true); else GW4_LAUNCH(4, 4, false); }
+#undef GW4_LAUNCH
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (rc_args && partial) {                                 // reduce + RoPE + cache scatter in one kernel
