@@ -502,8 +502,11 @@ def bench_prefill_attention(args, torch, ops):
     """Causal attention of a Llama-3-8B-shaped prefill step over the paged cache (32 q / 8 kv heads x 128, bf16,
     block 128): `llama3_8b_prefill_attention` = 4 prompts of 2048 tokens, `llama3_8b_chunked_prefill_attention` =
     4 sequences adding 512 tokens behind 3584 cached ones.  A step is one attention call; flops = 4 * D * heads *
-    (query, key) pairs inside the causal limit."""
-    nh, nkv, d, bs, dt = 32, 8, 128, 128, torch.bfloat16
+    (query, key) pairs inside the causal limit.  `deepseek_v3_mla_prefill_attention` = the prefill of multi-latent
+    attention (multi_latent_attention.py:405-432): 4 prompts of 2048 tokens, 128 heads, queries, keys and values 192
+    wide, taken from the step's own packed rows (no cache)."""
+    mla = args.workload == "deepseek_v3_mla_prefill_attention"
+    nh, nkv, d, bs, dt = (128, 128, 192, 128, torch.bfloat16) if mla else (32, 8, 128, 128, torch.bfloat16)
     chunked = args.workload == "llama3_8b_chunked_prefill_attention"
     lens = np.full(4, 4096 if chunked else 2048)
     q_lens = np.full(4, 512 if chunked else 2048)
@@ -516,9 +519,13 @@ def bench_prefill_attention(args, torch, ops):
         pos += n
     gen = torch.Generator(device="cuda")
     gen.manual_seed(3)
-    kc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
-    vc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
     t = int(q_lens.sum())
+    if mla:
+        kc = torch.randn(t, nkv * d, generator=gen, device="cuda").to(dt)
+        vc = torch.randn(t, nkv * d, generator=gen, device="cuda").to(dt)
+    else:
+        kc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
+        vc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
     q = torch.randn(t, nh * d, generator=gen, device="cuda").to(dt)
     starts = torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device="cuda")
     lens_t = torch.tensor(lens, dtype=torch.int32, device="cuda")
@@ -526,6 +533,8 @@ def bench_prefill_attention(args, torch, ops):
     out = torch.empty_like(q)
 
     def step():
+        if mla:
+            return ops.causal_attention_varlen(q, kc, vc, starts, nh, nkv, d ** -0.5, out=out)
         return ops.paged_attention_prefill(q, kc, vc, tb, lens_t, starts, nh, nkv, d ** -0.5, out=out)
     for _ in range(args.warmup):
         step()
@@ -541,12 +550,15 @@ def bench_prefill_attention(args, torch, ops):
     ach = flops / (us * 1e-6) / 1e12
     peak = 2500.0
     result = {
-        "metric": "prefill attention query tokens/sec per layer (Llama3-8B heads, bf16); % of dense bf16 MFMA peak",
+        "metric": f"prefill attention query tokens/sec per layer ({'DeepSeek-V3 MLA' if mla else 'Llama3-8B'} heads, bf16); "
+                  "% of dense bf16 MFMA peak",
         "value": round(t / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: causal attention over the paged cache, {len(lens)} sequences, "
-                               f"{int(q_lens[0])} new tokens each, context {int(lens[0])}, 32q/8kv heads x 128, block 128",
+        "config": {"workload": f"{args.workload}: causal attention over "
+                               f"{'the packed rows of the step' if mla else 'the paged cache'}, {len(lens)} sequences, "
+                               f"{int(q_lens[0])} new tokens each, context {int(lens[0])}, {nh}q/{nkv}kv heads x {d}"
+                               f"{'' if mla else ', block 128'}",
                    "launch": "eager", "flops_per_step": flops},
         "roofline": dict(bound="mfma", kernel="prefill_attention_kernel (+ partition reduce when partitioned)",
                          achieved=round(ach, 1), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4), traffic=None,
@@ -654,7 +666,8 @@ def main():
     if args.workload == "deepseek_v3_mla_decode":
         bench_mla_decode(args, torch, ops)
         return
-    if args.workload in ("llama3_8b_prefill_attention", "llama3_8b_chunked_prefill_attention"):
+    if args.workload in ("llama3_8b_prefill_attention", "llama3_8b_chunked_prefill_attention",
+                         "deepseek_v3_mla_prefill_attention"):
         bench_prefill_attention(args, torch, ops)
         return
 

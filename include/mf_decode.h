@@ -183,7 +183,10 @@ size_t mf_paged_attention_prefill_workspace_bytes(int batch, int total_q, int n_
  * query: total_q rows of n_heads * head_dim, q_row_stride elements apart (0 = dense); out: dense
  * [total_q, n_heads * head_dim].  q_starts: int32 [batch + 1], non-decreasing.  Rows of no sequence, and
  * rows beyond a sequence's context, are written as zeros.  scale must be positive.  Numerics as
- * mf_paged_attention_decode. */
+ * mf_paged_attention_decode.  head_dim in {32, 64, 128, 192}: 192 is the prefill of multi-latent attention, whose
+ * queries, keys and values all arrive 192 wide with n_kv_heads = n_heads
+ * (mindformers/parallel_core/inference/transformer/multi_latent_attention.py:405-432; the caller keeps the first
+ * v_head_dim columns of every head, :216-218). */
 int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache, const void* value_cache,
                                const int32_t* block_tables, const int32_t* context_lens,
                                const int32_t* q_starts, int batch, int total_q, int n_heads, int n_kv_heads,

@@ -513,16 +513,41 @@ constexpr int PF_COLS = 128;                                  // columns per wor
 constexpr int PF_TOK = 32;                                    // tokens per staged tile
 constexpr int PF_RING = 3;                                    // staged tiles
 
+// A staged K or V tile is one sub-tile of PF_TOK rows of W elements, W a power of two, or, for 192-wide heads (the
+// prefill of multi-latent attention: 128 + 64 rope dimensions), a 128-wide sub-tile followed by a 64-wide one: the
+// chunk permutations below need a power-of-two number of chunks per row, and the address each lane supplies to a
+// direct load is free, so the columns of a row can be split over two regions of the buffer.
+template <int W>
+struct PfSub {
+    static constexpr int ROWB = W * 2;                        // bytes per staged row
+    static constexpr int CPR = ROWB / 16;                     // 16-byte chunks per row
+    static constexpr int RPB = 16 / CPR;                      // rows per 256 bytes of LDS
+    static constexpr int RPI = 64 / CPR;                      // rows one wave-wide load covers
+    static constexpr int LOADS = PF_TOK / RPI;                // wave-wide loads per tile per tensor
+    static constexpr int LW = LOADS < PA_WAVES ? LOADS : PA_WAVES;   // waves that load
+    static constexpr int NI = LOADS / LW;                     // loads per loading wave per tile per tensor
+};
+template <>
+struct PfSub<0> {
+    static constexpr int ROWB = 0, CPR = 1, RPB = 1, RPI = 1, LOADS = 0, LW = PA_WAVES, NI = 0;
+};
+
 template <int D>
 struct PfSmem {
-    static constexpr int ROWB = D * 2;                        // bytes per staged row
-    static constexpr int KBYTES = PF_TOK * ROWB;
+    static constexpr int W0 = D == 192 ? 128 : D;             // widths of the two sub-tiles (the second may be empty)
+    static constexpr int W1 = D - W0;
+    using Sub0 = PfSub<W0>;
+    using Sub1 = PfSub<W1>;
+    static constexpr int NI = Sub0::NI + Sub1::NI;            // loads per loading wave per tile per tensor
+    static constexpr int KBYTES = PF_TOK * D * 2;
+    static constexpr int SUB1 = PF_TOK * W0 * 2;              // byte offset of the second sub-tile within a tile
     static constexpr int BUF = 2 * KBYTES;                    // K tile, then V tile
     static constexpr int BYTES = PF_RING * BUF;
 };
 
+// Three workgroups per compute unit; two at 192-wide heads (72 KB of LDS and 96 accumulator registers each).
 template <typename T, int D, bool TIB>
-__global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
+__global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
@@ -533,13 +558,11 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
     constexpr int KS = D / 16;                                // k-steps of the score product
     constexpr int DB = D / 32;                                // 32-row blocks of O^T
     constexpr int NV = 2 * DB;                                // PV MFMAs per tile
-    constexpr int ROWB = S::ROWB;
-    constexpr int CPR = ROWB / 16;                            // 16-byte chunks per row
-    constexpr int RPB = 16 / CPR;                             // rows per 256 bytes of LDS
-    constexpr int RPI = 64 / CPR;                             // rows one wave-wide load covers
-    constexpr int LOADS = PF_TOK / RPI;                       // wave-wide loads per tile per tensor
-    constexpr int LW = LOADS < PA_WAVES ? LOADS : PA_WAVES;   // waves that load
-    constexpr int NI = LOADS / LW;                            // loads per loading wave per tile per tensor
+    using S0 = typename S::Sub0;
+    using S1 = typename S::Sub1;
+    constexpr int NI = S::NI;
+    constexpr int KS0 = S::W0 / 16;                           // k-steps served by the first sub-tile
+    constexpr int DB0 = S::W0 / 32;                           // 32-row blocks of O^T served by the first sub-tile
 
     extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];
 
@@ -641,27 +664,32 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
     const int64_t row_bytes = kv_stride * 2;
 
-    // ---- tile loads: load i of wave w brings rows (LW i + w) RPI .. + RPI - 1; lane = (row in the group, LDS slot)
-    const int lrow = lane / CPR;
-    const int lslot = lane - lrow * CPR;
+    // ---- tile loads: load i of wave w into a sub-tile brings its rows (LW i + w) RPI .. + RPI - 1; lane = (row in
+    // the group, LDS slot).  The loads of the first sub-tile come first in the arrays.
     uint32_t kcol[NI], vcol[NI];                              // byte offset of this lane's chunk within a token row
     uint32_t kofs[NI], vofs[NI];
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int row = (LW * i + w) * RPI + lrow;
-        const int key = (row / RPB) & (CPR - 1);
-        const int key4 = (row / RPB) & (CPR / 4 - 1);
-        kcol[i] = (uint32_t)(kvh * D * 2 + 16 * (lslot ^ key));
-        vcol[i] = (uint32_t)(kvh * D * 2 + 16 * ((lslot - 4 * key4) & (CPR - 1)));
+    static_for<NI>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        constexpr bool second = i >= S0::NI;
+        using SS = std::conditional_t<second, S1, S0>;
+        constexpr int li = i - (second ? S0::NI : 0);
+        constexpr int col0 = second ? S::W0 * 2 : 0;          // first byte of the sub-tile's columns within a head
+        const int lrow = lane / SS::CPR;
+        const int lslot = lane - lrow * SS::CPR;
+        const int row = (SS::LW * li + w) * SS::RPI + lrow;
+        const int key = (row / SS::RPB) & (SS::CPR - 1);
+        const int key4 = (row / SS::RPB) & (SS::CPR / 4 - 1);
+        kcol[i] = (uint32_t)(kvh * D * 2 + col0 + 16 * (lslot ^ key));
+        vcol[i] = (uint32_t)(kvh * D * 2 + col0 + 16 * ((lslot - 4 * key4) & (SS::CPR - 1)));
         kofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + kcol[i];      // offsets within a whole tile
         vofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + vcol[i];
-    }
+    });
     const int part_end = min(Lwg, part_start + part_tokens);
     const int ntiles = (part_end - part_start + PF_TOK - 1) / PF_TOK;
 
     // rows past the group's range re-read its last row (their scores are masked)
     auto issue_tile = [&](int t) {
-        if (LW < PA_WAVES && w >= LW) return;
+        if (S0::LW < PA_WAVES && w >= S0::LW) return;         // narrow heads: a tile is fewer loads than waves
         const int ts = part_start + t * PF_TOK;
         uint8_t* kdst = pf_smem + (t % PF_RING) * S::BUF;
         int64_t slot0 = 0;
@@ -679,21 +707,27 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
         if (TIB && last_row >= PF_TOK - 1) {                  // whole tile inside one block: constant lane offsets
             const uint8_t* kb = (const uint8_t*)kc + slot0 * row_bytes;
             const uint8_t* vb = (const uint8_t*)vc + slot0 * row_bytes;
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int r0 = (LW * i + w) * RPI;
+            static_for<NI>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr bool second = i >= S0::NI;
+                using SS = std::conditional_t<second, S1, S0>;
+                constexpr int li = i - (second ? S0::NI : 0);
+                uint8_t* dst = kdst + (second ? S::SUB1 : 0) + (SS::LW * li + w) * SS::RPI * SS::ROWB;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb + kofs[i]),
-                                                 (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(vb + vofs[i]),
-                    (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB), 16, 0, 0);
-            }
+                                                 (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + vofs[i]),
+                                                 (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
+            });
             return;
         }
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int r0 = (LW * i + w) * RPI;
-            const int rc = min(r0 + lrow, last_row);
+        static_for<NI>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            constexpr bool second = i >= S0::NI;
+            using SS = std::conditional_t<second, S1, S0>;
+            constexpr int li = i - (second ? S0::NI : 0);
+            const int r0 = (SS::LW * li + w) * SS::RPI;
+            uint8_t* dst = kdst + (second ? S::SUB1 : 0) + r0 * SS::ROWB;
+            const int rc = min(r0 + lane / SS::CPR, last_row);
             const uint8_t *kp, *vp;
             if constexpr (TIB) {                              // uniform base, 32-bit lane offset
                 const uint32_t lo = (uint32_t)(rc * (int)row_bytes);
@@ -709,27 +743,36 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
                 vp = (const uint8_t*)vc + off + vcol[i];
             }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
-                                             (__attribute__((address_space(3))) void*)(kdst + r0 * ROWB), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
-                                             (__attribute__((address_space(3))) void*)(kdst + S::KBYTES + r0 * ROWB),
-                                             16, 0, 0);
-        }
+                                             (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
+        });
     };
 
     // ---- operand read addresses within a ring buffer (the buffer is a compile-time offset of the read)
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)pf_smem;
-    const uint32_t kx = (uint32_t)((16 * h) ^ (16 * ((rho / RPB) & (CPR - 1))));   // chunk 2 j + h, permuted
-    uint32_t klane[KS];                                       // K: row rho, chunk of k-step j
-#pragma unroll
-    for (int j = 0; j < KS; ++j) klane[j] = lds0 + rho * ROWB + ((32u * j) ^ kx);
+    uint32_t klane[KS];                                       // K: row rho, chunk 2 j + h of k-step j, permuted
+    static_for<KS>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        constexpr bool second = j >= KS0;
+        using SS = std::conditional_t<second, S1, S0>;
+        constexpr int lj = j - (second ? KS0 : 0);
+        const uint32_t kx = (uint32_t)((16 * h) ^ (16 * ((rho / SS::RPB) & (SS::CPR - 1))));
+        klane[j] = lds0 + (second ? S::SUB1 : 0) + rho * SS::ROWB + ((32u * lj) ^ kx);
+    });
     const int jj = rho & 15;
     const int tq = jj >> 2;                                   // token of the quad this lane names
-    const int vkey4 = ((4 * h + tq) / RPB) & (CPR / 4 - 1);
-    const int vchunk = (rho & 16) / 8 + ((jj & 3) >> 1) + 4 * vkey4;   // + 4 db, mod CPR
-    const uint32_t vrow = lds0 + S::KBYTES + (4 * h + tq) * ROWB + (jj & 1) * 8;
     uint32_t vlane[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) vlane[db] = vrow + 16 * ((vchunk + 4 * db) & (CPR - 1));
+    static_for<DB>([&](auto dc) {
+        constexpr int db = decltype(dc)::value;
+        constexpr bool second = db >= DB0;
+        using SS = std::conditional_t<second, S1, S0>;
+        constexpr int ldb = db - (second ? DB0 : 0);
+        const int vkey4 = ((4 * h + tq) / SS::RPB) & (SS::CPR / 4 - 1);
+        const int vchunk = (rho & 16) / 8 + ((jj & 3) >> 1) + 4 * vkey4;
+        const uint32_t vrow = lds0 + S::KBYTES + (second ? S::SUB1 : 0) + (4 * h + tq) * SS::ROWB + (jj & 1) * 8;
+        vlane[db] = vrow + 16 * ((vchunk + 4 * ldb) & (SS::CPR - 1));
+    });
 
     // a column can find a whole tile masked before it has seen any token; starting the running maximum above the
     // mask value makes those probabilities 2^(-huge) = 0 instead of 2^0.  Maxima are kept in raw score units: the
@@ -815,6 +858,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, 3) void prefill_attention_kernel(
                 constexpr int v = decltype(vc_)::value;
                 if constexpr (v < NV) {
                     constexpr int th = v / DB, db = v % DB;
+                    constexpr int ROWB = db >= DB0 ? S1::ROWB : S0::ROWB;
                     lo[v % P] = lds_read_tr16_at<OFF + 16 * th * ROWB>(vlane[db]);
                     hi[v % P] = lds_read_tr16_at<OFF + (16 * th + 8) * ROWB>(vlane[db]);
                 }
@@ -1289,8 +1333,8 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
     MF_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "paged_attention_prefill: n_heads (%d) must be a positive multiple of n_kv_heads (%d)", n_heads,
                n_kv_heads);
-    MF_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 128,
-               "paged_attention_prefill: head_dim %d not supported (32, 64, 128)", head_dim);
+    MF_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 128 || (head_dim == 192 && !kv8),
+               "paged_attention_prefill: head_dim %d not supported (32, 64, 128; 192 with a 16-bit cache)", head_dim);
     MF_REQUIRE(contiguous || (block_size > 0 && max_blocks_per_seq > 0 && num_blocks > 0),
                "paged_attention_prefill: bad block geometry");
     MF_REQUIRE(contiguous || (int64_t)block_size * max_blocks_per_seq <= 0x7fffffffLL,
@@ -1321,15 +1365,22 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
                                           batch, total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq,     \
                                           num_blocks, scale, q_row_stride, kv_row_stride, workspace, st, nullptr,  \
                                           nullptr)
+#define PF_CASE192(TT)                                                                                             \
+    return launch_pf<TT, 192, false>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, \
+                                     total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
+                                     q_row_stride, kv_row_stride, workspace, st, nullptr, nullptr)
     if (dtype == MF_BF16) {
         if (head_dim == 32) PF_CASE(BF16, 32);
         if (head_dim == 64) PF_CASE(BF16, 64);
+        if (head_dim == 192) PF_CASE192(BF16);
         PF_CASE(BF16, 128);
     } else {
         if (head_dim == 32) PF_CASE(FP16, 32);
         if (head_dim == 64) PF_CASE(FP16, 64);
+        if (head_dim == 192) PF_CASE192(FP16);
         PF_CASE(FP16, 128);
     }
+#undef PF_CASE192
 #undef PF_CASE
 }
 

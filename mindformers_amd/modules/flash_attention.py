@@ -69,8 +69,14 @@ class FlashAttention(nn.Module):
                                                           q2.shape[0])
             k2 = key if key.dim() == 2 else key.reshape(q2.shape[0], -1)
             v2 = value if value.dim() == 2 else value.reshape(q2.shape[0], -1)
-            out = ops.causal_attention_varlen(q2, k2, v2, starts, self.head_num,
-                                              self.pa_kv_head_num, self.scale_value)
+            # the kv head count of this step's keys: kv_head_num, which for multi-latent attention differs from the
+            # cache's (pa_kv_head_num = 1): its prefill attends over the up-projected 192-wide keys of every head
+            # (multi_latent_attention.py:405-432)
+            d = q2.shape[1] // self.head_num
+            if q2.shape[1] != self.head_num * d or k2.shape[1] % d or v2.shape[1] != k2.shape[1]:
+                raise ValueError(f"query / key / value widths {q2.shape[1]} / {k2.shape[1]} / {v2.shape[1]} do not "
+                                 f"fit {self.head_num} heads")
+            out = ops.causal_attention_varlen(q2, k2, v2, starts, self.head_num, k2.shape[1] // d, self.scale_value)
             return out.reshape(shape)
         if self.use_multi_latent_attention:                   # one latent cache, keys = values (flash_attention.py:136-139)
             out = ops.mla_paged_attention(q2, key_cache, block_tables, batch_valid_length, self.head_num,

@@ -296,6 +296,8 @@ def _prefill_case(rng, dtype, nh, nkv, d, bs, lens, q_lens, max_blocks=None, pad
     (torch.float16, 4, 4, 64, 32, [300], [300]),                            # MHA: 128 queries per workgroup
     (torch.float16, 16, 4, 128, 64, [1500, 33], [1500, 20]),                # many tiles per workgroup, fp16
     (torch.bfloat16, 8, 8, 128, 16, [200], [130]),                          # MHA behind a context, small blocks
+    (torch.bfloat16, 4, 4, 192, 32, [200, 77], [130, 77]),                  # 192-wide heads through the cache
+    (torch.float16, 4, 2, 192, 16, [90, 300], [90, 5]),                     # and with tiles that straddle blocks
 ])
 def test_paged_prefill_vs_oracle(dtype, nh, nkv, d, bs, lens, q_lens):
     rng = np.random.default_rng(nh * 100 + len(lens))
@@ -383,6 +385,9 @@ def test_chunked_prefill_matches_whole_prefill():
     (torch.bfloat16, 32, 8, 128, [130, 1, 64], True),
     (torch.float16, 8, 2, 64, [33, 200], False),
     (torch.bfloat16, 4, 4, 32, [17], False),
+    (torch.bfloat16, 16, 16, 192, [130, 1, 64], False),         # 192-wide heads: the prefill of multi-latent attention
+    (torch.float16, 8, 2, 192, [33, 200], True),                # the same width with grouped heads, strided rows
+    (torch.bfloat16, 2, 2, 192, [1500], False),                 # few columns: the context is cut into partitions
 ])
 def test_causal_attention_varlen_vs_oracle(dtype, nh, nkv, d, q_lens, fused):
     """Keys and values taken from this step's own packed rows (no cache), optionally as column slices of one fused

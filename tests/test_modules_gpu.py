@@ -734,6 +734,38 @@ def test_mcore_flash_attention_mla_decode_branch():
     assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA decode")
 
 
+def test_mcore_flash_attention_mla_prefill_branch():
+    """FlashAttention(pa_mla_v_dim=512) in prefill: MLASelfAttention hands over 192-wide queries, keys (the
+    up-projected 128 dimensions of every head followed by the shared rotary 64) and values (128 dimensions padded
+    with the same rotary 64), and keeps the first v_head_dim columns of every head of the result
+    (multi_latent_attention.py:405-432, 208-218).  The latent cache is the caller's to write and is not touched."""
+    from mindformers_amd.modules import FlashAttention
+    rng = np.random.default_rng(31)
+    nh, qk, rope, vd = 16, 128, 64, 128
+    q_lens = np.array([150, 1, 37, 260])
+    t = int(q_lens.sum())
+    scale = 1.0 / np.sqrt(qk + rope)
+    net = FlashAttention(head_num=nh, head_dim=qk + rope, kv_head_num=nh, scale_value=scale, next_tokens=0,
+                         pa_kv_head_num=1, pa_mla_v_dim=512)
+    assert net.is_prefill and net.use_multi_latent_attention
+    q = rounded(rng.normal(size=(t, nh, qk + rope)), BF)
+    k_pe = np.repeat(rounded(rng.normal(size=(t, 1, rope)), BF), nh, axis=1)
+    k = np.concatenate([rounded(rng.normal(size=(t, nh, qk)), BF), k_pe], axis=-1)
+    v = np.concatenate([rounded(rng.normal(size=(t, nh, vd)), BF), k_pe], axis=-1)
+    cache = torch.full((4, 32, 1, 576), 7.0, dtype=BF, device="cuda")
+    ends = torch.from_numpy(np.cumsum(q_lens).astype(np.int32)).cuda()
+    out = net(query=dev(q.reshape(t, -1), BF), key=dev(k.reshape(t, -1), BF), value=dev(v.reshape(t, -1), BF),
+              slot_mapping=None, actual_seq_qlen=ends, actual_seq_kvlen=ends, key_cache=cache, value_cache=None)
+    assert out.shape == (t, nh * (qk + rope))
+    assert bool((cache == 7.0).all())
+    ref = O.causal_prefill_attention(q.reshape(t, -1), k.reshape(t, -1), v.reshape(t, -1), q_lens, nh, nh, scale)
+    mag = O.causal_prefill_attention(q.reshape(t, -1), k.reshape(t, -1), np.abs(v.reshape(t, -1)), q_lens, nh, nh, scale)
+    assert_within(to_np(out), ref, mag, BF, ulps=1.5, what="FlashAttention MLA prefill")
+    kept = to_np(out).reshape(t, nh, qk + rope)[:, :, :vd]        # what MLASelfAttention passes to linear_proj
+    assert_within(kept, ref.reshape(t, nh, -1)[:, :, :vd], mag.reshape(t, nh, -1)[:, :, :vd], BF, ulps=1.5,
+                  what="MLA prefill, v_head_dim columns")
+
+
 def test_mcore_flash_attention_mla_decode_with_q_seq_lens():
     """MLA decode with several new tokens per sequence (q_seq_lens: parallel decoding / chunked prefill,
     flash_attention.py:140-143): every query row sees the latent cache up to its own position; a sequence without new
