@@ -66,12 +66,13 @@ __host__ __device__ inline int mla_free_slots(int batch, int head_blocks, int n_
 // Tokens per partition, chosen from the actual lengths so that the workgroups fit the chip's n_slots compute units in
 // one round (one workgroup is resident per unit): sum_b ceil(L_b / pt) * head_blocks <= total * head_blocks / pt +
 // batch * head_blocks, which is <= n_slots for pt >= total * head_blocks / (n_slots - batch * head_blocks).  Every
-// wave that calls this gets the same value (the main kernel and the reduce kernel both do).
+// wave that calls this gets the same value (the main kernel and the reduce kernel both do).  first: this lane's
+// entry of the first 64 lengths (0 beyond the batch), which the caller has loaded already.
 __device__ inline int mla_part_tokens(const int32_t* __restrict__ ctx_lens, int batch, int max_ctx, int head_blocks,
-                                      int n_slots) {
+                                      int n_slots, int first) {
     const int ln = threadIdx.x & 63;
-    int64_t total = 0;
-    for (int c0 = 0; c0 < batch; c0 += 64) {
+    int64_t total = first < 0 ? 0 : (first > max_ctx ? max_ctx : first);
+    for (int c0 = 64; c0 < batch; c0 += 64) {
         const int bb = c0 + ln;
         const int len = bb < batch ? ctx_lens[bb] : 0;
         total += len < 0 ? 0 : (len > max_ctx ? max_ctx : len);
@@ -93,9 +94,13 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     int num_blocks, int max_parts, int n_slots, float scale_log2, int64_t q_stride, int batch) {
     using vec8 = typename T::vec8;
     extern __shared__ __attribute__((aligned(16))) uint8_t mla_smem[];
-    const int part_tokens =
+    // the first 64 lengths serve the partition rule and the work list: one trip to memory for both
+    const int len_first = (int)(threadIdx.x & 63) < batch ? ctx_lens[threadIdx.x & 63] : 0;
+    // (made a scalar explicitly: the value comes out of a cross-lane reduction, and everything derived from it,
+    // the tile addresses and the branches on tile positions above all, would otherwise be computed per lane)
+    const int part_tokens = __builtin_amdgcn_readfirstlane(
         max_parts == 1 ? max_blocks * block_size
-                       : mla_part_tokens(ctx_lens, batch, max_blocks * block_size, head_blocks, n_slots);
+                       : mla_part_tokens(ctx_lens, batch, max_blocks * block_size, head_blocks, n_slots, len_first));
 
     // ---- work list: (sequence, partition, head block) triples that exist, from a prefix sum over the lengths
     int b = -1, part = 0, hb = 0, L = 0, nparts = 1;
@@ -105,7 +110,7 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         int base = 0;
         for (int c0 = 0; c0 < batch; c0 += 64) {
             const int bb = c0 + ln;
-            const int len = bb < batch ? min(ctx_lens[bb], max_blocks * block_size) : 0;
+            const int len = min(c0 == 0 ? len_first : (bb < batch ? ctx_lens[bb] : 0), max_blocks * block_size);
             int np = len > 0 ? (len + part_tokens - 1) / part_tokens : 0;
             np = np < max_parts ? np : max_parts;
             const int per_seq = np * head_blocks;
@@ -170,23 +175,55 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         const int pos = slot - row * MLA_CPR;
         lofs[i] = (uint32_t)(row * M2_ROWB + 16 * ((pos & ~7) | ((pos & 7) ^ m2_key(row))));   // its logical chunk
     }
-    auto issue_tile = [&](int t) {                            // a tile lies inside one block (host-checked)
+    // A tile lies inside one block (host-checked).  The table entry of the block being read stays in a scalar
+    // register and the next block's entry is fetched when the current one is entered, so that the lookup of a tile's
+    // block (a scalar load and its wait) is not on the path of every tile.
+    auto lookup = [&](int bi) {
+        int blk = bi < max_blocks ? table[bi] : 0;
+        return (blk < 0 || blk >= num_blocks) ? 0 : blk;      // never leave the cache allocation
+    };
+    int bi_cur = part_start / block_size;
+    int blk_cur = lookup(bi_cur), blk_nxt = lookup(bi_cur + 1);
+    // Where tile t comes from and goes to (tiles are asked for in order).
+    struct TileAddr {
+        const uint8_t* base;                                  // first row of the tile in the cache
+        uint8_t* dst;                                         // its ring buffer
+        int last_row;                                         // rows past the context re-read the last valid row
+    };
+    auto tile_addr = [&](int t) {
         const int ts = part_start + t * MLA_TILE;
         const int bi = ts / block_size;
-        int blk = table[bi];
-        blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;       // never leave the cache allocation
-        const uint8_t* base = (const uint8_t*)cache + ((int64_t)blk * block_size + (ts - bi * block_size)) * M2_ROWB;
-        uint8_t* dst = mla_smem + (t & (M2_RING - 1)) * M2_TILE_BYTES;
-        const int last_row = L - 1 - ts;                      // rows past the context re-read the last valid row
+        if (bi != bi_cur) {                                   // uniform: the tile enters the next block
+            bi_cur = bi;
+            blk_cur = blk_nxt;
+            blk_nxt = lookup(bi + 1);
+        }
+        TileAddr a;
+        a.base = (const uint8_t*)cache + ((int64_t)blk_cur * block_size + (ts - bi * block_size)) * M2_ROWB;
+        a.dst = mla_smem + (t & (M2_RING - 1)) * M2_TILE_BYTES;
+        a.last_row = L - 1 - ts;
+        return a;
+    };
+    // load i of a whole tile: constant lane offsets
+    auto issue_load = [&](const TileAddr& a, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.base + lofs[i]),
+                                         (__attribute__((address_space(3))) void*)(a.dst + 1024 * (M2_WAVES * i + w)),
+                                         16, 0, 0);
+    };
+    // all loads of a tile at once (the first tiles of a partition, and the last tile of a sequence, whose rows are
+    // clamped)
+    auto issue_tile = [&](const TileAddr& a) {
+        if (a.last_row >= MLA_TILE - 1) {
+            static_for<M2_LOADS>([&](auto ic) { issue_load(a, ic); });
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < M2_LOADS; ++i) {
-            uint32_t off = lofs[i];
-            if (last_row < MLA_TILE - 1) {                    // last tile of the sequence only
-                const int row = (int)(off / M2_ROWB);
-                off -= (uint32_t)(max(row - last_row, 0) * M2_ROWB);
-            }
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off),
-                                             (__attribute__((address_space(3))) void*)(dst + 1024 * (M2_WAVES * i + w)),
+            const int row = (int)(lofs[i] / M2_ROWB);
+            const uint32_t off = lofs[i] - (uint32_t)(max(row - a.last_row, 0) * M2_ROWB);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.base + off),
+                                             (__attribute__((address_space(3))) void*)(a.dst + 1024 * (M2_WAVES * i + w)),
                                              16, 0, 0);
         }
     };
@@ -230,9 +267,19 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     // One tile: scores, softmax, PV product.  With one wave per SIMD nothing is gained by interleaving the matrix and
     // vector instructions of different tiles (a wave runs its own MFMAs and vector instructions one after the other),
     // so the phases follow each other; the LDS reads run four operands ahead of the MFMAs that use them.
+    // The loads of tile t + 2 (its buffer is free: every wave has passed the barrier that ends tile t - 1) go out one
+    // at a time between the score MFMAs, each of which waits for its predecessor anyway: issued in a block they cost
+    // the wave about 60 cycles apiece.
     auto step = [&](int t, auto ring_c) {
         constexpr int R = decltype(ring_c)::value;
         constexpr int P = 4;
+        TileAddr nxt = {nullptr, nullptr, 0};
+        bool spread = false;                                  // uniform
+        if (t + 2 < ntiles) {
+            nxt = tile_addr(t + 2);
+            spread = nxt.last_row >= MLA_TILE - 1;
+            if (!spread) issue_tile(nxt);
+        }
         // ring buffers 2 and 3 lie beyond the 16-bit offset field of an LDS read: a second set of addresses
         constexpr int OFF = (R & 1) * M2_TILE_BYTES, HI = R >> 1;
         const int ts = part_start + t * MLA_TILE;
@@ -256,6 +303,10 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
                 if constexpr (m == 0) T::mfma32_first(sc, bitcast<vec8>(ka[m % P]), qreg[m]);
                 else T::mfma32_next(sc, bitcast<vec8>(ka[m % P]), qreg[m]);
                 __builtin_amdgcn_sched_barrier(0);
+                if constexpr (m % 4 == 1 && m / 4 < M2_LOADS) {
+                    if (spread) issue_load(nxt, std::integral_constant<int, m / 4>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 fetch(std::integral_constant<int, m + P>{});
             });
             // the compiler does not know that sc comes from matrix instructions: their 8 passes end here
@@ -276,14 +327,16 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         if (__builtin_amdgcn_ballot_w64(m_new != m_ref) != 0) {       // the reference point moves: rare
             const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * scale_log2);
             l_run *= alpha;
-            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      // the last PV MFMAs have written their registers
+            if (t != 0) {                                     // (the first tile always moves it, off zero accumulators)
+                asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last PV MFMAs have written their registers
 #pragma unroll
-            for (int db = 0; db < M2_DB; ++db) {
-                asm volatile("" : "+a"(acc[db]));
-                acc[db] *= alpha;
-                asm volatile("" : "+a"(acc[db]));
+                for (int db = 0; db < M2_DB; ++db) {
+                    asm volatile("" : "+a"(acc[db]));
+                    acc[db] *= alpha;
+                    asm volatile("" : "+a"(acc[db]));
+                }
+                asm volatile("s_nop 7" ::: "memory");
             }
-            asm volatile("s_nop 7" ::: "memory");
             m_ref = m_new;
         }
         const float nm = -m_ref * scale_log2;
@@ -324,19 +377,18 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         }
     };
 
-    issue_tile(0);
-    if (ntiles > 1) issue_tile(1);
+    issue_tile(tile_addr(0));
+    if (ntiles > 1) issue_tile(tile_addr(1));
 #pragma unroll
     for (int j = 0; j < M2_KS; ++j) asm volatile("" : "+v"(qreg[j]));   // the query is complete before the loop
-    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 2,
-    // whose buffer takes tile t + 2
+    // tile t has landed for every wave (tile t + 1 may still be on its way), and every wave is done with tile t - 1:
+    // the buffer of tile t - 2 may take tile t + 2 from here on
     auto sync_issue = [&](int t) {
         __builtin_amdgcn_sched_barrier(0);
         if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(M2_LOADS) : "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        if (t + 2 < ntiles) issue_tile(t + 2);
     };
     constexpr std::integral_constant<int, 0> r0{};
     constexpr std::integral_constant<int, 1> r1{};
@@ -401,19 +453,34 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         __builtin_amdgcn_wave_barrier();
         if (nparts == 1) {                                    // the only partition of its sequence: final rows
             // two heads per pass: lanes 0-31 one row, lanes 32-63 the next; 8 columns per lane
-            for (int r0 = 0; r0 < live; r0 += 2) {
-                const int r = r0 + h;
-                if (r >= live) continue;
-                const f32x4 lo = *(const f32x4*)(stage + r * OROW + rho * 32);
-                const f32x4 hi = *(const f32x4*)(stage + r * OROW + rho * 32 + 16);
-                const u32x4 o = {pack2<T>(lo[0], lo[1]), pack2<T>(lo[2], lo[3]), pack2<T>(hi[0], hi[1]),
-                                 pack2<T>(hi[2], hi[3])};
-                *(u32x4*)(out + ((int64_t)b * n_heads + head0 + r) * MLA_DV + 256 * hv + 8 * rho) = o;
+            for (int r0 = 0; r0 < live; r0 += 8) {            // 4 pairs of rows at a time
+                f32x4 lo[4], hi[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int r = min(r0 + 2 * i + h, 31);
+                    lo[i] = *(const f32x4*)(stage + r * OROW + rho * 32);
+                    hi[i] = *(const f32x4*)(stage + r * OROW + rho * 32 + 16);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int r = r0 + 2 * i + h;
+                    if (r >= live) continue;
+                    const u32x4 o = {pack2<T>(lo[i][0], lo[i][1]), pack2<T>(lo[i][2], lo[i][3]),
+                                     pack2<T>(hi[i][0], hi[i][1]), pack2<T>(hi[i][2], hi[i][3])};
+                    *(u32x4*)(out + ((int64_t)b * n_heads + head0 + r) * MLA_DV + 256 * hv + 8 * rho) = o;
+                }
             }
         } else {
-            for (int r = 0; r < live; ++r) {
-                const int64_t pi = ((int64_t)b * n_heads + head0 + r) * max_parts + part;
-                *(f32x4*)(part_out + pi * MLA_DV + 256 * hv + 4 * lane) = *(const f32x4*)(stage + r * OROW + lane * 16);
+            // 8 rows at a time: their LDS reads go out together, then their stores
+            float* dst = part_out + (((int64_t)b * n_heads + head0) * max_parts + part) * MLA_DV + 256 * hv + 4 * lane;
+            const int64_t rstride = (int64_t)max_parts * MLA_DV;
+            for (int r0 = 0; r0 < live; r0 += 8) {
+                f32x4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = *(const f32x4*)(stage + min(r0 + i, 31) * OROW + lane * 16);
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (r0 + i < live) *(f32x4*)(dst + (r0 + i) * rstride) = v[i];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -433,7 +500,9 @@ __global__ __launch_bounds__(MR_THREADS) void mla_reduce_kernel(uint16_t* __rest
                                                                 int max_parts, int batch, int head_blocks,
                                                                 int n_slots, int max_ctx) {
     const int h = blockIdx.x, b = blockIdx.y, d = 4 * threadIdx.x;
-    const int part_tokens = mla_part_tokens(ctx_lens, batch, max_ctx, head_blocks, n_slots);
+    const int ln = threadIdx.x & 63;
+    const int part_tokens = mla_part_tokens(ctx_lens, batch, max_ctx, head_blocks, n_slots,
+                                            ln < batch ? ctx_lens[ln] : 0);
     const int L = min(ctx_lens[b], max_ctx);
     const int64_t gh = (int64_t)b * n_heads + h;
     int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
