@@ -63,27 +63,65 @@ __host__ __device__ inline int mla_free_slots(int batch, int head_blocks, int n_
     const int f = n_slots - batch * head_blocks;
     return f > n_slots / 4 ? f : n_slots / 4;
 }
-// Tokens per partition, chosen from the actual lengths so that the workgroups fit the chip's n_slots compute units in
-// one round (one workgroup is resident per unit): sum_b ceil(L_b / pt) * head_blocks <= total * head_blocks / pt +
-// batch * head_blocks, which is <= n_slots for pt >= total * head_blocks / (n_slots - batch * head_blocks).  Every
-// wave that calls this gets the same value (the main kernel and the reduce kernel both do).  first: this lane's
-// entry of the first 64 lengths (0 beyond the batch), which the caller has loaded already.
-__device__ inline int mla_part_tokens(const int32_t* __restrict__ ctx_lens, int batch, int max_ctx, int head_blocks,
-                                      int n_slots, int first) {
+// Workgroups the launch provides: the partition rule never produces more.
+__host__ __device__ inline int mla_grid(int batch, int head_blocks, int n_slots) {
+    return mla_free_slots(batch, head_blocks, n_slots) + batch * head_blocks;
+}
+// The partition rule: the largest number of 32-token tiles a partition may hold, T, chosen from the actual lengths so
+// that the workgroups fit the chip's n_slots compute units in one round (one workgroup is resident per unit).
+// Sequence b with t_b tiles is cut into ceil(t_b / T) partitions of ceil(t_b / partitions) tiles each (equal up to one
+// tile).  T0 = total tiles * head_blocks / (n_slots - batch * head_blocks) always fits, because sum_b ceil(t_b / T) *
+// head_blocks <= total * head_blocks / T + batch * head_blocks; that bound charges every sequence a whole extra
+// partition, so four smaller candidates T0 - k max(1, T0 / 16) are counted exactly (one packed reduction) and the
+// smallest that fits wins: the longest workgroup, which sets the kernel's time, gets that much shorter.  Every wave
+// that calls this gets the same value (the main kernel and the reduce kernel both do).  first: this lane's entry of
+// the first 64 lengths (0 beyond the batch), which the caller has loaded already.
+__device__ inline int mla_tiles_of(int len, int max_ctx) {
+    const int l = len < 0 ? 0 : (len > max_ctx ? max_ctx : len);
+    return (l + MLA_TILE - 1) / MLA_TILE;
+}
+__device__ inline int mla_part_tiles(const int32_t* __restrict__ ctx_lens, int batch, int max_ctx, int head_blocks,
+                                     int n_slots, int first) {
     const int ln = threadIdx.x & 63;
-    int64_t total = first < 0 ? 0 : (first > max_ctx ? max_ctx : first);
+    const int t_first = mla_tiles_of(first, max_ctx);
+    int64_t total = t_first;
     for (int c0 = 64; c0 < batch; c0 += 64) {
         const int bb = c0 + ln;
-        const int len = bb < batch ? ctx_lens[bb] : 0;
-        total += len < 0 ? 0 : (len > max_ctx ? max_ctx : len);
+        total += mla_tiles_of(bb < batch ? ctx_lens[bb] : 0, max_ctx);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o, 64);
     const int64_t avail = mla_free_slots(batch, head_blocks, n_slots);
-    int64_t pt = (total * head_blocks + avail - 1) / avail;
-    pt = (pt + 31) / 32 * 32;
-    const int lo = mla_min_part(max_ctx);
-    return pt < lo ? lo : (int)pt;
+    const int lo = mla_min_part(max_ctx) / MLA_TILE;
+    const int64_t t0l = (total * head_blocks + avail - 1) / avail;
+    const int t0 = __builtin_amdgcn_readfirstlane(t0l < lo ? lo : (int)t0l);
+    const int step = t0 / 16 > 1 ? t0 / 16 : 1;
+    if (t0 - step < lo) return t0;
+    // partitions per candidate, 16 bits each (a chunk of 64 sequences adds at most 64 * 32 to a field)
+    int64_t cnt[4] = {0, 0, 0, 0};
+    for (int c0 = 0; c0 < batch; c0 += 64) {
+        const int bb = c0 + ln;
+        const int t = c0 == 0 ? t_first : mla_tiles_of(bb < batch ? ctx_lens[bb] : 0, max_ctx);
+        uint64_t packed = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int cand = t0 - (k + 1) * step;
+            const int parts = cand >= lo ? (t + cand - 1) / cand : 0;
+            packed |= (uint64_t)parts << (16 * k);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) packed += __shfl_xor(packed, o, 64);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) cnt[k] += (int64_t)((packed >> (16 * k)) & 0xffff);
+    }
+    const int64_t grid = mla_grid(batch, head_blocks, n_slots);
+    int best = t0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int cand = t0 - (k + 1) * step;
+        if (cand >= lo && cnt[k] * head_blocks <= grid) best = cand;      // counts grow with k: the last fit is the smallest
+    }
+    return __builtin_amdgcn_readfirstlane(best);
 }
 
 template <typename T>
@@ -91,16 +129,19 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ ctx_lens, int n_heads, int head_blocks, int block_size, int max_blocks,
-    int num_blocks, int max_parts, int n_slots, float scale_log2, int64_t q_stride, int batch) {
+    int num_blocks, int max_parts, int n_slots, float scale_log2, int64_t q_stride, int batch,
+    int32_t* __restrict__ plan_word) {
     using vec8 = typename T::vec8;
     extern __shared__ __attribute__((aligned(16))) uint8_t mla_smem[];
     // the first 64 lengths serve the partition rule and the work list: one trip to memory for both
     const int len_first = (int)(threadIdx.x & 63) < batch ? ctx_lens[threadIdx.x & 63] : 0;
-    // (made a scalar explicitly: the value comes out of a cross-lane reduction, and everything derived from it,
-    // the tile addresses and the branches on tile positions above all, would otherwise be computed per lane)
-    const int part_tokens = __builtin_amdgcn_readfirstlane(
-        max_parts == 1 ? max_blocks * block_size
-                       : mla_part_tokens(ctx_lens, batch, max_blocks * block_size, head_blocks, n_slots, len_first));
+    // (a scalar: it comes out of a cross-lane reduction, and everything derived from it, the tile addresses and the
+    // branches on tile positions above all, would otherwise be computed per lane)
+    const int max_ctx = max_blocks * block_size;
+    const int cap_tiles = __builtin_amdgcn_readfirstlane(
+        max_parts == 1 ? (max_ctx + MLA_TILE - 1) / MLA_TILE
+                       : mla_part_tiles(ctx_lens, batch, max_ctx, head_blocks, n_slots, len_first));
+    if (plan_word && blockIdx.x == 0 && threadIdx.x == 0) *plan_word = cap_tiles;   // for the reduce kernel
 
     // ---- work list: (sequence, partition, head block) triples that exist, from a prefix sum over the lengths
     int b = -1, part = 0, hb = 0, L = 0, nparts = 1;
@@ -110,8 +151,8 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         int base = 0;
         for (int c0 = 0; c0 < batch; c0 += 64) {
             const int bb = c0 + ln;
-            const int len = min(c0 == 0 ? len_first : (bb < batch ? ctx_lens[bb] : 0), max_blocks * block_size);
-            int np = len > 0 ? (len + part_tokens - 1) / part_tokens : 0;
+            const int len = min(c0 == 0 ? len_first : (bb < batch ? ctx_lens[bb] : 0), max_ctx);
+            int np = (mla_tiles_of(len, max_ctx) + cap_tiles - 1) / cap_tiles;
             np = np < max_parts ? np : max_parts;
             const int per_seq = np * head_blocks;
             int incl = per_seq;
@@ -161,6 +202,8 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
         }
     }
 
+    // the partitions of a sequence are equal up to one tile
+    const int part_tokens = ((L + MLA_TILE - 1) / MLA_TILE + nparts - 1) / nparts * MLA_TILE;
     const int part_start = part * part_tokens;
     const int part_end = min(L, part_start + part_tokens);
     const int ntiles = (part_end - part_start + MLA_TILE - 1) / MLA_TILE;      // >= 1 for a listed partition
@@ -487,53 +530,93 @@ __global__ __launch_bounds__(M2_WAVES * 64, 1) void mla_decode_kernel(
     }
 }
 
-// Combine the partitions of one (sequence, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p.
-// One workgroup of 128 threads (4 value columns each) per (head, sequence); the loads of up to 8 partitions are
-// issued together, so a row costs one round trip for the lengths, one for the (max, sum) pairs and one for the
-// accumulators.
+// Combine the partitions of (sequence, head) rows: out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p.
+// One workgroup of 128 threads (4 value columns each) per 4 heads of a sequence.  The partition rule's value comes
+// from the word the main kernel left behind the partials, so a row costs one round trip for that word and the
+// length and one for everything else: with up to 8 partitions the (max, sum) pairs and the accumulators of all four
+// heads are loaded together.
 constexpr int MR_THREADS = MLA_DV / 4;
+constexpr int MR_HEADS = 4;
 template <typename T>
 __global__ __launch_bounds__(MR_THREADS) void mla_reduce_kernel(uint16_t* __restrict__ out,
                                                                 const float* __restrict__ part_out,
                                                                 const float* __restrict__ part_ml,
-                                                                const int32_t* __restrict__ ctx_lens, int n_heads,
-                                                                int max_parts, int batch, int head_blocks,
-                                                                int n_slots, int max_ctx) {
-    const int h = blockIdx.x, b = blockIdx.y, d = 4 * threadIdx.x;
-    const int ln = threadIdx.x & 63;
-    const int part_tokens = mla_part_tokens(ctx_lens, batch, max_ctx, head_blocks, n_slots,
-                                            ln < batch ? ctx_lens[ln] : 0);
+                                                                const int32_t* __restrict__ ctx_lens,
+                                                                const int32_t* __restrict__ plan_word, int n_heads,
+                                                                int max_parts, int max_ctx) {
+    const int h0 = blockIdx.x * MR_HEADS, b = blockIdx.y, d = 4 * threadIdx.x;
+    const int cap_tiles = *plan_word;
     const int L = min(ctx_lens[b], max_ctx);
-    const int64_t gh = (int64_t)b * n_heads + h;
-    int np = L <= 0 ? 0 : (L + part_tokens - 1) / part_tokens;
+    int np = (mla_tiles_of(L, max_ctx) + cap_tiles - 1) / cap_tiles;
     np = np < max_parts ? np : max_parts;
-    if (np == 1) return;                                      // the main kernel wrote the final row
+    if (np == 1) return;                                      // the main kernel wrote the final rows
+    const int live = min(MR_HEADS, n_heads - h0);
+    const int64_t gh0 = (int64_t)b * n_heads + h0;
     if (np == 0) {
-        *(u32x2*)(out + gh * MLA_DV + d) = (u32x2){0u, 0u};
+        for (int hh = 0; hh < live; ++hh) *(u32x2*)(out + (gh0 + hh) * MLA_DV + d) = (u32x2){0u, 0u};
         return;
     }
-    const float* ml = part_ml + gh * max_parts * 2;
-    const float* po = part_out + gh * max_parts * MLA_DV + d;
-    float M = MLA_NEG;
-    for (int p = 0; p < np; ++p) M = fmaxf(M, ml[2 * p]);     // uniform addresses: broadcast loads
-    f32x4 num = {0.f, 0.f, 0.f, 0.f};
-    float den = 0.f;
-    for (int p0 = 0; p0 < np; p0 += 8) {
-        f32x4 v[8];
-        float f[8];
+    if (np <= 8) {
+        f32x4 v[MR_HEADS][8];
+        float m[MR_HEADS][8], l[MR_HEADS][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const bool on = p0 + i < np;
-            v[i] = on ? *(const f32x4*)(po + (int64_t)(p0 + i) * MLA_DV) : (f32x4){0.f, 0.f, 0.f, 0.f};
-            f[i] = on ? __builtin_amdgcn_exp2f(ml[2 * (p0 + i)] - M) : 0.f;
-            den += on ? f[i] * ml[2 * (p0 + i) + 1] : 0.f;
+        for (int hh = 0; hh < MR_HEADS; ++hh) {
+            const int64_t gh = gh0 + (hh < live ? hh : 0);
+            const float* ml = part_ml + gh * max_parts * 2;
+            const float* po = part_out + gh * max_parts * MLA_DV + d;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool on = i < np;
+                v[hh][i] = on ? *(const f32x4*)(po + (int64_t)i * MLA_DV) : (f32x4){0.f, 0.f, 0.f, 0.f};
+                m[hh][i] = on ? ml[2 * i] : MLA_NEG;
+                l[hh][i] = on ? ml[2 * i + 1] : 0.f;
+            }
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) num += v[i] * f[i];
+        for (int hh = 0; hh < MR_HEADS; ++hh) {
+            if (hh >= live) break;
+            float M = MLA_NEG;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) M = fmaxf(M, m[hh][i]);
+            f32x4 num = {0.f, 0.f, 0.f, 0.f};
+            float den = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float f = i < np ? __builtin_amdgcn_exp2f(m[hh][i] - M) : 0.f;
+                den += f * l[hh][i];
+                num += v[hh][i] * f;
+            }
+            const float inv = 1.0f / den;
+            *(u32x2*)(out + (gh0 + hh) * MLA_DV + d) =
+                (u32x2){pack2<T>(num[0] * inv, num[1] * inv), pack2<T>(num[2] * inv, num[3] * inv)};
+        }
+        return;
     }
-    const float inv = 1.0f / den;
-    *(u32x2*)(out + gh * MLA_DV + d) =
-        (u32x2){pack2<T>(num[0] * inv, num[1] * inv), pack2<T>(num[2] * inv, num[3] * inv)};
+    for (int hh = 0; hh < live; ++hh) {                       // long contexts: head by head, 8 partitions at a time
+        const int64_t gh = gh0 + hh;
+        const float* ml = part_ml + gh * max_parts * 2;
+        const float* po = part_out + gh * max_parts * MLA_DV + d;
+        float M = MLA_NEG;
+        for (int p = 0; p < np; ++p) M = fmaxf(M, ml[2 * p]);     // uniform addresses: broadcast loads
+        f32x4 num = {0.f, 0.f, 0.f, 0.f};
+        float den = 0.f;
+        for (int p0 = 0; p0 < np; p0 += 8) {
+            f32x4 v[8];
+            float f[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool on = p0 + i < np;
+                v[i] = on ? *(const f32x4*)(po + (int64_t)(p0 + i) * MLA_DV) : (f32x4){0.f, 0.f, 0.f, 0.f};
+                f[i] = on ? __builtin_amdgcn_exp2f(ml[2 * (p0 + i)] - M) : 0.f;
+                den += on ? f[i] * ml[2 * (p0 + i) + 1] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) num += v[i] * f[i];
+        }
+        const float inv = 1.0f / den;
+        *(u32x2*)(out + gh * MLA_DV + d) =
+            (u32x2){pack2<T>(num[0] * inv, num[1] * inv), pack2<T>(num[2] * inv, num[3] * inv)};
+    }
 }
 
 // zero the rows of sequences with no context when a single partition spans the context (the main kernel skips them)
@@ -581,6 +664,7 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
     const MlaPlan plan = mla_plan(n_heads, max_ctx);
     float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
     float* part_ml = part_out ? part_out + (int64_t)batch * n_heads * plan.max_parts * MLA_DV : nullptr;
+    int32_t* plan_word = part_ml ? (int32_t*)(part_ml + (int64_t)batch * n_heads * plan.max_parts * 2) : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
     if (plan.max_parts == 1) {
         hipLaunchKernelGGL(mla_zero_empty_kernel, dim3(batch), dim3(128), 0, st, (uint16_t*)out, context_lens,
@@ -588,18 +672,17 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
         const int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
-    const int64_t wgs = plan.max_parts == 1
-                            ? (int64_t)batch * plan.head_blocks
-                            : (int64_t)mla_free_slots(batch, plan.head_blocks, n_slots) + (int64_t)batch * plan.head_blocks;
+    const int64_t wgs = plan.max_parts == 1 ? (int64_t)batch * plan.head_blocks
+                                            : (int64_t)mla_grid(batch, plan.head_blocks, n_slots);
     hipLaunchKernelGGL(mla_decode_kernel<T>, dim3((unsigned)wgs), dim3(M2_WAVES * 64), M2_SMEM, st, (uint16_t*)out,
                        part_out, part_ml, (const uint16_t*)query, (const uint16_t*)cache, block_tables, context_lens,
                        n_heads, plan.head_blocks, block_size, max_blocks, num_blocks, plan.max_parts, n_slots,
-                       scale_log2, q_stride, batch);
+                       scale_log2, q_stride, batch, plan_word);
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
-        hipLaunchKernelGGL(mla_reduce_kernel<T>, dim3(n_heads, batch), dim3(MR_THREADS), 0, st, (uint16_t*)out, part_out,
-                           part_ml, context_lens, n_heads, plan.max_parts, batch, plan.head_blocks, n_slots,
+        hipLaunchKernelGGL(mla_reduce_kernel<T>, dim3((n_heads + MR_HEADS - 1) / MR_HEADS, batch), dim3(MR_THREADS), 0, st,
+                           (uint16_t*)out, part_out, part_ml, context_lens, plan_word, n_heads, plan.max_parts,
                            (int)max_ctx);
         rc = MF_LAUNCH_CHECK();
     }
@@ -612,7 +695,8 @@ extern "C" size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads,
     if (batch <= 0 || n_heads <= 0 || max_context <= 0) return 0;
     const MlaPlan plan = mla_plan(n_heads, max_context);
     if (plan.max_parts <= 1) return 0;
-    return (size_t)batch * n_heads * plan.max_parts * (MLA_DV + 2) * sizeof(float);
+    // partial accumulators, (max, sum) pairs, and the word that carries the partition rule's value to the reduce kernel
+    return (size_t)batch * n_heads * plan.max_parts * (MLA_DV + 2) * sizeof(float) + 16;
 }
 
 extern "C" int mf_mla_paged_attention_decode(void* out, const void* query, const void* latent_cache,
