@@ -1226,12 +1226,27 @@ static inline PfPlan pf_plan(int batch, int64_t total_q, int n_heads, int n_kv, 
     return p;
 }
 
-// zero the rows the single-partition prefill path never writes (rows of no sequence)
+// Zero the rows the single-partition prefill path never writes (rows of no sequence): one workgroup per sequence
+// takes the rows between the sequence's last query and the next sequence's first (the end of the output for the
+// last sequence), the first workgroup also those before the first sequence.  Usually there are none.
 __global__ void pf_zero_rows_kernel(uint16_t* __restrict__ out, const int32_t* __restrict__ q_starts,
                                     const int32_t* __restrict__ ctx_lens, bool contiguous, int max_ctx, int batch,
-                                    int row) {
-    if (pf_row_limit(blockIdx.x, q_starts, ctx_lens, contiguous, gridDim.x, max_ctx, batch) > 0) return;
-    for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)blockIdx.x * row + i] = 0;
+                                    int row, int rows) {
+    const int s = blockIdx.x;
+    int qs, ql, len;
+    pf_seq(s, q_starts, ctx_lens, contiguous, rows, max_ctx, batch, qs, ql, len);
+    const int64_t lo = qs < 0 ? 0 : (int64_t)qs + ql;
+    int64_t hi = s + 1 < batch ? q_starts[s + 1] : rows;
+    hi = hi > rows ? rows : hi;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t r = lo; r < hi; ++r)
+        for (int i = threadIdx.x * 8; i < row; i += blockDim.x * 8) *(u32x4*)(out + r * row + i) = z;
+    if (s == 0) {
+        int64_t first = q_starts[0];
+        first = first > rows ? rows : first;
+        for (int64_t r = 0; r < first; ++r)
+            for (int i = threadIdx.x * 8; i < row; i += blockDim.x * 8) *(u32x4*)(out + r * row + i) = z;
+    }
 }
 
 template <typename T, int D, bool KV8>
@@ -1252,8 +1267,8 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
         return 1;
     }
     if (plan.max_parts == 1) {
-        hipLaunchKernelGGL(pf_zero_rows_kernel, dim3(total_q), dim3(128), 0, st, (uint16_t*)out, q_starts,
-                           context_lens, contiguous, max_blocks * block_size, batch, n_heads * D);
+        hipLaunchKernelGGL(pf_zero_rows_kernel, dim3(batch), dim3(256), 0, st, (uint16_t*)out, q_starts, context_lens,
+                           contiguous, max_blocks * block_size, batch, n_heads * D, total_q);
         int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
