@@ -9,6 +9,10 @@ timed live with events on the launch stream) and the CPU restatement of the same
 cores on a bounded sample.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--no-cpu]
+
+Workloads: llama3_8b_w8a16 (default), llama3_8b_w8a16_kv8, tiny_llama_w8a16, qwen2_5_7b_w8a8, qwen2_5_72b_w8a16
+(layer steps); deepseek_v3_moe_w8a16 (one MoE layer step); deepseek_v3_mla_decode, llama3_8b_prefill_attention,
+llama3_8b_chunked_prefill_attention, deepseek_v3_mla_prefill_attention (one attention call per step).
 """
 import argparse
 import json
