@@ -478,6 +478,16 @@ def test_mla_paged_attention_large_batch():
     assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what="MLA paged attention, batch 210")
 
 
+def test_mla_paged_attention_partition_rule_over_several_chunks_of_sequences():
+    """More than 64 sequences with contexts long enough that the partition rule counts its smaller candidates over
+    two chunks of lengths, and sequences cut into 1 to 8 partitions equal up to one tile."""
+    rng = np.random.default_rng(78)
+    lens = rng.integers(300, 1500, 100)
+    lens[[3, 70]] = [33, 2900]
+    got, ref, mag = _mla_case(rng, torch.bfloat16, lens, 16, 32)
+    assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what="MLA paged attention, batch 100, long contexts")
+
+
 def test_attention_rejects_a_non_positive_scale():
     """Prefill and MLA decode take the maximum over raw scores: the scale must be positive (checked on the host)."""
     rng = np.random.default_rng(3)
