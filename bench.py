@@ -38,7 +38,9 @@ METRICS = {
     "deepseek_v3_moe_w8a16": "MoE layer tokens/sec (DeepSeek-V3 shape, 256 experts W8A16, 128 tokens); % of peak HBM GB/s",
 }
 TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-ATTENTION_SOURCE = os.path.join(ROOT, "mindformers_amd", "csrc", "paged_attention.hip")
+# the decode attention kernels and their launch rule (the prefill side lives in prefill_attention.hip)
+ATTENTION_SOURCES = [os.path.join(ROOT, "mindformers_amd", "csrc", n)
+                     for n in ("paged_attention_kernels.h", "paged_attention.hip")]
 
 
 def log(*a):
@@ -119,10 +121,13 @@ def kernel_breakdown(case, torch, ops, iters):
     return out
 
 
-def source_sha256(path):
+def source_sha256(paths):
     import hashlib
-    with open(path, "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()
+    h = hashlib.sha256()
+    for path in paths:
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
 
 
 def measured_traffic(workload, kv_bytes):
@@ -136,7 +141,7 @@ def measured_traffic(workload, kv_bytes):
         return None, "no counter record under profiles/"
     if rec.get("workload") != workload or rec.get("kv_bytes") != kv_bytes:
         return None, "the counter record covers another workload"
-    if rec.get("kernel_source_sha256") != source_sha256(ATTENTION_SOURCE):
+    if rec.get("kernel_source_sha256") != source_sha256(ATTENTION_SOURCES):
         return None, "the attention kernel source changed since the counters were read (record of commit %s)" % rec.get("commit")
     return int(rec["traffic_bytes"]), "profiles/hbm_traffic.json, commit %s" % rec.get("commit")
 
@@ -170,8 +175,9 @@ def record_traffic(fetch_csv, write_csv, workload, kv_bytes):
     commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
     rec = {"paged_attention": {"workload": workload, "kv_bytes": int(kv_bytes), "traffic_bytes": int(kib * 1024),
                                "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4),
-                               "commit": commit or "unknown", "kernel_source": "mindformers_amd/csrc/paged_attention.hip",
-                               "kernel_source_sha256": source_sha256(ATTENTION_SOURCE)}}
+                               "commit": commit or "unknown",
+                               "kernel_source": "mindformers_amd/csrc/paged_attention_kernels.h + paged_attention.hip",
+                               "kernel_source_sha256": source_sha256(ATTENTION_SOURCES)}}
     with open(TRAFFIC_RECORD, "w") as f:
         json.dump(rec, f, indent=1)
         f.write("\n")
@@ -250,13 +256,10 @@ def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
         max_abs_err=err, ref_max_abs=scale, rows=len(idx))
 
 
-def int8_gemm_roofline(case, torch, ops, iters):
+def int8_gemm_roofline(layer, x, torch, ops, iters):
     """The four int8 GEMMs of a W8A8 layer step (QKV, output, gate/up, down projection), each timed with events on
     the launch stream on the operands the layer feeds it: int8 ops (2 M N K, summed) over the summed durations
     against the dense int8 MFMA peak."""
-    layer = case["layers"][0]
-    kc, vc = case["caches"][0]
-    x = case["x"]
     m = x.shape[0]
     n1q = ops.rms_norm_dynamic_quant(x, layer.attn_norm, layer.eps, layer.qkv_smooth, tiled=True)
     qkv = ops.w8a8_linear(n1q[0], n1q[1], layer._packed["qkv"], out_dtype=layer.dtype)
@@ -287,6 +290,23 @@ def int8_gemm_roofline(case, torch, ops, iters):
                 peak=INT8_PEAK_TOPS, unit="TOP/s", frac=round(ach / INT8_PEAK_TOPS, 4), traffic=None,
                 ops_per_step=total_ops, avg_launch_us=round(total_us, 2), per_gemm_us=us,
                 weight_stream_gbps=round(weight_bytes / (total_us * 1e-6) / 1e9, 1))
+
+
+def w8a8_gemm_leg(torch, ops, synthetic, iters):
+    """int8_gemm_roofline on a freshly built Qwen2.5-7B-shape W8A8 layer (hidden 3584, ffn 18944, 28 q / 4 kv heads)
+    and 256 activation rows from N(0, 1): the configuration the int8 matrix-core target is quoted on."""
+    from mindformers_amd.decode_layer import QuantDecodeLayer
+    cfg = synthetic.CONFIGS["qwen2_5_7b_w8a8"]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    layer = synthetic.fill_layer(QuantDecodeLayer(cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"],
+                                                  cfg["ffn"], 1e-5, cfg["dtype"], True, device="cuda"), gen)
+    x = torch.randn(cfg["batch"], cfg["hidden"], generator=gen, device="cuda").to(cfg["dtype"])
+    out = int8_gemm_roofline(layer, x, torch, ops, iters)
+    out["workload"] = f"qwen2_5_7b_w8a8 GEMMs: {cfg['batch']} rows, hidden {cfg['hidden']}, ffn {cfg['ffn']}"
+    del layer
+    torch.cuda.empty_cache()
+    return out
 
 
 def bench_modules(case, torch, ops, args):
@@ -634,6 +654,7 @@ def main():
     ap.add_argument("--modules", action="store_true",
                     help="also time the step composed from the drop-in module cells (default for the headline workload)")
     ap.add_argument("--no-modules", action="store_true", help="skip the drop-in module leg")
+    ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg of the default workload")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: turn the counter_collection CSVs of two profiler runs of this command with "
                          "--calibrate-counters (--pmc FETCH_SIZE, --pmc WRITE_SIZE) into profiles/hbm_traffic.json")
@@ -769,9 +790,13 @@ def main():
         # W8A8: the figure of merit is the int8 matrix rate of the four projections at this batch; the attention
         # roofline moves to a second key
         extra["attention_roofline"] = roofline
-        roofline = int8_gemm_roofline(case, torch, ops, args.kernel_iters)
+        roofline = int8_gemm_roofline(case["layers"][0], case["x"], torch, ops, args.kernel_iters)
     if args.modules or (args.workload == "llama3_8b_w8a16" and not args.no_modules):
         extra["drop_in_modules"] = bench_modules(case, torch, ops, args)
+    if args.workload == "llama3_8b_w8a16" and not args.no_w8a8:
+        # the second figure of merit rides on the default line: the four int8 GEMMs of the Qwen2.5-7B-shape W8A8 layer
+        # at batch 256 (no KV cache needed), against the dense int8 matrix-core peak
+        extra["w8a8_int8_gemm_roofline"] = w8a8_gemm_leg(torch, ops, synthetic, args.kernel_iters)
 
     result = {
         "metric": METRICS.get(args.workload, METRICS["llama3_8b_w8a16"]),
@@ -786,7 +811,10 @@ def main():
                               else "eager"),
                    "algorithmic_bytes_per_layer": nbytes["total"]},
         "layer_hbm_gbps": round(layer_gbps, 1), "layer_hbm_frac": round(layer_gbps / HBM_PEAK_GBPS, 4),
-        "roofline": roofline, "breakdown_us": breakdown,
+        "roofline": roofline,
+        # each op of the unfused layer launched back to back on its own (not a split of ms_per_step: the timed step
+        # runs the fused entry points inside one graph)
+        "unfused_op_us": breakdown,
     }
     result.update(extra)
     if cfg.get("kv_int8"):

@@ -14,7 +14,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmf_decode.so")
 
-SOURCES = ["errors.cpp", "kv_cache.hip", "paged_attention.hip", "elementwise.hip", "w8a16_gemm.hip",
+SOURCES = ["errors.cpp", "kv_cache.hip", "paged_attention.hip", "prefill_attention.hip", "elementwise.hip", "w8a16_gemm.hip",
            "w8a8_gemm.hip", "moe.hip", "mla_attention.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

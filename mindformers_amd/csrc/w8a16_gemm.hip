@@ -380,13 +380,17 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
             uint32_t off = xlane[i] + (uint32_t)sc * (GW_KSTEP * 2);
+            uint32_t km = 0xffffffffu;
             if (KTAIL) {
-                // chunks past K (last, short step) re-read the row's last whole chunk: finite values that meet
-                // zero weights
+                // chunks past K (last, short step) re-read the row's last whole chunk and are zeroed with a mask (an
+                // AND, so that the load stays unconditional): the padded weight columns are zero, but an Inf or NaN
+                // among the last activations of a row must not meet them
                 const int over = sc * GW_KSTEP + xchunk8[i] - (K - 8);
                 off -= over > 0 ? 2u * over : 0u;
+                km = over > 0 ? 0u : 0xffffffffu;
             }
-            xreg[S][i] = *(const u32x4*)(xbase + off);
+            const u32x4 v = *(const u32x4*)(xbase + off);
+            xreg[S][i] = KTAIL ? (u32x4){v[0] & km, v[1] & km, v[2] & km, v[3] & km} : v;
         }
     };
     auto stage_x = [&](auto setc, int stage) {                // this wave's activation chunks of a set -> LDS stage

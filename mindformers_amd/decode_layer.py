@@ -34,6 +34,7 @@ class QuantDecodeLayer(nn.Module):
         self.eps, self.dtype, self.act_quant = eps, dtype, act_quant
         self.scale_value = 1.0 / math.sqrt(head_dim)
         self._packed = {}
+        self.raw_weights = {}                                 # host copies of released row-major weights
         shapes = {"qkv": ((n_head + 2 * n_kv_head) * head_dim, hidden), "wo": (hidden, n_head * head_dim),
                   "fc1": (2 * ffn, hidden), "fc2": (hidden, ffn)}
         for name, (n, k) in shapes.items():
@@ -60,10 +61,12 @@ class QuantDecodeLayer(nn.Module):
             return ops.w8a8_linear(xq, xs, packed, out_dtype=self.dtype, bias=b, residual=residual)
         return ops.w8a16_linear(x, packed, bias=b, residual=residual)
 
-    def prepare(self, release_raw=True):
-        """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights.
-        The packed copy is the only one the kernels read: with ``release_raw`` the row-major ``*_w`` buffers move to
-        host memory afterwards (still readable, e.g. for export), so the device holds every weight once."""
+    def prepare(self, release_raw=False):
+        """Pack the int8 weights into the tile order the GEMM kernels stream.  Call once after loading weights, and
+        again after loading new ones.  The packed copy is the only one the kernels read.  With ``release_raw`` the
+        row-major ``*_w`` tensors leave the module's buffers for host copies kept as plain attributes (``raw_weights``,
+        still readable, e.g. for export), so that the device holds every weight once and a later ``.to(device)`` does
+        not bring a second copy back; the ``*_w`` names then resolve to those host copies."""
         dev = self.attn_norm.device
         for name in self.NAMES:
             w, s = getattr(self, f"{name}_w").to(dev), getattr(self, f"{name}_s")
@@ -71,8 +74,21 @@ class QuantDecodeLayer(nn.Module):
             gated = name == "fc1" and not self.act_quant and getattr(self, "fc1_b") is None
             self._packed[name] = ops.pack_w8a16_gated(w, s, "halves") if gated else ops.pack_w8a16(w, s)
             if release_raw:
-                self._buffers[f"{name}_w"] = w.cpu()
+                self._buffers.pop(f"{name}_w", None)
+                self.raw_weights[f"{name}_w"] = w.cpu()
         return self
+
+    def __getattr__(self, name):
+        raw = self.__dict__.get("raw_weights")
+        if raw is not None and name in raw:
+            return raw[name]
+        return super().__getattr__(name)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # new weights invalidate the packed copies: the next forward asks for prepare() again
+        if any(k.startswith(prefix) and k[len(prefix):].rsplit("_", 1)[0] in self.NAMES for k in state_dict):
+            self._packed.clear()
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def set_kv_quant(self, scale, offset=None):
         """Per-channel parameters of int8 caches: x ~ (q - offset) * scale; float32 [2, n_kv_head * head_dim]."""

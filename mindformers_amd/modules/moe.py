@@ -125,11 +125,14 @@ class QuantGroupedMLP(nn.Module):
     def quantize_from_float(self, weight1, weight2):
         """weight1 [E, H, 2F], weight2 [E, F, H] float (reference layout) -> int8 per output channel."""
         for src, dst, sc in ((weight1, self.weight1, self.w1_scale), (weight2, self.weight2, self.w2_scale)):
-            w = src.detach().to(device=dst.device, dtype=torch.float32).transpose(1, 2).contiguous()     # [E, out, in]
-            scale = w.abs().amax(dim=2) / 127.0
-            safe = torch.where(scale > 0, scale, torch.ones_like(scale))
-            dst.copy_(torch.clamp(torch.round(w / safe[..., None]), -127, 127).to(torch.int8))
-            sc.copy_(scale)
+            # expert by expert in float64: the scale is max|w| / 127 rounded to float32 and the quotient is taken in
+            # float64, as the dense cells do, so that the int8 grid point does not depend on a float32 division
+            for e in range(src.shape[0]):
+                w = src[e].detach().to(device=dst.device, dtype=torch.float64).t()                       # [out, in]
+                scale = (w.abs().amax(dim=1) / 127.0).float()
+                safe = torch.where(scale > 0, scale, torch.ones_like(scale)).double()
+                dst[e].copy_(torch.clamp(torch.round(w / safe[:, None]), -127, 127).to(torch.int8))
+                sc[e].copy_(scale)
         self._p1 = self._p2 = None
         return self
 

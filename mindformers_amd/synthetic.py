@@ -62,7 +62,7 @@ def fill_layer(layer, gen, std=0.02):
             getattr(layer, f"{name}_smooth").copy_(torch.rand(k, generator=gen, device=dev) * 1.5 + 0.5)
     layer.attn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
     layer.ffn_norm.copy_(1.0 + 0.1 * torch.randn(layer.hidden, generator=gen, device=dev))
-    return layer.prepare()
+    return layer.prepare(release_raw=True)                      # the packed copy is the only one on the device
 
 
 def context_lens(name, seed=0, batch=None, ctx=None):

@@ -466,6 +466,71 @@ def test_long_context_layer_step_stage_by_stage(qwen72_case):
     _w8a16_stages(qwen72_case, 16, attn_rows=2)
 
 
+def test_long_context_stack_of_eight_layers_chained():
+    """The Qwen2.5-72B long-context configuration as the benchmark runs it: a stack of 8 layers, every layer handing
+    its output's norm under the next layer's gamma to the next one.  The chained stack must give the bits of eight
+    separate layer calls (hidden state and every cache), and its last hidden state must agree with the float32
+    restatement of the eight layers on the host for two of the sequences."""
+    from mindformers_amd import synthetic
+    from oracle import torch_cpu
+    case = synthetic.make_decode_case("qwen2_5_72b_w8a16", seed=11, layers=8)
+    cfg, layers = case["cfg"], case["layers"]
+    rest = (case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
+    n_seq = 2
+    t2, sel, slots2 = _sub_batch(case, n_seq)
+    before = [(kc[sel].float().cpu(), vc[sel].float().cpu()) for kc, vc in case["caches"]]   # the host's own copies
+
+    def run(chained):
+        caches = [(kc.clone(), vc.clone()) for kc, vc in case["caches"]] if not chained else case["caches"]
+        h, normed, states = case["x"], None, []
+        for i, (layer, (kc, vc)) in enumerate(zip(layers, caches)):
+            if chained and i + 1 < len(layers):
+                h, normed = layer(h, kc, vc, *rest, normed=normed, next_norm=(layers[i + 1].attn_norm, layers[i + 1].eps))
+            else:
+                h = layer(h, kc, vc, *rest, normed=normed if chained else None)
+            states.append(h)
+        return states, caches
+    s_sep, c_sep = run(False)
+    s_chain, c_chain = run(True)
+    for a, b in zip(s_sep, s_chain):
+        assert torch.equal(a, b)
+    for (k0, v0), (k1, v1) in zip(c_sep, c_chain):
+        assert torch.equal(k0, k1) and torch.equal(v0, v1)
+    del c_sep
+    torch.cuda.empty_cache()
+    # the host's float32 pass, two sequences: every layer on the hidden state the device fed it (the single-layer
+    # bound), and the eight layers in a row on the host's own hidden states
+    ocfg = dict(n_head=cfg["n_head"], n_kv_head=cfg["n_kv_head"], head_dim=cfg["head_dim"], eps=1e-5)
+    cos, sin = case["cos"][:n_seq].float().cpu(), case["sin"][:n_seq].float().cpu()
+    lens = case["context_lens_host"][:n_seq]
+    x_own = case["x"][:n_seq].float().cpu()
+    for i, (layer, (kc32, vc32)) in enumerate(zip(layers, before)):
+        p = {}
+        for n in layer.NAMES:
+            p[n + "_w"], p[n + "_s"] = to_np(getattr(layer, n + "_w")), to_np(getattr(layer, n + "_s"))
+        p["attn_norm"], p["ffn_norm"] = to_np(layer.attn_norm), to_np(layer.ffn_norm)
+        tp = torch_cpu.prepare_params(p)
+        del p
+        x_dev = (case["x"] if i == 0 else s_chain[i - 1])[:n_seq].float().cpu()
+        kc_a, vc_a = kc32.clone(), vc32.clone()
+        ref = torch_cpu.decode_layer_w8a16_fp32(x_dev, tp, ocfg, kc_a, vc_a, t2, lens, slots2, cos, sin,
+                                                act_dtype="bf16").numpy().astype(np.float64)
+        got = to_np(s_chain[i][:n_seq]).astype(np.float64)
+        err = np.abs(got - ref)
+        row_max = np.abs(ref).max(axis=1, keepdims=True)
+        tol = 8 * EPS[BF] * np.maximum(np.abs(ref), 0.05 * row_max) + 1e-4
+        assert float(np.mean(err > tol)) < 0.02, (i, float(np.mean(err > tol)), err.max())
+        assert np.all(err <= 8 * EPS[BF] * np.maximum(np.abs(ref), 0.25 * row_max) + 1e-4), (i, err.max())
+        x_own = torch_cpu.decode_layer_w8a16_fp32(x_own, tp, ocfg, kc32, vc32, t2, lens, slots2, cos, sin,
+                                                  act_dtype="bf16")
+        del tp
+    # end to end the one-step differences of intermediates travel through the residual path of every later layer:
+    # agreement in norm only
+    ref, got = x_own.numpy().astype(np.float64), to_np(s_chain[-1][:n_seq]).astype(np.float64)
+    rel = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert rel < 5e-2, rel
+
+
 # ------------------------------------------------------------------------------ DeepSeek-V3 MoE layer at full shape
 @pytest.fixture(scope="module")
 def moe_case():

@@ -847,6 +847,29 @@ def test_w8a16_exact_on_integer_grid():
     assert np.array_equal(to_np(y).astype(np.float64), rounded(exact, torch.float16).astype(np.float64))
 
 
+@pytest.mark.parametrize("m,n,k", [(37, 200, 1376), (64, 256, 1032), (5, 80, 72)])
+def test_w8a16_inf_in_the_last_columns_of_a_row_stays_in_that_row(m, n, k):
+    """K is not a multiple of 64, so the last k-step is short and its padding columns carry zero weights.  An Inf
+    among the last activations of one row gives that row +-Inf with the sign of the weight it meets (NaN where that
+    weight is zero), exactly as the sum over the real K columns does, and leaves every other row exact: no
+    activation may reach a padding column (Inf * 0 would turn the whole row into NaN)."""
+    rng = np.random.default_rng(k)
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    wq[::7, k - 3] = 0
+    s = (2.0 ** rng.integers(-9, -6, n)).astype(np.float32)
+    x = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    bad = m // 2
+    xt = dev(x, torch.float16)
+    xt[bad, k - 3] = float("inf")
+    y = to_np(ops.w8a16_linear(xt, torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())).astype(np.float64)
+    exact = rounded((x.astype(np.int64) @ wq.astype(np.int64).T).astype(np.float64) * s, torch.float16).astype(np.float64)
+    keep = np.arange(m) != bad
+    assert np.array_equal(y[keep], exact[keep])
+    w_hit = wq[:, k - 3].astype(np.float64)
+    assert np.isnan(y[bad][w_hit == 0]).all()
+    assert np.array_equal(y[bad][w_hit != 0], np.sign(w_hit[w_hit != 0]) * np.inf)
+
+
 def test_column_parallel_linear_reference_vectors(golden_dir):
     """The reference's linear vectors are for the bf16 cell; they pin the W8A16 path's layout ([out, in] weight,
     bias add): quantise the reference weight, run the kernel, compare with the oracle linear on the dequantised
