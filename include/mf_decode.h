@@ -216,6 +216,19 @@ int mf_mla_paged_attention_decode(void* out, const void* query, const void* late
                                   int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The weight-absorbed per-head projections around the multi-latent decode attention:
+ *   q_no_pe = mint.transpose(mint.matmul(mint.transpose(q_no_pe, -3, -2), q_absorb), -3, -2)
+ *   core_attn_out = mint.matmul(mint.transpose(core_attn_out, -3, -2), mint.transpose(out_absorb, -2, -1))
+ *   mindformers/parallel_core/inference/transformer/multi_latent_attention.py:434-448, :228-231
+ * out[t, h, :n] = x[t, h, :k] . w[h]^T with w [heads, n, k] dense (for the query side the slice of
+ * linear_kv_up_proj.weight is stored transposed once, so that both sides read rows of k).  x and out are addressed by
+ * element strides between tokens and between heads, so that q_no_pe can be read inside the [T, heads, 192] query
+ * projection and the result written into the first 512 columns of the [T, heads, 576] attention query.
+ * fp32 accumulation, one rounding.  k in {64, 128, 256, 512}; n a multiple of 16. */
+int mf_mla_absorb_bmm(void* out, const void* x, const void* w, int tokens, int heads, int n, int k,
+                      int64_t x_token_stride, int64_t x_head_stride, int64_t out_token_stride,
+                      int64_t out_head_stride, int dtype, void* stream);
+
 /* ---- norm / activation ---------------------------------------------------------------------------- */
 
 /* P.RmsNorm(eps)(x, gamma): mindformers/models/llama/llama_layer.py:195,225-228;

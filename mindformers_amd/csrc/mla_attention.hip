@@ -689,6 +689,194 @@ int launch_mla(void* out, const void* query, const void* cache, const int32_t* b
     return rc;
 }
 
+
+// ---- weight-absorbed per-head projections of a multi-latent attention layer --------------------------------------
+// out[t, h, n] = sum_k x[t, h, k] * w[h, n, k]: a batch of `heads` skinny GEMMs with a different [N, K] weight per
+// head and the token rows as the small side (decode: the query up-projection folded into the latent space,
+// [T, 128] x [128 -> 512] per head, and the value up-projection applied to the attention output, [T, 512] x
+// [512 -> 128]).  Weights (2 x 16.8 MB at 128 heads), activations and results should each cross the L2 once.  A
+// workgroup of 8 waves owns one head, 128 NT channels of it (all of them at the two decode shapes) and up to 64
+// tokens; wave w keeps the weight tiles of its 16 NT channels in registers, already in MFMA operand order (row, 8
+// consecutive k per lane: one 16-byte load per k-step), and walks the token tiles; the rows of a token tile are read
+// by all 8 waves and meet in the L1, the next tile's rows are in flight while the current one is multiplied.
+// Results leave as 16-byte pieces (neighbouring lanes first swap halves so that a lane holds 8 consecutive
+// channels).  No LDS, no barriers.
+constexpr int AB_WAVES = 8;
+
+template <typename T, int KS, int NT>
+__global__ __launch_bounds__(AB_WAVES * 64, 1) void mla_absorb_bmm_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int tokens, int N,
+    int wg_tokens, int64_t xs_t, int64_t xs_h, int64_t os_t, int64_t os_h) {
+    using vec8 = typename T::vec8;
+    constexpr int K = 32 * KS;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int h = blockIdx.y;
+    const int nb0 = blockIdx.x * (AB_WAVES * 16 * NT) + wave * (16 * NT);
+    if (nb0 >= N) return;                                     // uniform over the wave; there is no barrier below
+    const int t_begin = blockIdx.z * wg_tokens;
+    const int t_end = min(tokens, t_begin + wg_tokens);
+    vec8 wreg[NT][KS];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n = min(nb0 + 16 * j, N - 16) + r;          // tiles past N (a multiple of 16) repeat the last one
+        const uint16_t* wp = w + ((int64_t)h * N + n) * K + 8 * g;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) wreg[j][s] = *(const vec8*)(wp + 32 * s);
+    }
+    const uint16_t* xh = x + (int64_t)h * xs_h + 8 * g;
+    auto load_x = [&](vec8* xv, int t0) {
+        const int t = min(t0 + r, tokens - 1);                // rows past the end repeat the last one, never stored
+#pragma unroll
+        for (int s = 0; s < KS; ++s) xv[s] = *(const vec8*)(xh + (int64_t)t * xs_t + 32 * s);
+    };
+    auto tile = [&](const vec8* xv, int t0) {
+        u32x2 piece[NT];                                      // channels nb0 + 16 j + 4 g .. + 3 of token t0 + r
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s) acc = T::mfma16(wreg[j][s], xv[s], acc);
+            piece[j] = (u32x2){pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
+        }
+        const bool row_ok = t0 + r < t_end;
+        uint16_t* orow = out + (int64_t)(t0 + r) * os_t + (int64_t)h * os_h + nb0;
+        if constexpr (NT == 1) {
+            if (row_ok) *(u32x2*)(orow + 4 * g) = piece[0];
+        } else {
+            // lanes g and g ^ 1 swap one piece per tile pair: the even lane ends up with channels 4 g .. 4 g + 7 of
+            // the pair's first tile, the odd lane with channels 4 (g - 1) .. 4 g + 3 of its second
+            const bool odd = g & 1;
+#pragma unroll
+            for (int m = 0; m < NT / 2; ++m) {
+                const u32x2 send = odd ? piece[2 * m] : piece[2 * m + 1];
+                u32x2 recv;
+                recv[0] = __shfl_xor(send[0], 16, 64);
+                recv[1] = __shfl_xor(send[1], 16, 64);
+                const int j = 2 * m + (odd ? 1 : 0);
+                const u32x4 o = odd ? (u32x4){recv[0], recv[1], piece[j][0], piece[j][1]}
+                                    : (u32x4){piece[j][0], piece[j][1], recv[0], recv[1]};
+                if (row_ok && nb0 + 16 * j < N) *(u32x4*)(orow + 16 * j + 4 * (g & ~1)) = o;
+            }
+        }
+    };
+    // two register sets of token rows alternate: the next tile is fetched behind the current one's products
+    vec8 xa[KS], xb[KS];
+    load_x(xa, t_begin);
+    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+        load_x(xb, t0 + 16);
+        tile(xa, t0);
+        if (t0 + 16 >= t_end) break;
+        load_x(xa, t0 + 32);
+        tile(xb, t0 + 16);
+    }
+}
+
+// Long reductions (k = 256, 512: the output side, [T, 512] x [512 -> 128] per head): the token rows are the big
+// operand there, and eight waves fetching the same 16 KB tile each would pull it through the L2 eight times.  The
+// workgroup loads a token tile once, cooperatively and fully coalesced, into one of two LDS stages (one barrier per
+// tile; 16-byte chunk c of row r sits in slot c ^ r, which spreads the 16 rows an operand read touches over all
+// banks), and every wave reads its B operands from there.  One 16-channel tile per wave.
+template <typename T, int KS>
+__global__ __launch_bounds__(AB_WAVES * 64, 1) void mla_absorb_bmm_lds_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int tokens, int N,
+    int wg_tokens, int64_t xs_t, int64_t xs_h, int64_t os_t, int64_t os_h) {
+    using vec8 = typename T::vec8;
+    constexpr int K = 32 * KS;
+    constexpr int CPR = K / 8;                                // 16-byte chunks per token row
+    constexpr int STAGE = 16 * K * 2;
+    constexpr int XL = 16 * CPR / (AB_WAVES * 64);            // chunks per thread and tile
+    static_assert(XL >= 1 && CPR >= 16, "the chunk permutation needs at least 16 chunks per row");
+    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * STAGE];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int h = blockIdx.y;
+    const int nb0 = blockIdx.x * (AB_WAVES * 16) + wave * 16;
+    const bool active = nb0 < N;                              // idle waves still stage rows and meet the barriers
+    const int t_begin = blockIdx.z * wg_tokens;
+    const int t_end = min(tokens, t_begin + wg_tokens);
+    vec8 wreg[KS];
+    {
+        const int n = min(nb0, N - 16) + r;
+        const uint16_t* wp = w + ((int64_t)h * N + n) * K + 8 * g;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) wreg[s] = *(const vec8*)(wp + 32 * s);
+    }
+    const uint16_t* xh = x + (int64_t)h * xs_h;
+    u32x4 stg[XL];
+    auto fetch = [&](int t0) {                                // this thread's chunks of tile t0 -> registers
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int id = threadIdx.x + i * (AB_WAVES * 64);
+            const int row = id / CPR, c = id - row * CPR;
+            const int t = min(t0 + row, tokens - 1);
+            stg[i] = *(const u32x4*)(xh + (int64_t)t * xs_t + 8 * c);
+        }
+    };
+    auto park = [&](int stage) {                              // registers -> LDS stage
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int id = threadIdx.x + i * (AB_WAVES * 64);
+            const int row = id / CPR, c = id - row * CPR;
+            *(u32x4*)(smem + stage * STAGE + row * (K * 2) + ((c ^ row) << 4)) = stg[i];
+        }
+    };
+    fetch(t_begin);
+    park(0);
+    __syncthreads();
+    int stage = 0;
+    for (int t0 = t_begin; t0 < t_end; t0 += 16, stage ^= 1) {
+        const bool more = t0 + 16 < t_end;
+        if (more) fetch(t0 + 16);                             // in flight behind this tile's products
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const uint8_t* row = smem + stage * STAGE + r * (K * 2);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const u32x4 xb = *(const u32x4*)(row + (((4 * s + g) ^ r) << 4));
+            acc = T::mfma16(wreg[s], bitcast<vec8>(xb), acc);
+        }
+        if (active && t0 + r < t_end)
+            *(u32x2*)(out + (int64_t)(t0 + r) * os_t + (int64_t)h * os_h + nb0 + 4 * g) =
+                (u32x2){pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
+        if (more) park(stage ^ 1);                            // last read two tiles ago, before the previous barrier
+        __syncthreads();
+    }
+}
+
+template <typename T>
+int launch_absorb(void* out, const void* x, const void* w, int tokens, int heads, int n, int k, int64_t xs_t,
+                  int64_t xs_h, int64_t os_t, int64_t os_h, hipStream_t st) {
+    const int nt = k <= 128 ? 4 : 1;                          // 64 registers of weight tiles per wave (k <= 128)
+    const int n_blocks = (n + AB_WAVES * 16 * nt - 1) / (AB_WAVES * 16 * nt);
+    // up to 64 tokens per workgroup (the weights are re-read once per token slice, from L2); fewer when the launch
+    // would otherwise leave compute units idle
+    int wg_tokens = 64;
+    while (wg_tokens > 16 && (int64_t)n_blocks * heads * ((tokens + wg_tokens - 1) / wg_tokens) < 256) wg_tokens >>= 1;
+    const int tz = (tokens + wg_tokens - 1) / wg_tokens;
+    if (tz > 65535) {
+        mf_set_error("mla_absorb_bmm: %d tokens exceed the grid limit", tokens);
+        return 1;
+    }
+    const dim3 grid(n_blocks, heads, tz);
+#define ABSORB_LAUNCH(KSV, NTV)                                                                                 \
+    hipLaunchKernelGGL((mla_absorb_bmm_kernel<T, KSV, NTV>), grid, dim3(AB_WAVES * 64), 0, st, (uint16_t*)out,   \
+                       (const uint16_t*)x, (const uint16_t*)w, tokens, n, wg_tokens, xs_t, xs_h, os_t, os_h)
+    switch (k) {
+        case 64: ABSORB_LAUNCH(2, 4); break;
+        case 128: ABSORB_LAUNCH(4, 4); break;
+        case 256:
+            hipLaunchKernelGGL((mla_absorb_bmm_lds_kernel<T, 8>), grid, dim3(AB_WAVES * 64), 0, st, (uint16_t*)out,
+                               (const uint16_t*)x, (const uint16_t*)w, tokens, n, wg_tokens, xs_t, xs_h, os_t, os_h);
+            break;
+        default:
+            hipLaunchKernelGGL((mla_absorb_bmm_lds_kernel<T, 16>), grid, dim3(AB_WAVES * 64), 0, st, (uint16_t*)out,
+                               (const uint16_t*)x, (const uint16_t*)w, tokens, n, wg_tokens, xs_t, xs_h, os_t, os_h);
+            break;
+    }
+#undef ABSORB_LAUNCH
+    return MF_LAUNCH_CHECK();
+}
+
 }  // namespace
 
 extern "C" size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads, int max_context) {
@@ -732,4 +920,28 @@ extern "C" int mf_mla_paged_attention_decode(void* out, const void* query, const
                                 max_blocks_per_seq, num_blocks, scale, q_row_stride, workspace, st);
     return launch_mla<FP16>(out, query, latent_cache, block_tables, context_lens, batch, n_heads, block_size,
                             max_blocks_per_seq, num_blocks, scale, q_row_stride, workspace, st);
+}
+
+extern "C" int mf_mla_absorb_bmm(void* out, const void* x, const void* w, int tokens, int heads, int n, int k,
+                                 int64_t x_token_stride, int64_t x_head_stride, int64_t out_token_stride,
+                                 int64_t out_head_stride, int dtype, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "mla_absorb_bmm: dtype must be bf16 or fp16");
+    MF_REQUIRE(tokens >= 0 && heads >= 0, "mla_absorb_bmm: negative size");
+    if (tokens == 0 || heads == 0) return 0;
+    MF_REQUIRE(out && x && w, "mla_absorb_bmm: null argument");
+    MF_REQUIRE(k == 64 || k == 128 || k == 256 || k == 512, "mla_absorb_bmm: k = %d not supported (64, 128, 256, 512)", k);
+    MF_REQUIRE(n > 0 && n % 16 == 0, "mla_absorb_bmm: n (%d) must be a positive multiple of 16", n);
+    MF_REQUIRE(heads <= 65535, "mla_absorb_bmm: at most 65535 heads");
+    MF_REQUIRE(x_head_stride >= k && x_token_stride >= k && x_head_stride % 8 == 0 && x_token_stride % 8 == 0,
+               "mla_absorb_bmm: x strides must be >= k and multiples of 8 elements");
+    MF_REQUIRE(out_head_stride >= n && out_token_stride >= n && out_head_stride % 8 == 0 && out_token_stride % 8 == 0,
+               "mla_absorb_bmm: out strides must be >= n and multiples of 8 elements");
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0,
+               "mla_absorb_bmm: x / w / out must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MF_BF16)
+        return launch_absorb<BF16>(out, x, w, tokens, heads, n, k, x_token_stride, x_head_stride, out_token_stride,
+                                   out_head_stride, st);
+    return launch_absorb<FP16>(out, x, w, tokens, heads, n, k, x_token_stride, x_head_stride, out_token_stride,
+                               out_head_stride, st);
 }

@@ -6,6 +6,7 @@ from .layers import (AllQuantLinearInferCell, ColumnParallelLinear, Linear, QKVP
                      RowParallelLinear, WeightQuantLinearCell)
 from .mlp import MLP, LlamaFeedForward
 from .moe import GroupedMLP, MoELayer, QuantGroupedMLP, SharedExpertMLP, TopKRouter
+from .multi_latent_attention import MLASelfAttention, MLASelfAttentionSubmodules, MLATransformerConfig
 from .norm import LlamaRMSNorm, RMSNorm
 from .paged_attention_mgr import PagedAttentionMgr, QuantPagedAttentionMgr
 from .rotary import FreqsMgr, Llama3RotaryEmbedding, RotaryEmbedding, YaRNScalingRotaryEmbedding

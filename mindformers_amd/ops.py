@@ -245,6 +245,28 @@ def mla_paged_attention(query, latent_cache, block_tables, context_lens, n_heads
     return out
 
 
+def mla_absorb_bmm(x, w, out=None):
+    """Per-head projection out[t, h, :] = x[t, h, :] . w[h]^T (multi_latent_attention.py:434-448, :228-231):
+    x [T, H, K] and out [T, H, N] may be strided views with a unit last stride (a slice of a wider projection
+    output / of the attention query), w [H, N, K] contiguous."""
+    lib = _lib.load()
+    dev = _dev_of(x, w, out)
+    _need(x.dim() == 3 and w.dim() == 3 and w.is_contiguous(), "x must be [T, H, K], w a contiguous [H, N, K]")
+    t, h, k = x.shape
+    _need(w.shape[0] == h and w.shape[2] == k, f"w is {tuple(w.shape)}, x has {h} heads of {k}")
+    n = w.shape[1]
+    _need(x.dtype in _ACT and w.dtype == x.dtype, "x and w must be bf16/fp16 and agree")
+    _need(x.stride(2) == 1, "x needs a unit last stride")
+    if out is None:
+        out = torch.empty((t, h, n), dtype=x.dtype, device=dev)
+    _need(tuple(out.shape) == (t, h, n) and out.dtype == x.dtype and out.stride(2) == 1, "out must be a [T, H, N] view")
+    if t == 0 or h == 0:
+        return out
+    check(lib.mf_mla_absorb_bmm(ptr(out), ptr(x), ptr(w), t, h, n, k, x.stride(0), x.stride(1), out.stride(0),
+                                out.stride(1), dtype_code(x.dtype), stream_ptr(dev)), "mf_mla_absorb_bmm")
+    return out
+
+
 # --------------------------------------------------------------------------------------------- int8 KV cache
 def _kv_quant_params(scale, offset, row, dev):
     _need(isinstance(scale, torch.Tensor) and scale.dtype == torch.float32 and scale.numel() == 2 * row and

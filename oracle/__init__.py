@@ -20,6 +20,9 @@ Pinning status of each function (what fixes it besides its own formula):
                            causal_prefill_attention (tests); the golden prefill vectors through the cache
   mla_paged_attention_     its reduction to paged_attention_decode (pinned above) with one kv head: equal
    decode                  when v_dim = Dk, and its first v_dim columns otherwise (tests)
+  mla_self_attention_      the layer around it (oracle/mla.py): the decode form (absorbed weights, latent cache)
+   decode / _prefill       against the prefill form (up-projected keys / values: the definition) on the same
+                           tokens (tests); the pieces underneath are the pinned functions of this list
   rope tables / apply      reference vectors (rotary.npz: default, Llama3, YaRN; prefill+decode)
   rms_norm / layer_norm    reference vectors (norm.npz)
   silu_mul                 reference vectors (activation.npz)
@@ -55,3 +58,4 @@ from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,
                   grouped_matmul)
 from .layer import decode_layer_w8a16, decode_layer_w8a8
+from .mla import mla_project, mla_self_attention_decode, mla_self_attention_prefill

@@ -1209,3 +1209,42 @@ def test_grouped_w8a8_accumulators_bit_exact(counts, n, k):
         assert np.array_equal(got_acc[r0:r1], ref), ex
         yref = ref.astype(np.float64) * xs_n[r0:r1, None] * ws[ex].astype(np.float64)[None, :]
         assert np.all(np.abs(got_y[r0:r1] - yref) <= 1.01 * EPS[torch.bfloat16] * np.abs(yref) + 1e-6), ex
+
+
+# ------------------------------------------------------------------------------------------- MLA absorbed projections
+@pytest.mark.parametrize("dtype,t,h,k,n,strided", [
+    (torch.bfloat16, 64, 128, 128, 512, True),     # query side at DeepSeek-V3 geometry: q_no_pe inside [T, H, 192]
+    (torch.bfloat16, 64, 128, 512, 128, False),    # output side
+    (torch.float16, 5, 3, 512, 128, False),
+    (torch.bfloat16, 33, 16, 64, 48, True),        # ragged token tile, channel count not a multiple of 64
+    (torch.float16, 257, 2, 256, 16, False),       # few heads: the tokens are cut over workgroups
+    (torch.bfloat16, 1, 128, 128, 512, True),
+])
+def test_mla_absorb_bmm_vs_oracle(dtype, t, h, k, n, strided):
+    """out[t, h, :] = x[t, h, :] . w[h]^T against float64, x and out as strided slices of wider buffers (the query
+    projection [T, H, k + 64] and the attention query [T, H, n + 64]); the columns beside the output slice stay."""
+    rng = np.random.default_rng(t * 131 + n)
+    pad = 64 if strided else 0
+    xw = rounded(rng.normal(size=(t, h, k + pad)), dtype)
+    w = rounded(rng.normal(0, 0.1, (h, n, k)), dtype)
+    xd = dev(xw, dtype)
+    out_w = torch.full((t, h, n + pad), 7.0, dtype=dtype, device="cuda")
+    got = ops.mla_absorb_bmm(xd[..., :k], dev(w, dtype), out=out_w[..., :n])
+    x64, w64 = xw[..., :k].astype(np.float64), w.astype(np.float64)
+    ref = np.einsum("thk,hnk->thn", x64, w64)
+    mag = np.einsum("thk,hnk->thn", np.abs(x64), np.abs(w64))
+    assert_within(to_np(got), ref, np.abs(ref), dtype, ulps=1.0, extra=2.0 ** -18 * mag + 1e-9, what="absorb bmm")
+    if pad:
+        assert bool((out_w[..., n:] == 7.0).all())
+    fresh = ops.mla_absorb_bmm(xd[..., :k], dev(w, dtype))
+    assert fresh.is_contiguous() and torch.equal(fresh, out_w[..., :n])
+
+
+def test_mla_absorb_bmm_rejects_bad_operands():
+    x = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.mla_absorb_bmm(x, torch.zeros(2, 16, 64, dtype=torch.bfloat16, device="cuda"))      # k mismatch
+    with pytest.raises(RuntimeError):
+        ops.mla_absorb_bmm(x[..., :96], torch.zeros(2, 16, 96, dtype=torch.bfloat16, device="cuda"))   # k = 96
+    with pytest.raises(RuntimeError):
+        ops.mla_absorb_bmm(x, torch.zeros(2, 24, 128, dtype=torch.bfloat16, device="cuda"))     # n not a multiple of 16

@@ -964,3 +964,151 @@ def test_moe_layer_w8a8_experts_vs_oracle(granularity):
     ref = _r(O.moe_unpermute(_r(y, "bf16"), row_map, wgt), "bf16")
     assert np.abs(out - ref).max() <= 6 * EPS[BF] * np.abs(ref).max()
     assert np.mean(np.abs(out - ref) > 2 * EPS[BF] * np.abs(ref) + 1e-6) < 0.02
+
+
+# ------------------------------------------------------------------------------------------- multi-latent attention layer
+def _mla_module_and_params(rng, hidden, n, q_lora, rank=512, nope=128, rope=64, vd=128, rope_type="yarn"):
+    from mindformers_amd.modules import MLASelfAttention, MLATransformerConfig
+    cfg = MLATransformerConfig(hidden_size=hidden, num_attention_heads=n, q_lora_rank=q_lora, kv_lora_rank=rank,
+                               qk_head_dim=nope, qk_pos_emb_head_dim=rope, v_head_dim=vd, rope_type=rope_type,
+                               layernorm_epsilon=1e-6, compute_dtype="bfloat16", params_dtype="bfloat16")
+    net = MLASelfAttention(cfg, layer_number=1)
+    p = {}
+
+    def fill(cell, key, std):
+        w = rounded(rng.normal(0, std, tuple(cell.weight.shape)), BF)
+        cell.weight.data.copy_(dev(w, BF))
+        p[key] = w
+    if q_lora:
+        fill(net.linear_qkv_down_proj, "qkv_down_w", hidden ** -0.5)
+        fill(net.linear_q_up_proj, "q_up_w", q_lora ** -0.5)
+        g = (1 + 0.1 * rng.normal(size=q_lora)).astype(np.float32)
+        net.q_layernorm.weight.data.copy_(torch.from_numpy(g))
+        p["q_norm"] = g
+    else:
+        fill(net.linear_q_proj, "q_w", hidden ** -0.5)
+        fill(net.linear_kv_down_proj, "kv_down_w", hidden ** -0.5)
+    fill(net.linear_kv_up_proj, "kv_up_w", rank ** -0.5)
+    fill(net.linear_proj, "proj_w", (n * vd) ** -0.5)
+    g = (1 + 0.1 * rng.normal(size=rank)).astype(np.float32)
+    net.kv_layernorm.weight.data.copy_(torch.from_numpy(g))
+    p["kv_norm"] = g
+    ocfg = dict(n_head=n, qk_head_dim=nope, qk_pos_emb_head_dim=rope, kv_lora_rank=rank, v_head_dim=vd,
+                q_lora_rank=q_lora, eps=1e-6, rotary_scaling_factor=cfg.rotary_scaling_factor, mscale=cfg.mscale)
+    return net, cfg, p, ocfg
+
+
+@pytest.mark.parametrize("hidden,n,q_lora,rope_type", [(7168, 128, 1536, "yarn"), (1024, 16, None, "rope")])
+def test_mla_self_attention_prefill_then_decode_vs_oracle(hidden, n, q_lora, rope_type):
+    """MLASelfAttention at the DeepSeek-V3 geometry (128 heads, 512 + 64 latent, 128 + 64 query heads, q_lora 1536) and
+    at a small one without the query low-rank path: a prefill of three prompts writes the latent cache and returns the
+    up-projected attention, one decode step per sequence then runs on absorbed weights over that cache.  Both against
+    the float64 restatement rounded to bf16 where the module stores bf16; the caches must agree row for row."""
+    from mindformers_amd.modules import BlockTables
+    rng = np.random.default_rng(hidden + n)
+    net, cfg, p, ocfg = _mla_module_and_params(rng, hidden, n, q_lora, rope_type=rope_type)
+    rank, rope = cfg.kv_lora_rank, cfg.qk_pos_emb_head_dim
+    lens = [70, 5, 130]
+    bs = 32
+    need = [(l + 1 + bs - 1) // bs for l in lens]
+    nb = sum(need) + 2
+    perm = rng.permutation(nb)
+    tables = -np.ones((len(lens), max(need)), np.int32)
+    pos = 0
+    for i, k in enumerate(need):
+        tables[i, :k] = perm[pos:pos + k]
+        pos += k
+    cache = torch.zeros(nb, bs, 1, rank + rope, dtype=BF, device="cuda")
+    cache_ref = np.zeros((nb, bs, 1, rank + rope))
+    cos_t, sin_t = net.rotary_pos_emb.get_cos_sin_for_prefill()
+    # ---- prefill
+    total = sum(lens)
+    x = rounded(rng.normal(size=(total, hidden)), BF)
+    positions = np.concatenate([np.arange(l) for l in lens])
+    slots = np.concatenate([[tables[i, j // bs] * bs + j % bs for j in range(l)] for i, l in enumerate(lens)]).astype(np.int32)
+    pos_t = torch.from_numpy(positions).cuda()
+    cos, sin = cos_t.index_select(0, pos_t), sin_t.index_select(0, pos_t)
+    net.is_prefill = True
+    out = net(dev(x, BF), None, rotary_pos_cos=cos, rotary_pos_sin=sin, slot_mapping=dev(slots, torch.int32),
+              actual_seq_qlen=torch.tensor(np.cumsum(lens), dtype=torch.int32, device="cuda"),
+              actual_seq_kvlen=torch.tensor(np.cumsum(lens), dtype=torch.int32, device="cuda"), key_cache=cache)
+    ref = O.mla_self_attention_prefill(x, p, ocfg, cache_ref, slots, lens, to_np(cos), to_np(sin), act_dtype="bf16")
+    got = to_np(out)
+    assert got.shape == (total, hidden)
+    scale = np.abs(ref).max()
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 2e-2, np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert np.abs(got - ref).max() < 0.06 * scale, (np.abs(got - ref).max(), scale)
+    # the latent rows: one bf16 step at most apart (the norm output may round either way), untouched rows zero
+    c_got, c_ref = to_np(cache).reshape(-1, rank + rope), cache_ref.reshape(-1, rank + rope)
+    assert np.abs(c_got[slots] - c_ref[slots]).max() <= 4 * EPS[BF] * np.abs(c_ref[slots]).max()
+    keep = np.ones(c_got.shape[0], bool)
+    keep[slots] = False
+    assert not c_got[keep].any()
+    # ---- one decode step per sequence over the cache the device wrote (the oracle continues on the device's rows)
+    cache_ref = to_np(cache).astype(np.float64)
+    b = len(lens)
+    xd = rounded(rng.normal(size=(b, hidden)), BF)
+    new_lens = np.asarray(lens, np.int32) + 1
+    dslots = np.asarray([tables[i, lens[i] // bs] * bs + lens[i] % bs for i in range(b)], np.int32)
+    pos_t = torch.from_numpy(np.asarray(lens, np.int64)).cuda()
+    cos, sin = net.rotary_pos_emb.get_cos_sin_for_decode(pos_t)
+    net.is_prefill = False
+    out = net(dev(xd, BF), None, rotary_pos_cos=cos, rotary_pos_sin=sin, batch_valid_length=dev(new_lens, torch.int32),
+              block_tables=dev(tables, torch.int32), slot_mapping=dev(dslots, torch.int32), key_cache=cache)
+    ref = O.mla_self_attention_decode(xd, p, ocfg, cache_ref, tables, new_lens, dslots, to_np(cos), to_np(sin),
+                                      act_dtype="bf16")
+    got = to_np(out)
+    assert got.shape == (b, hidden)
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 2e-2, np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert np.abs(got - ref).max() < 0.06 * np.abs(ref).max()
+    c_got = to_np(cache).reshape(-1, rank + rope)
+    assert np.abs(c_got[dslots] - cache_ref.reshape(-1, rank + rope)[dslots]).max() <= 4 * EPS[BF] * np.abs(c_got[dslots]).max()
+    # the decode step equals the last row of a prefill over the same tokens (absorbed = up-projected), on the device
+    # too: sequence 1 (5 + 1 tokens) run again as one prompt
+    i = 1
+    xs = np.concatenate((x[lens[0]:lens[0] + lens[1]], xd[i:i + 1]))
+    pos_t = torch.arange(lens[i] + 1, device="cuda")
+    cos, sin = cos_t.index_select(0, pos_t), sin_t.index_select(0, pos_t)
+    net.is_prefill = True
+    seq = torch.tensor([lens[i] + 1], dtype=torch.int32, device="cuda")
+    again = net(dev(xs, BF), None, rotary_pos_cos=cos, rotary_pos_sin=sin, slot_mapping=None, actual_seq_qlen=seq,
+                actual_seq_kvlen=seq, key_cache=None)
+    d = to_np(again[-1]) - got[i]
+    assert np.linalg.norm(d) / np.linalg.norm(got[i]) < 2e-2
+
+
+def test_mla_self_attention_with_quantized_projections():
+    """The RTN quantizer converts the layer's projections (W8A16) and leaves linear_kv_up_proj, whose weight the
+    absorbed projections read, as a float cell; the decode step stays close to the float layer's."""
+    from mindformers_amd.modules import ColumnParallelLinear, WeightQuantLinearCell
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    rng = np.random.default_rng(5)
+    net, cfg, p, ocfg = _mla_module_and_params(rng, 1024, 16, 384)
+    rank, rope, bs = cfg.kv_lora_rank, cfg.qk_pos_emb_head_dim, 32
+    lens = np.asarray([40, 7], np.int32)
+    tables = np.asarray([[1, 0], [2, -1]], np.int32)
+    cache = dev(rounded(rng.normal(size=(4, bs, 1, rank + rope)), BF), BF)
+    x = dev(rounded(rng.normal(size=(2, 1024)), BF), BF)
+    slots = dev(np.asarray([tables[i, (lens[i] - 1) // bs] * bs + (lens[i] - 1) % bs for i in range(2)], np.int32), torch.int32)
+    cos, sin = net.rotary_pos_emb.get_cos_sin_for_decode(torch.from_numpy(lens.astype(np.int64) - 1).cuda())
+    args = dict(rotary_pos_cos=cos, rotary_pos_sin=sin, batch_valid_length=dev(lens, torch.int32),
+                block_tables=dev(tables, torch.int32), slot_mapping=slots)
+    net.is_prefill = False
+    ref = net(x, None, key_cache=cache.clone(), **args)
+    q = AutoQuantizer.from_config({"quant_method": "rtn", "weight_dtype": "int8",
+                                   "modules_to_not_convert": ["linear_kv_up_proj"]})
+    q.preprocess_model(net)
+    q.postprocess_model(net)
+    assert isinstance(net.linear_qkv_down_proj, WeightQuantLinearCell) and isinstance(net.linear_proj, WeightQuantLinearCell)
+    assert isinstance(net.linear_kv_up_proj, ColumnParallelLinear)
+    out = net(x, None, key_cache=cache.clone(), **args)
+    d = (out.float() - ref.float()).norm() / ref.float().norm()
+    assert float(d) < 0.05, float(d)
+    # a quantized linear_kv_up_proj cannot be absorbed: the layer says so
+    net2, *_ = _mla_module_and_params(rng, 1024, 16, 384)
+    q2 = AutoQuantizer.from_config({"quant_method": "rtn", "weight_dtype": "int8"})
+    q2.preprocess_model(net2)
+    q2.postprocess_model(net2)
+    net2.is_prefill = False
+    with pytest.raises(NotImplementedError):
+        net2(x, None, key_cache=cache.clone(), **args)

@@ -294,3 +294,68 @@ def test_float32_host_layer_follows_the_float64_oracle():
     assert np.array_equal(kc32.numpy().reshape(-1, row)[~written], kc.reshape(-1, row)[~written])
     assert np.abs(kc32.numpy() - kc64).max() <= 2 * 2.0 ** -8 * np.abs(kc64).max()
     assert np.abs(vc32.numpy() - vc64).max() <= 2 * 2.0 ** -8 * np.abs(vc64).max()
+
+
+# ------------------------------------------------------------------------------------------- multi-latent layer
+def _mla_case(rng, n=4, nope=16, rope=8, rank=32, vd=16, hidden=64, q_lora=24):
+    cfg = dict(n_head=n, qk_head_dim=nope, qk_pos_emb_head_dim=rope, kv_lora_rank=rank, v_head_dim=vd,
+               q_lora_rank=q_lora, eps=1e-6, rotary_scaling_factor=40.0, mscale=1.0)
+    p = dict(q_norm=1 + 0.1 * rng.normal(size=q_lora or 1), kv_norm=1 + 0.1 * rng.normal(size=rank),
+             kv_up_w=rng.normal(0, 0.3, (n * (nope + vd), rank)), proj_w=rng.normal(0, 0.3, (hidden, n * vd)))
+    if q_lora:
+        p["qkv_down_w"] = rng.normal(0, 0.3, (q_lora + rank + rope, hidden))
+        p["q_up_w"] = rng.normal(0, 0.3, (n * (nope + rope), q_lora))
+    else:
+        p["q_w"] = rng.normal(0, 0.3, (n * (nope + rope), hidden))
+        p["kv_down_w"] = rng.normal(0, 0.3, (rank + rope, hidden))
+    return cfg, p
+
+
+@pytest.mark.parametrize("q_lora", [24, None])
+def test_mla_decode_with_absorbed_weights_equals_the_prefill_definition(q_lora):
+    """multi_latent_attention.py:434-448 folds the key up-projection into the query and applies the value
+    up-projection to the attention output; :405-432 (prefill) up-projects keys and values and runs ordinary
+    attention.  Both are the same function of the tokens: the decode step of a sequence's last token over a cache
+    that the earlier tokens filled must equal the last row of a prefill over the whole sequence."""
+    rng = np.random.default_rng(17)
+    cfg, p = _mla_case(rng, q_lora=q_lora)
+    lens = [6, 1, 9]
+    bs, rope = 4, cfg["qk_pos_emb_head_dim"]
+    dk = cfg["kv_lora_rank"] + rope
+    need = [(l + bs - 1) // bs for l in lens]
+    nb = sum(need) + 1
+    perm = rng.permutation(nb)
+    tables = -np.ones((len(lens), max(need)), np.int32)
+    pos = 0
+    for i, k in enumerate(need):
+        tables[i, :k] = perm[pos:pos + k]
+        pos += k
+    total = sum(lens)
+    hidden = rng.normal(size=(total, 64))
+    inv = O.rope_inv_freq_default(rope, 10000.0)
+    cos_t, sin_t = O.rope_cos_sin_table(inv, 16)
+    positions = np.concatenate([np.arange(l) for l in lens])
+    cos, sin = cos_t[positions], sin_t[positions]
+    starts = np.cumsum([0] + lens)
+    slots = np.concatenate([[tables[i, j // bs] * bs + j % bs for j in range(l)] for i, l in enumerate(lens)]).astype(np.int32)
+    # the definition: prefill over whole sequences
+    cache_pf = np.zeros((nb, bs, 1, dk))
+    full = O.mla_self_attention_prefill(hidden, p, cfg, cache_pf, slots, lens, cos, sin)
+    # decode: earlier tokens through prefill (only their cache rows matter), the last token of each as a decode step
+    cache = np.zeros((nb, bs, 1, dk))
+    early = np.concatenate([np.arange(starts[i], starts[i + 1] - 1) for i in range(len(lens))]).astype(np.int64)
+    if len(early):
+        O.mla_self_attention_prefill(hidden[early], p, cfg, cache, slots[early], [l - 1 for l in lens if l > 1],
+                                     cos[early], sin[early])
+    last = starts[1:] - 1
+    dec = O.mla_self_attention_decode(hidden[last], p, cfg, cache, tables, np.asarray(lens, np.int32), slots[last],
+                                      cos[last], sin[last])
+    assert np.allclose(cache, cache_pf, rtol=0, atol=1e-12)
+    assert np.allclose(dec, full[last], rtol=1e-10, atol=1e-10)
+    # negative control: the two halves of linear_kv_up_proj swapped must not pass
+    bad = dict(p)
+    n, nope = cfg["n_head"], cfg["qk_head_dim"]
+    bad["kv_up_w"] = np.concatenate((p["kv_up_w"][n * nope:], p["kv_up_w"][: n * nope]))
+    dec_bad = O.mla_self_attention_decode(hidden[last], bad, cfg, cache.copy(), tables, np.asarray(lens, np.int32),
+                                          slots[last], cos[last], sin[last])
+    assert not np.allclose(dec_bad, full[last], rtol=1e-3, atol=1e-3)

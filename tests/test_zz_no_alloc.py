@@ -44,15 +44,19 @@ def test_static_scratch_decode_equals_the_workspace_entry_point_twice_in_a_row()
     # first call: 12 sequences, up to 16 partitions each, one without context
     lens = rng.integers(300, 4096, 12)
     lens[3] = 0
-    out, ref, need = _both(lib, rng, 12, 32, 8, 128, 128, np.maximum(lens, 1), 32, torch.bfloat16)
+    out, ref, need = _both(lib, rng, 12, 32, 8, 128, 128, lens, 32, torch.bfloat16)
     assert need > 0 and torch.equal(out, ref)
+    assert not out[3].any() and out[2].any()                   # the empty sequence's row is zeros
     # second call, smaller in every respect (batch, heads, partitions): the array still holds the first call's partials
     lens = rng.integers(100, 900, 3)
+    lens[1] = 0                                                # reads no partition: stale partials must not show
     out, ref, need = _both(lib, rng, 3, 8, 2, 64, 16, lens, 64, torch.float16)
     assert need > 0 and torch.equal(out, ref)
+    assert not out[1].any()
     # a single-partition shape uses no partials at all
-    out, ref, need = _both(lib, rng, 2, 4, 4, 32, 16, [5, 200], 16, torch.float16)
+    out, ref, need = _both(lib, rng, 3, 4, 4, 32, 16, [5, 0, 200], 16, torch.float16)
     assert need == 0 and torch.equal(out, ref)
+    assert not out[1].any()                                    # the single-partition path zeroes empty rows itself
 
 
 def test_static_scratch_decode_refuses_shapes_beyond_the_array():
