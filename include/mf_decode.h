@@ -248,6 +248,11 @@ int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, int layout, 
 /* out = a + b (residual add, llama_transformer.py:1057,1067). */
 int mf_add(void* out, const void* a, const void* b, int64_t n, int dtype, void* stream);
 
+/* out[m, k] = x[m, k] * scale[k], rounded once: the activation multiplier of an outlier-suppression pair (smooth /
+ * awq, mindformers/utils/quantization_config.py:413-414) in front of a weight-only GEMM, where no activation
+ * quantisation kernel is there to carry it.  cols % 8 == 0. */
+int mf_scale_columns(void* out, const void* x, const float* scale, int64_t rows, int cols, int dtype, void* stream);
+
 /* ---- quantized linear ----------------------------------------------------------------------------- */
 
 /* The W8A16 kernels stream the int8 weight in a tiled order (16 output channels x 64 input channels per
@@ -268,6 +273,22 @@ size_t mf_w8a16_workspace_bytes(int m, int n, int k);
  * K % 8 == 0. */
 int mf_w8a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
                   const void* residual, int m, int n, int k, int dtype, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
+/* 4-bit weights, weight-only (A16W4): WeightQuantBatchMatmul behind the golden-stick cell that
+ * PtqConfig(weight_dtype="qint4x2", weight_quant_granularity in {per_channel, per_group}, group_size in {0, 64, 128})
+ * selects (mindformers/utils/quantization_config.py:408-416,448-453; mindformers/modules/quantizers/
+ * ptq_quantizer.py:52-59).  mf_w4a16_pack_weight turns w [n, k] int8 holding the 4-bit values (-8 .. 7, one per byte)
+ * into 512-byte tiles of 16 channels x 64 columns in matrix-instruction operand order ([k-step][tile], nibbles
+ * q + 8); mf_w4a16_packed_bytes gives the size.  mf_w4a16_gemm: y = x . (w * scale)^T (+ bias) (+ residual) with
+ * scale [n] (group_size 0) or [k / group_size][n] (one scale per channel and group of columns).  The products of a
+ * group are summed in fp32 on the exact integer weights, then multiplied by the group's scale.  k a multiple of 64
+ * and of group_size; n a multiple of 4 with groups.  Workspace: mf_w4a16_workspace_bytes. */
+size_t mf_w4a16_packed_bytes(int n, int k);
+int mf_w4a16_pack_weight(void* packed, const int8_t* w, int n, int k, void* stream);
+size_t mf_w4a16_workspace_bytes(int m, int n, int k, int group_size);
+int mf_w4a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
+                  const void* residual, int m, int n, int k, int group_size, int dtype, void* workspace,
                   size_t workspace_bytes, void* stream);
 
 /* A row-parallel projection with its residual add, fused with the RMSNorm that follows it in the layer

@@ -42,9 +42,14 @@ SIGNATURES = {
     "mf_rmsnorm": (_I, [_P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P]),
     "mf_silu_mul": (_I, [_P, _P, _I, _I, _I, _I, _P]),
     "mf_add": (_I, [_P, _P, _P, _L, _I, _P]),
+    "mf_scale_columns": (_I, [_P, _P, _P, _L, _I, _I, _P]),
     "mf_w8a16_packed_bytes": (_Z, [_I, _I]),
     "mf_w8a16_pack_weight": (_I, [_P, _P, _I, _I, _P]),
     "mf_w8a16_workspace_bytes": (_Z, [_I, _I, _I]),
+    "mf_w4a16_packed_bytes": (_Z, [_I, _I]),
+    "mf_w4a16_pack_weight": (_I, [_P, _P, _I, _I, _P]),
+    "mf_w4a16_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "mf_w4a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm_add_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_qkv_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _I, _P, _Z, _P]),

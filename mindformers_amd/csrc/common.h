@@ -279,6 +279,30 @@ __device__ __forceinline__ f16x8 dequant8<FP16>(uint32_t lo, uint32_t hi) {
     return v;
 }
 
+// 8 unsigned nibbles holding q + 8 (q in -8 .. 7; nibble i = element i) -> 8 elements of T, exact.
+template <typename T>
+__device__ __forceinline__ typename T::vec8 dequant8_u4(uint32_t w);
+
+template <>
+__device__ __forceinline__ bf16x8 dequant8_u4<BF16>(uint32_t w) {
+    const uint32_t even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu;   // elements 0 2 4 6 / 1 3 5 7 as bytes
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float f0 = (float)((even >> (8 * i)) & 0xffu) - 8.0f;
+        const float f1 = (float)((odd >> (8 * i)) & 0xffu) - 8.0f;
+        v[i] = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);   // high halves: exact
+    }
+    return bitcast<bf16x8>(v);
+}
+template <>
+__device__ __forceinline__ f16x8 dequant8_u4<FP16>(uint32_t w) {
+    f16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (_Float16)((float)((w >> (4 * i)) & 0xfu) - 8.0f);
+    return v;
+}
+
 // Transposing 64-bit LDS read (ds_read_b64_tr_b16).  Within every group of 16 lanes, lane j names four consecutive
 // 16-bit values M[j][0..3]; lane i receives M[(i >> 2) + 4 e][i & 3] for e = 0..3.
 typedef __attribute__((ext_vector_type(4))) short s16x4;

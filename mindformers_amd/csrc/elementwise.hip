@@ -2,6 +2,8 @@
 // residual add), SiLU*mul, residual add, per-token dynamic int8 quantisation.
 // All are single-pass, HBM-bound, 16-byte lane accesses; one workgroup per row where a row reduction is
 // needed (the row is held in registers between the reduction and the scaled write).
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -124,6 +126,33 @@ __global__ void add_kernel(uint16_t* __restrict__ out, const uint16_t* __restric
     for (int64_t i = (nvec << 3) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
          i += (int64_t)gridDim.x * blockDim.x)
         out[i] = T::from_float(T::to_float(a[i]) + T::to_float(b[i]));
+}
+
+// out[m, k] = round_T(float32(x[m, k] * scale[k])): the activation side of an outlier-suppression pair (the multiplier that the
+// weights were divided by offline) in front of a weight-only GEMM.  8 elements per thread.
+template <typename T>
+__global__ void scale_columns_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
+                                     const float* __restrict__ scale, int64_t rows, int cols) {
+    const int cvec = cols >> 3;
+    const int64_t nvec = rows * cvec;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(i % cvec) * 8;
+        float v[8];
+        unpack8<T>(*(const u32x4*)(x + 8 * i), v);
+        const f32x4 s0 = *(const f32x4*)(scale + c), s1 = *(const f32x4*)(scale + c + 4);
+        u32x4 o;
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            p[j] = __fmul_rn(v[j], j < 4 ? s0[j] : s1[j - 4]);
+            // the float32 product is the value that is rounded to T: keep the compiler from folding the multiply
+            // into a mixed-precision instruction that rounds the exact product once (differs on near-ties)
+            asm volatile("" : "+v"(p[j]));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = pack2<T>(p[2 * j], p[2 * j + 1]);
+        *(u32x4*)(out + 8 * i) = o;
+    }
 }
 
 // Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
@@ -389,6 +418,24 @@ extern "C" int mf_add(void* out, const void* a, const void* b, int64_t n, int dt
     else
         hipLaunchKernelGGL(add_kernel<FP16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
                            (const uint16_t*)a, (const uint16_t*)b, n);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_scale_columns(void* out, const void* x, const float* scale, int64_t rows, int cols, int dtype,
+                                void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "scale_columns: dtype must be bf16 or fp16");
+    MF_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, "scale_columns: cols (%d) must be a positive multiple of 8", cols);
+    if (rows == 0) return 0;
+    MF_REQUIRE(out && x && scale, "scale_columns: null argument");
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)x | (uintptr_t)scale) & 15) == 0, "scale_columns: 16-byte alignment");
+    const int64_t nvec = rows * (cols >> 3);
+    const int blocks = (int)std::min<int64_t>((nvec + 255) / 256, 65535);
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(scale_columns_kernel<BF16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)x, scale, rows, cols);
+    else
+        hipLaunchKernelGGL(scale_columns_kernel<FP16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                           (const uint16_t*)x, scale, rows, cols);
     return MF_LAUNCH_CHECK();
 }
 

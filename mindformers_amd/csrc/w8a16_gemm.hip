@@ -52,7 +52,7 @@ __device__ __forceinline__ void store4(uint16_t* y, const uint16_t* bias, const 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         if (n + i < N) {
-            float v = dequant_bias<T>(acc[i], scale[n + i], bias, n + i);
+            float v = dequant_bias<T>(acc[i], scale ? scale[n + i] : 1.0f, bias, n + i);   // no scale: already applied
             if (residual) v = __fadd_rn(T::to_float(T::from_float(v)), T::to_float(residual[row_off + n + i]));
             o[i] = v;
         } else {
@@ -77,8 +77,8 @@ __device__ __forceinline__ void store_gated(uint16_t* y, const uint16_t* bias, c
     float o[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        float gv = dequant_bias<T>(acc[2 * h], scale[n + 2 * h], bias, n + 2 * h);
-        float uv = dequant_bias<T>(acc[2 * h + 1], scale[n + 2 * h + 1], bias, n + 2 * h + 1);
+        float gv = dequant_bias<T>(acc[2 * h], scale ? scale[n + 2 * h] : 1.0f, bias, n + 2 * h);
+        float uv = dequant_bias<T>(acc[2 * h + 1], scale ? scale[n + 2 * h + 1] : 1.0f, bias, n + 2 * h + 1);
         gv = T::to_float(T::from_float(gv));
         uv = T::to_float(T::from_float(uv));
         o[h] = T::to_float(T::from_float(silu_f(gv))) * uv;
@@ -324,14 +324,24 @@ struct G4 {
     static_assert(XL * XWRITERS == 2 * MT && XWRITERS <= WAVES && XL <= 2, "bad split of the activation loads");
 };
 
-template <typename T, int MT, int WAVES, bool KTAIL>
+// W4: the weights are 4-bit (unsigned nibbles holding q + 8, q in -8 .. 7; a 16 x 64 tile is 512 bytes, lane (r, g)
+// holds the 16 nibbles of row r, columns 16g .. 16g + 15 in 8 bytes, nibble i = column 16g + i).  GROUP (64 or 128,
+// W4 only): one scale per channel and GROUP columns, gscale [K / GROUP][N]: the products of a group are summed in
+// fp32 on the exact integer weights and enter the total times the group's scale; the epilogue's per-channel scale is
+// then 1.  GROUP = 0: one scale per channel, applied in the epilogue.
+template <typename T, int MT, int WAVES, bool KTAIL, bool W4 = false, int GROUP = 0>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_kernel(
     uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
     const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated, int split_major) {
+    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split, int gated, int split_major,
+    const float* __restrict__ gscale = nullptr) {
     using vec8 = typename T::vec8;
     using C = G4<MT, WAVES>;
     constexpr int D = C::DEPTH;
+    static_assert(!W4 || !KTAIL, "4-bit weights: K is a multiple of 64");
+    static_assert(GROUP == 0 || (W4 && (GROUP == 64 || GROUP == 128)), "groups of 64 or 128 columns, 4-bit weights");
+    constexpr int TB = W4 ? GW_TILE_BYTES / 2 : GW_TILE_BYTES;  // bytes of a weight tile
+    using wreg_t = std::conditional_t<W4, u32x2, u32x4>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * C::XTILE];
 
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -346,14 +356,18 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
     const int n0 = nblock * C::BN + wv * 16;                  // first output channel of this wave
     const int m0 = blockIdx.z * C::XROWS;
 
-    f32x4 acc[MT];
+    f32x4 acc[MT], tot[GROUP ? MT : 1];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < (GROUP ? MT : 1); ++mt) tot[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int n_tiles_total = (N + 15) >> 4;
-    const uint8_t* wtile = wp + (int64_t)min(n0 >> 4, n_tiles_total - 1) * GW_TILE_BYTES;   // wave-uniform
-    const int64_t wstride = (int64_t)n_tiles_total * GW_TILE_BYTES;
-    const uint32_t wlane = lane * 16;
+    const uint8_t* wtile = wp + (int64_t)min(n0 >> 4, n_tiles_total - 1) * TB;               // wave-uniform
+    const int64_t wstride = (int64_t)n_tiles_total * TB;
+    const uint32_t wlane = lane * (TB / 64);
+    // group scales of this lane's 4 output channels (clamped inside the row for channels past N: never stored)
+    const float* gsl = GROUP ? gscale + min(n0 + 4 * g, N - 4) : nullptr;
     const uint8_t* xbase = (const uint8_t*)(x + (int64_t)m0 * K);                            // wave-uniform
     uint32_t xlane[C::XL];
     int xchunk8[C::XL];
@@ -372,11 +386,14 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
     // front of the first use of every register (a hand-written wait cannot stop the register allocator from copying a
     // register whose load is still in flight).  For its count to stay exact, the main loop is free of conditional
     // steps: it runs over whole groups of D steps, the remaining 0 .. D-1 steps follow it.
-    u32x4 wreg[D], xreg[D][C::XL];
+    wreg_t wreg[D];
+    u32x4 xreg[D][C::XL];
+    f32x4 greg[GROUP ? D : 1];
     auto issue = [&](auto setc, int s) {
         constexpr int S = decltype(setc)::value;
         const int sc = min(s, s_last);
-        wreg[S] = *(const u32x4*)(wtile + sc * wstride + wlane);
+        wreg[S] = *(const wreg_t*)(wtile + sc * wstride + wlane);
+        if constexpr (GROUP != 0) greg[S] = *(const f32x4*)(gsl + (int64_t)(sc * GW_KSTEP / GROUP) * N);
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
             uint32_t off = xlane[i] + (uint32_t)sc * (GW_KSTEP * 2);
@@ -429,11 +446,19 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
         __builtin_amdgcn_sched_barrier(0);
         stage_x(std::integral_constant<int, JN>{}, P ^ 1);
         vec8 wa[2];
-        wa[0] = dequant8<T>(wreg[J][0], wreg[J][1]);
-        wa[1] = dequant8<T>(wreg[J][2], wreg[J][3]);
+        f32x4 gs = {1.f, 1.f, 1.f, 1.f};
+        if constexpr (W4) {
+            wa[0] = dequant8_u4<T>(wreg[J][0]);
+            wa[1] = dequant8_u4<T>(wreg[J][1]);
+            if constexpr (GROUP != 0) gs = greg[J];
+        } else {
+            wa[0] = dequant8<T>(wreg[J][0], wreg[J][1]);
+            wa[1] = dequant8<T>(wreg[J][2], wreg[J][3]);
+        }
         // the conversion happens here, before the set is reloaded (sunk below the reload it would keep the old
         // registers alive next to the new ones, and the sets would no longer rotate in place)
         asm volatile("" : "+v"(wa[0]), "+v"(wa[1]));
+        if constexpr (GROUP != 0) asm volatile("" : "+v"(gs));
         __builtin_amdgcn_sched_barrier(0);
         issue(jc, s + D);                                     // set J is free: weights converted, activations staged
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // this wave's LDS writes are done
@@ -445,6 +470,16 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[mt] = T::mfma16(wa[h], bitcast<vec8>(xb[P][mt][h]), acc[mt]);
+        if constexpr (GROUP != 0) {
+            if (GROUP == GW_KSTEP || (s & 1)) {               // the group's last step (splits begin on group borders)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) tot[mt][i] = __fmaf_rn(acc[mt][i], gs[i], tot[mt][i]);
+                    acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
     static_assert(D % 2 == 0 && D >= 4, "the two LDS stages alternate with the register sets");
@@ -462,19 +497,20 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
     for (int mt = 0; mt < MT; ++mt) {
         const int m = m0 + 16 * mt + r;
         if (m >= M) continue;
+        const f32x4 res = GROUP ? tot[mt] : acc[mt];
         if (partial) {
             float* p = partial + ((int64_t)split * M + m) * N + n;
             if (vec) {
-                *(f32x4*)p = acc[mt];
+                *(f32x4*)p = res;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (n + i < N) p[i] = acc[mt][i];
+                    if (n + i < N) p[i] = res[i];
             }
         } else if (gated) {
-            store_gated<T>(y, bias, scale, m, n, N, acc[mt]);
+            store_gated<T>(y, bias, scale, m, n, N, res);
         } else {
-            store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, acc[mt]);
+            store4<T>(y, bias, residual, scale, (int64_t)m * N, n, N, res);
         }
     }
 }
@@ -769,6 +805,27 @@ __global__ void w8a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __res
     }
 }
 
+// [N, K] row-major int8 holding 4-bit values (-8 .. 7) -> packed nibble tiles (q + 8).  One thread per 8 packed bytes.
+__global__ void w4a16_pack_kernel(uint8_t* __restrict__ dst, const int8_t* __restrict__ src, int N, int K,
+                                  int64_t chunks) {
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * blockDim.x) {
+        const int lane = (int)(c & 63);
+        const int64_t tile = c >> 6;
+        const int n_tiles = (N + 15) >> 4;
+        const int t = (int)(tile % n_tiles);
+        const int s = (int)(tile / n_tiles);
+        const int n = 16 * t + (lane & 15);
+        const int k0 = 64 * s + 16 * (lane >> 4);
+        uint32_t v[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int q = (n < N && k0 + j < K) ? (int)src[(int64_t)n * K + k0 + j] : 0;
+            v[j >> 3] |= (uint32_t)((q + 8) & 15) << (4 * (j & 7));
+        }
+        *(u32x2*)(dst + c * 8) = (u32x2){v[0], v[1]};
+    }
+}
+
 struct RopeCacheArgs {
     const void *cos, *sin;
     void *key_cache, *value_cache;
@@ -787,7 +844,7 @@ struct GemmPlan {
     int steps_per_split;
 };
 
-GemmPlan plan_w8a16(int m, int n, int k) {
+GemmPlan plan_w8a16(int m, int n, int k, int step_align = 1) {
     GemmPlan p;
     p.mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
     p.m_blocks = (m + 16 * p.mt - 1) / (16 * p.mt);
@@ -808,6 +865,7 @@ GemmPlan plan_w8a16(int m, int n, int k) {
     sk = sk > 16 ? 16 : sk;
     if (sk > 8) sk = 8 * (sk / 8);                             // multiples of 8 can run split-major
     p.steps_per_split = (total_steps + sk - 1) / sk;
+    p.steps_per_split = (p.steps_per_split + step_align - 1) / step_align * step_align;   // splits begin on group borders
     p.split_k = (total_steps + p.steps_per_split - 1) / p.steps_per_split;
     return p;
 }
@@ -816,8 +874,12 @@ template <typename T>
 int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
                  const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st,
                  void* norm_out = nullptr, const void* gamma = nullptr, float eps = 0.f, int gamma_dtype = MF_FP32,
-                 const RopeCacheArgs* rc_args = nullptr) {
-    const GemmPlan p = plan_w8a16(m, n, k);
+                 const RopeCacheArgs* rc_args = nullptr, int w4_group = -1) {
+    // w4_group >= 0: 4-bit weights; 0 = `scale` holds one value per channel, 64 / 128 = one per channel and group
+    // ([K / group][N]), applied inside the kernel (the epilogues then see no scale)
+    const GemmPlan p = plan_w8a16(m, n, k, w4_group == 128 ? 2 : 1);
+    const float* gscale = w4_group > 0 ? scale : nullptr;
+    if (w4_group > 0) scale = nullptr;
     float* partial = p.split_k > 1 ? (float*)workspace : nullptr;
     const int split_major = p.split_k % 8 == 0;
     dim3 grid(split_major ? p.split_k : p.n_blocks, split_major ? p.n_blocks : p.split_k, p.m_blocks);
@@ -826,11 +888,25 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     hipLaunchKernelGGL((w8a16_gemm4_kernel<T, MTV, WV, KT>), grid, dim3(WV * 64), 0, st, (uint16_t*)y, partial,  \
                        (const uint16_t*)x, wp, scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, k, \
                        p.steps_per_split, gated, split_major)
+#define GW4_LAUNCH_W4(MTV, WV, GV)                                                                               \
+    hipLaunchKernelGGL((w8a16_gemm4_kernel<T, MTV, WV, false, true, GV>), grid, dim3(WV * 64), 0, st, (uint16_t*)y, \
+                       partial, (const uint16_t*)x, wp, scale, (const uint16_t*)bias, (const uint16_t*)residual, m, n, \
+                       k, p.steps_per_split, gated, split_major, gscale)
+#define GW4_W4_BY_GROUP(MTV, WV)                                                                                 \
+    { if (w4_group == 0) GW4_LAUNCH_W4(MTV, WV, 0); else if (w4_group == 64) GW4_LAUNCH_W4(MTV, WV, 64);          \
+      else GW4_LAUNCH_W4(MTV, WV, 128); }
+    if (w4_group >= 0) {
+        if (p.mt == 1) GW4_W4_BY_GROUP(1, 4)
+        else if (p.mt == 2) GW4_W4_BY_GROUP(2, 4)
+        else GW4_W4_BY_GROUP(4, 8)
+    } else
     if (p.mt == 1) { if (ktail) GW4_LAUNCH(1, 4, true); else GW4_LAUNCH(1, 4, false); }
     else if (p.mt == 2) { if (ktail) GW4_LAUNCH(2, 4, true); else GW4_LAUNCH(2, 4, false); }
     else if (p.waves == 8) { if (ktail) GW4_LAUNCH(4, 8, true); else GW4_LAUNCH(4, 8, false); }
     else { if (ktail) GW4_LAUNCH(4, 4, true); else GW4_LAUNCH(4, 4, false); }
 #undef GW4_LAUNCH
+#undef GW4_LAUNCH_W4
+#undef GW4_W4_BY_GROUP
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (rc_args && partial) {                                 // reduce + RoPE + cache scatter in one kernel
@@ -1068,4 +1144,50 @@ extern "C" int mf_grouped_w8a16_gemm_silu_mul(void* y, const void* x, const void
                                               int dtype, void* stream) {
     return grouped_w8a16_entry("grouped_w8a16_gemm_silu_mul", y, x, w_packed, scale, offsets, n_experts, total_rows, n,
                                k, dtype, 1, stream);
+}
+
+// ---- 4-bit weights ---------------------------------------------------------------------------------------------------
+extern "C" size_t mf_w4a16_packed_bytes(int n, int k) {
+    if (n <= 0 || k <= 0) return 0;
+    return (size_t)((n + 15) / 16) * ((k + GW_KSTEP - 1) / GW_KSTEP) * (GW_TILE_BYTES / 2);
+}
+
+extern "C" int mf_w4a16_pack_weight(void* packed, const int8_t* w, int n, int k, void* stream) {
+    MF_REQUIRE(packed && w && n > 0 && k > 0, "w4a16_pack_weight: bad arguments");
+    MF_REQUIRE(((uintptr_t)packed & 15) == 0, "w4a16_pack_weight: packed buffer must be 16-byte aligned");
+    const int64_t chunks = (int64_t)mf_w4a16_packed_bytes(n, k) / 8;
+    const int blocks = (int)((chunks + 255) / 256 > 65535 ? 65535 : (chunks + 255) / 256);
+    hipLaunchKernelGGL(w4a16_pack_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint8_t*)packed, w, n, k,
+                       chunks);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" size_t mf_w4a16_workspace_bytes(int m, int n, int k, int group_size) {
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const GemmPlan p = plan_w8a16(m, n, k, group_size == 128 ? 2 : 1);
+    return p.split_k > 1 ? (size_t)p.split_k * m * n * sizeof(float) : 0;
+}
+
+extern "C" int mf_w4a16_gemm(void* y, const void* x, const void* w_packed, const float* scale, const void* bias,
+                             const void* residual, int m, int n, int k, int group_size, int dtype, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w4a16_gemm: dtype must be bf16 or fp16");
+    if (m == 0) return 0;
+    MF_REQUIRE(y && x && w_packed && scale, "w4a16_gemm: null argument");
+    MF_REQUIRE(m >= 0 && n > 0 && k > 0, "w4a16_gemm: bad sizes m=%d n=%d k=%d", m, n, k);
+    MF_REQUIRE(group_size == 0 || group_size == 64 || group_size == 128,
+               "w4a16_gemm: group_size %d not supported (0 = per channel, 64, 128)", group_size);
+    MF_REQUIRE(k % 64 == 0 && (group_size == 0 || k % group_size == 0),
+               "w4a16_gemm: K (%d) must be a multiple of 64 and of the group size", k);
+    MF_REQUIRE(group_size == 0 || n % 4 == 0, "w4a16_gemm: N (%d) must be a multiple of 4 with per-group scales", n);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)scale) & 15) == 0,
+               "w4a16_gemm: x, w_packed and scale must be 16-byte aligned");
+    const size_t need = mf_w4a16_workspace_bytes(m, n, k, group_size);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w4a16_gemm: 16-byte aligned workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
+                                  (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, nullptr, group_size);
+    return launch_w8a16<FP16>(y, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
+                              (hipStream_t)stream, nullptr, nullptr, 0.f, MF_FP32, nullptr, group_size);
 }

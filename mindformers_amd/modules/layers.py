@@ -146,15 +146,65 @@ class _QuantLinearBase(nn.Module):
 
 
 class WeightQuantLinearCell(_QuantLinearBase):
-    """W8A16 deploy cell (lowers to WeightQuantBatchMatmul in the reference stack)."""
+    """Weight-only deploy cell (lowers to WeightQuantBatchMatmul in the reference stack).  ``weight_bits`` 8: int8 per
+    output channel (W8A16).  ``weight_bits`` 4 (weight_dtype qint4x2, quantization_config.py:408-416): ``weight`` is
+    int8 [out, in / 2] with two 4-bit values per byte (element 2j in the low nibble), ``w_scale`` one value per output
+    channel (``group_size`` 0) or [in / group_size, out] (per_group, 64 or 128).  ``smooth``: the activations are
+    multiplied by ``smooth_scale`` [in] first (the activation side of awq / smooth outlier suppression, whose weight
+    side is folded into the checkpoint's weights)."""
+
+    def __init__(self, in_channels, out_channels, has_bias=False, compute_dtype=torch.bfloat16, device="cuda",
+                 layer=None, weight_bits=8, group_size=0, smooth=False):
+        super().__init__(in_channels, out_channels, has_bias, compute_dtype, device, layer)
+        if weight_bits not in (8, 4) or group_size not in (0, 64, 128):
+            raise ValueError(f"weight_bits must be 8 or 4 and group_size 0, 64 or 128, got {weight_bits} / {group_size}")
+        if weight_bits == 8 and group_size:
+            raise NotImplementedError("per_group scales are built for 4-bit weights only")
+        self.weight_bits, self.group_size = weight_bits, group_size
+        if weight_bits == 4:
+            if in_channels % 64 or (group_size and in_channels % group_size):
+                raise ValueError(f"in_channels ({in_channels}) must be a multiple of 64 and of the group size for 4-bit weights")
+            self.weight = torch.zeros(out_channels, in_channels // 2, dtype=torch.int8, device=device)
+            if group_size:
+                self.w_scale = torch.ones(in_channels // group_size, out_channels, dtype=torch.float32, device=device)
+        self.register_buffer("smooth_scale", torch.ones(in_channels, dtype=torch.float32, device=device) if smooth else None)
+
+    @torch.no_grad()
+    def quantize_from_float(self, weight, bias=None):
+        if self.weight_bits == 8:
+            return super().quantize_from_float(weight, bias)
+        # symmetric 4-bit, per channel or per channel and group: s = max|w| / 7, q = clip(rint(w / s), -8, 7), the
+        # quotient in float64
+        w = weight.detach().to(device=self.weight.device, dtype=torch.float64)
+        n, k = self.out_channels, self.in_channels
+        if tuple(w.shape) != (n, k):
+            raise ValueError(f"weight shape {tuple(w.shape)} != {(n, k)}")
+        g = self.group_size or k
+        wg = w.reshape(n, k // g, g)
+        scale = (wg.abs().amax(dim=2) / 7.0).float()
+        safe = torch.where(scale > 0, scale, torch.ones_like(scale)).double()
+        q = torch.clamp(torch.round(wg / safe[:, :, None]), -8, 7).to(torch.int8).reshape(n, k)
+        self.weight.copy_(((q[:, 0::2] & 15) | (q[:, 1::2] << 4)).to(torch.int8))
+        self.w_scale.copy_(scale[:, 0] if self.group_size == 0 else scale.t().contiguous())
+        if bias is not None and self.bias is not None:
+            self.bias.copy_(bias.to(self.bias.dtype))
+        self._packed = None
+        return self
 
     def prepare(self):
-        self._packed = ops.pack_w8a16(self.weight, self.w_scale)
+        if self.weight_bits == 4:
+            self._packed = ops.pack_w4a16(self.weight, self.w_scale, self.group_size, qint4x2=True)
+        else:
+            self._packed = ops.pack_w8a16(self.weight, self.w_scale)
         return self
 
     def _matmul(self, x, residual=None):
         if self._packed is None:
             self.prepare()
+        if self.smooth_scale is not None:
+            x = ops.scale_columns(x, self.smooth_scale)
+        if self.weight_bits == 4:
+            return ops.w4a16_linear(x, self._packed, bias=self.bias, residual=residual)
         return ops.w8a16_linear(x, self._packed, bias=self.bias, residual=residual)
 
     def forward(self, x, residual=None):

@@ -97,18 +97,25 @@ def _skipped(name, blacklist):
 
 def check_buildable(cfg):
     """Raise for configurations the reference's config classes accept but these kernels do not implement."""
-    if cfg.weight_quant_dtype != "int8":
-        raise NotImplementedError(f"weight_dtype {cfg.weight_quant_dtype!r}: only int8 per-channel weights are built")
-    if getattr(cfg, "weight_quant_granularity", "per_channel") != "per_channel":
-        raise NotImplementedError("per_group weight quantisation is not built")
+    if cfg.weight_quant_dtype not in ("int8", "int4x2"):
+        raise NotImplementedError(f"weight_dtype {cfg.weight_quant_dtype!r}: int8 and int4x2 weights are built")
+    per_group = getattr(cfg, "weight_quant_granularity", "per_channel") == "per_group"
+    if cfg.weight_quant_dtype == "int4x2" and cfg.act_quant_dtype is not None:
+        raise NotImplementedError("4-bit weights are built weight-only (A16W4); W4A8 is not")
+    if per_group and cfg.weight_quant_dtype != "int4x2":
+        raise NotImplementedError("per_group weight scales are built for int4x2 weights only")
+    if per_group and getattr(cfg, "group_size", 0) not in (64, 128):
+        raise NotImplementedError("per_group weights need group_size 64 or 128")
     if cfg.kvcache_quant_dtype not in (None, "int8"):
         raise NotImplementedError(f"kvcache_dtype {cfg.kvcache_quant_dtype!r}: only an int8 KV cache is built")
     if cfg.kvcache_quant_dtype == "int8" and getattr(cfg, "kvcache_quant_granularity", "per_channel") != "per_channel":
         raise NotImplementedError("per_token int8 KV cache is not built (per_channel only)")
     if getattr(cfg, "precision_recovery", "none") != "none":
         raise NotImplementedError("GPTQ precision recovery has no deploy-time kernel here")
-    if cfg.outliers_suppression not in ("none", "smooth"):
+    if cfg.outliers_suppression not in ("none", "smooth", "awq"):
         raise NotImplementedError(f"outliers_suppression {cfg.outliers_suppression!r} is not built")
+    if cfg.outliers_suppression == "awq" and cfg.act_quant_dtype is not None:
+        raise NotImplementedError("awq is built in front of weight-only cells (A16W4 / A16W8)")
     if cfg.act_quant_dtype == "int8" and cfg.act_quant_granularity not in ("per_token", "per_tensor"):
         raise NotImplementedError(f"act_quant_granularity {cfg.act_quant_granularity!r} is not built")
 
@@ -143,7 +150,11 @@ def convert_linears(model, cfg, layer_policies=None):
                                                    smooth=pol.outliers_suppression == "smooth",
                                                    act_quant_granularity=pol.act_quant_granularity)
                 else:
-                    cell = WeightQuantLinearCell(fin, fout, has_bias, cdt, dev, layer=child)
+                    per_group = getattr(pol, "weight_quant_granularity", "per_channel") == "per_group"
+                    cell = WeightQuantLinearCell(fin, fout, has_bias, cdt, dev, layer=child,
+                                                 weight_bits=4 if pol.weight_quant_dtype == "int4x2" else 8,
+                                                 group_size=pol.group_size if per_group else 0,
+                                                 smooth=pol.outliers_suppression in ("smooth", "awq"))
                 if child.weight is not None:
                     w = child.weight.data if getattr(child, "transpose_b", True) else child.weight.data.t()
                     cell.quantize_from_float(w, child.bias.data if has_bias else None)

@@ -483,6 +483,18 @@ def silu_mul(gate_up, interleaved=False):
     return out
 
 
+def scale_columns(x, scale):
+    """x * scale[None, :] rounded once (activation multiplier in front of a weight-only GEMM)."""
+    lib = _lib.load()
+    dev = _dev_ok(x, scale)
+    cols = x.shape[-1]
+    _need(x.dtype in _ACT and scale.dtype == torch.float32 and scale.numel() == cols, "x bf16/fp16, scale fp32 [cols]")
+    out = torch.empty_like(x)
+    check(lib.mf_scale_columns(ptr(out), ptr(x), ptr(scale), x.numel() // cols, cols, dtype_code(x.dtype),
+                               stream_ptr(dev)), "mf_scale_columns")
+    return out
+
+
 def add(a, b):
     lib = _lib.load()
     dev = _dev_ok(a, b)
@@ -554,6 +566,66 @@ class TiledInt8Activations:
 
     def __init__(self, data, shape):
         self.data, self.shape = data, tuple(shape)
+
+
+class PackedInt4Weight:
+    """A 4-bit weight [N, K] in the nibble-tile order the A16W4 kernel streams, with its scales: fp32 [N]
+    (``group_size`` 0) or [K / group_size, N]."""
+
+    def __init__(self, packed, scale, n, k, group_size):
+        self.packed, self.scale, self.n, self.k, self.group_size = packed, scale, n, k, group_size
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+
+def unpack_qint4x2(w):
+    """int8 [N, K/2] holding two signed 4-bit values per byte (element 2j in the low nibble, 2j + 1 in the high one)
+    -> int8 [N, K] of values -8 .. 7.  Data movement only."""
+    _need(w.dtype == torch.int8 and w.dim() == 2, "qint4x2 weight must be int8 [N, K/2]")
+    lo = (w << 4) >> 4                                            # arithmetic shifts sign-extend the nibbles
+    hi = w >> 4
+    return torch.stack((lo, hi), dim=-1).reshape(w.shape[0], -1).contiguous()
+
+
+def pack_w4a16(w_q, scale, group_size=0, qint4x2=False):
+    """Pack 4-bit weights for ``w4a16_linear``: ``w_q`` int8 [N, K] holding values -8 .. 7, or with ``qint4x2`` the
+    two-per-byte form [N, K/2] (see ``unpack_qint4x2``); scale fp32 [N] or [K / group_size, N]."""
+    lib = _lib.load()
+    dev = _dev_ok(w_q, scale)
+    _need(w_q.dtype == torch.int8 and w_q.dim() == 2, "weight must be int8 [N, K] (values -8..7) or qint4x2 [N, K/2]")
+    _need(scale.dtype == torch.float32 and group_size in (0, 64, 128), "scale must be fp32; group_size 0, 64 or 128")
+    if qint4x2:
+        w_q = unpack_qint4x2(w_q)
+    n, k = w_q.shape
+    _need(k % 64 == 0 and (group_size == 0 or k % group_size == 0), f"K ({k}) must be a multiple of 64 and of the group size")
+    want = (n,) if group_size == 0 else (k // group_size, n)
+    _need(tuple(scale.shape) == want, f"scale must be {want}, got {tuple(scale.shape)}")
+    _need(group_size == 0 or n % 4 == 0, "N must be a multiple of 4 with per-group scales")
+    packed = torch.empty(lib.mf_w4a16_packed_bytes(n, k), dtype=torch.uint8, device=dev)
+    check(lib.mf_w4a16_pack_weight(ptr(packed), ptr(w_q.contiguous()), n, k, stream_ptr(dev)), "mf_w4a16_pack_weight")
+    return PackedInt4Weight(packed, scale.contiguous(), n, k, group_size)
+
+
+def w4a16_linear(x, w, bias=None, residual=None):
+    """y = x . (w_int4 * scale)^T (+ bias) (+ residual): the A16W4 weight-only GEMM; ``w`` a PackedInt4Weight."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt4Weight), "w must be a PackedInt4Weight (pack_w4a16)")
+    dev = _dev_ok(x, bias, residual)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    n, k = w.n, w.k
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
+    m = x.numel() // k
+    y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=dev)
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    _need(residual is None or (residual.dtype == x.dtype and residual.shape == y.shape), "residual mismatch")
+    need = lib.mf_w4a16_workspace_bytes(m, n, k, w.group_size)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w4a16_gemm(ptr(y), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(residual), m, n, k, w.group_size,
+                            dtype_code(x.dtype), ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w4a16_gemm")
+    return y
 
 
 def w8a16_linear_add_rmsnorm(x, w, residual, gamma, eps, bias=None):

@@ -38,6 +38,10 @@ Pinning status of each function (what fixes it besides its own formula):
   dynamic_quant_per_token, pinned against exact integer matmul; rounding mode, clamp range
   static_quant_per_tensor,
   w8a8_linear              and dequant order are this build's declared convention.
+  quantize_weight_int4,    PARITY UNPINNED against the reference for the same reason (s = max|w| / 7 per channel or per
+  w4a16_linear             channel and group, q in -8 .. 7, the group's scale applied to the group's sum: declared);
+                           pinned against that convention by rails, the half-step round trip, exactness on
+                           power-of-two grids and the pack / unpack identity (tests/test_host_logic.py)
   quantize_kv_int8,        PARITY UNPINNED against the reference for the same reason (the convention, affine per
   dequantize_kv_int8       channel with ties to even and rails -128 / 127, is declared); the two functions
                            themselves are pinned against that convention by hand-computed values, the offset's
@@ -53,7 +57,8 @@ from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_ya
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp
 from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token, static_quant_per_tensor,
-                    int8_gemm_i32, w8a8_linear, quantize_kv_int8, dequantize_kv_int8)
+                    int8_gemm_i32, w8a8_linear, quantize_kv_int8, dequantize_kv_int8, quantize_weight_int4,
+                    w4a16_linear, pack_qint4x2, unpack_qint4x2)
 from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,
                   grouped_matmul)

@@ -97,3 +97,49 @@ def dequantize_kv_int8(q, scale, offset=None):
     if offset is not None:
         x = x - np.asarray(offset, dtype=np.float64)
     return x * np.asarray(scale, dtype=np.float64)
+
+
+def quantize_weight_int4(weight, group_size=0):
+    """Symmetric 4-bit weights, per output channel (group_size 0) or per channel and group of ``group_size`` input
+    columns: s = max|w| / 7 over the group (float32), q = clip(rint(w / s), -8, 7) with the quotient in float64.
+    Returns (q int8 [N, K] of values -8 .. 7, s float32 [N] or [K / group_size, N]).  PARITY UNPINNED against the
+    reference like the int8 convention (golden-stick's A16W4 arithmetic is not vendored); held to what the
+    mathematics fixes by tests/test_host_logic.py (rails, half-step round trip, exactness on power-of-two grids)."""
+    w = np.asarray(weight, dtype=np.float64)
+    n, k = w.shape
+    g = group_size or k
+    wg = w.reshape(n, k // g, g)
+    scale = (np.abs(wg).max(axis=2) / 7.0).astype(np.float32)                       # [N, K/g]
+    safe = np.where(scale > 0, scale, 1.0).astype(np.float64)
+    q = np.clip(np.rint(wg / safe[:, :, None]), -8, 7).astype(np.int8).reshape(n, k)
+    return q, (scale[:, 0] if group_size == 0 else np.ascontiguousarray(scale.T))
+
+
+def w4a16_linear(x, w_q, scale, group_size=0, bias=None):
+    """y = sum over groups of (x_g . q_g^T) * s_g (+ bias): integer weights times activations summed per group, the
+    group's scale applied to the group's sum.  float64."""
+    x = np.asarray(x, dtype=np.float64)
+    q = np.asarray(w_q, dtype=np.float64)
+    n, k = q.shape
+    g = group_size or k
+    s = np.asarray(scale, dtype=np.float64)
+    s = s.reshape(1, n) if group_size == 0 else s                                    # [K/g, N]
+    y = np.zeros((x.shape[0], n))
+    for i in range(k // g):
+        y += (x[:, i * g:(i + 1) * g] @ q[:, i * g:(i + 1) * g].T) * s[i][None, :]
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)
+    return y
+
+
+def pack_qint4x2(w_q):
+    """int8 [N, K] of values -8 .. 7 -> int8 [N, K/2]: element 2j in the low nibble of byte j, 2j + 1 in the high."""
+    u = (np.asarray(w_q).astype(np.int16) & 15).astype(np.uint8)
+    return (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8).view(np.int8)
+
+
+def unpack_qint4x2(w):
+    u = np.asarray(w).view(np.uint8)
+    lo, hi = (u & 15).astype(np.int8), (u >> 4).astype(np.int8)
+    lo, hi = np.where(lo > 7, lo - 16, lo), np.where(hi > 7, hi - 16, hi)
+    return np.stack((lo, hi), axis=-1).reshape(u.shape[0], -1).astype(np.int8)

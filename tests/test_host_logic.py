@@ -137,8 +137,15 @@ def test_unbuilt_quant_modes_are_rejected_at_conversion():
     from mindformers_amd.modules.quantizers.base import check_buildable
     from mindformers_amd.quantization_config import PtqConfig, SmoothQuantConfig
     check_buildable(SmoothQuantConfig())                 # static per-tensor activations + smooth: built
+    check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=64))   # A16W4: built
+    check_buildable(PtqConfig(weight_dtype="int4", outliers_suppression="awq", weight_quant_granularity="per_group",
+                              group_size=128))
+    with pytest.raises(NotImplementedError):             # per_group scales go with 4-bit weights
+        check_buildable(PtqConfig(weight_dtype="int8", weight_quant_granularity="per_group", group_size=64))
+    with pytest.raises(NotImplementedError):             # per_group without a group size
+        check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=0))
     with pytest.raises(NotImplementedError):
-        check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=64))
+        check_buildable(PtqConfig(weight_dtype="int4", precision_recovery="gptq"))
     with pytest.raises(NotImplementedError):             # an int8 cache is built per channel only
         check_buildable(PtqConfig(activation_dtype="int8", act_quant_granularity="per_token", kvcache_dtype="int8",
                                   kvcache_quant_granularity="per_token"))
@@ -313,3 +320,40 @@ def test_cache_sizing_follows_the_reference_formula():
     assert num_cache_blocks(1, 128, 8, 128, 32, 2) == 64
     assert num_cache_blocks(1, 128, 8, 128, 32, 1) == 128           # int8 cache
     assert num_cache_blocks(0, 128, 8, 128, 32, 2) == 0
+
+
+# ------------------------------------------------------------------------------------------- 4-bit weight convention
+@pytest.mark.parametrize("group", [0, 64, 128])
+def test_int4_weight_quantisation_is_held_to_what_the_mathematics_fixes(group):
+    """The declared A16W4 convention (s = max|w| / 7 per channel or per channel and group, q = clip(rint(w / s), -8, 7),
+    the group's scale on the group's sum): values on the grid come back exactly, everything comes back within half a
+    step, the extreme of every group sits on the rail, the two-per-byte form is a bijection, and on power-of-two scales
+    with integer activations the linear is the exact integer matmul.  A scale applied per channel where it is per
+    group, a transposed scale table or a swapped nibble order fails one of these."""
+    rng = np.random.default_rng(40 + group)
+    n, k = 12, 256
+    g = group or k
+    w = rng.normal(size=(n, k))
+    q, s = O.quantize_weight_int4(w, group)
+    assert q.dtype == np.int8 and q.min() >= -8 and q.max() <= 7
+    assert s.shape == ((n,) if group == 0 else (k // g, n)) and s.dtype == np.float32
+    s_full = (np.repeat(s[None, :], 1, 0).T if group == 0 else s.T)                  # [N, K/g]
+    deq = (q.reshape(n, k // g, g) * s_full[:, :, None].astype(np.float64)).reshape(n, k)
+    assert np.all(np.abs(deq - w) <= 0.5 * np.repeat(s_full, g, axis=1) * (1 + 1e-6))
+    amax = np.abs(w.reshape(n, k // g, g)).max(axis=2)
+    assert np.all(np.abs(q.reshape(n, k // g, g)).max(axis=2) == 7) and np.allclose(s_full, amax / 7, rtol=1e-6)
+    # a weight already on the grid of power-of-two scales is reproduced exactly, and the linear is the integer matmul
+    s2 = 2.0 ** rng.integers(-6, -2, s_full.shape)
+    q0 = rng.integers(-7, 8, (n, k)).astype(np.int8)
+    q0.reshape(n, k // g, g)[:, :, 0] = 7                                             # every group reaches the rail
+    w0 = (q0.reshape(n, k // g, g) * s2[:, :, None]).reshape(n, k)
+    q1, s1 = O.quantize_weight_int4(w0, group)
+    assert np.array_equal(q1, q0) and np.array_equal(s1, (s2[:, 0] if group == 0 else s2.T).astype(np.float32))
+    x = rng.integers(-3, 4, (5, k)).astype(np.float64)
+    y = O.w4a16_linear(x, q1, s1, group)
+    assert np.array_equal(y, x @ w0.T)
+    # two values per byte, element 2j in the low nibble
+    packed = O.pack_qint4x2(q0)
+    assert packed.shape == (n, k // 2) and np.array_equal(O.unpack_qint4x2(packed), q0)
+    one = O.pack_qint4x2(np.array([[-8, 7, 1, -1]], np.int8)).view(np.uint8)
+    assert one.tolist() == [[0x78, 0xF1]]

@@ -870,6 +870,87 @@ def test_w8a16_inf_in_the_last_columns_of_a_row_stays_in_that_row(m, n, k):
     assert np.array_equal(y[bad][w_hit != 0], np.sign(w_hit[w_hit != 0]) * np.inf)
 
 
+# ------------------------------------------------------------------------------------------- W4A16
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("group", [0, 64, 128])
+@pytest.mark.parametrize("m,n,k,bias,residual", [
+    (1, 4096, 4096, False, False), (16, 704, 512, True, False), (32, 512, 1408, True, True),
+    (64, 6144, 4096, False, True), (65, 132, 2048, False, False), (130, 256, 512, True, True),
+    (33, 64, 128, False, False), (4, 3584, 18944, False, False),
+])
+def test_w4a16_gemm(dtype, group, m, n, k, bias, residual):
+    """4-bit weight-only GEMM against the oracle: per-channel and per-group scales, row counts on both sides of every
+    tile height, shapes that split K and shapes that do not, from the two-per-byte and the one-per-byte weight forms."""
+    rng = np.random.default_rng(m * 7 + n + group)
+    w = rng.normal(0, 0.02, (n, k)).astype(np.float32)
+    wq, s = O.quantize_weight_int4(w, group)
+    x = rounded(rng.normal(size=(m, k)), dtype)
+    b = rounded(rng.normal(0, 0.1, n), dtype) if bias else None
+    r = rounded(rng.normal(size=(m, n)), dtype) if residual else None
+    s_t = torch.from_numpy(s).cuda()
+    packed = ops.pack_w4a16(torch.from_numpy(O.pack_qint4x2(wq)).cuda(), s_t, group, qint4x2=True)
+    same = ops.pack_w4a16(torch.from_numpy(wq).cuda(), s_t, group)
+    assert torch.equal(packed.packed, same.packed)
+    y = ops.w4a16_linear(dev(x, dtype), packed, dev(b, dtype) if bias else None, dev(r, dtype) if residual else None)
+    v = O.w4a16_linear(x, wq, s, group, b)
+    s_full = np.repeat(s.reshape(1, n) if group == 0 else s, (group or k), axis=0)          # [K, N]
+    dot_mag = np.abs(x).astype(np.float64) @ (np.abs(wq).astype(np.float64).T * s_full)
+    extra = 2.0 ** -18 * dot_mag + 1e-9
+    if residual:
+        vr = rounded(v, dtype).astype(np.float64)
+        ref, mag = vr + r, np.abs(vr + r) + 2 * np.abs(vr)
+    else:
+        ref, mag = v, np.abs(v)
+    assert_within(to_np(y), ref, mag, dtype, ulps=1.0, extra=extra, what=f"w4a16 g{group}")
+
+
+@pytest.mark.parametrize("group", [0, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(37, 200, 1408), (3, 64, 4096), (64, 1024, 256)])
+def test_w4a16_exact_on_integer_grid(group, m, n, k):
+    """Power-of-two scales (one per channel and group) and small-integer activations make every product and sum exact:
+    the kernel must return exactly the per-group integer matmul.  A group's scale applied to its neighbour, a swapped
+    nibble or a dropped k-step changes the result."""
+    rng = np.random.default_rng(group + k)
+    wq = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    s = (2.0 ** rng.integers(-9, -5, (n,) if group == 0 else (k // group, n))).astype(np.float32)
+    x = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    packed = ops.pack_w4a16(torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda(), group)
+    y = ops.w4a16_linear(dev(x, torch.float16), packed)
+    exact = O.w4a16_linear(x, wq, s, group)
+    assert np.array_equal(to_np(y).astype(np.float64), rounded(exact, torch.float16).astype(np.float64))
+
+
+def test_w4a16_rejects_bad_operands():
+    wq = torch.zeros(64, 128, dtype=torch.int8, device="cuda")
+    s = torch.ones(64, device="cuda")
+    with pytest.raises(ValueError):
+        ops.pack_w4a16(wq, s, 32)                                         # group size not built
+    with pytest.raises(ValueError):
+        ops.pack_w4a16(wq, s, 64)                                         # scale table of the wrong shape
+    with pytest.raises(ValueError):
+        ops.pack_w4a16(wq[:, :96].contiguous(), s, 0)                     # K not a multiple of 64
+    packed = ops.pack_w4a16(wq, s, 0)
+    with pytest.raises(ValueError):
+        ops.w4a16_linear(torch.zeros(2, 64, dtype=torch.bfloat16, device="cuda"), packed)
+    with pytest.raises(ValueError):
+        ops.w4a16_linear(torch.zeros(2, 128, dtype=torch.float32, device="cuda"), packed)
+    assert ops.w4a16_linear(torch.zeros(0, 128, dtype=torch.bfloat16, device="cuda"), packed).shape == (0, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (7, 104), (64, 18944), (0, 64)])
+def test_scale_columns_bit_exact(dtype, rows, cols):
+    """x * s per column: the float32 product rounded to the activation type, bit for bit (on the ~6e-5 of fp16
+    elements whose float32 product lands on a rounding tie this differs from rounding the exact product once, so
+    the large case also pins which of the two the kernel computes)."""
+    rng = np.random.default_rng(rows + cols)
+    x = rounded(rng.normal(size=(rows, cols)), dtype)
+    s = rng.uniform(0.25, 4.0, cols).astype(np.float32)
+    y = ops.scale_columns(dev(x, dtype), torch.from_numpy(s).cuda())
+    ref32 = (x.astype(np.float32) * s[None, :]).astype(np.float32)
+    assert np.array_equal(to_np(y), rounded(ref32, dtype))
+
+
 def test_column_parallel_linear_reference_vectors(golden_dir):
     """The reference's linear vectors are for the bf16 cell; they pin the W8A16 path's layout ([out, in] weight,
     bias add): quantise the reference weight, run the kernel, compare with the oracle linear on the dequantised

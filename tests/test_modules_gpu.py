@@ -313,6 +313,53 @@ def test_quantizer_swaps_cells_and_matches_oracle(method):
     assert out.shape == (7, 1000) and torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("granularity,group,suppression", [("per_channel", 0, "None"), ("per_group", 64, "None"),
+                                                           ("per_group", 128, "awq")])
+def test_quantizer_builds_four_bit_weight_only_cells(granularity, group, suppression):
+    """A16W4 (weight_dtype int4 -> qint4x2, quantization_config.py:33, :408-416), per channel or per group, with the
+    awq multiplier on the activations: the quantizer swaps in 4-bit WeightQuantLinearCells whose buffers hold two
+    values per byte and a scale table [in / group, out]; a checkpoint round trip (state_dict -> fresh cells) gives
+    the same output; the output equals the oracle's group-wise integer matmul."""
+    from mindformers_amd.modules import Linear, WeightQuantLinearCell
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    torch.manual_seed(0)
+    net = _tiny_model()
+    w_q, b_q = net.wq.weight.data.clone(), net.wq.bias.data.clone()
+    cfg = {"quant_method": "ptq", "weight_dtype": "int4", "weight_quant_granularity": granularity, "group_size": group,
+           "outliers_suppression": suppression, "modules_to_not_convert": ["lm_head"]}
+    quantizer = AutoQuantizer.from_config(cfg)
+    quantizer.preprocess_model(net)
+    assert isinstance(net.wq, WeightQuantLinearCell) and isinstance(net.lm_head, Linear)
+    assert net.wq.weight_bits == 4 and net.wq.group_size == group
+    assert net.wq.weight.shape == (512, 128) and net.wq.weight.dtype == torch.int8
+    assert net.wq.w_scale.shape == ((512,) if group == 0 else (256 // group, 512))
+    rng = np.random.default_rng(3)
+    smooth = None
+    if suppression == "awq":
+        smooth = rng.uniform(0.5, 2.0, 256).astype(np.float32)
+        net.wq.smooth_scale.copy_(torch.from_numpy(smooth))
+    else:
+        assert net.wq.smooth_scale is None
+    quantizer.postprocess_model(net)
+    x = rounded(rng.normal(size=(7, 256)), BF)
+    y = net.wq(dev(x, BF))
+    wq_i4, s = O.quantize_weight_int4(w_q.float().cpu().numpy(), group)
+    assert np.array_equal(to_np(net.wq.weight), O.pack_qint4x2(wq_i4)) and np.array_equal(to_np(net.wq.w_scale), s)
+    b = b_q.float().cpu().numpy()
+    xs = rounded(x * smooth[None, :], BF) if smooth is not None else x
+    ref = O.w4a16_linear(xs, wq_i4, s, group, b)
+    assert_within(to_np(y), ref, np.abs(ref) + np.abs(b), BF, ulps=1.0, extra=1e-5, what="4-bit cell")
+    # the deploy checkpoint carries the packed bytes and the scale table: fresh cells loaded from it agree bit for bit
+    fresh = _tiny_model()
+    q2 = AutoQuantizer.from_config(cfg)
+    q2.preprocess_model(fresh)
+    fresh.load_state_dict(net.state_dict())
+    q2.postprocess_model(fresh)
+    assert torch.equal(fresh.wq(dev(x, BF)), y)
+    out = net(dev(x, BF))
+    assert out.shape == (7, 1000) and torch.isfinite(out.float()).all()
+
+
 def test_smooth_quant_method_converts_to_static_per_tensor_cells():
     """The SmoothQuant method (A8W8, static per-tensor activations, smooth multiplier): the quantizer swaps in
     AllQuantLinearInferCell(act_quant_granularity="per_tensor"); with a calibrated scale and multiplier loaded, the
