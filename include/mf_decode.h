@@ -369,6 +369,20 @@ int mf_rmsnorm_dynamic_quant(int8_t* xq, float* x_scale, void* sum_out, const vo
 int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows, int cols,
                               int gate_up_layout, int dtype, int layout, void* stream);
 
+/* mf_dynamic_quant_per_token / mf_silu_mul_dynamic_quant for rows grouped by expert (the permuted rows in front of
+ * the routed experts' int8 GroupedMatmul, mindformers/parallel_core/inference/transformer/moe/experts.py:151-170, under
+ * outliers_suppression: smooth, mindformers/utils/quantization_config.py:413-414): rows offsets[e] ..
+ * offsets[e + 1] - 1 (offsets int32 [n_experts + 1], as mf_moe_permute writes it) are multiplied by row e of smooth
+ * fp32 [n_experts, k] before the per-token quantisation; rows at or past offsets[n_experts] use the last expert's.
+ * One multiplier vector per expert is this build's declared form of the suppression on stacked expert weights (the
+ * cell's arithmetic is not in the reference).  Everything else as the ungrouped calls. */
+int mf_grouped_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth,
+                                       const int32_t* offsets, int n_experts, int m, int k, int dtype, int layout,
+                                       void* stream);
+int mf_grouped_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth,
+                                      const int32_t* offsets, int n_experts, int rows, int cols, int gate_up_layout,
+                                      int dtype, int layout, void* stream);
+
 /* golden-stick QuantBatchMatmul: int8 x int8 -> int32 on MFMA, dequantised in the epilogue:
  * y[m,n] = acc[m,n] * x_scale[m] * w_scale[n] (+ bias[n]) (+ residual[m,n]) -> dtype.
  * xq int8 [M,K]: row-major (x_layout 0) or tiled (x_layout 1), as mf_dynamic_quant_per_token writes it; the tiled
@@ -406,6 +420,17 @@ int mf_w8a8_qkv_rope_and_cache(void* qkv, const int8_t* xq, const float* x_scale
                                int x_layout, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- mixture of experts --------------------------------------------------------------------------- */
+
+/* TopKRouter.gating — mindformers/parallel_core/inference/transformer/moe/router.py:49-63: the router's dense
+ * projection, logits = cast(x, router_dense_type) . w^T with w [n_experts, hidden] in the router's type.
+ * x [tokens, hidden] in `dtype`; w fp32 (w_dtype MF_FP32: products and sums in fp32) or of the activation type
+ * (w_dtype == dtype: a 16-bit router, whose projection output is rounded to that type); logits fp32
+ * [tokens, n_experts] (routing() casts to fp32 before scoring, router.py:127-128).  hidden % 4 == 0.  The sum over
+ * hidden is taken in a fixed order (slices of hidden added in sequence), so results do not depend on scheduling.
+ * workspace: mf_router_gate_workspace_bytes(tokens, n_experts, hidden) bytes (0 when hidden is not sliced). */
+size_t mf_router_gate_workspace_bytes(int tokens, int n_experts, int hidden);
+int mf_router_gate_gemm(float* logits, const void* x, const void* w, int tokens, int n_experts, int hidden, int dtype,
+                        int w_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* FusedAddTopKDiv(logits, bias, ...) — mindformers/parallel_core/inference/transformer/moe/router.py:129-140;
  * unfused form research/deepseek3/moe.py:763-778, mindformers/modules/transformer/moe.py:1529-1576.

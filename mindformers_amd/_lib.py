@@ -63,6 +63,10 @@ SIGNATURES = {
     "mf_w8a8_gemm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a8_gemm_add_rmsnorm_quant": (_I, [_P] * 11 + [_F] + [_I] * 7 + [_P, _Z, _P]),
     "mf_w8a8_qkv_rope_and_cache": (_I, [_P] * 11 + [_I] * 4 + [_L] + [_I] * 4 + [_P, _Z, _P]),
+    "mf_router_gate_workspace_bytes": (_Z, [_I, _I, _I]),
+    "mf_router_gate_gemm": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
+    "mf_grouped_dynamic_quant_per_token": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mf_grouped_silu_mul_dynamic_quant": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "mf_moe_route": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
     "mf_moe_permute": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mf_grouped_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),

@@ -155,15 +155,33 @@ __global__ void scale_columns_kernel(uint16_t* __restrict__ out, const uint16_t*
     }
 }
 
+// Rows grouped by expert (offsets int32 [groups + 1], rows offsets[e] .. offsets[e + 1] - 1 belong to e): the smooth
+// multiplier of a row is the row `e` of a [groups, cols] table.  The search is uniform over the workgroup.
+struct RowGroups {
+    const int32_t* offsets;       // null: one multiplier vector for every row
+    int groups;
+};
+__device__ __forceinline__ const float* smooth_of_row(const float* smooth, RowGroups rg, int row, int cols) {
+    if (!smooth || !rg.offsets) return smooth;
+    int lo = 0, hi = rg.groups - 1;                           // largest e with offsets[e] <= row
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (rg.offsets[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    return smooth + (int64_t)lo * cols;
+}
+
 // Per-token dynamic int8: xs = x*smooth; s = max|xs|/127; q = clip(rint(xs/s), -128, 127).
 // With static_scale (one float on the device: a calibrated per-tensor activation scale) s is that value for every
 // row and no maximum is taken; x_scale still receives s per row, which is what the int8 GEMM's epilogue reads.
 template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void dynamic_quant_kernel(int8_t* __restrict__ xq, float* __restrict__ x_scale,
                                                                const uint16_t* __restrict__ x,
-                                                               const float* __restrict__ smooth, int cols, int tiled,
-                                                               const float* __restrict__ static_scale) {
+                                                               const float* __restrict__ smooth_table, int cols,
+                                                               int tiled, const float* __restrict__ static_scale,
+                                                               RowGroups rg) {
     __shared__ float red[THREADS / 64];
+    const float* smooth = smooth_of_row(smooth_table, rg, blockIdx.x, cols);
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
     constexpr int ROW_THREADS = THREADS;
@@ -310,9 +328,10 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_quant_kernel(
 template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void silu_mul_quant_kernel(int8_t* __restrict__ xq, float* __restrict__ x_scale,
                                                                 const uint16_t* __restrict__ gu,
-                                                                const float* __restrict__ smooth, int cols, int layout,
-                                                                int tiled) {
+                                                                const float* __restrict__ smooth_table, int cols,
+                                                                int layout, int tiled, RowGroups rg) {
     __shared__ float red[THREADS / 64];
+    const float* smooth = smooth_of_row(smooth_table, rg, blockIdx.x, cols);
     const int nvec = cols >> 3;
     constexpr int ROW_THREADS = THREADS;
     constexpr int MAXV = ROW_MAX_COLS / 8 / THREADS;
@@ -440,7 +459,8 @@ extern "C" int mf_scale_columns(void* out, const void* x, const float* scale, in
 }
 
 static int quant_rows_entry(int8_t* xq, float* x_scale, const void* x, const float* smooth, const float* static_scale,
-                            int m, int k, int dtype, int layout, void* stream);
+                            int m, int k, int dtype, int layout, void* stream, const int32_t* group_offsets = nullptr,
+                            int groups = 0);
 
 extern "C" int mf_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth, int m,
                                           int k, int dtype, int layout, void* stream) {
@@ -454,8 +474,10 @@ extern "C" int mf_static_quant_per_tensor(int8_t* xq, float* x_scale, const void
 }
 
 static int quant_rows_entry(int8_t* xq, float* x_scale, const void* x, const float* smooth, const float* static_scale,
-                            int m, int k, int dtype, int layout, void* stream) {
+                            int m, int k, int dtype, int layout, void* stream, const int32_t* group_offsets, int groups) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(!group_offsets || groups > 0, "dynamic_quant: a group table needs groups > 0");
+    const RowGroups rg = {group_offsets, groups};
     MF_REQUIRE(layout == 0 || layout == 1, "dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
     if (m <= 0) return 0;
     MF_REQUIRE(xq && x_scale && x, "dynamic_quant: null argument");
@@ -466,7 +488,7 @@ static int quant_rows_entry(int8_t* xq, float* x_scale, const void* x, const flo
     if (m <= 0) return 0;
 #define DQ_LAUNCH(TT, TH)                                                                                        \
     hipLaunchKernelGGL((dynamic_quant_kernel<TT, TH>), dim3(m), dim3(TH), 0, (hipStream_t)stream, xq, x_scale,    \
-                       (const uint16_t*)x, smooth, k, layout, static_scale)
+                       (const uint16_t*)x, smooth, k, layout, static_scale, rg)
     const bool wide = k > 4096;
     if (dtype == MF_BF16) {
         if (wide) DQ_LAUNCH(BF16, ROW_THREADS_WIDE); else DQ_LAUNCH(BF16, ROW_THREADS);
@@ -523,9 +545,12 @@ int mf_detail_rmsnorm_quant_from_partial(int8_t* xq, float* x_scale, void* sum_o
     return MF_LAUNCH_CHECK();
 }
 
-extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows,
-                                         int cols, int gate_up_layout, int dtype, int layout, void* stream) {
+static int silu_mul_quant_entry(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows,
+                               int cols, int gate_up_layout, int dtype, int layout, void* stream,
+                               const int32_t* group_offsets, int groups) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "silu_mul_dynamic_quant: dtype must be bf16 or fp16");
+    MF_REQUIRE(!group_offsets || groups > 0, "silu_mul_dynamic_quant: a group table needs groups > 0");
+    const RowGroups rg = {group_offsets, groups};
     MF_REQUIRE(gate_up_layout == 0 || gate_up_layout == 1,
                "silu_mul_dynamic_quant: gate_up_layout must be 0 (halves) or 1 (interleaved)");
     MF_REQUIRE(layout == 0 || layout == 1, "silu_mul_dynamic_quant: layout must be 0 (row-major) or 1 (tiled)");
@@ -537,7 +562,7 @@ extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void*
                "silu_mul_dynamic_quant: gate_up/smooth must be 16-byte aligned, xq 8-byte aligned");
 #define SQ_LAUNCH(TT, TH)                                                                                        \
     hipLaunchKernelGGL((silu_mul_quant_kernel<TT, TH>), dim3(rows), dim3(TH), 0, (hipStream_t)stream, xq, x_scale, \
-                       (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout)
+                       (const uint16_t*)gate_up, smooth, cols, gate_up_layout, layout, rg)
     const bool wide = cols > 4096;
     if (dtype == MF_BF16) {
         if (wide) SQ_LAUNCH(BF16, ROW_THREADS_WIDE); else SQ_LAUNCH(BF16, ROW_THREADS);
@@ -546,4 +571,24 @@ extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void*
     }
 #undef SQ_LAUNCH
     return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth, int rows,
+                                         int cols, int gate_up_layout, int dtype, int layout, void* stream) {
+    return silu_mul_quant_entry(xq, x_scale, gate_up, smooth, rows, cols, gate_up_layout, dtype, layout, stream, nullptr, 0);
+}
+
+extern "C" int mf_grouped_dynamic_quant_per_token(int8_t* xq, float* x_scale, const void* x, const float* smooth,
+                                                  const int32_t* offsets, int n_experts, int m, int k, int dtype,
+                                                  int layout, void* stream) {
+    MF_REQUIRE(smooth && offsets && n_experts > 0, "grouped_dynamic_quant: smooth [n_experts, k] and offsets are needed");
+    return quant_rows_entry(xq, x_scale, x, smooth, nullptr, m, k, dtype, layout, stream, offsets, n_experts);
+}
+
+extern "C" int mf_grouped_silu_mul_dynamic_quant(int8_t* xq, float* x_scale, const void* gate_up, const float* smooth,
+                                                 const int32_t* offsets, int n_experts, int rows, int cols,
+                                                 int gate_up_layout, int dtype, int layout, void* stream) {
+    MF_REQUIRE(smooth && offsets && n_experts > 0, "grouped_silu_mul_dynamic_quant: smooth [n_experts, cols] and offsets are needed");
+    return silu_mul_quant_entry(xq, x_scale, gate_up, smooth, rows, cols, gate_up_layout, dtype, layout, stream, offsets,
+                                n_experts);
 }

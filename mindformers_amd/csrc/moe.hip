@@ -266,6 +266,121 @@ __global__ void moe_unpermute_kernel(uint16_t* __restrict__ out, const uint16_t*
     *(u32x4*)(out + (int64_t)t * hidden + i) = o;
 }
 
+
+// ---- router gate projection -------------------------------------------------------------------------
+// logits[t, e] = sum_h x[t, h] * w[e, h], products and sums in fp32 on the fp32 matrix instruction (16 x 16 x 4).
+// The weight (E x H, a few MB) is read once: a workgroup owns 16 experts and one slice of H for up to 64 tokens;
+// its 4 waves take the slice's 64-column chunks in turn and meet in LDS.  Lane (r = lane & 15, g = lane >> 4) loads
+// columns 16 j + 4 g .. + 3 of a chunk for expert r and for token r: the instruction's k index is any bijection as
+// long as both operands use the same one.  With more than one slice the workgroups write partial sums
+// [slice][token][expert] and router_gate_reduce_kernel adds the slices in order (no atomics: results do not depend
+// on scheduling).
+struct RG_F32 {};
+template <typename WT>
+__device__ __forceinline__ f32x4 rg_load4(const void* w, int64_t idx) {
+    if constexpr (std::is_same<WT, RG_F32>::value) {
+        return *(const f32x4*)((const float*)w + idx);
+    } else {
+        const u32x2 v = *(const u32x2*)((const uint16_t*)w + idx);
+        return (f32x4){WT::to_float((uint16_t)(v[0] & 0xffffu)), WT::to_float((uint16_t)(v[0] >> 16)),
+                       WT::to_float((uint16_t)(v[1] & 0xffffu)), WT::to_float((uint16_t)(v[1] >> 16))};
+    }
+}
+
+template <typename WT>
+__device__ __forceinline__ float rg_round(float v) {
+    // a 16-bit router computes in its own type: the projection's output is rounded to it before the cast to fp32
+    if constexpr (std::is_same<WT, RG_F32>::value) return v;
+    else return WT::to_float(WT::from_float(v));
+}
+
+constexpr int RG_TT = 4;                                      // token tiles of 16 per workgroup
+
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void router_gate_kernel(float* __restrict__ out, float* __restrict__ partial,
+                                                          const uint16_t* __restrict__ x, const void* __restrict__ w,
+                                                          int tokens, int E, int H, int k_per_split) {
+    __shared__ f32x4 red[4][RG_TT][64];
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int e0 = blockIdx.x * 16, t0 = blockIdx.z * (16 * RG_TT);
+    const int k_begin = blockIdx.y * k_per_split, k_end = min(H, k_begin + k_per_split);
+    const int64_t wrow = (int64_t)min(e0 + r, E - 1) * H;     // rows past the matrix re-read the last one, never stored
+    int64_t xrow[RG_TT];
+#pragma unroll
+    for (int tt = 0; tt < RG_TT; ++tt) xrow[tt] = (int64_t)min(t0 + 16 * tt + r, tokens - 1) * H;
+    f32x4 acc[RG_TT];
+#pragma unroll
+    for (int tt = 0; tt < RG_TT; ++tt) acc[tt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = k_begin + 64 * wv; k0 < k_end; k0 += 256) {
+        f32x4 wa[4], xb[RG_TT][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + 16 * j + 4 * g;
+            const bool in = k < k_end;                        // H and the slices are multiples of 4
+            const int kc = in ? k : k_begin;
+            wa[j] = rg_load4<WT>(w, wrow + kc);
+#pragma unroll
+            for (int tt = 0; tt < RG_TT; ++tt) xb[tt][j] = rg_load4<T>(x, xrow[tt] + kc);
+            if (!in) {
+                wa[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int tt = 0; tt < RG_TT; ++tt) xb[tt][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int tt = 0; tt < RG_TT; ++tt)
+                    acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[j][i], xb[tt][j][i], acc[tt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int tt = 0; tt < RG_TT; ++tt) red[wv][tt][lane] = acc[tt];
+    __syncthreads();
+    // thread (tt = wave, lane): the sum over the 4 waves, in order.  Lane (r, g) of the instruction's result holds
+    // token r, experts 4 g .. 4 g + 3 of the tile.
+    const int tt = wv;
+    f32x4 v = red[0][tt][lane];
+#pragma unroll
+    for (int q = 1; q < 4; ++q) {
+        const f32x4 u = red[q][tt][lane];
+        v = (f32x4){v[0] + u[0], v[1] + u[1], v[2] + u[2], v[3] + u[3]};
+    }
+    const int t = t0 + 16 * tt + r, e = e0 + 4 * g;
+    if (t >= tokens) return;
+    float* dst = partial ? partial + ((int64_t)blockIdx.y * tokens + t) * E + e : out + (int64_t)t * E + e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (e + i < E) dst[i] = partial ? v[i] : rg_round<WT>(v[i]);
+}
+
+template <typename WT>
+__global__ void router_gate_reduce_kernel(float* __restrict__ out, const float* __restrict__ partial, int64_t n,
+                                          int splits) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = partial[i];
+    for (int s = 1; s < splits; ++s) v += partial[s * n + i];
+    out[i] = rg_round<WT>(v);
+}
+
+struct GatePlan {
+    int splits, k_per_split;
+};
+GatePlan plan_router_gate(int tokens, int E, int H) {
+    const int wgs = ((E + 15) / 16) * ((tokens + 16 * RG_TT - 1) / (16 * RG_TT));
+    int s = 512 / wgs;
+    const int max_s = H / 256 < 1 ? 1 : H / 256;              // at least one chunk per wave
+    s = s < 1 ? 1 : (s > max_s ? max_s : s);
+    GatePlan p;
+    p.k_per_split = ((H + s - 1) / s + 63) / 64 * 64;
+    p.splits = (H + p.k_per_split - 1) / p.k_per_split;
+    return p;
+}
+
 }  // namespace
 
 extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* logits, const float* bias,
@@ -288,6 +403,49 @@ extern "C" int mf_moe_route(void* weights_out, int32_t* index_out, const float* 
     else
         hipLaunchKernelGGL(moe_route_kernel<FP16>, dim3(tokens), dim3(64), 0, (hipStream_t)stream, (uint16_t*)weights_out,
                            index_out, logits, bias, n_experts, k, n_group, topk_group, scale, renorm, biased_weights);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" size_t mf_router_gate_workspace_bytes(int tokens, int n_experts, int hidden) {
+    if (tokens <= 0 || n_experts <= 0 || hidden <= 0) return 0;
+    const GatePlan p = plan_router_gate(tokens, n_experts, hidden);
+    return p.splits > 1 ? (size_t)p.splits * tokens * n_experts * sizeof(float) : 0;
+}
+
+extern "C" int mf_router_gate_gemm(float* logits, const void* x, const void* w, int tokens, int n_experts, int hidden,
+                                   int dtype, int w_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "router_gate_gemm: dtype must be bf16 or fp16");
+    MF_REQUIRE(w_dtype == MF_FP32 || w_dtype == dtype, "router_gate_gemm: the weight is fp32 or of the activation type");
+    if (tokens <= 0) return 0;
+    MF_REQUIRE(logits && x && w, "router_gate_gemm: null argument");
+    MF_REQUIRE(n_experts > 0 && hidden > 0 && hidden % 4 == 0, "router_gate_gemm: hidden (%d) must be a multiple of 4", hidden);
+    MF_REQUIRE(((uintptr_t)x & 7) == 0 && ((uintptr_t)w & (w_dtype == MF_FP32 ? 15 : 7)) == 0,
+               "router_gate_gemm: x must be 8-byte aligned, w 16-byte (fp32) or 8-byte aligned");
+    const GatePlan p = plan_router_gate(tokens, n_experts, hidden);
+    const size_t need = mf_router_gate_workspace_bytes(tokens, n_experts, hidden);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), "router_gate_gemm: workspace of %zu bytes needed, %zu given",
+               need, workspace_bytes);
+    float* partial = p.splits > 1 ? (float*)workspace : nullptr;
+    const dim3 grid((n_experts + 15) / 16, p.splits, (tokens + 16 * RG_TT - 1) / (16 * RG_TT));
+    const int64_t n = (int64_t)tokens * n_experts;
+    const dim3 rgrid((unsigned)((n + 255) / 256));
+#define RG_LAUNCH(TT_, WT_)                                                                                      \
+    {                                                                                                            \
+        hipLaunchKernelGGL((router_gate_kernel<TT_, WT_>), grid, dim3(256), 0, (hipStream_t)stream, logits, partial, \
+                           (const uint16_t*)x, w, tokens, n_experts, hidden, p.k_per_split);                     \
+        if (partial) {                                                                                           \
+            int rc = MF_LAUNCH_CHECK();                                                                          \
+            if (rc) return rc;                                                                                   \
+            hipLaunchKernelGGL((router_gate_reduce_kernel<WT_>), rgrid, dim3(256), 0, (hipStream_t)stream, logits, \
+                               partial, n, p.splits);                                                            \
+        }                                                                                                        \
+    }
+    if (dtype == MF_BF16) {
+        if (w_dtype == MF_FP32) RG_LAUNCH(BF16, RG_F32) else RG_LAUNCH(BF16, BF16)
+    } else {
+        if (w_dtype == MF_FP32) RG_LAUNCH(FP16, RG_F32) else RG_LAUNCH(FP16, FP16)
+    }
+#undef RG_LAUNCH
     return MF_LAUNCH_CHECK();
 }
 

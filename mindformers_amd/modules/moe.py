@@ -2,10 +2,9 @@
 
 Follows mindformers/parallel_core/inference/transformer/moe/{router.py:88-159, experts.py:35-170,
 shared_experts.py:32-75, moe_layer.py:78-163}.  Router scoring, permute, the quantized grouped expert GEMMs and
-the weighted unpermute are HIP kernels; the small dense gate projection is a library GEMM in the router dtype.
+the weighted unpermute and the router's gate projection are HIP kernels.
 """
 import torch
-import torch.nn.functional as F
 from torch import nn
 
 from .. import ops
@@ -36,7 +35,14 @@ class TopKRouter(nn.Module):
         self.expert_bias = nn.Parameter(torch.zeros(self.num_experts, dtype=torch.float32, device=device), requires_grad=False)
 
     def gating(self, input_tensor):
-        return F.linear(input_tensor.to(self.router_dense_type), self.weight)
+        """logits = cast(x, router_dense_type) . weight^T (router.py:54-63), returned in fp32 (the cast of
+        router.py:128); a 16-bit router's projection output is rounded to its type first."""
+        x = input_tensor.reshape(-1, self.hidden)
+        if self.weight.dtype != torch.float32 and x.dtype != self.weight.dtype:
+            x = x.to(self.weight.dtype)
+        if x.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"router input of type {x.dtype}: the gate projection is built for bf16 / fp16 activations")
+        return ops.router_gate(x.contiguous(), self.weight)
 
     def routing(self, logits):
         input_dtype = logits.dtype
@@ -101,12 +107,17 @@ class QuantGroupedMLP(nn.Module):
     ``act_quant="per_token"`` / ``"per_tensor"`` (W8A8, the routed experts of a W8A8 checkpoint such as
     research/deepseek3/deepseek_r1_671b/predict_deepseek_r1_671b_w8a8.yaml:89-92): the permuted rows are quantised per
     token, or with one calibrated scale per projection (``act_scale1`` / ``act_scale2``, loaded with the checkpoint),
-    and both projections run on the int8 matrix cores with exact int32 accumulators."""
+    and both projections run on the int8 matrix cores with exact int32 accumulators.  ``smooth`` (per_token only):
+    the rows of expert e are multiplied by ``smooth_scale1[e]`` [H] in front of the first projection and the
+    activation product by ``smooth_scale2[e]`` [F] in front of the second (outliers_suppression: smooth; the weight
+    side of the pair is folded into the checkpoint's int8 weights)."""
 
-    def __init__(self, num_experts, config, device="cuda", act_quant=None):
+    def __init__(self, num_experts, config, device="cuda", act_quant=None, smooth=False):
         super().__init__()
         if act_quant not in (None, "per_token", "per_tensor"):
             raise ValueError(f"act_quant must be None, 'per_token' or 'per_tensor', got {act_quant!r}")
+        if smooth and act_quant != "per_token":
+            raise NotImplementedError("smooth multipliers on routed experts are built for per_token activations")
         self.config = config
         self.num_experts = num_experts
         self.act_quant = act_quant
@@ -119,6 +130,8 @@ class QuantGroupedMLP(nn.Module):
         static = act_quant == "per_tensor"
         self.register_buffer("act_scale1", torch.ones(1, dtype=torch.float32, device=device) if static else None)
         self.register_buffer("act_scale2", torch.ones(1, dtype=torch.float32, device=device) if static else None)
+        self.register_buffer("smooth_scale1", torch.ones(num_experts, h, dtype=torch.float32, device=device) if smooth else None)
+        self.register_buffer("smooth_scale2", torch.ones(num_experts, f, dtype=torch.float32, device=device) if smooth else None)
         self._p1 = self._p2 = None
 
     @torch.no_grad()
@@ -158,10 +171,15 @@ class QuantGroupedMLP(nn.Module):
             a = ops.grouped_w8a16_linear(hidden_states, self._p1, offsets)       # silu(gate) * hidden included
             return ops.grouped_w8a16_linear(a, self._p2, offsets)
         dt = hidden_states.dtype
-        xq, xs = self._quant(hidden_states.contiguous(), self.act_scale1)
+        if self.smooth_scale1 is not None:
+            xq, xs = ops.dynamic_quant(hidden_states.contiguous(), self.smooth_scale1, offsets=offsets)
+        else:
+            xq, xs = self._quant(hidden_states.contiguous(), self.act_scale1)
         h = ops.grouped_w8a8_linear(xq, xs, self._p1, offsets, out_dtype=dt)
         if self.act_quant == "per_tensor":
             aq, a_s = ops.static_quant(ops.silu_mul(h), self.act_scale2)
+        elif self.smooth_scale2 is not None:
+            aq, a_s = ops.silu_mul_dynamic_quant(h, self.smooth_scale2, offsets=offsets)
         else:
             aq, a_s = ops.silu_mul_dynamic_quant(h)
         return ops.grouped_w8a8_linear(aq, a_s, self._p2, offsets, out_dtype=dt)

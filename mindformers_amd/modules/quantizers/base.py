@@ -165,11 +165,10 @@ def convert_linears(model, cfg, layer_policies=None):
                 # parameters (filled from the checkpoint)
                 setattr(parent, child_name, QuantPagedAttentionMgr.from_float(child))
             elif isinstance(child, GroupedMLP):
-                if pol.act_quant_dtype == "int8" and pol.outliers_suppression == "smooth":
-                    raise NotImplementedError("smooth outlier suppression on routed experts is not built (a multiplier "
-                                              "per expert would have to follow the permuted rows)")
+                act8 = pol.act_quant_dtype == "int8"
                 cell = QuantGroupedMLP(child.num_experts, child.config, child.weight1.device,
-                                       act_quant=pol.act_quant_granularity if pol.act_quant_dtype == "int8" else None)
+                                       act_quant=pol.act_quant_granularity if act8 else None,
+                                       smooth=act8 and pol.outliers_suppression == "smooth")
                 cell.quantize_from_float(child.weight1.data, child.weight2.data)
                 setattr(parent, child_name, cell)
     return model

@@ -737,14 +737,29 @@ def w8a16_gated_linear(x, w, bias=None):
     return y
 
 
-def dynamic_quant(x, smooth=None, tiled=False):
+def _expert_smooth_ok(smooth, offsets, k):
+    _need(smooth is not None and smooth.dtype == torch.float32 and smooth.dim() == 2 and smooth.shape[1] == k
+          and smooth.is_contiguous(), "with offsets, smooth must be contiguous fp32 [E, K]")
+    _need(offsets.dtype == torch.int32 and offsets.numel() == smooth.shape[0] + 1, "offsets must be int32 [E + 1]")
+    return smooth.shape[0]
+
+
+def dynamic_quant(x, smooth=None, tiled=False, offsets=None):
     """DynamicQuant per token (with the smoothing vector folded in): returns (xq, scale fp32 [rows]); xq is int8
-    [..., K] row-major, or with ``tiled`` a TiledInt8Activations for ``w8a8_linear``."""
+    [..., K] row-major, or with ``tiled`` a TiledInt8Activations for ``w8a8_linear``.  With ``offsets`` (int32
+    [E + 1], the row groups of moe_permute) ``smooth`` is [E, K], one multiplier vector per expert."""
     lib = _lib.load()
-    dev = _dev_ok(x, smooth)
+    dev = _dev_ok(x, smooth, offsets)
     _need(x.dtype in _ACT, "x must be bf16/fp16")
     k = x.shape[-1]
     m = x.numel() // k
+    if offsets is not None:
+        e = _expert_smooth_ok(smooth, offsets, k)
+        xq, xs = _quant_out(lib, x.shape, m, k, tiled, dev)
+        check(lib.mf_grouped_dynamic_quant_per_token(ptr(xq), ptr(xs), ptr(x), ptr(smooth), ptr(offsets), e, m, k,
+                                                     dtype_code(x.dtype), 1 if tiled else 0, stream_ptr(dev)),
+              "mf_grouped_dynamic_quant_per_token")
+        return (TiledInt8Activations(xq, x.shape) if tiled else xq), xs
     _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [K]")
     if tiled:
         xq = torch.empty(lib.mf_w8a16_packed_bytes(max(m, 1), k), dtype=torch.int8, device=dev)
@@ -804,17 +819,24 @@ def rms_norm_dynamic_quant(x, gamma, eps, smooth=None, residual=None, tiled=Fals
     return (xq, xs, s) if residual is not None else (xq, xs)
 
 
-def silu_mul_dynamic_quant(gate_up, smooth=None, interleaved=False, tiled=False):
+def silu_mul_dynamic_quant(gate_up, smooth=None, interleaved=False, tiled=False, offsets=None):
     """silu(gate) * up followed by DynamicQuant per token in one kernel (the product is not materialised): returns
-    (xq, scale), bit-identical to silu_mul then dynamic_quant."""
+    (xq, scale), bit-identical to silu_mul then dynamic_quant (``offsets``: as there)."""
     lib = _lib.load()
-    dev = _dev_ok(gate_up, smooth)
+    dev = _dev_ok(gate_up, smooth, offsets)
     _need(gate_up.dtype in _ACT and gate_up.shape[-1] % 2 == 0, "gate_up must be bf16/fp16 with an even last dim")
     k = gate_up.shape[-1] // 2
     m = gate_up.numel() // (2 * k)
-    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [F]")
     shape = (*gate_up.shape[:-1], k)
     xq, xs = _quant_out(lib, shape, m, k, tiled, dev)
+    if offsets is not None:
+        e = _expert_smooth_ok(smooth, offsets, k)
+        check(lib.mf_grouped_silu_mul_dynamic_quant(ptr(xq), ptr(xs), ptr(gate_up), ptr(smooth), ptr(offsets), e, m, k,
+                                                    1 if interleaved else 0, dtype_code(gate_up.dtype),
+                                                    1 if tiled else 0, stream_ptr(dev)),
+              "mf_grouped_silu_mul_dynamic_quant")
+        return (TiledInt8Activations(xq, shape) if tiled else xq), xs
+    _need(smooth is None or (smooth.dtype == torch.float32 and smooth.numel() == k), "smooth must be fp32 [F]")
     check(lib.mf_silu_mul_dynamic_quant(ptr(xq), ptr(xs), ptr(gate_up), ptr(smooth), m, k, 1 if interleaved else 0,
                                         dtype_code(gate_up.dtype), 1 if tiled else 0, stream_ptr(dev)),
           "mf_silu_mul_dynamic_quant")
@@ -921,6 +943,25 @@ def w8a8_qkv_rope_and_cache(xq, x_scale, w, cos, sin, key_cache, value_cache, sl
 
 
 # --------------------------------------------------------------------------------------------- MoE
+def router_gate(x, weight):
+    """The router's dense projection: fp32 logits [T, E] = x . weight^T.  weight [E, H] fp32 (fp32 products and sums)
+    or of x's 16-bit type (the projection output is then rounded to that type, as a 16-bit dense cell returns it)."""
+    lib = _lib.load()
+    dev = _dev_ok(x, weight)
+    _need(x.dtype in _ACT and x.dim() == 2 and x.is_contiguous(), "x must be contiguous bf16/fp16 [T, H]")
+    _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.is_contiguous()
+          and weight.dtype in (torch.float32, x.dtype), "weight must be contiguous [E, H], fp32 or of x's type")
+    t, h = x.shape
+    e = weight.shape[0]
+    logits = torch.empty(t, e, dtype=torch.float32, device=dev)
+    need = lib.mf_router_gate_workspace_bytes(t, e, h)
+    ws = workspace(need, dev, "gemm") if need else None
+    w_code = 2 if weight.dtype == torch.float32 else dtype_code(weight.dtype)
+    check(lib.mf_router_gate_gemm(ptr(logits), ptr(x), ptr(weight), t, e, h, dtype_code(x.dtype), w_code, ptr(ws),
+                                  ws.numel() if ws is not None else 0, stream_ptr(dev)), "mf_router_gate_gemm")
+    return logits
+
+
 def moe_route(logits, expert_bias, k, n_group, topk_group, scale, out_dtype, renorm=True, biased_weights=False):
     """FusedAddTopKDiv: (expert_weight [T,k] out_dtype, expert_index [T,k] int32) from fp32 logits [T,E]."""
     lib = _lib.load()

@@ -1032,6 +1032,37 @@ def test_dynamic_quant_tiled_layout_bit_exact(m, k):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("counts,k", [([5, 0, 17, 1, 0, 40], 256), ([0, 0, 3], 7168), ([64] * 16, 2048), ([1], 64)])
+def test_grouped_dynamic_quant_bit_exact(dtype, tiled, counts, k):
+    """Rows grouped by expert, one multiplier vector per expert (empty experts, a single expert, an empty leading
+    run): every row is quantised exactly as the ungrouped call with its expert's vector quantises it, and the fused
+    SiLU * up form equals silu_mul followed by the grouped call."""
+    rng = np.random.default_rng(len(counts) + k)
+    e, m = len(counts), int(sum(counts))
+    offsets = np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
+    x = rounded(rng.normal(size=(m, k)) * 3, dtype)
+    sm = rng.uniform(0.5, 2.0, (e, k)).astype(np.float32)
+    sm_t, off_t = torch.from_numpy(sm).cuda(), torch.from_numpy(offsets).cuda()
+    xq, xs = ops.dynamic_quant(dev(x, dtype), sm_t, tiled=tiled, offsets=off_t)
+    got = untile_int8(to_np(xq.data), m, k) if tiled else to_np(xq)
+    for i in range(e):
+        a, b = offsets[i], offsets[i + 1]
+        q_ref, s_ref = O.dynamic_quant_per_token(x[a:b], sm[i])
+        assert np.array_equal(got[a:b], q_ref) and np.array_equal(to_np(xs)[a:b], s_ref), f"expert {i}"
+    gu = dev(rounded(rng.normal(size=(m, 2 * k)), dtype), dtype)
+    fq, fs = ops.silu_mul_dynamic_quant(gu, sm_t, tiled=tiled, offsets=off_t)
+    uq, us = ops.dynamic_quant(ops.silu_mul(gu), sm_t, tiled=tiled, offsets=off_t)
+    if tiled:                                                     # padding bytes of the tile order are left unwritten
+        assert np.array_equal(untile_int8(to_np(fq.data), m, k), untile_int8(to_np(uq.data), m, k))
+    else:
+        assert torch.equal(fq, uq)
+    assert torch.equal(fs, us)
+    with pytest.raises(ValueError):
+        ops.dynamic_quant(dev(x, dtype), sm_t[0], offsets=off_t)          # one vector where a table is needed
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,smooth,residual,tiled", [(256, 3584, True, False, True), (5, 512, False, True, False),
                                                        (33, 16384, True, True, True), (1, 64, True, False, False)])
 def test_rms_norm_dynamic_quant_equals_unfused(dtype, m, k, smooth, residual, tiled):
@@ -1153,6 +1184,37 @@ def test_w8a8_qkv_rope_and_cache_equals_unfused(dtype, t, n_head, n_kv, d, k, bi
     ops.rope_and_cache(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], cos, sin, kc2, vc2, slots_t, n_head)
     assert torch.equal(q1, qkv[:, :nq])
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,e,h,wdt", [(64, 256, 7168, "fp32"), (1, 256, 7168, "fp32"), (200, 64, 2048, "fp32"),
+                                       (7, 20, 260, "fp32"), (64, 256, 7168, "same"), (33, 8, 64, "same")])
+def test_router_gate_projection(dtype, t, e, h, wdt):
+    """The router's dense projection with fp32 accumulation: against the float64 product (an fp32 sum of h terms,
+    whatever its order, is within h * 2^-24 of sum |terms|); with small integers everywhere the result is exact, which
+    catches a dropped or doubled column at the slice and chunk borders (h = 260 ends inside a chunk); a 16-bit weight
+    gives logits that are values of that type."""
+    rng = np.random.default_rng(t + e + h)
+    x = rounded(rng.normal(size=(t, h)), dtype)
+    w = rng.normal(0, 0.02, (e, h)).astype(np.float32)
+    if wdt == "same":
+        w = rounded(w, dtype)
+    w_t = torch.from_numpy(w).cuda() if wdt == "fp32" else dev(w, dtype)
+    got = to_np(ops.router_gate(dev(x, dtype), w_t))
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    mag = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T
+    if wdt == "same":
+        assert np.array_equal(got, rounded(got, dtype))
+        assert_within(got, ref, np.abs(ref), dtype, ulps=1.0, extra=h * 2.0 ** -24 * mag, what="router gate (16-bit)")
+    else:
+        assert np.all(np.abs(got - ref) <= h * 2.0 ** -24 * mag + 1e-12)
+    xi = rng.integers(-3, 4, (t, h)).astype(np.float32)
+    wi = rng.integers(-4, 5, (e, h)).astype(np.float32)
+    wi_t = torch.from_numpy(wi).cuda() if wdt == "fp32" else dev(wi, dtype)
+    exact = xi.astype(np.int64) @ wi.astype(np.int64).T
+    got_i = to_np(ops.router_gate(dev(xi, dtype), wi_t)).astype(np.float64)
+    want = exact.astype(np.float64) if wdt == "fp32" else rounded(exact, dtype).astype(np.float64)
+    assert np.array_equal(got_i, want)
 
 
 @pytest.mark.parametrize("t,e,k,ng,tg", [(128, 256, 8, 8, 4), (16, 8, 2, 2, 2), (33, 64, 6, 8, 3), (5, 16, 4, 1, 1), (7, 96, 3, 4, 1),

@@ -945,7 +945,7 @@ def test_mcore_flash_attention_over_int8_caches():
     assert_within(to_np(out), ref, mag, dt, ulps=3.0, what="FlashAttention over int8 caches")
 
 
-@pytest.mark.parametrize("granularity", ["per_token", "per_tensor"])
+@pytest.mark.parametrize("granularity", ["per_token", "per_tensor", "per_token+smooth"])
 def test_moe_layer_w8a8_experts_vs_oracle(granularity):
     """The reference's own W8A8 recipe for the routed experts (quant_method ptq, int8 weights and activations,
     research/deepseek3/deepseek_r1_671b/predict_deepseek_r1_671b_w8a8.yaml:89-92; its default activation granularity is
@@ -962,6 +962,8 @@ def test_moe_layer_w8a8_experts_vs_oracle(granularity):
                             moe_router_num_groups=4, add_bias_linear=False, gated_linear_unit=True,
                             compute_dtype="bfloat16", params_dtype="bfloat16", moe_router_dtype="bfloat16",
                             moe_router_enable_expert_bias=True, moe_router_score_function="sigmoid")
+    smooth = granularity.endswith("+smooth")      # one multiplier vector per expert in front of each projection
+    granularity = granularity.split("+")[0]
     torch.manual_seed(3)
     net = MoELayer(cfg)
     net.router.weight.data.normal_(0, 0.3)
@@ -970,9 +972,19 @@ def test_moe_layer_w8a8_experts_vs_oracle(granularity):
     net.experts.weight2.data.normal_(0, 0.3)
     router_w, router_b = to_np(net.router.weight), to_np(net.router.expert_bias)
     q = AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8",
-                                   "act_quant_granularity": granularity, "modules_to_not_convert": ["router"]})
+                                   "act_quant_granularity": granularity, "modules_to_not_convert": ["router"],
+                                   "outliers_suppression": "smooth" if smooth else "None"})
     q.preprocess_model(net)
     assert isinstance(net.experts, QuantGroupedMLP) and net.experts.act_quant == granularity
+    sm_rng = np.random.default_rng(12)
+    sm1 = sm_rng.uniform(0.5, 2.0, (8, 64)).astype(np.float32) if smooth else None
+    sm2 = sm_rng.uniform(0.5, 2.0, (8, 32)).astype(np.float32) if smooth else None
+    if smooth:
+        assert net.experts.smooth_scale1.shape == (8, 64) and net.experts.smooth_scale2.shape == (8, 32)
+        net.experts.smooth_scale1.copy_(torch.from_numpy(sm1))
+        net.experts.smooth_scale2.copy_(torch.from_numpy(sm2))
+    else:
+        assert net.experts.smooth_scale1 is None
     s1, s2 = np.float32(0.03), np.float32(0.25)
     if granularity == "per_tensor":
         net.experts.act_scale1.fill_(float(s1))
@@ -988,12 +1000,21 @@ def test_moe_layer_w8a8_experts_vs_oracle(granularity):
     wgt = _r(wgt, "bf16")
     px, row_map, counts = O.moe_permute(x, idx, e)
 
-    def quant(a, s):
-        return O.dynamic_quant_per_token(a.astype(np.float32)) if granularity == "per_token" else \
-            O.static_quant_per_tensor(a.astype(np.float32), s)
+    def quant(a, s, sm=None):
+        if granularity == "per_tensor":
+            return O.static_quant_per_tensor(a.astype(np.float32), s)
+        if sm is None:
+            return O.dynamic_quant_per_token(a.astype(np.float32))
+        aq_, as_ = np.zeros(a.shape, np.int8), np.zeros(a.shape[0], np.float32)
+        st = 0
+        for i_, c_ in enumerate(counts):                          # the rows of expert i_ take its multiplier vector
+            c_ = int(c_)
+            aq_[st:st + c_], as_[st:st + c_] = O.dynamic_quant_per_token(a[st:st + c_].astype(np.float32), sm[i_])
+            st += c_
+        return aq_, as_
     y = np.zeros((px.shape[0], w2.shape[1]))
     start = 0
-    xq, xs = quant(px, s1)
+    xq, xs = quant(px, s1, sm1)
     h = np.zeros((px.shape[0], w1.shape[1]))
     for i, c in enumerate(counts):
         c = int(c)
@@ -1002,7 +1023,7 @@ def test_moe_layer_w8a8_experts_vs_oracle(granularity):
     h = _r(h, "bf16")
     f = h.shape[1] // 2
     a = _r(_r(Dn.silu(h[:, :f]), "bf16") * h[:, f:], "bf16")
-    aq, a_s = quant(a, s2)
+    aq, a_s = quant(a, s2, sm2)
     start = 0
     for i, c in enumerate(counts):
         c = int(c)
