@@ -154,6 +154,38 @@ int mf_paged_attention_prefill_int8kv(void* out, const void* query, const void* 
                                       int num_blocks, float scale, int64_t q_row_stride, int dtype,
                                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* int8 KV caches quantised per token (kvcache_quant_granularity per_token,
+ * mindformers/utils/quantization_config.py:206-207,296-300: needs an int8 cache): the cache write, and the two
+ * attention entry points on such caches.  Every cached token row (all kv heads of a token) has one fp32 scale in
+ * key_scale_cache / value_scale_cache [num_blocks * block_size], indexed by slot like the rows.
+ * mf_dynamic_quant_reshape_and_cache: s = max|row| / 127, q = clip(rint(x / s), -128, 127) in float32 as
+ * mf_dynamic_quant_per_token defines it (a zero row stores s = 0 and zeros); the int8 row and s go to
+ * slot_mapping[t]; negative or out-of-range slots are skipped.  Strides as mf_reshape_and_cache.
+ * Attention: K_b[j] = key_cache[slot j] * key_scale_cache[slot j], V_b[j] likewise; the score of token j is
+ * multiplied by its key scale, its probability by its value scale before the rounding to `dtype` in front of the PV
+ * product; the denominator sums the unscaled fp32 probabilities.  block_size % 4 == 0; scale caches 16-byte
+ * aligned.  Everything else as mf_paged_attention_decode / mf_paged_attention_prefill (paged form only).  The
+ * arithmetic of the reference's per-token cells is not in the reference: this is the build's declared convention. */
+int mf_dynamic_quant_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                                       float* key_scale_cache, float* value_scale_cache, const int32_t* slot_mapping,
+                                       int num_tokens, int n_kv_heads, int head_dim, int64_t num_slots,
+                                       int64_t key_row_stride, int64_t value_row_stride, int dtype, void* stream);
+int mf_paged_attention_decode_int8kv_per_token(void* out, const void* query, const void* key_cache,
+                                               const void* value_cache, const float* key_scale_cache,
+                                               const float* value_scale_cache, const int32_t* block_tables,
+                                               const int32_t* context_lens, int batch, int n_heads, int n_kv_heads,
+                                               int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                                               float scale, int64_t q_row_stride, int dtype, void* workspace,
+                                               size_t workspace_bytes, void* stream);
+int mf_paged_attention_prefill_int8kv_per_token(void* out, const void* query, const void* key_cache,
+                                                const void* value_cache, const float* key_scale_cache,
+                                                const float* value_scale_cache, const int32_t* block_tables,
+                                                const int32_t* context_lens, const int32_t* q_starts, int batch,
+                                                int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                                int max_blocks_per_seq, int num_blocks, float scale,
+                                                int64_t q_row_stride, int dtype, void* workspace,
+                                                size_t workspace_bytes, void* stream);
+
 /* ---- attention over several new tokens per sequence (prefill, chunked prefill, parallel decoding) -- */
 
 /* Bytes of scratch mf_paged_attention_prefill needs (0 when one partition spans the context).  max_context is

@@ -33,6 +33,11 @@ SIGNATURES = {
                                               _Z, _P]),
     "mf_paged_attention_prefill_int8kv": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _L,
                                                _I, _P, _Z, _P]),
+    "mf_dynamic_quant_reshape_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _P]),
+    "mf_paged_attention_decode_int8kv_per_token": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
+                                                        _L, _I, _P, _Z, _P]),
+    "mf_paged_attention_prefill_int8kv_per_token": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                                                         _I, _F, _L, _I, _P, _Z, _P]),
     "mf_mla_paged_attention_workspace_bytes": (_Z, [_I, _I, _I]),
     "mf_mla_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P, _Z, _P]),
     "mf_mla_absorb_bmm": (_I, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _I, _P]),

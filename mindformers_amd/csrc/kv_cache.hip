@@ -167,6 +167,33 @@ __global__ void quant_reshape_and_cache_kernel(const uint16_t* __restrict__ key,
     }
 }
 
+// Per-token int8 cache write: the row of all kv heads of a token is quantised as the per-token dynamic
+// quantisation defines it (s = max|row| / 127 in float32, q = clip(rint(x / s), -128, 127) with a true float32
+// division; a zero row gets s = 0 and zeros), the int8 row goes to the token's slot and s to the same slot of the
+// scale cache.  grid (tokens, 2): y = 0 keys, y = 1 values.
+template <typename T>
+__global__ __launch_bounds__(256) void dynamic_quant_reshape_and_cache_kernel(
+    const uint16_t* __restrict__ key, const uint16_t* __restrict__ value, int8_t* __restrict__ key_cache,
+    int8_t* __restrict__ value_cache, float* __restrict__ key_scale_cache, float* __restrict__ value_scale_cache,
+    const int32_t* __restrict__ slot_mapping, int row, int64_t num_slots, int64_t k_stride, int64_t v_stride) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, which = blockIdx.y;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0 || slot >= num_slots) return;                // uniform over the workgroup
+    const uint16_t* src = which ? value + (int64_t)t * v_stride : key + (int64_t)t * k_stride;
+    int8_t* dst = (which ? value_cache : key_cache) + slot * row;
+    float amax = 0.f;
+    for (int c = threadIdx.x; c < row; c += blockDim.x) amax = fmaxf(amax, fabsf(T::to_float(src[c])));
+    amax = block_max(amax, red);
+    const float s = __fdiv_rn(amax, 127.0f);
+    const float safe = s > 0.f ? s : 1.0f;
+    if (threadIdx.x == 0) (which ? value_scale_cache : key_scale_cache)[slot] = s;
+    for (int c = threadIdx.x; c < row; c += blockDim.x) {
+        const float q = rintf(__fdiv_rn(T::to_float(src[c]), safe));
+        dst[c] = (int8_t)fminf(fmaxf(q, -128.f), 127.f);
+    }
+}
+
 }  // namespace
 
 extern "C" int mf_quant_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
@@ -192,6 +219,37 @@ extern "C" int mf_quant_reshape_and_cache(const void* key, const void* value, vo
         hipLaunchKernelGGL(quant_reshape_and_cache_kernel<FP16>, grid, dim3(256), 0, (hipStream_t)stream,
                            (const uint16_t*)key, (const uint16_t*)value, (int8_t*)key_cache, (int8_t*)value_cache,
                            slot_mapping, scale, offset, row, num_slots, key_row_stride, value_row_stride);
+    return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_dynamic_quant_reshape_and_cache(const void* key, const void* value, void* key_cache,
+                                                  void* value_cache, float* key_scale_cache,
+                                                  float* value_scale_cache, const int32_t* slot_mapping,
+                                                  int num_tokens, int n_kv_heads, int head_dim, int64_t num_slots,
+                                                  int64_t key_row_stride, int64_t value_row_stride, int dtype,
+                                                  void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "dynamic_quant_reshape_and_cache: dtype must be bf16 or fp16");
+    if (num_tokens == 0) return 0;
+    MF_REQUIRE(key && value && key_cache && value_cache && key_scale_cache && value_scale_cache && slot_mapping,
+               "dynamic_quant_reshape_and_cache: null argument");
+    MF_REQUIRE(num_tokens > 0 && n_kv_heads > 0 && head_dim > 0 && num_slots > 0,
+               "dynamic_quant_reshape_and_cache: bad sizes");
+    const int row = n_kv_heads * head_dim;
+    if (key_row_stride <= 0) key_row_stride = row;
+    if (value_row_stride <= 0) value_row_stride = row;
+    MF_REQUIRE(key_row_stride >= row && value_row_stride >= row,
+               "dynamic_quant_reshape_and_cache: row stride smaller than a row");
+    dim3 grid(num_tokens, 2);
+    if (dtype == MF_BF16)
+        hipLaunchKernelGGL(dynamic_quant_reshape_and_cache_kernel<BF16>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)key, (const uint16_t*)value, (int8_t*)key_cache, (int8_t*)value_cache,
+                           key_scale_cache, value_scale_cache, slot_mapping, row, num_slots, key_row_stride,
+                           value_row_stride);
+    else
+        hipLaunchKernelGGL(dynamic_quant_reshape_and_cache_kernel<FP16>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)key, (const uint16_t*)value, (int8_t*)key_cache, (int8_t*)value_cache,
+                           key_scale_cache, value_scale_cache, slot_mapping, row, num_slots, key_row_stride,
+                           value_row_stride);
     return MF_LAUNCH_CHECK();
 }
 

@@ -12,8 +12,8 @@ static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 
 // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
 // first tile, merge) exposed: twice the tokens per workgroup at every context length (fewer partitions than the
 // workspace query, which does not know the cache type, sizes for).
-static inline int pa_launch_tiles_per_wave(int64_t max_context, bool kv8) {
-    return kv8 ? 4 : pa_tiles_per_wave(max_context);
+static inline int pa_launch_tiles_per_wave(int64_t max_context, int kvq) {
+    return kvq ? 4 : pa_tiles_per_wave(max_context);
 }
 
 // Per-token quantisation of the output rows requested together with the attention itself.
@@ -24,7 +24,7 @@ struct PaQuantArgs {
     int layout;
 };
 
-template <typename T, int D, bool KV8>
+template <typename T, int D, int KVQ>
 int launch_pa(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads, int n_kv,
               int block_size, int max_blocks, int num_blocks, float scale, int64_t q_stride, void* workspace,
@@ -32,7 +32,7 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    const int tpw = pa_launch_tiles_per_wave(max_ctx, KV8);
+    const int tpw = pa_launch_tiles_per_wave(max_ctx, KVQ);
     const int part_tokens = tpw * PA_WAVE_TOKENS;
     const int max_parts = (int)((max_ctx + part_tokens - 1) / part_tokens);
     float* part_out = (float*)workspace;
@@ -41,7 +41,7 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     dim3 grid((unsigned)((int64_t)batch * max_parts * n_kv * head_groups));
     const bool tib = block_size % PA_TILE == 0;               // a 32-token tile never straddles two blocks
 #define PA_LAUNCH(TPWV, TIBV)                                                                                    \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false, KV8, TIBV>), grid, dim3(PA_WAVES * 64), 0, st,  \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, TPWV, false, KVQ, TIBV>), grid, dim3(PA_WAVES * 64), 0, st,  \
                        (uint16_t*)out, part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,      \
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
@@ -95,10 +95,15 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
                            const int32_t* block_tables, const int32_t* context_lens, int batch, int n_heads,
                            int n_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
                            float scale, int64_t q_row_stride, int dtype, void* workspace, size_t workspace_bytes,
-                           void* stream, bool kv8, const float* kv_scale, const float* kv_offset,
+                           void* stream, int kvq, const float* kv_scale, const float* kv_offset,
                            const PaQuantArgs* qa = nullptr) {
+    // kvq: 0 = 16-bit caches, 1 = int8 with per-channel scale / offset, 2 = int8 with per-token key scales
+    // (kv_scale) and value scales (kv_offset), one float per cache slot
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention: dtype must be bf16 or fp16");
-    MF_REQUIRE(!kv8 || kv_scale, "paged_attention: an int8 cache needs its scales");
+    MF_REQUIRE(!kvq || kv_scale, "paged_attention: an int8 cache needs its scales");
+    MF_REQUIRE(kvq != 2 || (kv_offset && block_size % 4 == 0 && (((uintptr_t)kv_scale | (uintptr_t)kv_offset) & 15) == 0),
+               "paged_attention: per-token scales need both 16-byte aligned scale caches and a block size that is a "
+               "multiple of 4");
     if (batch == 0) return 0;
     MF_REQUIRE(out && query && key_cache && value_cache && block_tables && context_lens,
                "paged_attention: null argument");
@@ -121,7 +126,7 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
     hipStream_t st = (hipStream_t)stream;
     // with one partition the attention kernel writes the output rows itself and skips sequences without context
     const int64_t launch_part_tokens =
-        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kv8) * PA_WAVE_TOKENS;
+        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kvq) * PA_WAVE_TOKENS;
     if ((int64_t)max_blocks_per_seq * block_size <= launch_part_tokens) {
         hipLaunchKernelGGL(pa_zero_empty_kernel, dim3(batch), dim3(128), 0, st, (uint16_t*)out, context_lens,
                            n_heads * head_dim);
@@ -129,13 +134,16 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
         if (rc) return rc;
     }
     void* ws = need ? workspace : nullptr;
+#define PA_CASE_Q(TT, DD, QQ)                                                                                   \
+    return launch_pa<TT, DD, QQ>(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,  \
+                                 n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride, ws, st, \
+                                 kvq ? kv_scale : nullptr, kvq ? kv_offset : nullptr, qa)
 #define PA_CASE(TT, DD)                                                                                        \
-    return kv8 ? launch_pa<TT, DD, true>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
-                                         n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
-                                         q_row_stride, ws, st, kv_scale, kv_offset, qa)                        \
-               : launch_pa<TT, DD, false>(out, query, key_cache, value_cache, block_tables, context_lens, batch, \
-                                          n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
-                                          q_row_stride, ws, st, nullptr, nullptr, qa)
+    {                                                                                                          \
+        if (kvq == 2) PA_CASE_Q(TT, DD, 2);                                                                    \
+        if (kvq == 1) PA_CASE_Q(TT, DD, 1);                                                                    \
+        PA_CASE_Q(TT, DD, 0);                                                                                  \
+    }
     if (dtype == MF_BF16) {
         if (head_dim == 32) PA_CASE(BF16, 32);
         if (head_dim == 64) PA_CASE(BF16, 64);
@@ -146,6 +154,7 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
         PA_CASE(FP16, 128);
     }
 #undef PA_CASE
+#undef PA_CASE_Q
 }
 
 extern "C" int mf_paged_attention_decode(void* out, const void* query, const void* key_cache,
@@ -156,7 +165,7 @@ extern "C" int mf_paged_attention_decode(void* out, const void* query, const voi
                                          size_t workspace_bytes, void* stream) {
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
-                           dtype, workspace, workspace_bytes, stream, false, nullptr, nullptr);
+                           dtype, workspace, workspace_bytes, stream, 0, nullptr, nullptr);
 }
 
 extern "C" int mf_paged_attention_decode_dynamic_quant(void* out, int8_t* xq, float* x_scale, const float* smooth,
@@ -176,7 +185,7 @@ extern "C" int mf_paged_attention_decode_dynamic_quant(void* out, int8_t* xq, fl
     const PaQuantArgs qa = {xq, x_scale, smooth, xq_layout};
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
-                           dtype, workspace, workspace_bytes, stream, false, nullptr, nullptr, &qa);
+                           dtype, workspace, workspace_bytes, stream, 0, nullptr, nullptr, &qa);
 }
 
 extern "C" int mf_paged_attention_decode_int8kv(void* out, const void* query, const void* key_cache,
@@ -189,7 +198,20 @@ extern "C" int mf_paged_attention_decode_int8kv(void* out, const void* query, co
                                                 size_t workspace_bytes, void* stream) {
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
-                           dtype, workspace, workspace_bytes, stream, true, antiquant_scale, antiquant_offset);
+                           dtype, workspace, workspace_bytes, stream, 1, antiquant_scale, antiquant_offset);
+}
+
+extern "C" int mf_paged_attention_decode_int8kv_per_token(void* out, const void* query, const void* key_cache,
+                                                          const void* value_cache, const float* key_scale_cache,
+                                                          const float* value_scale_cache, const int32_t* block_tables,
+                                                          const int32_t* context_lens, int batch, int n_heads,
+                                                          int n_kv_heads, int head_dim, int block_size,
+                                                          int max_blocks_per_seq, int num_blocks, float scale,
+                                                          int64_t q_row_stride, int dtype, void* workspace,
+                                                          size_t workspace_bytes, void* stream) {
+    return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
+                           n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
+                           dtype, workspace, workspace_bytes, stream, 2, key_scale_cache, value_scale_cache);
 }
 
 // ---- decode attention for callers that cannot allocate ----------------------------------------------------------
@@ -237,5 +259,5 @@ extern "C" int mf_paged_attention_decode_static(void* out, const void* query, co
     // every partial a row's combine reads is written by this call's attention kernel first: nothing to clear
     return pa_decode_entry(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,
                            n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale, q_row_stride,
-                           dtype, ws, (size_t)MF_PA_STATIC_SCRATCH_BYTES, stream, false, nullptr, nullptr);
+                           dtype, ws, (size_t)MF_PA_STATIC_SCRATCH_BYTES, stream, 0, nullptr, nullptr);
 }

@@ -73,11 +73,16 @@ __device__ inline void pf_seq(int s, const int32_t* __restrict__ q_starts, const
 // folded into the query, the key offset shifts every score of a column by the same amount and drops out of the
 // softmax, the value scale and offset are applied once to the (accumulator, sum) pair; the int8 tiles are widened
 // to T (exactly) when they are staged in LDS, so the MFMA path is the same.
-template <typename T, int D, int TPW, bool PF, bool KV8, bool TIB>
+// KVQ = 2: int8 caches quantised per token (one scale per cached token row, shared by its heads): kv_scale points at
+// the key scales and kv_offset at the value scales, float [num_blocks * block_size] each, indexed by slot.  The score
+// of a token is multiplied by its key scale, its probability by its value scale before it is rounded to T for the PV
+// product (the denominator sums the unscaled probabilities).  The scales of a tile are loaded one tile ahead, like
+// the tile itself.  KVQ = 1 is the per-channel form above, 0 a 16-bit cache.
+template <typename T, int D, int TPW, bool PF, int KVQ, bool TIB>
 // Decode over an int8 cache keeps half the prefetch registers of a 16-bit one and fits four workgroups on a compute
 // unit (128 registers; measured 6 % faster than with three); the 16-bit kernel needs 166 registers for its two
 // prefetched tiles and gained nothing from a one-tile variant that fits four, so it stays at three.
-__global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void paged_attention_kernel(
+__global__ __launch_bounds__(PA_WAVES * 64, (!PF && KVQ == 1 && TIB) ? 4 : 3) void paged_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
@@ -85,6 +90,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
     float scale_log2, int64_t q_stride, int batch, const int32_t* __restrict__ q_starts, int pf_part_tokens,
     int64_t pf_kv_stride, int pf_rows, const float* __restrict__ kv_scale, const float* __restrict__ kv_offset) {
     using vec8 = typename T::vec8;
+    constexpr bool KV8 = KVQ != 0;
     constexpr int KS = D / 32;
     constexpr int VSTRIDE = PaSmem<D>::VSTRIDE;
     // tokens per partition: fixed by TPW in decode, chosen by the host (a multiple of 128) in PF, where the
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
         for (int j = 0; j < KS; ++j) {
             u32x4 v = {0u, 0u, 0u, 0u};
             if (head_ok) v = *(const u32x4*)(qp + 32 * j);
-            if constexpr (KV8) {                              // fold the per-channel key scale into the query
+            if constexpr (KVQ == 1) {                         // fold the per-channel key scale into the query
                 float f[8];
                 unpack8<T>(v, f);
                 const float* ks = kv_scale + kvh * D + 32 * j + 8 * g;
@@ -301,13 +307,37 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
         }
     };
 
+    // KVQ = 2: the scales of tokens tstart + 16 s + 4 g .. + 3 (the tokens whose scores this lane holds), s = 0, 1.
+    // Groups past the context read the scales of the sequence's first tokens: their scores are masked and their
+    // value scales replaced by zero where they are used.
+    auto load_scales = [&](f32x4* reg, const float* __restrict__ cache, int64_t slot0, int tstart) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            if constexpr (TIB) {
+                reg[s2] = *(const f32x4*)(cache + slot0 + 16 * s2 + 4 * g);       // inside the tile's block
+            } else {
+                int tok = tstart + 16 * s2 + 4 * g;                                // block sizes are multiples of 4
+                tok = tok < L ? tok : 0;
+                const int bi = tok / block_size;
+                int blk = table[bi];
+                blk = (blk < 0 || blk >= num_blocks) ? 0 : blk;
+                reg[s2] = *(const f32x4*)(cache + (int64_t)blk * block_size + (tok - bi * block_size));
+            }
+        }
+    };
+
     const int tstep = PA_WAVES * PA_TILE;
     const int tfirst = part_start + wu * PA_TILE;
     int64_t slot_cur = tile_slot(tfirst), slot_nxt = tile_slot(tfirst + tstep);
     u32x4 kreg[NI], vreg[NI];
+    [[maybe_unused]] f32x4 ksc[2], vsc[2];                    // KVQ = 2: token scales of the tile in kreg / vreg
     if (ntiles > 0) {
         load_tile(kreg, kc, slot_cur, tfirst);
         load_tile(vreg, vc, slot_cur, tfirst);
+        if constexpr (KVQ == 2) {
+            load_scales(ksc, kv_scale, slot_cur, tfirst);
+            load_scales(vsc, kv_offset, slot_cur, tfirst);
+        }
     }
     // the query is complete before the tile loop: a load still pending at the loop head from the entry path only
     // would make the compiler wait for every outstanding load at its first use inside the loop
@@ -342,13 +372,26 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
                 sc[s] = T::mfma16(bitcast<vec8>(ka), qreg[j], sc[s]);
             }
         }
+        // KVQ = 2: this tile's token scales leave their registers here; the next tile's follow one tile ahead of use
+        [[maybe_unused]] f32x4 kts[2], vts[2];
+        if constexpr (KVQ == 2) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                kts[s] = ksc[s] * scale_log2;
+                vts[s] = vsc[s];
+            }
+            if constexpr (more) {
+                load_scales(ksc, kv_scale, slot_nxt, tnext);
+                load_scales(vsc, kv_offset, slot_nxt, tnext);
+            }
+        }
         float tmax = PA_NEG;
         if (tstart + PA_TILE <= Lmask) {                      // every token of the tile is visible to every column
 #pragma unroll
             for (int s = 0; s < 2; ++s)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    sc[s][i] *= scale_log2;
+                    if constexpr (KVQ == 2) sc[s][i] *= kts[s][i]; else sc[s][i] *= scale_log2;
                     tmax = fmaxf(tmax, sc[s][i]);
                 }
         } else {
@@ -357,7 +400,14 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int tok = tstart + s * 16 + 4 * g + i;
-                    const float v = tok < Lcol ? sc[s][i] * scale_log2 : PA_NEG;
+                    float scaled;
+                    if constexpr (KVQ == 2) {
+                        scaled = sc[s][i] * kts[s][i];
+                        if (tok >= L) vts[s][i] = 0.f;        // whatever the cache holds there
+                    } else {
+                        scaled = sc[s][i] * scale_log2;
+                    }
+                    const float v = tok < Lcol ? scaled : PA_NEG;
                     sc[s][i] = v;
                     tmax = fmaxf(tmax, v);
                 }
@@ -373,6 +423,12 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
         for (int s = 0; s < 2; ++s) {
             float p0 = __builtin_amdgcn_exp2f(sc[s][0] - m_new), p1 = __builtin_amdgcn_exp2f(sc[s][1] - m_new);
             float p2 = __builtin_amdgcn_exp2f(sc[s][2] - m_new), p3 = __builtin_amdgcn_exp2f(sc[s][3] - m_new);
+            if constexpr (KVQ == 2) {                         // the value's token scale rides on its probability
+                psum += (p0 + p1) + (p2 + p3);
+                pp[2 * s] = pack2<T>(p0 * vts[s][0], p1 * vts[s][1]);
+                pp[2 * s + 1] = pack2<T>(p2 * vts[s][2], p3 * vts[s][3]);
+                continue;
+            }
             pp[2 * s] = pack2<T>(p0, p1);
             pp[2 * s + 1] = pack2<T>(p2, p3);
             // the denominator sums the probabilities as the PV product sees them (rounded to T)
@@ -460,7 +516,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KV8 && TIB) ? 4 : 3) void pa
             lt += sm_l[x][hr] * f;
             sum += *(const f32x4*)((const float*)(smem + x * (PA_TILE * VSTRIDE)) + hr * D + 4 * d4) * f;
         }
-        if constexpr (KV8) {                                  // value dequantisation, linear in (sum, lt)
+        if constexpr (KVQ == 1) {                             // value dequantisation, linear in (sum, lt)
             const float* vs = kv_scale + n_kv * D + kvh * D + 4 * d4;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {

@@ -515,7 +515,7 @@ __global__ void pf_zero_rows_kernel(uint16_t* __restrict__ out, const int32_t* _
     }
 }
 
-template <typename T, int D, bool KV8>
+template <typename T, int D, int KVQ>
 int launch_pf(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, const int32_t* q_starts, int batch,
               int total_q, int n_heads, int n_kv, int block_size, int max_blocks, int num_blocks, float scale,
@@ -527,6 +527,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
     float* part_ml = part_out ? part_out + (int64_t)total_q * n_heads * plan.max_parts * D : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
+    constexpr bool KV8 = KVQ != 0;
     const int64_t wgs = (KV8 ? plan.col_groups16 : plan.col_groups128) * n_kv * plan.max_parts;
     if (wgs > 0x7fffffffLL) {
         mf_set_error("paged_attention_prefill: %lld workgroups exceed the grid limit", (long long)wgs);
@@ -541,7 +542,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     if constexpr (KV8) {
         const bool tib = block_size % PA_TILE == 0;           // a 32-token tile never straddles two blocks
 #define PF_LAUNCH(TIBV)                                                                                           \
-    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, true, TIBV>), dim3((unsigned)wgs),                   \
+    hipLaunchKernelGGL((paged_attention_kernel<T, D, 2, true, KVQ, TIBV>), dim3((unsigned)wgs),                    \
                        dim3(PA_WAVES * 64), 0, st, (uint16_t*)out, part_out, part_ml, (const uint16_t*)query,      \
                        (const uint16_t*)key_cache, (const uint16_t*)value_cache, block_tables, context_lens,       \
                        n_heads, n_kv, n_rep, (n_rep + 15) / 16, block_size, max_blocks, num_blocks, plan.max_parts, \
@@ -602,9 +603,15 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
                             int batch, int total_q, int n_heads, int n_kv_heads, int head_dim, int block_size,
                             int max_blocks_per_seq, int num_blocks, float scale, int64_t q_row_stride,
                             int64_t kv_row_stride, int dtype, void* workspace, size_t workspace_bytes, void* stream,
-                            bool kv8, const float* kv_scale, const float* kv_offset) {
+                            int kvq, const float* kv_scale, const float* kv_offset) {
+    // kvq: 0 = 16-bit rows or caches, 1 = int8 caches with per-channel scale / offset, 2 = int8 caches with per-token
+    // key scales (kv_scale) and value scales (kv_offset), one float per cache slot
+    const bool kv8 = kvq != 0;
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "paged_attention_prefill: dtype must be bf16 or fp16");
     MF_REQUIRE(!kv8 || (kv_scale && block_tables), "paged_attention_prefill: an int8 cache needs its scales and a block table");
+    MF_REQUIRE(kvq != 2 || (kv_offset && block_size % 4 == 0 && (((uintptr_t)kv_scale | (uintptr_t)kv_offset) & 15) == 0),
+               "paged_attention_prefill: per-token scales need both 16-byte aligned scale caches and a block size that "
+               "is a multiple of 4");
     MF_REQUIRE(batch >= 0 && total_q >= 0, "paged_attention_prefill: negative batch or row count");
     if (batch == 0 || total_q == 0) return 0;
     MF_REQUIRE(out && query && key_cache && value_cache && q_starts, "paged_attention_prefill: null argument");
@@ -637,17 +644,19 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
     MF_REQUIRE(need == 0 || ((uintptr_t)workspace & 15) == 0,
                "paged_attention_prefill: workspace must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
+#define PF_CASE_Q(TT, DD, QQ)                                                                                      \
+    return launch_pf<TT, DD, QQ>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch,  \
+                                 total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale,  \
+                                 q_row_stride, kv_row_stride, workspace, st, kvq ? kv_scale : nullptr,             \
+                                 kvq ? kv_offset : nullptr)
 #define PF_CASE(TT, DD)                                                                                            \
-    return kv8 ? launch_pf<TT, DD, true>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, \
-                                         batch, total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq,      \
-                                         num_blocks, scale, q_row_stride, kv_row_stride, workspace, st, kv_scale,  \
-                                         kv_offset)                                                                \
-               : launch_pf<TT, DD, false>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, \
-                                          batch, total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq,     \
-                                          num_blocks, scale, q_row_stride, kv_row_stride, workspace, st, nullptr,  \
-                                          nullptr)
+    {                                                                                                              \
+        if (kvq == 2) PF_CASE_Q(TT, DD, 2);                                                                        \
+        if (kvq == 1) PF_CASE_Q(TT, DD, 1);                                                                        \
+        PF_CASE_Q(TT, DD, 0);                                                                                      \
+    }
 #define PF_CASE192(TT)                                                                                             \
-    return launch_pf<TT, 192, false>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, \
+    return launch_pf<TT, 192, 0>(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, \
                                      total_q, n_heads, n_kv_heads, block_size, max_blocks_per_seq, num_blocks, scale, \
                                      q_row_stride, kv_row_stride, workspace, st, nullptr, nullptr)
     if (dtype == MF_BF16) {
@@ -663,6 +672,7 @@ static int pa_prefill_entry(void* out, const void* query, const void* key_cache,
     }
 #undef PF_CASE192
 #undef PF_CASE
+#undef PF_CASE_Q
 }
 
 extern "C" int mf_paged_attention_prefill(void* out, const void* query, const void* key_cache,
@@ -674,7 +684,7 @@ extern "C" int mf_paged_attention_prefill(void* out, const void* query, const vo
                                           size_t workspace_bytes, void* stream) {
     return pa_prefill_entry(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, total_q,
                             n_heads, n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale,
-                            q_row_stride, kv_row_stride, dtype, workspace, workspace_bytes, stream, false, nullptr,
+                            q_row_stride, kv_row_stride, dtype, workspace, workspace_bytes, stream, 0, nullptr,
                             nullptr);
 }
 
@@ -688,7 +698,22 @@ extern "C" int mf_paged_attention_prefill_int8kv(void* out, const void* query, c
                                                  size_t workspace_bytes, void* stream) {
     return pa_prefill_entry(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, total_q,
                             n_heads, n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale,
-                            q_row_stride, 0, dtype, workspace, workspace_bytes, stream, true, antiquant_scale,
+                            q_row_stride, 0, dtype, workspace, workspace_bytes, stream, 1, antiquant_scale,
                             antiquant_offset);
+}
+
+extern "C" int mf_paged_attention_prefill_int8kv_per_token(void* out, const void* query, const void* key_cache,
+                                                           const void* value_cache, const float* key_scale_cache,
+                                                           const float* value_scale_cache,
+                                                           const int32_t* block_tables, const int32_t* context_lens,
+                                                           const int32_t* q_starts, int batch, int total_q,
+                                                           int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                                           int max_blocks_per_seq, int num_blocks, float scale,
+                                                           int64_t q_row_stride, int dtype, void* workspace,
+                                                           size_t workspace_bytes, void* stream) {
+    return pa_prefill_entry(out, query, key_cache, value_cache, block_tables, context_lens, q_starts, batch, total_q,
+                            n_heads, n_kv_heads, head_dim, block_size, max_blocks_per_seq, num_blocks, scale,
+                            q_row_stride, 0, dtype, workspace, workspace_bytes, stream, 2, key_scale_cache,
+                            value_scale_cache);
 }
 

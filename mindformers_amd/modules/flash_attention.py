@@ -33,17 +33,27 @@ class FlashAttention(nn.Module):
     def forward(self, query, key, value, slot_mapping=None, block_tables=None, batch_valid_length=None,
                 context_lens_tensor=None, q_seq_lens=None, actual_seq_qlen=None, actual_seq_kvlen=None,
                 attn_mask=None, padding_mask=None, prefix=None, key_cache=None, value_cache=None,
-                antiquant_scale=None, antiquant_offset=None):
+                antiquant_scale=None, antiquant_offset=None, key_scale_cache=None, value_scale_cache=None):
         """Forward process of the FlashAttention (flash_attention.py:109-145).  int8 caches (kvcache_dtype: int8) come
         with ``antiquant_scale`` / ``antiquant_offset`` float32 [2, n_kv * D] (keys, values), the arguments the
         reference's PagedAttention call has in positions 6-7: the scatter then quantises and the attention
-        dequantises."""
+        dequantises.  Caches quantised per token (kvcache_quant_granularity: per_token) come with
+        ``key_scale_cache`` / ``value_scale_cache`` float32 [num_blocks, block_size] instead: the scatter writes each
+        token's scale beside its row."""
         kv8 = key_cache is not None and key_cache.dtype == torch.int8
-        if kv8 and antiquant_scale is None:
-            raise ValueError("int8 caches need antiquant_scale (and optionally antiquant_offset)")
+        per_token = key_scale_cache is not None
+        if kv8 and not per_token and antiquant_scale is None:
+            raise ValueError("int8 caches need antiquant_scale (and optionally antiquant_offset), or the per-token "
+                             "scale caches")
+        if per_token and (not kv8 or value_scale_cache is None or antiquant_scale is not None):
+            raise ValueError("per-token scale caches go with int8 caches, both of them, and no per-channel parameters")
         if kv8 and self.use_multi_latent_attention:
             raise NotImplementedError("an int8 latent cache is not built")
-        if kv8:
+        token_scales = (key_scale_cache, value_scale_cache) if per_token else None
+        if per_token:
+            ops.dynamic_quant_reshape_and_cache(key, value, key_cache, value_cache, key_scale_cache, value_scale_cache,
+                                                slot_mapping)
+        elif kv8:
             ops.quant_reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, antiquant_scale,
                                         antiquant_offset)
         elif not self.use_multi_latent_attention:             # MLA: the caller has written the latent row already
@@ -86,7 +96,7 @@ class FlashAttention(nn.Module):
             starts = None if q_seq_lens is None else ops.q_starts_from_lens(q_seq_lens)
             out = ops.paged_attention_int8kv(q2, key_cache, value_cache, block_tables, batch_valid_length,
                                              antiquant_scale, antiquant_offset, self.head_num, self.pa_kv_head_num,
-                                             self.scale_value, q_starts=starts)
+                                             self.scale_value, q_starts=starts, token_scales=token_scales)
             return out.reshape(shape)
         if q_seq_lens is not None:                            # several new tokens per sequence (flash_attention.py:140-143)
             out = ops.paged_attention_prefill(q2, key_cache, value_cache, block_tables, batch_valid_length,

@@ -70,27 +70,42 @@ class QuantPagedAttentionMgr(PagedAttentionMgr):
     mindformers/modules/paged_attention_mgr.py:66-70; the cache dtype comes from the quantization config,
     mindformers/model_runner.py:364-368).  The cell itself belongs to golden-stick in the reference stack, so the
     parameter names are this build's: ``kv_scale`` / ``kv_offset`` float32 [2, n_kv_heads * head_dim] (keys, values),
-    x ~ (q - offset) * scale, loaded from the checkpoint or set with ``set_kv_quant``."""
+    x ~ (q - offset) * scale, loaded from the checkpoint or set with ``set_kv_quant``.
+
+    ``granularity="per_token"`` (kvcache_quant_granularity, mindformers/utils/quantization_config.py:206-207): nothing
+    is loaded; every token row is quantised with its own scale as it is written, and the scales live beside the rows
+    in ``key_scale_cache`` / ``value_scale_cache`` float32 [num_blocks, block_size]."""
 
     def __init__(self, n_heads, head_dim, n_kv_heads, kv_shape, seq_length=-1, compute_dtype=torch.float16,
-                 parallel_decoding=False, chunk_prefill=False, device="cuda"):
+                 parallel_decoding=False, chunk_prefill=False, device="cuda", granularity="per_channel"):
         super().__init__(n_heads, head_dim, n_kv_heads, (1,) + tuple(kv_shape[1:]), seq_length, compute_dtype,
                          parallel_decoding, chunk_prefill, device)
+        if granularity not in ("per_channel", "per_token"):
+            raise ValueError(f"kvcache_quant_granularity must be per_channel or per_token, got {granularity!r}")
+        self.granularity = granularity
         self.compute_dtype = compute_dtype
         self.register_buffer("key_cache", torch.zeros(kv_shape, dtype=torch.int8, device=device), persistent=False)
         self.register_buffer("value_cache", torch.zeros(kv_shape, dtype=torch.int8, device=device), persistent=False)
         row = n_kv_heads * head_dim
-        self.register_buffer("kv_scale", torch.ones(2, row, dtype=torch.float32, device=device))
-        self.register_buffer("kv_offset", torch.zeros(2, row, dtype=torch.float32, device=device))
+        per_token = granularity == "per_token"
+        if per_token and kv_shape[1] % 4:
+            raise ValueError(f"per_token int8 caches need a block size that is a multiple of 4, got {kv_shape[1]}")
+        self.register_buffer("kv_scale", None if per_token else torch.ones(2, row, dtype=torch.float32, device=device))
+        self.register_buffer("kv_offset", None if per_token else torch.zeros(2, row, dtype=torch.float32, device=device))
+        for name in ("key_scale_cache", "value_scale_cache"):
+            self.register_buffer(name, torch.zeros(kv_shape[:2], dtype=torch.float32, device=device) if per_token else None,
+                                 persistent=False)
 
     @classmethod
-    def from_float(cls, mgr):
+    def from_float(cls, mgr, granularity="per_channel"):
         """A quantised manager with the geometry of a float one."""
         kc = mgr.key_cache
         return cls(mgr.n_heads, mgr.head_dim, mgr.n_kv_heads, tuple(kc.shape), mgr.seq_length, kc.dtype,
-                   mgr.parallel_decoding, mgr.chunk_prefill, kc.device)
+                   mgr.parallel_decoding, mgr.chunk_prefill, kc.device, granularity=granularity)
 
     def set_kv_quant(self, scale, offset=None):
+        if self.granularity == "per_token":
+            raise ValueError("a per_token cache has no loaded parameters: its scales are written with the rows")
         self.kv_scale.copy_(scale.to(torch.float32))
         if offset is None:
             self.kv_offset.zero_()
@@ -99,6 +114,9 @@ class QuantPagedAttentionMgr(PagedAttentionMgr):
         return self
 
     def forward(self, key, value, slot_mapping, batch_valid_length=None):
+        if self.granularity == "per_token":
+            return ops.dynamic_quant_reshape_and_cache(key, value, self.key_cache, self.value_cache,
+                                                       self.key_scale_cache, self.value_scale_cache, slot_mapping)
         return ops.quant_reshape_and_cache(key, value, self.key_cache, self.value_cache, slot_mapping, self.kv_scale,
                                            self.kv_offset)
 
@@ -114,5 +132,7 @@ class QuantPagedAttentionMgr(PagedAttentionMgr):
             starts = ops.q_starts_from_lens(q_seq_lens)
         out = ops.paged_attention_int8kv(q2, self.key_cache, self.value_cache, block_tables, batch_valid_length,
                                          self.kv_scale, self.kv_offset, self.n_heads, self.n_kv_heads,
-                                         self.scale_value, q_starts=starts)
+                                         self.scale_value, q_starts=starts,
+                                         token_scales=(self.key_scale_cache, self.value_scale_cache)
+                                         if self.granularity == "per_token" else None)
         return out.reshape(shape)

@@ -108,8 +108,9 @@ def check_buildable(cfg):
         raise NotImplementedError("per_group weights need group_size 64 or 128")
     if cfg.kvcache_quant_dtype not in (None, "int8"):
         raise NotImplementedError(f"kvcache_dtype {cfg.kvcache_quant_dtype!r}: only an int8 KV cache is built")
-    if cfg.kvcache_quant_dtype == "int8" and getattr(cfg, "kvcache_quant_granularity", "per_channel") != "per_channel":
-        raise NotImplementedError("per_token int8 KV cache is not built (per_channel only)")
+    if cfg.kvcache_quant_dtype == "int8" and getattr(cfg, "kvcache_quant_granularity", "per_channel") not in (
+            "per_channel", "per_token"):
+        raise NotImplementedError("an int8 KV cache is quantised per_channel or per_token")
     if getattr(cfg, "precision_recovery", "none") != "none":
         raise NotImplementedError("GPTQ precision recovery has no deploy-time kernel here")
     if cfg.outliers_suppression not in ("none", "smooth", "awq"):
@@ -163,7 +164,8 @@ def convert_linears(model, cfg, layer_policies=None):
                   and pol.kvcache_quant_dtype == "int8"):
                 # kvcache_dtype: int8 - the manager owns int8 caches and hands the attention its dequantisation
                 # parameters (filled from the checkpoint)
-                setattr(parent, child_name, QuantPagedAttentionMgr.from_float(child))
+                setattr(parent, child_name, QuantPagedAttentionMgr.from_float(
+                    child, getattr(pol, "kvcache_quant_granularity", "per_channel")))
             elif isinstance(child, GroupedMLP):
                 act8 = pol.act_quant_dtype == "int8"
                 cell = QuantGroupedMLP(child.num_experts, child.config, child.weight1.device,

@@ -298,10 +298,43 @@ def quant_reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, sc
     return key
 
 
+def dynamic_quant_reshape_and_cache(key, value, key_cache, value_cache, key_scale_cache, value_scale_cache, slot_mapping):
+    """Quantise key / value rows per token (s = max|row| / 127 over all kv heads of the token, q = clip(rint(x / s),
+    -128, 127)) and scatter rows and scales: int8 caches [num_blocks, block_size, n_kv, D], fp32 scale caches
+    [num_blocks, block_size]."""
+    lib = _lib.load()
+    _dev_of(key, value)
+    dev = _dev_ok(key_cache, value_cache, key_scale_cache, value_scale_cache, slot_mapping)
+    _need(key_cache.dtype == torch.int8 and value_cache.dtype == torch.int8 and key_cache.dim() == 4 and
+          value_cache.shape == key_cache.shape, "caches must be int8 [blocks, block_size, n_kv, D]")
+    nb, bs, n_kv, d = key_cache.shape
+    _token_scale_caches(key_scale_cache, value_scale_cache, nb, bs)
+    row = n_kv * d
+    key, ks = _rows(key, row, "key")
+    value, vs = _rows(value, row, "value")
+    _need(key.dtype in _ACT and value.dtype == key.dtype, "key / value must be bf16 or fp16")
+    _need(slot_mapping.dtype == torch.int32, "slot_mapping must be int32")
+    t = slot_mapping.numel()
+    _need(key.numel() // row == t if key.is_contiguous() else key.shape[0] == t, "key rows != slots")
+    check(lib.mf_dynamic_quant_reshape_and_cache(ptr(key), ptr(value), ptr(key_cache), ptr(value_cache),
+                                                 ptr(key_scale_cache), ptr(value_scale_cache), ptr(slot_mapping), t,
+                                                 n_kv, d, nb * bs, ks, vs, dtype_code(key.dtype), stream_ptr(dev)),
+          "mf_dynamic_quant_reshape_and_cache")
+    return key
+
+
+def _token_scale_caches(key_scale_cache, value_scale_cache, nb, bs):
+    for c in (key_scale_cache, value_scale_cache):
+        _need(c is not None and c.dtype == torch.float32 and c.numel() == nb * bs and c.is_contiguous(),
+              "per-token scale caches must be contiguous fp32 [num_blocks, block_size]")
+
+
 def paged_attention_int8kv(query, key_cache, value_cache, block_tables, context_lens, antiquant_scale,
-                           antiquant_offset, n_heads, n_kv_heads, scale, q_starts=None, out=None):
+                           antiquant_offset, n_heads, n_kv_heads, scale, q_starts=None, out=None, token_scales=None):
     """PagedAttention(...)(query, key_cache, value_cache, block_tables, context_lens, antiquant_scale,
-    antiquant_offset[, mask, q_seq_lens]) on int8 caches; ``q_starts`` selects the several-rows-per-sequence form."""
+    antiquant_offset[, mask, q_seq_lens]) on int8 caches; ``q_starts`` selects the several-rows-per-sequence form.
+    ``token_scales`` = (key_scale_cache, value_scale_cache), fp32 [num_blocks, block_size]: caches quantised per
+    token (``dynamic_quant_reshape_and_cache``); antiquant_scale / antiquant_offset are then None."""
     lib = _lib.load()
     _dev_of(query)
     dev = _dev_ok(key_cache, value_cache, block_tables, context_lens, out)
@@ -312,7 +345,13 @@ def paged_attention_int8kv(query, key_cache, value_cache, block_tables, context_
     _need(n_kv == n_kv_heads and query.dtype in _ACT, "head count / dtype mismatch")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2, "block_tables must be int32 [B, max_blocks]")
     _need(context_lens.dtype == torch.int32 and context_lens.dim() == 1, "context_lens must be int32 [B]")
-    _kv_quant_params(antiquant_scale, antiquant_offset, n_kv * d, dev)
+    if token_scales is not None:
+        _need(antiquant_scale is None and antiquant_offset is None, "per-token caches take no per-channel parameters")
+        _dev_ok(*token_scales)
+        _token_scale_caches(token_scales[0], token_scales[1], nb, bs)
+        _need(bs % 4 == 0, "per-token scales need a block size that is a multiple of 4")
+    else:
+        _kv_quant_params(antiquant_scale, antiquant_offset, n_kv * d, dev)
     b = context_lens.numel()
     _need(block_tables.shape[0] == b, "block_tables rows != batch")
     max_blocks = block_tables.shape[1]
@@ -325,6 +364,13 @@ def paged_attention_int8kv(query, key_cache, value_cache, block_tables, context_
         _need(rows == b, f"query has {rows} rows for {b} sequences")
         need = lib.mf_paged_attention_workspace_bytes(b, n_heads, d, max_blocks * bs)
         ws = workspace(need, dev, "pa") if need else None
+        if token_scales is not None:
+            check(lib.mf_paged_attention_decode_int8kv_per_token(
+                ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(token_scales[0]), ptr(token_scales[1]),
+                ptr(block_tables), ptr(context_lens), b, n_heads, n_kv_heads, d, bs, max_blocks, nb, float(scale), qs,
+                dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+                "mf_paged_attention_decode_int8kv_per_token")
+            return out
         check(lib.mf_paged_attention_decode_int8kv(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache),
                                                    ptr(block_tables), ptr(context_lens), ptr(antiquant_scale),
                                                    ptr(antiquant_offset), b, n_heads, n_kv_heads, d, bs, max_blocks, nb,
@@ -335,6 +381,13 @@ def paged_attention_int8kv(query, key_cache, value_cache, block_tables, context_
         _need(_q_starts(q_starts, dev) == b, "q_starts must have batch + 1 entries")
         need = lib.mf_paged_attention_prefill_workspace_bytes(b, rows, n_heads, n_kv_heads, d, max_blocks * bs)
         ws = workspace(need, dev, "pa_prefill") if need else None
+        if token_scales is not None:
+            check(lib.mf_paged_attention_prefill_int8kv_per_token(
+                ptr(out), ptr(query), ptr(key_cache), ptr(value_cache), ptr(token_scales[0]), ptr(token_scales[1]),
+                ptr(block_tables), ptr(context_lens), ptr(q_starts), b, rows, n_heads, n_kv_heads, d, bs, max_blocks,
+                nb, float(scale), qs, dtype_code(query.dtype), ptr(ws), ws.numel() if ws is not None else 0,
+                stream_ptr(dev)), "mf_paged_attention_prefill_int8kv_per_token")
+            return out
         check(lib.mf_paged_attention_prefill_int8kv(ptr(out), ptr(query), ptr(key_cache), ptr(value_cache),
                                                     ptr(block_tables), ptr(context_lens), ptr(q_starts),
                                                     ptr(antiquant_scale), ptr(antiquant_offset), b, rows, n_heads,

@@ -54,7 +54,8 @@ class DecodeStackRunner:
             gran = (quantization_config.get("kvcache_quant_granularity", "per_channel") if isinstance(quantization_config, dict)
                     else getattr(quantization_config, "kvcache_quant_granularity", "per_channel"))
             if gran != "per_channel":
-                raise NotImplementedError("per_token int8 KV cache is not built (per_channel only)")
+                raise NotImplementedError("the fused layer step runs per_channel int8 caches; per_token caches are "
+                                          "served by the module path (QuantPagedAttentionMgr / FlashAttention)")
             if any(l.kv_scale is None for l in layers):
                 raise ValueError("kvcache_dtype int8: every layer needs set_kv_quant(scale, offset) first")
         self.kvcache_dtype = torch.int8 if kv_name == "int8" else self.dtype

@@ -57,7 +57,7 @@ from .rope import (rope_inv_freq_default, rope_inv_freq_llama3, rope_inv_freq_ya
                    yarn_mscale, rope_cos_sin_table, apply_rotary_half)
 from .dense import rms_norm, layer_norm, silu, silu_mul, linear, mlp
 from .quant import (quantize_weight_int8, w8a16_linear, dynamic_quant_per_token, static_quant_per_tensor,
-                    int8_gemm_i32, w8a8_linear, quantize_kv_int8, dequantize_kv_int8, quantize_weight_int4,
+                    int8_gemm_i32, w8a8_linear, quantize_kv_int8, quantize_kv_int8_per_token, dequantize_kv_int8, quantize_weight_int4,
                     w4a16_linear, pack_qint4x2, unpack_qint4x2)
 from . import checkpoint
 from .moe import (topk_router, moe_permute, grouped_mlp, moe_unpermute, moe_layer,

@@ -91,6 +91,14 @@ def quantize_kv_int8(x, scale, offset=None):
     return np.clip(np.rint(q), -128, 127).astype(np.int8)
 
 
+def quantize_kv_int8_per_token(x):
+    """Per-token int8 quantisation of key / value rows [T, n_kv * D] (kvcache_quant_granularity per_token,
+    quantization_config.py:206-207): one scale per token row over all its kv heads, the arithmetic of
+    dynamic_quant_per_token without a multiplier.  Returns (q int8, s float32 [T]); x ~ q * s.  PARITY UNPINNED like
+    the per-channel form: the reference only configures the mode."""
+    return dynamic_quant_per_token(x)
+
+
 def dequantize_kv_int8(q, scale, offset=None):
     """x ~ (q - offset) * scale in float64 (the inverse convention of quantize_kv_int8)."""
     x = np.asarray(q, dtype=np.float64)

@@ -146,9 +146,8 @@ def test_unbuilt_quant_modes_are_rejected_at_conversion():
         check_buildable(PtqConfig(weight_dtype="int4", weight_quant_granularity="per_group", group_size=0))
     with pytest.raises(NotImplementedError):
         check_buildable(PtqConfig(weight_dtype="int4", precision_recovery="gptq"))
-    with pytest.raises(NotImplementedError):             # an int8 cache is built per channel only
-        check_buildable(PtqConfig(activation_dtype="int8", act_quant_granularity="per_token", kvcache_dtype="int8",
-                                  kvcache_quant_granularity="per_token"))
+    check_buildable(PtqConfig(activation_dtype="int8", act_quant_granularity="per_token", kvcache_dtype="int8",
+                              kvcache_quant_granularity="per_token"))            # per-token int8 cache: built
     check_buildable(PtqConfig(kvcache_dtype="int8"))
     check_buildable(PtqConfig())
 

@@ -627,6 +627,114 @@ def test_paged_prefill_int8kv_vs_oracle():
     assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="prefill over an int8 cache")
 
 
+def _kv8_token_case(rng, dtype, b, nkv, d, bs, lens, max_blocks=None, poison=True):
+    """Random 16-bit caches quantised per token by the oracle: int8 caches, the float caches they stand for, the scale
+    caches [blocks, block_size] and the tables.  With ``poison`` the scales of every slot that holds no token of a
+    sequence are NaN, so a scale read past a context must not reach a result."""
+    kc, vc, tables, nb = make_paged_cache(rng, b, lens, nkv, d, bs, dtype, max_blocks=max_blocks)
+    row = nkv * d
+    k8, ks = O.quantize_kv_int8_per_token(kc.reshape(-1, row))
+    v8, vs = O.quantize_kv_int8_per_token(vc.reshape(-1, row))
+    kf = (k8.astype(np.float64) * ks[:, None]).reshape(kc.shape)
+    vf = (v8.astype(np.float64) * vs[:, None]).reshape(vc.shape)
+    if poison:
+        live = np.zeros(nb * bs, bool)
+        for i, n in enumerate(lens):
+            for j in range(int(n)):
+                live[tables[i, j // bs] * bs + j % bs] = True
+        ks, vs = np.where(live, ks, np.float32(np.nan)), np.where(live, vs, np.float32(np.nan))
+    return (k8.reshape(kc.shape), v8.reshape(vc.shape), kf, vf, ks.reshape(nb, bs).astype(np.float32),
+            vs.reshape(nb, bs).astype(np.float32), tables, nb)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dynamic_quant_reshape_and_cache_bit_exact(dtype):
+    """Per-token int8 cache write from strided key / value slices: rows and scales of the written slots equal the
+    oracle's per-token quantisation bit for bit (a zero row stores scale 0 and zeros); a -1 slot writes nothing and
+    every other slot keeps what it held."""
+    rng = np.random.default_rng(41)
+    t, nh, nkv, d, bs, nb = 37, 8, 2, 128, 16, 5
+    row = nkv * d
+    qkv = rounded(rng.normal(size=(t, (nh + 2 * nkv) * d)) * 2, dtype)
+    qkv[5, nh * d:nh * d + row] = 0                                # a key row of zeros
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    slots[11] = -1
+    qkv_t = dev(qkv, dtype)
+    kc = torch.full((nb, bs, nkv, d), 77, dtype=torch.int8, device="cuda")
+    vc = torch.full((nb, bs, nkv, d), -77, dtype=torch.int8, device="cuda")
+    ksc = torch.full((nb, bs), 3.0, dtype=torch.float32, device="cuda")
+    vsc = torch.full((nb, bs), 5.0, dtype=torch.float32, device="cuda")
+    ops.dynamic_quant_reshape_and_cache(qkv_t[:, nh * d:nh * d + row], qkv_t[:, nh * d + row:], kc, vc, ksc, vsc,
+                                        torch.from_numpy(slots).cuda())
+    k_ref, ks_ref = O.quantize_kv_int8_per_token(qkv[:, nh * d:nh * d + row])
+    v_ref, vs_ref = O.quantize_kv_int8_per_token(qkv[:, nh * d + row:])
+    want_k, want_v = np.full((nb * bs, row), 77, np.int8), np.full((nb * bs, row), -77, np.int8)
+    want_ks, want_vs = np.full(nb * bs, 3.0, np.float32), np.full(nb * bs, 5.0, np.float32)
+    for i, sl in enumerate(slots):
+        if sl >= 0:
+            want_k[sl], want_v[sl], want_ks[sl], want_vs[sl] = k_ref[i], v_ref[i], ks_ref[i], vs_ref[i]
+    assert ks_ref[5] == 0 and not k_ref[5].any()
+    assert np.array_equal(to_np(kc).reshape(-1, row), want_k) and np.array_equal(to_np(vc).reshape(-1, row), want_v)
+    assert np.array_equal(to_np(ksc).reshape(-1), want_ks) and np.array_equal(to_np(vsc).reshape(-1), want_vs)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,nh,nkv,d,bs,lo,hi", [(8, 32, 8, 128, 128, 1, 1500), (5, 8, 2, 64, 16, 1, 700),
+                                                 (3, 4, 4, 32, 32, 30, 300), (64, 28, 4, 128, 128, 500, 600),
+                                                 (2, 16, 2, 128, 20, 1, 90)])
+def test_paged_attention_int8kv_per_token_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi):
+    """Decode over int8 caches with one scale per cached token: against the oracle on the dequantised caches (block
+    sizes that hold whole 32-token tiles and block sizes that do not; contexts that end inside a tile; NaN in the
+    scale slots of tokens that do not exist)."""
+    rng = np.random.default_rng(b * 31 + bs)
+    lens = rng.integers(lo, hi + 1, b)
+    lens[0] = hi
+    k8, v8, kf, vf, ks, vs, tables, nb = _kv8_token_case(rng, dtype, b, nkv, d, bs, lens)
+    q = rounded(rng.normal(size=(b, nh * d)), dtype)
+    sc = 1.0 / np.sqrt(d)
+    out = ops.paged_attention_int8kv(dev(q, dtype), torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda(),
+                                     dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32), None, None,
+                                     nh, nkv, sc, token_scales=(torch.from_numpy(ks).cuda(), torch.from_numpy(vs).cuda()))
+    ref = O.paged_attention_decode(q, kf, vf, tables, lens, nh, nkv, sc)
+    mag = O.paged_attention_decode(q, kf, np.abs(vf), tables, lens, nh, nkv, sc)
+    assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="paged attention over a per-token int8 cache")
+
+
+@pytest.mark.parametrize("bs", [128, 16])
+def test_paged_prefill_int8kv_per_token_vs_oracle(bs):
+    rng = np.random.default_rng(34 + bs)
+    dtype, nh, nkv, d = torch.bfloat16, 16, 4, 128
+    lens, q_lens = np.array([300, 77, 520]), np.array([40, 77, 1])
+    k8, v8, kf, vf, ks, vs, tables, nb = _kv8_token_case(rng, dtype, 3, nkv, d, bs, lens)
+    t = int(q_lens.sum())
+    q = rounded(rng.normal(size=(t, nh * d)), dtype)
+    sc = 1.0 / np.sqrt(d)
+    out = ops.paged_attention_int8kv(dev(q, dtype), torch.from_numpy(k8).cuda(), torch.from_numpy(v8).cuda(),
+                                     dev(tables, torch.int32), dev(lens.astype(np.int32), torch.int32), None, None,
+                                     nh, nkv, sc, q_starts=dev(_starts(q_lens), torch.int32),
+                                     token_scales=(torch.from_numpy(ks).cuda(), torch.from_numpy(vs).cuda()))
+    ref = O.paged_attention_prefill(q, kf, vf, tables, lens, q_lens, nh, nkv, sc)
+    mag = O.paged_attention_prefill(q, kf, np.abs(vf), tables, lens, q_lens, nh, nkv, sc)
+    assert_within(to_np(out), ref, mag, dtype, ulps=3.0, what="prefill over a per-token int8 cache")
+
+
+def test_paged_attention_int8kv_per_token_rejects_bad_operands():
+    k8 = torch.zeros(2, 6, 1, 32, dtype=torch.int8, device="cuda")            # block size 6: not a multiple of 4
+    sc6 = torch.ones(2, 6, device="cuda")
+    q = torch.zeros(1, 32, dtype=torch.bfloat16, device="cuda")
+    tables = torch.zeros(1, 2, dtype=torch.int32, device="cuda")
+    lens = torch.ones(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        ops.paged_attention_int8kv(q, k8, k8, tables, lens, None, None, 1, 1, 1.0, token_scales=(sc6, sc6))
+    k8 = torch.zeros(2, 8, 1, 32, dtype=torch.int8, device="cuda")
+    with pytest.raises(ValueError):                                           # scale caches of the wrong size
+        ops.paged_attention_int8kv(q, k8, k8, tables, lens, None, None, 1, 1, 1.0, token_scales=(sc6, sc6))
+    sc8 = torch.ones(2, 8, device="cuda")
+    with pytest.raises(ValueError):                                           # both kinds of parameters at once
+        ops.paged_attention_int8kv(q, k8, k8, tables, lens, torch.ones(2, 32, device="cuda"), None, 1, 1, 1.0,
+                                   token_scales=(sc8, sc8))
+
+
 # ------------------------------------------------------------------------------------------- norm / activation
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,cols,gdt", [(64, 4096, torch.float32), (4, 512, torch.float16), (3, 8192, torch.bfloat16), (1, 32, torch.float32)])

@@ -868,10 +868,6 @@ def test_quantizer_swaps_in_the_int8_kv_manager_and_decode_matches_oracle(dynami
     mgr = net.infer_attention.paged_attention_mgr
     assert isinstance(mgr, QuantPagedAttentionMgr) and mgr.key_cache.dtype == torch.int8
     assert mgr.key_cache.shape == (nb, bs, n_kv, d) and mgr.kv_scale.shape == (2, n_kv * d)
-    with pytest.raises(NotImplementedError):                 # per-token cache granularity is refused, not ignored
-        AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8",
-                                   "act_quant_granularity": "per_token", "kvcache_dtype": "int8",
-                                   "kvcache_quant_granularity": "per_token"}).preprocess_model(Block())
     row = n_kv * d
     scale = (np.stack([np.abs(kc_f).reshape(-1, row).max(0), np.abs(vc_f).reshape(-1, row).max(0)]) / 110.0).astype(np.float32)
     offset = rng.integers(-12, 13, (2, row)).astype(np.float32)
@@ -909,6 +905,85 @@ def test_quantizer_swaps_in_the_int8_kv_manager_and_decode_matches_oracle(dynami
     keep = np.ones(nb * bs, bool)
     keep[slots] = False
     assert np.array_equal(mgr.key_cache.cpu().numpy().reshape(-1, row)[keep], k8.reshape(-1, row)[keep])
+
+
+@pytest.mark.parametrize("bs", [16, 128])
+def test_quantizer_swaps_in_the_per_token_int8_kv_manager(bs):
+    """`kvcache_dtype: int8` with `kvcache_quant_granularity: per_token` (quantization_config.py:206-207): the manager
+    the quantizer swaps in owns int8 caches and one scale per cached token.  A prefill through InferAttention writes
+    the prompt's rotated keys and values quantised per token, bit for bit as the oracle quantises them, and a decode
+    step attends over them - against the oracle's attention over the dequantised cache."""
+    from torch import nn
+    from mindformers_amd.modules import FreqsMgr, InferAttention, QuantPagedAttentionMgr
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    rng = np.random.default_rng(50 + bs)
+    b, n_head, n_kv, d, seq = 3, 8, 2, 64, 512
+    dt, row = BF, 2 * 64
+    lens = np.array([70, 5, 131])
+    _, _, tables, nb = make_paged_cache(rng, b, lens + 1, n_kv, d, bs, dt, max_blocks=seq // bs)
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.infer_attention = InferAttention(n_head, d, n_kv, scale_value=1 / np.sqrt(d), block_size=bs,
+                                                  num_blocks=nb, seq_length=seq, is_dynamic=True, rotary_cos_format=2,
+                                                  compute_dtype=dt)
+    net = Block()
+    AutoQuantizer.from_config({"quant_method": "ptq", "weight_dtype": "int8", "activation_dtype": "int8",
+                               "act_quant_granularity": "per_token", "kvcache_dtype": "int8",
+                               "kvcache_quant_granularity": "per_token"}).preprocess_model(net)
+    mgr = net.infer_attention.paged_attention_mgr
+    assert isinstance(mgr, QuantPagedAttentionMgr) and mgr.granularity == "per_token" and mgr.kv_scale is None
+    assert mgr.key_cache.dtype == torch.int8 and mgr.key_scale_cache.shape == (nb, bs)
+    with pytest.raises(ValueError):
+        mgr.set_kv_quant(torch.ones(2, row))
+    mgr.key_scale_cache.fill_(float("nan"))                   # a slot never written must never be read
+    mgr.value_scale_cache.fill_(float("nan"))
+    attn = net.infer_attention
+    freqs = FreqsMgr(d, seq_length=seq, max_position_embedding=seq, rotary_dtype=dt)
+    # ---- prefill: the prompts, packed
+    t = int(lens.sum())
+    q = rounded(rng.normal(size=(t, n_head * d)), dt)
+    k = rounded(rng.normal(size=(t, row)), dt)
+    v = rounded(rng.normal(size=(t, row)), dt)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    seq_of = np.repeat(np.arange(b), lens)
+    slots = (tables[seq_of, pos // bs] * bs + pos % bs).astype(np.int32)
+    lens_t = torch.from_numpy(lens.astype(np.int32)).cuda()
+    attn.is_first_iteration = True
+    cos_all, sin_all = to_np(freqs.freqs_cos), to_np(freqs.freqs_sin)
+    cos_t, sin_t = dev(cos_all[pos], dt), dev(sin_all[pos], dt)
+    attn(dev(q, dt), dev(k, dt), dev(v, dt), lens_t, torch.from_numpy(tables).cuda(), torch.from_numpy(slots).cuda(),
+         (cos_t, sin_t, None))
+    k_r = rounded(O.apply_rotary_half(k, cos_all[pos], sin_all[pos], n_kv), dt)
+    k8_ref, ks_ref = O.quantize_kv_int8_per_token(k_r)
+    v8_ref, vs_ref = O.quantize_kv_int8_per_token(v)
+    got_k = to_np(mgr.key_cache).reshape(-1, row)[slots].astype(np.int32)
+    assert np.abs(got_k - k8_ref).max() <= 1                  # a rotated key one rounding step away
+    assert np.array_equal(to_np(mgr.value_cache).reshape(-1, row)[slots], v8_ref)
+    assert np.array_equal(to_np(mgr.value_scale_cache).reshape(-1)[slots], vs_ref)
+    assert np.allclose(to_np(mgr.key_scale_cache).reshape(-1)[slots], ks_ref, rtol=2.0 ** -7)
+    # ---- decode: one more token per sequence over the cache the module wrote
+    attn.is_first_iteration = False
+    lens2 = lens + 1
+    slots2 = np.array([tables[i, (n - 1) // bs] * bs + (n - 1) % bs for i, n in enumerate(lens2)], np.int32)
+    lens2_t = torch.from_numpy(lens2.astype(np.int32)).cuda()
+    q2 = rounded(rng.normal(size=(b, n_head * d)), dt)
+    k2 = rounded(rng.normal(size=(b, row)), dt)
+    v2 = rounded(rng.normal(size=(b, row)), dt)
+    cos2, sin2 = cos_all[lens2 - 1], sin_all[lens2 - 1]
+    out = attn(dev(q2, dt), dev(k2, dt), dev(v2, dt), lens2_t, torch.from_numpy(tables).cuda(),
+               torch.from_numpy(slots2).cuda(), (dev(cos2, dt), dev(sin2, dt), None))
+    kq, vq = to_np(mgr.key_cache).astype(np.float64), to_np(mgr.value_cache).astype(np.float64)
+    ksc, vsc = to_np(mgr.key_scale_cache).astype(np.float64), to_np(mgr.value_scale_cache).astype(np.float64)
+    live = np.isfinite(ksc)
+    assert live.sum() == t + b and np.array_equal(live, np.isfinite(vsc))
+    kf = kq * np.where(live, ksc, 0.0)[:, :, None, None]
+    vf = vq * np.where(live, vsc, 0.0)[:, :, None, None]
+    q_r = rounded(O.apply_rotary_half(q2, cos2, sin2, n_head), dt)
+    ref = O.paged_attention_decode(q_r, kf, vf, tables, lens2, n_head, n_kv, 1 / np.sqrt(d))
+    mag = O.paged_attention_decode(q_r, kf, np.abs(vf), tables, lens2, n_head, n_kv, 1 / np.sqrt(d))
+    assert_within(to_np(out).reshape(b, -1), ref, mag, dt, ulps=4.0, what="InferAttention over a per-token int8 cache")
 
 
 def test_mcore_flash_attention_over_int8_caches():
