@@ -11,7 +11,8 @@ cores on a bounded sample.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--no-cpu]
 
 Workloads: llama3_8b_w8a16 (default), llama3_8b_w8a16_kv8, tiny_llama_w8a16, qwen2_5_7b_w8a8, qwen2_5_72b_w8a16
-(layer steps); deepseek_v3_moe_w8a16 (one MoE layer step); deepseek_v3_mla_decode, llama3_8b_prefill_attention,
+(layer steps); deepseek_v3_moe_w8a16 (one MoE layer step); deepseek_v3_mla_layer (one multi-latent attention layer step);
+deepseek_v3_mla_decode, llama3_8b_prefill_attention,
 llama3_8b_chunked_prefill_attention, deepseek_v3_mla_prefill_attention (one attention call per step).
 """
 import argparse
@@ -643,6 +644,124 @@ def bench_mla_decode(args, torch, ops):
     print(json.dumps(result), flush=True)
 
 
+def bench_mla_layer(args, torch, ops):
+    """DeepSeek-V3-shaped multi-latent self-attention layer, one decode step through the module surface
+    (MLASelfAttention): hidden 7168, 128 heads, q_lora_rank 1536, kv_lora_rank 512, 128 + 64 query dims, batch 64,
+    contexts uniform in [512, 4096], block 128, bf16; the down / up / output projections are W8A16 cells, the absorbed
+    per-head projections read linear_kv_up_proj's bf16 weight.  A step is one forward of the layer (projections,
+    norms, RoPE, latent-row scatter, absorbed query, attention over the latent cache, absorbed output, output
+    projection), replayed from a HIP graph of 4 steps on 4 separate weight sets."""
+    from mindformers_amd.modules import MLASelfAttention, MLATransformerConfig
+    from mindformers_amd.modules.quantizers import AutoQuantizer
+    hidden, nh, q_lora, rank, nope, rope, vd, bs, b, dt = 7168, 128, 1536, 512, 128, 64, 128, 128, 64, torch.bfloat16
+    rng = np.random.default_rng(1)
+    lens = rng.integers(512, 4097, b).astype(np.int32)
+    need = (lens + bs - 1) // bs
+    nb = int(need.sum()) + 2
+    tables = -np.ones((b, 4096 // bs), np.int32)
+    perm, pos = rng.permutation(nb), 0
+    for i, n in enumerate(need):
+        tables[i, :n] = perm[pos:pos + n]
+        pos += n
+    slots = np.array([tables[i, (l - 1) // bs] * bs + (l - 1) % bs for i, l in enumerate(lens)], np.int32)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4)
+    cfg = MLATransformerConfig(hidden_size=hidden, num_attention_heads=nh, q_lora_rank=q_lora, kv_lora_rank=rank,
+                               qk_head_dim=nope, qk_pos_emb_head_dim=rope, v_head_dim=vd, rope_type="yarn",
+                               layernorm_epsilon=1e-6, compute_dtype="bfloat16", params_dtype="bfloat16")
+    n_layers = 4
+    layers, caches = [], []
+    for _ in range(n_layers):
+        net = MLASelfAttention(cfg, layer_number=1)
+        for name in ("linear_qkv_down_proj", "linear_q_up_proj", "linear_kv_up_proj", "linear_proj"):
+            w = getattr(net, name).weight
+            w.data.copy_((torch.randn(w.shape, generator=gen, device="cuda") * w.shape[1] ** -0.5).to(dt))
+        q = AutoQuantizer.from_config({"quant_method": "rtn", "weight_dtype": "int8",
+                                       "modules_to_not_convert": ["linear_kv_up_proj"]})
+        q.preprocess_model(net)
+        q.postprocess_model(net)
+        net.prepare()
+        net.is_prefill = False
+        layers.append(net)
+        caches.append(torch.randn(nb, bs, 1, rank + rope, generator=gen, device="cuda").to(dt))
+    x = torch.randn(b, hidden, generator=gen, device="cuda").to(dt)
+    tb, lt, sl = torch.from_numpy(tables).cuda(), torch.from_numpy(lens).cuda(), torch.from_numpy(slots).cuda()
+    pos_t = (lt - 1).to(torch.int64)
+    cos, sin = layers[0].rotary_pos_emb.get_cos_sin_for_decode(pos_t)
+
+    def one(i):
+        return layers[i](x, rotary_pos_cos=cos, rotary_pos_sin=sin, batch_valid_length=lt, block_tables=tb,
+                         slot_mapping=sl, key_cache=caches[i])
+
+    def chain():
+        for i in range(n_layers):
+            one(i)
+    for _ in range(3):
+        chain()
+    torch.cuda.synchronize()
+    graph = None
+    if not args.no_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            chain()
+    run = graph.replay if graph is not None else chain
+    for _ in range(max(1, args.warmup // n_layers)):
+        run()
+    torch.cuda.synchronize()
+    reps = max(1, args.steps // n_layers)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / (reps * n_layers) * 1e3
+    # the pieces, each timed alone with events (eager launches, warm weights: lower bounds of their time in the layer)
+    net = layers[0]
+    xq = net.linear_qkv_down_proj(x)
+    q_c = net.q_layernorm(xq[:, :q_lora])
+    qq = net.linear_q_up_proj(q_c).reshape(b, nh, nope + rope)
+    query = torch.empty((b, nh, rank + rope), dtype=dt, device="cuda")
+    attn = torch.randn(b, nh, rank, generator=gen, device="cuda").to(dt)
+    core = torch.randn(b, nh * vd, generator=gen, device="cuda").to(dt)
+    qa_t, out_absorb = net._absorb
+    pieces = {
+        "qkv_down_proj": lambda: net.linear_qkv_down_proj(x),
+        "q_up_proj": lambda: net.linear_q_up_proj(q_c),
+        "absorb_query_bmm": lambda: ops.mla_absorb_bmm(qq[..., :nope], qa_t, out=query[..., :rank]),
+        "mla_paged_attention": lambda: ops.mla_paged_attention(query.reshape(b, -1), caches[0], tb, lt, nh, rank,
+                                                               net.softmax_scale),
+        "absorb_output_bmm": lambda: ops.mla_absorb_bmm(attn, out_absorb),
+        "linear_proj": lambda: net.linear_proj(core),
+    }
+    us = {}
+    for name, fn in pieces.items():
+        for _ in range(3):
+            fn()
+        us[name] = round(time_events(fn, args.kernel_iters, torch)[0] * 1e3, 2)
+    tokens = int(lens.astype(np.int64).sum())
+    w_bytes = (q_lora + rank + rope) * hidden + nh * (nope + rope) * q_lora + 2 * nh * (nope + vd) * rank + hidden * nh * vd
+    cache_bytes = tokens * (rank + rope) * 2
+    flops = 2.0 * (rank + rope + rank) * nh * tokens
+    ach = flops / (us["mla_paged_attention"] * 1e-6) / 1e12
+    result = {
+        "metric": "decode tokens/sec per multi-latent attention layer (DeepSeek-V3 shape, W8A16 projections, bs64)",
+        "value": round(b / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": reps * n_layers,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"deepseek_v3_mla_layer: MLASelfAttention decode step, batch {b}, hidden {hidden}, {nh} "
+                               f"heads, q_lora {q_lora}, latent {rank} + rope {rope}, ctx U[512,4096] (sum {tokens}), "
+                               f"block {bs}, W8A16 projections",
+                   "launch": "eager" if graph is None else f"hip_graph, {n_layers} layer steps on separate weights per replay",
+                   "algorithmic_bytes_per_layer": int(w_bytes + cache_bytes), "weight_bytes": int(w_bytes),
+                   "cache_bytes": int(cache_bytes)},
+        "layer_hbm_gbps": round((w_bytes + cache_bytes) / (ms * 1e-3) / 1e9, 1),
+        "unfused_op_us": us,
+        "roofline": dict(bound="mfma", kernel="mla_decode_kernel (+ mla_reduce_kernel)", achieved=round(ach, 1),
+                         peak=2500.0, unit="TFLOP/s", frac=round(ach / 2500.0, 4), traffic=None,
+                         flops_per_launch=flops, avg_launch_us=us["mla_paged_attention"]),
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -690,6 +809,9 @@ def main():
         return
     if args.workload == "deepseek_v3_mla_decode":
         bench_mla_decode(args, torch, ops)
+        return
+    if args.workload == "deepseek_v3_mla_layer":
+        bench_mla_layer(args, torch, ops)
         return
     if args.workload in ("llama3_8b_prefill_attention", "llama3_8b_chunked_prefill_attention",
                          "deepseek_v3_mla_prefill_attention"):

@@ -261,6 +261,25 @@ int mf_mla_absorb_bmm(void* out, const void* x, const void* w, int tokens, int h
                       int64_t x_token_stride, int64_t x_head_stride, int64_t out_token_stride,
                       int64_t out_head_stride, int dtype, void* stream);
 
+/* The element-wise work of MLASelfAttention.get_query_key_value_tensors between the down projections and the
+ * attention, in one launch - mindformers/parallel_core/inference/transformer/multi_latent_attention.py:391-403
+ * (kv_layernorm, rotary_pos_emb on q_pos_emb / k_pos_emb, concat + key-only reshape_and_cache) and :444-447 (the
+ * rotated query part behind the absorbed query):
+ *   kv [tokens, rank + rope] (rows kv_token_stride elements apart: a slice of the fused down projection): columns
+ *   [0, rank) are RMS-normalised with gamma / eps (rounded to dtype), columns [rank, rank + rope) rotated (rotate-half,
+ *   cos / sin [tokens, rope] rows gathered per token, table_dtype as mf_rope_half); both go to row slot_mapping[t] of
+ *   latent_cache [num_slots, rank + rope] (skipped for a negative / out-of-range slot or a NULL cache) and, where the
+ *   pointers are given, to the dense kv_norm_out [tokens, rank] and k_pe_out [tokens, rope];
+ *   q_rope points at the rotary part of head 0 of token 0 (head h of token t q_token_stride * t + q_head_stride * h
+ *   elements further); its rotation is stored likewise addressed at q_rope_out (q_rope_out == q_rope rotates in
+ *   place).  rank % 8 == 0, rope % 16 == 0, strides multiples of 8 elements, pointers 16-byte aligned. */
+int mf_mla_norm_rope_cache(void* q_rope_out, int64_t q_out_token_stride, int64_t q_out_head_stride,
+                           const void* q_rope, int64_t q_token_stride, int64_t q_head_stride, void* kv_norm_out,
+                           void* k_pe_out, const void* kv, int64_t kv_token_stride, const void* gamma, int gamma_dtype,
+                           float eps, const void* cos, const void* sin, int table_dtype, void* latent_cache,
+                           const int32_t* slot_mapping, int64_t num_slots, int tokens, int heads, int rank, int rope,
+                           int dtype, void* stream);
+
 /* ---- norm / activation ---------------------------------------------------------------------------- */
 
 /* P.RmsNorm(eps)(x, gamma): mindformers/models/llama/llama_layer.py:195,225-228;

@@ -877,6 +877,94 @@ int launch_absorb(void* out, const void* x, const void* w, int tokens, int heads
     return MF_LAUNCH_CHECK();
 }
 
+// ---- the element-wise work between the down projections and the attention, in one launch -------------------------
+// Per token: the latent part of the kv down projection is RMS-normalised, the shared rotary key part and the rotary
+// part of every head's query are rotated (rotate-half with the token's cos / sin row), the normalised latent row and
+// the rotated key part are written to the token's slot of the latent cache, and the rotated query part is stored
+// where the caller wants it (behind the absorbed query of a decode step, or back in place for a prefill).  Rounding
+// points as the separate kernels have them: the norm output is rounded to T, a rotation's two products and their
+// sum are rounded one by one (rope_pair) and the result to T.
+// grid (tokens, 1 + query parts): y = 0 handles the kv row (wave 0 the norm, wave 1 the key rotation), y >= 1 a
+// share of the heads; a work item is 8 consecutive elements of the first half of a rotary part and their partners.
+constexpr int MNR_THREADS = 256;
+
+template <typename T>
+__device__ __forceinline__ void mnr_rotate8(const uint16_t* src, uint16_t* dst0, uint16_t* dst1, const void* cos,
+                                            const void* sin, int64_t trow, int i0, int half, int table_dtype) {
+    float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8];
+    unpack8<T>(*(const u32x4*)(src + i0), x1);
+    unpack8<T>(*(const u32x4*)(src + half + i0), x2);
+    load8_as_float(cos, trow + i0, table_dtype, c1);
+    load8_as_float(sin, trow + i0, table_dtype, s1);
+    load8_as_float(cos, trow + half + i0, table_dtype, c2);
+    load8_as_float(sin, trow + half + i0, table_dtype, s2);
+    float o1[8], o2[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) rope_pair(x1[e], x2[e], c1[e], s1[e], c2[e], s2[e], o1[e], o2[e]);
+    const u32x4 a = {pack2<T>(o1[0], o1[1]), pack2<T>(o1[2], o1[3]), pack2<T>(o1[4], o1[5]), pack2<T>(o1[6], o1[7])};
+    const u32x4 b = {pack2<T>(o2[0], o2[1]), pack2<T>(o2[2], o2[3]), pack2<T>(o2[4], o2[5]), pack2<T>(o2[6], o2[7])};
+    *(u32x4*)(dst0 + i0) = a;
+    *(u32x4*)(dst0 + half + i0) = b;
+    if (dst1) {
+        *(u32x4*)(dst1 + i0) = a;
+        *(u32x4*)(dst1 + half + i0) = b;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(MNR_THREADS) void mla_norm_rope_cache_kernel(
+    uint16_t* __restrict__ q_rope_out, int64_t qo_token_stride, int64_t qo_head_stride, const uint16_t* __restrict__ q,
+    int64_t q_token_stride, int64_t q_head_stride, uint16_t* __restrict__ kv_norm_out, uint16_t* __restrict__ k_pe_out,
+    const uint16_t* __restrict__ kv, int64_t kv_token_stride, const void* __restrict__ gamma, int gamma_dtype, float eps,
+    const void* __restrict__ cos, const void* __restrict__ sin, int table_dtype, uint16_t* __restrict__ cache,
+    const int32_t* __restrict__ slot_mapping, int64_t num_slots, int heads, int rank, int rope) {
+    const int t = blockIdx.x;
+    const int half = rope >> 1;
+    const int64_t trow = (int64_t)t * rope;
+    const int per_head = half >> 3;                           // work items per rotary part
+    if (blockIdx.y > 0) {                                     // the rotary parts of the query heads
+        const int items = heads * per_head;
+        for (int it = (blockIdx.y - 1) * MNR_THREADS + threadIdx.x; it < items; it += (gridDim.y - 1) * MNR_THREADS) {
+            const int h = it / per_head, i0 = 8 * (it - h * per_head);
+            mnr_rotate8<T>(q + (int64_t)t * q_token_stride + (int64_t)h * q_head_stride,
+                           q_rope_out + (int64_t)t * qo_token_stride + (int64_t)h * qo_head_stride, nullptr, cos, sin,
+                           trow, i0, half, table_dtype);
+        }
+        return;
+    }
+    int64_t slot = cache ? slot_mapping[t] : -1;
+    uint16_t* crow = (slot >= 0 && slot < num_slots) ? cache + slot * (int64_t)(rank + rope) : nullptr;
+    const uint16_t* row = kv + (int64_t)t * kv_token_stride;
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wv == 0) {                                            // RMSNorm of the latent part: one wave
+        const int nvec = rank >> 3;
+        float ss = 0.f;
+        for (int c = lane; c < nvec; c += 64) {
+            float v[8];
+            unpack8<T>(*(const u32x4*)(row + 8 * c), v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[i], v[i], ss);
+        }
+        ss = wave_sum(ss);
+        const float inv = rsqrtf(ss / (float)rank + eps);
+        for (int c = lane; c < nvec; c += 64) {
+            float v[8], gm[8];
+            unpack8<T>(*(const u32x4*)(row + 8 * c), v);
+            load8_as_float(gamma, 8 * c, gamma_dtype, gm);
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = pack2<T>(v[2 * i] * inv * gm[2 * i], v[2 * i + 1] * inv * gm[2 * i + 1]);
+            if (kv_norm_out) *(u32x4*)(kv_norm_out + (int64_t)t * rank + 8 * c) = o;
+            if (crow) *(u32x4*)(crow + 8 * c) = o;
+        }
+    } else if (wv == 1) {                                     // the rotary key part, shared by the heads
+        // destinations: the dense copy when asked for, the cache row when the slot is live; with neither, nothing
+        uint16_t* d0 = k_pe_out ? k_pe_out + (int64_t)t * rope : (crow ? crow + rank : nullptr);
+        uint16_t* d1 = (k_pe_out && crow) ? crow + rank : nullptr;
+        if (d0 && lane < per_head) mnr_rotate8<T>(row + rank, d0, d1, cos, sin, trow, 8 * lane, half, table_dtype);
+    }
+}
+
 }  // namespace
 
 extern "C" size_t mf_mla_paged_attention_workspace_bytes(int batch, int n_heads, int max_context) {
@@ -944,4 +1032,41 @@ extern "C" int mf_mla_absorb_bmm(void* out, const void* x, const void* w, int to
                                    out_head_stride, st);
     return launch_absorb<FP16>(out, x, w, tokens, heads, n, k, x_token_stride, x_head_stride, out_token_stride,
                                out_head_stride, st);
+}
+
+extern "C" int mf_mla_norm_rope_cache(void* q_rope_out, int64_t q_out_token_stride, int64_t q_out_head_stride,
+                                      const void* q_rope, int64_t q_token_stride, int64_t q_head_stride,
+                                      void* kv_norm_out, void* k_pe_out, const void* kv, int64_t kv_token_stride,
+                                      const void* gamma, int gamma_dtype, float eps, const void* cos, const void* sin,
+                                      int table_dtype, void* latent_cache, const int32_t* slot_mapping,
+                                      int64_t num_slots, int tokens, int heads, int rank, int rope, int dtype,
+                                      void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "mla_norm_rope_cache: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32,
+               "mla_norm_rope_cache: bad gamma dtype");
+    MF_REQUIRE(table_dtype == MF_BF16 || table_dtype == MF_FP16 || table_dtype == MF_FP32,
+               "mla_norm_rope_cache: bad table dtype");
+    if (tokens <= 0) return 0;
+    MF_REQUIRE(q_rope_out && q_rope && kv && gamma && cos && sin, "mla_norm_rope_cache: null argument");
+    MF_REQUIRE(!latent_cache || (slot_mapping && num_slots > 0), "mla_norm_rope_cache: a cache needs slots");
+    MF_REQUIRE(heads > 0 && rank > 0 && rank % 8 == 0 && rope > 0 && rope % 16 == 0 && rope <= 1024,
+               "mla_norm_rope_cache: rank (%d) must be a multiple of 8, rope (%d) a multiple of 16", rank, rope);
+    MF_REQUIRE(q_out_token_stride % 8 == 0 && q_out_head_stride % 8 == 0 && q_token_stride % 8 == 0 &&
+                   q_head_stride % 8 == 0 && kv_token_stride % 8 == 0 && kv_token_stride >= rank + rope,
+               "mla_norm_rope_cache: strides must be multiples of 8 elements, kv rows at least rank + rope long");
+    MF_REQUIRE((((uintptr_t)q_rope_out | (uintptr_t)q_rope | (uintptr_t)kv | (uintptr_t)kv_norm_out |
+                 (uintptr_t)k_pe_out | (uintptr_t)latent_cache | (uintptr_t)gamma | (uintptr_t)cos | (uintptr_t)sin) & 15) == 0,
+               "mla_norm_rope_cache: pointers must be 16-byte aligned");
+    const int items = heads * (rope >> 4);
+    const dim3 grid(tokens, 1 + (items + MNR_THREADS - 1) / MNR_THREADS);
+#define MNR_LAUNCH(TT)                                                                                            \
+    hipLaunchKernelGGL(mla_norm_rope_cache_kernel<TT>, grid, dim3(MNR_THREADS), 0, (hipStream_t)stream,           \
+                       (uint16_t*)q_rope_out, q_out_token_stride, q_out_head_stride, (const uint16_t*)q_rope,     \
+                       q_token_stride, q_head_stride, (uint16_t*)kv_norm_out, (uint16_t*)k_pe_out,                \
+                       (const uint16_t*)kv, kv_token_stride, gamma, gamma_dtype, eps, cos, sin, table_dtype,      \
+                       (uint16_t*)latent_cache, slot_mapping, num_slots, heads, rank, rope)
+    if (dtype == MF_BF16) MNR_LAUNCH(BF16);
+    else MNR_LAUNCH(FP16);
+#undef MNR_LAUNCH
+    return MF_LAUNCH_CHECK();
 }

@@ -142,28 +142,45 @@ class MLASelfAttention(nn.Module):
         return super()._load_from_state_dict(*args, **kwargs)
 
     # ---- projections (:361-403) ------------------------------------------------------------------------------
-    def _project(self, hidden_states, rotary_pos_cos, rotary_pos_sin, slot_mapping, key_cache):
+    def _project(self, hidden_states, rotary_pos_cos, rotary_pos_sin, slot_mapping, key_cache, query_out=None):
+        """Down projections, norms, query up-projection, RoPE and the latent-row scatter.  Returns q [T, n, nope + rope]
+        and, for a prefill (``query_out`` None), the normalised latent rows and the rotated key part; the rotated query
+        parts go back into q, or, for a decode step, behind the absorbed query in ``query_out`` [T, n, rank + rope]."""
         c = self.config
         n, nope, rope, rank = c.num_attention_heads, c.qk_head_dim, c.qk_pos_emb_head_dim, c.kv_lora_rank
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
         if c.q_lora_rank is not None:
             qkv = self.linear_qkv_down_proj(x)
-            q_c, kv_c, k_pe = torch.split(qkv, [c.q_lora_rank, rank, rope], dim=-1)
-            q = self.linear_q_up_proj(self.q_layernorm(q_c))
+            kv = qkv[:, c.q_lora_rank:]                       # latent part, then the rotary key part
+            q = self.linear_q_up_proj(self.q_layernorm(qkv[:, : c.q_lora_rank]))
         else:
             kv = self.linear_kv_down_proj(x)
-            kv_c, k_pe = torch.split(kv, [rank, rope], dim=-1)
             q = self.linear_q_proj(x)
         t = x.shape[0]
         q = q.reshape(t, n, self.q_head_dim)
-        kv_c = self.kv_layernorm(kv_c)
-        q_pe = q[..., nope:].reshape(t, n * rope)                # a copy: the rotation wants dense rows
-        k_pe = k_pe.contiguous()
+        gamma = getattr(self.kv_layernorm, "weight", None)
+        if rotary_pos_cos is not None and rotary_pos_sin is not None and gamma is not None:
+            # kv_layernorm + RoPE + scatter + placement of the rotated query part: one launch
+            decode = query_out is not None
+            kv_c = None if decode else torch.empty((t, rank), dtype=q.dtype, device=q.device)
+            k_pe = None if decode else torch.empty((t, rope), dtype=q.dtype, device=q.device)
+            eps = getattr(self.kv_layernorm, "eps", c.layernorm_epsilon)
+            ops.mla_norm_rope_cache(q, nope, kv, gamma, eps, rotary_pos_cos.reshape(t, rope), rotary_pos_sin.reshape(t, rope),
+                                    latent_cache=key_cache, slot_mapping=slot_mapping,
+                                    q_rope_out=query_out[..., rank:] if decode else None, kv_norm_out=kv_c, k_pe_out=k_pe)
+            return q, kv_c, k_pe
+        # no rotary rows (or a norm cell without a gamma vector): the separate cells
+        kv_c = self.kv_layernorm(kv[:, :rank])
+        k_pe = kv[:, rank:].contiguous()
         if rotary_pos_cos is not None and rotary_pos_sin is not None:
+            q_pe = q[..., nope:].reshape(t, n * rope)
             self.rotary_pos_emb(q_pe, k_pe, rotary_pos_cos, rotary_pos_sin)
+            q[..., nope:] = q_pe.reshape(t, n, rope)
         if key_cache is not None:
             ops.reshape_and_cache(torch.cat((kv_c, k_pe), dim=-1), None, key_cache, None, slot_mapping)
-        return q, q_pe.reshape(t, n, rope), kv_c, k_pe
+        if query_out is not None:
+            query_out[..., rank:] = q[..., nope:]
+        return q, kv_c, k_pe
 
     def forward(self, hidden_states, attention_mask=None, key_value_states=None, rotary_pos_cos=None,
                 rotary_pos_sin=None, position_ids=None, batch_valid_length=None, block_tables=None, slot_mapping=None,
@@ -171,15 +188,14 @@ class MLASelfAttention(nn.Module):
                 value_cache=None):
         c = self.config
         n, nope, rope, rank, vd = c.num_attention_heads, c.qk_head_dim, c.qk_pos_emb_head_dim, c.kv_lora_rank, c.v_head_dim
-        q, q_pe, kv_c, k_pe = self._project(hidden_states, rotary_pos_cos, rotary_pos_sin, slot_mapping, key_cache)
-        t = q.shape[0]
         self.core_attention.is_prefill = self.is_prefill
         if self.is_prefill:
+            q, kv_c, k_pe = self._project(hidden_states, rotary_pos_cos, rotary_pos_sin, slot_mapping, key_cache)
+            t = q.shape[0]
             kv = self.linear_kv_up_proj(kv_c).reshape(t, -1)
             k_no_pe = kv[:, : n * nope].reshape(t, n, nope)
             value = kv[:, n * nope:].reshape(t, n, vd)
             k_rep = k_pe[:, None, :].expand(t, n, rope)
-            q[..., nope:] = q_pe                              # the rotated part back into the query rows
             key = torch.cat((k_no_pe, k_rep), dim=-1).reshape(t, n * self.q_head_dim)
             val = torch.cat((value, k_rep), dim=-1)
             if vd + rope != self.q_head_dim:
@@ -193,9 +209,10 @@ class MLASelfAttention(nn.Module):
             if self._absorb is None:
                 self.prepare()
             q_absorb_t, out_absorb = self._absorb
-            query = torch.empty((t, n, rank + rope), dtype=q.dtype, device=q.device)
+            t = hidden_states.reshape(-1, hidden_states.shape[-1]).shape[0]
+            query = torch.empty((t, n, rank + rope), dtype=self.compute_dtype, device=hidden_states.device)
+            q, _, _ = self._project(hidden_states, rotary_pos_cos, rotary_pos_sin, slot_mapping, key_cache, query_out=query)
             ops.mla_absorb_bmm(q[..., :nope], q_absorb_t, out=query[..., :rank])
-            query[..., rank:] = q_pe
             attn = self.core_attention(query.reshape(t, n * (rank + rope)), None, None, slot_mapping, block_tables,
                                        batch_valid_length, context_lens_tensor, q_seq_lens,
                                        actual_seq_qlen=actual_seq_qlen, actual_seq_kvlen=actual_seq_kvlen,

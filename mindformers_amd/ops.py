@@ -267,6 +267,48 @@ def mla_absorb_bmm(x, w, out=None):
     return out
 
 
+def mla_norm_rope_cache(q, nope, kv, gamma, eps, cos, sin, latent_cache=None, slot_mapping=None, q_rope_out=None,
+                        kv_norm_out=None, k_pe_out=None):
+    """kv_layernorm + RoPE of the rotary query / key parts + latent-row scatter in one launch
+    (multi_latent_attention.py:391-403, :444-447).  q [T, n, nope + rope] dense; kv [T, rank + rope] a view with a unit
+    last stride (latent part, then the rotary key part); gamma [rank]; cos / sin [T, rope].  The rotated query parts go
+    to ``q_rope_out`` (a [T, n, rope] view, e.g. the tail of the absorbed query) or back in place; the normalised
+    latent row and the rotated key part go to the cache row of the token's slot and, when given, to ``kv_norm_out``
+    [T, rank] / ``k_pe_out`` [T, rope]."""
+    lib = _lib.load()
+    dev = _dev_of(q, kv, gamma, cos, sin, latent_cache, slot_mapping, q_rope_out, kv_norm_out, k_pe_out)
+    _need(q.dim() == 3 and q.is_contiguous() and q.dtype in _ACT, "q must be a dense bf16/fp16 [T, n, nope + rope]")
+    t, n, qd = q.shape
+    rope = qd - nope
+    _need(kv.dim() == 2 and kv.shape[0] == t and kv.stride(1) == 1 and kv.dtype == q.dtype, "kv must be a [T, rank + rope] view")
+    rank = kv.shape[1] - rope
+    _need(rank > 0 and gamma.numel() == rank and gamma.is_contiguous(), "gamma must hold kv.shape[1] - rope values")
+    _need(cos.shape == (t, rope) and sin.shape == (t, rope) and cos.is_contiguous() and sin.is_contiguous() and
+          cos.dtype == sin.dtype, "cos / sin must be contiguous [T, rope]")
+    q_rope = q[..., nope:]
+    out = q_rope if q_rope_out is None else q_rope_out
+    _need(tuple(out.shape) == (t, n, rope) and out.stride(2) == 1 and out.dtype == q.dtype, "q_rope_out must be a [T, n, rope] view")
+    for buf, width, name in ((kv_norm_out, rank, "kv_norm_out"), (k_pe_out, rope, "k_pe_out")):
+        _need(buf is None or (tuple(buf.shape) == (t, width) and buf.is_contiguous() and buf.dtype == q.dtype),
+              f"{name} must be a contiguous [T, {width}]")
+    slots = 0
+    if latent_cache is not None:
+        _need(latent_cache.is_contiguous() and latent_cache.shape[-1] == rank + rope and latent_cache.dtype == q.dtype,
+              "latent_cache rows must hold rank + rope values of q's type")
+        _need(slot_mapping is not None and slot_mapping.dtype == torch.int32 and slot_mapping.numel() == t,
+              "slot_mapping must be int32 [T]")
+        slots = latent_cache.numel() // (rank + rope)
+    if t == 0:
+        return out
+    check(lib.mf_mla_norm_rope_cache(ptr(out), out.stride(0), out.stride(1), ptr(q_rope), q_rope.stride(0),
+                                     q_rope.stride(1), ptr(kv_norm_out), ptr(k_pe_out), ptr(kv), kv.stride(0), ptr(gamma),
+                                     dtype_code(gamma.dtype), float(eps), ptr(cos),
+                                     ptr(sin), dtype_code(cos.dtype),
+                                     ptr(latent_cache), ptr(slot_mapping), slots, t, n, rank, rope, dtype_code(q.dtype),
+                                     stream_ptr(dev)), "mf_mla_norm_rope_cache")
+    return out
+
+
 # --------------------------------------------------------------------------------------------- int8 KV cache
 def _kv_quant_params(scale, offset, row, dev):
     _need(isinstance(scale, torch.Tensor) and scale.dtype == torch.float32 and scale.numel() == 2 * row and

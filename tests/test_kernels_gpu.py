@@ -1491,6 +1491,61 @@ def test_mla_absorb_bmm_vs_oracle(dtype, t, h, k, n, strided):
     assert fresh.is_contiguous() and torch.equal(fresh, out_w[..., :n])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n,nope,rope,rank,q_lora,decode", [(64, 128, 128, 64, 512, 1536, True), (37, 16, 128, 64, 512, 0, False),
+                                                             (5, 3, 32, 16, 64, 8, True), (1, 128, 128, 64, 512, 1536, False)])
+def test_mla_norm_rope_cache_equals_the_separate_ops(dtype, t, n, nope, rope, rank, q_lora, decode):
+    """kv_layernorm + RoPE of the rotary query / key parts + latent-row scatter in one launch: the rotations are the
+    bits of apply_rotary_pos_emb, the normalised latent rows are within a rounding of rms_norm (the sum of squares is
+    taken in another order) and equal the oracle's norm to that bound; the cache rows of live slots hold [norm, rotated
+    key part], a -1 slot writes nothing, and the query part lands where it is asked for (in place, or behind the
+    absorbed query)."""
+    rng = np.random.default_rng(t + n + rope)
+    bs, nb = 16, (t + 15) // 16 + 2
+    q = rounded(rng.normal(size=(t, n, nope + rope)), dtype)
+    qkv = rounded(rng.normal(size=(t, q_lora + rank + rope)) * 2, dtype)
+    gamma = (1 + 0.1 * rng.normal(size=rank)).astype(np.float32)
+    ang = rng.uniform(0, 6, (t, rope // 2))
+    cos = rounded(np.concatenate((np.cos(ang), np.cos(ang)), 1), dtype)
+    sin = rounded(np.concatenate((np.sin(ang), np.sin(ang)), 1), dtype)
+    slots = rng.permutation(nb * bs)[:t].astype(np.int32)
+    if t > 2:
+        slots[t // 2] = -1
+    q_t, qkv_t = dev(q, dtype), dev(qkv, dtype)
+    cos_t, sin_t, g_t = dev(cos, dtype), dev(sin, dtype), torch.from_numpy(gamma).cuda()
+    cache = torch.full((nb, bs, 1, rank + rope), 3.0, dtype=dtype, device="cuda")
+    kv_view = qkv_t[:, q_lora:]
+    # the separate ops
+    q_pe_ref = q_t[..., nope:].reshape(t, n * rope).clone()       # copies: the separate op rotates in place
+    k_pe_ref = kv_view[:, rank:].clone()
+    ops.apply_rotary_pos_emb(q_pe_ref, k_pe_ref, cos_t, sin_t, n, 1, rope)
+    norm_ref = ops.rms_norm(kv_view[:, :rank].clone(), g_t, 1e-6)
+    if decode:
+        query = torch.full((t, n, rank + rope), 9.0, dtype=dtype, device="cuda")
+        ops.mla_norm_rope_cache(q_t, nope, kv_view, g_t, 1e-6, cos_t, sin_t, cache, torch.from_numpy(slots).cuda(),
+                                q_rope_out=query[..., rank:])
+        assert torch.equal(query[..., rank:].reshape(t, n * rope), q_pe_ref) and (query[..., :rank] == 9).all()
+        assert torch.equal(q_t, dev(q, dtype))                      # the source rows are left alone
+    else:
+        kv_norm, k_pe = torch.empty(t, rank, dtype=dtype, device="cuda"), torch.empty(t, rope, dtype=dtype, device="cuda")
+        ops.mla_norm_rope_cache(q_t, nope, kv_view, g_t, 1e-6, cos_t, sin_t, cache, torch.from_numpy(slots).cuda(),
+                                kv_norm_out=kv_norm, k_pe_out=k_pe)
+        assert torch.equal(q_t[..., nope:].reshape(t, n * rope), q_pe_ref)
+        assert torch.equal(q_t[..., :nope], dev(q, dtype)[..., :nope])
+        assert torch.equal(k_pe, k_pe_ref)
+        ref = O.rms_norm(qkv[:, q_lora:q_lora + rank], gamma, 1e-6)
+        assert_within(to_np(kv_norm), ref, np.abs(ref), dtype, ulps=1.0, extra=1e-7, what="latent norm")
+        assert (np.abs(to_np(kv_norm) - to_np(norm_ref)) <= EPS[dtype] * np.abs(to_np(norm_ref)) * 2 + 1e-7).all()
+    got = to_np(cache).reshape(nb * bs, rank + rope)
+    live = slots[slots >= 0]
+    rows = np.flatnonzero(slots >= 0)
+    assert np.array_equal(got[live][:, rank:], to_np(k_pe_ref)[rows])
+    assert (np.abs(got[live][:, :rank] - to_np(norm_ref)[rows]) <= EPS[dtype] * np.abs(to_np(norm_ref)[rows]) * 2 + 1e-7).all()
+    untouched = np.ones(nb * bs, bool)
+    untouched[live] = False
+    assert (got[untouched] == 3).all()
+
+
 def test_mla_absorb_bmm_rejects_bad_operands():
     x = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError):
