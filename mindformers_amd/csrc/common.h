@@ -21,6 +21,11 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define MF_WAVE 64
 #define MF_MAX_DEVICES 64                 // per-device one-off kernel configuration flags
+// The packed int8 operand format shared by both GEMM families (and by mf_w8a16_packed_bytes, which sizes it for
+// either): 1 KiB tiles of 16 rows x 64 columns.  Each family names the two constants its own way and asserts them
+// against these.
+constexpr int MF_PACK_KSTEP = 64;
+constexpr int MF_PACK_TILE_BYTES = 16 * MF_PACK_KSTEP;
 
 // Host-side argument error: remember the message, return hipErrorInvalidValue.
 void mf_set_error(const char* fmt, ...);

@@ -33,6 +33,7 @@ constexpr int GW_NT = 4;                    // 16-row weight tiles per wave
 constexpr int GW_BN = 16 * GW_NT;           // output channels per workgroup
 constexpr int GW_KSTEP = 64;
 constexpr int GW_TILE_BYTES = 16 * GW_KSTEP;
+static_assert(GW_KSTEP == MF_PACK_KSTEP && GW_TILE_BYTES == MF_PACK_TILE_BYTES, "the packed format is shared with the int8 GEMMs");
 constexpr int GW_DEPTH = 2;                 // weight k-steps in flight per wave beyond the current one
 
 // acc * scale (+ bias) with separately rounded operations: every epilogue below goes through here, so that the

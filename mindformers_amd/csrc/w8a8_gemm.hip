@@ -29,6 +29,7 @@ namespace {
 
 constexpr int Q_KSTEP = 64;
 constexpr int Q_TILE = 16 * Q_KSTEP;        // bytes of one packed weight tile
+static_assert(Q_KSTEP == MF_PACK_KSTEP && Q_TILE == MF_PACK_TILE_BYTES, "the int8 GEMMs read the shared packed format");
 
 // MSPLIT: wave grid of a workgroup.  0: 1 x 4 (64 rows, the waves own different channels); 1: 4 x 1 (256 rows, one
 // channel group).
