@@ -528,8 +528,9 @@ def bench_prefill_attention(args, torch, ops):
     block 128): `llama3_8b_prefill_attention` = 4 prompts of 2048 tokens, `llama3_8b_chunked_prefill_attention` =
     4 sequences adding 512 tokens behind 3584 cached ones.  A step is one attention call; flops = 4 * D * heads *
     (query, key) pairs inside the causal limit.  `deepseek_v3_mla_prefill_attention` = the prefill of multi-latent
-    attention (multi_latent_attention.py:405-432): 4 prompts of 2048 tokens, 128 heads, queries, keys and values 192
-    wide, taken from the step's own packed rows (no cache)."""
+    attention (multi_latent_attention.py:405-432): 4 prompts of 2048 tokens, 128 heads, queries and keys 192 wide,
+    values 128 wide (what the layer has; the reference pads them to 192 and drops the extra output columns), taken
+    from the step's own packed rows (no cache); flops = 2 * (192 + 128) * heads * pairs."""
     mla = args.workload == "deepseek_v3_mla_prefill_attention"
     nh, nkv, d, bs, dt = (128, 128, 192, 128, torch.bfloat16) if mla else (32, 8, 128, 128, torch.bfloat16)
     chunked = args.workload == "llama3_8b_chunked_prefill_attention"
@@ -547,7 +548,7 @@ def bench_prefill_attention(args, torch, ops):
     t = int(q_lens.sum())
     if mla:
         kc = torch.randn(t, nkv * d, generator=gen, device="cuda").to(dt)
-        vc = torch.randn(t, nkv * d, generator=gen, device="cuda").to(dt)
+        vc = torch.randn(t, nkv * 128, generator=gen, device="cuda").to(dt)
     else:
         kc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
         vc = torch.randn(nb, bs, nkv, d, generator=gen, device="cuda").to(dt)
@@ -555,7 +556,7 @@ def bench_prefill_attention(args, torch, ops):
     starts = torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device="cuda")
     lens_t = torch.tensor(lens, dtype=torch.int32, device="cuda")
     tb = torch.tensor(tables, device="cuda")
-    out = torch.empty_like(q)
+    out = torch.empty(t, nh * 128, dtype=dt, device="cuda") if mla else torch.empty_like(q)
 
     def step():
         if mla:
@@ -571,7 +572,7 @@ def bench_prefill_attention(args, torch, ops):
     ms = (time.perf_counter() - t0) / args.steps * 1e3
     us = time_events(step, args.kernel_iters, torch)[0] * 1e3
     pairs = int(sum(int(ql) * (int(L) - int(ql)) + int(ql) * (int(ql) + 1) // 2 for L, ql in zip(lens, q_lens)))
-    flops = 4.0 * d * nh * pairs
+    flops = (2.0 * (192 + 128) if mla else 4.0 * d) * nh * pairs
     ach = flops / (us * 1e-6) / 1e12
     peak = 2500.0
     result = {
@@ -583,6 +584,7 @@ def bench_prefill_attention(args, torch, ops):
         "config": {"workload": f"{args.workload}: causal attention over "
                                f"{'the packed rows of the step' if mla else 'the paged cache'}, {len(lens)} sequences, "
                                f"{int(q_lens[0])} new tokens each, context {int(lens[0])}, {nh}q/{nkv}kv heads x {d}"
+                               f"{' (values 128 wide)' if mla else ''}"
                                f"{'' if mla else ', block 128'}",
                    "launch": "eager", "flops_per_step": flops},
         "roofline": dict(bound="mfma", kernel="prefill_attention_kernel (+ partition reduce when partitioned)",

@@ -136,6 +136,19 @@ int mf_quant_reshape_and_cache(const void* key, const void* value, void* key_cac
                                int num_tokens, int n_kv_heads, int head_dim, int64_t num_slots,
                                int64_t key_row_stride, int64_t value_row_stride, int dtype, void* stream);
 
+/* FlashAttentionScore of the prefill of multi-latent attention -
+ * mindformers/parallel_core/inference/transformer/multi_latent_attention.py:405-432, :206-216: queries and keys have
+ * 192-wide heads (the up-projected 128 dimensions followed by the 64 rotary ones), values 128-wide heads.  The
+ * reference pads the values to 192 and keeps the first 128 output columns; this entry point takes the values as
+ * they are and returns out [total_q, n_heads * 128], the same numbers without the padded third of the PV product.
+ * Packed rows as mf_paged_attention_prefill with block_tables == NULL (causal, q_starts [batch + 1]); row strides
+ * in elements, 0 = dense.  Workspace: mf_paged_attention_prefill_workspace_bytes(batch, total_q, n_heads,
+ * n_kv_heads, 128, total_q). */
+int mf_causal_attention_qk192_v128(void* out, const void* query, const void* key, const void* value,
+                                   const int32_t* q_starts, int batch, int total_q, int n_heads, int n_kv_heads,
+                                   float scale, int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* mf_paged_attention_decode / _prefill on int8 caches: same arguments plus antiquant_scale / antiquant_offset
  * (offset may be NULL); workspaces as for the 16-bit entry points; paged keys only.  Scores use the query with
  * the key scale folded in (rounded to dtype); a key offset shifts all scores of a row equally and cancels in the

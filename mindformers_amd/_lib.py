@@ -38,6 +38,7 @@ SIGNATURES = {
                                                         _L, _I, _P, _Z, _P]),
     "mf_paged_attention_prefill_int8kv_per_token": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                                          _I, _F, _L, _I, _P, _Z, _P]),
+    "mf_causal_attention_qk192_v128": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _L, _L, _L, _I, _P, _Z, _P]),
     "mf_mla_paged_attention_workspace_bytes": (_Z, [_I, _I, _I]),
     "mf_mla_paged_attention_decode": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _L, _I, _P, _Z, _P]),
     "mf_mla_norm_rope_cache": (_I, [_P, _L, _L, _P, _L, _L, _P, _P, _P, _L, _P, _I, _F, _P, _P, _I, _P, _P, _L, _I, _I, _I,

@@ -66,21 +66,26 @@ struct PfSmem {
 };
 
 // Three workgroups per compute unit; two at 192-wide heads (72 KB of LDS and 96 accumulator registers each).
-template <typename T, int D, bool TIB>
+// DV: width of a value head and of an output head.  DV < D (the prefill of multi-latent attention: 192-wide queries
+// and keys, 128-wide values, packed rows only) loads and multiplies the first sub-tile of the value rows only.
+template <typename T, int D, bool TIB, int DV = D>
 __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_attention_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_out, float* __restrict__ part_ml,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx_lens, int n_heads, int n_kv,
     int n_rep, int block_size, int max_blocks, int num_blocks, int max_parts, float scale_log2, int64_t q_stride,
-    int batch, const int32_t* __restrict__ q_starts, int part_tokens, int64_t kv_stride, int rows) {
+    int batch, const int32_t* __restrict__ q_starts, int part_tokens, int64_t kv_stride, int rows,
+    int64_t v_stride) {
     using vec8 = typename T::vec8;
     using S = PfSmem<D>;
+    static_assert(DV == D || DV == S::W0, "value heads as wide as the key heads, or as their first sub-tile");
     constexpr int KS = D / 16;                                // k-steps of the score product
-    constexpr int DB = D / 32;                                // 32-row blocks of O^T
+    constexpr int DB = DV / 32;                               // 32-row blocks of O^T
     constexpr int NV = 2 * DB;                                // PV MFMAs per tile
     using S0 = typename S::Sub0;
     using S1 = typename S::Sub1;
     constexpr int NI = S::NI;
+    constexpr int NIV = DV == D ? NI : S0::NI;                // value loads per loading wave and tile
     constexpr int KS0 = S::W0 / 16;                           // k-steps served by the first sub-tile
     constexpr int DB0 = S::W0 / 32;                           // 32-row blocks of O^T served by the first sub-tile
 
@@ -183,6 +188,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
     const bool contiguous = block_tables == nullptr;
     const int32_t* table = block_tables + (int64_t)b * max_blocks;
     const int64_t row_bytes = kv_stride * 2;
+    const int64_t v_row_bytes = v_stride * 2;
 
     // ---- tile loads: load i of wave w into a sub-tile brings its rows (LW i + w) RPI .. + RPI - 1; lane = (row in
     // the group, LDS slot).  The loads of the first sub-tile come first in the arrays.
@@ -200,9 +206,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
         const int key = (row / SS::RPB) & (SS::CPR - 1);
         const int key4 = (row / SS::RPB) & (SS::CPR / 4 - 1);
         kcol[i] = (uint32_t)(kvh * D * 2 + col0 + 16 * (lslot ^ key));
-        vcol[i] = (uint32_t)(kvh * D * 2 + col0 + 16 * ((lslot - 4 * key4) & (SS::CPR - 1)));
+        vcol[i] = (uint32_t)(kvh * DV * 2 + col0 + 16 * ((lslot - 4 * key4) & (SS::CPR - 1)));
         kofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + kcol[i];      // offsets within a whole tile
-        vofs[i] = (uint32_t)(row * (int)(kv_stride * 2)) + vcol[i];
+        vofs[i] = (uint32_t)(row * (int)(v_stride * 2)) + vcol[i];
     });
     const int part_end = min(Lwg, part_start + part_tokens);
     const int ntiles = (part_end - part_start + PF_TOK - 1) / PF_TOK;
@@ -226,7 +232,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
         const int last_row = Lwg - 1 - ts;
         if (TIB && last_row >= PF_TOK - 1) {                  // whole tile inside one block: constant lane offsets
             const uint8_t* kb = (const uint8_t*)kc + slot0 * row_bytes;
-            const uint8_t* vb = (const uint8_t*)vc + slot0 * row_bytes;
+            const uint8_t* vb = (const uint8_t*)vc + slot0 * v_row_bytes;
             static_for<NI>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 constexpr bool second = i >= S0::NI;
@@ -235,8 +241,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
                 uint8_t* dst = kdst + (second ? S::SUB1 : 0) + (SS::LW * li + w) * SS::RPI * SS::ROWB;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb + kofs[i]),
                                                  (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + vofs[i]),
-                                                 (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
+                if constexpr (i < NIV)
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + vofs[i]),
+                                                     (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
             });
             return;
         }
@@ -250,9 +257,8 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
             const int rc = min(r0 + lane / SS::CPR, last_row);
             const uint8_t *kp, *vp;
             if constexpr (TIB) {                              // uniform base, 32-bit lane offset
-                const uint32_t lo = (uint32_t)(rc * (int)row_bytes);
-                kp = (const uint8_t*)kc + slot0 * row_bytes + (lo + kcol[i]);
-                vp = (const uint8_t*)vc + slot0 * row_bytes + (lo + vcol[i]);
+                kp = (const uint8_t*)kc + slot0 * row_bytes + ((uint32_t)(rc * (int)row_bytes) + kcol[i]);
+                vp = (const uint8_t*)vc + slot0 * v_row_bytes + ((uint32_t)(rc * (int)v_row_bytes) + vcol[i]);
             } else {
                 const int tok = ts + rc;
                 const int bi = tok / block_size;
@@ -264,8 +270,9 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
             }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
                                              (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
-                                             (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
+            if constexpr (i < NIV)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
+                                                 (__attribute__((address_space(3))) void*)(dst + S::KBYTES), 16, 0, 0);
         });
     };
 
@@ -406,7 +413,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
     // whose buffer takes tile t + 2
     auto sync_issue = [&](int t) {
         __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NI) : "memory");
+        if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NI + NIV) : "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -440,7 +447,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
     const int64_t gh = (int64_t)(q_start + qi) * n_heads + kvh * n_rep + hcol;
     if (max_parts == 1) {
         const float inv = 1.0f / l_run;
-        uint16_t* dst = out + gh * D + 4 * h;
+        uint16_t* dst = out + gh * DV + 4 * h;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -450,7 +457,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, D == 192 ? 2 : 3) void prefill_atten
                             pack2<T>(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv)};
     } else {
         const int64_t pi = gh * max_parts + part;
-        float* dst = part_out + pi * D + 4 * h;
+        float* dst = part_out + pi * DV + 4 * h;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -515,17 +522,19 @@ __global__ void pf_zero_rows_kernel(uint16_t* __restrict__ out, const int32_t* _
     }
 }
 
-template <typename T, int D, int KVQ>
+template <typename T, int D, int KVQ, int DV = D>
 int launch_pf(void* out, const void* query, const void* key_cache, const void* value_cache,
               const int32_t* block_tables, const int32_t* context_lens, const int32_t* q_starts, int batch,
               int total_q, int n_heads, int n_kv, int block_size, int max_blocks, int num_blocks, float scale,
               int64_t q_stride, int64_t kv_stride, void* workspace, hipStream_t st, const float* kv_scale,
-              const float* kv_offset) {
+              const float* kv_offset, int64_t v_stride = 0) {
+    static_assert(DV == D || KVQ == 0, "value heads narrower than the key heads: 16-bit packed rows only");
+    if (v_stride <= 0) v_stride = kv_stride;
     const int n_rep = n_heads / n_kv;
     const bool contiguous = block_tables == nullptr;
     const PfPlan plan = pf_plan(batch, total_q, n_heads, n_kv, contiguous ? total_q : (int64_t)max_blocks * block_size);
     float* part_out = plan.max_parts > 1 ? (float*)workspace : nullptr;
-    float* part_ml = part_out ? part_out + (int64_t)total_q * n_heads * plan.max_parts * D : nullptr;
+    float* part_ml = part_out ? part_out + (int64_t)total_q * n_heads * plan.max_parts * DV : nullptr;
     const float scale_log2 = scale * 1.4426950408889634f;
     constexpr bool KV8 = KVQ != 0;
     const int64_t wgs = (KV8 ? plan.col_groups16 : plan.col_groups128) * n_kv * plan.max_parts;
@@ -535,7 +544,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     }
     if (plan.max_parts == 1) {
         hipLaunchKernelGGL(pf_zero_rows_kernel, dim3(batch), dim3(256), 0, st, (uint16_t*)out, q_starts, context_lens,
-                           contiguous, max_blocks * block_size, batch, n_heads * D, total_q);
+                           contiguous, max_blocks * block_size, batch, n_heads * DV, total_q);
         int rc = MF_LAUNCH_CHECK();
         if (rc) return rc;
     }
@@ -559,7 +568,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
         if (e != hipSuccess) return (int)e;
 #define PF_LAUNCH(TIBV)                                                                                           \
     {                                                                                                             \
-        auto kern = prefill_attention_kernel<T, D, TIBV>;                                                         \
+        auto kern = prefill_attention_kernel<T, D, TIBV, DV>;                                                     \
         if (dev < 0 || dev >= MF_MAX_DEVICES || !lds_set[TIBV][dev]) {                                            \
             e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,                \
                                     PfSmem<D>::BYTES);                                                            \
@@ -570,7 +579,7 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
                            part_out, part_ml, (const uint16_t*)query, (const uint16_t*)key_cache,                 \
                            (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep,        \
                            block_size, max_blocks, num_blocks, plan.max_parts, scale_log2, q_stride, batch,       \
-                           q_starts, plan.part_tokens, kv_stride, total_q);                                       \
+                           q_starts, plan.part_tokens, kv_stride, total_q, v_stride);                             \
     }
         if (tib) PF_LAUNCH(true)
         else PF_LAUNCH(false)
@@ -579,8 +588,8 @@ int launch_pf(void* out, const void* query, const void* key_cache, const void* v
     int rc = MF_LAUNCH_CHECK();
     if (rc) return rc;
     if (plan.max_parts > 1) {
-        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, D, true>), dim3(n_heads, total_q),
-                           dim3(PA_REDUCE_THREADS<D>), 0, st,
+        hipLaunchKernelGGL((paged_attention_reduce_kernel<T, DV, true>), dim3(n_heads, total_q),
+                           dim3(PA_REDUCE_THREADS<DV>), 0, st,
                            (uint16_t*)out, part_out, part_ml, context_lens, n_heads, plan.max_parts,
                            plan.part_tokens, q_starts, batch, contiguous, max_blocks * block_size);
         rc = MF_LAUNCH_CHECK();
@@ -717,3 +726,38 @@ extern "C" int mf_paged_attention_prefill_int8kv_per_token(void* out, const void
                             value_scale_cache);
 }
 
+extern "C" int mf_causal_attention_qk192_v128(void* out, const void* query, const void* key, const void* value,
+                                              const int32_t* q_starts, int batch, int total_q, int n_heads,
+                                              int n_kv_heads, float scale, int64_t q_row_stride,
+                                              int64_t k_row_stride, int64_t v_row_stride, int dtype, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "causal_attention_qk192_v128: dtype must be bf16 or fp16");
+    MF_REQUIRE(batch >= 0 && total_q >= 0, "causal_attention_qk192_v128: negative batch or row count");
+    if (batch == 0 || total_q == 0) return 0;
+    MF_REQUIRE(out && query && key && value && q_starts, "causal_attention_qk192_v128: null argument");
+    MF_REQUIRE(scale > 0.f, "causal_attention_qk192_v128: the softmax scale must be positive");
+    MF_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+               "causal_attention_qk192_v128: n_heads (%d) must be a positive multiple of n_kv_heads (%d)", n_heads,
+               n_kv_heads);
+    if (q_row_stride <= 0) q_row_stride = (int64_t)n_heads * 192;
+    if (k_row_stride <= 0) k_row_stride = (int64_t)n_kv_heads * 192;
+    if (v_row_stride <= 0) v_row_stride = (int64_t)n_kv_heads * 128;
+    MF_REQUIRE(q_row_stride >= (int64_t)n_heads * 192 && k_row_stride >= (int64_t)n_kv_heads * 192 &&
+                   v_row_stride >= (int64_t)n_kv_heads * 128 && q_row_stride % 8 == 0 && k_row_stride % 8 == 0 &&
+                   v_row_stride % 8 == 0,
+               "causal_attention_qk192_v128: row strides must cover a row and be multiples of 8 elements");
+    MF_REQUIRE((((uintptr_t)out | (uintptr_t)query | (uintptr_t)key | (uintptr_t)value) & 15) == 0,
+               "causal_attention_qk192_v128: out / query / key / value must be 16-byte aligned");
+    const size_t need = mf_paged_attention_prefill_workspace_bytes(batch, total_q, n_heads, n_kv_heads, 128, total_q);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "causal_attention_qk192_v128: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MF_BF16)
+        return launch_pf<BF16, 192, 0, 128>(out, query, key, value, nullptr, nullptr, q_starts, batch, total_q, n_heads,
+                                            n_kv_heads, 0, 0, 0, scale, q_row_stride, k_row_stride, workspace, st,
+                                            nullptr, nullptr, v_row_stride);
+    return launch_pf<FP16, 192, 0, 128>(out, query, key, value, nullptr, nullptr, q_starts, batch, total_q, n_heads,
+                                        n_kv_heads, 0, 0, 0, scale, q_row_stride, k_row_stride, workspace, st, nullptr,
+                                        nullptr, v_row_stride);
+}

@@ -83,10 +83,13 @@ class FlashAttention(nn.Module):
             # cache's (pa_kv_head_num = 1): its prefill attends over the up-projected 192-wide keys of every head
             # (multi_latent_attention.py:405-432)
             d = q2.shape[1] // self.head_num
-            if q2.shape[1] != self.head_num * d or k2.shape[1] % d or v2.shape[1] != k2.shape[1]:
+            narrow_v = d == 192 and k2.shape[1] % d == 0 and v2.shape[1] == k2.shape[1] // d * 128
+            if q2.shape[1] != self.head_num * d or k2.shape[1] % d or (v2.shape[1] != k2.shape[1] and not narrow_v):
                 raise ValueError(f"query / key / value widths {q2.shape[1]} / {k2.shape[1]} / {v2.shape[1]} do not "
                                  f"fit {self.head_num} heads")
             out = ops.causal_attention_varlen(q2, k2, v2, starts, self.head_num, k2.shape[1] // d, self.scale_value)
+            if narrow_v:                                      # 128-wide value heads of multi-latent attention, unpadded
+                return out
             return out.reshape(shape)
         if self.use_multi_latent_attention:                   # one latent cache, keys = values (flash_attention.py:136-139)
             out = ops.mla_paged_attention(q2, key_cache, block_tables, batch_valid_length, self.head_num,

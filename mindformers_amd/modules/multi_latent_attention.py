@@ -197,14 +197,23 @@ class MLASelfAttention(nn.Module):
             value = kv[:, n * nope:].reshape(t, n, vd)
             k_rep = k_pe[:, None, :].expand(t, n, rope)
             key = torch.cat((k_no_pe, k_rep), dim=-1).reshape(t, n * self.q_head_dim)
-            val = torch.cat((value, k_rep), dim=-1)
-            if vd + rope != self.q_head_dim:
-                val = torch.nn.functional.pad(val, (0, self.q_head_dim - vd - rope))
-            out = self.core_attention(q.reshape(t, n * self.q_head_dim), key, val.reshape(t, n * self.q_head_dim),
+            if self.q_head_dim == 192 and vd == 128:
+                # the attention takes the 128-wide values as they are (the reference pads them to the key width with
+                # the rotary part and keeps the first 128 output columns: the same numbers)
+                val = value.reshape(t, n * vd)
+            else:
+                val = torch.cat((value, k_rep), dim=-1)
+                if vd + rope != self.q_head_dim:
+                    val = torch.nn.functional.pad(val, (0, self.q_head_dim - vd - rope))
+                val = val.reshape(t, n * self.q_head_dim)
+            out = self.core_attention(q.reshape(t, n * self.q_head_dim), key, val,
                                       slot_mapping, block_tables, batch_valid_length, context_lens_tensor, q_seq_lens,
                                       actual_seq_qlen=actual_seq_qlen, actual_seq_kvlen=actual_seq_kvlen,
                                       attn_mask=attention_mask, key_cache=key_cache, value_cache=value_cache)
-            core = out.reshape(t, n, self.q_head_dim)[..., :vd].reshape(t, n * vd)
+            if val.shape[1] == n * vd:
+                core = out.reshape(t, n * vd)
+            else:
+                core = out.reshape(t, n, self.q_head_dim)[..., :vd].reshape(t, n * vd)
         else:
             if self._absorb is None:
                 self.prepare()

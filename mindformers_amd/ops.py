@@ -498,7 +498,9 @@ def paged_attention_prefill(query, key_cache, value_cache, block_tables, context
 def causal_attention_varlen(query, key, value, q_starts, n_heads, n_kv_heads, scale, out=None):
     """FlashAttentionScore in the TH layout with a causal mask and actual_seq_qlen == actual_seq_kvlen: packed
     rows, sequence b owns rows q_starts[b] .. q_starts[b+1]-1 of query, key and value.  key / value may be column
-    slices of a fused projection output (equal row strides)."""
+    slices of a fused projection output (equal row strides).  With 192-wide query / key heads the value heads may be
+    128 wide (multi-latent attention): the result then has 128-wide heads, the numbers the 192-wide call gives on
+    zero-padded values in its first 128 columns."""
     lib = _lib.load()
     dev = _dev_of(query, key, value)
     _dev_ok(out)
@@ -508,11 +510,27 @@ def causal_attention_varlen(query, key, value, q_starts, n_heads, n_kv_heads, sc
     d = query.shape[1] // n_heads
     query, qs = _rows(query, n_heads * d, "query")
     key, ks = _rows(key, n_kv_heads * d, "key")
+    total_q = query.shape[0]
+    b = _q_starts(q_starts, dev)
+    if value.shape[1] != key.shape[1]:
+        # value heads narrower than the key heads: the prefill of multi-latent attention (192-wide keys, 128-wide values)
+        _need(d == 192 and value.shape[1] == n_kv_heads * 128, "narrower value heads are built for 192-wide keys with 128-wide values")
+        value, vs = _rows(value, n_kv_heads * 128, "value")
+        _need(key.shape[0] == total_q and value.shape[0] == total_q, "query, key and value must have the same number of rows")
+        if out is None:
+            out = torch.empty((total_q, n_heads * 128), dtype=query.dtype, device=dev)
+        else:
+            _need(out.numel() == total_q * n_heads * 128 and out.dtype == query.dtype and out.is_contiguous(), "out mismatch")
+        need = lib.mf_paged_attention_prefill_workspace_bytes(b, total_q, n_heads, n_kv_heads, 128, total_q)
+        ws = workspace(need, dev, "pa_prefill") if need else None
+        check(lib.mf_causal_attention_qk192_v128(ptr(out), ptr(query), ptr(key), ptr(value), ptr(q_starts), b, total_q,
+                                                 n_heads, n_kv_heads, float(scale), qs, ks, vs, dtype_code(query.dtype),
+                                                 ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+              "mf_causal_attention_qk192_v128")
+        return out
     value, vs = _rows(value, n_kv_heads * d, "value")
     _need(ks == vs, "key and value must have the same row stride")
-    total_q = query.shape[0]
     _need(key.shape[0] == total_q and value.shape[0] == total_q, "query, key and value must have the same number of rows")
-    b = _q_starts(q_starts, dev)
     if out is None:
         out = torch.empty((total_q, n_heads * d), dtype=query.dtype, device=dev)
     else:

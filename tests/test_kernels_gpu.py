@@ -407,6 +407,38 @@ def test_causal_attention_varlen_vs_oracle(dtype, nh, nkv, d, q_lens, fused):
     assert_within(out, ref, mag, dtype, ulps=1.5, what="varlen causal attention")
 
 
+@pytest.mark.parametrize("dtype,nh,nkv,q_lens,strided", [
+    (torch.bfloat16, 16, 16, [130, 1, 64], False), (torch.float16, 8, 2, [33, 200], True),
+    (torch.bfloat16, 2, 2, [1500], False), (torch.bfloat16, 128, 128, [40, 300], True),
+])
+def test_causal_attention_with_128_wide_values_under_192_wide_keys(dtype, nh, nkv, q_lens, strided):
+    """The prefill of multi-latent attention with the values as they are (128 wide) instead of padded to the key
+    width: against the oracle on the same values (its 128 output columns), and bit for bit the first 128 columns of
+    every head of the 192-wide call on zero-padded values, whose last 64 columns it never computes."""
+    rng = np.random.default_rng(nh + len(q_lens))
+    t = int(np.sum(q_lens))
+    q = rounded(rng.normal(size=(t, nh * 192)), dtype)
+    k = rounded(rng.normal(size=(t, nkv * 192)), dtype)
+    v = rounded(rng.normal(size=(t, nkv * 128)), dtype)
+    scale = 1.0 / np.sqrt(192)
+    starts = dev(_starts(q_lens), torch.int32)
+    if strided:                                                   # key and value as column slices of one buffer
+        kv_t = dev(np.concatenate((k, v), 1), dtype)
+        k_t, v_t = kv_t[:, :nkv * 192], kv_t[:, nkv * 192:]
+    else:
+        k_t, v_t = dev(k, dtype), dev(v, dtype)
+    out = ops.causal_attention_varlen(dev(q, dtype), k_t, v_t, starts, nh, nkv, scale)
+    assert out.shape == (t, nh * 128)
+    v_pad = np.concatenate((v.reshape(t, nkv, 128), np.zeros((t, nkv, 64), np.float32)), 2).reshape(t, nkv * 192)
+    wide = ops.causal_attention_varlen(dev(q, dtype), dev(k, dtype), dev(v_pad, dtype), starts, nh, nkv, scale)
+    assert torch.equal(out.reshape(t, nh, 128), wide.reshape(t, nh, 192)[..., :128])
+    ref = O.causal_prefill_attention(q, k, v_pad, q_lens, nh, nkv, scale).reshape(t, nh, 192)[..., :128]
+    mag = O.causal_prefill_attention(q, k, np.abs(v_pad), q_lens, nh, nkv, scale).reshape(t, nh, 192)[..., :128]
+    assert_within(to_np(out).reshape(t, nh, 128), ref, mag, dtype, ulps=1.5, what="192 / 128 causal attention")
+    with pytest.raises(ValueError):                               # other widths are not built
+        ops.causal_attention_varlen(dev(q, dtype), dev(k, dtype), dev(v[:, : nkv * 64].copy(), dtype), starts, nh, nkv, scale)
+
+
 @pytest.mark.parametrize("case,n_kv", [("1", 2), ("2", 1)])
 def test_prefill_reference_vectors(golden_dir, case, n_kv):
     """prefill_output_{1,2} of the reference's flash-attention unit test, from the packed rows and through the cache."""
