@@ -42,6 +42,7 @@ TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # the decode attention kernels and their launch rule (the prefill side lives in prefill_attention.hip)
 ATTENTION_SOURCES = [os.path.join(ROOT, "mindformers_amd", "csrc", n)
                      for n in ("paged_attention_kernels.h", "paged_attention.hip")]
+GEMM_SOURCES = [os.path.join(ROOT, "mindformers_amd", "csrc", "w8a16_gemm.hip")]
 
 
 def log(*a):
@@ -147,6 +148,22 @@ def measured_traffic(workload, kv_bytes):
     return int(rec["traffic_bytes"]), "profiles/hbm_traffic.json, commit %s" % rec.get("commit")
 
 
+def measured_gemm_chain(workload, weight_bytes):
+    """HBM bytes per layer step of the four weight-only GEMMs and the three kernels that carry their split-K sums
+    (from the same counter record), against the int8 weight bytes they must read.  Valid for the workload and the GEMM
+    source it was taken on: otherwise None."""
+    try:
+        with open(TRAFFIC_RECORD) as f:
+            rec = json.load(f)["gemm_chain"]
+    except (OSError, KeyError, ValueError):
+        return None
+    if rec.get("workload") != workload or rec.get("kernel_source_sha256") != source_sha256(GEMM_SOURCES):
+        return None
+    return {"traffic": int(rec["traffic_bytes"]), "algorithmic": int(weight_bytes),
+            "ratio": round(rec["traffic_bytes"] / weight_bytes, 3), "kernels": rec.get("kernels"),
+            "source": "profiles/hbm_traffic.json, commit %s" % rec.get("commit")}
+
+
 def record_traffic(fetch_csv, write_csv, workload, kv_bytes):
     """Write profiles/hbm_traffic.json from the counter_collection CSVs of two profiler runs of this benchmark with
     --calibrate-counters (one with --pmc FETCH_SIZE, one with --pmc WRITE_SIZE): mean counter value per dispatch of
@@ -173,16 +190,43 @@ def record_traffic(fetch_csv, write_csv, workload, kv_bytes):
     w_scale = 131072.0 / pick(write, "add_kernel")
     kib = (pick(fetch, "paged_attention_kernel") + pick(fetch, "paged_attention_reduce_kernel")) * f_scale + \
           (pick(write, "paged_attention_kernel") + pick(write, "paged_attention_reduce_kernel")) * w_scale
+
+    # the GEMM chain of a layer step: every dispatch of its kernels in a --layer-only run, per layer step (one
+    # w8a16_reduce_rope_cache_kernel dispatch each)
+    def totals(path, counter):
+        acc, steps = {}, 0
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") != counter:
+                    continue
+                name = row["Kernel_Name"]
+                for key in ("w8a16_gemm4_kernel", "w8a16_reduce_add_rmsnorm_kernel", "w8a16_reduce_rope_cache_kernel"):
+                    if key in name:
+                        acc[key] = acc.get(key, 0.0) + float(row["Counter_Value"])
+                        steps += key == "w8a16_reduce_rope_cache_kernel"
+        return acc, steps
+    cf, nf = totals(fetch_csv, "FETCH_SIZE")
+    cw, nw = totals(write_csv, "WRITE_SIZE")
+    chain = None
+    if nf and nw and cf.get("w8a16_gemm4_kernel"):
+        per_kernel = {k: int((cf.get(k, 0.0) / nf * f_scale + cw.get(k, 0.0) / nw * w_scale) * 1024) for k in cf}
+        chain = {"workload": workload, "traffic_bytes": int(sum(per_kernel.values())), "kernels": per_kernel,
+                 "layer_steps": nf, "kernel_source": "mindformers_amd/csrc/w8a16_gemm.hip",
+                 "kernel_source_sha256": source_sha256(GEMM_SOURCES)}
     commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
     rec = {"paged_attention": {"workload": workload, "kv_bytes": int(kv_bytes), "traffic_bytes": int(kib * 1024),
                                "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4),
                                "commit": commit or "unknown",
                                "kernel_source": "mindformers_amd/csrc/paged_attention_kernels.h + paged_attention.hip",
                                "kernel_source_sha256": source_sha256(ATTENTION_SOURCES)}}
+    if chain is not None:
+        chain["commit"] = commit or "unknown"
+        rec["gemm_chain"] = chain
     with open(TRAFFIC_RECORD, "w") as f:
         json.dump(rec, f, indent=1)
         f.write("\n")
-    log(f"[bench] wrote {TRAFFIC_RECORD}: {rec['paged_attention']['traffic_bytes']} bytes per launch")
+    log(f"[bench] wrote {TRAFFIC_RECORD}: {rec['paged_attention']['traffic_bytes']} bytes per attention launch" +
+        (f", {chain['traffic_bytes']} bytes per layer step for the GEMM chain" if chain else ""))
 
 
 def cpu_baseline(case, torch, sample_seqs, gpu_out, min_seconds=10.0):
@@ -781,6 +825,9 @@ def main():
                          "--calibrate-counters (--pmc FETCH_SIZE, --pmc WRITE_SIZE) into profiles/hbm_traffic.json")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-iters", type=int, default=50)
+    ap.add_argument("--layer-only", action="store_true",
+                    help="run the warm-up and the timed layer steps and nothing else (no per-op loops, no other legs): "
+                         "under a counter-collecting profiler every dispatch then belongs to a layer step")
     ap.add_argument("--calibrate-counters", action="store_true",
                     help="also launch add_kernel on 2 x 128 MiB inputs (reads 256 MiB, writes 128 MiB): the known-size "
                          "kernel that hardware traffic counters of a profiler run are scaled by")
@@ -887,6 +934,11 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     n_layers = cfg["layers"]
     tokens_per_s_layer = cfg["batch"] * n_layers * args.steps / elapsed
+    if args.layer_only:
+        print(json.dumps({"metric": METRICS.get(args.workload, METRICS["llama3_8b_w8a16"]),
+                          "value": round(tokens_per_s_layer, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "layer_only": True}), flush=True)
+        return
 
     # dominant kernel: paged attention, event-timed on the launch stream
     layer = case["layers"][0]
@@ -941,6 +993,9 @@ def main():
         "unfused_op_us": breakdown,
     }
     result.update(extra)
+    chain = None if cfg["act_quant"] else measured_gemm_chain(args.workload, nbytes["weights"])
+    if chain is not None:
+        result["gemm_chain"] = chain
     if cfg.get("kv_int8"):
         result["config"]["kv_cache"] = "int8, per-channel scales"
     if not args.no_cpu and not cfg.get("kv_int8"):            # the CPU restatement of the layer covers 16-bit caches
