@@ -50,11 +50,15 @@ def log(*a):
 
 
 def run_step(case, repeats=1):
-    """``repeats`` decode steps through every layer of the case (1 layer except the 8-layer long-context config),
-    each step taking the hidden state the step before it produced, as the layers of a model do."""
+    """``repeats`` decode steps of the config's layer stack (1 layer except the 8-layer long-context config), each
+    layer taking the hidden state the one before it produced, as the layers of a model do.  The case may hold
+    several separately allocated copies of the stack: consecutive steps then walk through them in turn, so that no
+    step finds its weights or its KV blocks in a cache because the step before it has just read them."""
     h, normed = case["x"], case.get("normed")
     layers = case["layers"]
-    for i, (layer, (kc, vc)) in ((i, lc) for _ in range(repeats) for i, lc in enumerate(zip(layers, case["caches"]))):
+    for j in range(repeats * case["cfg"]["layers"]):
+        i = j % len(layers)
+        layer, (kc, vc) = layers[i], case["caches"][i]
         # As in a stack of layers, every layer computes the attention norm of the layer after it (here: of the same
         # shape, the stack's first layer again after the last; W8A8: with its quantisation) in the kernel that
         # finishes its last projection, and takes its own normed input from the layer before it.  One step = every
@@ -366,39 +370,45 @@ def bench_modules(case, torch, ops, args):
     if layer.act_quant or cfg.get("kv_int8"):
         return {"skipped": "the module leg covers the W8A16 layer with 16-bit caches"}
     dt, dev = cfg["dtype"], case["x"].device
-    kc, vc = case["caches"][0]
-    cells = {}
-    for name in layer.NAMES:
-        w = getattr(layer, name + "_w")
-        cell = WeightQuantLinearCell(w.shape[1], w.shape[0], False, dt, device="meta")
-        cell.weight, cell.w_scale = w.to(dev), getattr(layer, name + "_s")
-        cell.prepare()
-        cell.weight = w                                         # the packed copy is what the kernels read
-        cells[name] = cell
-    norm1, norm2 = LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev), LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev)
-    norm1.weight.data, norm2.weight.data = layer.attn_norm, layer.ffn_norm
-    att = InferAttention(cfg["n_head"], cfg["head_dim"], cfg["n_kv_head"], scale_value=layer.scale_value,
-                         block_size=cfg["block_size"], num_blocks=1, rotary_cos_format=2, compute_dtype=dt, device=dev)
-    att.paged_attention_mgr.key_cache, att.paged_attention_mgr.value_cache = kc, vc     # the case's caches, not a copy
-    att.is_first_iteration = False
     nq, nkv = cfg["n_head"] * cfg["head_dim"], cfg["n_kv_head"] * cfg["head_dim"]
     freqs = (case["cos"], case["sin"], None)
 
-    def step(x):
-        qkv = cells["qkv"](norm1(x))
-        a = att(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], case["context_lens"], case["block_tables"],
-                case["slot_mapping"], freqs)
-        h = cells["wo"](a, residual=x)
-        return cells["fc2"](ops.silu_mul(cells["fc1"](norm2(h))), residual=h)
+    def compose(layer, kc, vc):
+        """The reference's cells around one layer's weights and caches; returns its step function."""
+        cells = {}
+        for name in layer.NAMES:
+            w = getattr(layer, name + "_w")
+            cell = WeightQuantLinearCell(w.shape[1], w.shape[0], False, dt, device="meta")
+            cell.weight, cell.w_scale = w.to(dev), getattr(layer, name + "_s")
+            cell.prepare()
+            cell.weight = w                                         # the packed copy is what the kernels read
+            cells[name] = cell
+        norm1, norm2 = LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev), LlamaRMSNorm(cfg["hidden"], layer.eps, device=dev)
+        norm1.weight.data, norm2.weight.data = layer.attn_norm, layer.ffn_norm
+        att = InferAttention(cfg["n_head"], cfg["head_dim"], cfg["n_kv_head"], scale_value=layer.scale_value,
+                             block_size=cfg["block_size"], num_blocks=1, rotary_cos_format=2, compute_dtype=dt, device=dev)
+        att.paged_attention_mgr.key_cache, att.paged_attention_mgr.value_cache = kc, vc     # the case's caches, not a copy
+        att.is_first_iteration = False
+
+        def step(x):
+            qkv = cells["qkv"](norm1(x))
+            a = att(qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], case["context_lens"], case["block_tables"],
+                    case["slot_mapping"], freqs)
+            h = cells["wo"](a, residual=x)
+            return cells["fc2"](ops.silu_mul(cells["fc1"](norm2(h))), residual=h)
+        return step
+    # one composition per separately allocated copy of the layer, walked through in turn like the fused leg
+    steps = [compose(l, kc, vc) for l, (kc, vc) in zip(case["layers"], case["caches"])]
+    kc, vc = case["caches"][0]
     ref = layer(case["x"], kc, vc, case["block_tables"], case["context_lens"], case["slot_mapping"], case["cos"], case["sin"])
-    out = step(case["x"])
+    out = steps[0](case["x"])
     same = bool(torch.equal(out, ref))
     per = next(g for g in (8, 4, 2, 1) if args.steps % g == 0)
 
     def chain():
         h = case["x"]
-        for _ in range(per):
-            h = step(h)
+        for j in range(per):
+            h = steps[j % len(steps)](h)
         return h
     launch = "eager"
     fn = chain
@@ -825,6 +835,9 @@ def main():
                          "--calibrate-counters (--pmc FETCH_SIZE, --pmc WRITE_SIZE) into profiles/hbm_traffic.json")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-iters", type=int, default=50)
+    ap.add_argument("--copies", type=int, default=8,
+                    help="separately allocated copies of the layer (weights and KV caches) the chained steps walk "
+                         "through; 1 = every step re-reads the same weights, which the memory-side cache may then hold")
     ap.add_argument("--layer-only", action="store_true",
                     help="run the warm-up and the timed layer steps and nothing else (no per-op loops, no other legs): "
                          "under a counter-collecting profiler every dispatch then belongs to a layer step")
@@ -868,7 +881,9 @@ def main():
         return
 
     t0 = time.perf_counter()
-    case = synthetic.make_decode_case(args.workload, seed=1)
+    stack = synthetic.CONFIGS[args.workload]["layers"]
+    copies = max(1, min(args.copies, 8 // stack))
+    case = synthetic.make_decode_case(args.workload, seed=1, copies=copies)
     cfg = case["cfg"]
     nbytes = synthetic.algorithmic_bytes(case)
     torch.cuda.synchronize()
@@ -984,7 +999,8 @@ def main():
                                f"ctx U[{cfg['ctx'][0]},{cfg['ctx'][1]}], block {cfg['block_size']}, "
                                f"{'W8A8' if cfg['act_quant'] else 'W8A16'}, layers {n_layers}",
                    "launch": (f"hip_graph, {per_replay} chained layer steps per replay" if graph is not None
-                              else "eager"),
+                              else "eager") + (f", over {copies} separately allocated copies of the layer"
+                                               if copies > 1 else ", every step on the same weights and caches"),
                    "algorithmic_bytes_per_layer": nbytes["total"]},
         "layer_hbm_gbps": round(layer_gbps, 1), "layer_hbm_frac": round(layer_gbps / HBM_PEAK_GBPS, 4),
         "roofline": roofline,

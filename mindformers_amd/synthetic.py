@@ -72,8 +72,10 @@ def context_lens(name, seed=0, batch=None, ctx=None):
     return np.random.default_rng(seed).integers(lo, hi + 1, batch if batch is not None else cfg["batch"]).astype(np.int32)
 
 
-def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=None):
-    """Build the layer(s) and one decode step's inputs for a named config.  Returns a dict."""
+def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=None, copies=1):
+    """Build the layer(s) and one decode step's inputs for a named config.  Returns a dict.  ``copies`` > 1 builds
+    that many separately allocated instances of the config's layer stack (own weights, own KV caches, same block
+    table and lengths), so that steps chained one after another read no byte an earlier step has left in a cache."""
     cfg = dict(CONFIGS[name])
     if batch is not None:
         cfg["batch"] = batch
@@ -101,7 +103,7 @@ def make_decode_case(name, seed=0, device="cuda", batch=None, ctx=None, layers=N
     layers_ = []
     caches = []
     kv_shape = (num_blocks, bs, cfg["n_kv_head"], cfg["head_dim"])
-    for _ in range(cfg["layers"]):
+    for _ in range(cfg["layers"] * copies):
         layer = QuantDecodeLayer(cfg["hidden"], cfg["n_head"], cfg["n_kv_head"], cfg["head_dim"], cfg["ffn"], 1e-5, dt,
                                  cfg["act_quant"], device=device)
         layers_.append(fill_layer(layer, gen))
