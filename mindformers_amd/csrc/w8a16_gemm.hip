@@ -36,6 +36,13 @@ constexpr int GW_TILE_BYTES = 16 * GW_KSTEP;
 static_assert(GW_KSTEP == MF_PACK_KSTEP && GW_TILE_BYTES == MF_PACK_TILE_BYTES, "the packed format is shared with the int8 GEMMs");
 constexpr int GW_DEPTH = 2;                 // weight k-steps in flight per wave beyond the current one
 
+// A weight byte is read once per launch.  The non-temporal hint lets the caches drop it first, which keeps the
+// activations, the partial sums and what the kernels around this one have left there.  Measured, it pays where many
+// expert matrices or a few activation rows are read (the grouped kernel, the 4-wave dense kernel: 2.5 - 3.5 % of the
+// layer step) and costs 1 % on the 8-wave dense kernel at 64 rows, which therefore keeps ordinary loads.
+template <typename V>
+__device__ __forceinline__ V gw_stream_load(const uint8_t* p) { return __builtin_nontemporal_load((const V*)p); }
+
 // acc * scale (+ bias) with separately rounded operations: every epilogue below goes through here, so that the
 // fused and the unfused paths give bit-identical values whatever the compiler would contract elsewhere.
 template <typename T>
@@ -145,7 +152,7 @@ __device__ __forceinline__ void w8a16_tile(uint16_t* __restrict__ y, float* __re
     auto load_w = [&](int slot, int s) {
         const int64_t off = (int64_t)min(s, s_last) * n_tiles_total * GW_TILE_BYTES;
 #pragma unroll
-        for (int nt = 0; nt < GW_NT; ++nt) wreg[slot][nt] = *(const u32x4*)(wbase[nt] + off);
+        for (int nt = 0; nt < GW_NT; ++nt) wreg[slot][nt] = gw_stream_load<u32x4>(wbase[nt] + off);
     };
     auto load_x = [&](int s) {
         const int kb = min(s, s_last) * GW_KSTEP;
@@ -248,20 +255,6 @@ struct GwSmem {
     // activation staging (4 waves x [16*MT, 64] bf16) and the cross-wave reduction ([4][16*MT][64] fp32) alias
     static constexpr int BYTES = GW_WAVES * 16 * MT * GW_BN * 4;
 };
-
-// Dense: grid = (ceil(N/64), split_k, ceil(M/(16*MT))).
-template <typename T, int MT, bool KTAIL>
-__global__ __launch_bounds__(GW_WAVES * 64, 2) void w8a16_gemm_kernel(
-    uint16_t* __restrict__ y, float* __restrict__ partial, const uint16_t* __restrict__ x,
-    const uint8_t* __restrict__ wp, const float* __restrict__ scale, const uint16_t* __restrict__ bias,
-    const uint16_t* __restrict__ residual, int M, int N, int K, int steps_per_split) {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[GwSmem<MT>::BYTES];
-    const int KS = (K + GW_KSTEP - 1) / GW_KSTEP;
-    const int s_begin = blockIdx.y * steps_per_split;
-    const int s_end = min(KS, s_begin + steps_per_split);
-    w8a16_tile<T, MT, KTAIL>(y, partial, x, wp, scale, bias, residual, M, N, K, KS, blockIdx.x * GW_BN,
-                      blockIdx.z * (16 * MT), s_begin, s_end, blockIdx.y, smem);
-}
 
 // ---- dense kernel: helpers ---------------------------------------------------------------------------
 constexpr int G2_WAVES = 4;
@@ -393,7 +386,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 3 : 1) void w8a16_gemm4_ke
     auto issue = [&](auto setc, int s) {
         constexpr int S = decltype(setc)::value;
         const int sc = min(s, s_last);
-        wreg[S] = *(const wreg_t*)(wtile + sc * wstride + wlane);
+        if constexpr (WAVES == 4) wreg[S] = gw_stream_load<wreg_t>(wtile + sc * wstride + wlane);
+        else wreg[S] = *(const wreg_t*)(wtile + sc * wstride + wlane);
         if constexpr (GROUP != 0) greg[S] = *(const f32x4*)(gsl + (int64_t)(sc * GW_KSTEP / GROUP) * N);
 #pragma unroll
         for (int i = 0; i < C::XL; ++i) {
