@@ -651,7 +651,8 @@ def bench_prefill_attention(args, torch, ops):
 def bench_mla_decode(args, torch, ops):
     """DeepSeek-V3-shaped multi-latent attention decode: 128 heads over one latent cache row per token (512 latent
     + 64 rotary, bf16), batch 64, context lengths uniform in [512, 4096], block 128.  A step is one attention call;
-    flops = 2 * (576 + 512) per (token, head)."""
+    consecutive calls walk through 4 separately allocated caches (170 MB each), as the layers of a model do, so that
+    no call finds its rows in the memory-side cache.  flops = 2 * (576 + 512) per (token, head)."""
     nh, dk, dv, bs, b, dt = 128, 576, 512, 128, 64, torch.bfloat16
     rng = np.random.default_rng(1)
     lens = rng.integers(512, 4097, b).astype(np.int32)
@@ -664,13 +665,16 @@ def bench_mla_decode(args, torch, ops):
         pos += n
     gen = torch.Generator(device="cuda")
     gen.manual_seed(4)
-    cache = torch.randn(nb, bs, 1, dk, generator=gen, device="cuda").to(dt)
+    caches = [torch.randn(nb, bs, 1, dk, generator=gen, device="cuda").to(dt) for _ in range(4)]
     q = torch.randn(b, nh * dk, generator=gen, device="cuda").to(dt)
     tb, lt = torch.from_numpy(tables).cuda(), torch.from_numpy(lens).cuda()
     out = torch.empty(b, nh * dv, dtype=dt, device="cuda")
 
+    turn = [0]
+
     def step():
-        return ops.mla_paged_attention(q, cache, tb, lt, nh, dv, 192 ** -0.5, out=out)
+        turn[0] = (turn[0] + 1) % len(caches)
+        return ops.mla_paged_attention(q, caches[turn[0]], tb, lt, nh, dv, 192 ** -0.5, out=out)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -690,7 +694,7 @@ def bench_mla_decode(args, torch, ops):
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"deepseek_v3_mla_decode: multi-latent attention decode, batch {b}, {nh} heads, latent "
-                               f"512 + rope 64, ctx U[512,4096] (sum {tokens}), block {bs}",
+                               f"512 + rope 64, ctx U[512,4096] (sum {tokens}), block {bs}, 4 caches in turn",
                    "launch": "eager", "flops_per_step": flops, "cache_bytes_per_step": kv_bytes},
         "hbm_gbps_on_cache_bytes": round(kv_bytes / (us * 1e-6) / 1e9, 1),
         "roofline": dict(bound="mfma", kernel="mla_decode_kernel (+ mla_reduce_kernel)", achieved=round(ach, 1),
@@ -779,11 +783,16 @@ def bench_mla_layer(args, torch, ops):
     attn = torch.randn(b, nh, rank, generator=gen, device="cuda").to(dt)
     core = torch.randn(b, nh * vd, generator=gen, device="cuda").to(dt)
     qa_t, out_absorb = net._absorb
+    turn = [0]
+
+    def next_cache():                                         # the layers' caches in turn: every call reads cold rows
+        turn[0] = (turn[0] + 1) % n_layers
+        return caches[turn[0]]
     pieces = {
         "qkv_down_proj": lambda: net.linear_qkv_down_proj(x),
         "q_up_proj": lambda: net.linear_q_up_proj(q_c),
         "absorb_query_bmm": lambda: ops.mla_absorb_bmm(qq[..., :nope], qa_t, out=query[..., :rank]),
-        "mla_paged_attention": lambda: ops.mla_paged_attention(query.reshape(b, -1), caches[0], tb, lt, nh, rank,
+        "mla_paged_attention": lambda: ops.mla_paged_attention(query.reshape(b, -1), next_cache(), tb, lt, nh, rank,
                                                                net.softmax_scale),
         "absorb_output_bmm": lambda: ops.mla_absorb_bmm(attn, out_absorb),
         "linear_proj": lambda: net.linear_proj(core),
