@@ -12,8 +12,19 @@ static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 
 // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
 // first tile, merge) exposed: twice the tokens per workgroup at every context length (fewer partitions than the
 // workspace query, which does not know the cache type, sizes for).
-static inline int pa_launch_tiles_per_wave(int64_t max_context, int kvq) {
-    return kvq ? 4 : pa_tiles_per_wave(max_context);
+// 16-bit caches: larger partitions (fewer fp32 partials to write and combine) where the batch still fills the
+// device several times over with them.  The lengths are on the device, so the count is taken on the context
+// capacity: 512 tokens from 3072 workgroups up (0.7 % off the layer step of the 64-sequence ragged batch), 1024
+// tokens from 2048 up if the sequences alone - one workgroup each per kv head - fill the 768 workgroup slots, so that
+// a ragged batch cannot leave the last round short (256 sequences of 2048 tokens, 4 kv heads: attention 212.7 ->
+// 185.2 us; the ragged 64-sequence batch gains nothing from 1024 and stays at 512).
+static inline int pa_launch_tiles_per_wave(int64_t max_context, int kvq, int64_t batch_kv_groups) {
+    if (kvq) return 4;
+    auto workgroups = [&](int tpw) {
+        return batch_kv_groups * ((max_context + tpw * PA_WAVE_TOKENS - 1) / (tpw * PA_WAVE_TOKENS));
+    };
+    if (batch_kv_groups >= 768 && workgroups(8) >= 2048) return 8;
+    return workgroups(4) >= 3072 ? 4 : pa_tiles_per_wave(max_context);
 }
 
 // Per-token quantisation of the output rows requested together with the attention itself.
@@ -32,7 +43,7 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     const int n_rep = n_heads / n_kv;
     const int head_groups = (n_rep + 15) / 16;
     const int64_t max_ctx = (int64_t)max_blocks * block_size;
-    const int tpw = pa_launch_tiles_per_wave(max_ctx, KVQ);
+    const int tpw = pa_launch_tiles_per_wave(max_ctx, KVQ, (int64_t)batch * n_kv * head_groups);
     const int part_tokens = tpw * PA_WAVE_TOKENS;
     const int max_parts = (int)((max_ctx + part_tokens - 1) / part_tokens);
     float* part_out = (float*)workspace;
@@ -46,7 +57,12 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
                        (const int32_t*)nullptr, 0, (int64_t)0, 0, kv_scale, kv_offset)
-    if (tpw == 2) {
+    if (tpw == 8) {
+        if constexpr (KVQ == 0) {                             // only 16-bit caches take 1024-token partitions
+            if (tib) PA_LAUNCH(8, true);
+            else PA_LAUNCH(8, false);
+        }
+    } else if (tpw == 2) {
         if (tib) PA_LAUNCH(2, true);
         else PA_LAUNCH(2, false);
     } else {
@@ -126,7 +142,9 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
     hipStream_t st = (hipStream_t)stream;
     // with one partition the attention kernel writes the output rows itself and skips sequences without context
     const int64_t launch_part_tokens =
-        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kvq) * PA_WAVE_TOKENS;
+        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kvq,
+                                          (int64_t)batch * n_kv_heads * ((n_heads / n_kv_heads + 15) / 16)) *
+        PA_WAVE_TOKENS;
     if ((int64_t)max_blocks_per_seq * block_size <= launch_part_tokens) {
         hipLaunchKernelGGL(pa_zero_empty_kernel, dim3(batch), dim3(128), 0, st, (uint16_t*)out, context_lens,
                            n_heads * head_dim);
