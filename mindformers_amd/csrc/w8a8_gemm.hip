@@ -751,13 +751,16 @@ __global__ __launch_bounds__(QRC_THREADS) void w8a8_reduce_rope_cache_kernel(
 // rows.  Decode batches route a handful of tokens to each expert, so the kernel is a weight stream: the waves
 // interleave the 64-wide k-steps, each loads its four 1 KiB weight tiles of a step straight into operand registers
 // (two steps ahead) and the 16 bytes per lane of each 16-row activation tile from the row-major int8 rows (a few KiB
-// per expert, served by L2), and the four waves' exact int32 sums meet in LDS at the end.  Up to 32 rows go through
-// one pass over the weights; experts with more rows repeat the pass per 32 rows.
+// per expert, served by L2), and the four waves' exact int32 sums meet in LDS at the end.  Up to 64 rows go through
+// one pass over the weights (16 / 32 / 64 by the expert's row count, as in the W8A16 grouped kernel); experts with
+// more rows repeat the pass.  Two builds of the kernel: passes of up to 32 rows (138 registers, three workgroups per
+// compute unit: the decode-sized case, a pure weight stream) and of up to 64 rows (197 registers, two per compute unit),
+// which the launch picks when the groups average more than 16 rows.
 constexpr int QG_WAVES = 4;
 constexpr int QG_NT = 4;                                      // 16-channel weight tiles per wave and step
 constexpr int QG_BN = 16 * QG_NT;
-constexpr int QG_MT_MAX = 2;                                  // 16-row activation tiles per pass
-constexpr int QG_SMEM = QG_WAVES * 16 * QG_MT_MAX * QG_BN * 4;
+template <int MTMAX>
+constexpr int QG_SMEM = QG_WAVES * 16 * MTMAX * QG_BN * 4;    // MTMAX 16-row activation tiles per pass
 
 template <typename T, int MT>
 __device__ __forceinline__ void w8a8_group_pass(uint16_t* __restrict__ y, int32_t* __restrict__ acc_out,
@@ -836,12 +839,12 @@ __device__ __forceinline__ void w8a8_group_pass(uint16_t* __restrict__ y, int32_
     }
 }
 
-template <typename T>
+template <typename T, int MTMAX>
 __global__ __launch_bounds__(QG_WAVES * 64, 2) void w8a8_grouped_kernel(
     uint16_t* __restrict__ y, int32_t* __restrict__ acc_out, const int8_t* __restrict__ xq,
     const float* __restrict__ x_scale, const uint8_t* __restrict__ wp, const float* __restrict__ w_scale,
     const int32_t* __restrict__ offsets, int total_rows, int N, int K, int64_t expert_bytes) {
-    __shared__ __attribute__((aligned(16))) int32_t red[QG_SMEM / 4];
+    __shared__ __attribute__((aligned(16))) int32_t red[QG_SMEM<MTMAX> / 4];
     const int e = blockIdx.y;
     int row0 = offsets[e], row1 = offsets[e + 1];
     row0 = max(0, min(row0, total_rows));
@@ -857,9 +860,12 @@ __global__ __launch_bounds__(QG_WAVES * 64, 2) void w8a8_grouped_kernel(
     const int n0 = blockIdx.x * QG_BN;
     if (rows <= 16) {
         w8a8_group_pass<T, 1>(ye, ae, xe, xse, we, se, rows, N, K, n0, 0, red);
+    } else if (rows <= 32 || MTMAX == 2) {
+        for (int m0 = 0; m0 < rows; m0 += 32)
+            w8a8_group_pass<T, 2>(ye, ae, xe, xse, we, se, rows, N, K, n0, m0, red);
     } else {
-        for (int m0 = 0; m0 < rows; m0 += 16 * QG_MT_MAX)
-            w8a8_group_pass<T, QG_MT_MAX>(ye, ae, xe, xse, we, se, rows, N, K, n0, m0, red);
+        for (int m0 = 0; m0 < rows; m0 += 16 * MTMAX)
+            w8a8_group_pass<T, MTMAX>(ye, ae, xe, xse, we, se, rows, N, K, n0, m0, red);
     }
 }
 
@@ -1127,13 +1133,19 @@ extern "C" int mf_grouped_w8a8_gemm(void* y, int32_t* acc_out, const int8_t* xq,
                "grouped_w8a8_gemm: xq and w_packed must be 16-byte aligned");
     const int64_t expert_bytes = (int64_t)mf_w8a16_packed_bytes(n, k);
     dim3 grid((n + QG_BN - 1) / QG_BN, n_experts);
-    if (out_dtype == MF_BF16)
-        hipLaunchKernelGGL(w8a8_grouped_kernel<BF16>, grid, dim3(QG_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
-                           acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, offsets, total_rows, n, k,
-                           expert_bytes);
-    else
-        hipLaunchKernelGGL(w8a8_grouped_kernel<FP16>, grid, dim3(QG_WAVES * 64), 0, (hipStream_t)stream, (uint16_t*)y,
-                           acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, offsets, total_rows, n, k,
-                           expert_bytes);
+    // groups that average more than 16 rows (prefill-sized) take the 64-row passes; both builds serve any row count
+    const bool big = (int64_t)total_rows > 16 * (int64_t)n_experts;
+#define QG_LAUNCH(TT, MTV)                                                                                      \
+    hipLaunchKernelGGL((w8a8_grouped_kernel<TT, MTV>), grid, dim3(QG_WAVES * 64), 0, (hipStream_t)stream,        \
+                       (uint16_t*)y, acc_out, xq, x_scale, (const uint8_t*)w_packed, w_scale, offsets, total_rows, n, \
+                       k, expert_bytes)
+    if (out_dtype == MF_BF16) {
+        if (big) QG_LAUNCH(BF16, 4);
+        else QG_LAUNCH(BF16, 2);
+    } else {
+        if (big) QG_LAUNCH(FP16, 4);
+        else QG_LAUNCH(FP16, 2);
+    }
+#undef QG_LAUNCH
     return MF_LAUNCH_CHECK();
 }

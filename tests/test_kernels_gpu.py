@@ -1484,11 +1484,12 @@ def test_grouped_w8a16_many_rows_and_gated_epilogue(dtype):
     assert fused.shape == (rows, f) and torch.equal(fused, ops.silu_mul(y))
 
 
-@pytest.mark.parametrize("counts,n,k", [([0, 5, 16, 20, 40, 1, 0, 3], 192, 208), ([4] * 16, 128, 1024), ([33], 80, 64)])
+@pytest.mark.parametrize("counts,n,k", [([0, 5, 16, 20, 40, 1, 0, 3], 192, 208), ([4] * 16, 128, 1024), ([33], 80, 64),
+                                        ([64, 65, 150, 32, 0, 129, 7], 144, 320)])
 def test_grouped_w8a8_accumulators_bit_exact(counts, n, k):
     """The grouped int8 GEMM: exact int32 accumulators per expert (against the integer matmul), dequantised outputs
-    within a rounding of acc * row scale * channel scale; ragged groups, empty experts, more than 32 rows (a repeated
-    pass), K not a multiple of 64, N not a multiple of 64."""
+    within a rounding of acc * row scale * channel scale; ragged groups, empty experts, every pass size (16, 32 and
+    64 rows), more than 64 rows (a repeated pass, whole and ragged), K not a multiple of 64, N not a multiple of 64."""
     rng = np.random.default_rng(n + k)
     counts, off = _ragged_groups(rng, counts)
     e, rows = len(counts), int(counts.sum())
