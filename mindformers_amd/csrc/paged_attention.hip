@@ -12,19 +12,24 @@ static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 
 // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
 // first tile, merge) exposed: twice the tokens per workgroup at every context length (fewer partitions than the
 // workspace query, which does not know the cache type, sizes for).
-// 16-bit caches: larger partitions (fewer fp32 partials to write and combine) where the batch still fills the
-// device several times over with them.  The lengths are on the device, so the count is taken on the context
-// capacity: 512 tokens from 3072 workgroups up (0.7 % off the layer step of the 64-sequence ragged batch), 1024
-// tokens from 2048 up if the sequences alone - one workgroup each per kv head - fill the 768 workgroup slots, so that
-// a ragged batch cannot leave the last round short (256 sequences of 2048 tokens, 4 kv heads: attention 212.7 ->
-// 185.2 us; the ragged 64-sequence batch gains nothing from 1024 and stays at 512), or if the capacity is above
-// 16384 tokens (16 sequences of 16-32 k tokens, 8 kv heads: 292.5 -> 282.3 us).
+// 16-bit caches: larger partitions (fewer fp32 partials to write and combine, fewer workgroups that find nothing to
+// do when the block table is wider than the contexts are long) where the batch still fills the device with them.
+// The lengths are on the device, so the count is taken on the context capacity:
+//   512 tokens from 3072 workgroups up (0.7 % off the layer step of the 64-sequence ragged batch, which gains nothing
+//   from more: 1024-token partitions leave it 1.8 rounds of workgroups);
+//   1024 / 2048 tokens where the sequences alone - one workgroup each per kv head - fill the 768 workgroup slots, so
+//   that a ragged batch cannot leave the last round short, or where the capacity is above 16384 tokens
+//   (256 sequences of 2048 tokens, 4 kv heads: attention 212.7 us with 256-token partitions, 198.8 with 1024, 186.5
+//   with 2048, which is one partition per sequence and no combine at all; 16 sequences of 16-32 k tokens, 8 kv heads:
+//   292.1 / 283.0 / 274.5 us with 512 / 1024 / 2048).
 static inline int pa_launch_tiles_per_wave(int64_t max_context, int kvq, int64_t batch_kv_groups) {
     if (kvq) return 4;
     auto workgroups = [&](int tpw) {
         return batch_kv_groups * ((max_context + tpw * PA_WAVE_TOKENS - 1) / (tpw * PA_WAVE_TOKENS));
     };
-    if ((batch_kv_groups >= 768 || max_context > 16384) && workgroups(8) >= 2048) return 8;
+    const bool full = batch_kv_groups >= 768, deep = max_context > 16384;
+    if ((full && workgroups(16) >= 1024) || (deep && workgroups(16) >= 2048)) return 16;
+    if ((full || deep) && workgroups(8) >= 2048) return 8;
     return workgroups(4) >= 3072 ? 4 : pa_tiles_per_wave(max_context);
 }
 
@@ -58,8 +63,13 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
                        (const uint16_t*)value_cache, block_tables, context_lens, n_heads, n_kv, n_rep, head_groups, \
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
                        (const int32_t*)nullptr, 0, (int64_t)0, 0, kv_scale, kv_offset)
-    if (tpw == 8) {
-        if constexpr (KVQ == 0) {                             // only 16-bit caches take 1024-token partitions
+    if (tpw == 16) {
+        if constexpr (KVQ == 0) {                             // only 16-bit caches take 1024- / 2048-token partitions
+            if (tib) PA_LAUNCH(16, true);
+            else PA_LAUNCH(16, false);
+        }
+    } else if (tpw == 8) {
+        if constexpr (KVQ == 0) {
             if (tib) PA_LAUNCH(8, true);
             else PA_LAUNCH(8, false);
         }

@@ -189,17 +189,19 @@ def test_paged_attention_long_contexts_vs_oracle(dtype, b, nh, nkv, d, bs, lens,
     assert_within(got, ref, mag, dtype, ulps=1.5, what="paged attention, long contexts")
 
 
-@pytest.mark.parametrize("b,nkv,max_blocks,part", [
-    (200, 2, 32, 512),      # 400 (sequence, kv head) pairs x 8 partitions of 512 tokens: 3200 workgroups
-    (400, 2, 24, 1024),     # 800 pairs fill the device by themselves: 1024-token partitions
+@pytest.mark.parametrize("b,nkv,max_blocks,part,hi", [
+    (200, 2, 32, 512, 4096),     # 400 (sequence, kv head) pairs x 8 partitions of 512 tokens: 3200 workgroups
+    (64, 2, 136, 1024, 3000),    # capacity 17408 tokens: 128 pairs x 17 partitions of 1024, too few of 2048
+    (400, 2, 24, 2048, 3072),    # 800 pairs fill the device by themselves: 2048-token partitions
+    (400, 2, 16, 2048, 2048),    # the same with one partition per sequence: no combine, rows written directly
 ])
-def test_paged_attention_large_batches_take_larger_partitions(b, nkv, max_blocks, part):
-    """Large batches of 16-bit caches run 512- or 1024-token partitions (chosen on the batch and the context
+def test_paged_attention_large_batches_take_larger_partitions(b, nkv, max_blocks, part, hi):
+    """Large batches of 16-bit caches run 512-, 1024- or 2048-token partitions (chosen on the batch and the context
     capacity); ragged lengths with empty sequences and lengths on and next to the partition borders."""
-    rng = np.random.default_rng(b + part)
+    rng = np.random.default_rng(b + part + max_blocks)
     cap = max_blocks * 128
-    lens = rng.integers(1, cap + 1, b)
-    lens[:8] = [0, 1, part - 1, part, part + 1, 2 * part, cap - 1, cap]
+    lens = rng.integers(1, hi + 1, b)
+    lens[:8] = [0, 1, part - 1, min(part, cap), min(part + 1, cap), min(2 * part, cap), cap - 1, cap]
     got, ref, mag = _pa_case(rng, torch.bfloat16, b, 2 * nkv, nkv, 32, 128, lens, max_blocks=max_blocks)
     assert not got[0].any()                                   # a sequence without context: zeros
     assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what=f"paged attention, {part}-token partitions")
