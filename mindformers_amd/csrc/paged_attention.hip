@@ -10,8 +10,8 @@ namespace {
 // the last round of workgroups short; very long contexts use 512 to halve the partial traffic.
 static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 16384 ? 4 : 2; }
 // int8 caches halve the bytes per tile, which leaves the fixed cost of a workgroup (work-list scan, query load,
-// first tile, merge) exposed: twice the tokens per workgroup at every context length (fewer partitions than the
-// workspace query, which does not know the cache type, sizes for).
+// first tile, merge) exposed: at least 512 tokens per workgroup at every context length (fewer partitions than the
+// workspace query, which does not know the cache type, sizes for), more by the rule below.
 // 16-bit caches: larger partitions (fewer fp32 partials to write and combine, fewer workgroups that find nothing to
 // do when the block table is wider than the contexts are long) where the batch still fills the device with them.
 // The lengths are on the device, so the count is taken on the context capacity:
@@ -23,14 +23,13 @@ static inline int pa_tiles_per_wave(int64_t max_context) { return max_context > 
 //   with 2048, which is one partition per sequence and no combine at all; 16 sequences of 16-32 k tokens, 8 kv heads:
 //   292.1 / 283.0 / 274.5 us with 512 / 1024 / 2048).
 static inline int pa_launch_tiles_per_wave(int64_t max_context, int kvq, int64_t batch_kv_groups) {
-    if (kvq) return 4;
     auto workgroups = [&](int tpw) {
         return batch_kv_groups * ((max_context + tpw * PA_WAVE_TOKENS - 1) / (tpw * PA_WAVE_TOKENS));
     };
     const bool full = batch_kv_groups >= 768, deep = max_context > 16384;
     if ((full && workgroups(16) >= 1024) || (deep && workgroups(16) >= 2048)) return 16;
     if ((full || deep) && workgroups(8) >= 2048) return 8;
-    return workgroups(4) >= 3072 ? 4 : pa_tiles_per_wave(max_context);
+    return (kvq || workgroups(4) >= 3072) ? 4 : pa_tiles_per_wave(max_context);
 }
 
 // Per-token quantisation of the output rows requested together with the attention itself.
@@ -64,15 +63,11 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
                        block_size, max_blocks, num_blocks, max_parts, scale_log2, q_stride, batch,                 \
                        (const int32_t*)nullptr, 0, (int64_t)0, 0, kv_scale, kv_offset)
     if (tpw == 16) {
-        if constexpr (KVQ == 0) {                             // only 16-bit caches take 1024- / 2048-token partitions
-            if (tib) PA_LAUNCH(16, true);
-            else PA_LAUNCH(16, false);
-        }
+        if (tib) PA_LAUNCH(16, true);
+        else PA_LAUNCH(16, false);
     } else if (tpw == 8) {
-        if constexpr (KVQ == 0) {
-            if (tib) PA_LAUNCH(8, true);
-            else PA_LAUNCH(8, false);
-        }
+        if (tib) PA_LAUNCH(8, true);
+        else PA_LAUNCH(8, false);
     } else if (tpw == 2) {
         if (tib) PA_LAUNCH(2, true);
         else PA_LAUNCH(2, false);

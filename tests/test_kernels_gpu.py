@@ -622,6 +622,7 @@ def test_quant_reshape_and_cache_bit_exact(dtype, with_offset):
     (torch.float16, 4, 8, 2, 64, 16, 10, 250, True),
     (torch.bfloat16, 2, 28, 4, 128, 128, 500, 600, False),    # n_rep = 7
     (torch.float16, 2, 4, 4, 32, 32, 1, 90, True),            # MHA, head_dim 32
+    (torch.bfloat16, 400, 4, 2, 32, 128, 1, 2100, True),      # 800 (sequence, kv head) pairs: 2048-token partitions
 ])
 def test_paged_attention_int8kv_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi, with_offset):
     """Attention over an int8 cache equals the oracle on the dequantised cache (the only extra rounding is the
@@ -731,7 +732,7 @@ def test_dynamic_quant_reshape_and_cache_bit_exact(dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("b,nh,nkv,d,bs,lo,hi", [(8, 32, 8, 128, 128, 1, 1500), (5, 8, 2, 64, 16, 1, 700),
                                                  (3, 4, 4, 32, 32, 30, 300), (64, 28, 4, 128, 128, 500, 600),
-                                                 (2, 16, 2, 128, 20, 1, 90)])
+                                                 (2, 16, 2, 128, 20, 1, 90), (400, 4, 2, 32, 128, 1, 2100)])
 def test_paged_attention_int8kv_per_token_vs_oracle(dtype, b, nh, nkv, d, bs, lo, hi):
     """Decode over int8 caches with one scale per cached token: against the oracle on the dequantised caches (block
     sizes that hold whole 32-token tiles and block sizes that do not; contexts that end inside a tile; NaN in the
