@@ -98,13 +98,6 @@ int launch_pa(void* out, const void* query, const void* key_cache, const void* v
     return rc;
 }
 
-// zero rows of sequences with no context when the single-partition path (which skips them) is used
-__global__ void pa_zero_empty_kernel(uint16_t* __restrict__ out, const int32_t* __restrict__ ctx_lens, int row) {
-    const int b = blockIdx.x;
-    if (ctx_lens[b] > 0) return;
-    for (int i = threadIdx.x; i < row; i += blockDim.x) out[(int64_t)b * row + i] = 0;
-}
-
 }  // namespace
 extern "C" size_t mf_paged_attention_workspace_bytes(int batch, int n_heads, int head_dim, int max_context) {
     const int part_tokens = pa_tiles_per_wave(max_context) * PA_WAVE_TOKENS;
@@ -146,17 +139,6 @@ static int pa_decode_entry(void* out, const void* query, const void* key_cache, 
                "paged_attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     MF_REQUIRE(need == 0 || ((uintptr_t)workspace & 15) == 0, "paged_attention: workspace must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    // with one partition the attention kernel writes the output rows itself and skips sequences without context
-    const int64_t launch_part_tokens =
-        (int64_t)pa_launch_tiles_per_wave((int64_t)max_blocks_per_seq * block_size, kvq,
-                                          (int64_t)batch * n_kv_heads * ((n_heads / n_kv_heads + 15) / 16)) *
-        PA_WAVE_TOKENS;
-    if ((int64_t)max_blocks_per_seq * block_size <= launch_part_tokens) {
-        hipLaunchKernelGGL(pa_zero_empty_kernel, dim3(batch), dim3(128), 0, st, (uint16_t*)out, context_lens,
-                           n_heads * head_dim);
-        int rc = MF_LAUNCH_CHECK();
-        if (rc) return rc;
-    }
     void* ws = need ? workspace : nullptr;
 #define PA_CASE_Q(TT, DD, QQ)                                                                                   \
     return launch_pa<TT, DD, QQ>(out, query, key_cache, value_cache, block_tables, context_lens, batch, n_heads,  \

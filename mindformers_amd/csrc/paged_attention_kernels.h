@@ -120,6 +120,7 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KVQ == 1 && TIB) ? 4 : 3) vo
     const int nkg = n_kv * head_groups;
     int b = -1, part = 0, L = 0, kg = 0;
     int q_len = 1, q_start = 0, col_groups = head_groups;     // PF: per sequence
+    int used = 0;                                             // work items that exist (known where none was found)
     {
         const int pidx = blockIdx.x;
         const int ln = threadIdx.x & 63;
@@ -162,9 +163,42 @@ __global__ __launch_bounds__(PA_WAVES * 64, (!PF && KVQ == 1 && TIB) ? 4 : 3) vo
             }
             base += total;
         }
+        used = base;
     }
     kg = __builtin_amdgcn_readfirstlane(kg);
-    if (b < 0) return;                                        // uniform over the workgroup
+    if (b < 0) {                                              // uniform over the workgroup
+        // Decode with one partition per sequence writes the output rows itself, and a sequence without context has no
+        // workgroup: the nkg workgroups it leaves over write its zeros (left-over workgroup u takes kv group
+        // u % nkg of the (u / nkg)-th empty sequence).
+        if constexpr (!PF) {
+            if (max_parts == 1) {
+                const int u = (int)blockIdx.x - used;
+                const int rank = u / nkg, kgz = u - rank * nkg;
+                const int ln = threadIdx.x & 63;
+                int seen = 0, target = -1;
+                for (int c0 = 0; c0 < batch; c0 += 64) {
+                    const int bb = c0 + ln;
+                    const bool empty = bb < batch && min(ctx_lens[bb], max_blocks * block_size) <= 0;
+                    const uint64_t m = __ballot(empty);
+                    const int cnt = __popcll(m);
+                    if (rank < seen + cnt) {
+                        const int before = __popcll(m & ((1ull << ln) - 1ull));
+                        const uint64_t hm = __ballot(empty && before == rank - seen);
+                        target = c0 + __ffsll((unsigned long long)hm) - 1;
+                        break;
+                    }
+                    seen += cnt;
+                }
+                if (target >= 0 && rank >= 0) {
+                    const int kvz = kgz / head_groups, hgz = kgz - kvz * head_groups;
+                    const int heads = min(16, n_rep - 16 * hgz);
+                    uint16_t* row = out + ((int64_t)target * n_heads + kvz * n_rep + 16 * hgz) * D;
+                    for (int i = threadIdx.x; i < heads * D; i += PA_WAVES * 64) row[i] = 0;
+                }
+            }
+        }
+        return;
+    }
     col_groups = __builtin_amdgcn_readfirstlane(col_groups);
     const int kvh = kg / col_groups;
     const int hg = kg - kvh * col_groups;                     // head group (decode) / column group (PF)

@@ -202,8 +202,10 @@ def test_paged_attention_large_batches_take_larger_partitions(b, nkv, max_blocks
     cap = max_blocks * 128
     lens = rng.integers(1, hi + 1, b)
     lens[:8] = [0, 1, part - 1, min(part, cap), min(part + 1, cap), min(2 * part, cap), cap - 1, cap]
+    empty = sorted({0, min(63, b - 2), min(64, b - 1), b - 1})   # no context, on both sides of a 64-wide scan chunk
+    lens[empty] = 0
     got, ref, mag = _pa_case(rng, torch.bfloat16, b, 2 * nkv, nkv, 32, 128, lens, max_blocks=max_blocks)
-    assert not got[0].any()                                   # a sequence without context: zeros
+    assert not got[empty].any()                               # a sequence without context: zeros
     assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what=f"paged attention, {part}-token partitions")
 
 
