@@ -4,11 +4,13 @@
 A "step" is one pass of one decode layer over one batch: the Llama-3.1-8B-shape W8A16 layer at batch 64
 (hidden 4096, 32 query / 8 KV heads, head_dim 128, FFN 14336, context lengths uniform in [512, 4096], bf16 KV
 cache in 128-token blocks behind a shuffled block table), synthetic seeded inputs already resident in HBM.
+The timed steps are chained in one HIP graph, each taking the hidden state of the one before, and walk through
+separately allocated copies of the layer (own weights, own KV caches; --copies), as the layers of a model do.
 Prints ONE JSON line: decode tokens/s per layer, the HBM roofline of the dominant kernel (paged attention,
 timed live with events on the launch stream) and the CPU restatement of the same path timed on the host
 cores on a bounded sample.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--no-cpu] [--copies C]
 
 Workloads: llama3_8b_w8a16 (default), llama3_8b_w8a16_kv8, tiny_llama_w8a16, qwen2_5_7b_w8a8, qwen2_5_72b_w8a16
 (layer steps); deepseek_v3_moe_w8a16 (one MoE layer step); deepseek_v3_mla_layer (one multi-latent attention layer step);
