@@ -303,6 +303,13 @@ int mf_mla_norm_rope_cache(void* q_rope_out, int64_t q_out_token_stride, int64_t
 int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* residual, const void* gamma, float eps,
                int rows, int cols, int dtype, int gamma_dtype, void* stream);
 
+/* The same norm over a column slice of a wider matrix: row i of x starts x_row_stride elements after row i - 1
+ * (>= cols, a multiple of 8); y is dense [rows, cols].  The latent norms of multi-latent attention read slices of the
+ * fused down projection: mindformers/parallel_core/inference/transformer/multi_latent_attention.py:367-374
+ * (q_layernorm on the first q_lora_rank columns, kv_layernorm on the next kv_lora_rank). */
+int mf_rmsnorm_strided(void* y, const void* x, int64_t x_row_stride, const void* gamma, float eps, int rows, int cols,
+                       int dtype, int gamma_dtype, void* stream);
+
 /* act(gate) * up with act = SiLU: mindformers/parallel_core/inference/transformer/mlp.py:135-140,
  * mindformers/models/llama/llama_layer.py:419-440.  gate_up is [rows, 2*cols]; layout 0 = contiguous halves
  * [gate | up] (mcore), 1 = interleaved columns g,u,g,u (legacy ffn_concat).  silu(gate) is rounded to dtype
@@ -365,6 +372,17 @@ int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* x, const vo
                               const void* bias, const void* residual, const void* gamma, float eps, int m, int n,
                               int k, int dtype, int gamma_dtype, void* workspace, size_t workspace_bytes,
                               void* stream);
+
+/* A projection whose leading columns feed an RMSNorm - the fused query / latent down projection of multi-latent
+ * attention followed by q_layernorm on its first q_lora_rank columns
+ * (mindformers/parallel_core/inference/transformer/multi_latent_attention.py:361-374): h_out [m, n] =
+ * round(x . w^T * scale + bias), y_norm [m, norm_cols] (dense) = RMSNorm(h_out[:, :norm_cols]) * gamma.  Bit-identical
+ * to mf_w8a16_gemm followed by mf_rmsnorm_strided on the slice; when K is split across workgroups the sum of the
+ * splits and the norm are one kernel.  N % 8 == 0, N <= 16384, norm_cols % 8 == 0, norm_cols <= N.  Workspace as for
+ * mf_w8a16_gemm. */
+int mf_w8a16_gemm_rmsnorm_leading(void* y_norm, void* h_out, const void* x, const void* w_packed, const float* scale,
+                                  const void* bias, const void* gamma, float eps, int m, int n, int k, int norm_cols,
+                                  int dtype, int gamma_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The fused QKV projection together with what follows it on the decode path: rotate-half RoPE on q and k and the
  * scatter of the rotated k and of v into the paged caches (mindformers/modules/infer_attention.py:441-463,

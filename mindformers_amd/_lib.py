@@ -48,6 +48,7 @@ SIGNATURES = {
     "mf_paged_attention_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _L, _L, _I,
                                         _P, _Z, _P]),
     "mf_rmsnorm": (_I, [_P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P]),
+    "mf_rmsnorm_strided": (_I, [_P, _P, _L, _P, _F, _I, _I, _I, _I, _P]),
     "mf_silu_mul": (_I, [_P, _P, _I, _I, _I, _I, _P]),
     "mf_add": (_I, [_P, _P, _P, _L, _I, _P]),
     "mf_scale_columns": (_I, [_P, _P, _P, _L, _I, _I, _P]),
@@ -60,6 +61,7 @@ SIGNATURES = {
     "mf_w4a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_gemm_add_rmsnorm": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P, _Z, _P]),
+    "mf_w8a16_gemm_rmsnorm_leading": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_qkv_rope_and_cache": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _L, _I, _I, _I, _P, _Z, _P]),
     "mf_w8a16_qkv_rope_and_quant_cache": (_I, [_P] * 12 + [_I] * 4 + [_L] + [_I] * 3 + [_P, _Z, _P]),
     "mf_w8a16_gemm_silu_mul": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P]),

@@ -30,7 +30,8 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(uint16_t* __restr
                                                              const uint16_t* __restrict__ x,
                                                              const uint16_t* __restrict__ residual,
                                                              const void* __restrict__ gamma, float eps, int cols,
-                                                             int gamma_dtype) {
+                                                             int gamma_dtype, int64_t x_stride) {
+    // x_stride: elements between two rows of x (a column slice of a wider matrix); every other tensor is dense
     __shared__ float red[NORM_THREADS / 64];
     const int64_t row = (int64_t)blockIdx.x * cols;
     const int nvec = cols >> 3;
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(uint16_t* __restr
     for (int it = 0; it < NORM_MAX_VEC; ++it) {
         const int c = threadIdx.x + it * NORM_THREADS;
         if (c < nvec) {
-            u32x4 raw = *(const u32x4*)(x + row + 8 * c);
+            u32x4 raw = *(const u32x4*)(x + (int64_t)blockIdx.x * x_stride + 8 * c);
             u32x4 rraw;
             if (residual) rraw = *(const u32x4*)(residual + row + 8 * c);
             load8_as_float(gamma, 8 * c, gamma_dtype, gm[it]);   // in flight together with the row, used after the sum
@@ -381,8 +382,8 @@ __global__ __launch_bounds__(THREADS) void silu_mul_quant_kernel(int8_t* __restr
 
 }  // namespace
 
-extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* residual, const void* gamma,
-                          float eps, int rows, int cols, int dtype, int gamma_dtype, void* stream) {
+static int rmsnorm_entry(void* y, void* sum_out, const void* x, int64_t x_row_stride, const void* residual,
+                         const void* gamma, float eps, int rows, int cols, int dtype, int gamma_dtype, void* stream) {
     MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "rmsnorm: dtype must be bf16 or fp16");
     MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32, "rmsnorm: bad gamma dtype");
     if (rows <= 0) return 0;
@@ -390,18 +391,30 @@ extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* res
     MF_REQUIRE(!residual || sum_out, "rmsnorm: residual given without sum_out");
     MF_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= NORM_THREADS * NORM_MAX_VEC * 8,
                "rmsnorm: cols (%d) must be a multiple of 8 and at most %d", cols, NORM_THREADS * NORM_MAX_VEC * 8);
+    MF_REQUIRE(x_row_stride >= cols && x_row_stride % 8 == 0,
+               "rmsnorm: the row stride of x (%lld) must be at least cols and a multiple of 8 elements",
+               (long long)x_row_stride);
     MF_REQUIRE((((uintptr_t)y | (uintptr_t)x | (uintptr_t)residual | (uintptr_t)sum_out | (uintptr_t)gamma) & 15) == 0,
                "rmsnorm: pointers must be 16-byte aligned");
-    if (rows <= 0) return 0;
     if (dtype == MF_BF16)
         hipLaunchKernelGGL(rmsnorm_kernel<BF16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
                            (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
-                           gamma_dtype);
+                           gamma_dtype, x_row_stride);
     else
         hipLaunchKernelGGL(rmsnorm_kernel<FP16>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (uint16_t*)y,
                            (uint16_t*)sum_out, (const uint16_t*)x, (const uint16_t*)residual, gamma, eps, cols,
-                           gamma_dtype);
+                           gamma_dtype, x_row_stride);
     return MF_LAUNCH_CHECK();
+}
+
+extern "C" int mf_rmsnorm(void* y, void* sum_out, const void* x, const void* residual, const void* gamma,
+                          float eps, int rows, int cols, int dtype, int gamma_dtype, void* stream) {
+    return rmsnorm_entry(y, sum_out, x, cols, residual, gamma, eps, rows, cols, dtype, gamma_dtype, stream);
+}
+
+extern "C" int mf_rmsnorm_strided(void* y, const void* x, int64_t x_row_stride, const void* gamma, float eps, int rows,
+                                  int cols, int dtype, int gamma_dtype, void* stream) {
+    return rmsnorm_entry(y, nullptr, x, x_row_stride, nullptr, gamma, eps, rows, cols, dtype, gamma_dtype, stream);
 }
 
 extern "C" int mf_silu_mul(void* out, const void* gate_up, int rows, int cols, int layout, int dtype,

@@ -588,11 +588,13 @@ constexpr int RN_THREADS = 512;
 constexpr int RN_MAX_VEC = 4;                                 // N <= 512 * 4 * 8 = 16384
 constexpr int RN_SPLITS = 8;                                  // splits whose loads are in flight together
 
+// norm_cols: the norm covers the leading norm_cols columns of a row (a multiple of 8; y is dense [M, norm_cols]); the
+// other columns are summed and written to h_out only.  residual may be null (no add).
 template <typename T>
 __global__ __launch_bounds__(RN_THREADS) void w8a16_reduce_add_rmsnorm_kernel(
     uint16_t* __restrict__ y, uint16_t* __restrict__ h_out, const float* __restrict__ partial,
     const float* __restrict__ scale, const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual,
-    const void* __restrict__ gamma, float eps, int M, int N, int split_k, int gamma_dtype) {
+    const void* __restrict__ gamma, float eps, int M, int N, int split_k, int gamma_dtype, int norm_cols) {
     __shared__ float red[RN_THREADS / 64];
     const int m = blockIdx.x;
     const int nvec = N >> 3;
@@ -604,10 +606,12 @@ __global__ __launch_bounds__(RN_THREADS) void w8a16_reduce_add_rmsnorm_kernel(
         const int c = threadIdx.x + it * RN_THREADS;
         if (c < nvec) {
             const int n = 8 * c;
+            const bool normed = n < norm_cols;
             const float* p = partial + (int64_t)m * N + n;
             const f32x4 s_lo = *(const f32x4*)(scale + n), s_hi = *(const f32x4*)(scale + n + 4);
-            const u32x4 rraw = *(const u32x4*)(residual + (int64_t)m * N + n);
-            load8_as_float(gamma, n, gamma_dtype, gm[it]);
+            u32x4 rraw = {0u, 0u, 0u, 0u};
+            if (residual) rraw = *(const u32x4*)(residual + (int64_t)m * N + n);
+            if (normed) load8_as_float(gamma, n, gamma_dtype, gm[it]);
             f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
             for (int s0 = 0; s0 < split_k; s0 += RN_SPLITS) {  // summed in split order
                 f32x4 a[RN_SPLITS], b[RN_SPLITS];
@@ -631,28 +635,31 @@ __global__ __launch_bounds__(RN_THREADS) void w8a16_reduce_add_rmsnorm_kernel(
             for (int i = 0; i < 4; ++i) {
                 const float t0 = dequant_bias<T>(lo[i], s_lo[i], bias, n + i);
                 const float t1 = dequant_bias<T>(hi[i], s_hi[i], bias, n + 4 + i);
-                v[it][i] = __fadd_rn(T::to_float(T::from_float(t0)), rr[i]);
-                v[it][4 + i] = __fadd_rn(T::to_float(T::from_float(t1)), rr[4 + i]);
+                const float r0 = T::to_float(T::from_float(t0)), r1 = T::to_float(T::from_float(t1));
+                v[it][i] = residual ? __fadd_rn(r0, rr[i]) : r0;
+                v[it][4 + i] = residual ? __fadd_rn(r1, rr[4 + i]) : r1;
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) hp[i] = pack2<T>(v[it][2 * i], v[it][2 * i + 1]);
             *(u32x4*)(h_out + (int64_t)m * N + n) = hp;
             unpack8<T>(hp, v[it]);                            // the norm sees the rounded h
+            if (normed) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[it][i], v[it][i], ss);
+                for (int i = 0; i < 8; ++i) ss = __fmaf_rn(v[it][i], v[it][i], ss);
+            }
         }
     }
     const float tot = rmsnorm_block_sum<RN_THREADS>(ss, red);
-    const float inv = rsqrtf(tot / (float)N + eps);
+    const float inv = rsqrtf(tot / (float)norm_cols + eps);
 #pragma unroll
     for (int it = 0; it < RN_MAX_VEC; ++it) {
         const int c = threadIdx.x + it * RN_THREADS;
-        if (c < nvec) {
+        if (c < nvec && 8 * c < norm_cols) {
             u32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 o[i] = pack2<T>(v[it][2 * i] * inv * gm[it][2 * i], v[it][2 * i + 1] * inv * gm[it][2 * i + 1]);
-            *(u32x4*)(y + (int64_t)m * N + 8 * c) = o;
+            *(u32x4*)(y + (int64_t)m * norm_cols + 8 * c) = o;
         }
     }
 }
@@ -869,7 +876,9 @@ template <typename T>
 int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, const void* bias,
                  const void* residual, int m, int n, int k, int gated, void* workspace, hipStream_t st,
                  void* norm_out = nullptr, const void* gamma = nullptr, float eps = 0.f, int gamma_dtype = MF_FP32,
-                 const RopeCacheArgs* rc_args = nullptr, int w4_group = -1) {
+                 const RopeCacheArgs* rc_args = nullptr, int w4_group = -1, int norm_cols = 0) {
+    // norm_cols: columns the norm in norm_out covers (the leading ones; 0 = the whole row)
+    if (norm_cols <= 0) norm_cols = n;
     // w4_group >= 0: 4-bit weights; 0 = `scale` holds one value per channel, 64 / 128 = one per channel and group
     // ([K / group][N]), applied inside the kernel (the epilogues then see no scale)
     const GemmPlan p = plan_w8a16(m, n, k, w4_group == 128 ? 2 : 1);
@@ -940,11 +949,11 @@ int launch_w8a16(void* y, const void* x, const uint8_t* wp, const float* scale, 
     if (norm_out && partial) {                                // reduce + residual + RMSNorm in one kernel
         hipLaunchKernelGGL((w8a16_reduce_add_rmsnorm_kernel<T>), dim3(m), dim3(RN_THREADS), 0, st, (uint16_t*)norm_out,
                            (uint16_t*)y, partial, scale, (const uint16_t*)bias, (const uint16_t*)residual, gamma, eps, m,
-                           n, p.split_k, gamma_dtype);
+                           n, p.split_k, gamma_dtype, norm_cols);
         return MF_LAUNCH_CHECK();
     }
     if (norm_out)                                             // no split: the GEMM wrote h; normalise it
-        return mf_rmsnorm(norm_out, nullptr, y, nullptr, gamma, eps, m, n, T::id, gamma_dtype, st);
+        return mf_rmsnorm_strided(norm_out, y, n, gamma, eps, m, norm_cols, T::id, gamma_dtype, st);
     if (!partial) return rc;
     const int64_t total = (int64_t)m * ((n + 3) / 4);
     const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
@@ -1029,6 +1038,35 @@ extern "C" int mf_w8a16_gemm_add_rmsnorm(void* y_norm, void* h_out, const void* 
                                   (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
     return launch_w8a16<FP16>(h_out, x, (const uint8_t*)w_packed, scale, bias, residual, m, n, k, 0, workspace,
                               (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype);
+}
+
+extern "C" int mf_w8a16_gemm_rmsnorm_leading(void* y_norm, void* h_out, const void* x, const void* w_packed,
+                                             const float* scale, const void* bias, const void* gamma, float eps, int m,
+                                             int n, int k, int norm_cols, int dtype, int gamma_dtype, void* workspace,
+                                             size_t workspace_bytes, void* stream) {
+    MF_REQUIRE(dtype == MF_BF16 || dtype == MF_FP16, "w8a16_gemm_rmsnorm_leading: dtype must be bf16 or fp16");
+    MF_REQUIRE(gamma_dtype == MF_BF16 || gamma_dtype == MF_FP16 || gamma_dtype == MF_FP32,
+               "w8a16_gemm_rmsnorm_leading: bad gamma dtype");
+    if (m == 0) return 0;
+    MF_REQUIRE(y_norm && h_out && x && w_packed && scale && gamma, "w8a16_gemm_rmsnorm_leading: null argument");
+    MF_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 8 == 0, "w8a16_gemm_rmsnorm_leading: bad sizes m=%d n=%d k=%d", m, n, k);
+    MF_REQUIRE(n % 8 == 0 && n <= RN_THREADS * RN_MAX_VEC * 8,
+               "w8a16_gemm_rmsnorm_leading: N (%d) must be a multiple of 8 and at most %d", n,
+               RN_THREADS * RN_MAX_VEC * 8);
+    MF_REQUIRE(norm_cols > 0 && norm_cols <= n && norm_cols % 8 == 0,
+               "w8a16_gemm_rmsnorm_leading: norm_cols (%d) must be a multiple of 8 in 8 .. N (%d)", norm_cols, n);
+    MF_REQUIRE((((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)y_norm | (uintptr_t)h_out | (uintptr_t)gamma |
+                 (uintptr_t)scale | (uintptr_t)bias) & 15) == 0,
+               "w8a16_gemm_rmsnorm_leading: pointers must be 16-byte aligned");
+    const size_t need = mf_w8a16_workspace_bytes(m, n, k);
+    MF_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0),
+               "w8a16_gemm_rmsnorm_leading: 16-byte aligned workspace of %zu bytes needed, %zu given", need,
+               workspace_bytes);
+    if (dtype == MF_BF16)
+        return launch_w8a16<BF16>(h_out, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                                  (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype, nullptr, -1, norm_cols);
+    return launch_w8a16<FP16>(h_out, x, (const uint8_t*)w_packed, scale, bias, nullptr, m, n, k, 0, workspace,
+                              (hipStream_t)stream, y_norm, gamma, eps, gamma_dtype, nullptr, -1, norm_cols);
 }
 
 extern "C" int mf_w8a16_qkv_rope_and_cache(void* qkv, const void* x, const void* w_packed, const float* scale,

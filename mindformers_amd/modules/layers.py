@@ -218,6 +218,23 @@ class WeightQuantLinearCell(_QuantLinearBase):
 
     construct = forward
 
+    def forward_with_leading_norm(self, x, gamma, eps):
+        """The projection together with an RMSNorm over its leading ``gamma.numel()`` output columns (the fused
+        query / latent down projection of multi-latent attention followed by q_layernorm): returns (y [T, out],
+        norm(y[:, :c]) * gamma [T, c]), the bits of ``forward`` followed by the norm on the column slice."""
+        x2 = x.reshape(-1, self.in_channels)
+        if x2.dtype != self.dtype:
+            x2 = x2.to(self.dtype)
+        if self.weight_bits != 8 or gamma.numel() % 8 or self.out_channels % 8 or self.out_channels > 16384:
+            y = self._matmul(x2.contiguous())
+            return y, ops.rms_norm(y[:, :gamma.numel()], gamma, eps)
+        if self._packed is None:
+            self.prepare()
+        x2 = x2.contiguous()
+        if self.smooth_scale is not None:
+            x2 = ops.scale_columns(x2, self.smooth_scale)
+        return ops.w8a16_linear_rmsnorm_leading(x2, self._packed, gamma, eps, bias=self.bias)
+
 
 class AllQuantLinearInferCell(_QuantLinearBase):
     """W8A8 deploy cell: per-token dynamic activation quantisation (with the SmoothQuant multiplier), or static

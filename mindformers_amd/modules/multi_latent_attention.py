@@ -150,9 +150,16 @@ class MLASelfAttention(nn.Module):
         n, nope, rope, rank = c.num_attention_heads, c.qk_head_dim, c.qk_pos_emb_head_dim, c.kv_lora_rank
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
         if c.q_lora_rank is not None:
-            qkv = self.linear_qkv_down_proj(x)
+            down, qn = self.linear_qkv_down_proj, self.q_layernorm
+            if hasattr(down, "forward_with_leading_norm") and isinstance(getattr(qn, "weight", None), torch.Tensor) \
+                    and hasattr(qn, "eps") and qn.weight.numel() == c.q_lora_rank:
+                # weight-only down projection: its split-K sum and q_layernorm are one kernel
+                qkv, q_c = down.forward_with_leading_norm(x, qn.weight, qn.eps)
+            else:
+                qkv = down(x)
+                q_c = qn(qkv[:, : c.q_lora_rank])             # the norm reads the column slice where it lies
             kv = qkv[:, c.q_lora_rank:]                       # latent part, then the rotary key part
-            q = self.linear_q_up_proj(self.q_layernorm(qkv[:, : c.q_lora_rank]))
+            q = self.linear_q_up_proj(q_c)
         else:
             kv = self.linear_kv_down_proj(x)
             q = self.linear_q_proj(x)

@@ -22,7 +22,7 @@ class LlamaRMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(dim, dtype=compute_type, device=device), requires_grad=False)
 
     def forward(self, x, residual=None):
-        return ops.rms_norm(x.contiguous(), self.weight, self.eps, residual=residual)
+        return ops.rms_norm(x, self.weight, self.eps, residual=residual)     # a column slice is read where it lies
 
     construct = forward
 
@@ -45,6 +45,6 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=ct, device=device), requires_grad=False)
 
     def forward(self, x, residual=None):
-        return ops.rms_norm(x.contiguous(), self.weight, self.eps, residual=residual)
+        return ops.rms_norm(x, self.weight, self.eps, residual=residual)     # a column slice is read where it lies
 
     construct = forward

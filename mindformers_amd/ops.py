@@ -566,13 +566,23 @@ def swap_cache(host_cache, device_cache, block_mapping, is_device_to_host):
 
 # --------------------------------------------------------------------------------------------- norm / activation
 def rms_norm(x, gamma, eps, residual=None):
-    """RmsNorm(eps)(x, gamma).  With ``residual``: returns (norm(x + residual), x + residual)."""
+    """RmsNorm(eps)(x, gamma).  With ``residual``: returns (norm(x + residual), x + residual).  Without it, x may
+    be a column slice of a wider 2-D matrix (unit column stride): the rows are read where they lie."""
     lib = _lib.load()
-    dev = _dev_ok(x, gamma, residual)
     _need(x.dtype in _ACT, "x must be bf16/fp16")
     cols = x.shape[-1]
-    rows = x.numel() // cols
     _need(gamma.numel() == cols, "gamma size")
+    if residual is None and x.dim() == 2 and not x.is_contiguous() and x.stride(1) == 1 and x.stride(0) % 8 == 0 \
+            and x.stride(0) >= cols and x.data_ptr() % 16 == 0:
+        dev = _dev_ok(gamma)
+        _need(x.is_cuda and x.device == dev, "all tensors must be on the same device")
+        y = torch.empty(x.shape, dtype=x.dtype, device=dev)
+        check(lib.mf_rmsnorm_strided(ptr(y), ptr(x), x.stride(0), ptr(gamma), float(eps), x.shape[0], cols,
+                                     dtype_code(x.dtype), dtype_code(gamma.dtype), stream_ptr(dev)), "mf_rmsnorm_strided")
+        return y
+    x = x.contiguous()
+    dev = _dev_ok(x, gamma, residual)
+    rows = x.numel() // cols
     y = torch.empty_like(x)
     s = None
     if residual is not None:
@@ -762,6 +772,30 @@ def w8a16_linear_add_rmsnorm(x, w, residual, gamma, eps, bias=None):
                                         ptr(gamma), float(eps), m, n, k, dtype_code(x.dtype), dtype_code(gamma.dtype),
                                         ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
           "mf_w8a16_gemm_add_rmsnorm")
+    return h, y
+
+
+def w8a16_linear_rmsnorm_leading(x, w, gamma, eps, bias=None):
+    """A projection whose leading ``gamma.numel()`` columns feed an RMSNorm (the fused query / latent down projection
+    of multi-latent attention with its q_layernorm): returns (h, norm(h[:, :c]) * gamma) with h = (x . w^T) * scale
+    (+bias).  Bit-identical to w8a16_linear followed by rms_norm on the column slice."""
+    lib = _lib.load()
+    _need(isinstance(w, PackedInt8Weight) and w.experts is None and not w.gated, "w must be a packed [N, K] weight")
+    dev = _dev_ok(x, bias, gamma)
+    _need(x.dtype in _ACT, "x must be bf16/fp16")
+    n, k, c = w.n, w.k, gamma.numel()
+    _need(x.shape[-1] == k, f"x has {x.shape[-1]} input channels, weight expects {k}")
+    _need(0 < c <= n and c % 8 == 0 and n % 8 == 0, "the normed columns must be a multiple of 8 within the output")
+    m = x.numel() // k
+    h = torch.empty(m, n, dtype=x.dtype, device=dev)
+    y = torch.empty(m, c, dtype=x.dtype, device=dev)
+    _need(bias is None or (bias.dtype == x.dtype and bias.numel() == n), "bias mismatch")
+    need = lib.mf_w8a16_workspace_bytes(m, n, k)
+    ws = workspace(need, dev, "gemm") if need else None
+    check(lib.mf_w8a16_gemm_rmsnorm_leading(ptr(y), ptr(h), ptr(x), ptr(w.packed), ptr(w.scale), ptr(bias), ptr(gamma),
+                                            float(eps), m, n, k, c, dtype_code(x.dtype), dtype_code(gamma.dtype),
+                                            ptr(ws), ws.numel() if ws is not None else 0, stream_ptr(dev)),
+          "mf_w8a16_gemm_rmsnorm_leading")
     return h, y
 
 

@@ -807,6 +807,18 @@ def test_rmsnorm(dtype, rows, cols, gdt):
     assert_within(to_np(y2), ref2, np.abs(ref2), dtype, ulps=1.0, extra=1e-7, what="add+rmsnorm")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,width,start,cols", [(64, 2112, 0, 1536), (5, 2112, 1536, 512), (3, 96, 8, 32)])
+def test_rmsnorm_on_a_column_slice_equals_the_dense_norm(dtype, rows, width, start, cols):
+    """The norm reads a column slice of a wider matrix where it lies: the bits of the norm of a dense copy."""
+    rng = np.random.default_rng(rows + width)
+    x = dev(rounded(rng.normal(size=(rows, width)), dtype), dtype)
+    g = torch.from_numpy(rng.normal(1.0, 0.1, cols).astype(np.float32)).cuda()
+    view = x[:, start:start + cols]
+    assert not view.is_contiguous()
+    assert torch.equal(ops.rms_norm(view, g, 1e-6), ops.rms_norm(view.contiguous(), g, 1e-6))
+
+
 def test_rmsnorm_reference_vectors(golden_dir):
     z = np.load(os.path.join(golden_dir, "norm.npz"))
     for name, eps in (("rmsnorm_output1", 1e-5), ("rmsnorm_output2", 0.1)):
@@ -928,6 +940,26 @@ def test_w8a16_linear_add_rmsnorm_equals_unfused(dtype, m, n, k, bias):
     y_ref = ops.rms_norm(h_ref, gamma, 1e-5)
     assert torch.equal(h, h_ref)
     assert torch.equal(y, y_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k,c,bias", [(64, 2112, 7168, 1536, False),    # the DeepSeek-V3 down projection: 8 k-splits
+                                          (20, 2112, 512, 1536, True),     # K too short to split: GEMM, then the norm
+                                          (7, 640, 1376, 640, True),       # the norm over the whole row, no residual
+                                          (130, 1024, 2048, 8, False)])
+def test_w8a16_linear_rmsnorm_leading_equals_unfused(dtype, m, n, k, c, bias):
+    """Projection + RMSNorm over its leading columns in one call: bit-identical to the GEMM followed by the norm of the
+    column slice, on shapes that split K (the split sum and the norm are one kernel) and shapes that do not."""
+    rng = np.random.default_rng(m + n + k + c)
+    wq, s = O.quantize_weight_int8(rng.normal(0, 0.02, (n, k)).astype(np.float32))
+    x = dev(rounded(rng.normal(size=(m, k)), dtype), dtype)
+    gamma = torch.from_numpy((1 + 0.1 * rng.normal(size=c)).astype(np.float32)).cuda()
+    b = dev(rounded(rng.normal(0, 0.1, n), dtype), dtype) if bias else None
+    packed = ops.pack_w8a16(torch.from_numpy(wq).cuda(), torch.from_numpy(s).cuda())
+    h, y = ops.w8a16_linear_rmsnorm_leading(x, packed, gamma, 1e-6, bias=b)
+    h_ref = ops.w8a16_linear(x, packed, bias=b)
+    assert torch.equal(h, h_ref)
+    assert y.shape == (m, c) and torch.equal(y, ops.rms_norm(h_ref[:, :c].contiguous(), gamma, 1e-6))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
