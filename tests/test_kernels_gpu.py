@@ -189,24 +189,26 @@ def test_paged_attention_long_contexts_vs_oracle(dtype, b, nh, nkv, d, bs, lens,
     assert_within(got, ref, mag, dtype, ulps=1.5, what="paged attention, long contexts")
 
 
-@pytest.mark.parametrize("b,nkv,max_blocks,part,hi", [
-    (200, 2, 32, 512, 4096),     # 400 (sequence, kv head) pairs x 8 partitions of 512 tokens: 3200 workgroups
-    (64, 2, 136, 1024, 3000),    # capacity 17408 tokens: 128 pairs x 17 partitions of 1024, too few of 2048
-    (400, 2, 24, 2048, 3072),    # 800 pairs fill the device by themselves: 2048-token partitions
-    (400, 2, 16, 2048, 2048),    # the same with one partition per sequence: no combine, rows written directly
+@pytest.mark.parametrize("dtype,b,nkv,d,bs,max_blocks,part,hi", [
+    (torch.bfloat16, 200, 2, 32, 128, 32, 512, 4096),    # 400 (sequence, kv head) pairs x 8 partitions of 512 tokens
+    (torch.bfloat16, 64, 2, 32, 128, 136, 1024, 3000),   # capacity 17408: 128 pairs x 17 partitions of 1024, too few of 2048
+    (torch.bfloat16, 400, 2, 32, 128, 24, 2048, 3072),   # 800 pairs fill the device by themselves: 2048-token partitions
+    (torch.bfloat16, 400, 2, 32, 128, 16, 2048, 2048),   # the same, one partition per sequence: no combine, rows written directly
+    (torch.float16, 400, 2, 64, 48, 64, 2048, 3072),     # blocks that 32-token tiles straddle, fp16, head_dim 64
+    (torch.bfloat16, 100, 8, 128, 128, 16, 2048, 2048),  # head_dim 128, 8 kv heads, one partition per sequence
 ])
-def test_paged_attention_large_batches_take_larger_partitions(b, nkv, max_blocks, part, hi):
+def test_paged_attention_large_batches_take_larger_partitions(dtype, b, nkv, d, bs, max_blocks, part, hi):
     """Large batches of 16-bit caches run 512-, 1024- or 2048-token partitions (chosen on the batch and the context
     capacity); ragged lengths with empty sequences and lengths on and next to the partition borders."""
     rng = np.random.default_rng(b + part + max_blocks)
-    cap = max_blocks * 128
+    cap = max_blocks * bs
     lens = rng.integers(1, hi + 1, b)
     lens[:8] = [0, 1, part - 1, min(part, cap), min(part + 1, cap), min(2 * part, cap), cap - 1, cap]
     empty = sorted({0, min(63, b - 2), min(64, b - 1), b - 1})   # no context, on both sides of a 64-wide scan chunk
     lens[empty] = 0
-    got, ref, mag = _pa_case(rng, torch.bfloat16, b, 2 * nkv, nkv, 32, 128, lens, max_blocks=max_blocks)
+    got, ref, mag = _pa_case(rng, dtype, b, 2 * nkv, nkv, d, bs, lens, max_blocks=max_blocks)
     assert not got[empty].any()                               # a sequence without context: zeros
-    assert_within(got, ref, mag, torch.bfloat16, ulps=1.5, what=f"paged attention, {part}-token partitions")
+    assert_within(got, ref, mag, dtype, ulps=1.5, what=f"paged attention, {part}-token partitions")
 
 
 def test_paged_attention_edge_lengths():
